@@ -1,0 +1,80 @@
+"""Builds libdgpp_amd.so (HIP kernels for gfx950 + the C ABI + host encoders) in-tree.
+
+hipcc cross-compiles without a GPU. Objects go to dgpp_amd/_build/, the library to
+dgpp_amd/lib/libdgpp_amd.so. Run as `python -m dgpp_amd.build`.
+"""
+from __future__ import annotations
+
+import concurrent.futures as cf
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+CSRC = PKG / "csrc"
+BUILD = PKG / "_build"
+LIB_DIR = PKG / "lib"
+LIB = LIB_DIR / "libdgpp_amd.so"
+
+HIP_SOURCES = [
+    "gemv_mxfp4.hip",
+    "gemv_nvfp4.hip",
+    "gemv_fp8f32.hip",
+    "gemv_fp8e8m0.hip",
+    "moe_misc.hip",
+    "capi.hip",
+]
+HOST_SOURCES = ["host_codec.cpp"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# Packed-FP32 instruction selection is switched off for all device code.
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result",
+]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-ffp-contract=off", "-pthread"]
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"command failed: {' '.join(cmd)}\n{proc.stdout}\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+
+
+def _stale(obj: Path, src: Path) -> bool:
+    if not obj.exists():
+        return True
+    newest = max(p.stat().st_mtime for p in list(CSRC.glob("*.hpp")) + [src, PKG.parent / "include" / "dgpp_amd.h"])
+    return obj.stat().st_mtime < newest
+
+
+def build(force: bool = True, jobs: int = 6) -> Path:
+    """Compiles every source (always, when force) and links the shared library."""
+    BUILD.mkdir(exist_ok=True)
+    LIB_DIR.mkdir(exist_ok=True)
+    tasks = []
+    objs = []
+    for name in HIP_SOURCES:
+        src, obj = CSRC / name, BUILD / (name + ".o")
+        objs.append(obj)
+        if force or _stale(obj, src):
+            tasks.append([HIPCC, *HIP_FLAGS, "-c", str(src), "-o", str(obj)])
+    for name in HOST_SOURCES:
+        src, obj = CSRC / name, BUILD / (name + ".o")
+        objs.append(obj)
+        if force or _stale(obj, src):
+            tasks.append([shutil.which("g++") or "g++", *HOST_FLAGS, "-c", str(src), "-o", str(obj)])
+    with cf.ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(_run, tasks))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)])
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--incremental" not in sys.argv))

@@ -1,0 +1,698 @@
+// The C ABI (include/dgpp_amd.h): argument validation mirroring the reference launchers'
+// std::invalid_argument rules, then dispatch to the kernels. Nothing here allocates or syncs.
+#include <hip/hip_runtime.h>
+
+#include <limits.h>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "../../include/dgpp_amd.h"
+#include "gemv_kernels.hpp"
+#include "moe_misc.hpp"
+
+using namespace dgpp_amd;
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail_arg(const std::string& what) {
+  g_last_error = what;
+  return DGPP_INVALID_ARGUMENT;
+}
+int finish(hipError_t err, const char* who) {
+  if (err == hipSuccess) return DGPP_OK;
+  g_last_error = std::string(who) + ": " + hipGetErrorString(err);
+  (void)hipGetLastError();  // drain the sticky error like the reference's check macro
+  return DGPP_RUNTIME_ERROR;
+}
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// src/kernels/fp4_gemv.cuh:110-125 (k_supported) and :771-788 (the compiled sets).
+bool fp4_k_supported(int k) { return k >= 32 && k % 32 == 0 && k <= 16384; }
+bool fp4_k_compiled(int k, int group) {
+  static const int nv[] = {32, 64, 128, 160, 256, 320, 384, 512, 640, 768, 1024, 1536, 2048, 2560, 3072, 4096, 5120, 6144, 7168, 12288};
+  static const int mx[] = {32, 64, 128, 256, 512, 576, 1024, 1152, 2048, 2304, 4096, 5120};
+  if (group == 32) {
+    for (int v : mx) if (v == k) return true;
+    return false;
+  }
+  for (int v : nv) if (v == k) return true;
+  return false;
+}
+// src/kernels/fp8_gemv.cuh:47-50: k a positive multiple of 16, 16-byte aligned payload, one row stageable.
+bool fp8_shape_ok(const void* payload, int k) {
+  return k > 0 && k % 16 == 0 && aligned16(payload) && stage_bytes(1, k) <= kMaxLdsBytes;
+}
+
+MatRef fp8_mat(const uint8_t* payload, const void* scales, int rs, int cs) {
+  MatRef m;
+  m.payload = payload;
+  m.scales = scales;
+  m.divisor = 1.f;
+  m.rs = rs;
+  m.cs = cs;
+  return m;
+}
+
+}  // namespace
+
+namespace dgpp_amd {
+hipError_t ensure_lds_impl(const void* kernel, size_t bytes) {
+  static std::mutex mu;
+  static std::unordered_map<const void*, size_t> raised;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = raised.find(kernel);
+  if (it != raised.end() && it->second >= bytes) return hipSuccess;
+  const hipError_t err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLdsBytes));
+  if (err == hipSuccess) raised[kernel] = kMaxLdsBytes;
+  return err;
+}
+
+hipError_t launch_dense(int fmt, const DenseArgs& a, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_dense_fmt<kFmtFp8F32>(a, s);
+    case kFmtFp8E8M0: return launch_dense_fmt<kFmtFp8E8M0>(a, s);
+    case kFmtNvfp4: return launch_dense_fmt<kFmtNvfp4>(a, s);
+    default: return launch_dense_fmt<kFmtMxfp4>(a, s);
+  }
+}
+hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_slot_gate_up_fmt<kFmtFp8F32>(a, s);
+    case kFmtNvfp4: return launch_slot_gate_up_fmt<kFmtNvfp4>(a, s);
+    default: return launch_slot_gate_up_fmt<kFmtMxfp4>(a, s);
+  }
+}
+hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_slot_down_fmt<kFmtFp8F32>(a, s);
+    case kFmtNvfp4: return launch_slot_down_fmt<kFmtNvfp4>(a, s);
+    default: return launch_slot_down_fmt<kFmtMxfp4>(a, s);
+  }
+}
+hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_grouped_fmt<kFmtFp8F32>(a, n_segs, z_ext, s);
+    case kFmtNvfp4: return launch_grouped_fmt<kFmtNvfp4>(a, n_segs, z_ext, s);
+    default: return launch_grouped_fmt<kFmtMxfp4>(a, n_segs, z_ext, s);
+  }
+}
+}  // namespace dgpp_amd
+
+namespace {
+
+// Dense GEMV over m rows in chunks the LDS can stage (each row's chain is the same whatever
+// the chunking). k == 0 zero-fills. `out_elem` is 2 (bf16) or 4 (f32).
+int dense_rows(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,
+               size_t out_stride, int out_f32, int m, int n, int k, hipStream_t stream, const char* who) {
+  const int max_rows = max_stage_rows(k);
+  const size_t esz = out_f32 ? 4 : 2;
+  for (int row0 = 0; row0 < m;) {
+    const int rows = std::min(max_rows, m - row0);
+    DenseArgs a;
+    a.act = act + static_cast<size_t>(row0) * act_stride;
+    a.act_stride = act_stride;
+    a.mat = mat;
+    a.global = global;
+    a.out = static_cast<uint8_t*>(out) + static_cast<size_t>(row0) * out_stride * esz;
+    a.out_stride = out_stride;
+    a.out_f32 = out_f32;
+    a.m = rows;
+    a.n = n;
+    a.k = k;
+    const int rc = finish(launch_dense(fmt, a, stream), who);
+    if (rc != DGPP_OK) return rc;
+    row0 += rows;
+  }
+  return DGPP_OK;
+}
+
+int fp4_gemv(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, void* out, int out_f32, int m, int n, int k,
+             void* stream) {
+  // src/kernels/fp4_gemv.cu:52-67
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  if (!w) return fail_arg("fp4_gemv: null pointer");
+  if (!act || !w->payload || !w->scales || !out) return fail_arg("fp4_gemv: null pointer");
+  if (w->scale_group != 16 && w->scale_group != 32)
+    return fail_arg("fp4_gemv: the scale group must be 16 (NVFP4) or 32 (MXFP4)");
+  if (w->scale_group == 16 && !w->global_scale) return fail_arg("fp4_gemv: an NVFP4 matrix needs its global scale");
+  if (w->rows < n || w->cols != k) return fail_arg("fp4_gemv: matrix geometry does not match n, k");
+  if (!fp4_k_supported(k) || !aligned16(w->payload) || !fp4_k_compiled(k, w->scale_group))
+    return fail_arg("fp4_gemv: K must be a multiple of 32 in the group's compiled set and the payload 16-byte aligned");
+  MatRef mat;
+  mat.payload = w->payload;
+  mat.scales = w->scales;
+  mat.divisor = 1.f;
+  mat.rs = 0;
+  mat.cs = 0;
+  return dense_rows(w->scale_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, mat, w->global_scale, out,
+                    static_cast<size_t>(n), out_f32, m, n, k, as_stream(stream), "fp4_gemv");
+}
+
+// src/kernels/scale_gemm.cu:280-365 (launch_scale_gemm) and :406-462 (launch_scale_gemm_grid):
+// every m takes the row-independent GEMV form here.
+int scale_gemm(const uint16_t* act, size_t act_stride, const uint8_t* payload, const void* scales, int e8m0, void* out,
+               int out_f32, int m, int n, int k, void* stream, size_t out_stride, int rs, int cs, int last_row_only,
+               int compact_row, bool grid_form, const char* who) {
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  if (!act || !payload || !scales || !out) return fail_arg(std::string(who) + ": null pointer");
+  if (grid_form) {
+    const bool row_grid = rs == 0 && cs >= 4;
+    if (!row_grid && (rs < 5 || rs > 7 || cs < 5 || cs > 7))
+      return fail_arg(std::string(who) + ": rs / cs must be 5..7 (32 .. 128 blocks) or a row grid (rs = 0, cs >= 4)");
+  }
+  if (out_stride == 0) out_stride = static_cast<size_t>(n);
+  if (out_stride < static_cast<size_t>(n)) return fail_arg(std::string(who) + ": output row stride narrower than n");
+  if (compact_row < -1 || compact_row >= m || (compact_row >= 0 && last_row_only))
+    return fail_arg(std::string(who) + ": invalid compact row selection");
+  const size_t esz = out_f32 ? 4 : 2;
+  uint8_t* o = static_cast<uint8_t*>(out);
+  if (last_row_only || compact_row >= 0) {
+    const int sel = compact_row >= 0 ? compact_row : m - 1;
+    act += static_cast<size_t>(sel) * act_stride;
+    if (last_row_only) o += static_cast<size_t>(sel) * out_stride * esz;
+    m = 1;
+  }
+  if (grid_form && (k <= 0 || k % 16 != 0)) return fail_arg(std::string(who) + ": k must be a positive multiple of 16");
+  if (k <= 0) {
+    // Degenerate contraction: zero outputs (src/kernels/scale_gemm.cu:303-309).
+    return finish(hipMemset2DAsync(o, out_stride * esz, 0, static_cast<size_t>(n) * esz, static_cast<size_t>(m),
+                                   as_stream(stream)),
+                  who);
+  }
+  if (!fp8_shape_ok(payload, k))
+    return fail_arg(std::string(who) + ": k must be a multiple of 16 with a 16-byte aligned payload");
+  return dense_rows(e8m0 ? kFmtFp8E8M0 : kFmtFp8F32, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, o,
+                    out_stride, out_f32, m, n, k, as_stream(stream), who);
+}
+
+// src/kernels/glm_moe.cu:1683-1703 (check_slot_args) and :2197-2228 (check_fp4_slot_args).
+int check_slot_common(const void* x, const int32_t* ids, const DgppMoeExpertView* views, const void* out, int n_routed,
+                      int k_routed, int n_shared, int k_shared, const char* who) {
+  if (!x || !ids || !views || !out) return fail_arg(std::string(who) + ": null pointer");
+  if (n_routed <= 0 || k_routed <= 0 || n_shared < 0 || k_shared < 0 || (n_shared > 0) != (k_shared > 0))
+    return fail_arg(std::string(who) + ": degenerate dims");
+  return DGPP_OK;
+}
+int check_fp4_slot(const void* x, const int32_t* ids, const DgppMoeExpertView* views, const void* out, int n_routed,
+                   int k_routed, int n_shared, int k_shared, int shared_view_base, int fp4_group, const char* who) {
+  if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
+  const int rc = check_slot_common(x, ids, views, out, n_routed, k_routed, n_shared, k_shared, who);
+  if (rc != DGPP_OK) return rc;
+  if (!fp4_k_supported(k_routed) || !fp4_k_compiled(k_routed, fp4_group))
+    return fail_arg(std::string(who) + ": routed k must be a multiple of 32 in the fp4 core's compiled set");
+  if (n_shared == 0) return DGPP_OK;
+  if (shared_view_base >= 0) {
+    if (k_shared != k_routed) return fail_arg(std::string(who) + ": the NVFP4 shared expert's k must equal the routed k");
+    return DGPP_OK;
+  }
+  if (k_shared % 16 != 0 || stage_bytes(1, k_shared) > kMaxLdsBytes)
+    return fail_arg(std::string(who) + ": shared k must be a multiple of 16");
+  return DGPP_OK;
+}
+
+SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                   const DgppMoeExpertView* views, void* out, int out_stride, int slots, int top_k, float limit) {
+  SlotArgs a{};
+  a.x = x;
+  a.x_stride = x_stride;
+  a.ids = ids;
+  a.order = order;
+  a.views = views;
+  a.out = out;
+  a.out_stride = out_stride;
+  a.slots = slots;
+  a.top_k = top_k;
+  a.limit = limit;
+  a.shared_view_base = -1;
+  return a;
+}
+
+int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
+            int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32, size_t out_stride,
+            int n, int k, void* stream, const char* who) {
+  if (max_rows <= 0) return fail_arg(std::string(who) + ": max_rows must be positive");
+  if (which < 0 || which > 2) return fail_arg(std::string(who) + ": which must be 0, 1 or 2");
+  const unsigned z_ext = rows_per_block > 0 ? static_cast<unsigned>((max_rows + rows_per_block - 1) / rows_per_block) : 1u;
+  if (n_segs > 65535 || z_ext > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
+  GroupedArgs a;
+  a.act = act;
+  a.act_stride = act_stride;
+  a.segs = segs;
+  a.views = views;
+  a.which = which;
+  a.out = out;
+  a.out_stride = out_stride;
+  a.out_f32 = out_f32;
+  a.n = n;
+  a.k = k;
+  a.rows_per_block = rows_per_block > 0 ? rows_per_block : INT_MAX;
+  a.group_rows = max_stage_rows(k);
+  return finish(launch_grouped(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* dgpp_last_error(void) { return g_last_error.c_str(); }
+const char* dgpp_target_arch(void) { return "gfx950"; }
+
+int dgpp_moe_config_validate(const DgppMoeConfig* c) {
+  // src/models/glm/moe.hpp:119-133
+  if (!c) return fail_arg("GlmMoeConfig: null");
+  if (c->hidden <= 0 || c->inter <= 0) return fail_arg("GlmMoeConfig: hidden/inter must be positive");
+  if (c->n_experts <= 0) return fail_arg("GlmMoeConfig: n_experts must be positive");
+  if (c->top_k <= 0 || c->top_k > 16) return fail_arg("GlmMoeConfig: top_k must be in [1, 16] (kernel register selection)");
+  if (c->top_k > c->n_experts) return fail_arg("GlmMoeConfig: top_k must not exceed n_experts");
+  if (c->n_experts > 4096) return fail_arg("GlmMoeConfig: n_experts must be <= 4096 (router smem: 2*n_experts floats)");
+  if (c->n_shared_experts != 0 && c->n_shared_experts != 1) return fail_arg("GlmMoeConfig: n_shared_experts must be 0 or 1");
+  if (!(c->swiglu_limit > 0)) return fail_arg("GlmMoeConfig: swiglu_limit must be positive");
+  if (c->router_mode < 0 || c->router_mode > 2) return fail_arg("GlmMoeConfig: unknown router mode");
+  return DGPP_OK;
+}
+
+int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const float* bias, int32_t* ids,
+                           float* weights, float* scores, float* biased, const DgppMoeConfig* cfg, int tokens,
+                           void* stream, int* counters, int allow_tiled) {
+  (void)counters;
+  (void)allow_tiled;
+  const int rc = dgpp_moe_config_validate(cfg);
+  if (rc != DGPP_OK) return rc;
+  if (tokens <= 0) return DGPP_OK;
+  const bool softmax = cfg->router_mode == DGPP_ROUTER_SOFTMAX_TOPK;
+  if (!hidden || !gate || (!softmax && !bias) || !ids || !weights || !scores || !biased)
+    return fail_arg("moe_router: null pointer");
+  if (scores == biased) return fail_arg("moe_router: scores and biased must not alias");
+  if (cfg->n_experts > 65535 || tokens > 65535) return fail_arg("moe_router: grid dimension overflow");
+  int r = finish(run_router_dots(cfg->router_mode, hidden, gate, bias, scores, biased, tokens, cfg->hidden,
+                                 cfg->n_experts, as_stream(stream)),
+                 "moe_router");
+  if (r != DGPP_OK) return r;
+  return finish(run_router_select(cfg->router_mode, scores, biased, ids, weights, tokens, cfg->n_experts, cfg->top_k,
+                                  cfg->routed_scaling_factor, cfg->norm_topk_prob ? 1 : 0, as_stream(stream)),
+                "moe_router");
+}
+
+int dgpp_launch_moe_router_select(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                  const DgppMoeConfig* cfg, int tokens, void* stream) {
+  const int rc = dgpp_moe_config_validate(cfg);
+  if (rc != DGPP_OK) return rc;
+  if (tokens <= 0) return DGPP_OK;
+  if (!scores || !biased || !ids || !weights) return fail_arg("moe_router_select: null pointer");
+  if (tokens > 65535) return fail_arg("moe_router_select: grid dimension overflow");
+  return finish(run_router_select(cfg->router_mode, scores, biased, ids, weights, tokens, cfg->n_experts, cfg->top_k,
+                                  cfg->routed_scaling_factor, cfg->norm_topk_prob ? 1 : 0, as_stream(stream)),
+                "moe_router_select");
+}
+
+int dgpp_launch_moe_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, float limit,
+                                 void* stream) {
+  if (n <= 0) return DGPP_OK;
+  if (!gate || !up || !out) return fail_arg("moe_swiglu: null pointer");
+  return finish(run_swiglu_clamp(gate, up, out, n, limit, as_stream(stream)), "moe_swiglu");
+}
+
+int dgpp_launch_moe_gather_rows(const uint16_t* src, const int32_t* rows, uint16_t* dst, int n_rows, int hidden,
+                                void* stream) {
+  if (n_rows <= 0) return DGPP_OK;
+  if (!src || !rows || !dst) return fail_arg("moe_gather: null pointer");
+  return finish(run_gather_rows(src, rows, dst, n_rows, hidden, as_stream(stream)), "moe_gather");
+}
+
+int dgpp_launch_moe_accum(float* acc, const float* y, const int32_t* rows, const float* row_weights, int n_rows,
+                          int hidden, void* stream) {
+  if (n_rows <= 0) return DGPP_OK;
+  if (!acc || !y || !rows || !row_weights) return fail_arg("moe_accum: null pointer");
+  return finish(run_accum(acc, y, rows, row_weights, n_rows, hidden, as_stream(stream)), "moe_accum");
+}
+
+int dgpp_launch_moe_round_bf16(uint16_t* out, const float* acc, int64_t n, void* stream) {
+  if (n <= 0) return DGPP_OK;
+  if (!out || !acc) return fail_arg("moe_round: null pointer");
+  return finish(run_round_bf16(out, acc, n, as_stream(stream)), "moe_round");
+}
+
+int dgpp_launch_moe_segment(const int32_t* ids, int tokens, int top_k, int n_experts, int32_t* rows,
+                            int32_t* slot_row, DgppMoeSegment* segs, void* stream) {
+  if (tokens <= 0) return DGPP_OK;
+  if (!ids || !rows || !slot_row || !segs) return fail_arg("moe segment: null pointer");
+  if (top_k < 1 || top_k > 16 || n_experts < 1 || n_experts > 1024)
+    return fail_arg("moe segment: top_k or n_experts out of range");
+  return finish(run_segment(ids, tokens, top_k, n_experts, rows, slot_row, segs, as_stream(stream)), "moe segment");
+}
+
+int dgpp_moe_tile_list_capacity(int n_segs, int total_rows, int tile_rows) {
+  return n_segs + (total_rows + tile_rows - 1) / tile_rows;
+}
+
+int dgpp_launch_moe_tile_list(const DgppMoeSegment* segs, int n_segs, int tile_rows, DgppMoeTile* tiles,
+                              int32_t* count, void* stream) {
+  if (!segs || !tiles || !count) return fail_arg("moe tile list: null pointer");
+  if (n_segs < 1 || n_segs > 65535 || tile_rows < 1) return fail_arg("moe tile list: n_segs or tile_rows out of range");
+  return finish(run_tile_list(segs, n_segs, tile_rows, tiles, count, as_stream(stream)), "moe tile list");
+}
+
+int dgpp_moe_run_groups_max(int slots) { return slots / 17 + 1; }
+
+int dgpp_launch_moe_slot_order(const int32_t* ids, int32_t* order, int slots, int top_k, int n_experts, void* stream,
+                               int shared_early, int32_t* runs) {
+  if (slots <= 0) return DGPP_OK;
+  if (!ids || !order) return fail_arg("moe_slot_order: null");
+  if (slots > 1024) return fail_arg("moe_slot_order: more slots than one block");
+  return finish(run_slot_order(ids, order, runs, slots, top_k, n_experts, shared_early ? 1 : 0, as_stream(stream)),
+                "moe_slot_order");
+}
+
+int dgpp_minimax_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* output, int experts, int capacity,
+                                  void* stream) {
+  if (!input || !output || input == output || experts < 1 || experts > 1024 || capacity < 1 || capacity > experts)
+    return fail_arg("MiniMax segment compaction geometry");
+  return finish(run_compact_segments(input, output, experts, capacity, as_stream(stream)), "minimax_compact_segments");
+}
+
+static int accum_ordered(void* out, int out_f32, const float* down, size_t down_stride, const int32_t* slot_row,
+                         const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens, int top_k,
+                         int hidden, void* stream) {
+  if (tokens <= 0) return DGPP_OK;
+  if (!out || !down || !slot_row || !slot_ids || !slot_w) return fail_arg("moe accum ordered: null pointer");
+  if (top_k < 1 || top_k > 16) return fail_arg("moe accum ordered: top_k outside [1, 16]");
+  return finish(run_accum_ordered(out, out_f32, down, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens,
+                                  top_k, hidden, as_stream(stream)),
+                "moe accum ordered");
+}
+int dgpp_launch_moe_accum_ordered(uint16_t* out, const float* down, size_t down_stride, const int32_t* slot_row,
+                                  const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens,
+                                  int top_k, int hidden, void* stream) {
+  return accum_ordered(out, 0, down, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens, top_k, hidden, stream);
+}
+int dgpp_launch_moe_accum_ordered_f32(float* out, const float* down, size_t down_stride, const int32_t* slot_row,
+                                      const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens,
+                                      int top_k, int hidden, void* stream) {
+  return accum_ordered(out, 1, down, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens, top_k, hidden, stream);
+}
+
+int dgpp_launch_moe_slot_accum(uint16_t* out, const float* contrib, const float* weights, int tokens, int hidden,
+                               int top_k, void* stream) {
+  if (tokens <= 0) return DGPP_OK;
+  if (!out || !contrib || !weights) return fail_arg("moe_slot_accum: null pointer");
+  return finish(run_slot_accum(out, 0, 1, contrib, weights, tokens, hidden, top_k, as_stream(stream)), "moe_slot_accum");
+}
+int dgpp_launch_moe_slot_accum_routed_f32(float* out, const float* contrib, const float* weights, int tokens,
+                                          int hidden, int top_k, void* stream) {
+  if (tokens <= 0) return DGPP_OK;
+  if (!out || !contrib || !weights) return fail_arg("moe_slot_accum_routed_f32: null pointer");
+  return finish(run_slot_accum(out, 1, 0, contrib, weights, tokens, hidden, top_k, as_stream(stream)),
+                "moe_slot_accum_routed_f32");
+}
+
+int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                                        const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                        int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                        const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                        int act_stride, int slots, int top_k, float limit, void* stream, int sh_rs,
+                                        int sh_cs) {
+  const char* who = "moe_slot_gate_up";
+  if (slots <= 0) return DGPP_OK;
+  int rc = check_slot_common(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, who);
+  if (rc != DGPP_OK) return rc;
+  if (k_routed % 16 != 0 || stage_bytes(1, k_routed) > kMaxLdsBytes)
+    return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
+  if (n_shared > 0 && (!sh_gate_payload || !sh_gate_scales || !sh_up_payload || !sh_up_scales ||
+                       !fp8_shape_ok(sh_gate_payload, k_shared) || !fp8_shape_ok(sh_up_payload, k_shared)))
+    return fail_arg(std::string(who) + ": shared payloads must be 16B-aligned with k % 16 == 0");
+  if (act_stride < n_routed || act_stride < n_shared) return fail_arg(std::string(who) + ": act_stride below n");
+  SlotArgs a = slot_args(x, x_stride, ids, order, views, act, act_stride, slots, top_k, limit);
+  a.n = n_routed;
+  a.k = k_routed;
+  a.want_shared = 0;
+  rc = finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who);
+  if (rc != DGPP_OK || n_shared == 0) return rc;
+  a.n = n_shared;
+  a.k = k_shared;
+  a.want_shared = 1;
+  a.sh[0] = fp8_mat(sh_gate_payload, sh_gate_scales, sh_rs, sh_cs);
+  a.sh[1] = fp8_mat(sh_up_payload, sh_up_scales, sh_rs, sh_cs);
+  return finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who);
+}
+
+int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                              const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared, int k_shared,
+                              const uint8_t* sh_payload, const float* sh_scales, float* out, int out_stride, int slots,
+                              int top_k, void* stream, int sh_rs, int sh_cs) {
+  const char* who = "moe_slot_down";
+  if (slots <= 0) return DGPP_OK;
+  int rc = check_slot_common(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, who);
+  if (rc != DGPP_OK) return rc;
+  if (k_routed % 16 != 0 || stage_bytes(1, k_routed) > kMaxLdsBytes)
+    return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
+  if (n_shared > 0 && (!sh_payload || !sh_scales || !fp8_shape_ok(sh_payload, k_shared)))
+    return fail_arg(std::string(who) + ": shared payload must be 16B-aligned with k % 16 == 0");
+  if (out_stride < n_routed || out_stride < n_shared) return fail_arg(std::string(who) + ": out_stride below n");
+  SlotArgs a = slot_args(act, act_stride, ids, order, views, out, out_stride, slots, top_k, 0.f);
+  a.n = n_routed;
+  a.k = k_routed;
+  a.want_shared = 0;
+  rc = finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
+  if (rc != DGPP_OK || n_shared == 0) return rc;
+  a.n = n_shared;
+  a.k = k_shared;
+  a.want_shared = 1;
+  a.sh[0] = fp8_mat(sh_payload, sh_scales, sh_rs, sh_cs);
+  return finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
+}
+
+int dgpp_launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                            const int32_t* order, const DgppMoeExpertView* views, int n_routed,
+                                            int k_routed, int n_shared, int k_shared, const uint8_t* sh_gate_payload,
+                                            const float* sh_gate_scales, const uint8_t* sh_up_payload,
+                                            const float* sh_up_scales, uint16_t* act, int act_stride, int slots,
+                                            int top_k, float limit, void* stream, int shared_view_base, int fp4_group,
+                                            int sh_rs, int sh_cs) {
+  const char* who = "moe_slot_gate_up_fp4";
+  if (slots <= 0) return DGPP_OK;
+  int rc = check_fp4_slot(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
+  if (rc != DGPP_OK) return rc;
+  const bool shared_fp4 = shared_view_base >= 0;
+  if (n_shared > 0 && !shared_fp4 &&
+      (!sh_gate_payload || !sh_gate_scales || !sh_up_payload || !sh_up_scales ||
+       !fp8_shape_ok(sh_gate_payload, k_shared) || !fp8_shape_ok(sh_up_payload, k_shared)))
+    return fail_arg(std::string(who) + ": shared payloads must be 16B-aligned with k % 16 == 0");
+  if (act_stride < n_routed || act_stride < n_shared) return fail_arg(std::string(who) + ": act_stride below n");
+  const int fmt = fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4;
+  SlotArgs a = slot_args(x, x_stride, ids, order, views, act, act_stride, slots, top_k, limit);
+  a.n = n_routed;
+  a.k = k_routed;
+  a.want_shared = 0;
+  rc = finish(launch_slot_gate_up(fmt, a, as_stream(stream)), who);
+  if (rc != DGPP_OK || n_shared == 0) return rc;
+  a.n = n_shared;
+  a.k = k_shared;
+  a.want_shared = 1;
+  if (shared_fp4) {
+    a.shared_view_base = shared_view_base;
+    return finish(launch_slot_gate_up(fmt, a, as_stream(stream)), who);
+  }
+  a.sh[0] = fp8_mat(sh_gate_payload, sh_gate_scales, sh_rs, sh_cs);
+  a.sh[1] = fp8_mat(sh_up_payload, sh_up_scales, sh_rs, sh_cs);
+  return finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who);
+}
+
+int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                  const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                  int k_shared, const uint8_t* sh_payload, const float* sh_scales, float* out,
+                                  int out_stride, int slots, int top_k, void* stream, int shared_view_base,
+                                  int fp4_group, int sh_rs, int sh_cs, int* tile_counter) {
+  const char* who = "moe_slot_down_fp4";
+  if (slots <= 0) return DGPP_OK;
+  if (tile_counter == nullptr) return fail_arg(std::string(who) + ": the stealing counter pair is required");
+  int rc = check_fp4_slot(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
+  if (rc != DGPP_OK) return rc;
+  const bool shared_fp4 = shared_view_base >= 0;
+  if (n_shared > 0 && !shared_fp4 && (!sh_payload || !sh_scales || !fp8_shape_ok(sh_payload, k_shared)))
+    return fail_arg(std::string(who) + ": shared payload must be 16B-aligned with k % 16 == 0");
+  if (out_stride < n_routed || out_stride < n_shared) return fail_arg(std::string(who) + ": out_stride below n");
+  const int fmt = fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4;
+  SlotArgs a = slot_args(act, act_stride, ids, order, views, out, out_stride, slots, top_k, 0.f);
+  a.n = n_routed;
+  a.k = k_routed;
+  a.want_shared = 0;
+  rc = finish(launch_slot_down(fmt, a, as_stream(stream)), who);
+  if (rc != DGPP_OK || n_shared == 0) return rc;
+  a.n = n_shared;
+  a.k = k_shared;
+  a.want_shared = 1;
+  if (shared_fp4) {
+    a.shared_view_base = shared_view_base;
+    return finish(launch_slot_down(fmt, a, as_stream(stream)), who);
+  }
+  a.sh[0] = fp8_mat(sh_payload, sh_scales, sh_rs, sh_cs);
+  return finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
+}
+
+static int grouped_fp8(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
+                       int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
+                       size_t out_stride, int n, int k, void* stream) {
+  // src/kernels/glm_moe.cu:1062-1090
+  const char* who = "moe grouped gemv";
+  if (n_segs <= 0 || n <= 0) return DGPP_OK;
+  if (!act || !segs || !views || !out) return fail_arg(std::string(who) + ": null pointer");
+  if (k <= 0 || k % 16 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 16");
+  if (stage_bytes(1, k) > kMaxLdsBytes) return fail_arg(std::string(who) + ": k exceeds the smem budget");
+  return grouped(kFmtFp8F32, act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_f32,
+                 out_stride, n, k, stream, who);
+}
+int dgpp_launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                      int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                      uint16_t* out, size_t out_stride, int n, int k, void* stream) {
+  return grouped_fp8(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 0, out_stride, n, k, stream);
+}
+int dgpp_launch_moe_grouped_gemv_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                     int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                     float* out, size_t out_stride, int n, int k, void* stream) {
+  return grouped_fp8(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 1, out_stride, n, k, stream);
+}
+
+static int grouped_fp4(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
+                       int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
+                       size_t out_stride, int n, int k, void* stream, int fp4_group) {
+  // src/kernels/glm_moe.cu:2231-2266
+  const char* who = "moe grouped gemv fp4";
+  if (n_segs <= 0 || n <= 0) return DGPP_OK;
+  if (!act || !segs || !views || !out) return fail_arg(std::string(who) + ": null pointer");
+  if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
+  if (!fp4_k_supported(k) || !fp4_k_compiled(k, fp4_group))
+    return fail_arg(std::string(who) + ": k must be a multiple of 32 in the fp4 core's compiled set");
+  return grouped(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
+                 which, out, out_f32, out_stride, n, k, stream, who);
+}
+int dgpp_launch_moe_grouped_gemv_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs,
+                                          int n_segs, int max_rows, int rows_per_block, const DgppMoeExpertView* views,
+                                          int which, uint16_t* out, size_t out_stride, int n, int k, void* stream,
+                                          int fp4_group) {
+  return grouped_fp4(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 0, out_stride, n, k,
+                     stream, fp4_group);
+}
+int dgpp_launch_moe_grouped_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                         int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                         float* out, size_t out_stride, int n, int k, void* stream, int fp4_group) {
+  return grouped_fp4(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 1, out_stride, n, k,
+                     stream, fp4_group);
+}
+
+int dgpp_launch_fp4_gemv_bf16(const uint16_t* act, size_t act_row_stride_elems, const DgppFp4Matrix* w, uint16_t* out,
+                              int m, int n, int k, void* stream) {
+  return fp4_gemv(act, act_row_stride_elems, w, out, 0, m, n, k, stream);
+}
+int dgpp_launch_fp4_gemv_f32(const uint16_t* act, size_t act_row_stride_elems, const DgppFp4Matrix* w, float* out,
+                             int m, int n, int k, void* stream) {
+  return fp4_gemv(act, act_row_stride_elems, w, out, 1, m, n, k, stream);
+}
+int dgpp_fp4_gemv_accepts(const DgppFp4Matrix* w) {
+  // src/kernels/fp4_gemv.cu:97-102
+  return w && w->payload && w->scales && (w->scale_group == 32 || w->global_scale) && w->cols > 0 && w->cols <= 16384 &&
+                 fp4_k_supported(static_cast<int>(w->cols)) && aligned16(w->payload) &&
+                 (w->scale_group == 16 || w->scale_group == 32) &&
+                 fp4_k_compiled(static_cast<int>(w->cols), w->scale_group)
+             ? 1
+             : 0;
+}
+
+int dgpp_launch_scale_gemm_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                const float* w_scales, uint16_t* out, int m, int n, int k, void* stream,
+                                size_t out_row_stride_elems, int mma_from_rows, void* ws, size_t ws_bytes) {
+  (void)mma_from_rows; (void)ws; (void)ws_bytes;
+  return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 0, m, n, k, stream, out_row_stride_elems, 7,
+                    7, 0, -1, false, "scale_gemm");
+}
+int dgpp_launch_scale_gemm_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                               const float* w_scales, float* out, int m, int n, int k, void* stream,
+                               size_t out_row_stride_elems, int mma_from_rows, int last_row_only, void* ws,
+                               size_t ws_bytes, int compact_row) {
+  (void)mma_from_rows; (void)ws; (void)ws_bytes;
+  return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 1, m, n, k, stream, out_row_stride_elems, 7,
+                    7, last_row_only, compact_row, false, "scale_gemm");
+}
+int dgpp_launch_scale_gemm_grid_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                     const float* w_scales, uint16_t* out, int m, int n, int k, void* stream,
+                                     size_t out_row_stride_elems, int rs, int cs, int decode_mma, void* ws,
+                                     size_t ws_bytes, int prefill_tile) {
+  (void)decode_mma; (void)ws; (void)ws_bytes; (void)prefill_tile;
+  return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 0, m, n, k, stream, out_row_stride_elems, rs,
+                    cs, 0, -1, true, "scale_gemm_grid");
+}
+int dgpp_launch_scale_gemm_grid_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                    const float* w_scales, float* out, int m, int n, int k, void* stream,
+                                    size_t out_row_stride_elems, int rs, int cs, int decode_mma, void* ws,
+                                    size_t ws_bytes, int prefill_tile) {
+  (void)decode_mma; (void)ws; (void)ws_bytes; (void)prefill_tile;
+  return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 1, m, n, k, stream, out_row_stride_elems, rs,
+                    cs, 0, -1, true, "scale_gemm_grid");
+}
+int dgpp_launch_scale_gemm_grid_e8m0_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                          const uint8_t* w_scales, uint16_t* out, int m, int n, int k, void* stream,
+                                          size_t out_row_stride_elems, int rs, int cs, void* ws, size_t ws_bytes,
+                                          int prefill_tile) {
+  (void)ws; (void)ws_bytes; (void)prefill_tile;
+  return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 1, out, 0, m, n, k, stream, out_row_stride_elems, rs,
+                    cs, 0, -1, true, "scale_gemm_grid_e8m0");
+}
+int dgpp_launch_scale_gemm_grid_e8m0_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                         const uint8_t* w_scales, float* out, int m, int n, int k, void* stream,
+                                         size_t out_row_stride_elems, int rs, int cs, void* ws, size_t ws_bytes,
+                                         int prefill_tile) {
+  (void)ws; (void)ws_bytes; (void)prefill_tile;
+  return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 1, out, 1, m, n, k, stream, out_row_stride_elems, rs,
+                    cs, 0, -1, true, "scale_gemm_grid_e8m0");
+}
+
+int dgpp_launch_scale_gemv_multi_bf16(const DgppFp8GemvProblem* problems, int n_problems, const uint16_t* act,
+                                      size_t act_row_stride_elems, int rows, int k, void* stream) {
+  // src/kernels/scale_gemm.cu:625-672: each problem's output is bitwise the single launcher's.
+  const char* who = "scale_gemv_multi";
+  if (n_problems <= 0 || rows <= 0) return DGPP_OK;
+  if (!problems || !act) return fail_arg(std::string(who) + ": null pointer");
+  if (n_problems > 4) return fail_arg(std::string(who) + ": at most four problems");
+  if (rows > kMaxActRows) return fail_arg(std::string(who) + ": at most eight rows");
+  for (int i = 0; i < n_problems; ++i) {
+    const DgppFp8GemvProblem& p = problems[i];
+    if (p.bf16_weight) return fail_arg(std::string(who) + ": bf16 problems are outside this library's path");
+    if (!p.payload || !p.scales || !p.out || p.n <= 0) return fail_arg(std::string(who) + ": null pointer");
+    if (!fp8_shape_ok(p.payload, k)) return fail_arg(std::string(who) + ": k must be a multiple of 16 with aligned payloads");
+  }
+  for (int i = 0; i < n_problems; ++i) {
+    const DgppFp8GemvProblem& p = problems[i];
+    const int rc = scale_gemm(act, act_row_stride_elems, p.payload, p.scales, 0, p.out, 0, rows, p.n, k, stream,
+                              p.out_stride, p.rs, p.cs, 0, -1, false, who);
+    if (rc != DGPP_OK) return rc;
+  }
+  return DGPP_OK;
+}
+
+int dgpp_fp8_gemv_can_stage(const void* w_payload, int k) { return fp8_shape_ok(w_payload, k) ? 1 : 0; }
+
+static int fp8_dequant(const uint8_t* payload, const void* scales, int e8m0, uint16_t* out, int64_t rows, int64_t cols,
+                       void* stream, int rs, int cs) {
+  // src/kernels/fp8_dequant.cu:52-72
+  if (rows <= 0 || cols <= 0) return fail_arg("fp8_dequant: rows and cols must be positive");
+  if (!payload || !scales || !out) return fail_arg("fp8_dequant: null pointer");
+  if (rs < 0 || cs < 4 || rs > 30 || cs > 30) return fail_arg("fp8_dequant: rs must be non-negative, cs >= 4");
+  if ((rows * cols + 255) / 256 > 2147483647LL) {
+    g_last_error = "fp8_dequant: grid too large";
+    return DGPP_RUNTIME_ERROR;
+  }
+  return finish(run_fp8_dequant(payload, scales, e8m0, out, rows, cols, rs, cs, as_stream(stream)), "fp8_dequant");
+}
+int dgpp_launch_fp8_dequant_blocks(const uint8_t* payload, const float* scales, uint16_t* out_bf16, int64_t rows,
+                                   int64_t cols, void* stream, int rs, int cs) {
+  return fp8_dequant(payload, scales, 0, out_bf16, rows, cols, stream, rs, cs);
+}
+int dgpp_launch_fp8_dequant_blocks_e8m0(const uint8_t* payload, const uint8_t* scales, uint16_t* out_bf16, int64_t rows,
+                                        int64_t cols, void* stream, int rs, int cs) {
+  return fp8_dequant(payload, scales, 1, out_bf16, rows, cols, stream, rs, cs);
+}
+
+}  // extern "C"

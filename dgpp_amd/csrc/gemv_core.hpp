@@ -1,0 +1,388 @@
+// The weight-streaming GEMV core for gfx950 (wave64), shared by the dense projection
+// launchers, the MoE decode-slot kernels and the grouped (segment-major) kernels.
+//
+// Shape of the computation. A weight row is a string of 16-byte CHUNKS (16 FP8 codes or
+// 32 FP4 codes). A row is covered by L = 2^l2 adjacent lanes (L <= 64); lane li of the row
+// owns chunks li, li + L, li + 2L, ... (P of them), so one load instruction of a row group
+// reads L consecutive chunks: fully coalesced 16-byte-per-lane global loads. A wavefront
+// carries 64 / L rows per step. Each lane decodes its chunks in registers to packed bf16
+// pairs (hardware FP4 / FP8 conversions of gfx950), multiplies them with the activation
+// vector staged in LDS through v_dot2_f32_bf16 (fp32 accumulate), and the L partial sums of
+// a row are folded by a fixed DPP / lane-permute butterfly. (row, activation-row) results
+// therefore depend only on (format, k): never on how many activation rows share the launch,
+// on the launcher, or on the grid — the property the slot / grouped / dense launchers'
+// bitwise-twin tests pin.
+//
+// Value semantics (reference: src/kernels/fp8_gemv.cuh:64-66, src/kernels/fp4_gemv.cuh:20-27):
+//   FP8 + F32 grid   w = bf16_rne(float(e4m3) * scale)               (the rounding is part of the value)
+//   FP8 + E8M0 grid  w = e4m3 * 2^(b-127), b == 0 -> 2^-127          (exact in bf16)
+//   NVFP4            w = e2m1 * e4m3(scale) exact; dot / global once  (we sum a 16-group unscaled,
+//                    then fold the group scale in with one fma: same sum, fp32 rounding order only)
+//   MXFP4            w = e2m1 * 2^(b-127) exact, b == 255 -> NaN
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "numerics.hpp"
+
+namespace dgpp_amd {
+
+enum : int { kFmtFp8F32 = 0, kFmtFp8E8M0 = 1, kFmtNvfp4 = 2, kFmtMxfp4 = 3 };
+
+constexpr int kWave = 64;
+constexpr int kBlockThreads = 256;
+constexpr int kWavesPerBlock = kBlockThreads / kWave;
+constexpr int kChunkBytes = 16;
+constexpr int kMaxActRows = 8;                 // activation rows one launch carries
+constexpr size_t kDefaultLdsBytes = 64 * 1024;  // dynamic LDS a block may take without opt-in
+constexpr size_t kMaxLdsBytes = 160 * 1024;     // LDS of one gfx950 CU: the ceiling after opt-in
+
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+
+template <int FMT>
+struct FmtTraits {
+  static constexpr bool kIsFp4 = FMT >= kFmtNvfp4;
+  static constexpr int kElemsPerChunk = kIsFp4 ? 32 : 16;
+  static constexpr int kPieces = kElemsPerChunk / 8;  // 16-byte activation vectors per chunk
+};
+
+// One weight matrix as the core reads it.
+struct MatRef {
+  const uint8_t* payload;   // [n, row_bytes]
+  const void* scales;       // FP8: float or e8m0 grid; FP4: per-row scale bytes
+  float divisor;            // NVFP4: the device global (dot divided by it); else unused
+  int rs, cs;               // FP8 scale grid log2 block sizes
+};
+
+// Row geometry as a function of the chunk count of a row.
+struct RowGeom {
+  int l2;      // log2 lanes per row
+  int P;       // chunks per lane
+  int nb;      // chunks per pass (a divisor of P, <= 8): the loads in flight per lane per row
+};
+__host__ __device__ inline RowGeom row_geom(int chunks) {
+  RowGeom g;
+  g.l2 = 0;
+  while (g.l2 < 6 && (chunks % (2 << g.l2)) == 0) ++g.l2;
+  g.P = chunks >> g.l2;
+  // Prefer four chunks per lane over very wide row groups: more bytes in flight per lane,
+  // and a row group keeps at least 128 contiguous bytes per load instruction (8 lanes).
+  while (g.P < 4 && g.l2 > 3) {
+    --g.l2;
+    g.P *= 2;
+  }
+  g.nb = 1;
+  for (int d = 8; d >= 1; --d)
+    if (d != 7 && g.P % d == 0) {
+      g.nb = d;
+      break;
+    }
+  return g;
+}
+
+// ---- activation staging -----------------------------------------------------------------
+// LDS layout: 16-byte vectors indexed [(r * kPieces + q) * chunks + c] for activation row r,
+// chunk c, piece q (elements 8q .. 8q+7 of the chunk). Lanes of a row group read consecutive
+// c for a fixed q: consecutive 16-byte vectors, bank-conflict free.
+template <int FMT>
+__device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x, size_t x_stride,
+                                                  int rows, int k, uint4* __restrict__ lds) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+  const int chunks = k / FmtTraits<FMT>::kElemsPerChunk;
+  const int vecs = k / 8;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && ((x_stride & 7u) == 0);
+  if (aligned) {
+    for (int i = threadIdx.x; i < rows * vecs; i += blockDim.x) {
+      const int r = i / vecs, v = i - r * vecs;
+      const int c = v / kPieces, q = v - c * kPieces;
+      lds[(r * kPieces + q) * chunks + c] =
+          *reinterpret_cast<const uint4*>(x + static_cast<size_t>(r) * x_stride + static_cast<size_t>(v) * 8);
+    }
+  } else {
+    uint16_t* l16 = reinterpret_cast<uint16_t*>(lds);
+    for (int i = threadIdx.x; i < rows * k; i += blockDim.x) {
+      const int r = i / k, e = i - r * k;
+      const int v = e >> 3, c = v / kPieces, q = v - c * kPieces;
+      l16[(static_cast<size_t>((r * kPieces + q) * chunks + c) << 3) + (e & 7)] =
+          x[static_cast<size_t>(r) * x_stride + e];
+    }
+  }
+}
+
+// ---- lane butterflies ---------------------------------------------------------------------
+template <int kCtrl>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xF, 0xF, true));
+}
+// Sum over the 2^l2 adjacent lanes of a row group; every lane of the group gets the sum.
+// Fixed order: distances 1, 2 (quad permutes), 4, 8 (half-row / row mirrors: after the
+// earlier steps every lane of a quad / octet already holds the same partial, so a mirror
+// pairs the same partials as an xor would), then 16 and 32 by lane permutes.
+__device__ __forceinline__ float group_sum(float v, int l2) {
+  if (l2 >= 1) v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+  if (l2 >= 2) v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+  if (l2 >= 3) v += dpp_move<0x141>(v);  // row_half_mirror
+  if (l2 >= 4) v += dpp_move<0x140>(v);  // row_mirror
+  if (l2 >= 5) v += __shfl_xor(v, 16);
+  if (l2 >= 6) v += __shfl_xor(v, 32);
+  return v;
+}
+
+// ---- per-chunk arithmetic -------------------------------------------------------------------
+__device__ __forceinline__ float dot2(bf16x2_t w, uint32_t xpair, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(w, __builtin_bit_cast(bf16x2_t, xpair), acc, false);
+}
+__device__ __forceinline__ bf16x2_t pack_bf16(float a, float b) {
+  f32x2_t v = {a, b};
+  return __builtin_convertvector(v, bf16x2_t);
+}
+
+// The raw bytes a lane holds for one chunk: 16 payload bytes and its scale word.
+struct ChunkRegs {
+  uint4 w;
+  uint32_t s;  // FP8-F32: float bits; FP8-E8M0 / MXFP4: the byte; NVFP4: two e4m3 bytes
+};
+
+// Issues the loads of chunk index c of the row whose payload / scale rows are given.
+template <int FMT>
+__device__ __forceinline__ void load_chunk(const uint8_t* __restrict__ payload_row,
+                                           const void* __restrict__ scale_row, int c, int cs,
+                                           ChunkRegs& out) {
+  out.w = *reinterpret_cast<const uint4*>(payload_row + static_cast<size_t>(c) * kChunkBytes);
+  if constexpr (FMT == kFmtFp8F32) {
+    out.s = reinterpret_cast<const uint32_t*>(scale_row)[(c * 16) >> cs];
+  } else if constexpr (FMT == kFmtFp8E8M0) {
+    out.s = reinterpret_cast<const uint8_t*>(scale_row)[(c * 16) >> cs];
+  } else if constexpr (FMT == kFmtNvfp4) {
+    out.s = reinterpret_cast<const uint16_t*>(scale_row)[c];
+  } else {
+    out.s = reinterpret_cast<const uint8_t*>(scale_row)[c];
+  }
+}
+
+// acc[r] += dot(chunk weights, activation row r's elements of chunk c) for r < m.
+// xl points at LDS vector [piece 0][chunk c] of activation row 0.
+template <int FMT, int MAXR>
+__device__ __forceinline__ void consume_chunk(const ChunkRegs& ch, const uint4* __restrict__ xl,
+                                              int chunks, int m, float (&acc)[MAXR]) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+  const uint32_t w[4] = {ch.w.x, ch.w.y, ch.w.z, ch.w.w};
+  if constexpr (FMT == kFmtMxfp4) {
+    if (ch.s >= 2u && ch.s <= 252u) {
+      // e2m1 * 2^(b-127) is a normal bf16 for every code: the scaled conversion is exact.
+      const float s = bits_f32(ch.s << 23);
+      bf16x2_t p[16];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        p[q * 4 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 0);
+        p[q * 4 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 1);
+        p[q * 4 + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 2);
+        p[q * 4 + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 3);
+      }
+#pragma unroll
+      for (int r = 0; r < MAXR; ++r) {
+        if (r < m) {
+          float a = acc[r];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint4 xv = xl[(r * kPieces + q) * chunks];
+            a = dot2(p[q * 4 + 0], xv.x, a);
+            a = dot2(p[q * 4 + 1], xv.y, a);
+            a = dot2(p[q * 4 + 2], xv.z, a);
+            a = dot2(p[q * 4 + 3], xv.w, a);
+          }
+          acc[r] = a;
+        }
+      }
+    } else {
+      // Scale bytes at the ends of the range (2^-127, 2^-126, >= 2^126, NaN): exact fp32 path.
+      const float s = e8m0_to_f32(static_cast<uint8_t>(ch.s));
+#pragma unroll
+      for (int r = 0; r < MAXR; ++r) {
+        if (r < m) {
+          float a = acc[r];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint4 xv = xl[(r * kPieces + q) * chunks];
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const uint32_t byte = (w[q] >> (8 * j)) & 0xFFu;
+              a = fmaf(e2m1_to_f32(byte & 0xFu) * s, bits_f32(xw[j] << 16), a);
+              a = fmaf(e2m1_to_f32(byte >> 4) * s, bits_f32(xw[j] & 0xFFFF0000u), a);
+            }
+          }
+          acc[r] = a;
+        }
+      }
+    }
+  } else if constexpr (FMT == kFmtNvfp4) {
+    bf16x2_t p[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      p[q * 4 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 0);
+      p[q * 4 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 1);
+      p[q * 4 + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 2);
+      p[q * 4 + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 3);
+    }
+    // The two e4m3 group scales of the chunk (codes 0..15 and 16..31), NaN codes propagate.
+    const float s0 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 0);
+    const float s1 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 1);
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      if (r < m) {
+        float a = acc[r];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          float part = 0.f;
+#pragma unroll
+          for (int q = 2 * h; q < 2 * h + 2; ++q) {
+            const uint4 xv = xl[(r * kPieces + q) * chunks];
+            part = dot2(p[q * 4 + 0], xv.x, part);
+            part = dot2(p[q * 4 + 1], xv.y, part);
+            part = dot2(p[q * 4 + 2], xv.z, part);
+            part = dot2(p[q * 4 + 3], xv.w, part);
+          }
+          a = fmaf(part, h == 0 ? s0 : s1, a);
+        }
+        acc[r] = a;
+      }
+    }
+  } else {
+    // FP8: 16 codes -> 8 packed bf16 pairs.
+    bf16x2_t p[8];
+    bool fast = true;
+    if constexpr (FMT == kFmtFp8E8M0) fast = ch.s >= 10u && ch.s <= 245u;
+    if constexpr (FMT == kFmtFp8E8M0) {
+      if (fast) {
+        const float s = bits_f32(ch.s << 23);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          p[q * 2 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], s, false);
+          p[q * 2 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], s, true);
+        }
+      }
+    }
+    if (FMT == kFmtFp8F32 || !fast) {
+      // float(e4m3) * scale in fp32, one RNE rounding to bf16. The E8M0 bridge reads byte b
+      // as the float with exponent field b (0 -> 2^-127), src/kernels/fp8_dequant.cu:28-31.
+      const float s = FMT == kFmtFp8F32 ? bits_f32(ch.s) : (ch.s ? bits_f32(ch.s << 23) : bits_f32(0x00400000u));
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[q], false);
+        const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[q], true);
+        p[q * 2 + 0] = pack_bf16(lo.x * s, lo.y * s);
+        p[q * 2 + 1] = pack_bf16(hi.x * s, hi.y * s);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < MAXR; ++r) {
+      if (r < m) {
+        float a = acc[r];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const uint4 xv = xl[(r * kPieces + q) * chunks];
+          a = dot2(p[q * 4 + 0], xv.x, a);
+          a = dot2(p[q * 4 + 1], xv.y, a);
+          a = dot2(p[q * 4 + 2], xv.z, a);
+          a = dot2(p[q * 4 + 3], xv.w, a);
+        }
+        acc[r] = a;
+      }
+    }
+  }
+}
+
+// ---- a wavefront's row step --------------------------------------------------------------------
+// Per-lane addressing of one row step: which row this lane helps with and where its chunks start.
+struct LaneRow {
+  const uint8_t* payload_row;
+  const void* scale_row;
+  int row;       // absolute row (may be >= n: the lane then works on row n-1 and its result is dropped)
+  int li;        // lane index inside the row group
+};
+
+template <int FMT>
+__device__ __forceinline__ LaneRow lane_row(const MatRef& mat, int row0, int n, int k, int l2) {
+  const int lane = threadIdx.x & (kWave - 1);
+  LaneRow lr;
+  lr.li = lane & ((1 << l2) - 1);
+  lr.row = row0 + (lane >> l2);
+  const int r = lr.row < n ? lr.row : n - 1;
+  if constexpr (FMT == kFmtFp8F32 || FMT == kFmtFp8E8M0) {
+    lr.payload_row = mat.payload + static_cast<size_t>(r) * k;
+    const size_t scale_cols = (static_cast<size_t>(k) + (1u << mat.cs) - 1) >> mat.cs;
+    const size_t esz = FMT == kFmtFp8F32 ? 4 : 1;
+    lr.scale_row = reinterpret_cast<const uint8_t*>(mat.scales) + (static_cast<size_t>(r >> mat.rs) * scale_cols) * esz;
+  } else {
+    lr.payload_row = mat.payload + static_cast<size_t>(r) * (k / 2);
+    lr.scale_row = reinterpret_cast<const uint8_t*>(mat.scales) +
+                   static_cast<size_t>(r) * (k / (FMT == kFmtNvfp4 ? 16 : 32));
+  }
+  return lr;
+}
+
+// Loads one pass (NB chunks) of a row for this lane.
+template <int FMT, int NB>
+__device__ __forceinline__ void issue_pass(const LaneRow& lr, int pass, int l2, int cs,
+                                           ChunkRegs (&regs)[NB]) {
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+    load_chunk<FMT>(lr.payload_row, lr.scale_row, ((pass * NB + i) << l2) + lr.li, cs, regs[i]);
+}
+
+template <int FMT, int MAXR, int NB>
+__device__ __forceinline__ void consume_pass(const ChunkRegs (&regs)[NB], const LaneRow& lr, int pass,
+                                             int l2, const uint4* __restrict__ lds, int chunks, int m,
+                                             float (&acc)[MAXR]) {
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int c = ((pass * NB + i) << l2) + lr.li;
+    consume_chunk<FMT, MAXR>(regs[i], lds + c, chunks, m, acc);
+  }
+}
+
+// Full dot products of this lane's row against m staged activation rows; after the call every
+// lane of the row group holds the finished sums (the NVFP4 division is the caller's epilogue).
+template <int FMT, int MAXR, int NB>
+__device__ __forceinline__ void row_dots(const LaneRow& lr, const RowGeom& g, int cs,
+                                         const uint4* __restrict__ lds, int chunks, int m,
+                                         float (&acc)[MAXR]) {
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) acc[r] = 0.f;
+  const int passes = g.P / NB;
+  ChunkRegs cur[NB];
+  issue_pass<FMT, NB>(lr, 0, g.l2, cs, cur);
+  for (int p = 0; p < passes; ++p) {
+    ChunkRegs nxt[NB];
+    if (p + 1 < passes) issue_pass<FMT, NB>(lr, p + 1, g.l2, cs, nxt);
+    consume_pass<FMT, MAXR, NB>(cur, lr, p, g.l2, lds, chunks, m, acc);
+    if (p + 1 < passes) {
+#pragma unroll
+      for (int i = 0; i < NB; ++i) cur[i] = nxt[i];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r)
+    if (r < m) acc[r] = group_sum(acc[r], g.l2);
+}
+
+// Dispatches a callable on the compile-time pass width.
+template <class F>
+inline void dispatch_nb(int nb, F&& f) {
+  switch (nb) {
+    case 8: f(std::integral_constant<int, 8>{}); break;
+    case 6: f(std::integral_constant<int, 6>{}); break;
+    case 5: f(std::integral_constant<int, 5>{}); break;
+    case 4: f(std::integral_constant<int, 4>{}); break;
+    case 3: f(std::integral_constant<int, 3>{}); break;
+    case 2: f(std::integral_constant<int, 2>{}); break;
+    default: f(std::integral_constant<int, 1>{}); break;
+  }
+}
+
+}  // namespace dgpp_amd

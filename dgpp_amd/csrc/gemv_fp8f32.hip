@@ -1,0 +1,10 @@
+// Instantiates the GEMV-core kernels for one weight format (kFmtFp8F32).
+#define DGPP_GEMV_IMPL
+#include "gemv_kernels.hpp"
+
+namespace dgpp_amd {
+template hipError_t launch_dense_fmt<kFmtFp8F32>(const DenseArgs&, hipStream_t);
+template hipError_t launch_slot_gate_up_fmt<kFmtFp8F32>(const SlotArgs&, hipStream_t);
+template hipError_t launch_slot_down_fmt<kFmtFp8F32>(const SlotArgs&, hipStream_t);
+template hipError_t launch_grouped_fmt<kFmtFp8F32>(const GroupedArgs&, int, int, hipStream_t);
+}  // namespace dgpp_amd

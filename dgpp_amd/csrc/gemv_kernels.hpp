@@ -1,0 +1,382 @@
+// Kernels built on the GEMV core: the dense projection, the MoE decode-slot kernels (fused
+// gate/up + SwiGLU, down) and the grouped (segment-major) twin. One template per kernel,
+// instantiated per weight format in gemv_fp8.hip / gemv_fp4.hip.
+//
+// Reference counterparts: src/kernels/fp4_gemv.cu:16-95, src/kernels/scale_gemm.cu:168-197,
+// src/kernels/glm_moe.cu:572-667 (FP8 slot kernels), :1863-1953 and :2061-2144 (FP4 slot kernels),
+// :999-1059 and :2149-2195 (grouped kernels).
+#pragma once
+
+#include <type_traits>
+
+#include "../../include/dgpp_amd.h"
+#include "gemv_core.hpp"
+
+namespace dgpp_amd {
+
+// ---- epilogues ------------------------------------------------------------------------------
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// SwiGLU on the bf16-rounded dots with the reference's rounding points
+// (src/kernels/glm_moe.cu:659-666): gate clamped above only, up on both sides.
+__device__ __forceinline__ uint16_t swiglu_bf16(float gate_dot, float up_dot, float limit) {
+  float g = bf16_to_f32(f32_to_bf16(gate_dot));
+  float u = bf16_to_f32(f32_to_bf16(up_dot));
+  if (g > limit) g = limit;
+  u = fminf(fmaxf(u, -limit), limit);
+  const uint16_t t = f32_to_bf16(g * sigmoid_f32(g));
+  return f32_to_bf16(bf16_to_f32(t) * u);
+}
+
+template <int FMT>
+__device__ __forceinline__ float finish_dot(float acc, float divisor) {
+  if constexpr (FMT == kFmtNvfp4) return acc / divisor;  // one correctly rounded division
+  return acc;
+}
+
+template <int FMT>
+__device__ __forceinline__ float load_divisor(const float* global) {
+  if constexpr (FMT == kFmtNvfp4) return *global;
+  return 1.0f;
+}
+
+// rows a block covers: waves x rows-per-wave x steps
+__host__ __device__ inline int block_rows(const RowGeom& g, int steps) {
+  return kWavesPerBlock * (kWave >> g.l2) * steps;
+}
+
+// ---- dense projection -------------------------------------------------------------------------
+struct DenseArgs {
+  const uint16_t* act;
+  size_t act_stride;
+  MatRef mat;
+  const float* global;   // NVFP4 device global
+  void* out;
+  size_t out_stride;
+  int out_f32;
+  int m, n, k;
+};
+
+template <int FMT, int MAXR, int NB>
+__global__ __launch_bounds__(kBlockThreads) void gemv_dense_kernel(DenseArgs a, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  stage_activations<FMT>(a.act, a.act_stride, a.m, a.k, lds);
+  __syncthreads();
+  const float divisor = load_divisor<FMT>(a.global);
+  const int rpw = kWave >> g.l2;
+  const int wave = threadIdx.x >> 6;
+  int row0 = blockIdx.x * block_rows(g, steps) + wave * rpw;
+  for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+    if (row0 >= a.n) break;
+    const LaneRow lr = lane_row<FMT>(a.mat, row0, a.n, a.k, g.l2);
+    float acc[MAXR];
+    row_dots<FMT, MAXR, NB>(lr, g, a.mat.cs, lds, chunks, a.m, acc);
+    if (lr.li == 0 && lr.row < a.n) {
+#pragma unroll
+      for (int r = 0; r < MAXR; ++r) {
+        if (r < a.m) {
+          const float v = finish_dot<FMT>(acc[r], divisor);
+          const size_t at = static_cast<size_t>(r) * a.out_stride + lr.row;
+          if (a.out_f32)
+            static_cast<float*>(a.out)[at] = v;
+          else
+            static_cast<uint16_t*>(a.out)[at] = f32_to_bf16(v);
+        }
+      }
+    }
+  }
+}
+
+// ---- MoE decode slots ----------------------------------------------------------------------------
+// Slot layout (src/kernels/glm_moe_launch.hpp:216-226): slot = t * (top_k + 1) + j, j < top_k the
+// token's j-th routed expert (ascending id), j == top_k the shared expert.
+struct SlotArgs {
+  const uint16_t* x;        // gate/up: token rows; down: slot activation rows
+  size_t x_stride;
+  const int32_t* ids;
+  const int32_t* order;     // nullable: blockIdx.y -> logical slot
+  const DgppMoeExpertView* views;
+  MatRef sh[2];             // shared expert matrices given as launch arguments (FP8)
+  void* out;                // gate/up: bf16 act [slots, out_stride]; down: f32 [slots, out_stride]
+  int out_stride;
+  int n, k;                 // the dims of the slots this launch computes
+  int slots, top_k;
+  float limit;
+  int want_shared;          // 0: routed slots, 1: shared slots (others exit)
+  int shared_view_base;     // >= 0: shared matrices come from views[base + which]
+};
+
+template <int FMT>
+__device__ __forceinline__ MatRef mat_of_view(const DgppMoeExpertView& v, const float** global) {
+  MatRef m;
+  m.payload = v.payload;
+  if constexpr (FMT == kFmtFp8F32) {
+    m.scales = v.scales;
+    m.rs = v.scale_shift_rows;
+    m.cs = v.scale_shift_cols;
+    *global = nullptr;
+  } else {
+    m.scales = v.fp4_scales;
+    m.rs = 0;
+    m.cs = 0;
+    *global = v.fp4_global;
+  }
+  m.divisor = 1.0f;
+  return m;
+}
+
+// Resolves the slot of this block; false when the block has nothing to do.
+__device__ __forceinline__ bool resolve_slot(const SlotArgs& a, int& slot, int& token, int& view_base) {
+  if (static_cast<int>(blockIdx.y) >= a.slots) return false;
+  slot = a.order ? a.order[blockIdx.y] : static_cast<int>(blockIdx.y);
+  token = slot / (a.top_k + 1);
+  const int j = slot - token * (a.top_k + 1);
+  const bool shared = j == a.top_k;
+  if (shared != (a.want_shared != 0)) return false;
+  view_base = shared ? a.shared_view_base : a.ids[static_cast<size_t>(token) * a.top_k + j] * 3;
+  return true;
+}
+
+template <int FMT, int NB>
+__global__ __launch_bounds__(kBlockThreads) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  int slot, token, base;
+  if (!resolve_slot(a, slot, token, base)) return;
+  const int rows_per_block = block_rows(g, steps);
+  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
+  MatRef mg, mu;
+  const float *gg = nullptr, *gu = nullptr;
+  if (base >= 0) {
+    mg = mat_of_view<FMT>(a.views[base + 0], &gg);
+    mu = mat_of_view<FMT>(a.views[base + 1], &gu);
+  } else {
+    mg = a.sh[0];
+    mu = a.sh[1];
+  }
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  stage_activations<FMT>(a.x + static_cast<size_t>(token) * a.x_stride, a.x_stride, 1, a.k, lds);
+  __syncthreads();
+  const float dg = load_divisor<FMT>(gg), du = load_divisor<FMT>(gu);
+  const int rpw = kWave >> g.l2;
+  const int wave = threadIdx.x >> 6;
+  uint16_t* act_row = static_cast<uint16_t*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
+  int row0 = blockIdx.x * rows_per_block + wave * rpw;
+  for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+    if (row0 >= a.n) break;
+    const LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
+    const LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
+    float ag[1], au[1];
+    row_dots<FMT, 1, NB>(lg, g, mg.cs, lds, chunks, 1, ag);
+    row_dots<FMT, 1, NB>(lu, g, mu.cs, lds, chunks, 1, au);
+    if (lg.li == 0 && lg.row < a.n)
+      act_row[lg.row] = swiglu_bf16(finish_dot<FMT>(ag[0], dg), finish_dot<FMT>(au[0], du), a.limit);
+  }
+}
+
+template <int FMT, int NB>
+__global__ __launch_bounds__(kBlockThreads) void slot_down_kernel(SlotArgs a, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  int slot, token, base;
+  if (!resolve_slot(a, slot, token, base)) return;
+  const int rows_per_block = block_rows(g, steps);
+  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
+  MatRef md;
+  const float* gd = nullptr;
+  if (base >= 0)
+    md = mat_of_view<FMT>(a.views[base + 2], &gd);
+  else
+    md = a.sh[0];
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  // The down projection consumes this slot's own activation row.
+  stage_activations<FMT>(a.x + static_cast<size_t>(slot) * a.x_stride, a.x_stride, 1, a.k, lds);
+  __syncthreads();
+  const float dd = load_divisor<FMT>(gd);
+  const int rpw = kWave >> g.l2;
+  const int wave = threadIdx.x >> 6;
+  float* out_row = static_cast<float*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
+  int row0 = blockIdx.x * rows_per_block + wave * rpw;
+  for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+    if (row0 >= a.n) break;
+    const LaneRow lr = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
+    float acc[1];
+    row_dots<FMT, 1, NB>(lr, g, md.cs, lds, chunks, 1, acc);
+    if (lr.li == 0 && lr.row < a.n) out_row[lr.row] = finish_dot<FMT>(acc[0], dd);
+  }
+}
+
+// ---- grouped (segment-major) twin ------------------------------------------------------------------
+struct GroupedArgs {
+  const uint16_t* act;
+  size_t act_stride;
+  const DgppMoeSegment* segs;
+  const DgppMoeExpertView* views;
+  int which;
+  void* out;
+  size_t out_stride;
+  int out_f32;
+  int n, k;
+  int rows_per_block;  // segment rows per z block
+  int group_rows;      // activation rows staged per pass (<= kMaxActRows)
+};
+
+template <int FMT, int NB>
+__global__ __launch_bounds__(kBlockThreads) void grouped_gemv_kernel(GroupedArgs a, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  const DgppMoeSegment seg = a.segs[blockIdx.y];
+  const int z0 = static_cast<int>(blockIdx.z) * a.rows_per_block;
+  if (z0 >= seg.rows) return;
+  const int z1 = min(seg.rows, z0 + a.rows_per_block);
+  const float* gp = nullptr;
+  const MatRef mat = mat_of_view<FMT>(a.views[seg.expert * 3 + a.which], &gp);
+  const float divisor = load_divisor<FMT>(gp);
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  const int rpw = kWave >> g.l2;
+  const int wave = threadIdx.x >> 6;
+  for (int g0 = z0; g0 < z1; g0 += a.group_rows) {
+    const int m = min(a.group_rows, z1 - g0);
+    if (g0 > z0) __syncthreads();  // the previous group is done reading the staged rows
+    stage_activations<FMT>(a.act + static_cast<size_t>(seg.row0 + g0) * a.act_stride, a.act_stride, m, a.k, lds);
+    __syncthreads();
+    int row0 = blockIdx.x * block_rows(g, steps) + wave * rpw;
+    for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+      if (row0 >= a.n) break;
+      const LaneRow lr = lane_row<FMT>(mat, row0, a.n, a.k, g.l2);
+      float acc[kMaxActRows];
+      row_dots<FMT, kMaxActRows, NB>(lr, g, mat.cs, lds, chunks, m, acc);
+      if (lr.li == 0 && lr.row < a.n) {
+#pragma unroll
+        for (int r = 0; r < kMaxActRows; ++r) {
+          if (r < m) {
+            const float v = finish_dot<FMT>(acc[r], divisor);
+            const size_t at = static_cast<size_t>(seg.row0 + g0 + r) * a.out_stride + lr.row;
+            if (a.out_f32)
+              static_cast<float*>(a.out)[at] = v;
+            else
+              static_cast<uint16_t*>(a.out)[at] = f32_to_bf16(v);
+          }
+        }
+      }
+    }
+  }
+}
+
+// ---- host launch helpers (defined per format in gemv_fp8.hip / gemv_fp4.hip) ---------------------------
+// Elements per chunk by format, and the LDS bytes `rows` staged activation rows take.
+inline int elems_per_chunk(int fmt) { return fmt >= kFmtNvfp4 ? 32 : 16; }
+inline size_t stage_bytes(int rows, int k) { return static_cast<size_t>(rows) * static_cast<size_t>(k) * 2; }
+
+// Row steps per block: enough blocks to fill the 256 CUs several times over while amortising
+// the activation staging of a block over more weight rows on large problems.
+inline int pick_steps(long long block_steps_total) {
+  long long s = (block_steps_total + 4095) / 4096;
+  if (s < 1) s = 1;
+  if (s > 8) s = 8;
+  return static_cast<int>(s);
+}
+
+hipError_t launch_dense(int fmt, const DenseArgs& a, hipStream_t stream);
+hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t stream);
+hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t stream);
+hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
+
+// Per-format implementations.
+template <int FMT> hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream);
+template <int FMT> hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream);
+template <int FMT> hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream);
+template <int FMT> hipError_t launch_grouped_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
+
+// Raises a kernel's dynamic LDS ceiling (once per kernel) when a launch needs more than the
+// default 64 KB; gfx950 offers 160 KB per workgroup.
+hipError_t ensure_lds_impl(const void* kernel, size_t bytes);
+template <class K>
+inline hipError_t ensure_lds(K kernel, size_t bytes) {
+  if (bytes <= kDefaultLdsBytes) return hipSuccess;
+  return ensure_lds_impl(reinterpret_cast<const void*>(kernel), bytes);
+}
+// Activation rows one launch may stage for a k-wide row (at most kMaxActRows).
+inline int max_stage_rows(int k) {
+  const size_t per_row = static_cast<size_t>(k) * 2;
+  const size_t fit = per_row ? kMaxLdsBytes / per_row : kMaxActRows;
+  return static_cast<int>(fit < 1 ? 1 : (fit > kMaxActRows ? kMaxActRows : fit));
+}
+
+// The bodies, included by the per-format translation units.
+#ifdef DGPP_GEMV_IMPL
+template <int FMT>
+hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
+  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
+  const long long block_steps = (a.n + rows_per_step - 1) / rows_per_step;
+  const int steps = pick_steps(block_steps);
+  const dim3 grid(static_cast<unsigned>((block_steps + steps - 1) / steps));
+  const size_t lds = stage_bytes(a.m, a.k);
+  hipError_t err = hipSuccess;
+  dispatch_nb(g.nb, [&](auto nbc) {
+    constexpr int NB = decltype(nbc)::value;
+    auto go = [&](auto rc) {
+      constexpr int MAXR = decltype(rc)::value;
+      auto kern = gemv_dense_kernel<FMT, MAXR, NB>;
+      err = ensure_lds(kern, lds);
+      if (err != hipSuccess) return;
+      hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
+    };
+    if (a.m == 1) go(std::integral_constant<int, 1>{});
+    else if (a.m == 2) go(std::integral_constant<int, 2>{});
+    else if (a.m <= 4) go(std::integral_constant<int, 4>{});
+    else go(std::integral_constant<int, 8>{});
+  });
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+template <int FMT>
+hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
+  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
+  const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
+  const int steps = pick_steps(per_slot * a.slots);
+  const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
+  hipError_t err = hipSuccess;
+  dispatch_nb(g.nb, [&](auto nbc) {
+    constexpr int NB = decltype(nbc)::value;
+    hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g, steps);
+  });
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+template <int FMT>
+hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
+  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
+  const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
+  const int steps = pick_steps(per_slot * a.slots);
+  const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
+  dispatch_nb(g.nb, [&](auto nbc) {
+    constexpr int NB = decltype(nbc)::value;
+    hipLaunchKernelGGL((slot_down_kernel<FMT, NB>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g, steps);
+  });
+  return hipGetLastError();
+}
+
+template <int FMT>
+hipError_t launch_grouped_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {
+  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
+  const long long per_seg = (a.n + rows_per_step - 1) / rows_per_step;
+  const int steps = pick_steps(per_seg * n_segs);
+  const dim3 grid(static_cast<unsigned>((per_seg + steps - 1) / steps), static_cast<unsigned>(n_segs),
+                  static_cast<unsigned>(z_ext));
+  const size_t lds = stage_bytes(a.group_rows, a.k);
+  hipError_t err = hipSuccess;
+  dispatch_nb(g.nb, [&](auto nbc) {
+    constexpr int NB = decltype(nbc)::value;
+    auto kern = grouped_gemv_kernel<FMT, NB>;
+    err = ensure_lds(kern, lds);
+    if (err != hipSuccess) return;
+    hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
+  });
+  return err != hipSuccess ? err : hipGetLastError();
+}
+#endif  // DGPP_GEMV_IMPL
+
+}  // namespace dgpp_amd

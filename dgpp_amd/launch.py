@@ -1,0 +1,288 @@
+"""Python mirror of the reference's `dgpp::launch_*` operator surface over the C ABI.
+
+Same names, argument order and meaning as the reference headers (src/kernels/glm_moe_launch.hpp,
+fp4_gemv.hpp, scale_gemm.hpp, fp8_dequant.hpp, minimax.hpp); the reference's
+std::invalid_argument becomes InvalidArgument (a ValueError), its std::runtime_error a
+RuntimeError. Pointer arguments accept torch tensors (their data_ptr()), ints or None; torch
+only supplies device memory and streams here.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+from . import _lib
+from ._lib import Fp4Matrix, Fp8GemvProblem, MoeConfig, MoeExpertView, MoeSegment, MoeTile  # noqa: F401
+
+ROUTER_SIGMOID_BIAS, ROUTER_SOFTMAX_TOPK, ROUTER_SQRT_SOFTPLUS_BIAS = 0, 1, 2
+K_FP4_GROUP, K_MXFP4_GROUP = 16, 32
+
+
+class InvalidArgument(ValueError):
+    """The reference launcher would have thrown std::invalid_argument; nothing was launched."""
+
+
+def _p(x):
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    if isinstance(x, (C.Structure, C.Array)):
+        return C.addressof(x)
+    raise TypeError(f"cannot take a pointer of {type(x)!r}")
+
+
+def _stream(stream):
+    if stream is None:
+        return None
+    if isinstance(stream, int):
+        return stream or None
+    return stream.cuda_stream or None  # torch.cuda.Stream
+
+
+def _check(rc: int) -> None:
+    if rc == _lib.OK:
+        return
+    msg = _lib.load().dgpp_last_error().decode()
+    if rc == _lib.INVALID_ARGUMENT:
+        raise InvalidArgument(msg)
+    raise RuntimeError(msg)
+
+
+def make_config(hidden, inter, n_experts, top_k, *, n_shared_experts=1, routed_scaling_factor=2.5,
+                norm_topk_prob=True, swiglu_limit=10.0, router_mode=ROUTER_SIGMOID_BIAS) -> MoeConfig:
+    return MoeConfig(hidden, inter, n_experts, top_k, n_shared_experts, routed_scaling_factor,
+                     1 if norm_topk_prob else 0, swiglu_limit, router_mode)
+
+
+def validate_config(cfg: MoeConfig) -> None:
+    _check(_lib.load().dgpp_moe_config_validate(C.addressof(cfg)))
+
+
+# ---- router -------------------------------------------------------------------------------------
+def launch_moe_router(hidden, gate, bias, ids, weights, scores, biased, cfg: MoeConfig, tokens, stream=None,
+                      counters=None, allow_tiled=True):
+    _check(_lib.load().dgpp_launch_moe_router(_p(hidden), _p(gate), _p(bias), _p(ids), _p(weights), _p(scores),
+                                              _p(biased), C.addressof(cfg), tokens, _stream(stream), _p(counters),
+                                              1 if allow_tiled else 0))
+
+
+def launch_moe_router_select(scores, biased, ids, weights, cfg: MoeConfig, tokens, stream=None):
+    _check(_lib.load().dgpp_launch_moe_router_select(_p(scores), _p(biased), _p(ids), _p(weights), C.addressof(cfg),
+                                                     tokens, _stream(stream)))
+
+
+# ---- elementwise --------------------------------------------------------------------------------
+def launch_moe_swiglu_clamp(gate, up, out, n, limit, stream=None):
+    _check(_lib.load().dgpp_launch_moe_swiglu_clamp(_p(gate), _p(up), _p(out), n, limit, _stream(stream)))
+
+
+def launch_moe_gather_rows(src, rows, dst, n_rows, hidden, stream=None):
+    _check(_lib.load().dgpp_launch_moe_gather_rows(_p(src), _p(rows), _p(dst), n_rows, hidden, _stream(stream)))
+
+
+def launch_moe_accum(acc, y, rows, row_weights, n_rows, hidden, stream=None):
+    _check(_lib.load().dgpp_launch_moe_accum(_p(acc), _p(y), _p(rows), _p(row_weights), n_rows, hidden, _stream(stream)))
+
+
+def launch_moe_round_bf16(out, acc, n, stream=None):
+    _check(_lib.load().dgpp_launch_moe_round_bf16(_p(out), _p(acc), n, _stream(stream)))
+
+
+# ---- grouping -------------------------------------------------------------------------------------
+def launch_moe_segment(ids, tokens, top_k, n_experts, rows, slot_row, segs, stream=None):
+    _check(_lib.load().dgpp_launch_moe_segment(_p(ids), tokens, top_k, n_experts, _p(rows), _p(slot_row), _p(segs),
+                                               _stream(stream)))
+
+
+def moe_tile_list_capacity(n_segs, total_rows, tile_rows) -> int:
+    return _lib.load().dgpp_moe_tile_list_capacity(n_segs, total_rows, tile_rows)
+
+
+def launch_moe_tile_list(segs, n_segs, tile_rows, tiles, count, stream=None):
+    _check(_lib.load().dgpp_launch_moe_tile_list(_p(segs), n_segs, tile_rows, _p(tiles), _p(count), _stream(stream)))
+
+
+def moe_run_groups_max(slots) -> int:
+    return _lib.load().dgpp_moe_run_groups_max(slots)
+
+
+def launch_moe_slot_order(ids, order, slots, top_k, n_experts, stream=None, shared_early=False, runs=None):
+    _check(_lib.load().dgpp_launch_moe_slot_order(_p(ids), _p(order), slots, top_k, n_experts, _stream(stream),
+                                                  1 if shared_early else 0, _p(runs)))
+
+
+def minimax_compact_segments(input, output, experts, capacity, stream=None):
+    _check(_lib.load().dgpp_minimax_compact_segments(_p(input), _p(output), experts, capacity, _stream(stream)))
+
+
+# ---- accumulation -----------------------------------------------------------------------------------
+def launch_moe_accum_ordered(out, down, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens, top_k, hidden,
+                             stream=None):
+    _check(_lib.load().dgpp_launch_moe_accum_ordered(_p(out), _p(down), down_stride, _p(slot_row), _p(slot_ids),
+                                                     _p(slot_w), shared_row0, tokens, top_k, hidden, _stream(stream)))
+
+
+def launch_moe_accum_ordered_f32(out, down, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens, top_k,
+                                 hidden, stream=None):
+    _check(_lib.load().dgpp_launch_moe_accum_ordered_f32(_p(out), _p(down), down_stride, _p(slot_row), _p(slot_ids),
+                                                         _p(slot_w), shared_row0, tokens, top_k, hidden,
+                                                         _stream(stream)))
+
+
+def launch_moe_slot_accum(out, contrib, weights, tokens, hidden, top_k, stream=None):
+    _check(_lib.load().dgpp_launch_moe_slot_accum(_p(out), _p(contrib), _p(weights), tokens, hidden, top_k,
+                                                  _stream(stream)))
+
+
+def launch_moe_slot_accum_routed_f32(out, contrib, weights, tokens, hidden, top_k, stream=None):
+    _check(_lib.load().dgpp_launch_moe_slot_accum_routed_f32(_p(out), _p(contrib), _p(weights), tokens, hidden, top_k,
+                                                             _stream(stream)))
+
+
+# ---- decode-slot kernels ------------------------------------------------------------------------------
+def launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                   sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride,
+                                   slots, top_k, limit, stream=None, sh_rs=7, sh_cs=7):
+    _check(_lib.load().dgpp_launch_moe_slot_gate_up_swiglu(
+        _p(x), x_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_gate_payload),
+        _p(sh_gate_scales), _p(sh_up_payload), _p(sh_up_scales), _p(act), act_stride, slots, top_k, limit,
+        _stream(stream), sh_rs, sh_cs))
+
+
+def launch_moe_slot_down(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared, sh_payload,
+                         sh_scales, out, out_stride, slots, top_k, stream=None, sh_rs=7, sh_cs=7):
+    _check(_lib.load().dgpp_launch_moe_slot_down(
+        _p(act), act_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_payload),
+        _p(sh_scales), _p(out), out_stride, slots, top_k, _stream(stream), sh_rs, sh_cs))
+
+
+def launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                       sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride,
+                                       slots, top_k, limit, stream=None, shared_view_base=-1, fp4_group=16, sh_rs=7,
+                                       sh_cs=7):
+    _check(_lib.load().dgpp_launch_moe_slot_gate_up_swiglu_fp4(
+        _p(x), x_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_gate_payload),
+        _p(sh_gate_scales), _p(sh_up_payload), _p(sh_up_scales), _p(act), act_stride, slots, top_k, limit,
+        _stream(stream), shared_view_base, fp4_group, sh_rs, sh_cs))
+
+
+def launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared, sh_payload,
+                             sh_scales, out, out_stride, slots, top_k, stream=None, shared_view_base=-1, fp4_group=16,
+                             sh_rs=7, sh_cs=7, tile_counter=None):
+    _check(_lib.load().dgpp_launch_moe_slot_down_fp4(
+        _p(act), act_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_payload),
+        _p(sh_scales), _p(out), out_stride, slots, top_k, _stream(stream), shared_view_base, fp4_group, sh_rs, sh_cs,
+        _p(tile_counter)))
+
+
+# ---- grouped twins ---------------------------------------------------------------------------------------
+def launch_moe_grouped_gemv_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
+                                 out_stride, n, k, stream=None):
+    _check(_lib.load().dgpp_launch_moe_grouped_gemv_bf16(_p(act), act_stride, _p(segs), n_segs, max_rows,
+                                                         rows_per_block, _p(views), which, _p(out), out_stride, n, k,
+                                                         _stream(stream)))
+
+
+def launch_moe_grouped_gemv_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
+                                out_stride, n, k, stream=None):
+    _check(_lib.load().dgpp_launch_moe_grouped_gemv_f32(_p(act), act_stride, _p(segs), n_segs, max_rows,
+                                                        rows_per_block, _p(views), which, _p(out), out_stride, n, k,
+                                                        _stream(stream)))
+
+
+def launch_moe_grouped_gemv_fp4_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
+                                     out_stride, n, k, stream=None, fp4_group=16):
+    _check(_lib.load().dgpp_launch_moe_grouped_gemv_fp4_bf16(_p(act), act_stride, _p(segs), n_segs, max_rows,
+                                                             rows_per_block, _p(views), which, _p(out), out_stride, n,
+                                                             k, _stream(stream), fp4_group))
+
+
+def launch_moe_grouped_gemv_fp4_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
+                                    out_stride, n, k, stream=None, fp4_group=16):
+    _check(_lib.load().dgpp_launch_moe_grouped_gemv_fp4_f32(_p(act), act_stride, _p(segs), n_segs, max_rows,
+                                                            rows_per_block, _p(views), which, _p(out), out_stride, n,
+                                                            k, _stream(stream), fp4_group))
+
+
+# ---- dense projections --------------------------------------------------------------------------------------
+def launch_fp4_gemv_bf16(act, act_row_stride_elems, w: Fp4Matrix, out, m, n, k, stream=None):
+    _check(_lib.load().dgpp_launch_fp4_gemv_bf16(_p(act), act_row_stride_elems, C.addressof(w), _p(out), m, n, k,
+                                                 _stream(stream)))
+
+
+def launch_fp4_gemv_f32(act, act_row_stride_elems, w: Fp4Matrix, out, m, n, k, stream=None):
+    _check(_lib.load().dgpp_launch_fp4_gemv_f32(_p(act), act_row_stride_elems, C.addressof(w), _p(out), m, n, k,
+                                                _stream(stream)))
+
+
+def fp4_gemv_accepts(w: Fp4Matrix) -> bool:
+    return bool(_lib.load().dgpp_fp4_gemv_accepts(C.addressof(w)))
+
+
+def launch_scale_gemm_bf16(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream=None,
+                           out_row_stride_elems=0, mma_from_rows=0, ws=None, ws_bytes=0):
+    _check(_lib.load().dgpp_launch_scale_gemm_bf16(_p(act), act_row_stride_elems, _p(w_payload), _p(w_scales), _p(out),
+                                                   m, n, k, _stream(stream), out_row_stride_elems, mma_from_rows,
+                                                   _p(ws), ws_bytes))
+
+
+def launch_scale_gemm_f32(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream=None,
+                          out_row_stride_elems=0, mma_from_rows=0, last_row_only=False, ws=None, ws_bytes=0,
+                          compact_row=-1):
+    _check(_lib.load().dgpp_launch_scale_gemm_f32(_p(act), act_row_stride_elems, _p(w_payload), _p(w_scales), _p(out),
+                                                  m, n, k, _stream(stream), out_row_stride_elems, mma_from_rows,
+                                                  1 if last_row_only else 0, _p(ws), ws_bytes, compact_row))
+
+
+def launch_scale_gemm_grid_bf16(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                                out_row_stride_elems, rs, cs, decode_mma=False, ws=None, ws_bytes=0,
+                                prefill_tile=False):
+    _check(_lib.load().dgpp_launch_scale_gemm_grid_bf16(_p(act), act_row_stride_elems, _p(w_payload), _p(w_scales),
+                                                        _p(out), m, n, k, _stream(stream), out_row_stride_elems, rs,
+                                                        cs, int(decode_mma), _p(ws), ws_bytes, int(prefill_tile)))
+
+
+def launch_scale_gemm_grid_f32(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                               out_row_stride_elems, rs, cs, decode_mma=False, ws=None, ws_bytes=0,
+                               prefill_tile=False):
+    _check(_lib.load().dgpp_launch_scale_gemm_grid_f32(_p(act), act_row_stride_elems, _p(w_payload), _p(w_scales),
+                                                       _p(out), m, n, k, _stream(stream), out_row_stride_elems, rs,
+                                                       cs, int(decode_mma), _p(ws), ws_bytes, int(prefill_tile)))
+
+
+def launch_scale_gemm_grid_e8m0_bf16(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                                     out_row_stride_elems, rs, cs, ws=None, ws_bytes=0, prefill_tile=False):
+    _check(_lib.load().dgpp_launch_scale_gemm_grid_e8m0_bf16(_p(act), act_row_stride_elems, _p(w_payload),
+                                                             _p(w_scales), _p(out), m, n, k, _stream(stream),
+                                                             out_row_stride_elems, rs, cs, _p(ws), ws_bytes,
+                                                             int(prefill_tile)))
+
+
+def launch_scale_gemm_grid_e8m0_f32(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                                    out_row_stride_elems, rs, cs, ws=None, ws_bytes=0, prefill_tile=False):
+    _check(_lib.load().dgpp_launch_scale_gemm_grid_e8m0_f32(_p(act), act_row_stride_elems, _p(w_payload),
+                                                            _p(w_scales), _p(out), m, n, k, _stream(stream),
+                                                            out_row_stride_elems, rs, cs, _p(ws), ws_bytes,
+                                                            int(prefill_tile)))
+
+
+def launch_scale_gemv_multi_bf16(problems, act, act_row_stride_elems, rows, k, stream=None):
+    arr = (Fp8GemvProblem * len(problems))(*problems)
+    _check(_lib.load().dgpp_launch_scale_gemv_multi_bf16(C.addressof(arr), len(problems), _p(act),
+                                                         act_row_stride_elems, rows, k, _stream(stream)))
+
+
+def fp8_gemv_can_stage(w_payload, k) -> bool:
+    return bool(_lib.load().dgpp_fp8_gemv_can_stage(_p(w_payload), k))
+
+
+def launch_fp8_dequant_blocks(payload, scales, out_bf16, rows, cols, stream=None, rs=7, cs=7):
+    _check(_lib.load().dgpp_launch_fp8_dequant_blocks(_p(payload), _p(scales), _p(out_bf16), rows, cols,
+                                                      _stream(stream), rs, cs))
+
+
+def launch_fp8_dequant_blocks_e8m0(payload, scales, out_bf16, rows, cols, stream, rs, cs):
+    _check(_lib.load().dgpp_launch_fp8_dequant_blocks_e8m0(_p(payload), _p(scales), _p(out_bf16), rows, cols,
+                                                           _stream(stream), rs, cs))

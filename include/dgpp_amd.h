@@ -1,0 +1,336 @@
+/*
+ * dgpp_amd — C ABI of the MI355X (gfx950) quantized MoE expert GEMV path.
+ *
+ * One `extern "C"` entry point per kernel launcher of the reference's operator surface for this
+ * path (src/kernels/glm_moe_launch.hpp, fp4_gemv.hpp, scale_gemm.hpp, fp8_dequant.hpp,
+ * minimax.hpp), same argument order and meaning. Differences that the C ABI forces:
+ *   - the stream is an opaque `void*` holding a hipStream_t (null = the default stream);
+ *   - C++ default arguments are spelled out;
+ *   - instead of throwing, every launcher returns DGPP_OK, DGPP_INVALID_ARGUMENT (the
+ *     reference's std::invalid_argument: nothing was launched) or DGPP_RUNTIME_ERROR (the
+ *     reference's std::runtime_error from a failed runtime call); dgpp_last_error() returns the
+ *     message of the calling thread's last failure. include/dgpp_amd.hpp re-throws them.
+ *
+ * Conventions (reference: src/kernels/glm_moe_launch.hpp:211-243, src/kernels/scale_gemm.hpp:27-36):
+ * bf16 travels as uint16_t bit patterns; e4m3 / e2m1 pairs / e8m0 as uint8_t; every pointer is
+ * a DEVICE pointer unless the parameter is documented as host; matrices are row-major W[n, k]
+ * and the product is D = Act * W^T; strides are in ELEMENTS; launchers are asynchronous on the
+ * given stream, allocate nothing, never synchronise, and are deterministic run to run.
+ */
+#ifndef DGPP_AMD_H
+#define DGPP_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DGPP_OK 0
+#define DGPP_INVALID_ARGUMENT 1
+#define DGPP_RUNTIME_ERROR 2
+
+/* Message of the calling thread's most recent failed call ("" when none). */
+const char* dgpp_last_error(void);
+/* "gfx950" — the only architecture the library carries code for. */
+const char* dgpp_target_arch(void);
+
+/* ---- POD types shared with device code -------------------------------------------------- */
+
+/* Device-side expert table entry, read by the slot and grouped kernels.
+ * Layout-identical (96 bytes, same offsets) to the reference's MoeExpertView,
+ * src/models/glm/moe.hpp:232-292. Fields the path does not use are kept as reserved space. */
+typedef struct DgppMoeExpertView {
+  const uint8_t* payload;     /*  0  fp8: e4m3 [n, k]; fp4: e2m1 pairs [n, k/2]            */
+  const float* scales;        /*  8  fp8: F32 block scales (fp4: null)                     */
+  const uint8_t* fp4_scales;  /* 16  NVFP4: e4m3 [n, k/16]; MXFP4: e8m0 [n, k/32]          */
+  const float* fp4_global;    /* 24  NVFP4: the matrix's F32 global scale (MXFP4: null)    */
+  int32_t scale_shift_rows;   /* 32  fp8 scale grid, log2 block rows (7 = 128)             */
+  int32_t scale_shift_cols;   /* 36  fp8 scale grid, log2 block cols                       */
+  int32_t fp4_group;          /* 40  16 = NVFP4, 32 = MXFP4                                */
+  int32_t reserved0;          /* 44                                                        */
+  const void* reserved1;      /* 48  (reference: packed_scales)                            */
+  int32_t reserved2[2];       /* 56  (reference: bits, packed_scale_fmt)                   */
+  const void* reserved3[2];   /* 64  (reference: exl3_suh, exl3_svh)                       */
+  int32_t reserved4[4];       /* 80  (reference: exl3_bits, exl3_rows, exl3_cols, pad)     */
+} DgppMoeExpertView;
+
+/* src/kernels/glm_moe_launch.hpp:67-71 */
+typedef struct DgppMoeSegment {
+  int32_t row0;   /* first row of the segment in act / out */
+  int32_t rows;   /* rows in the segment */
+  int32_t expert; /* view-table expert index (the shared expert last) */
+} DgppMoeSegment;
+
+/* src/kernels/glm_moe_launch.hpp:151-154 */
+typedef struct DgppMoeTile {
+  int32_t seg; /* index into the segment table */
+  int32_t m0;  /* first row of the tile within the segment */
+} DgppMoeTile;
+
+/* src/models/quant_matrix.hpp:117-138 (GlmFp4Matrix), same 56-byte layout. */
+typedef struct DgppFp4Matrix {
+  const uint8_t* payload;     /* U8 [rows, cols/2], low nibble = even element */
+  const uint8_t* scales;      /* e4m3 [rows, cols/16] or e8m0 [rows, cols/32] */
+  const float* global_scale;  /* F32 [1] on the device; null under MXFP4 */
+  int64_t rows;
+  int64_t cols;               /* logical K (elements) */
+  int32_t scale_group;        /* 16: NVFP4, 32: MXFP4 */
+  int32_t reserved0;
+  const void* reserved1;      /* (reference: tma) */
+} DgppFp4Matrix;
+
+/* Router scoring rule, src/models/glm/moe.hpp:49. */
+#define DGPP_ROUTER_SIGMOID_BIAS 0
+#define DGPP_ROUTER_SOFTMAX_TOPK 1
+#define DGPP_ROUTER_SQRT_SOFTPLUS_BIAS 2
+
+/* The router-relevant fields of the reference's GlmMoeConfig, src/models/glm/moe.hpp:51-134.
+ * dgpp_moe_config_validate applies validate_config's rules (moe.hpp:119-133). */
+typedef struct DgppMoeConfig {
+  int32_t hidden;
+  int32_t inter;
+  int32_t n_experts;
+  int32_t top_k;
+  int32_t n_shared_experts;
+  float routed_scaling_factor;
+  int32_t norm_topk_prob;
+  float swiglu_limit;
+  int32_t router_mode;
+} DgppMoeConfig;
+int dgpp_moe_config_validate(const DgppMoeConfig* cfg);
+
+/* ---- router ------------------------------------------------------------------------------ */
+/* src/kernels/glm_moe_launch.hpp:23 (launch_moe_router). counters (nullable) is accepted for
+ * signature parity; the two-kernel form is used either way and the counters stay zero. */
+int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const float* bias,
+                           int32_t* ids, float* weights, float* scores, float* biased,
+                           const DgppMoeConfig* cfg, int tokens, void* stream, int* counters,
+                           int allow_tiled);
+/* The selection half of launch_moe_router alone (src/kernels/glm_moe.cu:314-329,
+ * moe_router_select_kernel): scores / biased f32 [tokens, n_experts] already on the device
+ * (softmax mode: the bf16-rounded logits in both) -> ids ascending, weights. */
+int dgpp_launch_moe_router_select(const float* scores, const float* biased, int32_t* ids,
+                                  float* weights, const DgppMoeConfig* cfg, int tokens,
+                                  void* stream);
+
+/* ---- elementwise pieces -------------------------------------------------------------------- */
+/* src/kernels/glm_moe_launch.hpp:43 */
+int dgpp_launch_moe_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out,
+                                 int64_t n, float limit, void* stream);
+/* src/kernels/glm_moe_launch.hpp:48 */
+int dgpp_launch_moe_gather_rows(const uint16_t* src, const int32_t* rows, uint16_t* dst,
+                                int n_rows, int hidden, void* stream);
+/* src/kernels/glm_moe_launch.hpp:56 */
+int dgpp_launch_moe_accum(float* acc, const float* y, const int32_t* rows,
+                          const float* row_weights, int n_rows, int hidden, void* stream);
+/* src/kernels/glm_moe_launch.hpp:195 */
+int dgpp_launch_moe_round_bf16(uint16_t* out, const float* acc, int64_t n, void* stream);
+
+/* ---- grouping ------------------------------------------------------------------------------- */
+/* src/kernels/glm_moe_launch.hpp:134 */
+int dgpp_launch_moe_segment(const int32_t* ids, int tokens, int top_k, int n_experts,
+                            int32_t* rows, int32_t* slot_row, DgppMoeSegment* segs, void* stream);
+/* src/kernels/glm_moe_launch.hpp:155-160 */
+int dgpp_moe_tile_list_capacity(int n_segs, int total_rows, int tile_rows);
+int dgpp_launch_moe_tile_list(const DgppMoeSegment* segs, int n_segs, int tile_rows,
+                              DgppMoeTile* tiles, int32_t* count, void* stream);
+/* src/kernels/glm_moe_launch.hpp:244; runs (nullable) holds slots + dgpp_moe_run_groups_max(slots)
+ * entries (glm_moe_launch.hpp:207-209). */
+int dgpp_moe_run_groups_max(int slots);
+int dgpp_launch_moe_slot_order(const int32_t* ids, int32_t* order, int slots, int top_k,
+                               int n_experts, void* stream, int shared_early, int32_t* runs);
+/* src/kernels/minimax.hpp:11 */
+int dgpp_minimax_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* output,
+                                  int experts, int capacity, void* stream);
+
+/* ---- ordered accumulation -------------------------------------------------------------------- */
+/* src/kernels/glm_moe_launch.hpp:168-180 */
+int dgpp_launch_moe_accum_ordered(uint16_t* out, const float* down, size_t down_stride,
+                                  const int32_t* slot_row, const int32_t* slot_ids,
+                                  const float* slot_w, int shared_row0, int tokens, int top_k,
+                                  int hidden, void* stream);
+int dgpp_launch_moe_accum_ordered_f32(float* out, const float* down, size_t down_stride,
+                                      const int32_t* slot_row, const int32_t* slot_ids,
+                                      const float* slot_w, int shared_row0, int tokens, int top_k,
+                                      int hidden, void* stream);
+/* src/kernels/glm_moe_launch.hpp:273-283 */
+int dgpp_launch_moe_slot_accum(uint16_t* out, const float* contrib, const float* weights,
+                               int tokens, int hidden, int top_k, void* stream);
+int dgpp_launch_moe_slot_accum_routed_f32(float* out, const float* contrib, const float* weights,
+                                          int tokens, int hidden, int top_k, void* stream);
+
+/* ---- FP8 block-scaled decode-slot kernels ------------------------------------------------------ */
+/* src/kernels/glm_moe_launch.hpp:247-253 */
+int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                        const int32_t* order, const DgppMoeExpertView* views,
+                                        int n_routed, int k_routed, int n_shared, int k_shared,
+                                        const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                        const uint8_t* sh_up_payload, const float* sh_up_scales,
+                                        uint16_t* act, int act_stride, int slots, int top_k,
+                                        float limit, void* stream, int sh_rs, int sh_cs);
+/* src/kernels/glm_moe_launch.hpp:258-265 */
+int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                              const int32_t* order, const DgppMoeExpertView* views, int n_routed,
+                              int k_routed, int n_shared, int k_shared, const uint8_t* sh_payload,
+                              const float* sh_scales, float* out, int out_stride, int slots,
+                              int top_k, void* stream, int sh_rs, int sh_cs);
+
+/* ---- NVFP4 / MXFP4 decode-slot kernels ----------------------------------------------------------- */
+/* src/kernels/glm_moe_launch.hpp:392-399 */
+int dgpp_launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                            const int32_t* order, const DgppMoeExpertView* views,
+                                            int n_routed, int k_routed, int n_shared, int k_shared,
+                                            const uint8_t* sh_gate_payload,
+                                            const float* sh_gate_scales,
+                                            const uint8_t* sh_up_payload, const float* sh_up_scales,
+                                            uint16_t* act, int act_stride, int slots, int top_k,
+                                            float limit, void* stream, int shared_view_base,
+                                            int fp4_group, int sh_rs, int sh_cs);
+/* src/kernels/glm_moe_launch.hpp:400-408. tile_counter (two device ints zeroed once by the
+ * caller) is accepted for signature parity and left untouched: this build's down kernel uses a
+ * static grid. */
+int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                  const int32_t* order, const DgppMoeExpertView* views,
+                                  int n_routed, int k_routed, int n_shared, int k_shared,
+                                  const uint8_t* sh_payload, const float* sh_scales, float* out,
+                                  int out_stride, int slots, int top_k, void* stream,
+                                  int shared_view_base, int fp4_group, int sh_rs, int sh_cs,
+                                  int* tile_counter);
+
+/* ---- grouped (segment-major) GEMV twins ------------------------------------------------------------ */
+/* src/kernels/glm_moe_launch.hpp:77-87 */
+int dgpp_launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride,
+                                      const DgppMoeSegment* segs, int n_segs, int max_rows,
+                                      int rows_per_block, const DgppMoeExpertView* views, int which,
+                                      uint16_t* out, size_t out_stride, int n, int k, void* stream);
+int dgpp_launch_moe_grouped_gemv_f32(const uint16_t* act, size_t act_stride,
+                                     const DgppMoeSegment* segs, int n_segs, int max_rows,
+                                     int rows_per_block, const DgppMoeExpertView* views, int which,
+                                     float* out, size_t out_stride, int n, int k, void* stream);
+/* src/kernels/glm_moe_launch.hpp:375-386 */
+int dgpp_launch_moe_grouped_gemv_fp4_bf16(const uint16_t* act, size_t act_stride,
+                                          const DgppMoeSegment* segs, int n_segs, int max_rows,
+                                          int rows_per_block, const DgppMoeExpertView* views,
+                                          int which, uint16_t* out, size_t out_stride, int n, int k,
+                                          void* stream, int fp4_group);
+int dgpp_launch_moe_grouped_gemv_fp4_f32(const uint16_t* act, size_t act_stride,
+                                         const DgppMoeSegment* segs, int n_segs, int max_rows,
+                                         int rows_per_block, const DgppMoeExpertView* views,
+                                         int which, float* out, size_t out_stride, int n, int k,
+                                         void* stream, int fp4_group);
+
+/* ---- dense NVFP4 / MXFP4 projection GEMV -------------------------------------------------------------- */
+/* src/kernels/fp4_gemv.hpp:23-32. `w` is a HOST struct holding device pointers. */
+int dgpp_launch_fp4_gemv_bf16(const uint16_t* act, size_t act_row_stride_elems,
+                              const DgppFp4Matrix* w, uint16_t* out, int m, int n, int k,
+                              void* stream);
+int dgpp_launch_fp4_gemv_f32(const uint16_t* act, size_t act_row_stride_elems,
+                             const DgppFp4Matrix* w, float* out, int m, int n, int k, void* stream);
+/* 1 when the core accepts the matrix, else 0. */
+int dgpp_fp4_gemv_accepts(const DgppFp4Matrix* w);
+
+/* ---- dense FP8 block-scaled projection GEMV ------------------------------------------------------------ */
+/* src/kernels/scale_gemm.hpp:57-79. mma_from_rows, ws and ws_bytes are accepted for signature
+ * parity; every m takes the row-independent GEMV form here. */
+int dgpp_launch_scale_gemm_bf16(const uint16_t* act, size_t act_row_stride_elems,
+                                const uint8_t* w_payload, const float* w_scales, uint16_t* out,
+                                int m, int n, int k, void* stream, size_t out_row_stride_elems,
+                                int mma_from_rows, void* ws, size_t ws_bytes);
+int dgpp_launch_scale_gemm_f32(const uint16_t* act, size_t act_row_stride_elems,
+                               const uint8_t* w_payload, const float* w_scales, float* out, int m,
+                               int n, int k, void* stream, size_t out_row_stride_elems,
+                               int mma_from_rows, int last_row_only, void* ws, size_t ws_bytes,
+                               int compact_row);
+/* src/kernels/scale_gemm.hpp:140-149 (decode_mma / ws / prefill_tile accepted, GEMV form). */
+int dgpp_launch_scale_gemm_grid_bf16(const uint16_t* act, size_t act_row_stride_elems,
+                                     const uint8_t* w_payload, const float* w_scales, uint16_t* out,
+                                     int m, int n, int k, void* stream,
+                                     size_t out_row_stride_elems, int rs, int cs, int decode_mma,
+                                     void* ws, size_t ws_bytes, int prefill_tile);
+int dgpp_launch_scale_gemm_grid_f32(const uint16_t* act, size_t act_row_stride_elems,
+                                    const uint8_t* w_payload, const float* w_scales, float* out,
+                                    int m, int n, int k, void* stream, size_t out_row_stride_elems,
+                                    int rs, int cs, int decode_mma, void* ws, size_t ws_bytes,
+                                    int prefill_tile);
+/* src/kernels/scale_gemm.hpp:155-162: the scale grid as e8m0 bytes (MXFP8: rs = 0, cs = 5). */
+int dgpp_launch_scale_gemm_grid_e8m0_bf16(const uint16_t* act, size_t act_row_stride_elems,
+                                          const uint8_t* w_payload, const uint8_t* w_scales,
+                                          uint16_t* out, int m, int n, int k, void* stream,
+                                          size_t out_row_stride_elems, int rs, int cs, void* ws,
+                                          size_t ws_bytes, int prefill_tile);
+int dgpp_launch_scale_gemm_grid_e8m0_f32(const uint16_t* act, size_t act_row_stride_elems,
+                                         const uint8_t* w_payload, const uint8_t* w_scales,
+                                         float* out, int m, int n, int k, void* stream,
+                                         size_t out_row_stride_elems, int rs, int cs, void* ws,
+                                         size_t ws_bytes, int prefill_tile);
+/* src/kernels/scale_gemm.hpp:85-107: up to four [n_i, k] fp8 matrices against the same rows.
+ * `problems` is a HOST array. bf16_weight must be null (that form is outside this path). */
+typedef struct DgppFp8GemvProblem {
+  const uint8_t* payload;
+  const float* scales;
+  uint16_t* out;
+  int32_t n;
+  int32_t reserved0;
+  size_t out_stride;
+  int32_t rs;
+  int32_t cs;
+  const uint16_t* bf16_weight;
+} DgppFp8GemvProblem;
+int dgpp_launch_scale_gemv_multi_bf16(const DgppFp8GemvProblem* problems, int n_problems,
+                                      const uint16_t* act, size_t act_row_stride_elems, int rows,
+                                      int k, void* stream);
+/* src/kernels/scale_gemm.hpp:171: 1 when the fp8 GEMV can stage this payload at one row. */
+int dgpp_fp8_gemv_can_stage(const void* w_payload, int k);
+
+/* ---- FP8 -> BF16 dequant bridge ---------------------------------------------------------------------------- */
+/* src/kernels/fp8_dequant.hpp:22-29 */
+int dgpp_launch_fp8_dequant_blocks(const uint8_t* payload, const float* scales, uint16_t* out_bf16,
+                                   int64_t rows, int64_t cols, void* stream, int rs, int cs);
+int dgpp_launch_fp8_dequant_blocks_e8m0(const uint8_t* payload, const uint8_t* scales,
+                                        uint16_t* out_bf16, int64_t rows, int64_t cols,
+                                        void* stream, int rs, int cs);
+
+/* ---- host-side weight encoders and synthetic data (no GPU involved) ------------------------------------------ */
+/* Scalar codecs, src/common/dtypes.hpp:83-190, src/kernels/latent_format.hpp:117-162. */
+float dgpp_bf16_to_f32(uint16_t bits);
+uint16_t dgpp_f32_to_bf16(float v);
+float dgpp_e4m3_to_f32(uint8_t code);
+uint8_t dgpp_f32_to_e4m3(float v);
+float dgpp_e2m1_to_f32(uint8_t code);
+uint8_t dgpp_f32_to_e2m1(float v);
+float dgpp_e8m0_to_f32(uint8_t code);
+uint8_t dgpp_e8m0_ceil_log2(float v);
+/* Block FP8 encoder, src/loaders/fp8_quant.hpp:32-46 generalised to any block size:
+ * scale_b = amax/448 (zero block: 1), code = e4m3_rne_sat(w / scale_b). src bf16 [rows, cols]. */
+void dgpp_encode_fp8_blocks(const uint16_t* src_bf16, int64_t rows, int64_t cols, int block_rows,
+                            int block_cols, uint8_t* payload, float* scales, int threads);
+/* NVFP4 encoder, src/loaders/nvfp4_quant.hpp:25-55. Returns weight_scale_2; the DEVICE global the
+ * kernels divide by is 1 / weight_scale_2. src f32 [rows, cols], cols % 16 == 0. */
+float dgpp_encode_nvfp4(const float* src, int64_t rows, int64_t cols, uint8_t* payload,
+                        uint8_t* scales, int threads);
+/* MXFP4 / MXFP8 encoders: one e8m0 byte per 32 elements chosen by the reference's own e8m0
+ * producers' rule, b = 127 + ceil(log2(amax / fmt_max)) from the IEEE fields
+ * (src/kernels/latent_format.hpp:117-123, src/kernels/mxfp8_gemm.cu:61-66), codes RNE saturating;
+ * an all-zero block stores byte 0 and zero codes. src f32 [rows, cols], cols % 32 == 0. */
+void dgpp_encode_mxfp4(const float* src, int64_t rows, int64_t cols, uint8_t* payload,
+                       uint8_t* scales, int threads);
+void dgpp_encode_mxfp8(const float* src, int64_t rows, int64_t cols, uint8_t* payload,
+                       uint8_t* scales, int threads);
+/* Seeded synthetic data: xorshift64 (tests/cuda/scale_gemm_test_helpers.hpp:29-47's generator
+ * family) + Box-Muller; element i of a stream depends on (seed, i / 4096) only, so the output does
+ * not depend on `threads`. */
+void dgpp_fill_normal_f32(uint64_t seed, float mean, float stddev, int64_t n, float* out,
+                          int threads);
+void dgpp_fill_normal_bf16(uint64_t seed, float mean, float stddev, int64_t n, uint16_t* out,
+                           int threads);
+/* top_k distinct expert ids per token drawn without replacement from Zipf(s) popularity over
+ * n_experts (expert e has weight 1/(e+1)^s), ids ascending per token. */
+void dgpp_fill_zipf_routes(uint64_t seed, double s, int tokens, int top_k, int n_experts,
+                           int32_t* ids);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DGPP_AMD_H */
