@@ -1,0 +1,58 @@
+"""The C ABI library loads without a GPU and exports every symbol include/dgpp_amd.h declares."""
+import ctypes
+import re
+from pathlib import Path
+
+from dgpp_amd import _lib
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def declared_symbols():
+    text = (ROOT / "include" / "dgpp_amd.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dgpp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = declared_symbols()
+    assert len(names) >= 50
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/dgpp_amd.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(names)
+    assert lib.dgpp_target_arch() == b"gfx950"
+
+
+def test_struct_layouts_match_the_reference_abi():
+    V = _lib.MoeExpertView
+    assert ctypes.sizeof(V) == 96
+    offs = {f: getattr(V, f).offset for f in ("payload", "scales", "fp4_scales", "fp4_global", "scale_shift_rows",
+                                              "scale_shift_cols", "fp4_group")}
+    assert offs == {"payload": 0, "scales": 8, "fp4_scales": 16, "fp4_global": 24, "scale_shift_rows": 32,
+                    "scale_shift_cols": 36, "fp4_group": 40}
+    assert ctypes.sizeof(_lib.MoeSegment) == 12 and ctypes.sizeof(_lib.MoeTile) == 8
+    assert ctypes.sizeof(_lib.Fp4Matrix) == 56 and _lib.Fp4Matrix.scale_group.offset == 40
+
+
+def test_host_side_argument_checks_need_no_gpu():
+    from dgpp_amd import launch as L
+    import pytest
+    cfg = L.make_config(64, 64, 8, 9)            # top_k > n_experts
+    with pytest.raises(L.InvalidArgument):
+        L.validate_config(cfg)
+    with pytest.raises(L.InvalidArgument):
+        L.validate_config(L.make_config(64, 64, 8, 17))
+    L.validate_config(L.make_config(4096, 1024, 256, 8, n_shared_experts=0, router_mode=L.ROUTER_SOFTMAX_TOPK))
+    assert L.moe_tile_list_capacity(5, 33, 16) == 5 + 3 and L.moe_run_groups_max(72) == 72 // 17 + 1
+    w = L.Fp4Matrix(0x1000, 0x2000, None, 8, 1024, 16, 0, None)
+    assert not L.fp4_gemv_accepts(w)            # NVFP4 without a global
+    w.scale_group = 32
+    assert L.fp4_gemv_accepts(w)
+    w.cols = 3072
+    assert not L.fp4_gemv_accepts(w)            # not in the MXFP4 set
+    assert L.fp8_gemv_can_stage(0x1000, 4096) and not L.fp8_gemv_can_stage(0x1001, 4096)
+    with pytest.raises(L.InvalidArgument):      # null pointers are refused before any launch
+        L.launch_moe_segment(None, 4, 8, 16, None, None, None)
+    L.launch_moe_segment(None, 0, 8, 16, None, None, None)      # tokens <= 0 returns silently
