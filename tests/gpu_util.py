@@ -69,3 +69,37 @@ def fp4_view(payload_d, scales_d, global_d, group) -> MoeExpertView:
 
 def segments_to_numpy(t: torch.Tensor) -> np.ndarray:
     return host(t).view(np.int32).reshape(-1, 3)
+
+
+class DeviceMoe:
+    """A MoeProblem (tests/moe_data.py) uploaded to the GPU: per-matrix tensors and the expert-view table
+    ([E * 3] routed entries, then the shared triple when it is an FP4 expert read through the table)."""
+
+    def __init__(self, p):
+        self.p = p
+        self.keep = []
+        entries = []
+        for e in p.experts:
+            for m in e:
+                entries.append(self._view(m))
+        self.shared_view_base = -1
+        self.sh = None
+        if p.shared is not None:
+            if p.shared_kind in ("nvfp4", "mxfp4"):
+                self.shared_view_base = len(entries)
+                for m in p.shared:
+                    entries.append(self._view(m))
+            else:
+                self.sh = [(dev(m.payload), dev(m.scales)) for m in p.shared]
+        self.views = view_table(entries)
+        self.x = dev(p.x)
+        self.fp4_group = 32 if p.kind == "mxfp4" else 16
+
+    def _view(self, m):
+        pd, sd = dev(m.payload), dev(m.scales)
+        self.keep += [pd, sd]
+        if m.kind == "fp8":
+            return fp8_view(pd, sd, m.rs, m.cs)
+        gd = dev(m.glob) if m.glob is not None else None
+        self.keep.append(gd)
+        return fp4_view(pd, sd, gd, 16 if m.kind == "nvfp4" else 32)

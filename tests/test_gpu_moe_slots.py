@@ -1,0 +1,239 @@
+"""The decode-slot kernels (fused gate/up + SwiGLU, down), their grouped twins and the full
+decode layer against the oracle.
+
+Budgets: a single GEMV stage keeps the strict comparator (2 bf16 ulps / 1e-3 floor / 0 mismatches);
+SwiGLU adds at most one bf16 ulp (tests/cuda/glm_moe_test.cu:1588); the layer keeps the reference's
+expert-path budget — hard 12 ulps, soft 4 ulps on < 2 % of elements, l2 < 4e-3, floor 2 % of the
+output RMS (tests/cuda/glm_moe_test.cu:606-658) — and the north-star measure stays <= 2e-3.
+"""
+import numpy as np
+import pytest
+
+import moe_data
+import oracle_lib as orc
+from dgpp_amd import hostgen as hg, launch as L
+from gpu_util import DeviceMoe, dev, dev_empty, host, sync
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_stage_outputs(p, ids):
+    """Per-slot oracle intermediates: act bf16 [slots, maxI] and down f64 [slots, H] (unrounded)."""
+    import np_ref
+    T, K = ids.shape
+    slots = T * (K + 1)
+    maxI = max(p.I, p.shared_I if p.shared else 0)
+    act = np.zeros((slots, maxI), np.uint16)
+    down = np.zeros((slots, p.H), np.float64)
+    used = np.zeros(slots, bool)
+    for t in range(T):
+        x = p.x[t:t + 1]
+        for j in range(K + 1):
+            if j == K and p.shared is None:
+                continue
+            mats = p.shared if j == K else p.experts[int(ids[t, j])]
+            I = p.shared_I if j == K else p.I
+            outs = []
+            for m in mats[:2]:
+                if m.kind in ("fp8", "mxfp8"):
+                    outs.append(orc.gemv_fp8(x, m.payload, m.scales, 1, I, p.H, m.rs, m.cs, True, m.kind == "mxfp8")[0])
+                else:
+                    outs.append(orc.gemv_fp4(x, m.payload, m.scales, float(m.glob[0]) if m.glob is not None else 1.0,
+                                             16 if m.kind == "nvfp4" else 32, 1, I, p.H)[0])
+            gb, ub = orc.bf16_round(outs[0]), orc.bf16_round(outs[1])
+            a = np.empty(I, np.uint16)
+            orc.oracle().orc_swiglu(orc.p(gb), orc.p(ub), I, p.limit, orc.p(a))
+            s = t * (K + 1) + j
+            act[s, :I] = a
+            m = mats[2]
+            arow = np.ascontiguousarray(a[None, :])
+            if m.kind in ("fp8", "mxfp8"):
+                down[s] = orc.gemv_fp8(arow, m.payload, m.scales, 1, p.H, I, m.rs, m.cs, True, m.kind == "mxfp8")[0]
+            else:
+                down[s] = orc.gemv_fp4(arow, m.payload, m.scales, float(m.glob[0]) if m.glob is not None else 1.0,
+                                       16 if m.kind == "nvfp4" else 32, 1, p.H, I)[0]
+            used[s] = True
+    return act, down, used
+
+
+def run_slot_path(p, d, ids, weights, use_order=True, shared_early=False):
+    """The reference's decode call order (src/models/glm/moe_layer.cpp:1415-1680) through the launchers."""
+    T, K = ids.shape
+    slots = T * (K + 1)
+    n_shared = p.shared_I if p.shared else 0
+    maxI = max(p.I, n_shared)
+    ids_d, w_d = dev(ids), dev(weights)
+    order_d = None
+    if use_order and T > 1:
+        order_d = dev_empty(slots, np.int32)
+        L.launch_moe_slot_order(ids_d, order_d, slots, K, p.E, None, shared_early)
+    act_d = dev_empty((slots, maxI), np.uint16)
+    act_d.zero_()
+    down_d = dev_empty((slots, p.H), np.float32)
+    down_d.zero_()
+    sh = d.sh
+    if p.kind == "fp8":
+        L.launch_moe_slot_gate_up_swiglu(d.x, p.H, ids_d, order_d, d.views, p.I, p.H, n_shared, p.H if n_shared else 0,
+                                         sh[0][0] if sh else None, sh[0][1] if sh else None, sh[1][0] if sh else None,
+                                         sh[1][1] if sh else None, act_d, maxI, slots, K, p.limit, None)
+        L.launch_moe_slot_down(act_d, maxI, ids_d, order_d, d.views, p.H, p.I, p.H if n_shared else 0, n_shared,
+                               sh[2][0] if sh else None, sh[2][1] if sh else None, down_d, p.H, slots, K, None)
+    else:
+        counter = dev(np.zeros(2, np.int32))
+        L.launch_moe_slot_gate_up_swiglu_fp4(d.x, p.H, ids_d, order_d, d.views, p.I, p.H, n_shared,
+                                             p.H if n_shared else 0, sh[0][0] if sh else None, sh[0][1] if sh else None,
+                                             sh[1][0] if sh else None, sh[1][1] if sh else None, act_d, maxI, slots, K,
+                                             p.limit, None, d.shared_view_base, d.fp4_group)
+        L.launch_moe_slot_down_fp4(act_d, maxI, ids_d, order_d, d.views, p.H, p.I, p.H if n_shared else 0, n_shared,
+                                   sh[2][0] if sh else None, sh[2][1] if sh else None, down_d, p.H, slots, K, None,
+                                   d.shared_view_base, d.fp4_group, 7, 7, counter)
+    out_d = dev_empty((T, p.H), np.uint16)
+    outf_d = dev_empty((T, p.H), np.float32)
+    if p.shared:
+        L.launch_moe_slot_accum(out_d, down_d, w_d, T, p.H, K, None)
+    else:
+        L.launch_moe_slot_accum_routed_f32(outf_d, down_d, w_d, T, p.H, K, None)
+        L.launch_moe_round_bf16(out_d, outf_d, T * p.H, None)
+    sync()
+    return host(act_d, np.uint16), host(down_d), host(out_d, np.uint16)
+
+
+def expert_budget(got_bits, raw, label):
+    """tests/cuda/glm_moe_test.cu:606-658."""
+    strict = hg.bf16_to_f32(orc.bf16_round(raw)).astype(np.float64)
+    rms = float(np.sqrt(np.mean(raw ** 2)))
+    floor_frac = 0.02 * rms / max(np.abs(strict).max(), 1e-30)
+    hard = orc.compare_bf16(got_bits, strict, 12.0, floor_frac)
+    soft = orc.compare_bf16(got_bits, strict, 4.0, floor_frac)
+    assert hard.mismatches == 0 and hard.nan_pattern_errors == 0, f"{label}: hard budget, max {hard.max_ulps:.1f} ulps"
+    assert soft.mismatches < 0.02 * soft.total, f"{label}: soft budget {soft.mismatches}/{soft.total}"
+    assert hard.l2_rel < 4e-3, f"{label}: l2 {hard.l2_rel}"
+    ns = orc.north_star_rel(got_bits, raw, floor_frac)
+    assert ns <= 2e-3, f"{label}: north-star rel {ns}"
+
+
+CASES = [
+    # E, H, I, K, T, kind, shared_kind, shared_I, limit
+    (16, 256, 128, 4, 1, "fp8", "fp8", 128, 10.0),
+    (16, 256, 128, 4, 5, "fp8", "fp8", 256, 10.0),
+    (12, 384, 96, 3, 3, "fp8", None, None, float("inf")),
+    (16, 256, 128, 4, 4, "nvfp4", "fp8", 128, 10.0),
+    (10, 512, 64, 2, 3, "nvfp4", "nvfp4", 64, 10.0),
+    (16, 1024, 256, 8, 2, "nvfp4", None, None, float("inf")),
+    (32, 1024, 256, 8, 4, "mxfp4", None, None, float("inf")),
+    (8, 512, 128, 2, 6, "mxfp4", "fp8", 384, 7.0),
+    (9, 256, 64, 3, 2, "mxfp4", "mxfp4", 64, 10.0),
+]
+
+
+@pytest.mark.parametrize("E,H,I,K,T,kind,shared,sI,limit", CASES)
+def test_slot_kernels_and_layer_vs_oracle(gpu, E, H, I, K, T, kind, shared, sI, limit):
+    p = moe_data.make_problem(E, H, I, K, T, kind, 300 + E + T, shared_kind=shared, shared_I=sI, limit=limit, std=0.05)
+    d = DeviceMoe(p)
+    mode = 1 if shared is None else 0
+    ids, w, _, _ = moe_data.orc_router(p, mode, 1.0 if mode == 1 else 2.5, True)
+    act, down, out = run_slot_path(p, d, ids, w)
+    o_act, o_down, used = oracle_stage_outputs(p, ids)
+    # gate/up + SwiGLU: the two dots carry the GEMV budget and SwiGLU one more ulp; compare act rows
+    a_rep = orc.compare_bf16(act[used], hg.bf16_to_f32(o_act[used]).astype(np.float64), 4.0, 2e-3)
+    assert a_rep.mismatches <= 0.001 * a_rep.total and a_rep.nan_pattern_errors == 0, f"act: {a_rep.mismatches}"
+    assert a_rep.l2_rel < 3e-3
+    # down from the DEVICE's own act rows (isolates the down kernel): strict fp32-vs-fp64 comparison
+    p2_down = np.zeros_like(o_down)
+    for s in np.nonzero(used)[0]:
+        t, j = divmod(int(s), K + 1)
+        m = (p.shared if j == K else p.experts[int(ids[t, j])])[2]
+        Iw = p.shared_I if j == K else p.I
+        arow = np.ascontiguousarray(act[s:s + 1, :Iw])
+        if m.kind == "fp8":
+            p2_down[s] = orc.gemv_fp8(arow, m.payload, m.scales, 1, p.H, Iw, m.rs, m.cs, True)[0]
+        else:
+            p2_down[s] = orc.gemv_fp4(arow, m.payload, m.scales, float(m.glob[0]) if m.glob is not None else 1.0,
+                                      16 if m.kind == "nvfp4" else 32, 1, p.H, Iw)[0]
+    d_rep = orc.compare_f32(down[used], p2_down[used], 0.05, 1e-4)   # 0.05 bf16 ulps ~ 2e-4 relative
+    assert d_rep.mismatches == 0, f"down: {d_rep.mismatches} beyond fp32 accumulation noise, max_rel {d_rep.max_rel}"
+    # full layer
+    raw, bits = moe_data.orc_forward(p, ids, w)
+    expert_budget(out, raw, f"layer {kind}/{shared} T{T}")
+    # execution order does not change any bit; a second run is bitwise identical
+    act2, down2, out2 = run_slot_path(p, d, ids, w, use_order=False)
+    assert np.array_equal(out, out2) and np.array_equal(down, down2) and np.array_equal(act, act2)
+    if shared and T > 1:
+        _, _, out3 = run_slot_path(p, d, ids, w, use_order=True, shared_early=True)
+        assert np.array_equal(out, out3)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "nvfp4", "mxfp4"])
+def test_slot_path_is_bitwise_the_grouped_path_and_the_dense_launcher(gpu, kind):
+    """tests/cuda/glm_moe_test.cu:942-1023, 1679-1752: slot == grouped == single-matrix launcher per row."""
+    E, H, I, K, T = 12, 512, 128, 3, 7
+    p = moe_data.make_problem(E, H, I, K, T, kind, 77, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    act, down, out = run_slot_path(p, d, ids, w)
+    # grouped path: segment -> gather -> grouped gate, up -> swiglu -> grouped down -> ordered accumulation
+    ids_d = dev(ids)
+    rows_d, sr_d, segs_d = dev_empty(T * K + T, np.int32), dev_empty(T * K, np.int32), dev_empty((E + 1, 3), np.int32)
+    L.launch_moe_segment(ids_d, T, K, E, rows_d, sr_d, segs_d, None)
+    xg = dev_empty((T * K, H), np.uint16)
+    L.launch_moe_gather_rows(d.x, rows_d, xg, T * K, H, None)
+    g_d, u_d, a_d = (dev_empty((T * K, I), np.uint16) for _ in range(3))
+    dn_d = dev_empty((T * K, H), np.float32)
+    max_rows = T
+    if kind == "fp8":
+        L.launch_moe_grouped_gemv_bf16(xg, H, segs_d, E, max_rows, 0, d.views, 0, g_d, I, I, H, None)
+        L.launch_moe_grouped_gemv_bf16(xg, H, segs_d, E, max_rows, 0, d.views, 1, u_d, I, I, H, None)
+    else:
+        L.launch_moe_grouped_gemv_fp4_bf16(xg, H, segs_d, E, max_rows, 0, d.views, 0, g_d, I, I, H, None, d.fp4_group)
+        L.launch_moe_grouped_gemv_fp4_bf16(xg, H, segs_d, E, max_rows, 3, d.views, 1, u_d, I, I, H, None, d.fp4_group)
+    L.launch_moe_swiglu_clamp(g_d, u_d, a_d, T * K * I, p.limit, None)
+    if kind == "fp8":
+        L.launch_moe_grouped_gemv_f32(a_d, I, segs_d, E, max_rows, 0, d.views, 2, dn_d, H, H, I, None)
+    else:
+        L.launch_moe_grouped_gemv_fp4_f32(a_d, I, segs_d, E, max_rows, 0, d.views, 2, dn_d, H, H, I, None, d.fp4_group)
+    out_g = dev_empty((T, H), np.uint16)
+    L.launch_moe_accum_ordered(out_g, dn_d, H, sr_d, ids_d, dev(w), -1, T, K, H, None)
+    sync()
+    slot_row = host(sr_d)
+    a_g, dn_g = host(a_d, np.uint16), host(dn_d)
+    for t in range(T):
+        for j in range(K):
+            s, r = t * (K + 1) + j, slot_row[t * K + j]
+            assert np.array_equal(act[s, :I], a_g[r]), "slot act row != grouped act row"
+            assert np.array_equal(down[s], dn_g[r]), "slot down row != grouped down row"
+    assert np.array_equal(out, host(out_g, np.uint16)), "slot layer output != grouped layer output"
+    # the single-matrix launcher on one expert's gate matrix, one token: bitwise the grouped row
+    e = int(ids[2, 1])
+    m = p.experts[e][0]
+    one = dev_empty((1, I), np.uint16)
+    xrow = dev(p.x[2:3])
+    if kind == "fp8":
+        L.launch_scale_gemm_bf16(xrow, H, dev(m.payload), dev(m.scales), one, 1, I, H, None)
+    else:
+        from gpu_util import fp4_matrix
+        wm = fp4_matrix(dev(m.payload), dev(m.scales), dev(m.glob) if m.glob is not None else None, I, H, d.fp4_group)
+        L.launch_fp4_gemv_bf16(xrow, H, wm, one, 1, I, H, None)
+    sync()
+    assert np.array_equal(host(one, np.uint16)[0], host(g_d, np.uint16)[slot_row[2 * K + 1]])
+
+
+def test_slot_launcher_argument_errors(gpu):
+    p = moe_data.make_problem(4, 256, 64, 2, 1, "nvfp4", 5, std=0.05)
+    d = DeviceMoe(p)
+    ids = dev(np.array([[0, 1]], np.int32))
+    act = dev_empty((3, 64), np.uint16)
+    out = dev_empty((3, 256), np.float32)
+    args = (d.x, 256, ids, None, d.views)
+    with pytest.raises(L.InvalidArgument):   # k outside the compiled set
+        L.launch_moe_slot_gate_up_swiglu_fp4(*args, 64, 96, 0, 0, None, None, None, None, act, 64, 3, 2, 10.0, None, -1, 16)
+    with pytest.raises(L.InvalidArgument):   # bad group
+        L.launch_moe_slot_gate_up_swiglu_fp4(*args, 64, 256, 0, 0, None, None, None, None, act, 64, 3, 2, 10.0, None, -1, 8)
+    with pytest.raises(L.InvalidArgument):   # act_stride below n
+        L.launch_moe_slot_gate_up_swiglu_fp4(*args, 64, 256, 0, 0, None, None, None, None, act, 32, 3, 2, 10.0, None, -1, 16)
+    with pytest.raises(L.InvalidArgument):   # n_shared without k_shared
+        L.launch_moe_slot_gate_up_swiglu_fp4(*args, 64, 256, 64, 0, None, None, None, None, act, 64, 3, 2, 10.0, None, -1, 16)
+    with pytest.raises(L.InvalidArgument):   # the counter pair is required
+        L.launch_moe_slot_down_fp4(act, 64, ids, None, d.views, 256, 64, 0, 0, None, None, out, 256, 3, 2, None, -1, 16, 7, 7, None)
+    with pytest.raises(L.InvalidArgument):   # fp8: k not a multiple of 16
+        L.launch_moe_slot_gate_up_swiglu(*args, 64, 250, 0, 0, None, None, None, None, act, 64, 3, 2, 10.0, None)
+    L.launch_moe_slot_gate_up_swiglu_fp4(*args, 64, 256, 0, 0, None, None, None, None, act, 64, 0, 2, 10.0, None, -1, 16)  # slots <= 0
