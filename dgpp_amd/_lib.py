@@ -121,6 +121,32 @@ SIGNATURES = {
     "dgpp_fill_zipf_routes": (None, [C.c_uint64, C.c_double, _I, _I, _I, _P]),
 }
 
+
+
+class MoeLayerDesc(C.Structure):
+    """include/dgpp_amd_layer.h: DgppMoeLayerDesc."""
+    _fields_ = [
+        ("cfg", MoeConfig), ("expert_format", C.c_int32), ("max_tokens", C.c_int32), ("views", C.c_void_p),
+        ("shared_in_table", C.c_int32), ("shared_inter", C.c_int32), ("sh_payload", C.c_void_p * 3),
+        ("sh_scales", C.c_void_p * 3), ("sh_rs", C.c_int32), ("sh_cs", C.c_int32), ("router_gate", C.c_void_p),
+        ("router_bias", C.c_void_p),
+    ]
+
+
+# include/dgpp_amd_layer.h
+LAYER_SIGNATURES = {
+    "dgpp_moe_layer_last_error": (C.c_char_p, []),
+    "dgpp_moe_layer_scratch_bytes": (C.c_size_t, [_P, _I, _I]),
+    "dgpp_moe_layer_create": (_I, [_P, _P]),
+    "dgpp_moe_layer_destroy": (None, [_P]),
+    "dgpp_moe_layer_enqueue_decode": (_I, [_P, _P, _Z, _P, _P, _I, _P]),
+    "dgpp_moe_layer_enqueue_decode_scores": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
+    "dgpp_moe_layer_enqueue_decode_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
+    "dgpp_moe_layer_enqueue_grouped_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
+    "dgpp_moe_layer_ids": (_P, [_P]),
+    "dgpp_moe_layer_weights": (_P, [_P]),
+}
+
 _lib = None
 
 
@@ -134,7 +160,7 @@ def load() -> C.CDLL:
             f"{LIB_PATH} is missing: build it with `python -m dgpp_amd.build` "
             "(there is no CPU fallback for the HIP path)")
     lib = C.CDLL(str(LIB_PATH))
-    for name, (res, args) in SIGNATURES.items():
+    for name, (res, args) in {**SIGNATURES, **LAYER_SIGNATURES}.items():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

@@ -27,6 +27,8 @@ HIP_SOURCES = [
     "capi.hip",
 ]
 HOST_SOURCES = ["host_codec.cpp"]
+# Host C++ that needs the HIP runtime headers (compiled by hipcc as plain host code).
+HIP_HOST_SOURCES = ["moe_layer.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed-FP32 instruction selection is switched off for all device code.
@@ -50,7 +52,7 @@ def _run(cmd: list[str]) -> None:
 def _stale(obj: Path, src: Path) -> bool:
     if not obj.exists():
         return True
-    newest = max(p.stat().st_mtime for p in list(CSRC.glob("*.hpp")) + [src, PKG.parent / "include" / "dgpp_amd.h"])
+    newest = max(p.stat().st_mtime for p in list(CSRC.glob("*.hpp")) + [src] + list((PKG.parent / "include").glob("*.h*")))
     return obj.stat().st_mtime < newest
 
 
@@ -65,6 +67,12 @@ def build(force: bool = True, jobs: int = 6) -> Path:
         objs.append(obj)
         if force or _stale(obj, src):
             tasks.append([HIPCC, *HIP_FLAGS, "-c", str(src), "-o", str(obj)])
+    for name in HIP_HOST_SOURCES:
+        src, obj = CSRC / name, BUILD / (name + ".o")
+        objs.append(obj)
+        if force or _stale(obj, src):
+            tasks.append([HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-c", str(src),
+                          "-o", str(obj)])
     for name in HOST_SOURCES:
         src, obj = CSRC / name, BUILD / (name + ".o")
         objs.append(obj)

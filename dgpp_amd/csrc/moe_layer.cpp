@@ -1,0 +1,337 @@
+#include "moe_layer.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <stdexcept>
+#include <string>
+
+#include "../../include/dgpp_amd_layer.h"
+
+namespace dgpp {
+namespace {
+
+void hip_ok(hipError_t e, const char* what) {
+  if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+
+// Buffer sizes in bytes, in the order they are carved (each rounded to 256).
+struct Layout {
+  size_t views, ids, weights, scores, biased, order, slot_act, slot_down, acc, counter, rows, slot_row, segs, gather,
+      gate, up, total;
+};
+Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t n_views) {
+  const size_t M = static_cast<size_t>(std::max(max_tokens, 0)), H = c.hidden, K = c.top_k, E = c.n_experts;
+  const size_t I = static_cast<size_t>(std::max(c.inter, shared_inter));
+  const size_t slots = M * (K + 1);
+  Layout l{};
+  l.views = align_up(n_views * sizeof(MoeExpertView));
+  l.ids = align_up(M * K * 4);
+  l.weights = align_up(M * K * 4);
+  l.scores = align_up(M * E * 4);
+  l.biased = align_up(M * E * 4);
+  l.order = align_up(slots * 4);
+  l.slot_act = align_up(slots * I * 2);
+  l.slot_down = align_up(slots * H * 4);
+  l.acc = align_up(M * H * 4);
+  l.counter = align_up(2 * sizeof(int));
+  l.rows = align_up(slots * 4);
+  l.slot_row = align_up(M * K * 4);
+  l.segs = align_up((E + 1) * sizeof(MoeSegment));
+  l.gather = align_up(slots * H * 2);
+  l.gate = align_up(slots * I * 2);
+  l.up = align_up(slots * I * 2);
+  l.total = l.views + l.ids + l.weights + l.scores + l.biased + l.order + l.slot_act + l.slot_down + l.acc + l.counter +
+            l.rows + l.slot_row + l.segs + l.gather + l.gate + l.up;
+  return l;
+}
+
+}  // namespace
+
+size_t GlmMoeLayer::scratch_bytes(const GlmMoeConfig& cfg, int max_tokens, int shared_inter) {
+  return layout_of(cfg, max_tokens, shared_inter, static_cast<size_t>(cfg.n_experts + 1) * 3).total;
+}
+
+GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, int max_tokens)
+    : cfg_(cfg), w_(w), max_tokens_(max_tokens) {
+  GlmMoeConfig::validate_config(cfg);
+  if (max_tokens <= 0) throw std::invalid_argument("GlmMoeLayer: max_tokens must be positive");
+  const size_t E = static_cast<size_t>(cfg.n_experts);
+  const bool fp4 = w.format != GlmExpertFormat::Fp8;
+  fp4_group_ = w.format == GlmExpertFormat::Mxfp4 ? kMxfp4Group : kFp4Group;
+  if (w.views.size() != (E + (w.shared_in_table ? 1 : 0)) * 3)
+    throw std::runtime_error("GlmMoeLayer: the expert view table must hold n_experts (+1 shared) triples");
+  // One format, one scale group and (FP8) one scale grid per matrix index across the table;
+  // NVFP4 matrices carry a global (src/models/glm/moe_layer.cpp:527-583).
+  auto grid_ok = [](int s) { return s >= 4 && s <= 7; };
+  for (size_t i = 0; i < w.views.size(); ++i) {
+    const MoeExpertView& v = w.views[i];
+    if (!v.payload) throw std::runtime_error("GlmMoeLayer: inconsistent routed expert matrices (null payload)");
+    if (fp4) {
+      if (!v.fp4_scales || v.fp4_group != fp4_group_ || (fp4_group_ == kFp4Group && !v.fp4_global))
+        throw std::runtime_error("GlmMoeLayer: inconsistent fp4 routed expert matrices (entry " + std::to_string(i) + ")");
+    } else {
+      const MoeExpertView& g = w.views[i % 3];
+      if (!v.scales || v.scale_shift_rows != g.scale_shift_rows || v.scale_shift_cols != g.scale_shift_cols ||
+          !grid_ok(v.scale_shift_rows) || !grid_ok(v.scale_shift_cols))
+        throw std::runtime_error("GlmMoeLayer: inconsistent or unsupported expert scale grid (entry " +
+                                 std::to_string(i) + ")");
+    }
+  }
+  if (w.shared_in_table) {
+    if (!fp4) throw std::runtime_error("GlmMoeLayer: a table-resident shared expert needs an fp4 table");
+    if (w.shared_inter != cfg.inter)
+      throw std::runtime_error(
+          "GlmMoeLayer: the NVFP4 shared expert's inter must equal the routed experts' (the slot kernels' K)");
+  } else if (w.shared_inter > 0) {
+    for (int i = 0; i < 3; ++i)
+      if (!w.sh_payload[i] || !w.sh_scales[i]) throw std::runtime_error("GlmMoeLayer: inconsistent shared matrices");
+  }
+  if ((cfg.n_shared_experts != 0) != (w.shared_inter > 0))
+    throw std::runtime_error("GlmMoeLayer: n_shared_experts does not match the shared weights");
+  max_inter_ = std::max(cfg.inter, w.shared_inter);
+
+  const Layout l = layout_of(cfg, max_tokens, w.shared_inter, w.views.size());
+  hip_ok(hipMalloc(&arena_, l.total), "GlmMoeLayer: hipMalloc");
+  uint8_t* p = static_cast<uint8_t*>(arena_);
+  auto carve = [&p](size_t bytes) {
+    uint8_t* q = p;
+    p += bytes;
+    return q;
+  };
+  d_views_ = reinterpret_cast<MoeExpertView*>(carve(l.views));
+  d_ids_ = reinterpret_cast<int32_t*>(carve(l.ids));
+  d_weights_ = reinterpret_cast<float*>(carve(l.weights));
+  d_scores_ = reinterpret_cast<float*>(carve(l.scores));
+  d_biased_ = reinterpret_cast<float*>(carve(l.biased));
+  d_order_ = reinterpret_cast<int32_t*>(carve(l.order));
+  d_slot_act_ = reinterpret_cast<uint16_t*>(carve(l.slot_act));
+  d_slot_down_ = reinterpret_cast<float*>(carve(l.slot_down));
+  d_acc_ = reinterpret_cast<float*>(carve(l.acc));
+  d_tile_counter_ = reinterpret_cast<int*>(carve(l.counter));
+  d_rows_ = reinterpret_cast<int32_t*>(carve(l.rows));
+  d_slot_row_ = reinterpret_cast<int32_t*>(carve(l.slot_row));
+  d_segs_ = reinterpret_cast<MoeSegment*>(carve(l.segs));
+  d_gather_ = reinterpret_cast<uint16_t*>(carve(l.gather));
+  d_gate_ = reinterpret_cast<uint16_t*>(carve(l.gate));
+  d_up_ = reinterpret_cast<uint16_t*>(carve(l.up));
+  // The device expert table is uploaded once (the reference's capture form prepares a per-binding
+  // device table once too, src/models/glm/moe_layer.cpp:364-396); the counter pair is zero at rest.
+  hip_ok(hipMemcpy(d_views_, w.views.data(), w.views.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
+         "GlmMoeLayer: table upload");
+  hip_ok(hipMemset(d_tile_counter_, 0, 2 * sizeof(int)), "GlmMoeLayer: counter");
+}
+
+GlmMoeLayer::~GlmMoeLayer() {
+  if (arena_) (void)hipFree(arena_);
+}
+
+void GlmMoeLayer::check_tokens(int tokens) const {
+  if (tokens > max_tokens_) throw std::invalid_argument("GlmMoeLayer: tokens exceed the layer's max_tokens");
+}
+
+void GlmMoeLayer::enqueue_decode(const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32, int tokens,
+                                 hipStream_t stream) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  if (!w_.router_gate) throw std::invalid_argument("GlmMoeLayer: the router gate is not bound");
+  launch_moe_router(x, w_.router_gate, w_.router_bias, d_ids_, d_weights_, d_scores_, d_biased_, cfg_, tokens, stream);
+  expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream);
+}
+
+void GlmMoeLayer::enqueue_decode_scores(const uint16_t* x, size_t x_stride, const float* scores, const float* biased,
+                                        uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  launch_moe_router_select(scores, biased, d_ids_, d_weights_, cfg_, tokens, stream);
+  expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream);
+}
+
+void GlmMoeLayer::enqueue_decode_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                                        uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  expert_chain_slots(x, x_stride, ids, weights, out_bf16, out_f32, tokens, stream);
+}
+
+// Steps 4-7 of the reference's decode call order (src/models/glm/moe_layer.cpp:1555-1677).
+void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                                     uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
+  const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter;
+  const int slots = tokens * (K + 1);
+  if (slots > 1024 && tokens > 1)
+    throw std::invalid_argument("GlmMoeLayer: the decode-slot path takes at most 1024 slots; use the grouped path");
+  const int32_t* order = nullptr;
+  if (tokens > 1) {
+    launch_moe_slot_order(ids, d_order_, slots, K, cfg_.n_experts, stream, cfg_.shared_slots_early);
+    order = d_order_;
+  }
+  const bool sh_args = has_shared() && !w_.shared_in_table;
+  const int n_sh = has_shared() ? w_.shared_inter : 0;
+  const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
+  if (w_.format == GlmExpertFormat::Fp8) {
+    launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
+                                   w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
+                                   K, cfg_.swiglu_limit, stream, w_.sh_rs, w_.sh_cs);
+    launch_moe_slot_down(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
+                         n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, stream, w_.sh_rs, w_.sh_cs);
+  } else {
+    const int base = w_.shared_in_table ? cfg_.n_experts * 3 : -1;
+    launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
+                                       sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
+                                       sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
+                                       d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, stream, base, fp4_group_,
+                                       w_.sh_rs, w_.sh_cs);
+    launch_moe_slot_down_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
+                             has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
+                             sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, stream, base, fp4_group_,
+                             w_.sh_rs, w_.sh_cs, d_tile_counter_);
+  }
+  if (has_shared()) {
+    if (out_f32) {
+      // The shared chain, unrounded: the ordered form over the slot layout's rows.
+      throw std::invalid_argument("GlmMoeLayer: an unrounded output with a shared expert is not a decode form");
+    }
+    launch_moe_slot_accum(out_bf16, d_slot_down_, weights, tokens, H, K, stream);
+  } else if (out_f32) {
+    launch_moe_slot_accum_routed_f32(out_f32, d_slot_down_, weights, tokens, H, K, stream);
+  } else {
+    launch_moe_slot_accum_routed_f32(d_acc_, d_slot_down_, weights, tokens, H, K, stream);
+    launch_moe_round_bf16(out_bf16, d_acc_, static_cast<int64_t>(tokens) * H, stream);
+  }
+}
+
+// The device-segmented grouped path (src/models/glm/moe_layer.cpp:906-934, :1054-1379 GEMV form).
+void GlmMoeLayer::enqueue_grouped_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                                         uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  if (has_shared())
+    throw std::invalid_argument("GlmMoeLayer: the grouped path here covers the routed experts (no shared segment)");
+  if (x_stride != static_cast<size_t>(cfg_.hidden))
+    throw std::invalid_argument("GlmMoeLayer: the grouped path gathers dense [tokens, hidden] rows");
+  const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter, E = cfg_.n_experts;
+  const int tk = tokens * K;
+  launch_moe_segment(ids, tokens, K, E, d_rows_, d_slot_row_, d_segs_, stream);
+  launch_moe_gather_rows(x, d_rows_, d_gather_, tk, H, stream);
+  const int max_rows = tokens;  // a segment holds at most one row per token
+  if (w_.format == GlmExpertFormat::Fp8) {
+    launch_moe_grouped_gemv_bf16(d_gather_, H, d_segs_, E, max_rows, 0, d_views_, 0, d_gate_, I, I, H, stream);
+    launch_moe_grouped_gemv_bf16(d_gather_, H, d_segs_, E, max_rows, 0, d_views_, 1, d_up_, I, I, H, stream);
+  } else {
+    launch_moe_grouped_gemv_fp4_bf16(d_gather_, H, d_segs_, E, max_rows, 0, d_views_, 0, d_gate_, I, I, H, stream,
+                                     fp4_group_);
+    launch_moe_grouped_gemv_fp4_bf16(d_gather_, H, d_segs_, E, max_rows, 0, d_views_, 1, d_up_, I, I, H, stream,
+                                     fp4_group_);
+  }
+  launch_moe_swiglu_clamp(d_gate_, d_up_, d_slot_act_, static_cast<int64_t>(tk) * I, cfg_.swiglu_limit, stream);
+  if (w_.format == GlmExpertFormat::Fp8)
+    launch_moe_grouped_gemv_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream);
+  else
+    launch_moe_grouped_gemv_fp4_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream,
+                                    fp4_group_);
+  if (out_f32)
+    launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+  else
+    launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+}
+
+}  // namespace dgpp
+
+// ---- C wrappers -------------------------------------------------------------------------------------------
+namespace {
+thread_local std::string g_layer_error;
+template <class Fn>
+int guarded(Fn fn) {
+  try {
+    fn();
+    return DGPP_OK;
+  } catch (const std::invalid_argument& e) {
+    g_layer_error = e.what();
+    return DGPP_INVALID_ARGUMENT;
+  } catch (const std::exception& e) {
+    g_layer_error = e.what();
+    return DGPP_RUNTIME_ERROR;
+  }
+}
+dgpp::GlmMoeConfig cpp_config(const DgppMoeConfig& c) {
+  dgpp::GlmMoeConfig g;
+  g.hidden = c.hidden;
+  g.inter = c.inter;
+  g.n_experts = c.n_experts;
+  g.top_k = c.top_k;
+  g.n_shared_experts = c.n_shared_experts;
+  g.routed_scaling_factor = c.routed_scaling_factor;
+  g.norm_topk_prob = c.norm_topk_prob != 0;
+  g.swiglu_limit = c.swiglu_limit;
+  g.router_mode = static_cast<dgpp::MoeRouterMode>(c.router_mode);
+  return g;
+}
+}  // namespace
+
+struct DgppMoeLayer {
+  dgpp::GlmMoeLayer impl;
+  DgppMoeLayer(const dgpp::GlmMoeConfig& c, const dgpp::GlmMoeLayerWeights& w, int m) : impl(c, w, m) {}
+};
+
+extern "C" {
+
+const char* dgpp_moe_layer_last_error(void) { return g_layer_error.c_str(); }
+
+size_t dgpp_moe_layer_scratch_bytes(const DgppMoeConfig* cfg, int max_tokens, int shared_inter) {
+  return dgpp::GlmMoeLayer::scratch_bytes(cpp_config(*cfg), max_tokens, shared_inter);
+}
+
+int dgpp_moe_layer_create(const DgppMoeLayerDesc* d, DgppMoeLayer** out) {
+  return guarded([&] {
+    if (!d || !out || !d->views) throw std::invalid_argument("moe_layer_create: null pointer");
+    dgpp::GlmMoeLayerWeights w;
+    w.format = static_cast<dgpp::GlmExpertFormat>(d->expert_format);
+    const size_t n = (static_cast<size_t>(d->cfg.n_experts) + (d->shared_in_table ? 1 : 0)) * 3;
+    w.views.assign(d->views, d->views + n);
+    w.shared_in_table = d->shared_in_table != 0;
+    w.shared_inter = d->shared_inter;
+    for (int i = 0; i < 3; ++i) {
+      w.sh_payload[i] = d->sh_payload[i];
+      w.sh_scales[i] = d->sh_scales[i];
+    }
+    w.sh_rs = d->sh_rs;
+    w.sh_cs = d->sh_cs;
+    w.router_gate = d->router_gate;
+    w.router_bias = d->router_bias;
+    *out = new DgppMoeLayer(cpp_config(d->cfg), w, d->max_tokens);
+  });
+}
+
+void dgpp_moe_layer_destroy(DgppMoeLayer* layer) { delete layer; }
+
+int dgpp_moe_layer_enqueue_decode(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, uint16_t* out_bf16,
+                                  float* out_f32, int tokens, void* stream) {
+  return guarded([&] { l->impl.enqueue_decode(x, x_stride, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream)); });
+}
+int dgpp_moe_layer_enqueue_decode_scores(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, const float* scores,
+                                         const float* biased, uint16_t* out_bf16, float* out_f32, int tokens,
+                                         void* stream) {
+  return guarded([&] {
+    l->impl.enqueue_decode_scores(x, x_stride, scores, biased, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
+  });
+}
+int dgpp_moe_layer_enqueue_decode_routed(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                         const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
+                                         void* stream) {
+  return guarded([&] {
+    l->impl.enqueue_decode_routed(x, x_stride, ids, weights, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
+  });
+}
+int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                          const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
+                                          void* stream) {
+  return guarded([&] {
+    l->impl.enqueue_grouped_routed(x, x_stride, ids, weights, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
+  });
+}
+const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* l) { return l->impl.ids(); }
+const float* dgpp_moe_layer_weights(const DgppMoeLayer* l) { return l->impl.weights(); }
+
+}  // extern "C"

@@ -1,0 +1,86 @@
+// Host-side driver of one quantized MoE layer over the launcher surface (include/dgpp_amd.hpp):
+// the counterpart of the reference's GlmMoeLayer (src/models/glm/moe_layer.hpp:50). It owns the
+// layer's device scratch and device expert table, checks the weight geometry the way the
+// reference's binding does (src/models/glm/moe_layer.cpp:527-583) and issues the reference's call
+// order for the sync-free decode path (:1415-1680) and the device-segmented grouped path
+// (:775-817, :906-934). All work is enqueued on the caller's stream; nothing synchronises.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <vector>
+
+#include "../../include/dgpp_amd.hpp"
+
+namespace dgpp {
+
+enum class GlmExpertFormat { Fp8 = 0, Nvfp4 = 1, Mxfp4 = 2 };
+
+struct GlmMoeLayerWeights {
+  GlmExpertFormat format = GlmExpertFormat::Fp8;
+  std::vector<MoeExpertView> views;   // [E * 3] (+3 when the shared expert is an FP4 table entry)
+  bool shared_in_table = false;
+  int shared_inter = 0;               // 0: no shared expert
+  const uint8_t* sh_payload[3] = {nullptr, nullptr, nullptr};
+  const float* sh_scales[3] = {nullptr, nullptr, nullptr};
+  int sh_rs = 7, sh_cs = 7;
+  const uint16_t* router_gate = nullptr;
+  const float* router_bias = nullptr;
+};
+
+class GlmMoeLayer {
+ public:
+  GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, int max_tokens);
+  ~GlmMoeLayer();
+  GlmMoeLayer(const GlmMoeLayer&) = delete;
+  GlmMoeLayer& operator=(const GlmMoeLayer&) = delete;
+
+  static size_t scratch_bytes(const GlmMoeConfig& cfg, int max_tokens, int shared_inter);
+
+  // out_f32 non-null: the unrounded chain goes there and out_bf16 is not written.
+  void enqueue_decode(const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32, int tokens,
+                      hipStream_t stream);
+  void enqueue_decode_scores(const uint16_t* x, size_t x_stride, const float* scores, const float* biased,
+                             uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
+  void enqueue_decode_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                             uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
+  void enqueue_grouped_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                              uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
+
+  const int32_t* ids() const { return d_ids_; }
+  const float* weights() const { return d_weights_; }
+  bool has_shared() const { return w_.shared_inter > 0; }
+
+ private:
+  void check_tokens(int tokens) const;
+  void expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                          uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
+
+  GlmMoeConfig cfg_;
+  GlmMoeLayerWeights w_;
+  int max_tokens_ = 0;
+  int fp4_group_ = 16;
+  int max_inter_ = 0;
+  // One device allocation carved into the buffers below.
+  void* arena_ = nullptr;
+  MoeExpertView* d_views_ = nullptr;
+  int32_t* d_ids_ = nullptr;
+  float* d_weights_ = nullptr;
+  float* d_scores_ = nullptr;
+  float* d_biased_ = nullptr;
+  int32_t* d_order_ = nullptr;
+  uint16_t* d_slot_act_ = nullptr;   // [slots, max_inter]
+  float* d_slot_down_ = nullptr;     // [slots, hidden]
+  float* d_acc_ = nullptr;           // [tokens, hidden]
+  int* d_tile_counter_ = nullptr;    // [2]
+  int32_t* d_rows_ = nullptr;        // grouped path
+  int32_t* d_slot_row_ = nullptr;
+  MoeSegment* d_segs_ = nullptr;
+  uint16_t* d_gather_ = nullptr;     // [rows_total, hidden]
+  uint16_t* d_gate_ = nullptr;       // [rows_total, max_inter]
+  uint16_t* d_up_ = nullptr;
+};
+
+}  // namespace dgpp

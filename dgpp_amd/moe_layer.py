@@ -1,0 +1,84 @@
+"""Python handle on the C++ host layer driver (dgpp_amd/csrc/moe_layer.cpp, include/dgpp_amd_layer.h),
+the counterpart of the reference's GlmMoeLayer (src/models/glm/moe_layer.hpp:50). Tests and the
+benchmark drive the decode path through it; pointers are torch tensors / ints as in dgpp_amd.launch."""
+from __future__ import annotations
+
+import ctypes as C
+
+from . import _lib
+from ._lib import MoeConfig, MoeExpertView, MoeLayerDesc
+from .launch import InvalidArgument, _p, _stream
+
+EXPERTS_FP8, EXPERTS_NVFP4, EXPERTS_MXFP4 = 0, 1, 2
+
+
+def _check(rc: int) -> None:
+    if rc == _lib.OK:
+        return
+    msg = _lib.load().dgpp_moe_layer_last_error().decode()
+    if rc == _lib.INVALID_ARGUMENT:
+        raise InvalidArgument(msg)
+    raise RuntimeError(msg)
+
+
+def scratch_bytes(cfg: MoeConfig, max_tokens: int, shared_inter: int = 0) -> int:
+    return _lib.load().dgpp_moe_layer_scratch_bytes(C.addressof(cfg), max_tokens, shared_inter)
+
+
+class MoeLayer:
+    """Owns the layer's device scratch and expert table; every enqueue_* is asynchronous on `stream`."""
+
+    def __init__(self, cfg: MoeConfig, expert_format: int, views: list[MoeExpertView], max_tokens: int, *,
+                 shared_in_table: bool = False, shared_inter: int = 0, sh_payload=(None, None, None),
+                 sh_scales=(None, None, None), sh_rs: int = 7, sh_cs: int = 7, router_gate=None, router_bias=None):
+        self._lib = _lib.load()
+        arr = (MoeExpertView * len(views))(*views)
+        d = MoeLayerDesc()
+        d.cfg = cfg
+        d.expert_format = expert_format
+        d.max_tokens = max_tokens
+        d.views = C.addressof(arr)
+        d.shared_in_table = 1 if shared_in_table else 0
+        d.shared_inter = shared_inter
+        for i in range(3):
+            d.sh_payload[i] = _p(sh_payload[i])
+            d.sh_scales[i] = _p(sh_scales[i])
+        d.sh_rs, d.sh_cs = sh_rs, sh_cs
+        d.router_gate = _p(router_gate)
+        d.router_bias = _p(router_bias)
+        self.cfg = cfg
+        self._keep = (sh_payload, sh_scales, router_gate, router_bias)
+        handle = C.c_void_p()
+        _check(self._lib.dgpp_moe_layer_create(C.addressof(d), C.addressof(handle)))
+        self._h = handle
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._lib.dgpp_moe_layer_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def enqueue_decode(self, x, x_stride, out_bf16, tokens, stream=None, out_f32=None):
+        _check(self._lib.dgpp_moe_layer_enqueue_decode(self._h, _p(x), x_stride, _p(out_bf16), _p(out_f32), tokens,
+                                                       _stream(stream)))
+
+    def enqueue_decode_scores(self, x, x_stride, scores, biased, out_bf16, tokens, stream=None, out_f32=None):
+        _check(self._lib.dgpp_moe_layer_enqueue_decode_scores(self._h, _p(x), x_stride, _p(scores), _p(biased),
+                                                              _p(out_bf16), _p(out_f32), tokens, _stream(stream)))
+
+    def enqueue_decode_routed(self, x, x_stride, ids, weights, out_bf16, tokens, stream=None, out_f32=None):
+        _check(self._lib.dgpp_moe_layer_enqueue_decode_routed(self._h, _p(x), x_stride, _p(ids), _p(weights),
+                                                              _p(out_bf16), _p(out_f32), tokens, _stream(stream)))
+
+    def enqueue_grouped_routed(self, x, x_stride, ids, weights, out_bf16, tokens, stream=None, out_f32=None):
+        _check(self._lib.dgpp_moe_layer_enqueue_grouped_routed(self._h, _p(x), x_stride, _p(ids), _p(weights),
+                                                               _p(out_bf16), _p(out_f32), tokens, _stream(stream)))
+
+    @property
+    def ids_ptr(self) -> int:
+        return self._lib.dgpp_moe_layer_ids(self._h)
+
+    @property
+    def weights_ptr(self) -> int:
+        return self._lib.dgpp_moe_layer_weights(self._h)

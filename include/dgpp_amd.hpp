@@ -1,0 +1,314 @@
+// C++ face of the C ABI (dgpp_amd.h): the reference's `dgpp::launch_*` free functions with their
+// own names, argument order, default arguments and error behaviour (std::invalid_argument for a
+// refused call, std::runtime_error for a failed runtime call), so host code written against
+// src/kernels/glm_moe_launch.hpp, fp4_gemv.hpp, scale_gemm.hpp, fp8_dequant.hpp and minimax.hpp
+// compiles against this header with `cudaStream_t` replaced by `hipStream_t`. Header-only.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "dgpp_amd.h"
+
+namespace dgpp {
+
+using MoeExpertView = DgppMoeExpertView;   // src/models/glm/moe.hpp:232
+using MoeSegment = DgppMoeSegment;         // src/kernels/glm_moe_launch.hpp:67
+using MoeTile = DgppMoeTile;               // src/kernels/glm_moe_launch.hpp:151
+using GlmFp4Matrix = DgppFp4Matrix;        // src/models/quant_matrix.hpp:117
+using Fp8GemvProblem = DgppFp8GemvProblem; // src/kernels/scale_gemm.hpp:85
+
+constexpr int kFp4Group = 16;
+constexpr int kMxfp4Group = 32;
+
+// src/models/quant_matrix.hpp:16-47 (the fields the path reads).
+struct GlmQuantMatrix {
+  const uint8_t* payload = nullptr;
+  const float* scales = nullptr;
+  const uint8_t* scales_e8m0 = nullptr;
+  int64_t rows = 0;
+  int64_t cols = 0;
+  int scale_block_rows = 128;
+  int scale_block_cols = 128;
+};
+
+enum class MoeRouterMode { SigmoidBias = 0, SoftmaxTopk = 1, SqrtSoftplusBias = 2 };
+
+// src/models/glm/moe.hpp:51-134 (the fields the path reads).
+struct GlmMoeConfig {
+  int hidden = 4096;
+  int inter = 2048;
+  int n_experts = 288;
+  int top_k = 8;
+  int n_shared_experts = 1;
+  float routed_scaling_factor = 2.5f;
+  bool norm_topk_prob = true;
+  float swiglu_limit = 10.0f;
+  bool shared_slots_early = false;
+  MoeRouterMode router_mode = MoeRouterMode::SigmoidBias;
+
+  DgppMoeConfig c_config() const {
+    return DgppMoeConfig{hidden, inter, n_experts, top_k, n_shared_experts, routed_scaling_factor,
+                         norm_topk_prob ? 1 : 0, swiglu_limit, static_cast<int32_t>(router_mode)};
+  }
+  static void validate_config(const GlmMoeConfig& c);
+};
+
+namespace detail {
+inline void check(int rc) {
+  if (rc == DGPP_OK) return;
+  const std::string msg = dgpp_last_error();
+  if (rc == DGPP_INVALID_ARGUMENT) throw std::invalid_argument(msg);
+  throw std::runtime_error(msg);
+}
+inline int shift_of(int block) {
+  int s = 0;
+  while ((1 << s) < block) ++s;
+  return s;
+}
+}  // namespace detail
+
+inline void GlmMoeConfig::validate_config(const GlmMoeConfig& c) {
+  const DgppMoeConfig cc = c.c_config();
+  detail::check(dgpp_moe_config_validate(&cc));
+}
+
+// MoeExpertView::of (src/models/glm/moe.hpp:248-256)
+inline MoeExpertView expert_view_of(const GlmQuantMatrix& m) {
+  MoeExpertView v{};
+  v.payload = m.payload;
+  v.scales = m.scales;
+  v.scale_shift_rows = detail::shift_of(m.scale_block_rows);
+  v.scale_shift_cols = detail::shift_of(m.scale_block_cols);
+  v.fp4_group = kFp4Group;
+  return v;
+}
+inline MoeExpertView expert_view_of(const GlmFp4Matrix& m) {
+  MoeExpertView v{};
+  v.payload = m.payload;
+  v.fp4_scales = m.scales;
+  v.fp4_global = m.global_scale;
+  v.scale_shift_rows = 7;
+  v.scale_shift_cols = 7;
+  v.fp4_group = m.scale_group;
+  return v;
+}
+
+// ---- src/kernels/glm_moe_launch.hpp ---------------------------------------------------------------
+inline void launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const float* bias, int32_t* ids,
+                              float* weights, float* scores, float* biased, const GlmMoeConfig& cfg, int tokens,
+                              hipStream_t stream, int* counters = nullptr, bool allow_tiled = true) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_router(hidden, gate, bias, ids, weights, scores, biased, &c, tokens, stream, counters,
+                                       allow_tiled ? 1 : 0));
+}
+// The selection half alone (src/kernels/glm_moe.cu:314-329).
+inline void launch_moe_router_select(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                     const GlmMoeConfig& cfg, int tokens, hipStream_t stream) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_router_select(scores, biased, ids, weights, &c, tokens, stream));
+}
+inline void launch_moe_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, float limit,
+                                    hipStream_t stream) {
+  detail::check(dgpp_launch_moe_swiglu_clamp(gate, up, out, n, limit, stream));
+}
+inline void launch_moe_gather_rows(const uint16_t* src, const int32_t* rows, uint16_t* dst, int n_rows, int hidden,
+                                   hipStream_t stream) {
+  detail::check(dgpp_launch_moe_gather_rows(src, rows, dst, n_rows, hidden, stream));
+}
+inline void launch_moe_accum(float* acc, const float* y, const int32_t* rows, const float* row_weights, int n_rows,
+                             int hidden, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_accum(acc, y, rows, row_weights, n_rows, hidden, stream));
+}
+inline void launch_moe_round_bf16(uint16_t* out, const float* acc, int64_t n, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_round_bf16(out, acc, n, stream));
+}
+inline void launch_moe_segment(const int32_t* ids, int tokens, int top_k, int n_experts, int32_t* rows,
+                               int32_t* slot_row, MoeSegment* segs, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_segment(ids, tokens, top_k, n_experts, rows, slot_row, segs, stream));
+}
+inline int moe_tile_list_capacity(int n_segs, int total_rows, int tile_rows) {
+  return dgpp_moe_tile_list_capacity(n_segs, total_rows, tile_rows);
+}
+inline void launch_moe_tile_list(const MoeSegment* segs, int n_segs, int tile_rows, MoeTile* tiles, int32_t* count,
+                                 hipStream_t stream) {
+  detail::check(dgpp_launch_moe_tile_list(segs, n_segs, tile_rows, tiles, count, stream));
+}
+inline int moe_run_groups_max(int slots) { return dgpp_moe_run_groups_max(slots); }
+inline void launch_moe_slot_order(const int32_t* ids, int32_t* order, int slots, int top_k, int n_experts,
+                                  hipStream_t stream, bool shared_early = false, int32_t* runs = nullptr) {
+  detail::check(dgpp_launch_moe_slot_order(ids, order, slots, top_k, n_experts, stream, shared_early ? 1 : 0, runs));
+}
+inline void launch_moe_accum_ordered(uint16_t* out, const float* down, size_t down_stride, const int32_t* slot_row,
+                                     const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens,
+                                     int top_k, int hidden, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_accum_ordered(out, down, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens,
+                                              top_k, hidden, stream));
+}
+inline void launch_moe_accum_ordered_f32(float* out, const float* down, size_t down_stride, const int32_t* slot_row,
+                                         const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens,
+                                         int top_k, int hidden, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_accum_ordered_f32(out, down, down_stride, slot_row, slot_ids, slot_w, shared_row0,
+                                                  tokens, top_k, hidden, stream));
+}
+inline void launch_moe_slot_accum(uint16_t* out, const float* contrib, const float* weights, int tokens, int hidden,
+                                  int top_k, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_slot_accum(out, contrib, weights, tokens, hidden, top_k, stream));
+}
+inline void launch_moe_slot_accum_routed_f32(float* out, const float* contrib, const float* weights, int tokens,
+                                             int hidden, int top_k, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_slot_accum_routed_f32(out, contrib, weights, tokens, hidden, top_k, stream));
+}
+inline void launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                                           const MoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                           int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                           const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                           int act_stride, int slots, int top_k, float limit, hipStream_t stream,
+                                           int sh_rs = 7, int sh_cs = 7) {
+  detail::check(dgpp_launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, views, n_routed, k_routed, n_shared,
+                                                    k_shared, sh_gate_payload, sh_gate_scales, sh_up_payload,
+                                                    sh_up_scales, act, act_stride, slots, top_k, limit, stream, sh_rs,
+                                                    sh_cs));
+}
+inline void launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                 const MoeExpertView* views, int n_routed, int k_routed, int n_shared, int k_shared,
+                                 const uint8_t* sh_payload, const float* sh_scales, float* out, int out_stride,
+                                 int slots, int top_k, hipStream_t stream, int sh_rs = 7, int sh_cs = 7) {
+  detail::check(dgpp_launch_moe_slot_down(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                          sh_payload, sh_scales, out, out_stride, slots, top_k, stream, sh_rs, sh_cs));
+}
+inline void launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                               const int32_t* order, const MoeExpertView* views, int n_routed,
+                                               int k_routed, int n_shared, int k_shared,
+                                               const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                               const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                               int act_stride, int slots, int top_k, float limit, hipStream_t stream,
+                                               int shared_view_base = -1, int fp4_group = 16, int sh_rs = 7,
+                                               int sh_cs = 7) {
+  detail::check(dgpp_launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, views, n_routed, k_routed, n_shared,
+                                                        k_shared, sh_gate_payload, sh_gate_scales, sh_up_payload,
+                                                        sh_up_scales, act, act_stride, slots, top_k, limit, stream,
+                                                        shared_view_base, fp4_group, sh_rs, sh_cs));
+}
+inline void launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                     const MoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                     int k_shared, const uint8_t* sh_payload, const float* sh_scales, float* out,
+                                     int out_stride, int slots, int top_k, hipStream_t stream,
+                                     int shared_view_base = -1, int fp4_group = 16, int sh_rs = 7, int sh_cs = 7,
+                                     int* tile_counter = nullptr) {
+  detail::check(dgpp_launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_routed, n_shared,
+                                              k_shared, sh_payload, sh_scales, out, out_stride, slots, top_k, stream,
+                                              shared_view_base, fp4_group, sh_rs, sh_cs, tile_counter));
+}
+inline void launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                         int max_rows, int rows_per_block, const MoeExpertView* views, int which,
+                                         uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_grouped_gemv_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which,
+                                                  out, out_stride, n, k, stream));
+}
+inline void launch_moe_grouped_gemv_f32(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                        int max_rows, int rows_per_block, const MoeExpertView* views, int which,
+                                        float* out, size_t out_stride, int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_grouped_gemv_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which,
+                                                 out, out_stride, n, k, stream));
+}
+inline void launch_moe_grouped_gemv_fp4_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                             int max_rows, int rows_per_block, const MoeExpertView* views, int which,
+                                             uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream,
+                                             int fp4_group = 16) {
+  detail::check(dgpp_launch_moe_grouped_gemv_fp4_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
+                                                      which, out, out_stride, n, k, stream, fp4_group));
+}
+inline void launch_moe_grouped_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                            int max_rows, int rows_per_block, const MoeExpertView* views, int which,
+                                            float* out, size_t out_stride, int n, int k, hipStream_t stream,
+                                            int fp4_group = 16) {
+  detail::check(dgpp_launch_moe_grouped_gemv_fp4_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
+                                                     which, out, out_stride, n, k, stream, fp4_group));
+}
+
+// ---- src/kernels/minimax.hpp:11 -----------------------------------------------------------------------
+inline void minimax_compact_segments(const MoeSegment* input, MoeSegment* output, int experts, int capacity,
+                                     hipStream_t stream) {
+  detail::check(dgpp_minimax_compact_segments(input, output, experts, capacity, stream));
+}
+
+// ---- src/kernels/fp4_gemv.hpp ---------------------------------------------------------------------------
+inline void launch_fp4_gemv_bf16(const uint16_t* act, size_t act_row_stride_elems, const GlmFp4Matrix& w,
+                                 uint16_t* out, int m, int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_fp4_gemv_bf16(act, act_row_stride_elems, &w, out, m, n, k, stream));
+}
+inline void launch_fp4_gemv_f32(const uint16_t* act, size_t act_row_stride_elems, const GlmFp4Matrix& w, float* out,
+                                int m, int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_fp4_gemv_f32(act, act_row_stride_elems, &w, out, m, n, k, stream));
+}
+inline bool fp4_gemv_accepts(const GlmFp4Matrix& w) { return dgpp_fp4_gemv_accepts(&w) != 0; }
+
+// ---- src/kernels/scale_gemm.hpp ---------------------------------------------------------------------------
+inline void launch_scale_gemm_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                   const float* w_scales, uint16_t* out, int m, int n, int k, hipStream_t stream,
+                                   size_t out_row_stride_elems = 0, int mma_from_rows = 0, void* ws = nullptr,
+                                   size_t ws_bytes = 0) {
+  detail::check(dgpp_launch_scale_gemm_bf16(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                                            out_row_stride_elems, mma_from_rows, ws, ws_bytes));
+}
+inline void launch_scale_gemm_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                  const float* w_scales, float* out, int m, int n, int k, hipStream_t stream,
+                                  size_t out_row_stride_elems = 0, int mma_from_rows = 0, bool last_row_only = false,
+                                  void* ws = nullptr, size_t ws_bytes = 0, int compact_row = -1) {
+  detail::check(dgpp_launch_scale_gemm_f32(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                                           out_row_stride_elems, mma_from_rows, last_row_only ? 1 : 0, ws, ws_bytes,
+                                           compact_row));
+}
+inline void launch_scale_gemm_grid_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                        const float* w_scales, uint16_t* out, int m, int n, int k, hipStream_t stream,
+                                        size_t out_row_stride_elems, int rs, int cs, bool decode_mma = false,
+                                        void* ws = nullptr, size_t ws_bytes = 0, bool prefill_tile = false) {
+  detail::check(dgpp_launch_scale_gemm_grid_bf16(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                                                 out_row_stride_elems, rs, cs, decode_mma, ws, ws_bytes, prefill_tile));
+}
+inline void launch_scale_gemm_grid_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                       const float* w_scales, float* out, int m, int n, int k, hipStream_t stream,
+                                       size_t out_row_stride_elems, int rs, int cs, bool decode_mma = false,
+                                       void* ws = nullptr, size_t ws_bytes = 0, bool prefill_tile = false) {
+  detail::check(dgpp_launch_scale_gemm_grid_f32(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream,
+                                                out_row_stride_elems, rs, cs, decode_mma, ws, ws_bytes, prefill_tile));
+}
+inline void launch_scale_gemm_grid_e8m0_bf16(const uint16_t* act, size_t act_row_stride_elems,
+                                             const uint8_t* w_payload, const uint8_t* w_scales, uint16_t* out, int m,
+                                             int n, int k, hipStream_t stream, size_t out_row_stride_elems, int rs,
+                                             int cs, void* ws = nullptr, size_t ws_bytes = 0,
+                                             bool prefill_tile = false) {
+  detail::check(dgpp_launch_scale_gemm_grid_e8m0_bf16(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k,
+                                                      stream, out_row_stride_elems, rs, cs, ws, ws_bytes, prefill_tile));
+}
+inline void launch_scale_gemm_grid_e8m0_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                            const uint8_t* w_scales, float* out, int m, int n, int k,
+                                            hipStream_t stream, size_t out_row_stride_elems, int rs, int cs,
+                                            void* ws = nullptr, size_t ws_bytes = 0, bool prefill_tile = false) {
+  detail::check(dgpp_launch_scale_gemm_grid_e8m0_f32(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k,
+                                                     stream, out_row_stride_elems, rs, cs, ws, ws_bytes, prefill_tile));
+}
+constexpr int kFp8GemvMaxProblems = 4;
+inline void launch_scale_gemv_multi_bf16(const Fp8GemvProblem* problems, int n_problems, const uint16_t* act,
+                                         size_t act_row_stride_elems, int rows, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_scale_gemv_multi_bf16(problems, n_problems, act, act_row_stride_elems, rows, k, stream));
+}
+inline bool fp8_gemv_can_stage(const void* w_payload, int k) { return dgpp_fp8_gemv_can_stage(w_payload, k) != 0; }
+
+// ---- src/kernels/fp8_dequant.hpp ----------------------------------------------------------------------------
+inline void launch_fp8_dequant_blocks(const uint8_t* payload, const float* scales, uint16_t* out_bf16, int64_t rows,
+                                      int64_t cols, hipStream_t stream, int rs = 7, int cs = 7) {
+  detail::check(dgpp_launch_fp8_dequant_blocks(payload, scales, out_bf16, rows, cols, stream, rs, cs));
+}
+inline void launch_fp8_dequant_blocks_e8m0(const uint8_t* payload, const uint8_t* scales, uint16_t* out_bf16,
+                                           int64_t rows, int64_t cols, hipStream_t stream, int rs, int cs) {
+  detail::check(dgpp_launch_fp8_dequant_blocks_e8m0(payload, scales, out_bf16, rows, cols, stream, rs, cs));
+}
+
+}  // namespace dgpp

@@ -1,0 +1,74 @@
+/*
+ * C entry points of the host-side MoE layer driver (dgpp_amd/csrc/moe_layer.{hpp,cpp}): the
+ * counterpart of the reference's GlmMoeLayer (src/models/glm/moe_layer.hpp:50, call order of
+ * enqueue_decode_impl at src/models/glm/moe_layer.cpp:1415-1680 and of the device-segmented grouped
+ * path at :775-817, :906-934). The driver is C++ above the kernel ABI of dgpp_amd.h; these wrappers
+ * let tests and the benchmark drive it through ctypes. Unlike the launchers, create / destroy
+ * allocate and free device memory (the layer's scratch and its device expert table).
+ */
+#ifndef DGPP_AMD_LAYER_H
+#define DGPP_AMD_LAYER_H
+
+#include "dgpp_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DGPP_EXPERTS_FP8 0
+#define DGPP_EXPERTS_NVFP4 1
+#define DGPP_EXPERTS_MXFP4 2
+
+typedef struct DgppMoeLayer DgppMoeLayer;
+/* Message of the calling thread's last failed layer call. */
+const char* dgpp_moe_layer_last_error(void);
+
+typedef struct DgppMoeLayerDesc {
+  DgppMoeConfig cfg;
+  int32_t expert_format;              /* DGPP_EXPERTS_* */
+  int32_t max_tokens;
+  const DgppMoeExpertView* views;     /* HOST array: [n_experts * 3] gate,up,down, then the shared
+                                         triple when shared_in_table != 0 */
+  int32_t shared_in_table;            /* the shared expert is an FP4 triple at views[n_experts * 3 ..] */
+  int32_t shared_inter;               /* the shared expert's intermediate width (0: no shared expert) */
+  const uint8_t* sh_payload[3];       /* FP8 shared expert given as launch arguments (gate, up, down) */
+  const float* sh_scales[3];
+  int32_t sh_rs, sh_cs;
+  const uint16_t* router_gate;        /* bf16 [n_experts, hidden] (may be null when only
+                                         enqueue_decode_scores is used) */
+  const float* router_bias;           /* f32 [n_experts] (null in softmax mode) */
+} DgppMoeLayerDesc;
+
+/* Device bytes the layer's scratch takes for max_tokens (reference: GlmMoeLayer::scratch_bytes,
+ * src/models/glm/moe_layer.cpp:72-129, decode-slot and grouped buffers). */
+size_t dgpp_moe_layer_scratch_bytes(const DgppMoeConfig* cfg, int max_tokens, int shared_inter);
+int dgpp_moe_layer_create(const DgppMoeLayerDesc* desc, DgppMoeLayer** out);
+void dgpp_moe_layer_destroy(DgppMoeLayer* layer);
+
+/* The decode path: router -> slot order (tokens > 1) -> gate/up+SwiGLU -> down -> accumulate, all
+ * on `stream`, no host sync. out_bf16 [tokens, hidden]; out_f32 (nullable) receives the unrounded
+ * chain instead when given. x bf16 [tokens, x_stride]. */
+int dgpp_moe_layer_enqueue_decode(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, uint16_t* out_bf16,
+                                  float* out_f32, int tokens, void* stream);
+/* The same with the router's scores given (f32 [tokens, n_experts] scores and biased rows; softmax
+ * mode: the bf16-rounded logits in both): only the selection half of the router runs. */
+int dgpp_moe_layer_enqueue_decode_scores(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride,
+                                         const float* scores, const float* biased, uint16_t* out_bf16,
+                                         float* out_f32, int tokens, void* stream);
+/* The same with the routes given (ids ascending per token, weights): no router at all. */
+int dgpp_moe_layer_enqueue_decode_routed(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride,
+                                         const int32_t* ids, const float* weights, uint16_t* out_bf16,
+                                         float* out_f32, int tokens, void* stream);
+/* The grouped (segment-major) path over given routes: device segmentation -> gather -> grouped
+ * gate, up -> SwiGLU -> grouped down -> ordered accumulation. Bitwise the decode path's output. */
+int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride,
+                                          const int32_t* ids, const float* weights, uint16_t* out_bf16,
+                                          float* out_f32, int tokens, void* stream);
+/* Device pointers of the last routes the layer computed: ids int32 [tokens, top_k], weights f32. */
+const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* layer);
+const float* dgpp_moe_layer_weights(const DgppMoeLayer* layer);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -8,8 +8,8 @@ from dgpp_amd import _lib
 ROOT = Path(__file__).resolve().parent.parent
 
 
-def declared_symbols():
-    text = (ROOT / "include" / "dgpp_amd.h").read_text()
+def declared_symbols(header="dgpp_amd.h"):
+    text = (ROOT / "include" / header).read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(dgpp_[a-z0-9_]+)\s*\(", text)))
 
@@ -22,6 +22,10 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} is declared in include/dgpp_amd.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert set(_lib.SIGNATURES) == set(names)
+    layer = declared_symbols("dgpp_amd_layer.h")
+    assert set(layer) == set(_lib.LAYER_SIGNATURES)
+    for n in layer:
+        assert hasattr(lib, n), f"{n} is declared in include/dgpp_amd_layer.h but not exported"
     assert lib.dgpp_target_arch() == b"gfx950"
 
 
