@@ -1,0 +1,301 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized MoE expert GEMV path on one MI355X.
+
+A "step" is one pass of the hot path over one batch: one MXFP4 MoE decode layer (router top-8
+selection from given logits -> slot order -> fused gate/up + SwiGLU -> down -> ordered
+accumulation) at the BASELINE shape (256 experts, hidden 4096, expert intermediate 1024, top-8,
+no shared expert), T tokens. Consecutive steps walk DIFFERENT layers' weights (a ring of
+`--layers` full layers, as a model's decode step walks its MoE layers), so every step streams its
+experts from HBM, not from the 256 MB Infinity Cache / L2. The steps are captured once in a HIP
+graph (the serving form of the reference's decode walk) and timed with events on the launch stream.
+
+Prints ONE JSON line: whole-layer achieved HBM GB/s (algorithmic bytes / time), µs per layer,
+the dominant kernel's roofline, and the CPU oracle timed on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+E, H, I, K = 256, 4096, 1024, 8          # BASELINE config 3 (MXFP4 MoE decode layer)
+EXPERT_BYTES = 3 * I * H // 2 + 3 * I * H // 32          # payload + e8m0 scales of gate, up, down
+GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
+DOWN_BYTES = H * I // 2 + H * I // 32
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--tokens", type=int, default=8, help="decode batch of the headline number (1..8)")
+    ap.add_argument("--layers", type=int, default=16, help="ring of distinct layers' weights (cold-cache rotation)")
+    ap.add_argument("--experts", type=int, default=E, help="experts per layer (256 = the BASELINE shape)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="'layer', 'gate_up' or 'down': run only that timed graph (for profiling)")
+    ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU (the path shards by experts or by the intermediate "
+              "dimension with a single all-reduce after the layer; no multi-GPU figure is produced). "
+              "Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from dgpp_amd import _lib, hostgen as hg, launch as L, moe_layer as ML
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    lib = _lib.load()   # fails loudly when the HIP library has not been built
+    for kv in filter(None, args.tune.split(",")):
+        k, v = kv.split("=")
+        lib.dgpp_tune_set(int(k), int(v))
+    dev = torch.device("cuda:0")
+    nE, nL = args.experts, args.layers
+    t_build = time.time()
+
+    # ---- layer 0: host-generated N(0, 0.02) weights, MXFP4-quantised with the library's encoder ----------
+    gu_p = torch.empty((nE, 2, I, H // 2), dtype=torch.uint8)
+    gu_s = torch.empty((nE, 2, I, H // 32), dtype=torch.uint8)
+    dn_p = torch.empty((nE, H, I // 2), dtype=torch.uint8)
+    dn_s = torch.empty((nE, H, I // 32), dtype=torch.uint8)
+    for e in range(nE):
+        seed = 0xD6990000 + 3 * 16 + e * 3
+        for m in range(2):
+            p, s = hg.encode_mxfp4(hg.normal_f32(seed + m, (I, H), 0.02))
+            gu_p[e, m], gu_s[e, m] = torch.from_numpy(p), torch.from_numpy(s)
+        p, s = hg.encode_mxfp4(hg.normal_f32(seed + 2, (H, I), 0.02))
+        dn_p[e], dn_s[e] = torch.from_numpy(p), torch.from_numpy(s)
+    host_layer0 = (gu_p, gu_s, dn_p, dn_s)
+    # ---- the ring: layer l is layer 0 with its experts rotated by 37*l (distinct addresses) ------------
+    layers, keep = [], []
+    cfg = L.make_config(H, I, nE, K, n_shared_experts=0, routed_scaling_factor=1.0, swiglu_limit=float("inf"),
+                        router_mode=L.ROUTER_SOFTMAX_TOPK)
+    max_t = 8
+    d0 = [t.to(dev) for t in host_layer0]
+    for l in range(nL):
+        if l == 0:
+            bufs = d0
+        else:
+            sh = (37 * l) % nE
+            bufs = [torch.roll(t, shifts=sh, dims=0).contiguous() for t in d0]
+        keep.append(bufs)
+        views = []
+        for e in range(nE):
+            for m in range(3):
+                v = L.MoeExpertView()
+                if m < 2:
+                    v.payload, v.fp4_scales = bufs[0][e, m].data_ptr(), bufs[1][e, m].data_ptr()
+                else:
+                    v.payload, v.fp4_scales = bufs[2][e].data_ptr(), bufs[3][e].data_ptr()
+                v.scale_shift_rows = v.scale_shift_cols = 7
+                v.fp4_group = 32
+                views.append(v)
+        layers.append(ML.MoeLayer(cfg, ML.EXPERTS_MXFP4, views, max_t))
+    build_s = time.time() - t_build
+
+    def inputs(T):
+        xs = torch.from_numpy(hg.normal_bf16(0xD6990000 + 3 * 16 + T, (nL, T, H)).view(np.int16)).to(dev)
+        lg = hg.bf16_to_f32(hg.normal_bf16(0xD6990100 + T, (nL, T, nE)))        # router logits N(0,1), bf16 values
+        return xs, torch.from_numpy(lg).to(dev), lg
+
+    stream = torch.cuda.Stream()
+
+    def time_graph(enqueue, steps, warmup):
+        """Captures `steps` calls of enqueue(i) in one graph, replays it once untimed (plus `warmup` eager
+        steps before capture) and once timed with events on the launch stream. Returns seconds per step."""
+        with torch.cuda.stream(stream):
+            for i in range(max(warmup, 1)):
+                enqueue(i)
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for i in range(steps):
+                    enqueue(i)
+            g.replay()
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            g.replay()
+            e1.record(stream)
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / steps
+
+    def measure(T, steps, warmup, only=""):
+        xs, lg_d, lg = inputs(T)
+        outs = torch.empty((nL, T, H), dtype=torch.int16, device=dev)
+        # distinct experts per layer-step (the algorithmic bytes count each distinct expert once)
+        l64 = lg.astype(np.float64)
+        uniq = []
+        for l in range(nL):
+            top = np.argsort(-l64[l], axis=1, kind="stable")[:, :K]
+            uniq.append(len(np.unique(top)))
+        u_mean = float(np.mean([uniq[i % nL] for i in range(steps)]))
+        layer_bytes = u_mean * EXPERT_BYTES + T * (H * 2 * 2) + T * K * 8
+        res = {"tokens": T, "distinct_experts_mean": u_mean, "algorithmic_bytes": layer_bytes}
+
+        def full(i):
+            l = i % nL
+            layers[l].enqueue_decode_scores(xs[l], H, lg_d[l], lg_d[l], outs[l], T, stream)
+
+        if only in ("", "layer"):
+            sec = time_graph(full, steps, warmup)
+            res["us_per_layer"] = sec * 1e6
+            res["gbps"] = layer_bytes / sec / 1e9
+            res["frac_of_peak"] = res["gbps"] / HBM_PEAK_GBPS
+        # the dominant kernel alone: the fused gate/up + SwiGLU slot kernel on the routes the layers hold
+        slots = T * (K + 1)
+        acts = torch.empty((nL, slots, I), dtype=torch.int16, device=dev)
+        orders = []
+        with torch.cuda.stream(stream):
+            for l in range(nL):
+                full(l)                                       # leaves ids / weights in the layer's scratch
+                o = torch.empty(slots, dtype=torch.int32, device=dev)
+                if T > 1:
+                    L.launch_moe_slot_order(layers[l].ids_ptr, o, slots, K, nE, stream)
+                orders.append(o)
+            stream.synchronize()
+        def gate_up(i):
+            l = i % nL
+            L.launch_moe_slot_gate_up_swiglu_fp4(xs[l], H, layers[l].ids_ptr, orders[l] if T > 1 else None,
+                                                 layers[l]._views_ptr, I, H, 0, 0, None, None, None, None, acts[l], I,
+                                                 slots, K, float("inf"), stream, -1, 32)
+
+        if only in ("", "gate_up"):
+            sec_k = time_graph(gate_up, steps, warmup)
+            kbytes = u_mean * GATE_UP_BYTES + T * H * 2 + T * K * I * 2
+            res["gate_up_us"] = sec_k * 1e6
+            res["gate_up_bytes"] = kbytes
+            res["gate_up_gbps"] = kbytes / sec_k / 1e9
+        downs = torch.empty((nL, slots, H), dtype=torch.float32, device=dev)
+        counter = torch.zeros(2, dtype=torch.int32, device=dev)
+
+        def down(i):
+            l = i % nL
+            L.launch_moe_slot_down_fp4(acts[l], I, layers[l].ids_ptr, orders[l] if T > 1 else None, layers[l]._views_ptr,
+                                       H, I, 0, 0, None, None, downs[l], H, slots, K, stream, -1, 32, 7, 7, counter)
+
+        if only in ("", "down"):
+            sec_d = time_graph(down, steps, warmup)
+            dbytes = u_mean * DOWN_BYTES + T * K * I * 2 + T * K * H * 4
+            res["down_us"] = sec_d * 1e6
+            res["down_bytes"] = dbytes
+            res["down_gbps"] = dbytes / sec_d / 1e9
+        return res
+
+    for lyr in layers:     # device pointer of the layer's expert table, for the single-kernel leg
+        lyr._views_ptr = lyr.views_ptr
+
+    T = args.tokens
+    main_res = measure(T, args.steps, args.warmup, args.only)
+    others = {}
+    if not args.only and not args.tune:
+        for t in (1, 4, 8):
+            if t != T:
+                others[f"T{t}"] = measure(t, args.steps, args.warmup)
+
+    # ---- CPU baseline: the oracle's layer forward (dequantise to double, fp64 dots) on a bounded sample ----
+    cpu = None
+    if not args.no_cpu and not args.only:
+        sys.path.insert(0, str(ROOT / "tests"))
+        import oracle_lib as orc
+        xs, lg_d, lg = inputs(1)
+        l64 = lg[0].astype(np.float64)
+        ids = np.empty((1, K), np.int32)
+        w = np.empty((1, K), np.float32)
+        orc.oracle().orc_router_select(orc.p(l64), orc.p(l64.copy()), 1, 1, nE, K, 1.0, 1, orc.p(ids), orc.p(w))
+        mats, hold = [], []
+        zero8 = np.zeros(1, np.uint8)
+        used = set(int(v) for v in ids.ravel())
+        for e in range(nE):
+            for m in range(3):
+                if e in used:
+                    pa = (gu_p[e, m] if m < 2 else dn_p[e]).numpy()
+                    sa = (gu_s[e, m] if m < 2 else dn_s[e]).numpy()
+                    hold += [pa, sa]
+                    mats.append(orc.make_matrix(1, pa, sa, group=32))
+                else:
+                    mats.append(orc.make_matrix(1, zero8, zero8, group=32))
+        x1 = hg.normal_bf16(0xD6990000 + 3 * 16 + 1, (nL, 1, H))[0]
+        cores = min(16, os.cpu_count() or 1)
+        t0 = time.time()
+        raw1, _ = orc.moe_forward(x1, ids, w, H, I, I, mats, None, float("inf"), threads=1)
+        t_one = time.time() - t0
+        t0 = time.time()
+        rawn, _ = orc.moe_forward(x1, ids, w, H, I, I, mats, None, float("inf"), threads=cores)
+        t_many = time.time() - t0
+        bytes1 = K * EXPERT_BYTES + 2 * H * 2 + K * 8
+        cpu = {"value": bytes1 / t_many / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+               "sample": "one layer pass at T=1 (8 experts, 53.5 MB) through the CPU oracle: weights dequantised "
+                         "to double, fp64 dots, reference rounding points",
+               "us_per_layer": t_many * 1e6, "single_thread_us_per_layer": t_one * 1e6,
+               "single_thread_gbps": bytes1 / t_one / 1e9}
+        # the same pass on the GPU must agree with what was just computed on the CPU
+        out1 = torch.empty((1, H), dtype=torch.int16, device=dev)
+        layers[0].enqueue_decode_scores(xs[0], H, lg_d[0], lg_d[0], out1, 1, None)
+        torch.cuda.synchronize()
+        got = hg.bf16_to_f32(out1.cpu().numpy().view(np.uint16)).astype(np.float64)[0]
+        ref = raw1[0]
+        floor = 0.02 * float(np.sqrt(np.mean(ref ** 2)))
+        cpu["gpu_vs_cpu_max_rel"] = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+
+    sec = main_res.get("us_per_layer", float("nan")) * 1e-6
+    line = {
+        "metric": "MXFP4 MoE decode layer achieved HBM GB/s (algorithmic bytes / time) on 1 MI355X",
+        "value": main_res.get("gbps"),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec * 1e3,
+        "us_per_layer": main_res.get("us_per_layer"),
+        "frac_of_hbm_peak": main_res.get("frac_of_peak"),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic: layer 0 host-generated N(0,0.02) weights MXFP4-quantised (E2M1 + E8M0/32, ceil-pow2 "
+                "scales); the other ring layers are device copies with the experts rotated; x ~ N(0,1) bf16, "
+                "router logits ~ N(0,1)",
+        "config": {"workload": f"BASELINE config 3: MXFP4 MoE decode layer, {nE} experts, hidden {H}, inter {I}, "
+                               f"top-{K} softmax-renormalised, no shared expert, T={T} tokens",
+                   "tokens": T, "ring_layers": nL, "timing": "HIP graph of `steps` layer passes, events on the "
+                   "launch stream, weights cold (ring >= 2x the 256 MB cache)",
+                   "distinct_experts_mean": main_res["distinct_experts_mean"],
+                   "algorithmic_bytes_per_layer": main_res["algorithmic_bytes"]},
+        "roofline": None,
+        "cpu_baseline": cpu,
+        "other_batches": others,
+        "build_seconds": build_s,
+    }
+    if "gate_up_us" in main_res:
+        line["roofline"] = {"kernel": "slot_gate_up_kernel<MXFP4> (fused gate/up GEMV + SwiGLU)", "bound": "hbm",
+                            "achieved": main_res["gate_up_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                            "frac": main_res["gate_up_gbps"] / HBM_PEAK_GBPS, "traffic": None,
+                            "bytes_per_launch": main_res["gate_up_bytes"], "us_per_launch": main_res["gate_up_us"]}
+        if "down_us" in main_res:
+            line["roofline"]["second_kernel"] = {
+                "kernel": "slot_down_kernel<MXFP4> (down GEMV, f32 out)", "achieved": main_res["down_gbps"],
+                "frac": main_res["down_gbps"] / HBM_PEAK_GBPS, "bytes_per_launch": main_res["down_bytes"],
+                "us_per_launch": main_res["down_us"]}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

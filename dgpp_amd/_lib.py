@@ -66,6 +66,8 @@ _P, _I, _F, _Z, _L = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_int64
 SIGNATURES = {
     "dgpp_last_error": (C.c_char_p, []),
     "dgpp_target_arch": (C.c_char_p, []),
+    "dgpp_tune_set": (None, [_I, _I]),
+    "dgpp_tune_get": (_I, [_I]),
     "dgpp_moe_config_validate": (_I, [_P]),
     "dgpp_launch_moe_router": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_launch_moe_router_select": (_I, [_P, _P, _P, _P, _P, _I, _P]),
@@ -83,6 +85,7 @@ SIGNATURES = {
     "dgpp_launch_moe_accum_ordered_f32": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _I, _P]),
     "dgpp_launch_moe_slot_accum": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dgpp_launch_moe_slot_accum_routed_f32": (_I, [_P, _P, _P, _I, _I, _I, _P]),
+    "dgpp_launch_moe_slot_accum_routed_bf16": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dgpp_launch_moe_slot_gate_up_swiglu": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I]),
     "dgpp_launch_moe_slot_down": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_launch_moe_slot_gate_up_swiglu_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I, _I, _I]),
@@ -143,6 +146,7 @@ LAYER_SIGNATURES = {
     "dgpp_moe_layer_enqueue_decode_scores": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_decode_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_grouped_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
+    "dgpp_moe_layer_views": (_P, [_P]),
     "dgpp_moe_layer_ids": (_P, [_P]),
     "dgpp_moe_layer_weights": (_P, [_P]),
 }

@@ -60,6 +60,9 @@ MatRef fp8_mat(const uint8_t* payload, const void* scales, int rs, int cs) {
 }  // namespace
 
 namespace dgpp_amd {
+static int g_tune[kTuneCount] = {0};
+int tune_get(int key) { return key >= 0 && key < kTuneCount ? g_tune[key] : 0; }
+
 hipError_t ensure_lds_impl(const void* kernel, size_t bytes) {
   static std::mutex mu;
   static std::unordered_map<const void*, size_t> raised;
@@ -260,6 +263,10 @@ extern "C" {
 
 const char* dgpp_last_error(void) { return g_last_error.c_str(); }
 const char* dgpp_target_arch(void) { return "gfx950"; }
+void dgpp_tune_set(int key, int value) {
+  if (key >= 0 && key < kTuneCount) g_tune[key] = value;
+}
+int dgpp_tune_get(int key) { return tune_get(key); }
 
 int dgpp_moe_config_validate(const DgppMoeConfig* c) {
   // src/models/glm/moe.hpp:119-133
@@ -407,6 +414,14 @@ int dgpp_launch_moe_slot_accum_routed_f32(float* out, const float* contrib, cons
   if (!out || !contrib || !weights) return fail_arg("moe_slot_accum_routed_f32: null pointer");
   return finish(run_slot_accum(out, 1, 0, contrib, weights, tokens, hidden, top_k, as_stream(stream)),
                 "moe_slot_accum_routed_f32");
+}
+
+int dgpp_launch_moe_slot_accum_routed_bf16(uint16_t* out, const float* contrib, const float* weights, int tokens,
+                                           int hidden, int top_k, void* stream) {
+  if (tokens <= 0) return DGPP_OK;
+  if (!out || !contrib || !weights) return fail_arg("moe_slot_accum_routed_bf16: null pointer");
+  return finish(run_slot_accum(out, 0, 0, contrib, weights, tokens, hidden, top_k, as_stream(stream)),
+                "moe_slot_accum_routed_bf16");
 }
 
 int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,

@@ -15,7 +15,8 @@
 //
 // Value semantics (reference: src/kernels/fp8_gemv.cuh:64-66, src/kernels/fp4_gemv.cuh:20-27):
 //   FP8 + F32 grid   w = bf16_rne(float(e4m3) * scale)               (the rounding is part of the value)
-//   FP8 + E8M0 grid  w = e4m3 * 2^(b-127), b == 0 -> 2^-127          (exact in bf16)
+//   FP8 + E8M0 grid  w = e4m3 * 2^(b-127), b == 0 -> 2^-127          (exact in bf16; byte 255 gives NaN, the
+//                    E8M0 encoding's meaning, where the reference's dequant bridge reads it as +inf)
 //   NVFP4            w = e2m1 * e4m3(scale) exact; dot / global once  (we sum a 16-group unscaled,
 //                    then fold the group scale in with one fma: same sum, fp32 rounding order only)
 //   MXFP4            w = e2m1 * 2^(b-127) exact, b == 255 -> NaN
@@ -64,14 +65,20 @@ struct RowGeom {
   int P;       // chunks per lane
   int nb;      // chunks per pass (a divisor of P, <= 8): the loads in flight per lane per row
 };
-__host__ __device__ inline RowGeom row_geom(int chunks) {
+// Bench A/B switches (host side, process-wide; 0 = the default behaviour). Set through
+// dgpp_tune_set; launchers read them when they pick a geometry or a kernel form.
+enum : int { kTunePreferP = 0, kTuneSlotForm = 1, kTuneSlotSteps = 2, kTuneCount = 8 };
+int tune_get(int key);
+
+__host__ __device__ inline RowGeom row_geom(int chunks, int prefer_p = 4) {
   RowGeom g;
   g.l2 = 0;
   while (g.l2 < 6 && (chunks % (2 << g.l2)) == 0) ++g.l2;
   g.P = chunks >> g.l2;
-  // Prefer four chunks per lane over very wide row groups: more bytes in flight per lane,
-  // and a row group keeps at least 128 contiguous bytes per load instruction (8 lanes).
-  while (g.P < 4 && g.l2 > 3) {
+  // Prefer at least `prefer_p` chunks per lane over very wide row groups (a row group keeps at
+  // least 128 contiguous bytes per load instruction: 8 lanes). Four measured a few percent faster
+  // than two on the MoE shapes (more bytes in flight per lane).
+  while (g.P < prefer_p && g.l2 > 3) {
     --g.l2;
     g.P *= 2;
   }
@@ -164,137 +171,115 @@ __device__ __forceinline__ void load_chunk(const uint8_t* __restrict__ payload_r
   }
 }
 
-// acc[r] += dot(chunk weights, activation row r's elements of chunk c) for r < m.
-// xl points at LDS vector [piece 0][chunk c] of activation row 0.
-template <int FMT, int MAXR>
-__device__ __forceinline__ void consume_chunk(const ChunkRegs& ch, const uint4* __restrict__ xl,
-                                              int chunks, int m, float (&acc)[MAXR]) {
-  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+// Where a chunk's activation vectors come from: LDS (any number of staged rows) ...
+template <int FMT>
+struct XLds {
+  const uint4* base;  // LDS vector [piece 0][chunk c] of activation row 0
+  int chunks;
+  __device__ __forceinline__ uint4 get(int r, int q) const { return base[(r * FmtTraits<FMT>::kPieces + q) * chunks]; }
+};
+// ... or registers (one activation row, the lane's own chunk columns loaded once per wavefront).
+template <int FMT>
+struct XReg {
+  const uint4* v;     // [kPieces] vectors of this chunk
+  __device__ __forceinline__ uint4 get(int, int q) const { return v[q]; }
+};
+
+// ---- per-chunk arithmetic, split in decode and dot ------------------------------------------------
+// A chunk decoded to packed bf16 pairs (element pairs in k order); NVFP4 keeps its two group scales
+// aside because they are folded in once per 16-group, after the unscaled partial sum.
+template <int FMT>
+struct Decoded {
+  bf16x2_t p[FmtTraits<FMT>::kElemsPerChunk / 2];
+  float s0, s1;
+};
+
+template <int FMT>
+__device__ __forceinline__ void decode_chunk(const ChunkRegs& ch, Decoded<FMT>& d) {
   const uint32_t w[4] = {ch.w.x, ch.w.y, ch.w.z, ch.w.w};
-  if constexpr (FMT == kFmtMxfp4) {
-    if (ch.s >= 2u && ch.s <= 252u) {
-      // e2m1 * 2^(b-127) is a normal bf16 for every code: the scaled conversion is exact.
-      const float s = bits_f32(ch.s << 23);
-      bf16x2_t p[16];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        p[q * 4 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 0);
-        p[q * 4 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 1);
-        p[q * 4 + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 2);
-        p[q * 4 + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 3);
-      }
-#pragma unroll
-      for (int r = 0; r < MAXR; ++r) {
-        if (r < m) {
-          float a = acc[r];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint4 xv = xl[(r * kPieces + q) * chunks];
-            a = dot2(p[q * 4 + 0], xv.x, a);
-            a = dot2(p[q * 4 + 1], xv.y, a);
-            a = dot2(p[q * 4 + 2], xv.z, a);
-            a = dot2(p[q * 4 + 3], xv.w, a);
-          }
-          acc[r] = a;
-        }
-      }
-    } else {
-      // Scale bytes at the ends of the range (2^-127, 2^-126, >= 2^126, NaN): exact fp32 path.
-      const float s = e8m0_to_f32(static_cast<uint8_t>(ch.s));
-#pragma unroll
-      for (int r = 0; r < MAXR; ++r) {
-        if (r < m) {
-          float a = acc[r];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint4 xv = xl[(r * kPieces + q) * chunks];
-            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const uint32_t byte = (w[q] >> (8 * j)) & 0xFFu;
-              a = fmaf(e2m1_to_f32(byte & 0xFu) * s, bits_f32(xw[j] << 16), a);
-              a = fmaf(e2m1_to_f32(byte >> 4) * s, bits_f32(xw[j] & 0xFFFF0000u), a);
-            }
-          }
-          acc[r] = a;
-        }
-      }
-    }
-  } else if constexpr (FMT == kFmtNvfp4) {
-    bf16x2_t p[16];
+  if constexpr (FMT == kFmtMxfp4 || FMT == kFmtNvfp4) {
+    // MXFP4: the scaled conversion takes the E8M0 byte as the exponent field of a float and is exact
+    // for EVERY byte on gfx950 (0 -> 2^-127 with subnormal bf16 results, 255 -> NaN), checked over all
+    // 256 x 16 (byte, code) pairs on the hardware.
+    const float s = FMT == kFmtMxfp4 ? bits_f32(ch.s << 23) : 1.0f;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      p[q * 4 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 0);
-      p[q * 4 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 1);
-      p[q * 4 + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 2);
-      p[q * 4 + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], 1.0f, 3);
+      d.p[q * 4 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 0);
+      d.p[q * 4 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 1);
+      d.p[q * 4 + 2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 2);
+      d.p[q * 4 + 3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 3);
     }
-    // The two e4m3 group scales of the chunk (codes 0..15 and 16..31), NaN codes propagate.
-    const float s0 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 0);
-    const float s1 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 1);
+    if constexpr (FMT == kFmtNvfp4) {
+      // The two e4m3 group scales (codes 0..15 and 16..31); NaN codes propagate.
+      d.s0 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 0);
+      d.s1 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 1);
+    }
+  } else if constexpr (FMT == kFmtFp8E8M0) {
+    const float s = bits_f32(ch.s << 23);
 #pragma unroll
-    for (int r = 0; r < MAXR; ++r) {
-      if (r < m) {
-        float a = acc[r];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          float part = 0.f;
-#pragma unroll
-          for (int q = 2 * h; q < 2 * h + 2; ++q) {
-            const uint4 xv = xl[(r * kPieces + q) * chunks];
-            part = dot2(p[q * 4 + 0], xv.x, part);
-            part = dot2(p[q * 4 + 1], xv.y, part);
-            part = dot2(p[q * 4 + 2], xv.z, part);
-            part = dot2(p[q * 4 + 3], xv.w, part);
-          }
-          a = fmaf(part, h == 0 ? s0 : s1, a);
-        }
-        acc[r] = a;
-      }
+    for (int q = 0; q < 4; ++q) {
+      d.p[q * 2 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], s, false);
+      d.p[q * 2 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], s, true);
     }
   } else {
-    // FP8: 16 codes -> 8 packed bf16 pairs.
-    bf16x2_t p[8];
-    bool fast = true;
-    if constexpr (FMT == kFmtFp8E8M0) fast = ch.s >= 10u && ch.s <= 245u;
-    if constexpr (FMT == kFmtFp8E8M0) {
-      if (fast) {
-        const float s = bits_f32(ch.s << 23);
+    // float(e4m3) * scale in fp32, one RNE rounding to bf16: the rounding is part of the value.
+    const float s = bits_f32(ch.s);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          p[q * 2 + 0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], s, false);
-          p[q * 2 + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[q], s, true);
-        }
-      }
-    }
-    if (FMT == kFmtFp8F32 || !fast) {
-      // float(e4m3) * scale in fp32, one RNE rounding to bf16. The E8M0 bridge reads byte b
-      // as the float with exponent field b (0 -> 2^-127), src/kernels/fp8_dequant.cu:28-31.
-      const float s = FMT == kFmtFp8F32 ? bits_f32(ch.s) : (ch.s ? bits_f32(ch.s << 23) : bits_f32(0x00400000u));
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[q], false);
-        const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[q], true);
-        p[q * 2 + 0] = pack_bf16(lo.x * s, lo.y * s);
-        p[q * 2 + 1] = pack_bf16(hi.x * s, hi.y * s);
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < MAXR; ++r) {
-      if (r < m) {
-        float a = acc[r];
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          const uint4 xv = xl[(r * kPieces + q) * chunks];
-          a = dot2(p[q * 4 + 0], xv.x, a);
-          a = dot2(p[q * 4 + 1], xv.y, a);
-          a = dot2(p[q * 4 + 2], xv.z, a);
-          a = dot2(p[q * 4 + 3], xv.w, a);
-        }
-        acc[r] = a;
-      }
+    for (int q = 0; q < 4; ++q) {
+      const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[q], false);
+      const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[q], true);
+      d.p[q * 2 + 0] = pack_bf16(lo.x * s, lo.y * s);
+      d.p[q * 2 + 1] = pack_bf16(hi.x * s, hi.y * s);
     }
   }
+}
+
+// acc + dot(decoded chunk, the chunk's activation vectors x[0 .. kPieces)).
+template <int FMT>
+__device__ __forceinline__ float dot_chunk(const Decoded<FMT>& d, const uint4* x, float acc) {
+  if constexpr (FMT == kFmtNvfp4) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      float part = 0.f;
+#pragma unroll
+      for (int q = 2 * h; q < 2 * h + 2; ++q) {
+        part = dot2(d.p[q * 4 + 0], x[q].x, part);
+        part = dot2(d.p[q * 4 + 1], x[q].y, part);
+        part = dot2(d.p[q * 4 + 2], x[q].z, part);
+        part = dot2(d.p[q * 4 + 3], x[q].w, part);
+      }
+      acc = fmaf(part, h == 0 ? d.s0 : d.s1, acc);
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < FmtTraits<FMT>::kPieces; ++q) {
+      acc = dot2(d.p[q * 4 + 0], x[q].x, acc);
+      acc = dot2(d.p[q * 4 + 1], x[q].y, acc);
+      acc = dot2(d.p[q * 4 + 2], x[q].z, acc);
+      acc = dot2(d.p[q * 4 + 3], x[q].w, acc);
+    }
+  }
+  return acc;
+}
+
+// acc[r] += dot(chunk weights, activation row r's elements of the chunk) for r < m.
+template <int FMT, int MAXR, class X>
+__device__ __forceinline__ void consume_chunk(const ChunkRegs& ch, const X& xs, int m, float (&acc)[MAXR]) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+  Decoded<FMT> d;
+  decode_chunk<FMT>(ch, d);
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) {
+    if (r < m) {
+      uint4 xv[kPieces];
+#pragma unroll
+      for (int q = 0; q < kPieces; ++q) xv[q] = xs.get(r, q);
+      acc[r] = dot_chunk<FMT>(d, xv, acc[r]);
+    }
+  }
+  // Keep the scheduler from hoisting the next chunk's decode above this chunk's dots: that trades
+  // a few cycles of overlap for dozens of live registers (and spills) per lane.
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 // ---- a wavefront's row step --------------------------------------------------------------------
@@ -342,7 +327,7 @@ __device__ __forceinline__ void consume_pass(const ChunkRegs (&regs)[NB], const 
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     const int c = ((pass * NB + i) << l2) + lr.li;
-    consume_chunk<FMT, MAXR>(regs[i], lds + c, chunks, m, acc);
+    consume_chunk<FMT, MAXR>(regs[i], XLds<FMT>{lds + c, chunks}, m, acc);
   }
 }
 
@@ -355,20 +340,52 @@ __device__ __forceinline__ void row_dots(const LaneRow& lr, const RowGeom& g, in
 #pragma unroll
   for (int r = 0; r < MAXR; ++r) acc[r] = 0.f;
   const int passes = g.P / NB;
-  ChunkRegs cur[NB];
-  issue_pass<FMT, NB>(lr, 0, g.l2, cs, cur);
   for (int p = 0; p < passes; ++p) {
-    ChunkRegs nxt[NB];
-    if (p + 1 < passes) issue_pass<FMT, NB>(lr, p + 1, g.l2, cs, nxt);
+    ChunkRegs cur[NB];
+    issue_pass<FMT, NB>(lr, p, g.l2, cs, cur);
     consume_pass<FMT, MAXR, NB>(cur, lr, p, g.l2, lds, chunks, m, acc);
-    if (p + 1 < passes) {
-#pragma unroll
-      for (int i = 0; i < NB; ++i) cur[i] = nxt[i];
-    }
   }
 #pragma unroll
   for (int r = 0; r < MAXR; ++r)
     if (r < m) acc[r] = group_sum(acc[r], g.l2);
+}
+
+// One activation row already in registers: acc + dot(chunk, x).
+template <int FMT>
+__device__ __forceinline__ float chunk_dot1(const ChunkRegs& ch, const uint4* xv, float acc) {
+  Decoded<FMT> d;
+  decode_chunk<FMT>(ch, d);
+  acc = dot_chunk<FMT>(d, xv, acc);
+  __builtin_amdgcn_sched_barrier(0);
+  return acc;
+}
+
+// Two weight rows of the same geometry (a slot's gate and up rows) against ONE staged activation
+// row: both rows' loads are issued together and each chunk column's activation vectors are read
+// from LDS once for the pair. Each row's chain is row_dots' chain, bit for bit.
+template <int FMT, int NB>
+__device__ __forceinline__ void row_dots_pair(const LaneRow& la, const LaneRow& lb, const RowGeom& g, int csa,
+                                              int csb, const uint4* __restrict__ lds, int chunks, float& ra,
+                                              float& rb) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+  float a = 0.f, b = 0.f;
+  const int passes = g.P / NB;
+  for (int p = 0; p < passes; ++p) {
+    ChunkRegs ca[NB], cb[NB];
+    issue_pass<FMT, NB>(la, p, g.l2, csa, ca);
+    issue_pass<FMT, NB>(lb, p, g.l2, csb, cb);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int c = ((p * NB + i) << g.l2) + la.li;
+      uint4 xv[kPieces];
+#pragma unroll
+      for (int q = 0; q < kPieces; ++q) xv[q] = lds[q * chunks + c];
+      a = chunk_dot1<FMT>(ca[i], xv, a);
+      b = chunk_dot1<FMT>(cb[i], xv, b);
+    }
+  }
+  ra = group_sum(a, g.l2);
+  rb = group_sum(b, g.l2);
 }
 
 // Dispatches a callable on the compile-time pass width.

@@ -14,6 +14,14 @@
 
 namespace dgpp_amd {
 
+// Every GEMV kernel is compiled for at least this many resident wavefronts per SIMD (a cap of 128
+// VGPRs): the streams are latency-bound, and the compiler otherwise trades occupancy for hoisting
+// every decode of a pass ahead of the first dot.
+#ifndef DGPP_MIN_WAVES_PER_SIMD
+#define DGPP_MIN_WAVES_PER_SIMD 2
+#endif
+constexpr int kMinWavesPerSimd = DGPP_MIN_WAVES_PER_SIMD;
+
 // ---- epilogues ------------------------------------------------------------------------------
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
 
@@ -40,6 +48,14 @@ __device__ __forceinline__ float load_divisor(const float* global) {
   return 1.0f;
 }
 
+// The row geometry every launcher uses for a k-wide row of format FMT (one function, so the slot,
+// grouped and dense forms agree bit for bit).
+template <int FMT>
+inline RowGeom geom_for(int k) {
+  const int prefer = tune_get(kTunePreferP);
+  return row_geom(k / FmtTraits<FMT>::kElemsPerChunk, prefer > 0 ? prefer : 4);
+}
+
 // rows a block covers: waves x rows-per-wave x steps
 __host__ __device__ inline int block_rows(const RowGeom& g, int steps) {
   return kWavesPerBlock * (kWave >> g.l2) * steps;
@@ -58,7 +74,7 @@ struct DenseArgs {
 };
 
 template <int FMT, int MAXR, int NB>
-__global__ __launch_bounds__(kBlockThreads) void gemv_dense_kernel(DenseArgs a, RowGeom g, int steps) {
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_kernel(DenseArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
   stage_activations<FMT>(a.act, a.act_stride, a.m, a.k, lds);
@@ -105,6 +121,7 @@ struct SlotArgs {
   float limit;
   int want_shared;          // 0: routed slots, 1: shared slots (others exit)
   int shared_view_base;     // >= 0: shared matrices come from views[base + which]
+  int debug_nomath;         // bench probe: loads only
 };
 
 template <int FMT>
@@ -139,7 +156,7 @@ __device__ __forceinline__ bool resolve_slot(const SlotArgs& a, int& slot, int& 
 }
 
 template <int FMT, int NB>
-__global__ __launch_bounds__(kBlockThreads) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   int slot, token, base;
   if (!resolve_slot(a, slot, token, base)) return;
@@ -166,16 +183,15 @@ __global__ __launch_bounds__(kBlockThreads) void slot_gate_up_kernel(SlotArgs a,
     if (row0 >= a.n) break;
     const LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
     const LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
-    float ag[1], au[1];
-    row_dots<FMT, 1, NB>(lg, g, mg.cs, lds, chunks, 1, ag);
-    row_dots<FMT, 1, NB>(lu, g, mu.cs, lds, chunks, 1, au);
+    float ag, au;
+    row_dots_pair<FMT, NB>(lg, lu, g, mg.cs, mu.cs, lds, chunks, ag, au);
     if (lg.li == 0 && lg.row < a.n)
-      act_row[lg.row] = swiglu_bf16(finish_dot<FMT>(ag[0], dg), finish_dot<FMT>(au[0], du), a.limit);
+      act_row[lg.row] = swiglu_bf16(finish_dot<FMT>(ag, dg), finish_dot<FMT>(au, du), a.limit);
   }
 }
 
 template <int FMT, int NB>
-__global__ __launch_bounds__(kBlockThreads) void slot_down_kernel(SlotArgs a, RowGeom g, int steps) {
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   int slot, token, base;
   if (!resolve_slot(a, slot, token, base)) return;
@@ -205,6 +221,165 @@ __global__ __launch_bounds__(kBlockThreads) void slot_down_kernel(SlotArgs a, Ro
   }
 }
 
+// ---- decode slots, register-resident activations ---------------------------------------------------
+// The slot kernels' fast form when a row fits ONE pass (P == NB chunks per lane) and the activation
+// row is 16-byte aligned: a lane's chunk columns are the same for every weight row it visits, so it
+// loads its own slice of the activation row into registers ONCE (straight from global memory: no
+// LDS, no barrier) and then streams weight rows: both matrices of a step are issued together and
+// the next step's loads are issued before the current step is consumed, so a lane keeps up to
+// 4 * NB 16-byte loads in flight. The per-(row) arithmetic — chunk order per lane, dot2 order,
+// butterfly — is exactly the LDS form's: the two are bitwise twins.
+template <int FMT, int NB>
+struct XSlice {
+  uint4 v[NB * FmtTraits<FMT>::kPieces];
+};
+template <int FMT, int NB>
+__device__ __forceinline__ void load_x_slice(const uint16_t* __restrict__ x, int li, int l2, XSlice<FMT, NB>& xs) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int c = (i << l2) + li;
+#pragma unroll
+    for (int q = 0; q < kPieces; ++q)
+      xs.v[i * kPieces + q] = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(c * kPieces + q) * 8);
+  }
+}
+template <int FMT, int NB>
+__device__ __forceinline__ float dot_pass_reg(const ChunkRegs (&regs)[NB], const XSlice<FMT, NB>& xs, int l2) {
+  float acc[1] = {0.f};
+#pragma unroll
+  for (int i = 0; i < NB; ++i)
+    consume_chunk<FMT, 1>(regs[i], XReg<FMT>{xs.v + i * FmtTraits<FMT>::kPieces}, 1, acc);
+  return group_sum(acc[0], l2);
+}
+
+template <int FMT, int NB, bool PREFETCH>
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_reg_kernel(SlotArgs a, RowGeom g, int steps) {
+  int slot, token, base;
+  if (!resolve_slot(a, slot, token, base)) return;
+  const int rows_per_block = block_rows(g, steps);
+  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
+  MatRef mg, mu;
+  const float *gg = nullptr, *gu = nullptr;
+  if (base >= 0) {
+    mg = mat_of_view<FMT>(a.views[base + 0], &gg);
+    mu = mat_of_view<FMT>(a.views[base + 1], &gu);
+  } else {
+    mg = a.sh[0];
+    mu = a.sh[1];
+  }
+  const int rpw = kWave >> g.l2;
+  const int wave = threadIdx.x >> 6;
+  const int stride = kWavesPerBlock * rpw;
+  int row0 = blockIdx.x * rows_per_block + wave * rpw;
+  if (row0 >= a.n) return;
+  // The first step's weight loads go out before anything else (the longest latency of the block).
+  LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
+  LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
+  ChunkRegs cg[NB], cu[NB];
+  issue_pass<FMT, NB>(lg, 0, g.l2, mg.cs, cg);
+  issue_pass<FMT, NB>(lu, 0, g.l2, mu.cs, cu);
+  XSlice<FMT, NB> xs;
+  load_x_slice<FMT, NB>(a.x + static_cast<size_t>(token) * a.x_stride, lg.li, g.l2, xs);
+  const float dg = load_divisor<FMT>(gg), du = load_divisor<FMT>(gu);
+  uint16_t* act_row = static_cast<uint16_t*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
+  for (int s = 0; s < steps; ++s) {
+    const int next0 = row0 + stride;
+    const bool has_next = s + 1 < steps && next0 < a.n;
+    ChunkRegs ng[NB], nu[NB];
+    LaneRow lgn = lg, lun = lu;
+    if (has_next) {
+      lgn = lane_row<FMT>(mg, next0, a.n, a.k, g.l2);
+      lun = lane_row<FMT>(mu, next0, a.n, a.k, g.l2);
+      if constexpr (PREFETCH) {
+        issue_pass<FMT, NB>(lgn, 0, g.l2, mg.cs, ng);
+        issue_pass<FMT, NB>(lun, 0, g.l2, mu.cs, nu);
+      }
+    }
+    float ag, au;
+    if (a.debug_nomath) {
+      uint32_t t = 0;
+#pragma unroll
+      for (int i = 0; i < NB; ++i) t ^= cg[i].w.x ^ cg[i].w.y ^ cg[i].w.z ^ cg[i].w.w ^ cu[i].w.x ^ cu[i].w.y ^ cu[i].w.z ^ cu[i].w.w ^ cg[i].s ^ cu[i].s;
+      ag = au = bits_f32(t & 0x3FFFFFFFu);
+    } else {
+      ag = dot_pass_reg<FMT, NB>(cg, xs, g.l2);
+      au = dot_pass_reg<FMT, NB>(cu, xs, g.l2);
+    }
+    if (lg.li == 0 && lg.row < a.n)
+      act_row[lg.row] = swiglu_bf16(finish_dot<FMT>(ag, dg), finish_dot<FMT>(au, du), a.limit);
+    if (!has_next) break;
+    if constexpr (PREFETCH) {
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        cg[i] = ng[i];
+        cu[i] = nu[i];
+      }
+    } else {
+      issue_pass<FMT, NB>(lgn, 0, g.l2, mg.cs, cg);
+      issue_pass<FMT, NB>(lun, 0, g.l2, mu.cs, cu);
+    }
+    lg = lgn;
+    lu = lun;
+    row0 = next0;
+  }
+}
+
+template <int FMT, int NB, bool PREFETCH>
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_reg_kernel(SlotArgs a, RowGeom g, int steps) {
+  int slot, token, base;
+  if (!resolve_slot(a, slot, token, base)) return;
+  const int rows_per_block = block_rows(g, steps);
+  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
+  MatRef md;
+  const float* gd = nullptr;
+  if (base >= 0)
+    md = mat_of_view<FMT>(a.views[base + 2], &gd);
+  else
+    md = a.sh[0];
+  const int rpw = kWave >> g.l2;
+  const int wave = threadIdx.x >> 6;
+  const int stride = kWavesPerBlock * rpw;
+  int row0 = blockIdx.x * rows_per_block + wave * rpw;
+  if (row0 >= a.n) return;
+  LaneRow lr = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
+  ChunkRegs cur[NB];
+  issue_pass<FMT, NB>(lr, 0, g.l2, md.cs, cur);
+  XSlice<FMT, NB> xs;
+  load_x_slice<FMT, NB>(a.x + static_cast<size_t>(slot) * a.x_stride, lr.li, g.l2, xs);
+  const float dd = load_divisor<FMT>(gd);
+  float* out_row = static_cast<float*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
+  for (int s = 0; s < steps; ++s) {
+    const int next0 = row0 + stride;
+    const bool has_next = s + 1 < steps && next0 < a.n;
+    ChunkRegs nxt[NB];
+    LaneRow ln = lr;
+    if (has_next) {
+      ln = lane_row<FMT>(md, next0, a.n, a.k, g.l2);
+      if constexpr (PREFETCH) issue_pass<FMT, NB>(ln, 0, g.l2, md.cs, nxt);
+    }
+    const float acc = dot_pass_reg<FMT, NB>(cur, xs, g.l2);
+    if (lr.li == 0 && lr.row < a.n) out_row[lr.row] = finish_dot<FMT>(acc, dd);
+    if (!has_next) break;
+    if constexpr (PREFETCH) {
+#pragma unroll
+      for (int i = 0; i < NB; ++i) cur[i] = nxt[i];
+    } else {
+      issue_pass<FMT, NB>(ln, 0, g.l2, md.cs, cur);
+    }
+    lr = ln;
+    row0 = next0;
+  }
+}
+
+// The register form applies when the whole row is one pass and the lane's activation slice stays
+// within 64 registers.
+template <int FMT>
+inline bool slot_reg_form_ok(const RowGeom& g, const SlotArgs& a) {
+  const int xregs = g.P * FmtTraits<FMT>::kPieces * 4;
+  return g.P == g.nb && xregs <= 64 && ((reinterpret_cast<uintptr_t>(a.x) & 15u) == 0) && ((a.x_stride & 7u) == 0);
+}
+
 // ---- grouped (segment-major) twin ------------------------------------------------------------------
 struct GroupedArgs {
   const uint16_t* act;
@@ -221,7 +396,7 @@ struct GroupedArgs {
 };
 
 template <int FMT, int NB>
-__global__ __launch_bounds__(kBlockThreads) void grouped_gemv_kernel(GroupedArgs a, RowGeom g, int steps) {
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void grouped_gemv_kernel(GroupedArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   const DgppMoeSegment seg = a.segs[blockIdx.y];
   const int z0 = static_cast<int>(blockIdx.z) * a.rows_per_block;
@@ -305,7 +480,7 @@ inline int max_stage_rows(int k) {
 #ifdef DGPP_GEMV_IMPL
 template <int FMT>
 hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
-  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long block_steps = (a.n + rows_per_step - 1) / rows_per_step;
   const int steps = pick_steps(block_steps);
@@ -329,30 +504,64 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
   return err != hipSuccess ? err : hipGetLastError();
 }
 
+// Row steps per block of a slot launch: about four resident rounds of blocks over the 256 CUs.
+inline int pick_slot_steps(long long block_steps_total) {
+  long long s = (block_steps_total + 2047) / 2048;
+  if (s < 1) s = 1;
+  if (s > 16) s = 16;
+  return static_cast<int>(s);
+}
+
 template <int FMT>
 hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
-  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
-  const int steps = pick_steps(per_slot * a.slots);
+  const int form = tune_get(kTuneSlotForm);   // 0 auto, 1 LDS, 2 registers + prefetch, 3 registers
+  const_cast<SlotArgs&>(a).debug_nomath = tune_get(3);
+  const bool reg = form >= 2 && slot_reg_form_ok<FMT>(g, a);
+  int steps = reg ? pick_slot_steps(per_slot * a.slots) : pick_steps(per_slot * a.slots);
+  if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
-  hipError_t err = hipSuccess;
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
+    if constexpr (NB * FmtTraits<FMT>::kPieces * 4 <= 64) {
+      if (reg && form == 2) {
+        hipLaunchKernelGGL((slot_gate_up_reg_kernel<FMT, NB, true>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
+        return;
+      }
+      if (reg) {
+        hipLaunchKernelGGL((slot_gate_up_reg_kernel<FMT, NB, false>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
+        return;
+      }
+    }
     hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g, steps);
   });
-  return err != hipSuccess ? err : hipGetLastError();
+  return hipGetLastError();
 }
 
 template <int FMT>
 hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
-  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
-  const int steps = pick_steps(per_slot * a.slots);
+  const int form = tune_get(kTuneSlotForm);
+  const bool reg = form >= 2 && slot_reg_form_ok<FMT>(g, a);
+  int steps = reg ? pick_slot_steps(per_slot * a.slots) : pick_steps(per_slot * a.slots);
+  if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
+    if constexpr (NB * FmtTraits<FMT>::kPieces * 4 <= 64) {
+      if (reg && form == 2) {
+        hipLaunchKernelGGL((slot_down_reg_kernel<FMT, NB, true>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
+        return;
+      }
+      if (reg) {
+        hipLaunchKernelGGL((slot_down_reg_kernel<FMT, NB, false>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
+        return;
+      }
+    }
     hipLaunchKernelGGL((slot_down_kernel<FMT, NB>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g, steps);
   });
   return hipGetLastError();
@@ -360,7 +569,7 @@ hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
 
 template <int FMT>
 hipError_t launch_grouped_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {
-  const RowGeom g = row_geom(a.k / FmtTraits<FMT>::kElemsPerChunk);
+  const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_seg = (a.n + rows_per_step - 1) / rows_per_step;
   const int steps = pick_steps(per_seg * n_segs);

@@ -197,8 +197,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   } else if (out_f32) {
     launch_moe_slot_accum_routed_f32(out_f32, d_slot_down_, weights, tokens, H, K, stream);
   } else {
-    launch_moe_slot_accum_routed_f32(d_acc_, d_slot_down_, weights, tokens, H, K, stream);
-    launch_moe_round_bf16(out_bf16, d_acc_, static_cast<int64_t>(tokens) * H, stream);
+    launch_moe_slot_accum_routed_bf16(out_bf16, d_slot_down_, weights, tokens, H, K, stream);
   }
 }
 
@@ -331,6 +330,7 @@ int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* l, const uint16_t* x, si
     l->impl.enqueue_grouped_routed(x, x_stride, ids, weights, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
   });
 }
+const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* l) { return l->impl.views(); }
 const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* l) { return l->impl.ids(); }
 const float* dgpp_moe_layer_weights(const DgppMoeLayer* l) { return l->impl.weights(); }
 

@@ -49,6 +49,7 @@ class GlmMoeLayer {
   void enqueue_grouped_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                               uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
 
+  const MoeExpertView* views() const { return d_views_; }
   const int32_t* ids() const { return d_ids_; }
   const float* weights() const { return d_weights_; }
   bool has_shared() const { return w_.shared_inter > 0; }

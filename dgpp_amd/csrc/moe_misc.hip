@@ -185,6 +185,138 @@ __global__ __launch_bounds__(kWaveSize) void router_select_kernel(
   }
 }
 
+// The same selection for up to 64 * PER_LANE experts with the whole row in registers (expert e
+// lives in lane e % 64, slot e / 64): no LDS, no barriers, DPP reductions inside 16-lane rows and
+// four lane reads across them. Ordering keys are (value, ~id) pairs compared lexicographically, so
+// the maximum is the largest value and, among equal values, the LOWEST id — the strict '>' scan's
+// outcome. -0 is folded into +0 first (they compare equal as floats); a NaN key never wins.
+template <int kCtrl>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), kCtrl, 0xF, 0xF, true));
+}
+template <int kCtrl>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return bits_f32(dpp_u32<kCtrl>(f32_bits(v)));
+}
+__device__ __forceinline__ float row_lane(float v, int lane) {
+  return bits_f32(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(f32_bits(v)), lane)));
+}
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v += dpp_f32<0xB1>(v);
+  v += dpp_f32<0x4E>(v);
+  v += dpp_f32<0x141>(v);
+  v += dpp_f32<0x140>(v);
+  return (row_lane(v, 0) + row_lane(v, 16)) + (row_lane(v, 32) + row_lane(v, 48));
+}
+__device__ __forceinline__ float wave_max_dpp(float v) {
+  v = fmaxf(v, dpp_f32<0xB1>(v));
+  v = fmaxf(v, dpp_f32<0x4E>(v));
+  v = fmaxf(v, dpp_f32<0x141>(v));
+  v = fmaxf(v, dpp_f32<0x140>(v));
+  return fmaxf(fmaxf(row_lane(v, 0), row_lane(v, 16)), fmaxf(row_lane(v, 32), row_lane(v, 48)));
+}
+__device__ __forceinline__ void key_max(uint32_t& hi, uint32_t& lo, uint32_t ohi, uint32_t olo) {
+  const bool take = ohi > hi || (ohi == hi && olo > lo);
+  hi = take ? ohi : hi;
+  lo = take ? olo : lo;
+}
+template <int kCtrl>
+__device__ __forceinline__ void key_max_dpp(uint32_t& hi, uint32_t& lo) {
+  key_max(hi, lo, dpp_u32<kCtrl>(hi), dpp_u32<kCtrl>(lo));
+}
+__device__ __forceinline__ uint32_t order_key(float v) {
+  if (v != v) return 0u;                       // NaN: below every real key
+  const uint32_t u = f32_bits(v + 0.0f);       // -0 -> +0
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+template <int kMode, int PER_LANE>
+__global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
+    const float* __restrict__ scores, const float* __restrict__ biased, int32_t* __restrict__ ids,
+    float* __restrict__ weights, int tokens, int n_experts, int top_k, float scaling, int norm_topk) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  if (t >= tokens) return;
+  const size_t row = static_cast<size_t>(t) * n_experts;
+  float sc[PER_LANE];
+  uint32_t key[PER_LANE];
+#pragma unroll
+  for (int j = 0; j < PER_LANE; ++j) {
+    const int e = lane + j * kWaveSize;
+    const bool live = e < n_experts;
+    sc[j] = live ? scores[row + e] : -INFINITY;
+    key[j] = live ? order_key(biased[row + e]) : 0u;
+  }
+  if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
+    float m = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) m = fmaxf(m, sc[j]);
+    m = wave_max_dpp(m);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+      sc[j] = lane + j * kWaveSize < n_experts ? expf(sc[j] - m) : 0.f;
+      sum += sc[j];
+    }
+    sum = wave_sum_dpp(sum);
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) sc[j] = sc[j] / sum;
+  }
+  int sel[16];
+  float wsel[16];
+  for (int r = 0; r < top_k; ++r) {
+    uint32_t hi = 0u, lo = 0u;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) key_max(hi, lo, key[j], ~static_cast<uint32_t>(lane + j * kWaveSize));
+    key_max_dpp<0xB1>(hi, lo);
+    key_max_dpp<0x4E>(hi, lo);
+    key_max_dpp<0x141>(hi, lo);
+    key_max_dpp<0x140>(hi, lo);
+    uint32_t bh = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 0));
+    uint32_t bl = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 0));
+    key_max(bh, bl, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 16)),
+            static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 16)));
+    key_max(bh, bl, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 32)),
+            static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 32)));
+    key_max(bh, bl, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 48)),
+            static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 48)));
+    int best = static_cast<int>(~bl);
+    if (bh == 0u || best < 0 || best >= n_experts) best = 0;   // a row of NaN keys: stay in bounds
+    const int owner = best & (kWaveSize - 1), slot = best >> 6;
+    float mine = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+      if (j == slot) {
+        mine = sc[j];
+        if (lane == owner) key[j] = 0u;          // taken: below every real key
+      }
+    }
+    sel[r] = best;
+    wsel[r] = __shfl(mine, owner);
+  }
+  if (lane != 0) return;
+  for (int i = 1; i < top_k; ++i) {  // ascending expert id
+    const int id = sel[i];
+    const float w = wsel[i];
+    int j = i - 1;
+    while (j >= 0 && sel[j] > id) {
+      sel[j + 1] = sel[j];
+      wsel[j + 1] = wsel[j];
+      --j;
+    }
+    sel[j + 1] = id;
+    wsel[j + 1] = w;
+  }
+  float denom = 0.f;
+  for (int i = 0; i < top_k; ++i) denom += wsel[i];
+  denom += 1e-20f;
+  for (int i = 0; i < top_k; ++i) {
+    float w = norm_topk ? (wsel[i] / denom) * scaling : wsel[i] * scaling;
+    if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) w = bf16_to_f32(f32_to_bf16(w));
+    ids[static_cast<size_t>(t) * top_k + i] = sel[i];
+    weights[static_cast<size_t>(t) * top_k + i] = w;
+  }
+}
+
 // ---- elementwise ------------------------------------------------------------------------------
 __global__ void swiglu_clamp_kernel(const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up,
                                     uint16_t* __restrict__ out, int64_t n, float limit) {
@@ -461,13 +593,31 @@ hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gat
 
 hipError_t run_router_select(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
                              int tokens, int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream) {
-  const size_t lds = 2 * static_cast<size_t>(n_experts) * sizeof(float);
-  if (mode == DGPP_ROUTER_SOFTMAX_TOPK)
-    hipLaunchKernelGGL(router_select_kernel<DGPP_ROUTER_SOFTMAX_TOPK>, dim3(tokens), dim3(kWaveSize), lds, stream, scores,
-                       biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk);
-  else
-    hipLaunchKernelGGL(router_select_kernel<DGPP_ROUTER_SIGMOID_BIAS>, dim3(tokens), dim3(kWaveSize), lds, stream, scores,
-                       biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk);
+  const bool softmax = mode == DGPP_ROUTER_SOFTMAX_TOPK;
+  const dim3 grid(tokens), block(kWaveSize);
+  if (n_experts <= 4 * kWaveSize) {
+    if (softmax)
+      hipLaunchKernelGGL((router_select_reg_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 4>), grid, block, 0, stream, scores, biased,
+                         ids, weights, tokens, n_experts, top_k, scaling, norm_topk);
+    else
+      hipLaunchKernelGGL((router_select_reg_kernel<DGPP_ROUTER_SIGMOID_BIAS, 4>), grid, block, 0, stream, scores, biased,
+                         ids, weights, tokens, n_experts, top_k, scaling, norm_topk);
+  } else if (n_experts <= 8 * kWaveSize) {
+    if (softmax)
+      hipLaunchKernelGGL((router_select_reg_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 8>), grid, block, 0, stream, scores, biased,
+                         ids, weights, tokens, n_experts, top_k, scaling, norm_topk);
+    else
+      hipLaunchKernelGGL((router_select_reg_kernel<DGPP_ROUTER_SIGMOID_BIAS, 8>), grid, block, 0, stream, scores, biased,
+                         ids, weights, tokens, n_experts, top_k, scaling, norm_topk);
+  } else {
+    const size_t lds = 2 * static_cast<size_t>(n_experts) * sizeof(float);
+    if (softmax)
+      hipLaunchKernelGGL(router_select_kernel<DGPP_ROUTER_SOFTMAX_TOPK>, grid, block, lds, stream, scores, biased, ids,
+                         weights, tokens, n_experts, top_k, scaling, norm_topk);
+    else
+      hipLaunchKernelGGL(router_select_kernel<DGPP_ROUTER_SIGMOID_BIAS>, grid, block, lds, stream, scores, biased, ids,
+                         weights, tokens, n_experts, top_k, scaling, norm_topk);
+  }
   return hipGetLastError();
 }
 

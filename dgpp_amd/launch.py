@@ -141,6 +141,12 @@ def launch_moe_slot_accum_routed_f32(out, contrib, weights, tokens, hidden, top_
                                                              _stream(stream)))
 
 
+def launch_moe_slot_accum_routed_bf16(out, contrib, weights, tokens, hidden, top_k, stream=None):
+    """launch_moe_slot_accum_routed_f32 + launch_moe_round_bf16 in one launch (no reference counterpart)."""
+    _check(_lib.load().dgpp_launch_moe_slot_accum_routed_bf16(_p(out), _p(contrib), _p(weights), tokens, hidden, top_k,
+                                                              _stream(stream)))
+
+
 # ---- decode-slot kernels ------------------------------------------------------------------------------
 def launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
                                    sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride,

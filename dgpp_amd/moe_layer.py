@@ -76,6 +76,11 @@ class MoeLayer:
                                                                _p(out_bf16), _p(out_f32), tokens, _stream(stream)))
 
     @property
+    def views_ptr(self) -> int:
+        """Device address of the layer's expert table."""
+        return self._lib.dgpp_moe_layer_views(self._h)
+
+    @property
     def ids_ptr(self) -> int:
         return self._lib.dgpp_moe_layer_ids(self._h)
 

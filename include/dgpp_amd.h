@@ -36,6 +36,15 @@ const char* dgpp_last_error(void);
 /* "gfx950" — the only architecture the library carries code for. */
 const char* dgpp_target_arch(void);
 
+/* Bench A/B switches, process-wide, not thread-safe against concurrent launches (the reference
+ * keeps such a switch in its launcher header too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90).
+ * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: decode-slot kernel
+ * form (0 / 1 LDS-staged activations, 2 register activations + next-step prefetch, 3 register
+ * activations); key 2: row steps per block of the slot launches (0 = automatic). Outputs do not
+ * depend on keys 1 and 2; key 0 changes the fp32 summation order (every launcher follows it alike). */
+void dgpp_tune_set(int key, int value);
+int dgpp_tune_get(int key);
+
 /* ---- POD types shared with device code -------------------------------------------------- */
 
 /* Device-side expert table entry, read by the slot and grouped kernels.
@@ -160,6 +169,12 @@ int dgpp_launch_moe_slot_accum(uint16_t* out, const float* contrib, const float*
                                int tokens, int hidden, int top_k, void* stream);
 int dgpp_launch_moe_slot_accum_routed_f32(float* out, const float* contrib, const float* weights,
                                           int tokens, int hidden, int top_k, void* stream);
+
+/* No counterpart in the reference: launch_moe_slot_accum_routed_f32 followed by launch_moe_round_bf16
+ * (src/kernels/glm_moe_launch.hpp:280, :195) in ONE launch — the routed chain alone rounded once to
+ * bf16, bit for bit the two-launch form. */
+int dgpp_launch_moe_slot_accum_routed_bf16(uint16_t* out, const float* contrib, const float* weights,
+                                           int tokens, int hidden, int top_k, void* stream);
 
 /* ---- FP8 block-scaled decode-slot kernels ------------------------------------------------------ */
 /* src/kernels/glm_moe_launch.hpp:247-253 */

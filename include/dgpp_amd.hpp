@@ -164,6 +164,11 @@ inline void launch_moe_slot_accum_routed_f32(float* out, const float* contrib, c
                                              int hidden, int top_k, hipStream_t stream) {
   detail::check(dgpp_launch_moe_slot_accum_routed_f32(out, contrib, weights, tokens, hidden, top_k, stream));
 }
+// launch_moe_slot_accum_routed_f32 + launch_moe_round_bf16 in one launch (no reference counterpart).
+inline void launch_moe_slot_accum_routed_bf16(uint16_t* out, const float* contrib, const float* weights, int tokens,
+                                              int hidden, int top_k, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_slot_accum_routed_bf16(out, contrib, weights, tokens, hidden, top_k, stream));
+}
 inline void launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
                                            const MoeExpertView* views, int n_routed, int k_routed, int n_shared,
                                            int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,

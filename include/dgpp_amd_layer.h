@@ -65,6 +65,7 @@ int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* layer, const uint16_t* x
                                           const int32_t* ids, const float* weights, uint16_t* out_bf16,
                                           float* out_f32, int tokens, void* stream);
 /* Device pointers of the last routes the layer computed: ids int32 [tokens, top_k], weights f32. */
+const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* layer); /* the device expert table */
 const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* layer);
 const float* dgpp_moe_layer_weights(const DgppMoeLayer* layer);
 

@@ -218,6 +218,9 @@ def test_slot_accum_and_ordered_accum_bit_exact(gpu, T, H, K):
     L.launch_moe_slot_accum_routed_f32(outf, dev(contrib), dev(w), T, H, K, None)
     sync()
     assert np.array_equal(host(outf), f32_want)
+    L.launch_moe_slot_accum_routed_bf16(out, dev(contrib), dev(w), T, H, K, None)   # the fused form
+    sync()
+    assert np.array_equal(host(out, np.uint16), hg.f32_to_bf16(f32_want))
     # grouped layout: rows found through slot_row, slots visited in ascending expert id
     ids = np.stack([rng.permutation(64)[:K] for _ in range(T)]).astype(np.int32)
     slot_row = rng.permutation(T * K).astype(np.int32)
