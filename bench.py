@@ -219,7 +219,7 @@ def main():
         l64 = lg[0].astype(np.float64)
         ids = np.empty((1, K), np.int32)
         w = np.empty((1, K), np.float32)
-        orc.oracle().orc_router_select(orc.p(l64), orc.p(l64.copy()), 1, 1, nE, K, 1.0, 1, orc.p(ids), orc.p(w))
+        orc.oracle().orc_router_select(orc.p(l64), orc.p(l64), 1, 1, nE, K, 1.0, 1, orc.p(ids), orc.p(w))
         mats, hold = [], []
         zero8 = np.zeros(1, np.uint8)
         used = set(int(v) for v in ids.ravel())

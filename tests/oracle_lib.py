@@ -3,6 +3,7 @@ compiled reference oracle (oracle/_ref/libdgpp_ref.so). Test infrastructure only
 from __future__ import annotations
 
 import ctypes as C
+import sys
 import subprocess
 from pathlib import Path
 
@@ -92,6 +93,9 @@ def p(a):
     if a is None:
         return None
     assert a.flags["C_CONTIGUOUS"], "oracle inputs must be contiguous"
+    # The address outlives this call only if the caller holds the array: a temporary (held by
+    # nothing but the call's own stack slot, this frame and getrefcount) would be freed first.
+    assert sys.getrefcount(a) > 3, "pass a named array: the address of a temporary dangles before the C call"
     return a.ctypes.data
 
 

@@ -100,7 +100,7 @@ def test_layer_from_given_scores_softmax(gpu):
     sync()
     l64 = logits.astype(np.float64)
     ids, w = np.empty((T, K), np.int32), np.empty((T, K), np.float32)
-    orc.oracle().orc_router_select(orc.p(l64), orc.p(l64.copy()), 1, T, E, K, 1.0, 1, orc.p(ids), orc.p(w))
+    orc.oracle().orc_router_select(orc.p(l64), orc.p(l64), 1, T, E, K, 1.0, 1, orc.p(ids), orc.p(w))
     raw, _ = moe_data.orc_forward(p, ids, w)
     expert_budget(host(out, np.uint16), raw, "scores-driven layer")
     layer.close()

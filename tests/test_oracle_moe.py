@@ -67,7 +67,7 @@ def test_router_tie_rule_all_equal_scores():
     scores = np.full((T, E), 0.5)
     ids = np.empty((T, K), np.int32)
     w = np.empty((T, K), np.float32)
-    orc.oracle().orc_router_select(orc.p(scores), orc.p(scores.copy()), 0, T, E, K, 2.5, 1, orc.p(ids), orc.p(w))
+    orc.oracle().orc_router_select(orc.p(scores), orc.p(scores), 0, T, E, K, 2.5, 1, orc.p(ids), orc.p(w))
     assert np.array_equal(ids, np.tile(np.arange(K, dtype=np.int32), (T, 1)))
     assert np.allclose(w, 0.5 / (K * 0.5) * 2.5, rtol=1e-7)
     # selection key and weight source are different rows: pick by biased, weigh by scores
@@ -85,7 +85,7 @@ def test_router_select_brute_force():
     scores = hg.bf16_to_f32(hg.f32_to_bf16(scores.astype(np.float32))).astype(np.float64)
     ids = np.empty((T, K), np.int32)
     w = np.empty((T, K), np.float32)
-    orc.oracle().orc_router_select(orc.p(scores), orc.p(scores.copy()), 1, T, E, K, 1.0, 1, orc.p(ids), orc.p(w))
+    orc.oracle().orc_router_select(orc.p(scores), orc.p(scores), 1, T, E, K, 1.0, 1, orc.p(ids), orc.p(w))
     for t in range(T):
         order = sorted(range(E), key=lambda e: (-scores[t, e], e))[:K]
         assert list(ids[t]) == sorted(order)
