@@ -31,6 +31,10 @@ HBM_PEAK_GBPS = 8000.0
 E, H, I, K = 256, 4096, 1024, 8          # BASELINE config 3 (MXFP4 MoE decode layer)
 EXPERT_BYTES = 3 * I * H // 2 + 3 * I * H // 32          # payload + e8m0 scales of gate, up, down
 GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
+# HBM-side bytes per launch of the two GEMV kernels at the default workload (T = 8, 256 experts), from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the library's plain copy kernel (the summary under
+# profiles/ holds the commands and the raw counters). A counter cannot be read from inside this process.
+MEASURED_TRAFFIC = {"gate_up": 287.3e6, "down": 145.0e6}
 DOWN_BYTES = H * I // 2 + H * I // 32
 
 
@@ -44,6 +48,10 @@ def parse():
     ap.add_argument("--experts", type=int, default=E, help="experts per layer (256 = the BASELINE shape)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="'layer', 'gate_up' or 'down': run only that timed graph (for profiling)")
+    ap.add_argument("--no-others", action="store_true", help="skip the T=1/4/8 side measurements")
+    ap.add_argument("--eager", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
+    ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
+                    help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -123,6 +131,14 @@ def main():
             for i in range(max(warmup, 1)):
                 enqueue(i)
             stream.synchronize()
+            if args.eager:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for i in range(steps):
+                    enqueue(i)
+                e1.record(stream)
+                torch.cuda.synchronize()
+                return e0.elapsed_time(e1) * 1e-3 / steps
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=stream):
                 for i in range(steps):
@@ -202,10 +218,21 @@ def main():
     for lyr in layers:     # device pointer of the layer's expert table, for the single-kernel leg
         lyr._views_ptr = lyr.views_ptr
 
+    if args.probe_copy > 0:
+        nbytes = args.probe_copy << 20
+        src = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        with torch.cuda.stream(stream):
+            for _ in range(3):
+                if lib.dgpp_probe_copy(dst.data_ptr(), src.data_ptr(), nbytes, stream.cuda_stream) != 0:
+                    raise RuntimeError(lib.dgpp_last_error().decode())
+            stream.synchronize()
+        del src, dst
+
     T = args.tokens
     main_res = measure(T, args.steps, args.warmup, args.only)
     others = {}
-    if not args.only and not args.tune:
+    if not args.only and not args.tune and not args.no_others:
         for t in (1, 4, 8):
             if t != T:
                 others[f"T{t}"] = measure(t, args.steps, args.warmup)
@@ -287,7 +314,8 @@ def main():
     if "gate_up_us" in main_res:
         line["roofline"] = {"kernel": "slot_gate_up_kernel<MXFP4> (fused gate/up GEMV + SwiGLU)", "bound": "hbm",
                             "achieved": main_res["gate_up_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                            "frac": main_res["gate_up_gbps"] / HBM_PEAK_GBPS, "traffic": None,
+                            "frac": main_res["gate_up_gbps"] / HBM_PEAK_GBPS,
+                            "traffic": MEASURED_TRAFFIC["gate_up"] if (T == 8 and nE == E and not args.tune) else None,
                             "bytes_per_launch": main_res["gate_up_bytes"], "us_per_launch": main_res["gate_up_us"]}
         if "down_us" in main_res:
             line["roofline"]["second_kernel"] = {

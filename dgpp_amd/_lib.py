@@ -68,6 +68,7 @@ SIGNATURES = {
     "dgpp_target_arch": (C.c_char_p, []),
     "dgpp_tune_set": (None, [_I, _I]),
     "dgpp_tune_get": (_I, [_I]),
+    "dgpp_probe_copy": (_I, [_P, _P, C.c_size_t, _P]),
     "dgpp_moe_config_validate": (_I, [_P]),
     "dgpp_launch_moe_router": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_launch_moe_router_select": (_I, [_P, _P, _P, _P, _P, _I, _P]),

@@ -263,6 +263,14 @@ extern "C" {
 
 const char* dgpp_last_error(void) { return g_last_error.c_str(); }
 const char* dgpp_target_arch(void) { return "gfx950"; }
+int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
+  const char* who = "probe copy";
+  if (bytes == 0) return DGPP_OK;
+  if (!dst || !src) return fail_arg(std::string(who) + ": null pointer");
+  if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0)
+    return fail_arg(std::string(who) + ": bytes and both pointers must be multiples of 16");
+  return finish(run_probe_copy(dst, src, bytes, as_stream(stream)), who);
+}
 void dgpp_tune_set(int key, int value) {
   if (key >= 0 && key < kTuneCount) g_tune[key] = value;
 }

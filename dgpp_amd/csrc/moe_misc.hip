@@ -679,6 +679,23 @@ hipError_t run_accum_ordered(void* out, int out_f32, const float* down, size_t d
   return hipGetLastError();
 }
 
+// Plain streaming copy, 16 bytes per lane per step, grid-stride: the calibration workload for
+// a profiler's HBM byte counters.
+__global__ __launch_bounds__(256) void probe_copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n16) {
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride)
+    dst[i] = src[i];
+}
+
+hipError_t run_probe_copy(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+  const size_t n16 = bytes / 16;
+  const size_t want = (n16 + 255) / 256;
+  const unsigned blocks = static_cast<unsigned>(want < 1 ? 1 : (want > 16384 ? 16384 : want));
+  hipLaunchKernelGGL(probe_copy_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<uint4*>(dst),
+                     static_cast<const uint4*>(src), n16);
+  return hipGetLastError();
+}
+
 hipError_t run_segment(const int32_t* ids, int tokens, int top_k, int n_experts, int32_t* rows, int32_t* slot_row,
                        DgppMoeSegment* segs, hipStream_t stream) {
   hipLaunchKernelGGL(segment_kernel, dim3(n_experts + 1), dim3(kSegThreads), 0, stream, ids, tokens, top_k, n_experts,

@@ -33,6 +33,7 @@ hipError_t run_tile_list(const DgppMoeSegment* segs, int n_segs, int tile_rows, 
                          hipStream_t stream);
 hipError_t run_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* output, int experts, int capacity,
                                 hipStream_t stream);
+hipError_t run_probe_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 hipError_t run_fp8_dequant(const uint8_t* payload, const void* scales, int e8m0, uint16_t* out, int64_t rows,
                            int64_t cols, int rs, int cs, hipStream_t stream);
 

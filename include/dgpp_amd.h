@@ -45,6 +45,11 @@ const char* dgpp_target_arch(void);
 void dgpp_tune_set(int key, int value);
 int dgpp_tune_get(int key);
 
+/* Measurement aid with no counterpart in the reference: a plain streaming copy of `bytes`
+ * (a multiple of 16; both pointers 16-byte aligned) on `stream`. A profiler's HBM byte counters
+ * are calibrated against it: it reads `bytes` and writes `bytes`, nothing else. */
+int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
+
 /* ---- POD types shared with device code -------------------------------------------------- */
 
 /* Device-side expert table entry, read by the slot and grouped kernels.

@@ -23,6 +23,11 @@ using MoeTile = DgppMoeTile;               // src/kernels/glm_moe_launch.hpp:151
 using GlmFp4Matrix = DgppFp4Matrix;        // src/models/quant_matrix.hpp:117
 using Fp8GemvProblem = DgppFp8GemvProblem; // src/kernels/scale_gemm.hpp:85
 
+// The device code reads these by offset: the sizes are part of the ABI.
+static_assert(sizeof(MoeExpertView) == 96 && sizeof(MoeSegment) == 12 && sizeof(MoeTile) == 8 &&
+                  sizeof(GlmFp4Matrix) == 56,
+              "POD layouts shared with the kernels");
+
 constexpr int kFp4Group = 16;
 constexpr int kMxfp4Group = 32;
 
