@@ -91,6 +91,8 @@ SIGNATURES = {
     "dgpp_launch_moe_slot_down": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_launch_moe_slot_gate_up_swiglu_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I, _I, _I]),
     "dgpp_launch_moe_slot_down_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _P]),
+    "dgpp_launch_moe_slot_down_accum": (_I, [_P, _Z, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
+    "dgpp_launch_moe_slot_down_accum_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P, _I]),
     "dgpp_launch_moe_grouped_gemv_bf16": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
     "dgpp_launch_moe_grouped_gemv_f32": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
     "dgpp_launch_moe_grouped_gemv_fp4_bf16": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _I]),

@@ -556,6 +556,54 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
   return finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
 }
 
+// Routed-only down + ordered accumulation in one launch (no counterpart in the reference, which runs
+// launch_moe_slot_down* and launch_moe_slot_accum* back to back).
+static int slot_down_accum(int fmt, const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                           const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride, int slots,
+                           int top_k, const float* weights, uint16_t* out_bf16, float* out_f32, int* arrive,
+                           size_t arrive_len, void* stream, const char* who) {
+  if (slots <= 0) return DGPP_OK;
+  if (!act || !ids || !views || !slot_down || !weights || !arrive || (!out_bf16 && !out_f32))
+    return fail_arg(std::string(who) + ": null pointer");
+  if (n <= 0 || k <= 0 || top_k <= 0 || slots % (top_k + 1) != 0) return fail_arg(std::string(who) + ": degenerate dims");
+  if (out_stride < n) return fail_arg(std::string(who) + ": out_stride below n");
+  const size_t tokens = static_cast<size_t>(slots / (top_k + 1));
+  if (arrive_len < tokens * static_cast<size_t>((n + 3) / 4))
+    return fail_arg(std::string(who) + ": the arrival counters must hold tokens * ceil(n / 4) ints");
+  SlotArgs a = slot_args(act, act_stride, ids, order, views, slot_down, out_stride, slots, top_k, 0.f);
+  a.n = n;
+  a.k = k;
+  a.want_shared = 0;
+  a.arrive = arrive;
+  a.arrivals = top_k;
+  a.weights = weights;
+  a.final_out = out_f32 ? static_cast<void*>(out_f32) : static_cast<void*>(out_bf16);
+  a.final_f32 = out_f32 != nullptr;
+  a.final_shared = 0;
+  return finish(launch_slot_down(fmt, a, as_stream(stream)), who);
+}
+int dgpp_launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                    const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride,
+                                    int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
+                                    int* arrive, size_t arrive_len, void* stream) {
+  const char* who = "moe_slot_down_accum";
+  if (slots > 0 && (k % 16 != 0 || stage_bytes(1, k) > kMaxLdsBytes))
+    return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
+  return slot_down_accum(kFmtFp8F32, act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots, top_k,
+                         weights, out_bf16, out_f32, arrive, arrive_len, stream, who);
+}
+int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                        const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride,
+                                        int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
+                                        int* arrive, size_t arrive_len, void* stream, int fp4_group) {
+  const char* who = "moe_slot_down_accum_fp4";
+  if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
+  if (slots > 0 && (!fp4_k_supported(k) || !fp4_k_compiled(k, fp4_group)))
+    return fail_arg(std::string(who) + ": k must be a multiple of 32 in the fp4 core's compiled set");
+  return slot_down_accum(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, ids, order, views, n, k, slot_down,
+                         out_stride, slots, top_k, weights, out_bf16, out_f32, arrive, arrive_len, stream, who);
+}
+
 static int grouped_fp8(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
                        int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
                        size_t out_stride, int n, int k, void* stream) {

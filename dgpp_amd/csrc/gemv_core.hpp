@@ -67,7 +67,7 @@ struct RowGeom {
 };
 // Bench A/B switches (host side, process-wide; 0 = the default behaviour). Set through
 // dgpp_tune_set; launchers read them when they pick a geometry or a kernel form.
-enum : int { kTunePreferP = 0, kTuneSlotForm = 1, kTuneSlotSteps = 2, kTuneCount = 8 };
+enum : int { kTunePreferP = 0, kTuneSlotRun = 1, kTuneSlotSteps = 2, kTuneCount = 8 };
 int tune_get(int key);
 
 __host__ __device__ inline RowGeom row_geom(int chunks, int prefer_p = 4) {
@@ -360,15 +360,17 @@ __device__ __forceinline__ float chunk_dot1(const ChunkRegs& ch, const uint4* xv
   return acc;
 }
 
-// Two weight rows of the same geometry (a slot's gate and up rows) against ONE staged activation
-// row: both rows' loads are issued together and each chunk column's activation vectors are read
-// from LDS once for the pair. Each row's chain is row_dots' chain, bit for bit.
-template <int FMT, int NB>
+// Two weight rows of the same geometry (a slot's gate and up rows) against the SAME m staged
+// activation rows: both rows' loads are issued together and each chunk column's activation vectors
+// are read from LDS once for the pair. Each (row, activation row) chain is row_dots' chain, bit for
+// bit.
+template <int FMT, int NB, int MAXM>
 __device__ __forceinline__ void row_dots_pair(const LaneRow& la, const LaneRow& lb, const RowGeom& g, int csa,
-                                              int csb, const uint4* __restrict__ lds, int chunks, float& ra,
-                                              float& rb) {
+                                              int csb, const uint4* __restrict__ lds, int chunks, int m,
+                                              float (&ra)[MAXM], float (&rb)[MAXM]) {
   constexpr int kPieces = FmtTraits<FMT>::kPieces;
-  float a = 0.f, b = 0.f;
+#pragma unroll
+  for (int r = 0; r < MAXM; ++r) ra[r] = rb[r] = 0.f;
   const int passes = g.P / NB;
   for (int p = 0; p < passes; ++p) {
     ChunkRegs ca[NB], cb[NB];
@@ -377,15 +379,25 @@ __device__ __forceinline__ void row_dots_pair(const LaneRow& la, const LaneRow& 
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       const int c = ((p * NB + i) << g.l2) + la.li;
-      uint4 xv[kPieces];
+      if constexpr (MAXM == 1) {
+        uint4 xv[kPieces];
 #pragma unroll
-      for (int q = 0; q < kPieces; ++q) xv[q] = lds[q * chunks + c];
-      a = chunk_dot1<FMT>(ca[i], xv, a);
-      b = chunk_dot1<FMT>(cb[i], xv, b);
+        for (int q = 0; q < kPieces; ++q) xv[q] = lds[q * chunks + c];
+        ra[0] = chunk_dot1<FMT>(ca[i], xv, ra[0]);
+        rb[0] = chunk_dot1<FMT>(cb[i], xv, rb[0]);
+      } else {
+        consume_chunk<FMT, MAXM>(ca[i], XLds<FMT>{lds + c, chunks}, m, ra);
+        consume_chunk<FMT, MAXM>(cb[i], XLds<FMT>{lds + c, chunks}, m, rb);
+      }
     }
   }
-  ra = group_sum(a, g.l2);
-  rb = group_sum(b, g.l2);
+#pragma unroll
+  for (int r = 0; r < MAXM; ++r) {
+    if (r < m) {
+      ra[r] = group_sum(ra[r], g.l2);
+      rb[r] = group_sum(rb[r], g.l2);
+    }
+  }
 }
 
 // Dispatches a callable on the compile-time pass width.

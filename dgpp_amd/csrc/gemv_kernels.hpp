@@ -121,7 +121,13 @@ struct SlotArgs {
   float limit;
   int want_shared;          // 0: routed slots, 1: shared slots (others exit)
   int shared_view_base;     // >= 0: shared matrices come from views[base + which]
-  int debug_nomath;         // bench probe: loads only
+  // Down only, optional: the ordered accumulation fused behind the last slot of a token.
+  int* arrive;              // [tokens, row tiles] arrival counters, zero at rest (left zero); null = not fused
+  int arrivals;             // slots per token whose down rows this launch produces
+  const float* weights;     // [tokens, top_k]
+  void* final_out;          // [tokens, n] bf16 bits or f32
+  int final_f32;
+  int final_shared;         // the chain ends with the token's shared slot (weight 1)
 };
 
 template <int FMT>
@@ -143,241 +149,196 @@ __device__ __forceinline__ MatRef mat_of_view(const DgppMoeExpertView& v, const 
   return m;
 }
 
-// Resolves the slot of this block; false when the block has nothing to do.
-__device__ __forceinline__ bool resolve_slot(const SlotArgs& a, int& slot, int& token, int& view_base) {
-  if (static_cast<int>(blockIdx.y) >= a.slots) return false;
-  slot = a.order ? a.order[blockIdx.y] : static_cast<int>(blockIdx.y);
+// The slots one block serves: a RUN of up to MAXM slots that follow each other in `order` and use
+// the same expert (the order sorts slots by expert; the shared slots of all tokens form one run).
+// The expert's rows are then read once for the whole run. A position is the run's leader when the
+// count of same-expert positions right before it is a multiple of MAXM; other blocks exit.
+template <int MAXM>
+struct SlotRun {
+  int m;
+  int slot[MAXM];
+  int token[MAXM];
+  int view_base;   // index of the expert's gate view, or < 0: matrices from the launch arguments
+};
+
+// Expert key of a logical slot (-1 for the shared slot) and its token.
+__device__ __forceinline__ int slot_key(const SlotArgs& a, int slot, int& token) {
   token = slot / (a.top_k + 1);
   const int j = slot - token * (a.top_k + 1);
-  const bool shared = j == a.top_k;
-  if (shared != (a.want_shared != 0)) return false;
-  view_base = shared ? a.shared_view_base : a.ids[static_cast<size_t>(token) * a.top_k + j] * 3;
+  return j == a.top_k ? -1 : a.ids[static_cast<size_t>(token) * a.top_k + j];
+}
+
+template <int MAXM>
+__device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& run) {
+  const int p = static_cast<int>(blockIdx.y);
+  if (p >= a.slots) return false;
+  const int slot0 = a.order ? a.order[p] : p;
+  int token0;
+  const int key0 = slot_key(a, slot0, token0);
+  if ((key0 < 0) != (a.want_shared != 0)) return false;
+  run.m = 1;
+  run.slot[0] = slot0;
+  run.token[0] = token0;
+  run.view_base = key0 < 0 ? a.shared_view_base : key0 * 3;
+  if constexpr (MAXM > 1) {
+    if (a.order) {
+      int back = 0, t;
+      while (p - back - 1 >= 0 && slot_key(a, a.order[p - back - 1], t) == key0) ++back;
+      if (back % MAXM != 0) return false;
+      bool alive = true;
+#pragma unroll
+      for (int r = 1; r < MAXM; ++r) {
+        run.slot[r] = slot0;
+        run.token[r] = token0;
+        if (alive && p + r < a.slots) {
+          const int s = a.order[p + r];
+          if (slot_key(a, s, t) == key0) {
+            run.slot[r] = s;
+            run.token[r] = t;
+            run.m = r + 1;
+          } else {
+            alive = false;
+          }
+        } else {
+          alive = false;
+        }
+      }
+    }
+  }
   return true;
 }
 
-template <int FMT, int NB>
+template <int FMT, int NB, int MAXM>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
-  int slot, token, base;
-  if (!resolve_slot(a, slot, token, base)) return;
+  SlotRun<MAXM> run;
+  if (!resolve_run<MAXM>(a, run)) return;
   const int rows_per_block = block_rows(g, steps);
   if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
   MatRef mg, mu;
   const float *gg = nullptr, *gu = nullptr;
-  if (base >= 0) {
-    mg = mat_of_view<FMT>(a.views[base + 0], &gg);
-    mu = mat_of_view<FMT>(a.views[base + 1], &gu);
+  if (run.view_base >= 0) {
+    mg = mat_of_view<FMT>(a.views[run.view_base + 0], &gg);
+    mu = mat_of_view<FMT>(a.views[run.view_base + 1], &gu);
   } else {
     mg = a.sh[0];
     mu = a.sh[1];
   }
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
-  stage_activations<FMT>(a.x + static_cast<size_t>(token) * a.x_stride, a.x_stride, 1, a.k, lds);
+  const int row_vecs = FmtTraits<FMT>::kPieces * chunks;
+#pragma unroll
+  for (int r = 0; r < MAXM; ++r)
+    if (r < run.m)
+      stage_activations<FMT>(a.x + static_cast<size_t>(run.token[r]) * a.x_stride, a.x_stride, 1, a.k, lds + r * row_vecs);
   __syncthreads();
   const float dg = load_divisor<FMT>(gg), du = load_divisor<FMT>(gu);
   const int rpw = kWave >> g.l2;
   const int wave = threadIdx.x >> 6;
-  uint16_t* act_row = static_cast<uint16_t*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
+  uint16_t* act = static_cast<uint16_t*>(a.out);
   int row0 = blockIdx.x * rows_per_block + wave * rpw;
   for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
     if (row0 >= a.n) break;
     const LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
     const LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
-    float ag, au;
-    row_dots_pair<FMT, NB>(lg, lu, g, mg.cs, mu.cs, lds, chunks, ag, au);
-    if (lg.li == 0 && lg.row < a.n)
-      act_row[lg.row] = swiglu_bf16(finish_dot<FMT>(ag, dg), finish_dot<FMT>(au, du), a.limit);
+    float ag[MAXM], au[MAXM];
+    row_dots_pair<FMT, NB, MAXM>(lg, lu, g, mg.cs, mu.cs, lds, chunks, run.m, ag, au);
+    if (lg.li == 0 && lg.row < a.n) {
+#pragma unroll
+      for (int r = 0; r < MAXM; ++r)
+        if (r < run.m)
+          act[static_cast<size_t>(run.slot[r]) * a.out_stride + lg.row] =
+              swiglu_bf16(finish_dot<FMT>(ag[r], dg), finish_dot<FMT>(au[r], du), a.limit);
+    }
   }
 }
 
-template <int FMT, int NB>
+// Down rows of a run of slots, unrounded f32. With `arrive` set, the block that completes a token's
+// last outstanding slot for its row tile also runs that token's accumulation chain over the tile
+// (a = 0; a = fma(w_j, y_j, a) for j ascending; the shared row last with weight 1; one rounding):
+// every block counts in once per slot after publishing its rows, the counter names the last one, so
+// no block ever waits for another. The chain's order is fixed, whoever runs it.
+template <int FMT, int NB, int MAXM>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
-  int slot, token, base;
-  if (!resolve_slot(a, slot, token, base)) return;
+  __shared__ int s_last[MAXM];
+  SlotRun<MAXM> run;
+  if (!resolve_run<MAXM>(a, run)) return;
   const int rows_per_block = block_rows(g, steps);
-  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
+  const int tile_row0 = static_cast<int>(blockIdx.x) * rows_per_block;
+  if (tile_row0 >= a.n) return;
   MatRef md;
   const float* gd = nullptr;
-  if (base >= 0)
-    md = mat_of_view<FMT>(a.views[base + 2], &gd);
+  if (run.view_base >= 0)
+    md = mat_of_view<FMT>(a.views[run.view_base + 2], &gd);
   else
     md = a.sh[0];
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
-  // The down projection consumes this slot's own activation row.
-  stage_activations<FMT>(a.x + static_cast<size_t>(slot) * a.x_stride, a.x_stride, 1, a.k, lds);
+  const int row_vecs = FmtTraits<FMT>::kPieces * chunks;
+  // The down projection consumes each slot's own activation row.
+#pragma unroll
+  for (int r = 0; r < MAXM; ++r)
+    if (r < run.m)
+      stage_activations<FMT>(a.x + static_cast<size_t>(run.slot[r]) * a.x_stride, a.x_stride, 1, a.k, lds + r * row_vecs);
   __syncthreads();
   const float dd = load_divisor<FMT>(gd);
   const int rpw = kWave >> g.l2;
   const int wave = threadIdx.x >> 6;
-  float* out_row = static_cast<float*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
-  int row0 = blockIdx.x * rows_per_block + wave * rpw;
+  float* out = static_cast<float*>(a.out);
+  int row0 = tile_row0 + wave * rpw;
   for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
     if (row0 >= a.n) break;
     const LaneRow lr = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
-    float acc[1];
-    row_dots<FMT, 1, NB>(lr, g, md.cs, lds, chunks, 1, acc);
-    if (lr.li == 0 && lr.row < a.n) out_row[lr.row] = finish_dot<FMT>(acc[0], dd);
-  }
-}
-
-// ---- decode slots, register-resident activations ---------------------------------------------------
-// The slot kernels' fast form when a row fits ONE pass (P == NB chunks per lane) and the activation
-// row is 16-byte aligned: a lane's chunk columns are the same for every weight row it visits, so it
-// loads its own slice of the activation row into registers ONCE (straight from global memory: no
-// LDS, no barrier) and then streams weight rows: both matrices of a step are issued together and
-// the next step's loads are issued before the current step is consumed, so a lane keeps up to
-// 4 * NB 16-byte loads in flight. The per-(row) arithmetic — chunk order per lane, dot2 order,
-// butterfly — is exactly the LDS form's: the two are bitwise twins.
-template <int FMT, int NB>
-struct XSlice {
-  uint4 v[NB * FmtTraits<FMT>::kPieces];
-};
-template <int FMT, int NB>
-__device__ __forceinline__ void load_x_slice(const uint16_t* __restrict__ x, int li, int l2, XSlice<FMT, NB>& xs) {
-  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+    float acc[MAXM];
+    row_dots<FMT, MAXM, NB>(lr, g, md.cs, lds, chunks, run.m, acc);
+    if (lr.li == 0 && lr.row < a.n) {
 #pragma unroll
-  for (int i = 0; i < NB; ++i) {
-    const int c = (i << l2) + li;
-#pragma unroll
-    for (int q = 0; q < kPieces; ++q)
-      xs.v[i * kPieces + q] = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(c * kPieces + q) * 8);
+      for (int r = 0; r < MAXM; ++r)
+        if (r < run.m) out[static_cast<size_t>(run.slot[r]) * a.out_stride + lr.row] = finish_dot<FMT>(acc[r], dd);
+    }
   }
-}
-template <int FMT, int NB>
-__device__ __forceinline__ float dot_pass_reg(const ChunkRegs (&regs)[NB], const XSlice<FMT, NB>& xs, int l2) {
-  float acc[1] = {0.f};
+  if (a.arrive == nullptr) return;
+  // Publish this block's rows, then count in once per slot of the run.
+  __threadfence();
+  __syncthreads();
+  if (static_cast<int>(threadIdx.x) < MAXM) {
+    int last = 0;
 #pragma unroll
-  for (int i = 0; i < NB; ++i)
-    consume_chunk<FMT, 1>(regs[i], XReg<FMT>{xs.v + i * FmtTraits<FMT>::kPieces}, 1, acc);
-  return group_sum(acc[0], l2);
-}
-
-template <int FMT, int NB, bool PREFETCH>
-__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_reg_kernel(SlotArgs a, RowGeom g, int steps) {
-  int slot, token, base;
-  if (!resolve_slot(a, slot, token, base)) return;
-  const int rows_per_block = block_rows(g, steps);
-  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
-  MatRef mg, mu;
-  const float *gg = nullptr, *gu = nullptr;
-  if (base >= 0) {
-    mg = mat_of_view<FMT>(a.views[base + 0], &gg);
-    mu = mat_of_view<FMT>(a.views[base + 1], &gu);
-  } else {
-    mg = a.sh[0];
-    mu = a.sh[1];
-  }
-  const int rpw = kWave >> g.l2;
-  const int wave = threadIdx.x >> 6;
-  const int stride = kWavesPerBlock * rpw;
-  int row0 = blockIdx.x * rows_per_block + wave * rpw;
-  if (row0 >= a.n) return;
-  // The first step's weight loads go out before anything else (the longest latency of the block).
-  LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
-  LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
-  ChunkRegs cg[NB], cu[NB];
-  issue_pass<FMT, NB>(lg, 0, g.l2, mg.cs, cg);
-  issue_pass<FMT, NB>(lu, 0, g.l2, mu.cs, cu);
-  XSlice<FMT, NB> xs;
-  load_x_slice<FMT, NB>(a.x + static_cast<size_t>(token) * a.x_stride, lg.li, g.l2, xs);
-  const float dg = load_divisor<FMT>(gg), du = load_divisor<FMT>(gu);
-  uint16_t* act_row = static_cast<uint16_t*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
-  for (int s = 0; s < steps; ++s) {
-    const int next0 = row0 + stride;
-    const bool has_next = s + 1 < steps && next0 < a.n;
-    ChunkRegs ng[NB], nu[NB];
-    LaneRow lgn = lg, lun = lu;
-    if (has_next) {
-      lgn = lane_row<FMT>(mg, next0, a.n, a.k, g.l2);
-      lun = lane_row<FMT>(mu, next0, a.n, a.k, g.l2);
-      if constexpr (PREFETCH) {
-        issue_pass<FMT, NB>(lgn, 0, g.l2, mg.cs, ng);
-        issue_pass<FMT, NB>(lun, 0, g.l2, mu.cs, nu);
+    for (int r = 0; r < MAXM; ++r) {
+      if (r == static_cast<int>(threadIdx.x) && r < run.m) {
+        int* counter = a.arrive + static_cast<size_t>(run.token[r]) * gridDim.x + blockIdx.x;
+        if (atomicAdd(counter, 1) == a.arrivals - 1) {
+          *counter = 0;   // zero at rest: nobody else touches this counter before the next launch
+          last = 1;
+        }
       }
     }
-    float ag, au;
-    if (a.debug_nomath) {
-      uint32_t t = 0;
+    s_last[threadIdx.x] = last;
+  }
+  __syncthreads();
+  const int tile_end = min(a.n, tile_row0 + rows_per_block);
 #pragma unroll
-      for (int i = 0; i < NB; ++i) t ^= cg[i].w.x ^ cg[i].w.y ^ cg[i].w.z ^ cg[i].w.w ^ cu[i].w.x ^ cu[i].w.y ^ cu[i].w.z ^ cu[i].w.w ^ cg[i].s ^ cu[i].s;
-      ag = au = bits_f32(t & 0x3FFFFFFFu);
-    } else {
-      ag = dot_pass_reg<FMT, NB>(cg, xs, g.l2);
-      au = dot_pass_reg<FMT, NB>(cu, xs, g.l2);
-    }
-    if (lg.li == 0 && lg.row < a.n)
-      act_row[lg.row] = swiglu_bf16(finish_dot<FMT>(ag, dg), finish_dot<FMT>(au, du), a.limit);
-    if (!has_next) break;
-    if constexpr (PREFETCH) {
-#pragma unroll
-      for (int i = 0; i < NB; ++i) {
-        cg[i] = ng[i];
-        cu[i] = nu[i];
+  for (int r = 0; r < MAXM; ++r) {
+    if (r >= run.m || !s_last[r]) continue;
+    __threadfence();   // the other slots' rows, published before their blocks counted in
+    const int t = run.token[r];
+    const size_t slot_base = static_cast<size_t>(t) * (a.top_k + 1);
+    for (int row = tile_row0 + static_cast<int>(threadIdx.x); row < tile_end; row += kBlockThreads) {
+      float v = 0.f;
+      for (int j = 0; j < a.top_k; ++j) {
+        const float y = __hip_atomic_load(out + (slot_base + j) * a.out_stride + row, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT);
+        v = fmaf(a.weights[static_cast<size_t>(t) * a.top_k + j], y, v);
       }
-    } else {
-      issue_pass<FMT, NB>(lgn, 0, g.l2, mg.cs, cg);
-      issue_pass<FMT, NB>(lun, 0, g.l2, mu.cs, cu);
+      if (a.final_shared)
+        v = fmaf(1.0f, __hip_atomic_load(out + (slot_base + a.top_k) * a.out_stride + row, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT), v);
+      const size_t at = static_cast<size_t>(t) * a.n + row;
+      if (a.final_f32)
+        static_cast<float*>(a.final_out)[at] = v;
+      else
+        static_cast<uint16_t*>(a.final_out)[at] = f32_to_bf16(v);
     }
-    lg = lgn;
-    lu = lun;
-    row0 = next0;
   }
-}
-
-template <int FMT, int NB, bool PREFETCH>
-__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_reg_kernel(SlotArgs a, RowGeom g, int steps) {
-  int slot, token, base;
-  if (!resolve_slot(a, slot, token, base)) return;
-  const int rows_per_block = block_rows(g, steps);
-  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
-  MatRef md;
-  const float* gd = nullptr;
-  if (base >= 0)
-    md = mat_of_view<FMT>(a.views[base + 2], &gd);
-  else
-    md = a.sh[0];
-  const int rpw = kWave >> g.l2;
-  const int wave = threadIdx.x >> 6;
-  const int stride = kWavesPerBlock * rpw;
-  int row0 = blockIdx.x * rows_per_block + wave * rpw;
-  if (row0 >= a.n) return;
-  LaneRow lr = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
-  ChunkRegs cur[NB];
-  issue_pass<FMT, NB>(lr, 0, g.l2, md.cs, cur);
-  XSlice<FMT, NB> xs;
-  load_x_slice<FMT, NB>(a.x + static_cast<size_t>(slot) * a.x_stride, lr.li, g.l2, xs);
-  const float dd = load_divisor<FMT>(gd);
-  float* out_row = static_cast<float*>(a.out) + static_cast<size_t>(slot) * a.out_stride;
-  for (int s = 0; s < steps; ++s) {
-    const int next0 = row0 + stride;
-    const bool has_next = s + 1 < steps && next0 < a.n;
-    ChunkRegs nxt[NB];
-    LaneRow ln = lr;
-    if (has_next) {
-      ln = lane_row<FMT>(md, next0, a.n, a.k, g.l2);
-      if constexpr (PREFETCH) issue_pass<FMT, NB>(ln, 0, g.l2, md.cs, nxt);
-    }
-    const float acc = dot_pass_reg<FMT, NB>(cur, xs, g.l2);
-    if (lr.li == 0 && lr.row < a.n) out_row[lr.row] = finish_dot<FMT>(acc, dd);
-    if (!has_next) break;
-    if constexpr (PREFETCH) {
-#pragma unroll
-      for (int i = 0; i < NB; ++i) cur[i] = nxt[i];
-    } else {
-      issue_pass<FMT, NB>(ln, 0, g.l2, md.cs, cur);
-    }
-    lr = ln;
-    row0 = next0;
-  }
-}
-
-// The register form applies when the whole row is one pass and the lane's activation slice stays
-// within 64 registers.
-template <int FMT>
-inline bool slot_reg_form_ok(const RowGeom& g, const SlotArgs& a) {
-  const int xregs = g.P * FmtTraits<FMT>::kPieces * 4;
-  return g.P == g.nb && xregs <= 64 && ((reinterpret_cast<uintptr_t>(a.x) & 15u) == 0) && ((a.x_stride & 7u) == 0);
 }
 
 // ---- grouped (segment-major) twin ------------------------------------------------------------------
@@ -504,12 +465,17 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
   return err != hipSuccess ? err : hipGetLastError();
 }
 
-// Row steps per block of a slot launch: about four resident rounds of blocks over the 256 CUs.
-inline int pick_slot_steps(long long block_steps_total) {
-  long long s = (block_steps_total + 2047) / 2048;
-  if (s < 1) s = 1;
-  if (s > 16) s = 16;
-  return static_cast<int>(s);
+// Slots of a run one block serves: a shared expert read once for up to this many slots. Bounded by the
+// LDS a block may take without giving up residency (16 KB of staged activations) and by the
+// accumulators a lane holds.
+constexpr int kGateUpRun = 2;
+constexpr int kDownRun = 4;
+inline int run_cap_for(const SlotArgs& a, int max_run) {
+  if (a.order == nullptr) return 1;            // slots in layout order: no two neighbours share an expert
+  const int tuned = tune_get(kTuneSlotRun);
+  int cap = tuned > 0 ? tuned : max_run;
+  while (cap > 1 && (cap > max_run || stage_bytes(cap, a.k) > 16 * 1024)) --cap;
+  return cap;
 }
 
 template <int FMT>
@@ -517,52 +483,53 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
-  const int form = tune_get(kTuneSlotForm);   // 0 auto, 1 LDS, 2 registers + prefetch, 3 registers
-  const_cast<SlotArgs&>(a).debug_nomath = tune_get(3);
-  const bool reg = form >= 2 && slot_reg_form_ok<FMT>(g, a);
-  int steps = reg ? pick_slot_steps(per_slot * a.slots) : pick_steps(per_slot * a.slots);
+  int steps = pick_steps(per_slot * a.slots);
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
+  const int cap = run_cap_for(a, kGateUpRun);
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
-    if constexpr (NB * FmtTraits<FMT>::kPieces * 4 <= 64) {
-      if (reg && form == 2) {
-        hipLaunchKernelGGL((slot_gate_up_reg_kernel<FMT, NB, true>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
-        return;
-      }
-      if (reg) {
-        hipLaunchKernelGGL((slot_gate_up_reg_kernel<FMT, NB, false>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
-        return;
-      }
-    }
-    hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g, steps);
+    if (cap >= kGateUpRun)
+      hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, kGateUpRun>), grid, dim3(kBlockThreads),
+                         stage_bytes(kGateUpRun, a.k), stream, a, g, steps);
+    else
+      hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, 1>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a,
+                         g, steps);
   });
   return hipGetLastError();
 }
 
+// Row tiles (grid x) of a down launch: the arrival counters of the fused accumulation are indexed
+// [token, tile].
 template <int FMT>
-hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
-  const RowGeom g = geom_for<FMT>(a.k);
+inline void slot_down_grid(const SlotArgs& a, RowGeom& g, int& steps, unsigned& tiles) {
+  g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
-  const int form = tune_get(kTuneSlotForm);
-  const bool reg = form >= 2 && slot_reg_form_ok<FMT>(g, a);
-  int steps = reg ? pick_slot_steps(per_slot * a.slots) : pick_steps(per_slot * a.slots);
+  steps = pick_steps(per_slot * a.slots);
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
-  const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
+  tiles = static_cast<unsigned>((per_slot + steps - 1) / steps);
+}
+
+template <int FMT>
+hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
+  RowGeom g;
+  int steps;
+  unsigned tiles;
+  slot_down_grid<FMT>(a, g, steps, tiles);
+  const dim3 grid(tiles, static_cast<unsigned>(a.slots));
+  const int cap = run_cap_for(a, kDownRun);
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
-    if constexpr (NB * FmtTraits<FMT>::kPieces * 4 <= 64) {
-      if (reg && form == 2) {
-        hipLaunchKernelGGL((slot_down_reg_kernel<FMT, NB, true>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
-        return;
-      }
-      if (reg) {
-        hipLaunchKernelGGL((slot_down_reg_kernel<FMT, NB, false>), grid, dim3(kBlockThreads), 0, stream, a, g, steps);
-        return;
-      }
-    }
-    hipLaunchKernelGGL((slot_down_kernel<FMT, NB>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g, steps);
+    if (cap >= kDownRun)
+      hipLaunchKernelGGL((slot_down_kernel<FMT, NB, kDownRun>), grid, dim3(kBlockThreads), stage_bytes(kDownRun, a.k),
+                         stream, a, g, steps);
+    else if (cap >= 2)
+      hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 2>), grid, dim3(kBlockThreads), stage_bytes(2, a.k), stream, a, g,
+                         steps);
+    else
+      hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 1>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g,
+                         steps);
   });
   return hipGetLastError();
 }

@@ -76,6 +76,9 @@ class GlmMoeLayer {
   float* d_slot_down_ = nullptr;     // [slots, hidden]
   float* d_acc_ = nullptr;           // [tokens, hidden]
   int* d_tile_counter_ = nullptr;    // [2]
+  int* d_arrive_ = nullptr;          // [max_tokens, ceil(hidden / 4)] arrival counters of the fused down + accumulate
+  size_t arrive_len_ = 0;
+  bool fuse_accum_ = true;
   int32_t* d_rows_ = nullptr;        // grouped path
   int32_t* d_slot_row_ = nullptr;
   MoeSegment* d_segs_ = nullptr;

@@ -183,6 +183,22 @@ def launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_rou
         _p(tile_counter)))
 
 
+def launch_moe_slot_down_accum(act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots, top_k, weights,
+                               out_bf16, out_f32, arrive, arrive_len, stream=None):
+    """Extension: routed down rows + the ordered accumulation in one launch (FP8 experts)."""
+    _check(_lib.load().dgpp_launch_moe_slot_down_accum(
+        _p(act), act_stride, _p(ids), _p(order), _p(views), n, k, _p(slot_down), out_stride, slots, top_k,
+        _p(weights), _p(out_bf16), _p(out_f32), _p(arrive), arrive_len, _stream(stream)))
+
+
+def launch_moe_slot_down_accum_fp4(act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots, top_k,
+                                   weights, out_bf16, out_f32, arrive, arrive_len, stream=None, fp4_group=16):
+    """Extension: routed down rows + the ordered accumulation in one launch (NVFP4 / MXFP4 experts)."""
+    _check(_lib.load().dgpp_launch_moe_slot_down_accum_fp4(
+        _p(act), act_stride, _p(ids), _p(order), _p(views), n, k, _p(slot_down), out_stride, slots, top_k,
+        _p(weights), _p(out_bf16), _p(out_f32), _p(arrive), arrive_len, _stream(stream), fp4_group))
+
+
 # ---- grouped twins ---------------------------------------------------------------------------------------
 def launch_moe_grouped_gemv_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                  out_stride, n, k, stream=None):

@@ -38,10 +38,10 @@ const char* dgpp_target_arch(void);
 
 /* Bench A/B switches, process-wide, not thread-safe against concurrent launches (the reference
  * keeps such a switch in its launcher header too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90).
- * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: decode-slot kernel
- * form (0 / 1 LDS-staged activations, 2 register activations + next-step prefetch, 3 register
- * activations); key 2: row steps per block of the slot launches (0 = automatic). Outputs do not
- * depend on keys 1 and 2; key 0 changes the fp32 summation order (every launcher follows it alike). */
+ * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: slots of one expert a
+ * decode-slot block serves together (0 = default: 2 gate/up, 4 down; 1 = one slot per block);
+ * key 2: row steps per block of the slot launches (0 = automatic). Outputs do not depend on keys 1
+ * and 2; key 0 changes the fp32 summation order (every launcher follows it alike). */
 void dgpp_tune_set(int key, int value);
 int dgpp_tune_get(int key);
 
@@ -220,6 +220,24 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
                                   int* tile_counter);
 
 /* ---- grouped (segment-major) GEMV twins ------------------------------------------------------------ */
+/* Extension (no counterpart in the reference, which runs launch_moe_slot_down* and
+ * launch_moe_slot_accum* back to back): the routed slots' down rows AND the token's ordered
+ * accumulation chain in one launch. `slot_down` [slots, out_stride] f32 receives the unrounded down
+ * rows as launch_moe_slot_down* writes them; the block that finishes a token's last outstanding slot
+ * for a row tile then runs the chain of launch_moe_slot_accum_routed_* over that tile into out_f32
+ * (when given) or out_bf16, [tokens, n]. `arrive` holds at least tokens * ceil(n / 4) ints, zero before
+ * the first call and left zero by every call; calls sharing it must be ordered on one stream.
+ * Results are bit-identical to the two-launch form. No shared slot: chain it separately. */
+int dgpp_launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                    const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride,
+                                    int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
+                                    int* arrive, size_t arrive_len, void* stream);
+int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                        const int32_t* order, const DgppMoeExpertView* views, int n, int k,
+                                        float* slot_down, int out_stride, int slots, int top_k, const float* weights,
+                                        uint16_t* out_bf16, float* out_f32, int* arrive, size_t arrive_len,
+                                        void* stream, int fp4_group);
+
 /* src/kernels/glm_moe_launch.hpp:77-87 */
 int dgpp_launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride,
                                       const DgppMoeSegment* segs, int n_segs, int max_rows,

@@ -215,6 +215,23 @@ inline void launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, con
                                               k_shared, sh_payload, sh_scales, out, out_stride, slots, top_k, stream,
                                               shared_view_base, fp4_group, sh_rs, sh_cs, tile_counter));
 }
+// Extensions: down rows + ordered accumulation in one launch (see dgpp_amd.h).
+inline void launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                       const MoeExpertView* views, int n, int k, float* slot_down, int out_stride,
+                                       int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
+                                       int* arrive, size_t arrive_len, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_slot_down_accum(act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots,
+                                                top_k, weights, out_bf16, out_f32, arrive, arrive_len, stream));
+}
+inline void launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                           const int32_t* order, const MoeExpertView* views, int n, int k,
+                                           float* slot_down, int out_stride, int slots, int top_k, const float* weights,
+                                           uint16_t* out_bf16, float* out_f32, int* arrive, size_t arrive_len,
+                                           hipStream_t stream, int fp4_group = 16) {
+  detail::check(dgpp_launch_moe_slot_down_accum_fp4(act, act_stride, ids, order, views, n, k, slot_down, out_stride,
+                                                    slots, top_k, weights, out_bf16, out_f32, arrive, arrive_len,
+                                                    stream, fp4_group));
+}
 inline void launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
                                          int max_rows, int rows_per_block, const MoeExpertView* views, int which,
                                          uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream) {
