@@ -72,6 +72,7 @@ SIGNATURES = {
     "dgpp_moe_config_validate": (_I, [_P]),
     "dgpp_launch_moe_router": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_launch_moe_router_select": (_I, [_P, _P, _P, _P, _P, _I, _P]),
+    "dgpp_launch_moe_router_select_order": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P]),
     "dgpp_launch_moe_swiglu_clamp": (_I, [_P, _P, _P, _L, _F, _P]),
     "dgpp_launch_moe_gather_rows": (_I, [_P, _P, _P, _I, _I, _P]),
     "dgpp_launch_moe_accum": (_I, [_P, _P, _P, _P, _I, _I, _P]),

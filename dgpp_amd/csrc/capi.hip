@@ -324,6 +324,27 @@ int dgpp_launch_moe_router_select(const float* scores, const float* biased, int3
                 "moe_router_select");
 }
 
+int dgpp_launch_moe_router_select_order(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                        int32_t* order, const DgppMoeConfig* cfg, int tokens, int shared_early,
+                                        void* stream) {
+  const char* who = "moe_router_select_order";
+  const int rc = dgpp_moe_config_validate(cfg);
+  if (rc != DGPP_OK) return rc;
+  if (tokens <= 0) return DGPP_OK;
+  if (!scores || !biased || !ids || !weights) return fail_arg(std::string(who) + ": null pointer");
+  const int slots = tokens * (cfg->top_k + 1);
+  if (order != nullptr && slots > 1024) return fail_arg(std::string(who) + ": at most 1024 slots");
+  if (tokens <= 16 && cfg->n_experts <= 8 * 64)
+    return finish(run_router_select_order(cfg->router_mode, scores, biased, ids, weights, order, tokens, cfg->n_experts,
+                                          cfg->top_k, cfg->routed_scaling_factor, cfg->norm_topk_prob ? 1 : 0,
+                                          shared_early, as_stream(stream)),
+                  who);
+  const int rc2 = dgpp_launch_moe_router_select(scores, biased, ids, weights, cfg, tokens, stream);
+  if (rc2 != DGPP_OK || order == nullptr) return rc2;
+  return finish(run_slot_order(ids, order, nullptr, slots, cfg->top_k, cfg->n_experts, shared_early, as_stream(stream)),
+                who);
+}
+
 int dgpp_launch_moe_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, float limit,
                                  void* stream) {
   if (n <= 0) return DGPP_OK;

@@ -148,8 +148,11 @@ void GlmMoeLayer::enqueue_decode_scores(const uint16_t* x, size_t x_stride, cons
                                         uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
   if (tokens <= 0) return;
   check_tokens(tokens);
-  launch_moe_router_select(scores, biased, d_ids_, d_weights_, cfg_, tokens, stream);
-  expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream);
+  // Selection and slot order in one launch; the chain below then finds its order ready.
+  const bool with_order = tokens > 1 && tokens * (cfg_.top_k + 1) <= 1024;
+  launch_moe_router_select_order(scores, biased, d_ids_, d_weights_, with_order ? d_order_ : nullptr, cfg_, tokens, stream,
+                                 cfg_.shared_slots_early);
+  expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream, /*order_ready=*/true);
 }
 
 void GlmMoeLayer::enqueue_decode_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
@@ -161,20 +164,21 @@ void GlmMoeLayer::enqueue_decode_routed(const uint16_t* x, size_t x_stride, cons
 
 // Steps 4-7 of the reference's decode call order (src/models/glm/moe_layer.cpp:1555-1677).
 void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
-                                     uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
+                                     uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
+                                     bool order_ready) {
   const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter;
   const int slots = tokens * (K + 1);
   if (slots > 1024 && tokens > 1)
     throw std::invalid_argument("GlmMoeLayer: the decode-slot path takes at most 1024 slots; use the grouped path");
   const int32_t* order = nullptr;
   if (tokens > 1) {
-    launch_moe_slot_order(ids, d_order_, slots, K, cfg_.n_experts, stream, cfg_.shared_slots_early);
+    if (!order_ready) launch_moe_slot_order(ids, d_order_, slots, K, cfg_.n_experts, stream, cfg_.shared_slots_early);
     order = d_order_;
   }
   const bool sh_args = has_shared() && !w_.shared_in_table;
   const int n_sh = has_shared() ? w_.shared_inter : 0;
   const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
-  const bool fused = !has_shared() && fuse_accum_;   // down rows + accumulation in one launch
+  const bool fused = !has_shared() && dgpp_tune_get(4) == 1;   // down rows + accumulation in one launch
   if (w_.format == GlmExpertFormat::Fp8) {
     launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
                                    w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,

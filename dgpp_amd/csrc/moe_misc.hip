@@ -230,21 +230,20 @@ __device__ __forceinline__ uint32_t order_key(float v) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// One wavefront selects for one token. On return lane p < top_k holds the token's p-th expert in
+// ascending id order and its final weight; no private arrays, no LDS.
 template <int kMode, int PER_LANE>
-__global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
-    const float* __restrict__ scores, const float* __restrict__ biased, int32_t* __restrict__ ids,
-    float* __restrict__ weights, int tokens, int n_experts, int top_k, float scaling, int norm_topk) {
-  const int t = blockIdx.x, lane = threadIdx.x;
-  if (t >= tokens) return;
-  const size_t row = static_cast<size_t>(t) * n_experts;
+__device__ __forceinline__ void select_token(const float* __restrict__ scores, const float* __restrict__ biased,
+                                             int n_experts, int top_k, float scaling, int norm_topk, int lane,
+                                             int& out_id, float& out_w) {
   float sc[PER_LANE];
   uint32_t key[PER_LANE];
 #pragma unroll
   for (int j = 0; j < PER_LANE; ++j) {
     const int e = lane + j * kWaveSize;
     const bool live = e < n_experts;
-    sc[j] = live ? scores[row + e] : -INFINITY;
-    key[j] = live ? order_key(biased[row + e]) : 0u;
+    sc[j] = live ? scores[e] : -INFINITY;
+    key[j] = live ? order_key(biased[e]) : 0u;
   }
   if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
     float m = -INFINITY;
@@ -261,8 +260,9 @@ __global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) sc[j] = sc[j] / sum;
   }
-  int sel[16];
-  float wsel[16];
+  // Pick r lands in lane r.
+  int my_id = INT_MAX;
+  float my_w = 0.f;
   for (int r = 0; r < top_k; ++r) {
     uint32_t hi = 0u, lo = 0u;
 #pragma unroll
@@ -290,31 +290,85 @@ __global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
         if (lane == owner) key[j] = 0u;          // taken: below every real key
       }
     }
-    sel[r] = best;
-    wsel[r] = __shfl(mine, owner);
-  }
-  if (lane != 0) return;
-  for (int i = 1; i < top_k; ++i) {  // ascending expert id
-    const int id = sel[i];
-    const float w = wsel[i];
-    int j = i - 1;
-    while (j >= 0 && sel[j] > id) {
-      sel[j + 1] = sel[j];
-      wsel[j + 1] = wsel[j];
-      --j;
+    const float w = row_lane(mine, owner);
+    if (lane == r) {
+      my_id = best;
+      my_w = w;
     }
-    sel[j + 1] = id;
-    wsel[j + 1] = w;
   }
-  float denom = 0.f;
-  for (int i = 0; i < top_k; ++i) denom += wsel[i];
-  denom += 1e-20f;
+  // Ascending expert id, stable in pick order: rank of lane's pick, then the inverse permutation.
+  int rank = 0;
   for (int i = 0; i < top_k; ++i) {
-    float w = norm_topk ? (wsel[i] / denom) * scaling : wsel[i] * scaling;
-    if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) w = bf16_to_f32(f32_to_bf16(w));
-    ids[static_cast<size_t>(t) * top_k + i] = sel[i];
-    weights[static_cast<size_t>(t) * top_k + i] = w;
+    const int oid = __builtin_amdgcn_readlane(my_id, i);
+    rank += (oid < my_id) || (oid == my_id && i < lane);
   }
+  int src = 0;
+  for (int i = 0; i < top_k; ++i)
+    if (__builtin_amdgcn_readlane(rank, i) == lane) src = i;
+  const int sid = __shfl(my_id, src);
+  const float sw = __shfl(my_w, src);
+  float denom = 0.f;
+  for (int i = 0; i < top_k; ++i) denom += row_lane(sw, i);   // fp32 adds in id order
+  denom += 1e-20f;
+  float w = norm_topk ? (sw / denom) * scaling : sw * scaling;
+  if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) w = bf16_to_f32(f32_to_bf16(w));
+  out_id = sid;
+  out_w = w;
+}
+
+template <int kMode, int PER_LANE>
+__global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
+    const float* __restrict__ scores, const float* __restrict__ biased, int32_t* __restrict__ ids,
+    float* __restrict__ weights, int tokens, int n_experts, int top_k, float scaling, int norm_topk) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  if (t >= tokens) return;
+  const size_t row = static_cast<size_t>(t) * n_experts;
+  int id;
+  float w;
+  select_token<kMode, PER_LANE>(scores + row, biased + row, n_experts, top_k, scaling, norm_topk, lane, id, w);
+  if (lane < top_k) {
+    ids[static_cast<size_t>(t) * top_k + lane] = id;
+    weights[static_cast<size_t>(t) * top_k + lane] = w;
+  }
+}
+
+// Selection and slot order in ONE launch for a decode batch: one wavefront per token selects, the
+// block then ranks the slots by (expert, slot) exactly as slot_order_kernel does (key = expert id,
+// or n_experts for the token's shared slot). tokens * 64 threads, tokens <= 16.
+template <int kMode, int PER_LANE>
+__global__ __launch_bounds__(1024) void router_select_order_kernel(
+    const float* __restrict__ scores, const float* __restrict__ biased, int32_t* __restrict__ ids,
+    float* __restrict__ weights, int32_t* __restrict__ order, int tokens, int n_experts, int top_k, float scaling,
+    int norm_topk, int shared_early) {
+  __shared__ int32_t keys[16 * 17];
+  const int t = threadIdx.x >> 6, lane = threadIdx.x & (kWaveSize - 1);
+  const size_t row = static_cast<size_t>(t) * n_experts;
+  int id;
+  float w;
+  select_token<kMode, PER_LANE>(scores + row, biased + row, n_experts, top_k, scaling, norm_topk, lane, id, w);
+  if (lane < top_k) {
+    ids[static_cast<size_t>(t) * top_k + lane] = id;
+    weights[static_cast<size_t>(t) * top_k + lane] = w;
+    keys[t * (top_k + 1) + lane] = id;
+  } else if (lane == top_k) {
+    keys[t * (top_k + 1) + lane] = n_experts;
+  }
+  if (order == nullptr) return;
+  __syncthreads();
+  const int slots = tokens * (top_k + 1);
+  const int s = threadIdx.x;
+  if (s >= slots) return;
+  const int mine = keys[s];
+  int pos = 0;
+  for (int o = 0; o < slots; ++o) {
+    const int k = keys[o];
+    pos += (k < mine) || (k == mine && o < s);
+  }
+  if (shared_early) {
+    const int routed = tokens * top_k;
+    pos = pos < routed ? pos + (pos < tokens ? pos : tokens) : 2 * (pos - routed) + 1;
+  }
+  order[pos] = s;
 }
 
 // ---- elementwise ------------------------------------------------------------------------------
@@ -617,6 +671,29 @@ hipError_t run_router_select(int mode, const float* scores, const float* biased,
     else
       hipLaunchKernelGGL(router_select_kernel<DGPP_ROUTER_SIGMOID_BIAS>, grid, block, lds, stream, scores, biased, ids,
                          weights, tokens, n_experts, top_k, scaling, norm_topk);
+  }
+  return hipGetLastError();
+}
+
+hipError_t run_router_select_order(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
+                                   int32_t* order, int tokens, int n_experts, int top_k, float scaling, int norm_topk,
+                                   int shared_early, hipStream_t stream) {
+  const bool softmax = mode == DGPP_ROUTER_SOFTMAX_TOPK;
+  const dim3 grid(1), block(tokens * kWaveSize);
+  if (n_experts <= 4 * kWaveSize) {
+    if (softmax)
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 4>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
+    else
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SIGMOID_BIAS, 4>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
+  } else {
+    if (softmax)
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 8>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
+    else
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SIGMOID_BIAS, 8>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
   }
   return hipGetLastError();
 }

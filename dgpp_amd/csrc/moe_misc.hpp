@@ -13,6 +13,10 @@ hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gat
                            float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream);
 hipError_t run_router_select(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
                              int tokens, int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream);
+// tokens <= 16, n_experts <= 512, top_k <= 16; order may be null (selection only).
+hipError_t run_router_select_order(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
+                                   int32_t* order, int tokens, int n_experts, int top_k, float scaling, int norm_topk,
+                                   int shared_early, hipStream_t stream);
 hipError_t run_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, float limit,
                             hipStream_t stream);
 hipError_t run_gather_rows(const uint16_t* src, const int32_t* rows, uint16_t* dst, int n_rows, int hidden,

@@ -73,6 +73,14 @@ def launch_moe_router_select(scores, biased, ids, weights, cfg: MoeConfig, token
                                                      tokens, _stream(stream)))
 
 
+def launch_moe_router_select_order(scores, biased, ids, weights, order, cfg: MoeConfig, tokens, shared_early=False,
+                                   stream=None):
+    """Extension: selection + slot order in one launch (order may be None)."""
+    _check(_lib.load().dgpp_launch_moe_router_select_order(_p(scores), _p(biased), _p(ids), _p(weights), _p(order),
+                                                           C.addressof(cfg), tokens, 1 if shared_early else 0,
+                                                           _stream(stream)))
+
+
 # ---- elementwise --------------------------------------------------------------------------------
 def launch_moe_swiglu_clamp(gate, up, out, n, limit, stream=None):
     _check(_lib.load().dgpp_launch_moe_swiglu_clamp(_p(gate), _p(up), _p(out), n, limit, _stream(stream)))

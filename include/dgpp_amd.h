@@ -130,6 +130,13 @@ int dgpp_launch_moe_router_select(const float* scores, const float* biased, int3
                                   void* stream);
 
 /* ---- elementwise pieces -------------------------------------------------------------------- */
+/* Extension: the selection of dgpp_launch_moe_router_select and, when `order` is given, the slot
+ * order of dgpp_launch_moe_slot_order (same outputs, bit for bit) in one launch for decode batches
+ * (tokens <= 16 and n_experts <= 512; larger problems run the two kernels). */
+int dgpp_launch_moe_router_select_order(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                        int32_t* order, const DgppMoeConfig* cfg, int tokens, int shared_early,
+                                        void* stream);
+
 /* src/kernels/glm_moe_launch.hpp:43 */
 int dgpp_launch_moe_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out,
                                  int64_t n, float limit, void* stream);

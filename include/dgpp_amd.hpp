@@ -118,6 +118,14 @@ inline void launch_moe_router_select(const float* scores, const float* biased, i
   const DgppMoeConfig c = cfg.c_config();
   detail::check(dgpp_launch_moe_router_select(scores, biased, ids, weights, &c, tokens, stream));
 }
+// Extension: selection + slot order in one launch (see dgpp_amd.h).
+inline void launch_moe_router_select_order(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                           int32_t* order, const GlmMoeConfig& cfg, int tokens, hipStream_t stream,
+                                           bool shared_early = false) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_router_select_order(scores, biased, ids, weights, order, &c, tokens,
+                                                    shared_early ? 1 : 0, stream));
+}
 inline void launch_moe_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, float limit,
                                     hipStream_t stream) {
   detail::check(dgpp_launch_moe_swiglu_clamp(gate, up, out, n, limit, stream));

@@ -233,3 +233,33 @@ def test_slot_accum_and_ordered_accum_bit_exact(gpu, T, H, K):
         L.launch_moe_accum_ordered_f32(outf, dev(down), H + 8, dev(slot_row), dev(ids), dev(sw), shared_row0, T, K, H, None)
         sync()
         assert np.array_equal(host(out, np.uint16), bf_want) and np.array_equal(host(outf), f32_want)
+
+
+@pytest.mark.parametrize("mode,E,K,T,early", [(1, 256, 8, 8, False), (1, 256, 8, 1, False), (0, 288, 8, 5, True),
+                                              (0, 40, 4, 16, False), (1, 512, 16, 3, False), (1, 600, 8, 4, False),
+                                              (0, 64, 8, 40, False)])
+def test_router_select_order_is_bitwise_select_then_slot_order(gpu, mode, E, K, T, early):
+    """The one-launch extension (selection + slot order) against the two launchers it stands for,
+    including the shapes it hands back to them (more than 16 tokens, more than 512 experts)."""
+    rng = np.random.default_rng(7 * E + T)
+    scores = rng.uniform(0.05, 0.95, (T, E)).astype(np.float32) if mode == 0 else \
+        hg.bf16_to_f32(hg.normal_bf16(E + T, (T, E)))
+    biased = (scores + rng.normal(0, 0.05, (T, E))).astype(np.float32) if mode == 0 else scores
+    scores[0, : E // 2] = scores[0, 0]          # a row with many exact ties: lower id wins
+    if mode == 0:
+        biased[0] = scores[0]
+    cfg = L.make_config(64, 64, E, K, router_mode=mode, routed_scaling_factor=1.0 if mode else 2.5, n_shared_experts=0)
+    slots = T * (K + 1)
+    s_d, b_d = dev(scores), dev(biased)
+    ids1, w1, o1 = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32), dev_empty(slots, np.int32)
+    L.launch_moe_router_select(s_d, b_d, ids1, w1, cfg, T, None)
+    L.launch_moe_slot_order(ids1, o1, slots, K, E, None, early)
+    ids2, w2, o2 = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32), dev_empty(slots, np.int32)
+    L.launch_moe_router_select_order(s_d, b_d, ids2, w2, o2, cfg, T, early, None)
+    ids3, w3 = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32)
+    L.launch_moe_router_select_order(s_d, b_d, ids3, w3, None, cfg, T, early, None)
+    sync()
+    assert np.array_equal(host(ids1), host(ids2)) and np.array_equal(host(ids1), host(ids3))
+    assert np.array_equal(host(w1), host(w2)) and np.array_equal(host(w1), host(w3))
+    assert np.array_equal(host(o1), host(o2))
+    assert np.array_equal(np.sort(host(o2)), np.arange(slots))
