@@ -187,9 +187,9 @@ __global__ __launch_bounds__(kWaveSize) void router_select_kernel(
 
 // The same selection for up to 64 * PER_LANE experts with the whole row in registers (expert e
 // lives in lane e % 64, slot e / 64): no LDS, no barriers, DPP reductions inside 16-lane rows and
-// four lane reads across them. Ordering keys are (value, ~id) pairs compared lexicographically, so
-// the maximum is the largest value and, among equal values, the LOWEST id — the strict '>' scan's
-// outcome. -0 is folded into +0 first (they compare equal as floats); a NaN key never wins.
+// four lane reads across them. A value's ordering key is a monotone unsigned image of the float
+// (-0 folded into +0 first: they compare equal as floats; NaN maps to 0 and never wins); among
+// equal keys the LOWEST id is taken — the strict '>' scan's outcome.
 template <int kCtrl>
 __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
   return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), kCtrl, 0xF, 0xF, true));
@@ -215,14 +215,9 @@ __device__ __forceinline__ float wave_max_dpp(float v) {
   v = fmaxf(v, dpp_f32<0x140>(v));
   return fmaxf(fmaxf(row_lane(v, 0), row_lane(v, 16)), fmaxf(row_lane(v, 32), row_lane(v, 48)));
 }
-__device__ __forceinline__ void key_max(uint32_t& hi, uint32_t& lo, uint32_t ohi, uint32_t olo) {
-  const bool take = ohi > hi || (ohi == hi && olo > lo);
-  hi = take ? ohi : hi;
-  lo = take ? olo : lo;
-}
-template <int kCtrl>
-__device__ __forceinline__ void key_max_dpp(uint32_t& hi, uint32_t& lo) {
-  key_max(hi, lo, dpp_u32<kCtrl>(hi), dpp_u32<kCtrl>(lo));
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+__device__ __forceinline__ uint32_t lane_u32(uint32_t v, int lane) {
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane));
 }
 __device__ __forceinline__ uint32_t order_key(float v) {
   if (v != v) return 0u;                       // NaN: below every real key
@@ -260,27 +255,31 @@ __device__ __forceinline__ void select_token(const float* __restrict__ scores, c
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) sc[j] = sc[j] / sum;
   }
-  // Pick r lands in lane r.
+  // Pick r lands in lane r. A round takes the wave-wide maximum key (one DPP max per step), then the
+  // LOWEST expert id among the lanes and slots that hold it: slot-major ids (e = lane + 64 * slot),
+  // so the first slot with a match wins and, inside it, the lowest matching lane.
   int my_id = INT_MAX;
   float my_w = 0.f;
   for (int r = 0; r < top_k; ++r) {
-    uint32_t hi = 0u, lo = 0u;
+    uint32_t m = key[0];
 #pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) key_max(hi, lo, key[j], ~static_cast<uint32_t>(lane + j * kWaveSize));
-    key_max_dpp<0xB1>(hi, lo);
-    key_max_dpp<0x4E>(hi, lo);
-    key_max_dpp<0x141>(hi, lo);
-    key_max_dpp<0x140>(hi, lo);
-    uint32_t bh = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 0));
-    uint32_t bl = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 0));
-    key_max(bh, bl, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 16)),
-            static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 16)));
-    key_max(bh, bl, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 32)),
-            static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 32)));
-    key_max(bh, bl, static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(hi), 48)),
-            static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(lo), 48)));
-    int best = static_cast<int>(~bl);
-    if (bh == 0u || best < 0 || best >= n_experts) best = 0;   // a row of NaN keys: stay in bounds
+    for (int j = 1; j < PER_LANE; ++j) m = m > key[j] ? m : key[j];
+    m = umax(m, dpp_u32<0xB1>(m));
+    m = umax(m, dpp_u32<0x4E>(m));
+    m = umax(m, dpp_u32<0x141>(m));
+    m = umax(m, dpp_u32<0x140>(m));
+    const uint32_t top = umax(umax(lane_u32(m, 0), lane_u32(m, 16)), umax(lane_u32(m, 32), lane_u32(m, 48)));
+    int best = 0;
+    bool found = false;
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+      const uint64_t hit = __builtin_amdgcn_ballot_w64(key[j] == top);
+      if (!found && hit != 0) {
+        best = j * kWaveSize + __builtin_ctzll(hit);
+        found = true;
+      }
+    }
+    if (top == 0u || best >= n_experts) best = 0;   // a row of NaN keys: stay in bounds
     const int owner = best & (kWaveSize - 1), slot = best >> 6;
     float mine = 0.f;
 #pragma unroll
