@@ -52,6 +52,8 @@ def parse():
     ap.add_argument("--eager", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
+    ap.add_argument("--configs", default="c1,c2", help="other BASELINE configurations to time beside the headline, "
+                    "comma separated out of c1,c2,c4,c5 ('' for none; c4 and c5 take a minute of set-up each)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -237,6 +239,169 @@ def main():
             if t != T:
                 others[f"T{t}"] = measure(t, args.steps, args.warmup)
 
+    # ---- the other BASELINE configurations (reported beside the headline, never part of `value`) ------------
+    def ring_copies(tensors, nbytes, want=2 * 256 * 2**20 + 64 * 2**20):
+        """Device copies of a weight set so that consecutive timed launches never find it in the caches."""
+        n = max(2, -(-want // nbytes))
+        return [[t.clone() for t in tensors] if i else list(tensors) for i in range(n)]
+
+    def bench_c1():
+        n = k = 4096
+        payload, scales = hg.encode_fp8_blocks(hg.f32_to_bf16(hg.normal_f32(0xD6990010, (n, k), 0.02)), 128, 128)
+        ring = ring_copies([torch.from_numpy(payload).to(dev), torch.from_numpy(scales).to(dev)], payload.nbytes)
+        act = torch.from_numpy(hg.normal_bf16(0xD6990011, (1, k)).view(np.int16)).to(dev)
+        out = torch.empty((len(ring), n), dtype=torch.int16, device=dev)
+        def step(i):
+            r = i % len(ring)
+            L.launch_scale_gemm_bf16(act, k, ring[r][0], ring[r][1], out[r], 1, n, k, stream)
+        sec = time_graph(step, args.steps, args.warmup)
+        nbytes = n * k + (n // 128) * (k // 128) * 4 + k * 2 + n * 2
+        return {"workload": "C1 dense FP8 block-128 GEMV 4096x4096, batch 1", "us": sec * 1e6, "algorithmic_bytes": nbytes,
+                "gbps": nbytes / sec / 1e9, "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+
+    def bench_c2():
+        n, k = 17408, 5120
+        payload, scales, ws2 = hg.encode_nvfp4(hg.normal_f32(0xD6990020, (n, k), 0.02))
+        glob = torch.tensor([1.0 / np.float32(ws2)], dtype=torch.float32, device=dev)
+        ring = ring_copies([torch.from_numpy(payload).to(dev), torch.from_numpy(scales).to(dev)],
+                           payload.nbytes + scales.nbytes)
+        mats = [L.Fp4Matrix(r[0].data_ptr(), r[1].data_ptr(), glob.data_ptr(), n, k, 16, 0, None) for r in ring]
+        res = {}
+        for m in (1, 8):
+            act = torch.from_numpy(hg.normal_bf16(0xD6990021, (m, k)).view(np.int16)).to(dev)
+            out = torch.empty((len(ring), m, n), dtype=torch.int16, device=dev)
+            def step(i):
+                r = i % len(ring)
+                L.launch_fp4_gemv_bf16(act, k, mats[r], out[r], m, n, k, stream)
+            sec = time_graph(step, args.steps, args.warmup)
+            nbytes = n * k // 2 + n * k // 16 + 4 + m * (k * 2 + n * 2)
+            res[f"batch{m}"] = {"us": sec * 1e6, "algorithmic_bytes": nbytes, "gbps": nbytes / sec / 1e9,
+                                "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+        res["workload"] = "C2 dense NVFP4 GEMV 17408x5120 (gate_up shape), batch 1 and 8 (one weight pass)"
+        return res
+
+    def expert_table(per_expert_views, n_exp):
+        return [v for e in range(n_exp) for v in per_expert_views[e]]
+
+    def bench_c4():
+        cE, cH, cI, cK, cT = 128, 2048, 768, 8, 32
+        gen = []
+        for e in range(cE):   # every expert its own weights: 604 MB per layer, far beyond the caches
+            mats = []
+            for mi, (r, c) in enumerate(((cI, cH), (cI, cH), (cH, cI))):
+                pw, sw = hg.encode_fp8_blocks(hg.f32_to_bf16(hg.normal_f32(0xD6994000 + e * 3 + mi, (r, c), 0.02)), 128, 128)
+                mats.append((torch.from_numpy(pw).to(dev), torch.from_numpy(sw).to(dev)))
+            gen.append(mats)
+        ring = [gen, [[(a.clone(), b.clone()) for a, b in mats] for mats in gen]]
+        cfg4 = L.make_config(cH, cI, cE, cK, n_shared_experts=0, routed_scaling_factor=1.0, swiglu_limit=float("inf"),
+                             router_mode=L.ROUTER_SOFTMAX_TOPK)
+        lay = []
+        for g in ring:
+            views = []
+            for e in range(cE):
+                for pw, sw in g[e]:
+                    v = L.MoeExpertView()
+                    v.payload, v.scales = pw.data_ptr(), sw.data_ptr()
+                    v.scale_shift_rows = v.scale_shift_cols = 7
+                    v.fp4_group = 16
+                    views.append(v)
+            lay.append(ML.MoeLayer(cfg4, ML.EXPERTS_FP8, views, cT))
+        ids = hg.zipf_routes(0xD6990040 + cT, 1.1, cT, cK, cE)
+        lg = hg.bf16_to_f32(hg.normal_bf16(0xD6990041, (cT, cK))).astype(np.float64)
+        wts = np.exp(lg - lg.max(1, keepdims=True))
+        wts = (wts / wts.sum(1, keepdims=True)).astype(np.float32)
+        x = torch.from_numpy(hg.normal_bf16(0xD6990042, (cT, cH)).view(np.int16)).to(dev)
+        ids_d, w_d = torch.from_numpy(ids).to(dev), torch.from_numpy(wts).to(dev)
+        out = torch.empty((2, cT, cH), dtype=torch.int16, device=dev)
+        uniq = len(np.unique(ids))
+        nbytes = uniq * (3 * cI * cH + 3 * (cI // 128) * (cH // 128) * 4) + cT * cH * 4
+        res = {"workload": f"C4 FP8 block-128 MoE layer, 128 experts, hidden 2048, inter 768, top-8, T=32 Zipf(1.1) "
+                           f"routing ({uniq} distinct experts, busiest {int(np.bincount(ids.ravel()).max())} tokens)",
+               "algorithmic_bytes": nbytes}
+        for name, fn in (("decode_slots", lambda i: lay[i % 2].enqueue_decode_routed(x, cH, ids_d, w_d, out[i % 2], cT, stream)),
+                         ("grouped", lambda i: lay[i % 2].enqueue_grouped_routed(x, cH, ids_d, w_d, out[i % 2], cT, stream))):
+            sec = time_graph(fn, max(args.steps // 4, 10), args.warmup)
+            res[name] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9, "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+        for l_ in lay:
+            l_.close()
+        return res
+
+    def bench_c5():
+        cE, cH, cI, cK, cT, cSI, G = 256, 6144, 2048, 8, 64, 4096, 8
+        keep5, gen = [], []
+        for g in range(G):    # G generated experts; the 256 table entries are device COPIES of them (own addresses)
+            mats = []
+            for mi, (r, c) in enumerate(((cI, cH), (cI, cH), (cH, cI))):
+                pw, sw, ws2 = hg.encode_nvfp4(hg.normal_f32(0xD6995000 + g * 3 + mi, (r, c), 0.02))
+                mats.append((torch.from_numpy(pw).to(dev), torch.from_numpy(sw).to(dev),
+                             torch.tensor([1.0 / np.float32(ws2)], dtype=torch.float32, device=dev)))
+            gen.append(mats)
+        views = []
+        for e in range(cE):
+            for pw, sw, gl in gen[e % G]:
+                pc, sc_ = (pw, sw) if e < G else (pw.clone(), sw.clone())
+                keep5 += [pc, sc_]
+                v = L.MoeExpertView()
+                v.payload, v.fp4_scales, v.fp4_global = pc.data_ptr(), sc_.data_ptr(), gl.data_ptr()
+                v.scale_shift_rows = v.scale_shift_cols = 7
+                v.fp4_group = 16
+                views.append(v)
+        cfg5 = L.make_config(cH, cI, cE, cK, n_shared_experts=0, routed_scaling_factor=1.0, swiglu_limit=float("inf"),
+                             router_mode=L.ROUTER_SOFTMAX_TOPK)
+        lay = ML.MoeLayer(cfg5, ML.EXPERTS_NVFP4, views, cT)
+        x = torch.from_numpy(hg.normal_bf16(0xD6990050, (cT, cH)).view(np.int16)).to(dev)
+        lg_h = hg.bf16_to_f32(hg.normal_bf16(0xD6990051, (cT, cE)))
+        lg5 = torch.from_numpy(lg_h).to(dev)
+        uniq = len(np.unique(np.argsort(-lg_h.astype(np.float64), axis=1, kind="stable")[:, :cK]))
+        sh = []
+        for mi, (r, c) in enumerate(((cSI, cH), (cSI, cH), (cH, cSI))):
+            pw, sw = hg.encode_mxfp8(hg.normal_f32(0xD6995900 + mi, (r, c), 0.02))
+            sh.append((torch.from_numpy(pw).to(dev), torch.from_numpy(sw).to(dev)))
+        routed = torch.empty((cT, cH), dtype=torch.float32, device=dev)
+        g_d, u_d, a_d = (torch.empty((cT, cSI), dtype=torch.int16, device=dev) for _ in range(3))
+        shared_down = torch.empty((cT, cH), dtype=torch.float32, device=dev)
+        rows_id = torch.arange(cT, dtype=torch.int32, device=dev)
+        ones = torch.ones(cT, dtype=torch.float32, device=dev)
+        out = torch.empty((cT, cH), dtype=torch.int16, device=dev)
+
+        def routed_part(i):
+            lay.enqueue_decode_scores(x, cH, lg5, lg5, None, cT, stream, out_f32=routed)
+
+        def shared_part(i):
+            L.launch_scale_gemm_grid_e8m0_bf16(x, cH, sh[0][0], sh[0][1], g_d, cT, cSI, cH, stream, 0, 0, 5)
+            L.launch_scale_gemm_grid_e8m0_bf16(x, cH, sh[1][0], sh[1][1], u_d, cT, cSI, cH, stream, 0, 0, 5)
+            L.launch_moe_swiglu_clamp(g_d, u_d, a_d, cT * cSI, float("inf"), stream)
+            L.launch_scale_gemm_grid_e8m0_f32(a_d, cSI, sh[2][0], sh[2][1], shared_down, cT, cH, cSI, stream, 0, 0, 5)
+            L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
+            L.launch_moe_round_bf16(out, routed, cT * cH, stream)
+
+        def full(i):
+            routed_part(i)
+            shared_part(i)
+
+        n_steps = max(args.steps // 10, 5)
+        per_expert = 3 * cI * cH // 2 + 3 * cI * cH // 16 + 12
+        shared_bytes = 3 * cSI * cH + 3 * cSI * cH // 32
+        nbytes = uniq * per_expert + shared_bytes + cT * cH * 4
+        res = {"workload": f"C5 NVFP4 routed MoE (256 experts, hidden 6144, inter 2048, top-8, {uniq} distinct) + MXFP8 "
+                           f"shared expert (inter 4096), T=64; routed expert weights = device copies of {G} generated experts",
+               "algorithmic_bytes": nbytes}
+        for name, fn, nb in (("layer", full, nbytes), ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
+                             ("shared_only", shared_part, shared_bytes + cT * cH * 4)):
+            sec = time_graph(fn, n_steps, 2)
+            res[name] = {"us": sec * 1e6, "algorithmic_bytes": nb, "gbps": nb / sec / 1e9,
+                         "frac_of_peak": nb / sec / 1e9 / HBM_PEAK_GBPS}
+        lay.close()
+        return res
+
+    other_configs = {}
+    if not args.only and not args.tune:
+        for name in filter(None, args.configs.split(",")):
+            t0 = time.time()
+            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5}[name]()
+            other_configs[name]["setup_and_run_seconds"] = time.time() - t0
+            torch.cuda.empty_cache()
+
     # ---- CPU baseline: the oracle's layer forward (dequantise to double, fp64 dots) on a bounded sample ----
     cpu = None
     if not args.no_cpu and not args.only:
@@ -293,6 +458,8 @@ def main():
         "ms_per_step": sec * 1e3,
         "us_per_layer": main_res.get("us_per_layer"),
         "frac_of_hbm_peak": main_res.get("frac_of_peak"),
+        # the reference's own bench counts rows * top_k * per-expert bytes ("no expert sharing", benchmarks/micro/moe_slot_bench.cu:238-264)
+        "reference_style_slot_gbps": (T * K * EXPERT_BYTES / sec / 1e9) if sec == sec else None,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -309,6 +476,7 @@ def main():
         "roofline": None,
         "cpu_baseline": cpu,
         "other_batches": others,
+        "other_configs": other_configs,
         "build_seconds": build_s,
     }
     if "gate_up_us" in main_res:
