@@ -277,6 +277,12 @@ def main():
             nbytes = n * k // 2 + n * k // 16 + 4 + m * (k * 2 + n * 2)
             res[f"batch{m}"] = {"us": sec * 1e6, "algorithmic_bytes": nbytes, "gbps": nbytes / sec / 1e9,
                                 "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+            def step_mma(i):
+                r = i % len(ring)
+                L.launch_dense_mma_fp4_bf16(act, k, mats[r], out[r], m, n, k, stream)
+            sec = time_graph(step_mma, args.steps, args.warmup)
+            res[f"batch{m}_matrix_core"] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9,
+                                            "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
         res["workload"] = "C2 dense NVFP4 GEMV 17408x5120 (gate_up shape), batch 1 and 8 (one weight pass)"
         return res
 
@@ -319,7 +325,9 @@ def main():
                            f"routing ({uniq} distinct experts, busiest {int(np.bincount(ids.ravel()).max())} tokens)",
                "algorithmic_bytes": nbytes}
         for name, fn in (("decode_slots", lambda i: lay[i % 2].enqueue_decode_routed(x, cH, ids_d, w_d, out[i % 2], cT, stream)),
-                         ("grouped", lambda i: lay[i % 2].enqueue_grouped_routed(x, cH, ids_d, w_d, out[i % 2], cT, stream))):
+                         ("grouped", lambda i: lay[i % 2].enqueue_grouped_routed(x, cH, ids_d, w_d, out[i % 2], cT, stream)),
+                         ("grouped_matrix_core",
+                          lambda i: lay[i % 2].enqueue_prefill_routed(x, cH, ids_d, w_d, out[i % 2], cT, stream))):
             sec = time_graph(fn, max(args.steps // 4, 10), args.warmup)
             res[name] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9, "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
         for l_ in lay:
@@ -375,19 +383,36 @@ def main():
             L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
             L.launch_moe_round_bf16(out, routed, cT * cH, stream)
 
+        ids5 = torch.empty((cT, cK), dtype=torch.int32, device=dev)
+        w5 = torch.empty((cT, cK), dtype=torch.float32, device=dev)
+        L.launch_moe_router_select(lg5, lg5, ids5, w5, cfg5, cT, stream)
+
+        def routed_mc(i):
+            lay.enqueue_prefill_routed(x, cH, ids5, w5, None, cT, stream, out_f32=routed)
+
+        def shared_mc(i):
+            L.launch_mma_gemv_fp8e8m0_bf16(x, cH, sh[0][0], sh[0][1], g_d, cT, cSI, cH, 0, 0, 5, stream)
+            L.launch_mma_gemv_fp8e8m0_bf16(x, cH, sh[1][0], sh[1][1], u_d, cT, cSI, cH, 0, 0, 5, stream)
+            L.launch_moe_swiglu_clamp(g_d, u_d, a_d, cT * cSI, float("inf"), stream)
+            L.launch_mma_gemv_fp8e8m0_f32(a_d, cSI, sh[2][0], sh[2][1], shared_down, cT, cH, cSI, 0, 0, 5, stream)
+            L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
+            L.launch_moe_round_bf16(out, routed, cT * cH, stream)
+
         def full(i):
             routed_part(i)
-            shared_part(i)
+            shared_mc(i)
 
         n_steps = max(args.steps // 10, 5)
         per_expert = 3 * cI * cH // 2 + 3 * cI * cH // 16 + 12
         shared_bytes = 3 * cSI * cH + 3 * cSI * cH // 32
         nbytes = uniq * per_expert + shared_bytes + cT * cH * 4
-        res = {"workload": f"C5 NVFP4 routed MoE (256 experts, hidden 6144, inter 2048, top-8, {uniq} distinct) + MXFP8 "
-                           f"shared expert (inter 4096), T=64; routed expert weights = device copies of {G} generated experts",
+        res = {"workload": f"C5 NVFP4 routed MoE (256 experts, hidden 6144, inter 2048, top-8, {uniq} distinct; decode slots) "
+                           f"+ MXFP8 shared expert (inter 4096; matrix-core launchers), T=64; routed expert weights = device copies of {G} generated experts",
                "algorithmic_bytes": nbytes}
         for name, fn, nb in (("layer", full, nbytes), ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
-                             ("shared_only", shared_part, shared_bytes + cT * cH * 4)):
+                             ("routed_only_matrix_core", routed_mc, uniq * per_expert + cT * cH * 6),
+                             ("shared_only_gemv_launchers", shared_part, shared_bytes + cT * cH * 4),
+                             ("shared_only", shared_mc, shared_bytes + cT * cH * 4)):
             sec = time_graph(fn, n_steps, 2)
             res[name] = {"us": sec * 1e6, "algorithmic_bytes": nb, "gbps": nb / sec / 1e9,
                          "frac_of_peak": nb / sec / 1e9 / HBM_PEAK_GBPS}

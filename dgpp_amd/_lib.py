@@ -92,8 +92,18 @@ SIGNATURES = {
     "dgpp_launch_moe_slot_down": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_launch_moe_slot_gate_up_swiglu_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I, _I, _I]),
     "dgpp_launch_moe_slot_down_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _P]),
-    "dgpp_launch_moe_slot_down_accum": (_I, [_P, _Z, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P]),
-    "dgpp_launch_moe_slot_down_accum_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _P, _I, _I, _I, _P, _P, _P, _P, _Z, _P, _I]),
+    "dgpp_launch_dense_mma_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _Z]),
+    "dgpp_launch_dense_mma_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _Z]),
+    "dgpp_launch_dense_mma_fp4_bf16": (_I, [_P, _Z, _P, _P, _I, _I, _I, _P]),
+    "dgpp_launch_dense_mma_fp4_f32": (_I, [_P, _Z, _P, _P, _I, _I, _I, _P]),
+    "dgpp_launch_mma_gemv_fp8_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
+    "dgpp_launch_mma_gemv_fp8_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
+    "dgpp_launch_mma_gemv_fp8e8m0_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
+    "dgpp_launch_mma_gemv_fp8e8m0_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
+    "dgpp_launch_moe_grouped_mma_bf16": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _P]),
+    "dgpp_launch_moe_grouped_mma_f32": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _P]),
+    "dgpp_launch_moe_grouped_mma_fp4_bf16": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _P, _I, _I]),
+    "dgpp_launch_moe_grouped_mma_fp4_f32": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _P, _I, _I]),
     "dgpp_launch_moe_grouped_gemv_bf16": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
     "dgpp_launch_moe_grouped_gemv_f32": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
     "dgpp_launch_moe_grouped_gemv_fp4_bf16": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _I]),
@@ -150,6 +160,7 @@ LAYER_SIGNATURES = {
     "dgpp_moe_layer_enqueue_decode_scores": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_decode_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_grouped_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
+    "dgpp_moe_layer_enqueue_prefill_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_views": (_P, [_P]),
     "dgpp_moe_layer_ids": (_P, [_P]),
     "dgpp_moe_layer_weights": (_P, [_P]),

@@ -103,6 +103,21 @@ hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, 
     default: return launch_grouped_fmt<kFmtMxfp4>(a, n_segs, z_ext, s);
   }
 }
+hipError_t launch_dense_mma(int fmt, const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_dense_mma_fmt<kFmtFp8F32>(a, ws, ws_bytes, s);
+    case kFmtFp8E8M0: return launch_dense_mma_fmt<kFmtFp8E8M0>(a, ws, ws_bytes, s);
+    case kFmtNvfp4: return launch_dense_mma_fmt<kFmtNvfp4>(a, ws, ws_bytes, s);
+    default: return launch_dense_mma_fmt<kFmtMxfp4>(a, ws, ws_bytes, s);
+  }
+}
+hipError_t launch_grouped_mma(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_grouped_mma_fmt<kFmtFp8F32>(a, n_segs, z_ext, s);
+    case kFmtNvfp4: return launch_grouped_mma_fmt<kFmtNvfp4>(a, n_segs, z_ext, s);
+    default: return launch_grouped_mma_fmt<kFmtMxfp4>(a, n_segs, z_ext, s);
+  }
+}
 }  // namespace dgpp_amd
 
 namespace {
@@ -111,7 +126,8 @@ namespace {
 // the chunking). k == 0 zero-fills. `out_elem` is 2 (bf16) or 4 (f32).
 int dense_rows(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,
                size_t out_stride, int out_f32, int m, int n, int k, hipStream_t stream, const char* who) {
-  const int max_rows = max_stage_rows(k);
+  // The matrix-core form takes every row in one launch (16 per weight pass); the vector form what LDS can stage.
+  const int max_rows = tune_get(kTuneCore) == 2 ? m : max_stage_rows(k);
   const size_t esz = out_f32 ? 4 : 2;
   for (int row0 = 0; row0 < m;) {
     const int rows = std::min(max_rows, m - row0);
@@ -236,7 +252,7 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
 
 int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
             int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32, size_t out_stride,
-            int n, int k, void* stream, const char* who) {
+            int n, int k, void* stream, const char* who, bool mma = false, const int32_t* act_rows = nullptr) {
   if (max_rows <= 0) return fail_arg(std::string(who) + ": max_rows must be positive");
   if (which < 0 || which > 2) return fail_arg(std::string(who) + ": which must be 0, 1 or 2");
   const unsigned z_ext = rows_per_block > 0 ? static_cast<unsigned>((max_rows + rows_per_block - 1) / rows_per_block) : 1u;
@@ -254,6 +270,8 @@ int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegmen
   a.k = k;
   a.rows_per_block = rows_per_block > 0 ? rows_per_block : INT_MAX;
   a.group_rows = max_stage_rows(k);
+  a.act_rows = act_rows;
+  if (mma) return finish(launch_grouped_mma(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
   return finish(launch_grouped(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
 }
 
@@ -577,52 +595,149 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
   return finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
 }
 
-// Routed-only down + ordered accumulation in one launch (no counterpart in the reference, which runs
-// launch_moe_slot_down* and launch_moe_slot_accum* back to back).
-static int slot_down_accum(int fmt, const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
-                           const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride, int slots,
-                           int top_k, const float* weights, uint16_t* out_bf16, float* out_f32, int* arrive,
-                           size_t arrive_len, void* stream, const char* who) {
-  if (slots <= 0) return DGPP_OK;
-  if (!act || !ids || !views || !slot_down || !weights || !arrive || (!out_bf16 && !out_f32))
-    return fail_arg(std::string(who) + ": null pointer");
-  if (n <= 0 || k <= 0 || top_k <= 0 || slots % (top_k + 1) != 0) return fail_arg(std::string(who) + ": degenerate dims");
-  if (out_stride < n) return fail_arg(std::string(who) + ": out_stride below n");
-  const size_t tokens = static_cast<size_t>(slots / (top_k + 1));
-  if (arrive_len < tokens * static_cast<size_t>((n + 3) / 4))
-    return fail_arg(std::string(who) + ": the arrival counters must hold tokens * ceil(n / 4) ints");
-  SlotArgs a = slot_args(act, act_stride, ids, order, views, slot_down, out_stride, slots, top_k, 0.f);
+// ---- matrix-core launchers (src/kernels/glm_moe_launch.hpp:103-125, :311-345; src/kernels/mma_gemv.hpp:65-85) -----
+static int dense_mma(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,
+                     int out_f32, size_t out_stride, int m, int n, int k, void* ws, size_t ws_bytes, void* stream,
+                     const char* who) {
+  if (out_stride == 0) out_stride = static_cast<size_t>(n);
+  if (out_stride < static_cast<size_t>(n)) return fail_arg(std::string(who) + ": output row stride narrower than n");
+  if ((m + kTileCols - 1) / kTileCols > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
+  DenseArgs a;
+  a.act = act;
+  a.act_stride = act_stride;
+  a.mat = mat;
+  a.global = global;
+  a.out = out;
+  a.out_stride = out_stride;
+  a.out_f32 = out_f32;
+  a.m = m;
   a.n = n;
   a.k = k;
-  a.want_shared = 0;
-  a.arrive = arrive;
-  a.arrivals = top_k;
-  a.weights = weights;
-  a.final_out = out_f32 ? static_cast<void*>(out_f32) : static_cast<void*>(out_bf16);
-  a.final_f32 = out_f32 != nullptr;
-  a.final_shared = 0;
-  return finish(launch_slot_down(fmt, a, as_stream(stream)), who);
+  return finish(launch_dense_mma(fmt, a, static_cast<float*>(ws), ws_bytes, as_stream(stream)), who);
 }
-int dgpp_launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
-                                    const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride,
-                                    int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
-                                    int* arrive, size_t arrive_len, void* stream) {
-  const char* who = "moe_slot_down_accum";
-  if (slots > 0 && (k % 16 != 0 || stage_bytes(1, k) > kMaxLdsBytes))
-    return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
-  return slot_down_accum(kFmtFp8F32, act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots, top_k,
-                         weights, out_bf16, out_f32, arrive, arrive_len, stream, who);
+
+static int dense_mma_fp8(const uint16_t* act, size_t act_stride, const uint8_t* payload, const void* scales, int e8m0,
+                         void* out, int out_f32, int m, int n, int k, size_t out_stride, int rs, int cs, void* ws,
+                         size_t ws_bytes, void* stream, const char* who) {
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  if (!act || !payload || !scales || !out) return fail_arg(std::string(who) + ": null pointer");
+  const bool row_grid = rs == 0 && cs >= 4;
+  if (!row_grid && (rs < 4 || rs > 7 || cs < 4 || cs > 7))
+    return fail_arg(std::string(who) + ": rs / cs must be 4..7 or a row grid (rs = 0, cs >= 4)");
+  if (k <= 0 || !fp8_shape_ok(payload, k))
+    return fail_arg(std::string(who) + ": k must be a positive multiple of 16 with a 16-byte aligned payload");
+  return dense_mma(e8m0 ? kFmtFp8E8M0 : kFmtFp8F32, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, out,
+                   out_f32, out_stride, m, n, k, ws, ws_bytes, stream, who);
 }
-int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
-                                        const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride,
-                                        int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
-                                        int* arrive, size_t arrive_len, void* stream, int fp4_group) {
-  const char* who = "moe_slot_down_accum_fp4";
+int dgpp_launch_dense_mma_bf16(const uint16_t* act, size_t act_stride, const uint8_t* payload, const float* scales,
+                               uint16_t* out, int m, int n, int k, void* stream, size_t out_stride) {
+  return dense_mma_fp8(act, act_stride, payload, scales, 0, out, 0, m, n, k, out_stride, 7, 7, nullptr, 0, stream, "dense_mma");
+}
+int dgpp_launch_dense_mma_f32(const uint16_t* act, size_t act_stride, const uint8_t* payload, const float* scales,
+                              float* out, int m, int n, int k, void* stream, size_t out_stride) {
+  return dense_mma_fp8(act, act_stride, payload, scales, 0, out, 1, m, n, k, out_stride, 7, 7, nullptr, 0, stream, "dense_mma");
+}
+int dgpp_launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
+                                  uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
+                                  void* ws, size_t ws_bytes) {
+  return dense_mma_fp8(act, act_stride, w, scales, 0, out, 0, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream, "mma_gemv_fp8");
+}
+int dgpp_launch_mma_gemv_fp8_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales, float* out,
+                                 int m, int n, int k, size_t out_stride, int rs, int cs, void* stream, void* ws,
+                                 size_t ws_bytes) {
+  return dense_mma_fp8(act, act_stride, w, scales, 0, out, 1, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream, "mma_gemv_fp8");
+}
+int dgpp_launch_mma_gemv_fp8e8m0_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
+                                      uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
+                                      void* ws, size_t ws_bytes) {
+  return dense_mma_fp8(act, act_stride, w, scales, 1, out, 0, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream,
+                       "mma_gemv_fp8e8m0");
+}
+int dgpp_launch_mma_gemv_fp8e8m0_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
+                                     float* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
+                                     void* ws, size_t ws_bytes) {
+  return dense_mma_fp8(act, act_stride, w, scales, 1, out, 1, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream,
+                       "mma_gemv_fp8e8m0");
+}
+
+static int dense_mma_fp4(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, void* out, int out_f32, int m,
+                         int n, int k, void* stream) {
+  const char* who = "dense_mma_fp4";
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  if (!w || !act || !w->payload || !w->scales || !out) return fail_arg(std::string(who) + ": null pointer");
+  if (w->scale_group != 16 && w->scale_group != 32)
+    return fail_arg(std::string(who) + ": the scale group must be 16 (NVFP4) or 32 (MXFP4)");
+  if (w->scale_group == 16 && !w->global_scale) return fail_arg(std::string(who) + ": an NVFP4 matrix needs its global scale");
+  if (w->rows < n || w->cols != k) return fail_arg(std::string(who) + ": matrix geometry does not match n, k");
+  if (k <= 0 || k % 32 != 0 || !aligned16(w->payload))
+    return fail_arg(std::string(who) + ": k must be a multiple of 32 and the payload 16-byte aligned");
+  MatRef mat;
+  mat.payload = w->payload;
+  mat.scales = w->scales;
+  mat.divisor = 1.f;
+  mat.rs = 0;
+  mat.cs = 0;
+  return dense_mma(w->scale_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, mat, w->global_scale, out, out_f32,
+                   static_cast<size_t>(n), m, n, k, nullptr, 0, stream, who);
+}
+int dgpp_launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out, int m,
+                                   int n, int k, void* stream) {
+  return dense_mma_fp4(act, act_stride, w, out, 0, m, n, k, stream);
+}
+int dgpp_launch_dense_mma_fp4_f32(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, float* out, int m, int n,
+                                  int k, void* stream) {
+  return dense_mma_fp4(act, act_stride, w, out, 1, m, n, k, stream);
+}
+
+static int grouped_mma_fp8(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
+                           int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
+                           size_t out_stride, int n, int k, void* stream, const int32_t* act_rows) {
+  const char* who = "moe grouped mma";
+  if (n_segs <= 0 || n <= 0) return DGPP_OK;
+  if (!act || !segs || !views || !out) return fail_arg(std::string(who) + ": null pointer");
+  if (k <= 0 || k % 16 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 16");
+  return grouped(kFmtFp8F32, act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_f32,
+                 out_stride, n, k, stream, who, true, act_rows);
+}
+int dgpp_launch_moe_grouped_mma_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                     int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                     uint16_t* out, size_t out_stride, int n, int k, void* stream,
+                                     const int32_t* act_rows) {
+  return grouped_mma_fp8(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 0, out_stride, n, k,
+                         stream, act_rows);
+}
+int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                    int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which, float* out,
+                                    size_t out_stride, int n, int k, void* stream, const int32_t* act_rows) {
+  return grouped_mma_fp8(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 1, out_stride, n, k,
+                         stream, act_rows);
+}
+static int grouped_mma_fp4(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
+                           int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
+                           size_t out_stride, int n, int k, void* stream, const int32_t* act_rows, int fp4_group) {
+  const char* who = "moe grouped mma fp4";
+  if (n_segs <= 0 || n <= 0) return DGPP_OK;
+  if (!act || !segs || !views || !out) return fail_arg(std::string(who) + ": null pointer");
   if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
-  if (slots > 0 && (!fp4_k_supported(k) || !fp4_k_compiled(k, fp4_group)))
-    return fail_arg(std::string(who) + ": k must be a multiple of 32 in the fp4 core's compiled set");
-  return slot_down_accum(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, ids, order, views, n, k, slot_down,
-                         out_stride, slots, top_k, weights, out_bf16, out_f32, arrive, arrive_len, stream, who);
+  if (k <= 0 || k % 32 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 32");
+  return grouped(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
+                 which, out, out_f32, out_stride, n, k, stream, who, true, act_rows);
+}
+int dgpp_launch_moe_grouped_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                         int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                         uint16_t* out, size_t out_stride, int n, int k, void* stream,
+                                         const int32_t* act_rows, int fp4_group, int tile_rows) {
+  (void)tile_rows;   // the reference's activation ring depth; one 16-row tile per weight pass here
+  return grouped_mma_fp4(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 0, out_stride, n, k,
+                         stream, act_rows, fp4_group);
+}
+int dgpp_launch_moe_grouped_mma_fp4_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                        int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                        float* out, size_t out_stride, int n, int k, void* stream, const int32_t* act_rows,
+                                        int fp4_group, int tile_rows) {
+  (void)tile_rows;
+  return grouped_mma_fp4(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, 1, out_stride, n, k,
+                         stream, act_rows, fp4_group);
 }
 
 static int grouped_fp8(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,

@@ -121,13 +121,6 @@ struct SlotArgs {
   float limit;
   int want_shared;          // 0: routed slots, 1: shared slots (others exit)
   int shared_view_base;     // >= 0: shared matrices come from views[base + which]
-  // Down only, optional: the ordered accumulation fused behind the last slot of a token.
-  int* arrive;              // [tokens, row tiles] arrival counters, zero at rest (left zero); null = not fused
-  int arrivals;             // slots per token whose down rows this launch produces
-  const float* weights;     // [tokens, top_k]
-  void* final_out;          // [tokens, n] bf16 bits or f32
-  int final_f32;
-  int final_shared;         // the chain ends with the token's shared slot (weight 1)
 };
 
 template <int FMT>
@@ -252,15 +245,10 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_
   }
 }
 
-// Down rows of a run of slots, unrounded f32. With `arrive` set, the block that completes a token's
-// last outstanding slot for its row tile also runs that token's accumulation chain over the tile
-// (a = 0; a = fma(w_j, y_j, a) for j ascending; the shared row last with weight 1; one rounding):
-// every block counts in once per slot after publishing its rows, the counter names the last one, so
-// no block ever waits for another. The chain's order is fixed, whoever runs it.
+// Down rows of a run of slots, unrounded f32.
 template <int FMT, int NB, int MAXM>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
-  __shared__ int s_last[MAXM];
   SlotRun<MAXM> run;
   if (!resolve_run<MAXM>(a, run)) return;
   const int rows_per_block = block_rows(g, steps);
@@ -296,49 +284,6 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_ker
         if (r < run.m) out[static_cast<size_t>(run.slot[r]) * a.out_stride + lr.row] = finish_dot<FMT>(acc[r], dd);
     }
   }
-  if (a.arrive == nullptr) return;
-  // Publish this block's rows, then count in once per slot of the run.
-  __threadfence();
-  __syncthreads();
-  if (static_cast<int>(threadIdx.x) < MAXM) {
-    int last = 0;
-#pragma unroll
-    for (int r = 0; r < MAXM; ++r) {
-      if (r == static_cast<int>(threadIdx.x) && r < run.m) {
-        int* counter = a.arrive + static_cast<size_t>(run.token[r]) * gridDim.x + blockIdx.x;
-        if (atomicAdd(counter, 1) == a.arrivals - 1) {
-          *counter = 0;   // zero at rest: nobody else touches this counter before the next launch
-          last = 1;
-        }
-      }
-    }
-    s_last[threadIdx.x] = last;
-  }
-  __syncthreads();
-  const int tile_end = min(a.n, tile_row0 + rows_per_block);
-#pragma unroll
-  for (int r = 0; r < MAXM; ++r) {
-    if (r >= run.m || !s_last[r]) continue;
-    __threadfence();   // the other slots' rows, published before their blocks counted in
-    const int t = run.token[r];
-    const size_t slot_base = static_cast<size_t>(t) * (a.top_k + 1);
-    for (int row = tile_row0 + static_cast<int>(threadIdx.x); row < tile_end; row += kBlockThreads) {
-      float v = 0.f;
-      for (int j = 0; j < a.top_k; ++j) {
-        const float y = __hip_atomic_load(out + (slot_base + j) * a.out_stride + row, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-        v = fmaf(a.weights[static_cast<size_t>(t) * a.top_k + j], y, v);
-      }
-      if (a.final_shared)
-        v = fmaf(1.0f, __hip_atomic_load(out + (slot_base + a.top_k) * a.out_stride + row, __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT), v);
-      const size_t at = static_cast<size_t>(t) * a.n + row;
-      if (a.final_f32)
-        static_cast<float*>(a.final_out)[at] = v;
-      else
-        static_cast<uint16_t*>(a.final_out)[at] = f32_to_bf16(v);
-    }
-  }
 }
 
 // ---- grouped (segment-major) twin ------------------------------------------------------------------
@@ -354,6 +299,7 @@ struct GroupedArgs {
   int n, k;
   int rows_per_block;  // segment rows per z block
   int group_rows;      // activation rows staged per pass (<= kMaxActRows)
+  const int32_t* act_rows;  // matrix-core form only, nullable: activation row of each segment row
 };
 
 template <int FMT, int NB>
@@ -397,6 +343,12 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void grouped_gemv_
   }
 }
 
+}  // namespace dgpp_amd
+
+#include "gemv_mfma_kernels.hpp"
+
+namespace dgpp_amd {
+
 // ---- host launch helpers (defined per format in gemv_fp8.hip / gemv_fp4.hip) ---------------------------
 // Elements per chunk by format, and the LDS bytes `rows` staged activation rows take.
 inline int elems_per_chunk(int fmt) { return fmt >= kFmtNvfp4 ? 32 : 16; }
@@ -415,6 +367,12 @@ hipError_t launch_dense(int fmt, const DenseArgs& a, hipStream_t stream);
 hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t stream);
 hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t stream);
 hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
+
+// The matrix-core launchers proper (the *_mma_* entry points).
+hipError_t launch_dense_mma(int fmt, const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t stream);
+hipError_t launch_grouped_mma(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
+template <int FMT> hipError_t launch_dense_mma_fmt(const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t stream);
+template <int FMT> hipError_t launch_grouped_mma_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
 
 // Per-format implementations.
 template <int FMT> hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream);
@@ -439,8 +397,93 @@ inline int max_stage_rows(int k) {
 
 // The bodies, included by the per-format translation units.
 #ifdef DGPP_GEMV_IMPL
+// The GEMV launchers run the vector ALU core (fastest while one or two activation rows ride on a weight
+// pass); the bench switch moves them to the matrix-core form, which the *_mma_* launchers always use.
+inline bool use_mfma_core() { return tune_get(kTuneCore) == 2; }
+
+// `ws` (nullable) holds parts * m * n floats: the K parts then run in separate blocks and a second
+// launch folds them (same bits); worth it only when the unsplit grid leaves the chip under-filled.
+template <int FMT>
+hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, size_t ws_bytes) {
+  const MGeom g = mgeom<FMT>(a.k);
+  const unsigned gx = static_cast<unsigned>((a.n + 63) / 64), gy = static_cast<unsigned>((a.m + kTileCols - 1) / kTileCols);
+  const size_t need = static_cast<size_t>(g.parts) * a.m * a.n * sizeof(float);
+  const bool split = ws != nullptr && g.parts > 1 && ws_bytes >= need && static_cast<size_t>(gx) * gy < 1024;
+  const dim3 grid(gx, gy, split ? g.parts : 1);
+  hipLaunchKernelGGL((mfma_dense_kernel<FMT, kMfmaNB>), grid, dim3(kBlockThreads), 2 * kStageUnits * sizeof(uint4), stream,
+                     a, g, split ? ws : nullptr);
+  if (split) {
+    const int64_t total = static_cast<int64_t>(a.m) * a.n;
+    hipLaunchKernelGGL(fold_parts_kernel<FMT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream, ws,
+                       g.parts, a.m, a.n, a.global, a.out, a.out_f32, a.out_stride);
+  }
+  return hipGetLastError();
+}
+
+template <int FMT>
+hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {
+  const MGeom g = mgeom<FMT>(a.k);
+  const dim3 grid(static_cast<unsigned>((a.n + 63) / 64), static_cast<unsigned>(n_segs), static_cast<unsigned>(z_ext));
+  hipLaunchKernelGGL((mfma_grouped_kernel<FMT, kMfmaNB>), grid, dim3(kBlockThreads), 2 * kStageUnits * sizeof(uint4),
+                     stream, a, g);
+  return hipGetLastError();
+}
+
+// Slots per run in the matrix-core slot kernels: bounded by the LDS of the per-wavefront stages.
+template <int FMT>
+inline int mfma_run_cap(const SlotArgs& a, const MGeom& g, int max_run) {
+  if (a.order == nullptr) return 1;
+  const int tuned = tune_get(kTuneSlotRun);
+  int cap = tuned > 0 && tuned < max_run ? tuned : max_run;
+  while (cap > 1 && (kWavesPerBlock * slot_wave_units<FMT>(cap, g) + kSlotRedUnits) * sizeof(uint4) > 48 * 1024) --cap;
+  return cap;
+}
+template <int FMT>
+inline size_t mfma_slot_lds(int maxm, const MGeom& g) {
+  return (static_cast<size_t>(kWavesPerBlock) * slot_wave_units<FMT>(maxm, g) + kSlotRedUnits) * sizeof(uint4);
+}
+
+template <int FMT>
+hipError_t launch_slot_gate_up_mfma(const SlotArgs& a, hipStream_t stream) {
+  const MGeom g = mgeom<FMT>(a.k);
+  const int rows_per_block = kWavesPerBlock / g.parts * kGroupRows;
+  const dim3 grid(static_cast<unsigned>((a.n + rows_per_block - 1) / rows_per_block), static_cast<unsigned>(a.slots));
+  const int cap = mfma_run_cap<FMT>(a, g, 2);
+  hipError_t err = hipSuccess;
+  auto go = [&](auto mc) {
+    constexpr int MAXM = decltype(mc)::value;
+    auto kern = slot_gate_up_mfma_kernel<FMT, kMfmaNB, MAXM>;
+    const size_t lds = mfma_slot_lds<FMT>(MAXM, g);
+    err = ensure_lds(kern, lds);
+    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g);
+  };
+  if (cap >= 2) go(std::integral_constant<int, 2>{});
+  else go(std::integral_constant<int, 1>{});
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+template <int FMT>
+hipError_t launch_slot_down_mfma(const SlotArgs& a, hipStream_t stream) {
+  const MGeom g = mgeom<FMT>(a.k);
+  const int rows_per_block = kWavesPerBlock / g.parts * kGroupRows;
+  const dim3 grid(static_cast<unsigned>((a.n + rows_per_block - 1) / rows_per_block), static_cast<unsigned>(a.slots));
+  const int cap = mfma_run_cap<FMT>(a, g, 2);
+  hipError_t err = hipSuccess;
+  auto go = [&](auto mc) {
+    constexpr int MAXM = decltype(mc)::value;
+    auto kern = slot_down_mfma_kernel<FMT, kMfmaNB, MAXM>;
+    const size_t lds = mfma_slot_lds<FMT>(MAXM, g);
+    err = ensure_lds(kern, lds);
+    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g);
+  };
+  if (cap >= 2) go(std::integral_constant<int, 2>{});
+  else go(std::integral_constant<int, 1>{});
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
 template <int FMT>
 hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
+  if (use_mfma_core()) return launch_dense_mfma<FMT>(a, stream, nullptr, 0);
   const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long block_steps = (a.n + rows_per_step - 1) / rows_per_step;
@@ -480,6 +523,7 @@ inline int run_cap_for(const SlotArgs& a, int max_run) {
 
 template <int FMT>
 hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
+  if (use_mfma_core()) return launch_slot_gate_up_mfma<FMT>(a, stream);
   const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
@@ -499,7 +543,7 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// Row tiles (grid x) of a down launch: the arrival counters of the fused accumulation are indexed
+// Row tiles (grid x) and steps of a vector-form down launch.
 // [token, tile].
 template <int FMT>
 inline void slot_down_grid(const SlotArgs& a, RowGeom& g, int& steps, unsigned& tiles) {
@@ -513,6 +557,7 @@ inline void slot_down_grid(const SlotArgs& a, RowGeom& g, int& steps, unsigned& 
 
 template <int FMT>
 hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
+  if (use_mfma_core()) return launch_slot_down_mfma<FMT>(a, stream);
   RowGeom g;
   int steps;
   unsigned tiles;
@@ -535,7 +580,17 @@ hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
 }
 
 template <int FMT>
+hipError_t launch_dense_mma_fmt(const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t stream) {
+  return launch_dense_mfma<FMT>(a, stream, ws, ws_bytes);
+}
+template <int FMT>
+hipError_t launch_grouped_mma_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {
+  return launch_grouped_mfma<FMT>(a, n_segs, z_ext, stream);
+}
+
+template <int FMT>
 hipError_t launch_grouped_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {
+  if (use_mfma_core()) return launch_grouped_mfma<FMT>(a, n_segs, z_ext, stream);
   const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_seg = (a.n + rows_per_step - 1) / rows_per_step;

@@ -1,0 +1,218 @@
+// The matrix-core form of the weight-streaming GEMV for gfx950: the same launchers, the same
+// layouts in memory, but the dot products run on v_mfma_f32_16x16x32_bf16 instead of the vector
+// ALU, so the per-weight vector work is the decode alone and up to 16 activation rows ride on one
+// pass over the weights.
+//
+// Shape. A wavefront owns a ROW GROUP of 16 weight rows. Lane (r = lane % 16, q = lane / 16) loads
+// 16 bytes of row r per STEP at byte offset step * 64 + q * 16: one load instruction reads 64
+// contiguous bytes of each of the 16 rows (128 FP4 or 64 FP8 elements per row and step). The lane
+// decodes its 16 bytes to bf16 in registers (hardware FP4 / FP8 conversions, block scale folded
+// in) and feeds them, 8 elements at a time, as the A operand; the B operand is the matching 8
+// activations of activation row (lane % 16), read as one 16-byte vector from an LDS stage laid
+// out [8-element block][activation row]. D[weight row][activation row] accumulates in fp32: lane
+// (r, q) ends up with weight rows 4q .. 4q+3 of activation row r.
+//
+// K is cut in PARTS (1, 2 or 4, a function of k alone): each part accumulates on its own and the
+// parts are added in ascending order at the end. The decode-slot kernels give each part to its own
+// wavefront (that is where a one-token batch gets its parallelism from); the dense and grouped
+// kernels walk the parts one after the other with one accumulator each. Both therefore run the
+// SAME arithmetic per (weight row, activation row): results do not depend on the launcher, the
+// grid, or how many activation rows share the pass.
+//
+// Value semantics are the vector core's (gemv_core.hpp); NVFP4 weights are formed as
+// bf16(e2m1 * e4m3), which is exact.
+#pragma once
+
+#include "gemv_core.hpp"
+
+namespace dgpp_amd {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+template <int FMT>
+struct MTraits {
+  static constexpr int kLoadElems = FmtTraits<FMT>::kElemsPerChunk;  // k elements of one 16-byte lane load
+  static constexpr int kSub = kLoadElems / 8;                        // MFMA operands per lane load
+  static constexpr int kStepElems = 4 * kLoadElems;                  // k elements per row and step
+  static constexpr int kStepBlocks = 4 * kSub;                       // 8-element blocks per row and step
+};
+
+constexpr int kMaxParts = 4;
+constexpr int kGroupRows = 16;       // weight rows of a row group
+constexpr int kTileCols = 16;        // activation rows of one MFMA tile
+
+struct MGeom {
+  int parts;       // 1, 2 or 4
+  int part_steps;  // steps per part (the last part may be shorter)
+  int steps;       // steps covering k
+};
+template <int FMT>
+__host__ __device__ inline MGeom mgeom(int k) {
+  constexpr int se = MTraits<FMT>::kStepElems;
+  MGeom g;
+  g.parts = k >= 4096 ? 4 : (k >= 2048 ? 2 : 1);
+  g.steps = (k + se - 1) / se;
+  g.part_steps = (g.steps + g.parts - 1) / g.parts;
+  return g;
+}
+
+union Frag {
+  bf16x8_t v;
+  bf16x2_t p[4];
+};
+
+// The MFMA A operands of one 16-byte lane load.
+template <int FMT>
+__device__ __forceinline__ void decode_frags(const ChunkRegs& ch, Frag (&f)[MTraits<FMT>::kSub]) {
+  const uint32_t w[4] = {ch.w.x, ch.w.y, ch.w.z, ch.w.w};
+  if constexpr (FMT == kFmtMxfp4) {
+    const float s = bits_f32(ch.s << 23);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      f[q].p[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 0);
+      f[q].p[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 1);
+      f[q].p[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 2);
+      f[q].p[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w[q], s, 3);
+    }
+  } else if constexpr (FMT == kFmtNvfp4) {
+    const float s0 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 0);
+    const float s1 = __builtin_amdgcn_cvt_f32_fp8(ch.s, 1);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float s = q < 2 ? s0 : s1;
+      const f32x2_t v0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[q], 1.0f, 0);
+      const f32x2_t v1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[q], 1.0f, 1);
+      const f32x2_t v2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[q], 1.0f, 2);
+      const f32x2_t v3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[q], 1.0f, 3);
+      f[q].p[0] = pack_bf16(v0.x * s, v0.y * s);
+      f[q].p[1] = pack_bf16(v1.x * s, v1.y * s);
+      f[q].p[2] = pack_bf16(v2.x * s, v2.y * s);
+      f[q].p[3] = pack_bf16(v3.x * s, v3.y * s);
+    }
+  } else if constexpr (FMT == kFmtFp8E8M0) {
+    const float s = bits_f32(ch.s << 23);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      f[q].p[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * q], s, false);
+      f[q].p[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * q], s, true);
+      f[q].p[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * q + 1], s, false);
+      f[q].p[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w[2 * q + 1], s, true);
+    }
+  } else {
+    const float s = bits_f32(ch.s);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[2 * q + h], false);
+        const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[2 * q + h], true);
+        f[q].p[2 * h + 0] = pack_bf16(lo.x * s, lo.y * s);
+        f[q].p[2 * h + 1] = pack_bf16(hi.x * s, hi.y * s);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ f32x4_t mfma_bf16(const Frag& a, const uint4& b, f32x4_t acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+}
+
+// Per-lane addressing of a row group: lane (r, q) of the group starting at row0.
+struct GroupLane {
+  const uint8_t* payload_row;
+  const void* scale_row;
+  int q;
+};
+template <int FMT>
+__device__ __forceinline__ GroupLane group_lane(const MatRef& mat, int row0, int n, int k) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row = row0 + (lane & 15);
+  const int r = row < n ? row : n - 1;   // rows past the end redo the last row; their results are dropped
+  GroupLane gl;
+  gl.q = lane >> 4;
+  if constexpr (FMT == kFmtFp8F32 || FMT == kFmtFp8E8M0) {
+    gl.payload_row = mat.payload + static_cast<size_t>(r) * k;
+    const size_t scale_cols = (static_cast<size_t>(k) + (1u << mat.cs) - 1) >> mat.cs;
+    const size_t esz = FMT == kFmtFp8F32 ? 4 : 1;
+    gl.scale_row = reinterpret_cast<const uint8_t*>(mat.scales) + (static_cast<size_t>(r >> mat.rs) * scale_cols) * esz;
+  } else {
+    gl.payload_row = mat.payload + static_cast<size_t>(r) * (k / 2);
+    gl.scale_row = reinterpret_cast<const uint8_t*>(mat.scales) +
+                   static_cast<size_t>(r) * (k / (FMT == kFmtNvfp4 ? 16 : 32));
+  }
+  return gl;
+}
+
+// The lane's 16 bytes of step `step` (chunk index step * 4 + q of the row), or zeros past k.
+template <int FMT>
+__device__ __forceinline__ void load_step(const GroupLane& gl, int step, int chunks, int cs, ChunkRegs& out) {
+  const int c = step * 4 + gl.q;
+  if (c < chunks) {
+    load_chunk<FMT>(gl.payload_row, gl.scale_row, c, cs, out);
+  } else {
+    out.w = make_uint4(0u, 0u, 0u, 0u);   // code 0 is +0 in e2m1 and e4m3
+    out.s = 0u;
+  }
+}
+
+// One 8-element block of an activation row as a 16-byte vector; zeros past k.
+__device__ __forceinline__ uint4 load_act_block(const uint16_t* __restrict__ row, int k0, int k, bool aligned) {
+  if (k0 >= k) return make_uint4(0u, 0u, 0u, 0u);
+  if (aligned) return *reinterpret_cast<const uint4*>(row + k0);
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = static_cast<uint32_t>(row[k0 + 2 * i]) | (static_cast<uint32_t>(row[k0 + 2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// acc += sum over the NB steps of `regs` (steps step0 ... relative to the stage at `stage`):
+// stage unit of (step t, lane q, sub j, activation row c) is ((t * 4 + q) * kSub + j) * m + c.
+// Only the first `valid` steps of the chunk exist (the rest hold zeros and their stage units may
+// never have been written, so they must not reach the matrix core).
+template <int FMT, int NB>
+__device__ __forceinline__ void mfma_chunk(const ChunkRegs (&regs)[NB], const uint4* __restrict__ lane_stage, int m,
+                                           int valid, f32x4_t& acc) {
+  constexpr int kSub = MTraits<FMT>::kSub;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    if (i < valid) {
+      Frag f[kSub];
+      decode_frags<FMT>(regs[i], f);
+#pragma unroll
+      for (int j = 0; j < kSub; ++j) acc = mfma_bf16(f[j], lane_stage[(i * 4 * kSub + j) * m], acc);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+template <int FMT, int NB>
+__device__ __forceinline__ void mfma_chunk_pair(const ChunkRegs (&ra)[NB], const ChunkRegs (&rb)[NB],
+                                                const uint4* __restrict__ lane_stage, int m, int valid,
+                                                f32x4_t& acc_a, f32x4_t& acc_b) {
+  constexpr int kSub = MTraits<FMT>::kSub;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    if (i < valid) {
+      Frag fa[kSub], fb[kSub];
+      decode_frags<FMT>(ra[i], fa);
+      decode_frags<FMT>(rb[i], fb);
+#pragma unroll
+      for (int j = 0; j < kSub; ++j) {
+        const uint4 b = lane_stage[(i * 4 * kSub + j) * m];
+        acc_a = mfma_bf16(fa[j], b, acc_a);
+        acc_b = mfma_bf16(fb[j], b, acc_b);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// The parts' sums in ascending order (parts is 1, 2 or 4).
+__device__ __forceinline__ f32x4_t fold_parts(const f32x4_t (&acc)[kMaxParts], int parts) {
+  f32x4_t s = acc[0];
+  if (parts >= 2) s = s + acc[1];
+  if (parts >= 4) s = (s + acc[2]) + acc[3];
+  return s;
+}
+
+}  // namespace dgpp_amd

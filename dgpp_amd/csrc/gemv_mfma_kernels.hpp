@@ -1,0 +1,336 @@
+// Kernels of the matrix-core GEMV form (gemv_mfma.hpp): dense projection and grouped segments
+// (block-shared, double-buffered activation stages), decode slots (one K part per wavefront).
+// Included by gemv_kernels.hpp after the argument structs.
+#pragma once
+
+#include "gemv_mfma.hpp"
+
+namespace dgpp_amd {
+
+constexpr int kStageUnits = 1024;   // 16-byte units of one block-shared activation stage (16 KB)
+constexpr int kMfmaNB = 4;          // lane loads in flight per row group and pass
+
+// Steps of one block-shared stage for mt activation rows: a multiple of kMfmaNB within the unit budget.
+template <int FMT>
+__host__ __device__ inline int stage_steps_for(int mt, int part_steps) {
+  int s = kStageUnits / (mt * MTraits<FMT>::kStepBlocks);
+  s -= s % kMfmaNB;
+  if (s < kMfmaNB) s = kMfmaNB;
+  const int cover = (part_steps + kMfmaNB - 1) / kMfmaNB * kMfmaNB;
+  return s < cover ? s : cover;
+}
+
+// 64 weight rows (one row group per wavefront) against mt <= 16 activation rows, all of K: the
+// block walks K in stages; a stage's activations sit in LDS as [8-element block][row], fetched one
+// stage ahead into registers. acc[p] receives part p's sum. Every thread of the block must call.
+// Parts [p_lo, p_hi) only (the others stay zero). `act_rows`, when given, names the activation
+// row of each of the mt rows (a gather folded into the stage load).
+template <int FMT, int NB>
+__device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_t* __restrict__ act, size_t act_stride,
+                                                const int32_t* __restrict__ act_rows, int mt, int n, int k, int row0,
+                                                const MGeom& g, int p_lo, int p_hi, uint4* __restrict__ lds,
+                                                f32x4_t (&acc)[kMaxParts]) {
+  constexpr int kSub = MTraits<FMT>::kSub;
+  constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
+  constexpr int kStepElems = MTraits<FMT>::kStepElems;
+  const int chunks = k / MTraits<FMT>::kLoadElems;
+  const GroupLane gl = group_lane<FMT>(mat, row0, n, k);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int cc = min(lane & 15, mt - 1);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(act) & 15u) == 0) && ((act_stride & 7u) == 0);
+  const int stage_steps = stage_steps_for<FMT>(mt, g.part_steps);
+  const int spp = (g.part_steps + stage_steps - 1) / stage_steps;
+  const int total = (p_hi - p_lo) * spp;
+  const int units = stage_steps * kStepBlocks * mt;
+  uint4 pre[4];
+  auto fetch = [&](int s) {
+    const int p = p_lo + s / spp, ls = s - (p - p_lo) * spp;
+    const int k_base = (p * g.part_steps + ls * stage_steps) * kStepElems;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = threadIdx.x + i * kBlockThreads;
+      if (idx < units) {
+        const int kb = idx / mt, c = idx - kb * mt;
+        const size_t arow = act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(c);
+        pre[i] = load_act_block(act + arow * act_stride, k_base + kb * 8, k, aligned);
+      }
+    }
+  };
+  auto put = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = threadIdx.x + i * kBlockThreads;
+      if (idx < units) lds[buf * kStageUnits + idx] = pre[i];
+    }
+  };
+#pragma unroll
+  for (int p = 0; p < kMaxParts; ++p) acc[p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  put(0);
+  __syncthreads();
+  int s = 0;
+#pragma unroll
+  for (int p = 0; p < kMaxParts; ++p) {
+    if (p >= p_lo && p < p_hi) {
+      for (int ls = 0; ls < spp; ++ls, ++s) {
+        const bool more = s + 1 < total;
+        if (more) fetch(s + 1);
+        const uint4* lane_stage = lds + (s & 1) * kStageUnits + (gl.q * kSub) * mt + cc;
+        const int step0 = p * g.part_steps + ls * stage_steps;
+        const int nsteps = min(stage_steps, g.part_steps - ls * stage_steps);
+        for (int t = 0; t < nsteps; t += NB) {
+          ChunkRegs regs[NB];
+#pragma unroll
+          for (int i = 0; i < NB; ++i) load_step<FMT>(gl, t + i < nsteps ? step0 + t + i : g.steps, chunks, mat.cs, regs[i]);
+          mfma_chunk<FMT, NB>(regs, lane_stage + (t * kStepBlocks) * mt, mt, min(NB, nsteps - t), acc[p]);
+        }
+        if (more) put((s + 1) & 1);
+        __syncthreads();
+      }
+    }
+  }
+}
+
+// Stores a folded tile: lane (c = lane % 16, q = lane / 16) holds weight rows row0 + 4q .. + 3 of
+// activation row c.
+template <int FMT>
+__device__ __forceinline__ void store_tile(const f32x4_t& v, float divisor, void* out, int out_f32, size_t out_row,
+                                           int row0, int n, bool live) {
+  if (!live) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int r = row0 + (lane >> 4) * 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (r + i < n) {
+      const float x = finish_dot<FMT>(v[i], divisor);
+      if (out_f32)
+        static_cast<float*>(out)[out_row + r + i] = x;
+      else
+        static_cast<uint16_t*>(out)[out_row + r + i] = f32_to_bf16(x);
+    }
+  }
+}
+
+// `partials` null: all parts in one block, folded and stored. Otherwise blockIdx.z names the ONE part
+// this block computes and its raw sums go to partials[part][row of out][n] (fp32); fold_parts_kernel
+// then adds the parts in the same ascending order — the split form's bits are the unsplit form's.
+template <int FMT, int NB>
+__global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs a, MGeom g, float* partials) {
+  extern __shared__ uint4 lds[];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int row0 = (static_cast<int>(blockIdx.x) * kWavesPerBlock + wave) * kGroupRows;
+  const int c0 = static_cast<int>(blockIdx.y) * kTileCols;
+  const int mt = min(kTileCols, a.m - c0);
+  const int c = lane & 15;
+  f32x4_t acc[kMaxParts];
+  if (partials == nullptr) {
+    block_rows_mfma<FMT, NB>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k,
+                             row0, g, 0, g.parts, lds, acc);
+    store_tile<FMT>(fold_parts(acc, g.parts), load_divisor<FMT>(a.global), a.out, a.out_f32,
+                    static_cast<size_t>(c0 + c) * a.out_stride, row0, a.n, c < mt);
+    return;
+  }
+  const int part = static_cast<int>(blockIdx.z);
+  block_rows_mfma<FMT, NB>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k, row0,
+                           g, part, part + 1, lds, acc);
+  f32x4_t mine = acc[0];
+#pragma unroll
+  for (int p = 1; p < kMaxParts; ++p) mine = part == p ? acc[p] : mine;
+  store_tile<kFmtMxfp4>(mine, 1.0f, partials, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
+}
+
+// out[r][j] = finish(((p0 + p1) + p2) + p3) over partials[part][r][j].
+template <int FMT>
+__global__ void fold_parts_kernel(const float* __restrict__ partials, int parts, int m, int n, const float* global,
+                                  void* out, int out_f32, size_t out_stride) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= static_cast<int64_t>(m) * n) return;
+  const int r = static_cast<int>(i / n), j = static_cast<int>(i - static_cast<int64_t>(r) * n);
+  const size_t plane = static_cast<size_t>(m) * n;
+  float s = partials[i];
+  if (parts >= 2) s = s + partials[plane + i];
+  if (parts >= 4) s = (s + partials[2 * plane + i]) + partials[3 * plane + i];
+  const float x = finish_dot<FMT>(s, load_divisor<FMT>(global));
+  const size_t at = static_cast<size_t>(r) * out_stride + j;
+  if (out_f32)
+    static_cast<float*>(out)[at] = x;
+  else
+    static_cast<uint16_t*>(out)[at] = f32_to_bf16(x);
+}
+
+template <int FMT, int NB>
+__global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedArgs a, MGeom g) {
+  extern __shared__ uint4 lds[];
+  const DgppMoeSegment seg = a.segs[blockIdx.y];
+  const int z0 = static_cast<int>(blockIdx.z) * a.rows_per_block;
+  if (z0 >= seg.rows) return;
+  const int z1 = min(seg.rows, z0 + a.rows_per_block);
+  const float* gp = nullptr;
+  const MatRef mat = mat_of_view<FMT>(a.views[seg.expert * 3 + a.which], &gp);
+  const float divisor = load_divisor<FMT>(gp);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int row0 = (static_cast<int>(blockIdx.x) * kWavesPerBlock + wave) * kGroupRows;
+  const int c = lane & 15;
+  for (int c0 = z0; c0 < z1; c0 += kTileCols) {
+    const int mt = min(kTileCols, z1 - c0);
+    f32x4_t acc[kMaxParts];
+    const size_t first = static_cast<size_t>(seg.row0 + c0);
+    block_rows_mfma<FMT, NB>(mat, a.act_rows ? a.act : a.act + first * a.act_stride, a.act_stride,
+                             a.act_rows ? a.act_rows + first : nullptr, mt, a.n, a.k, row0, g, 0, g.parts, lds, acc);
+    store_tile<FMT>(fold_parts(acc, g.parts), divisor, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, c < mt);
+  }
+}
+
+// ---- decode slots: one K part per wavefront ----------------------------------------------------------
+// A block's four wavefronts are 4 / parts row groups times `parts` K parts. Each wavefront stages
+// ITS part of the run's activation rows ([block][row], m <= MAXM rows) in its own LDS region, streams
+// its 16 rows over that part, and the part sums meet in LDS, added in ascending part order by the
+// part-0 wavefront (fold_parts' order).
+template <int FMT>
+__host__ __device__ inline int slot_wave_units(int maxm, const MGeom& g) {
+  return maxm * g.part_steps * MTraits<FMT>::kStepBlocks;
+}
+constexpr int kSlotRedUnits = kWavesPerBlock * 2 * kWave;   // f32x4 per lane, two tiles per wavefront
+
+template <int MAXM>
+__device__ __forceinline__ int pick_slot(const int (&v)[MAXM], int c) {
+  int s = v[0];
+#pragma unroll
+  for (int r = 1; r < MAXM; ++r) s = c == r ? v[r] : s;
+  return s;
+}
+
+// Stages rows x + idx[0 .. m-1] * x_stride (k bf16 values each) of this wavefront's K part.
+template <int FMT, int MAXM>
+__device__ __forceinline__ void stage_wave_part(const uint16_t* __restrict__ x, size_t x_stride, const int (&idx)[MAXM],
+                                                int m, int k, int part, const MGeom& g, uint4* __restrict__ stage) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int k_base = part * g.part_steps * MTraits<FMT>::kStepElems;
+  const int units = g.part_steps * MTraits<FMT>::kStepBlocks * m;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) && ((x_stride & 7u) == 0);
+  for (int u = lane; u < units; u += kWave) {
+    const int kb = u / m, r = u - kb * m;
+    const uint16_t* row = x + static_cast<size_t>(pick_slot<MAXM>(idx, r)) * x_stride;
+    stage[u] = load_act_block(row, k_base + kb * 8, k, aligned);
+  }
+}
+
+template <int FMT, int NB, int MAXM>
+__global__ __launch_bounds__(kBlockThreads, 2) void slot_gate_up_mfma_kernel(SlotArgs a, MGeom g) {
+  extern __shared__ uint4 lds[];
+  SlotRun<MAXM> run;
+  if (!resolve_run<MAXM>(a, run)) return;
+  const int gpb = kWavesPerBlock / g.parts;   // row groups per block
+  if (static_cast<int>(blockIdx.x) * gpb * kGroupRows >= a.n) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int grp = wave / g.parts, part = wave - grp * g.parts;
+  const int row0 = (static_cast<int>(blockIdx.x) * gpb + grp) * kGroupRows;
+  MatRef mg, mu;
+  const float *gg = nullptr, *gu = nullptr;
+  if (run.view_base >= 0) {
+    mg = mat_of_view<FMT>(a.views[run.view_base + 0], &gg);
+    mu = mat_of_view<FMT>(a.views[run.view_base + 1], &gu);
+  } else {
+    mg = a.sh[0];
+    mu = a.sh[1];
+  }
+  const int m = run.m;
+  const int wave_units = slot_wave_units<FMT>(MAXM, g);
+  uint4* stage = lds + wave * wave_units;
+  f32x4_t* red = reinterpret_cast<f32x4_t*>(lds + kWavesPerBlock * wave_units);
+  stage_wave_part<FMT, MAXM>(a.x, a.x_stride, run.token, m, a.k, part, g, stage);
+  __syncthreads();
+  constexpr int kSub = MTraits<FMT>::kSub;
+  constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
+  const int chunks = a.k / MTraits<FMT>::kLoadElems;
+  const GroupLane lg = group_lane<FMT>(mg, row0, a.n, a.k);
+  const GroupLane lu = group_lane<FMT>(mu, row0, a.n, a.k);
+  const int cc = min(lane & 15, m - 1);
+  const uint4* lane_stage = stage + (lg.q * kSub) * m + cc;
+  const int step0 = part * g.part_steps;
+  const int nsteps = min(g.part_steps, g.steps - step0);
+  f32x4_t ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < nsteps; t += NB) {
+    ChunkRegs rg[NB], ru[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int st = t + i < nsteps ? step0 + t + i : g.steps;
+      load_step<FMT>(lg, st, chunks, mg.cs, rg[i]);
+      load_step<FMT>(lu, st, chunks, mu.cs, ru[i]);
+    }
+    mfma_chunk_pair<FMT, NB>(rg, ru, lane_stage + (t * kStepBlocks) * m, m, min(NB, nsteps - t), ag, au);
+  }
+  if (g.parts > 1) {
+    if (part != 0) {
+      red[(wave * 2 + 0) * kWave + lane] = ag;
+      red[(wave * 2 + 1) * kWave + lane] = au;
+    }
+    __syncthreads();
+    if (part != 0) return;
+    ag = ag + red[((wave + 1) * 2 + 0) * kWave + lane];
+    au = au + red[((wave + 1) * 2 + 1) * kWave + lane];
+    if (g.parts == 4) {
+      ag = (ag + red[((wave + 2) * 2 + 0) * kWave + lane]) + red[((wave + 3) * 2 + 0) * kWave + lane];
+      au = (au + red[((wave + 2) * 2 + 1) * kWave + lane]) + red[((wave + 3) * 2 + 1) * kWave + lane];
+    }
+  }
+  const int c = lane & 15;
+  if (c >= m) return;
+  const float dg = load_divisor<FMT>(gg), du = load_divisor<FMT>(gu);
+  uint16_t* act_row = static_cast<uint16_t*>(a.out) + static_cast<size_t>(pick_slot<MAXM>(run.slot, c)) * a.out_stride;
+  const int r = row0 + (lane >> 4) * 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (r + i < a.n) act_row[r + i] = swiglu_bf16(finish_dot<FMT>(ag[i], dg), finish_dot<FMT>(au[i], du), a.limit);
+}
+
+template <int FMT, int NB, int MAXM>
+__global__ __launch_bounds__(kBlockThreads, 2) void slot_down_mfma_kernel(SlotArgs a, MGeom g) {
+  extern __shared__ uint4 lds[];
+  SlotRun<MAXM> run;
+  if (!resolve_run<MAXM>(a, run)) return;
+  const int gpb = kWavesPerBlock / g.parts;
+  if (static_cast<int>(blockIdx.x) * gpb * kGroupRows >= a.n) return;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int grp = wave / g.parts, part = wave - grp * g.parts;
+  const int row0 = (static_cast<int>(blockIdx.x) * gpb + grp) * kGroupRows;
+  MatRef md;
+  const float* gd = nullptr;
+  if (run.view_base >= 0)
+    md = mat_of_view<FMT>(a.views[run.view_base + 2], &gd);
+  else
+    md = a.sh[0];
+  const int m = run.m;
+  const int wave_units = slot_wave_units<FMT>(MAXM, g);
+  uint4* stage = lds + wave * wave_units;
+  f32x4_t* red = reinterpret_cast<f32x4_t*>(lds + kWavesPerBlock * wave_units);
+  stage_wave_part<FMT, MAXM>(a.x, a.x_stride, run.slot, m, a.k, part, g, stage);
+  __syncthreads();
+  constexpr int kSub = MTraits<FMT>::kSub;
+  constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
+  const int chunks = a.k / MTraits<FMT>::kLoadElems;
+  const GroupLane ld = group_lane<FMT>(md, row0, a.n, a.k);
+  const int cc = min(lane & 15, m - 1);
+  const uint4* lane_stage = stage + (ld.q * kSub) * m + cc;
+  const int step0 = part * g.part_steps;
+  const int nsteps = min(g.part_steps, g.steps - step0);
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < nsteps; t += NB) {
+    ChunkRegs regs[NB];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) load_step<FMT>(ld, t + i < nsteps ? step0 + t + i : g.steps, chunks, md.cs, regs[i]);
+    mfma_chunk<FMT, NB>(regs, lane_stage + (t * kStepBlocks) * m, m, min(NB, nsteps - t), acc);
+  }
+  if (g.parts > 1) {
+    if (part != 0) red[wave * kWave + lane] = acc;
+    __syncthreads();
+    if (part != 0) return;
+    acc = acc + red[(wave + 1) * kWave + lane];
+    if (g.parts == 4) acc = (acc + red[(wave + 2) * kWave + lane]) + red[(wave + 3) * kWave + lane];
+  }
+  const int c = lane & 15;
+  store_tile<FMT>(acc, load_divisor<FMT>(gd), a.out, 1,
+                  static_cast<size_t>(pick_slot<MAXM>(run.slot, c)) * a.out_stride, row0, a.n, c < m);
+}
+
+}  // namespace dgpp_amd

@@ -18,8 +18,8 @@ size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 
 // Buffer sizes in bytes, in the order they are carved (each rounded to 256).
 struct Layout {
-  size_t views, ids, weights, scores, biased, order, slot_act, slot_down, acc, counter, arrive, rows, slot_row, segs,
-      gather, gate, up, total;
+  size_t views, ids, weights, scores, biased, order, slot_act, slot_down, acc, counter, rows, slot_row, segs, gather,
+      gate, up, total;
 };
 Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t n_views) {
   const size_t M = static_cast<size_t>(std::max(max_tokens, 0)), H = c.hidden, K = c.top_k, E = c.n_experts;
@@ -36,7 +36,6 @@ Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t
   l.slot_down = align_up(slots * H * 4);
   l.acc = align_up(M * H * 4);
   l.counter = align_up(2 * sizeof(int));
-  l.arrive = align_up(M * ((H + 3) / 4) * sizeof(int));
   l.rows = align_up(slots * 4);
   l.slot_row = align_up(M * K * 4);
   l.segs = align_up((E + 1) * sizeof(MoeSegment));
@@ -44,7 +43,7 @@ Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t
   l.gate = align_up(slots * I * 2);
   l.up = align_up(slots * I * 2);
   l.total = l.views + l.ids + l.weights + l.scores + l.biased + l.order + l.slot_act + l.slot_down + l.acc + l.counter +
-            l.arrive + l.rows + l.slot_row + l.segs + l.gather + l.gate + l.up;
+            l.rows + l.slot_row + l.segs + l.gather + l.gate + l.up;
   return l;
 }
 
@@ -111,8 +110,6 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   d_slot_down_ = reinterpret_cast<float*>(carve(l.slot_down));
   d_acc_ = reinterpret_cast<float*>(carve(l.acc));
   d_tile_counter_ = reinterpret_cast<int*>(carve(l.counter));
-  d_arrive_ = reinterpret_cast<int*>(carve(l.arrive));
-  arrive_len_ = l.arrive / sizeof(int);
   d_rows_ = reinterpret_cast<int32_t*>(carve(l.rows));
   d_slot_row_ = reinterpret_cast<int32_t*>(carve(l.slot_row));
   d_segs_ = reinterpret_cast<MoeSegment*>(carve(l.segs));
@@ -124,7 +121,6 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   hip_ok(hipMemcpy(d_views_, w.views.data(), w.views.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
          "GlmMoeLayer: table upload");
   hip_ok(hipMemset(d_tile_counter_, 0, 2 * sizeof(int)), "GlmMoeLayer: counter");
-  hip_ok(hipMemset(d_arrive_, 0, l.arrive), "GlmMoeLayer: arrival counters");
 }
 
 GlmMoeLayer::~GlmMoeLayer() {
@@ -178,16 +174,10 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   const bool sh_args = has_shared() && !w_.shared_in_table;
   const int n_sh = has_shared() ? w_.shared_inter : 0;
   const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
-  const bool fused = !has_shared() && dgpp_tune_get(4) == 1;   // down rows + accumulation in one launch
   if (w_.format == GlmExpertFormat::Fp8) {
     launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
                                    w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
                                    K, cfg_.swiglu_limit, stream, w_.sh_rs, w_.sh_cs);
-    if (fused) {
-      launch_moe_slot_down_accum(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, d_slot_down_,
-                                 H, slots, K, weights, out_bf16, out_f32, d_arrive_, arrive_len_, stream);
-      return;
-    }
     launch_moe_slot_down(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
                          n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, stream, w_.sh_rs, w_.sh_cs);
   } else {
@@ -197,12 +187,6 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
                                        sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
                                        d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, stream, base, fp4_group_,
                                        w_.sh_rs, w_.sh_cs);
-    if (fused) {
-      launch_moe_slot_down_accum_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
-                                     d_slot_down_, H, slots, K, weights, out_bf16, out_f32, d_arrive_, arrive_len_,
-                                     stream, fp4_group_);
-      return;
-    }
     launch_moe_slot_down_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
                              has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
                              sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, stream, base, fp4_group_,
@@ -250,6 +234,40 @@ void GlmMoeLayer::enqueue_grouped_routed(const uint16_t* x, size_t x_stride, con
   else
     launch_moe_grouped_gemv_fp4_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream,
                                     fp4_group_);
+  if (out_f32)
+    launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+  else
+    launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+}
+
+// The matrix-core grouped path (the reference's prefill form, src/models/glm/moe_layer.cpp:775-817): the same
+// stages as enqueue_grouped_routed with the gather folded into the gate / up launches (act_rows) and 16 token
+// rows per weight pass.
+void GlmMoeLayer::enqueue_prefill_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                                         uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  if (has_shared())
+    throw std::invalid_argument("GlmMoeLayer: the grouped path here covers the routed experts (no shared segment)");
+  const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter, E = cfg_.n_experts;
+  const int tk = tokens * K;
+  launch_moe_segment(ids, tokens, K, E, d_rows_, d_slot_row_, d_segs_, stream);
+  const int max_rows = tokens;
+  if (w_.format == GlmExpertFormat::Fp8) {
+    launch_moe_grouped_mma_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 0, d_gate_, I, I, H, stream, d_rows_);
+    launch_moe_grouped_mma_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 1, d_up_, I, I, H, stream, d_rows_);
+  } else {
+    launch_moe_grouped_mma_fp4_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 0, d_gate_, I, I, H, stream, d_rows_,
+                                    fp4_group_);
+    launch_moe_grouped_mma_fp4_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 1, d_up_, I, I, H, stream, d_rows_,
+                                    fp4_group_);
+  }
+  launch_moe_swiglu_clamp(d_gate_, d_up_, d_slot_act_, static_cast<int64_t>(tk) * I, cfg_.swiglu_limit, stream);
+  if (w_.format == GlmExpertFormat::Fp8)
+    launch_moe_grouped_mma_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream);
+  else
+    launch_moe_grouped_mma_fp4_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream,
+                                   nullptr, fp4_group_);
   if (out_f32)
     launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
   else
@@ -348,6 +366,13 @@ int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* l, const uint16_t* x, si
                                           void* stream) {
   return guarded([&] {
     l->impl.enqueue_grouped_routed(x, x_stride, ids, weights, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
+  });
+}
+int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                          const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
+                                          void* stream) {
+  return guarded([&] {
+    l->impl.enqueue_prefill_routed(x, x_stride, ids, weights, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
   });
 }
 const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* l) { return l->impl.views(); }

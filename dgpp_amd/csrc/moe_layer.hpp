@@ -48,6 +48,9 @@ class GlmMoeLayer {
                              uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
   void enqueue_grouped_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                               uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
+  // The same through the matrix-core grouped launchers (gather folded in, 16 token rows per weight pass).
+  void enqueue_prefill_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                              uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
 
   const MoeExpertView* views() const { return d_views_; }
   const int32_t* ids() const { return d_ids_; }
@@ -77,9 +80,6 @@ class GlmMoeLayer {
   float* d_slot_down_ = nullptr;     // [slots, hidden]
   float* d_acc_ = nullptr;           // [tokens, hidden]
   int* d_tile_counter_ = nullptr;    // [2]
-  int* d_arrive_ = nullptr;          // [max_tokens, ceil(hidden / 4)] arrival counters of the fused down + accumulate
-  size_t arrive_len_ = 0;
-  bool fuse_accum_ = true;
   int32_t* d_rows_ = nullptr;        // grouped path
   int32_t* d_slot_row_ = nullptr;
   MoeSegment* d_segs_ = nullptr;

@@ -191,22 +191,6 @@ def launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_rou
         _p(tile_counter)))
 
 
-def launch_moe_slot_down_accum(act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots, top_k, weights,
-                               out_bf16, out_f32, arrive, arrive_len, stream=None):
-    """Extension: routed down rows + the ordered accumulation in one launch (FP8 experts)."""
-    _check(_lib.load().dgpp_launch_moe_slot_down_accum(
-        _p(act), act_stride, _p(ids), _p(order), _p(views), n, k, _p(slot_down), out_stride, slots, top_k,
-        _p(weights), _p(out_bf16), _p(out_f32), _p(arrive), arrive_len, _stream(stream)))
-
-
-def launch_moe_slot_down_accum_fp4(act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots, top_k,
-                                   weights, out_bf16, out_f32, arrive, arrive_len, stream=None, fp4_group=16):
-    """Extension: routed down rows + the ordered accumulation in one launch (NVFP4 / MXFP4 experts)."""
-    _check(_lib.load().dgpp_launch_moe_slot_down_accum_fp4(
-        _p(act), act_stride, _p(ids), _p(order), _p(views), n, k, _p(slot_down), out_stride, slots, top_k,
-        _p(weights), _p(out_bf16), _p(out_f32), _p(arrive), arrive_len, _stream(stream), fp4_group))
-
-
 # ---- grouped twins ---------------------------------------------------------------------------------------
 def launch_moe_grouped_gemv_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                  out_stride, n, k, stream=None):
@@ -316,3 +300,75 @@ def launch_fp8_dequant_blocks(payload, scales, out_bf16, rows, cols, stream=None
 def launch_fp8_dequant_blocks_e8m0(payload, scales, out_bf16, rows, cols, stream, rs, cs):
     _check(_lib.load().dgpp_launch_fp8_dequant_blocks_e8m0(_p(payload), _p(scales), _p(out_bf16), rows, cols,
                                                            _stream(stream), rs, cs))
+
+
+# ---- matrix-core launchers (src/kernels/glm_moe_launch.hpp:103-125, :311-345; src/kernels/mma_gemv.hpp:65-85) ----
+def launch_dense_mma_bf16(act, act_stride, payload, scales, out, m, n, k, stream=None, out_stride=0):
+    _check(_lib.load().dgpp_launch_dense_mma_bf16(_p(act), act_stride, _p(payload), _p(scales), _p(out), m, n, k,
+                                                  _stream(stream), out_stride))
+
+
+def launch_dense_mma_f32(act, act_stride, payload, scales, out, m, n, k, stream=None, out_stride=0):
+    _check(_lib.load().dgpp_launch_dense_mma_f32(_p(act), act_stride, _p(payload), _p(scales), _p(out), m, n, k,
+                                                 _stream(stream), out_stride))
+
+
+def launch_dense_mma_fp4_bf16(act, act_stride, w: Fp4Matrix, out, m, n, k, stream=None):
+    _check(_lib.load().dgpp_launch_dense_mma_fp4_bf16(_p(act), act_stride, C.addressof(w), _p(out), m, n, k, _stream(stream)))
+
+
+def launch_dense_mma_fp4_f32(act, act_stride, w: Fp4Matrix, out, m, n, k, stream=None):
+    _check(_lib.load().dgpp_launch_dense_mma_fp4_f32(_p(act), act_stride, C.addressof(w), _p(out), m, n, k, _stream(stream)))
+
+
+def _mma_gemv(name, act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws, ws_bytes):
+    _check(getattr(_lib.load(), name)(_p(act), act_stride, _p(w), _p(scales), _p(out), m, n, k, out_stride, rs, cs,
+                                      _stream(stream), _p(ws), ws_bytes))
+
+
+def launch_mma_gemv_fp8_bf16(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream=None, ws=None, ws_bytes=0):
+    _mma_gemv("dgpp_launch_mma_gemv_fp8_bf16", act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws, ws_bytes)
+
+
+def launch_mma_gemv_fp8_f32(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream=None, ws=None, ws_bytes=0):
+    _mma_gemv("dgpp_launch_mma_gemv_fp8_f32", act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws, ws_bytes)
+
+
+def launch_mma_gemv_fp8e8m0_bf16(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream=None, ws=None,
+                                 ws_bytes=0):
+    _mma_gemv("dgpp_launch_mma_gemv_fp8e8m0_bf16", act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws,
+              ws_bytes)
+
+
+def launch_mma_gemv_fp8e8m0_f32(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream=None, ws=None,
+                                ws_bytes=0):
+    _mma_gemv("dgpp_launch_mma_gemv_fp8e8m0_f32", act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws,
+              ws_bytes)
+
+
+def launch_moe_grouped_mma_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_stride, n,
+                                k, stream=None, act_rows=None):
+    _check(_lib.load().dgpp_launch_moe_grouped_mma_bf16(_p(act), act_stride, _p(segs), n_segs, max_rows, rows_per_block,
+                                                        _p(views), which, _p(out), out_stride, n, k, _stream(stream),
+                                                        _p(act_rows)))
+
+
+def launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_stride, n, k,
+                               stream=None, act_rows=None):
+    _check(_lib.load().dgpp_launch_moe_grouped_mma_f32(_p(act), act_stride, _p(segs), n_segs, max_rows, rows_per_block,
+                                                       _p(views), which, _p(out), out_stride, n, k, _stream(stream),
+                                                       _p(act_rows)))
+
+
+def launch_moe_grouped_mma_fp4_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_stride,
+                                    n, k, stream=None, act_rows=None, fp4_group=16, tile_rows=64):
+    _check(_lib.load().dgpp_launch_moe_grouped_mma_fp4_bf16(_p(act), act_stride, _p(segs), n_segs, max_rows, rows_per_block,
+                                                            _p(views), which, _p(out), out_stride, n, k, _stream(stream),
+                                                            _p(act_rows), fp4_group, tile_rows))
+
+
+def launch_moe_grouped_mma_fp4_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_stride,
+                                   n, k, stream=None, act_rows=None, fp4_group=16, tile_rows=64):
+    _check(_lib.load().dgpp_launch_moe_grouped_mma_fp4_f32(_p(act), act_stride, _p(segs), n_segs, max_rows, rows_per_block,
+                                                           _p(views), which, _p(out), out_stride, n, k, _stream(stream),
+                                                           _p(act_rows), fp4_group, tile_rows))

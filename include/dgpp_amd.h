@@ -40,8 +40,9 @@ const char* dgpp_target_arch(void);
  * keeps such a switch in its launcher header too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90).
  * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: slots of one expert a
  * decode-slot block serves together (0 = default: 2 gate/up, 4 down; 1 = one slot per block);
- * key 2: row steps per block of the slot launches (0 = automatic). Outputs do not depend on keys 1
- * and 2; key 0 changes the fp32 summation order (every launcher follows it alike). */
+ * key 2: row steps per block of the slot launches (0 = automatic); key 5: 2 moves the GEMV launchers
+ * to the matrix-core form (another fp32 summation order, all launchers alike). Outputs do not depend on
+ * keys 1 and 2; key 0 changes the fp32 summation order (every launcher follows it alike). */
 void dgpp_tune_set(int key, int value);
 int dgpp_tune_get(int key);
 
@@ -227,24 +228,6 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
                                   int* tile_counter);
 
 /* ---- grouped (segment-major) GEMV twins ------------------------------------------------------------ */
-/* Extension (no counterpart in the reference, which runs launch_moe_slot_down* and
- * launch_moe_slot_accum* back to back): the routed slots' down rows AND the token's ordered
- * accumulation chain in one launch. `slot_down` [slots, out_stride] f32 receives the unrounded down
- * rows as launch_moe_slot_down* writes them; the block that finishes a token's last outstanding slot
- * for a row tile then runs the chain of launch_moe_slot_accum_routed_* over that tile into out_f32
- * (when given) or out_bf16, [tokens, n]. `arrive` holds at least tokens * ceil(n / 4) ints, zero before
- * the first call and left zero by every call; calls sharing it must be ordered on one stream.
- * Results are bit-identical to the two-launch form. No shared slot: chain it separately. */
-int dgpp_launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
-                                    const DgppMoeExpertView* views, int n, int k, float* slot_down, int out_stride,
-                                    int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
-                                    int* arrive, size_t arrive_len, void* stream);
-int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
-                                        const int32_t* order, const DgppMoeExpertView* views, int n, int k,
-                                        float* slot_down, int out_stride, int slots, int top_k, const float* weights,
-                                        uint16_t* out_bf16, float* out_f32, int* arrive, size_t arrive_len,
-                                        void* stream, int fp4_group);
-
 /* src/kernels/glm_moe_launch.hpp:77-87 */
 int dgpp_launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride,
                                       const DgppMoeSegment* segs, int n_segs, int max_rows,
@@ -267,6 +250,53 @@ int dgpp_launch_moe_grouped_gemv_fp4_f32(const uint16_t* act, size_t act_stride,
                                          void* stream, int fp4_group);
 
 /* ---- dense NVFP4 / MXFP4 projection GEMV -------------------------------------------------------------- */
+/* ---- matrix-core launchers ------------------------------------------------------------------
+ * The reference's tensor-core forms of the same products (src/kernels/glm_moe_launch.hpp:103-125 dense and
+ * grouped FP8, :311-345 grouped and dense FP4; src/kernels/mma_gemv.hpp:65-85 FP8 with a scale grid given
+ * as shifts, F32 or E8M0). Here they run on v_mfma_f32_16x16x32_bf16: 16 activation rows ride on one pass
+ * over the weights, any m (16-row tiles). A (weight row, activation row) result does not depend on m, on
+ * the launcher (dense == grouped == split form, bit for bit) or on `ws`; it is NOT bitwise the GEMV
+ * launchers' (another summation order) and is held to the same oracle tolerance.
+ * act_rows (nullable): segment row i reads activation row act_rows[i] (the gather folded in).
+ * ws / ws_bytes (nullable): room for parts(k) * m * n floats lets an under-filled grid run the K parts in
+ * separate blocks plus one folding launch. rows_per_block: segment rows per z block (0 = all).
+ * tile_rows is accepted for the signature and ignored. */
+int dgpp_launch_dense_mma_bf16(const uint16_t* act, size_t act_stride, const uint8_t* payload, const float* scales,
+                               uint16_t* out, int m, int n, int k, void* stream, size_t out_stride);
+int dgpp_launch_dense_mma_f32(const uint16_t* act, size_t act_stride, const uint8_t* payload, const float* scales,
+                              float* out, int m, int n, int k, void* stream, size_t out_stride);
+int dgpp_launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out, int m,
+                                   int n, int k, void* stream);
+int dgpp_launch_dense_mma_fp4_f32(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, float* out, int m, int n,
+                                  int k, void* stream);
+int dgpp_launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
+                                  uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
+                                  void* ws, size_t ws_bytes);
+int dgpp_launch_mma_gemv_fp8_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales, float* out,
+                                 int m, int n, int k, size_t out_stride, int rs, int cs, void* stream, void* ws,
+                                 size_t ws_bytes);
+int dgpp_launch_mma_gemv_fp8e8m0_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
+                                      uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
+                                      void* ws, size_t ws_bytes);
+int dgpp_launch_mma_gemv_fp8e8m0_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
+                                     float* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
+                                     void* ws, size_t ws_bytes);
+int dgpp_launch_moe_grouped_mma_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                     int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                     uint16_t* out, size_t out_stride, int n, int k, void* stream,
+                                     const int32_t* act_rows);
+int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                    int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which, float* out,
+                                    size_t out_stride, int n, int k, void* stream, const int32_t* act_rows);
+int dgpp_launch_moe_grouped_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                         int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                         uint16_t* out, size_t out_stride, int n, int k, void* stream,
+                                         const int32_t* act_rows, int fp4_group, int tile_rows);
+int dgpp_launch_moe_grouped_mma_fp4_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
+                                        int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
+                                        float* out, size_t out_stride, int n, int k, void* stream, const int32_t* act_rows,
+                                        int fp4_group, int tile_rows);
+
 /* src/kernels/fp4_gemv.hpp:23-32. `w` is a HOST struct holding device pointers. */
 int dgpp_launch_fp4_gemv_bf16(const uint16_t* act, size_t act_row_stride_elems,
                               const DgppFp4Matrix* w, uint16_t* out, int m, int n, int k,

@@ -223,23 +223,6 @@ inline void launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, con
                                               k_shared, sh_payload, sh_scales, out, out_stride, slots, top_k, stream,
                                               shared_view_base, fp4_group, sh_rs, sh_cs, tile_counter));
 }
-// Extensions: down rows + ordered accumulation in one launch (see dgpp_amd.h).
-inline void launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
-                                       const MoeExpertView* views, int n, int k, float* slot_down, int out_stride,
-                                       int slots, int top_k, const float* weights, uint16_t* out_bf16, float* out_f32,
-                                       int* arrive, size_t arrive_len, hipStream_t stream) {
-  detail::check(dgpp_launch_moe_slot_down_accum(act, act_stride, ids, order, views, n, k, slot_down, out_stride, slots,
-                                                top_k, weights, out_bf16, out_f32, arrive, arrive_len, stream));
-}
-inline void launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
-                                           const int32_t* order, const MoeExpertView* views, int n, int k,
-                                           float* slot_down, int out_stride, int slots, int top_k, const float* weights,
-                                           uint16_t* out_bf16, float* out_f32, int* arrive, size_t arrive_len,
-                                           hipStream_t stream, int fp4_group = 16) {
-  detail::check(dgpp_launch_moe_slot_down_accum_fp4(act, act_stride, ids, order, views, n, k, slot_down, out_stride,
-                                                    slots, top_k, weights, out_bf16, out_f32, arrive, arrive_len,
-                                                    stream, fp4_group));
-}
 inline void launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
                                          int max_rows, int rows_per_block, const MoeExpertView* views, int which,
                                          uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream) {
@@ -283,6 +266,76 @@ inline void launch_fp4_gemv_f32(const uint16_t* act, size_t act_row_stride_elems
   detail::check(dgpp_launch_fp4_gemv_f32(act, act_row_stride_elems, &w, out, m, n, k, stream));
 }
 inline bool fp4_gemv_accepts(const GlmFp4Matrix& w) { return dgpp_fp4_gemv_accepts(&w) != 0; }
+
+// ---- matrix-core launchers: src/kernels/glm_moe_launch.hpp:103-125, :311-345; src/kernels/mma_gemv.hpp:65-85 ----
+inline void launch_dense_mma_bf16(const uint16_t* act, size_t act_stride, const uint8_t* payload, const float* scales,
+                                  uint16_t* out, int m, int n, int k, hipStream_t stream, size_t out_stride = 0) {
+  detail::check(dgpp_launch_dense_mma_bf16(act, act_stride, payload, scales, out, m, n, k, stream, out_stride));
+}
+inline void launch_dense_mma_f32(const uint16_t* act, size_t act_stride, const uint8_t* payload, const float* scales,
+                                 float* out, int m, int n, int k, hipStream_t stream, size_t out_stride = 0) {
+  detail::check(dgpp_launch_dense_mma_f32(act, act_stride, payload, scales, out, m, n, k, stream, out_stride));
+}
+inline void launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const GlmFp4Matrix& w, uint16_t* out, int m,
+                                      int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_dense_mma_fp4_bf16(act, act_stride, &w, out, m, n, k, stream));
+}
+inline void launch_dense_mma_fp4_f32(const uint16_t* act, size_t act_stride, const GlmFp4Matrix& w, float* out, int m, int n,
+                                     int k, hipStream_t stream) {
+  detail::check(dgpp_launch_dense_mma_fp4_f32(act, act_stride, &w, out, m, n, k, stream));
+}
+inline void launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
+                                     uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs,
+                                     hipStream_t stream, void* ws = nullptr, size_t ws_bytes = 0) {
+  detail::check(dgpp_launch_mma_gemv_fp8_bf16(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws, ws_bytes));
+}
+inline void launch_mma_gemv_fp8_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales, float* out,
+                                    int m, int n, int k, size_t out_stride, int rs, int cs, hipStream_t stream,
+                                    void* ws = nullptr, size_t ws_bytes = 0) {
+  detail::check(dgpp_launch_mma_gemv_fp8_f32(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws, ws_bytes));
+}
+inline void launch_mma_gemv_fp8e8m0_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
+                                         uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs,
+                                         hipStream_t stream, void* ws = nullptr, size_t ws_bytes = 0) {
+  detail::check(dgpp_launch_mma_gemv_fp8e8m0_bf16(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws,
+                                                  ws_bytes));
+}
+inline void launch_mma_gemv_fp8e8m0_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
+                                        float* out, int m, int n, int k, size_t out_stride, int rs, int cs,
+                                        hipStream_t stream, void* ws = nullptr, size_t ws_bytes = 0) {
+  detail::check(dgpp_launch_mma_gemv_fp8e8m0_f32(act, act_stride, w, scales, out, m, n, k, out_stride, rs, cs, stream, ws,
+                                                 ws_bytes));
+}
+inline void launch_moe_grouped_mma_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                        int max_rows, int rows_per_block, const MoeExpertView* views, int which,
+                                        uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream,
+                                        const int32_t* act_rows = nullptr) {
+  detail::check(dgpp_launch_moe_grouped_mma_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
+                                                 out_stride, n, k, stream, act_rows));
+}
+inline void launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                       int max_rows, int rows_per_block, const MoeExpertView* views, int which, float* out,
+                                       size_t out_stride, int n, int k, hipStream_t stream,
+                                       const int32_t* act_rows = nullptr) {
+  detail::check(dgpp_launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
+                                                out_stride, n, k, stream, act_rows));
+}
+inline void launch_moe_grouped_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                            int max_rows, int rows_per_block, const MoeExpertView* views, int which,
+                                            uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream,
+                                            const int32_t* act_rows = nullptr, int fp4_group = kFp4Group,
+                                            int tile_rows = 64) {
+  detail::check(dgpp_launch_moe_grouped_mma_fp4_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which,
+                                                     out, out_stride, n, k, stream, act_rows, fp4_group, tile_rows));
+}
+inline void launch_moe_grouped_mma_fp4_f32(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                           int max_rows, int rows_per_block, const MoeExpertView* views, int which,
+                                           float* out, size_t out_stride, int n, int k, hipStream_t stream,
+                                           const int32_t* act_rows = nullptr, int fp4_group = kFp4Group,
+                                           int tile_rows = 64) {
+  detail::check(dgpp_launch_moe_grouped_mma_fp4_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which,
+                                                    out, out_stride, n, k, stream, act_rows, fp4_group, tile_rows));
+}
 
 // ---- src/kernels/scale_gemm.hpp ---------------------------------------------------------------------------
 inline void launch_scale_gemm_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,

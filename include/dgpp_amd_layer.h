@@ -64,6 +64,11 @@ int dgpp_moe_layer_enqueue_decode_routed(DgppMoeLayer* layer, const uint16_t* x,
 int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride,
                                           const int32_t* ids, const float* weights, uint16_t* out_bf16,
                                           float* out_f32, int tokens, void* stream);
+/* The grouped path through the matrix-core launchers (the reference's prefill form,
+ * src/models/glm/moe_layer.cpp:775-817): gather folded into the gate / up launches. */
+int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                          const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
+                                          void* stream);
 /* Device pointers of the last routes the layer computed: ids int32 [tokens, top_k], weights f32. */
 const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* layer); /* the device expert table */
 const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* layer);

@@ -1,0 +1,156 @@
+"""The matrix-core launchers (dense, scale-grid and grouped forms) against the CPU oracle, and the
+properties the reference pins for its tensor-core kernels (tests/cuda/glm_moe_test.cu grouped-vs-dense
+per segment, tests/cuda/scale_gemm_test.cu:255-330 rows bitwise the rows alone): a (weight row,
+activation row) result does not depend on how many rows ride in the launch, on the launcher, or on the
+split form. Budget: the strict single-GEMV comparator of test_gpu_dense_gemv.check.
+"""
+import numpy as np
+import pytest
+
+import moe_data
+import oracle_lib as orc
+from dgpp_amd import _lib, hostgen as hg, launch as L
+from gpu_util import DeviceMoe, dev, dev_empty, fp4_matrix, host, sync
+from test_gpu_dense_gemv import check, make_fp4
+
+pytestmark = pytest.mark.gpu
+
+FP4_SHAPES = [(1, 520, 4096), (5, 200, 1024), (16, 100, 2048), (37, 130, 5120), (8, 64, 160), (3, 33, 576),
+              (20, 77, 6144), (2, 16, 32)]
+
+
+@pytest.mark.parametrize("group", [16, 32])
+@pytest.mark.parametrize("m,n,k", FP4_SHAPES)
+def test_dense_mma_fp4_matches_oracle_and_rows_are_independent(gpu, group, m, n, k):
+    act, payload, scales, glob = make_fp4(m, n, k, 0x3A0 + n + k + group, group)
+    raw = orc.gemv_fp4(act, payload, scales, float(glob[0]) if glob is not None else 1.0, group, m, n, k)
+    act_d, p_d, s_d = dev(act), dev(payload), dev(scales)
+    g_d = dev(glob) if glob is not None else None
+    w = fp4_matrix(p_d, s_d, g_d, n, k, group)
+    out, outf, one = dev_empty((m, n), np.uint16), dev_empty((m, n), np.float32), dev_empty((1, n), np.uint16)
+    L.launch_dense_mma_fp4_bf16(act_d, k, w, out, m, n, k, None)
+    L.launch_dense_mma_fp4_f32(act_d, k, w, outf, m, n, k, None)
+    last = act_d[m - 1:m].contiguous()
+    L.launch_dense_mma_fp4_bf16(last, k, w, one, 1, n, k, None)
+    sync()
+    got = host(out, np.uint16)
+    check(got, raw, f"dense mma fp4 g{group} {m}x{n}x{k}")
+    assert np.array_equal(hg.f32_to_bf16(host(outf)), got), "bf16(out_f32) == out_bf16"
+    assert np.array_equal(host(one, np.uint16)[0], got[m - 1]), "a row's bits do not depend on the rows beside it"
+
+
+@pytest.mark.parametrize("e8m0,rs,cs", [(False, 7, 7), (False, 5, 6), (False, 0, 12), (True, 0, 5)])
+@pytest.mark.parametrize("m,n,k", [(1, 300, 4096), (9, 130, 2048), (33, 96, 1024), (16, 50, 304), (64, 128, 6144)])
+def test_mma_gemv_fp8_matches_oracle_split_and_unsplit(gpu, e8m0, rs, cs, m, n, k):
+    if e8m0 and k % 32:
+        k -= k % 32                      # the 1 x 32 grid needs whole blocks
+    rng = np.random.default_rng(n + k + rs)
+    w = hg.f32_to_bf16(hg.normal_f32(0x8A0 + n + k, (n, k), 0.02))
+    act = hg.normal_bf16(0x8A1 + n, (m, k))
+    if e8m0:
+        payload, scales = hg.encode_mxfp8(hg.bf16_to_f32(w))
+    else:
+        payload, _ = hg.encode_fp8_blocks(w, 128, 128)
+        br, bc = 1 << rs, 1 << cs
+        scales = rng.uniform(0.5, 2.0, ((n + br - 1) // br, (k + bc - 1) // bc)).astype(np.float32) * 1e-3
+    raw = orc.gemv_fp8(act, payload, scales, m, n, k, rs, cs, True, e8m0)
+    a_d, p_d, s_d = dev(act), dev(payload), dev(scales)
+    fn_b = L.launch_mma_gemv_fp8e8m0_bf16 if e8m0 else L.launch_mma_gemv_fp8_bf16
+    fn_f = L.launch_mma_gemv_fp8e8m0_f32 if e8m0 else L.launch_mma_gemv_fp8_f32
+    stride = n + 8
+    out, outf, outs = dev_empty((m, stride), np.uint16), dev_empty((m, n), np.float32), dev_empty((m, n), np.uint16)
+    out.zero_()
+    ws = dev_empty(4 * m * n, np.float32)
+    fn_b(a_d, k, p_d, s_d, out, m, n, k, stride, rs, cs, None)
+    fn_f(a_d, k, p_d, s_d, outf, m, n, k, 0, rs, cs, None)
+    fn_b(a_d, k, p_d, s_d, outs, m, n, k, 0, rs, cs, None, ws, 4 * m * n * 4)
+    sync()
+    got = host(out, np.uint16)
+    assert not got[:, n:].any(), "columns past n are left alone"
+    got = np.ascontiguousarray(got[:, :n])
+    check(got, raw, f"mma gemv fp8 e8m0={e8m0} {m}x{n}x{k} rs{rs} cs{cs}")
+    assert np.array_equal(hg.f32_to_bf16(host(outf)), got)
+    assert np.array_equal(host(outs, np.uint16), got), "the split form's bits are the unsplit form's"
+    if not e8m0 and rs == 7 and cs == 7:
+        outd = dev_empty((m, n), np.uint16)
+        L.launch_dense_mma_bf16(a_d, k, p_d, s_d, outd, m, n, k, None)
+        sync()
+        assert np.array_equal(host(outd, np.uint16), got)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "nvfp4", "mxfp4"])
+def test_grouped_mma_is_bitwise_the_dense_mma_per_segment_with_and_without_the_gather(gpu, kind):
+    E, H, I, K, T = 6, 512, 160 if kind != "fp8" else 144, 3, 23          # segments of up to 23 rows: two tiles
+    p = moe_data.make_problem(E, H, I, K, T, kind, 41, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    ids_d = dev(ids)
+    rows_d, sr_d, segs_d = dev_empty(T * K + T, np.int32), dev_empty(T * K, np.int32), dev_empty((E + 1, 3), np.int32)
+    L.launch_moe_segment(ids_d, T, K, E, rows_d, sr_d, segs_d, None)
+    xg = dev_empty((T * K, H), np.uint16)
+    L.launch_moe_gather_rows(d.x, rows_d, xg, T * K, H, None)
+    g1, g2, g3 = (dev_empty((T * K, I), np.uint16) for _ in range(3))
+    gf = dev_empty((T * K, I), np.float32)
+    if kind == "fp8":
+        L.launch_moe_grouped_mma_bf16(xg, H, segs_d, E, T, 0, d.views, 0, g1, I, I, H, None)
+        L.launch_moe_grouped_mma_bf16(d.x, H, segs_d, E, T, 0, d.views, 0, g2, I, I, H, None, rows_d)
+        L.launch_moe_grouped_mma_bf16(xg, H, segs_d, E, T, 16, d.views, 0, g3, I, I, H, None)
+        L.launch_moe_grouped_mma_f32(xg, H, segs_d, E, T, 0, d.views, 0, gf, I, I, H, None)
+    else:
+        L.launch_moe_grouped_mma_fp4_bf16(xg, H, segs_d, E, T, 0, d.views, 0, g1, I, I, H, None, None, d.fp4_group)
+        L.launch_moe_grouped_mma_fp4_bf16(d.x, H, segs_d, E, T, 0, d.views, 0, g2, I, I, H, None, rows_d, d.fp4_group)
+        L.launch_moe_grouped_mma_fp4_bf16(xg, H, segs_d, E, T, 16, d.views, 0, g3, I, I, H, None, None, d.fp4_group)
+        L.launch_moe_grouped_mma_fp4_f32(xg, H, segs_d, E, T, 0, d.views, 0, gf, I, I, H, None, None, d.fp4_group)
+    sync()
+    a = host(g1, np.uint16)
+    assert np.array_equal(a, host(g2, np.uint16)), "the folded gather reads the gathered buffer's values"
+    assert np.array_equal(a, host(g3, np.uint16)), "the z split does not change a row"
+    assert np.array_equal(hg.f32_to_bf16(host(gf)), a)
+    segs, rows = host(segs_d).reshape(-1, 3), host(rows_d)
+    xh = host(xg, np.uint16)
+    for e in range(E):
+        r0, cnt, _ = (int(v) for v in segs[e])
+        if cnt == 0:
+            continue
+        m = p.experts[e][0]
+        xs = dev(xh[r0:r0 + cnt])
+        one = dev_empty((cnt, I), np.uint16)
+        if kind == "fp8":
+            L.launch_dense_mma_bf16(xs, H, dev(m.payload), dev(m.scales), one, cnt, I, H, None)
+            raw = orc.gemv_fp8(xh[r0:r0 + cnt], m.payload, m.scales, cnt, I, H, 7, 7, True)
+        else:
+            wm = fp4_matrix(dev(m.payload), dev(m.scales), dev(m.glob) if m.glob is not None else None, I, H, d.fp4_group)
+            L.launch_dense_mma_fp4_bf16(xs, H, wm, one, cnt, I, H, None)
+            raw = orc.gemv_fp4(xh[r0:r0 + cnt], m.payload, m.scales, float(m.glob[0]) if m.glob is not None else 1.0,
+                               d.fp4_group, cnt, I, H)
+        sync()
+        assert np.array_equal(host(one, np.uint16), a[r0:r0 + cnt]), f"segment {e}: grouped == dense, bitwise"
+        check(np.ascontiguousarray(a[r0:r0 + cnt]), raw, f"grouped mma {kind} segment {e}")
+
+
+@pytest.mark.parametrize("kind", ["fp8", "nvfp4", "mxfp4"])
+def test_prefill_path_matches_oracle_and_gemv_launchers_on_the_matrix_core_are_its_twins(gpu, kind):
+    """The layer's matrix-core grouped path against the oracle's layer budget; then, with the bench switch that
+    moves the GEMV launchers onto the matrix core, the decode-slot kernels give the same bits as that path."""
+    from dgpp_amd import moe_layer as ML
+    from test_gpu_moe_layer import make_layer
+    from test_gpu_moe_slots import expert_budget, run_slot_path
+    E, H, I, K, T = 10, 2048, 256, 4, 21
+    p = moe_data.make_problem(E, H, I, K, T, kind, 58, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    layer = make_layer(p, d, 1, 1.0, T)
+    out = dev_empty((T, H), np.uint16)
+    layer.enqueue_prefill_routed(d.x, H, dev(ids), dev(w), out, T)
+    sync()
+    got = host(out, np.uint16)
+    raw, _ = moe_data.orc_forward(p, ids, w)
+    expert_budget(got, raw, f"prefill {kind}")
+    lib = _lib.load()
+    lib.dgpp_tune_set(5, 2)
+    try:
+        _, _, out_slots = run_slot_path(p, d, ids, w)
+    finally:
+        lib.dgpp_tune_set(5, 0)
+    assert np.array_equal(out_slots, got), "slot kernels on the matrix core == grouped matrix-core path, bitwise"
+    layer.close()

@@ -248,45 +248,3 @@ def test_slot_launcher_argument_errors(gpu):
     with pytest.raises(L.InvalidArgument):   # fp8: k not a multiple of 16
         L.launch_moe_slot_gate_up_swiglu(*args, 64, 250, 0, 0, None, None, None, None, act, 64, 3, 2, 10.0, None)
     L.launch_moe_slot_gate_up_swiglu_fp4(*args, 64, 256, 0, 0, None, None, None, None, act, 64, 0, 2, 10.0, None, -1, 16)  # slots <= 0
-
-
-@pytest.mark.parametrize("kind,E,H,I,K,T", [("fp8", 12, 384, 96, 3, 7), ("nvfp4", 16, 1024, 256, 8, 2),
-                                            ("mxfp4", 6, 1024, 256, 4, 8), ("mxfp4", 32, 1024, 256, 8, 1)])
-def test_fused_down_accumulate_is_bitwise_the_two_launch_form(gpu, kind, E, H, I, K, T):
-    """The extension launcher (down rows + the token's ordered chain in one launch) against
-    launch_moe_slot_down* followed by launch_moe_slot_accum_routed_f32 / round: same bits, counters left zero,
-    a second call on the same counters gives the same bits again."""
-    p = moe_data.make_problem(E, H, I, K, T, kind, 900 + E + T, shared_kind=None, limit=float("inf"), std=0.05)
-    d = DeviceMoe(p)
-    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
-    act, down, out = run_slot_path(p, d, ids, w)
-    slots = T * (K + 1)
-    ids_d, w_d, act_d = dev(ids), dev(w), dev(act)
-    order_d = None
-    if T > 1:
-        order_d = dev_empty(slots, np.int32)
-        L.launch_moe_slot_order(ids_d, order_d, slots, K, E, None, False)
-    n_arrive = T * ((H + 3) // 4)
-    arrive = dev(np.zeros(n_arrive, np.int32))
-    for rep in range(2):
-        down_d = dev_empty((slots, H), np.float32)
-        down_d.zero_()
-        out_b, out_f = dev_empty((T, H), np.uint16), dev_empty((T, H), np.float32)
-        if kind == "fp8":
-            L.launch_moe_slot_down_accum(act_d, I, ids_d, order_d, d.views, H, I, down_d, H, slots, K, w_d, out_b, None,
-                                         arrive, n_arrive, None)
-            L.launch_moe_slot_down_accum(act_d, I, ids_d, order_d, d.views, H, I, down_d, H, slots, K, w_d, None, out_f,
-                                         arrive, n_arrive, None)
-        else:
-            L.launch_moe_slot_down_accum_fp4(act_d, I, ids_d, order_d, d.views, H, I, down_d, H, slots, K, w_d, out_b,
-                                             None, arrive, n_arrive, None, d.fp4_group)
-            L.launch_moe_slot_down_accum_fp4(act_d, I, ids_d, order_d, d.views, H, I, down_d, H, slots, K, w_d, None,
-                                             out_f, arrive, n_arrive, None, d.fp4_group)
-        sync()
-        assert np.array_equal(host(down_d), down), "down rows"
-        assert np.array_equal(host(out_b, np.uint16), out), f"fused bf16 output (call {rep})"
-        assert np.array_equal(hg.f32_to_bf16(host(out_f)), out), f"fused f32 output (call {rep})"
-        assert not host(arrive).any(), "arrival counters are zero at rest"
-    with pytest.raises(L.InvalidArgument):   # counters too small
-        L.launch_moe_slot_down_accum_fp4(act_d, I, ids_d, order_d, d.views, H, 256 if kind == "fp8" else I, down_d, H,
-                                         slots, K, w_d, out_b, None, arrive, n_arrive - 1, None, 32)
