@@ -3,10 +3,10 @@
 // ALU, so the per-weight vector work is the decode alone and up to 16 activation rows ride on one
 // pass over the weights.
 //
-// Shape. A wavefront owns a ROW GROUP of 16 weight rows. Lane (r = lane % 16, q = lane / 16) loads
-// 16 bytes of row r per STEP at byte offset step * 64 + q * 16: one load instruction reads 64
-// contiguous bytes of each of the 16 rows (128 FP4 or 64 FP8 elements per row and step). The lane
-// decodes its 16 bytes to bf16 in registers (hardware FP4 / FP8 conversions, block scale folded
+// Shape. A wavefront owns a ROW GROUP of 16 weight rows. Per STEP one load instruction reads 64
+// contiguous bytes of each of the 16 rows (128 FP4 or 64 FP8 elements per row and step), 16 bytes
+// per lane; after a lane permute lane (r = lane % 16, q = lane / 16) holds bytes q * 16 .. + 15 of
+// row r's 64. The lane decodes its 16 bytes to bf16 in registers (hardware FP4 / FP8 conversions, block scale folded
 // in) and feeds them, 8 elements at a time, as the A operand; the B operand is the matching 8
 // activations of activation row (lane % 16), read as one 16-byte vector from an LDS stage laid
 // out [8-element block][activation row]. D[weight row][activation row] accumulates in fp32: lane
@@ -118,19 +118,24 @@ __device__ __forceinline__ f32x4_t mfma_bf16(const Frag& a, const uint4& b, f32x
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
 }
 
-// Per-lane addressing of a row group: lane (r, q) of the group starting at row0.
+// Per-lane LOAD addressing of a row group starting at row0. Loads are issued row-major — lane l reads
+// piece l % 4 of row l / 4, so a quarter wavefront touches 4 rows x 64 contiguous bytes instead of 16
+// rows x 16 bytes — and a lane permute (to_operand_layout) then hands lane (r, q) = r + 16 q the 16
+// bytes of row r, piece q that the matrix core expects from it.
 struct GroupLane {
   const uint8_t* payload_row;
   const void* scale_row;
-  int q;
+  int q;          // the piece this lane LOADS
+  int from;       // byte address (lane * 4) of the lane whose load this lane consumes
 };
 template <int FMT>
 __device__ __forceinline__ GroupLane group_lane(const MatRef& mat, int row0, int n, int k) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int row = row0 + (lane & 15);
+  const int row = row0 + (lane >> 2);
   const int r = row < n ? row : n - 1;   // rows past the end redo the last row; their results are dropped
   GroupLane gl;
-  gl.q = lane >> 4;
+  gl.q = lane & 3;
+  gl.from = (4 * (lane & 15) + (lane >> 4)) * 4;
   if constexpr (FMT == kFmtFp8F32 || FMT == kFmtFp8E8M0) {
     gl.payload_row = mat.payload + static_cast<size_t>(r) * k;
     const size_t scale_cols = (static_cast<size_t>(k) + (1u << mat.cs) - 1) >> mat.cs;
@@ -156,6 +161,14 @@ __device__ __forceinline__ void load_step(const GroupLane& gl, int step, int chu
   }
 }
 
+__device__ __forceinline__ void to_operand_layout(const GroupLane& gl, ChunkRegs& r) {
+  r.w.x = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.w.x)));
+  r.w.y = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.w.y)));
+  r.w.z = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.w.z)));
+  r.w.w = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.w.w)));
+  r.s = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.s)));
+}
+
 // One 8-element block of an activation row as a 16-byte vector; zeros past k.
 __device__ __forceinline__ uint4 load_act_block(const uint16_t* __restrict__ row, int k0, int k, bool aligned) {
   if (k0 >= k) return make_uint4(0u, 0u, 0u, 0u);
@@ -171,12 +184,13 @@ __device__ __forceinline__ uint4 load_act_block(const uint16_t* __restrict__ row
 // Only the first `valid` steps of the chunk exist (the rest hold zeros and their stage units may
 // never have been written, so they must not reach the matrix core).
 template <int FMT, int NB>
-__device__ __forceinline__ void mfma_chunk(const ChunkRegs (&regs)[NB], const uint4* __restrict__ lane_stage, int m,
-                                           int valid, f32x4_t& acc) {
+__device__ __forceinline__ void mfma_chunk(const GroupLane& gl, ChunkRegs (&regs)[NB], const uint4* __restrict__ lane_stage,
+                                           int m, int valid, f32x4_t& acc) {
   constexpr int kSub = MTraits<FMT>::kSub;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     if (i < valid) {
+      to_operand_layout(gl, regs[i]);
       Frag f[kSub];
       decode_frags<FMT>(regs[i], f);
 #pragma unroll
@@ -186,13 +200,15 @@ __device__ __forceinline__ void mfma_chunk(const ChunkRegs (&regs)[NB], const ui
   }
 }
 template <int FMT, int NB>
-__device__ __forceinline__ void mfma_chunk_pair(const ChunkRegs (&ra)[NB], const ChunkRegs (&rb)[NB],
+__device__ __forceinline__ void mfma_chunk_pair(const GroupLane& gl, ChunkRegs (&ra)[NB], ChunkRegs (&rb)[NB],
                                                 const uint4* __restrict__ lane_stage, int m, int valid,
                                                 f32x4_t& acc_a, f32x4_t& acc_b) {
   constexpr int kSub = MTraits<FMT>::kSub;
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
     if (i < valid) {
+      to_operand_layout(gl, ra[i]);
+      to_operand_layout(gl, rb[i]);
       Frag fa[kSub], fb[kSub];
       decode_frags<FMT>(ra[i], fa);
       decode_frags<FMT>(rb[i], fb);

@@ -75,14 +75,14 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
       for (int ls = 0; ls < spp; ++ls, ++s) {
         const bool more = s + 1 < total;
         if (more) fetch(s + 1);
-        const uint4* lane_stage = lds + (s & 1) * kStageUnits + (gl.q * kSub) * mt + cc;
+        const uint4* lane_stage = lds + (s & 1) * kStageUnits + ((lane >> 4) * kSub) * mt + cc;
         const int step0 = p * g.part_steps + ls * stage_steps;
         const int nsteps = min(stage_steps, g.part_steps - ls * stage_steps);
         for (int t = 0; t < nsteps; t += NB) {
           ChunkRegs regs[NB];
 #pragma unroll
           for (int i = 0; i < NB; ++i) load_step<FMT>(gl, t + i < nsteps ? step0 + t + i : g.steps, chunks, mat.cs, regs[i]);
-          mfma_chunk<FMT, NB>(regs, lane_stage + (t * kStepBlocks) * mt, mt, min(NB, nsteps - t), acc[p]);
+          mfma_chunk<FMT, NB>(gl, regs, lane_stage + (t * kStepBlocks) * mt, mt, min(NB, nsteps - t), acc[p]);
         }
         if (more) put((s + 1) & 1);
         __syncthreads();
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void slot_gate_up_mfma_kernel(Slo
   const GroupLane lg = group_lane<FMT>(mg, row0, a.n, a.k);
   const GroupLane lu = group_lane<FMT>(mu, row0, a.n, a.k);
   const int cc = min(lane & 15, m - 1);
-  const uint4* lane_stage = stage + (lg.q * kSub) * m + cc;
+  const uint4* lane_stage = stage + ((lane >> 4) * kSub) * m + cc;
   const int step0 = part * g.part_steps;
   const int nsteps = min(g.part_steps, g.steps - step0);
   f32x4_t ag = {0.f, 0.f, 0.f, 0.f}, au = {0.f, 0.f, 0.f, 0.f};
@@ -258,7 +258,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void slot_gate_up_mfma_kernel(Slo
       load_step<FMT>(lg, st, chunks, mg.cs, rg[i]);
       load_step<FMT>(lu, st, chunks, mu.cs, ru[i]);
     }
-    mfma_chunk_pair<FMT, NB>(rg, ru, lane_stage + (t * kStepBlocks) * m, m, min(NB, nsteps - t), ag, au);
+    mfma_chunk_pair<FMT, NB>(lg, rg, ru, lane_stage + (t * kStepBlocks) * m, m, min(NB, nsteps - t), ag, au);
   }
   if (g.parts > 1) {
     if (part != 0) {
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void slot_down_mfma_kernel(SlotAr
   const int chunks = a.k / MTraits<FMT>::kLoadElems;
   const GroupLane ld = group_lane<FMT>(md, row0, a.n, a.k);
   const int cc = min(lane & 15, m - 1);
-  const uint4* lane_stage = stage + (ld.q * kSub) * m + cc;
+  const uint4* lane_stage = stage + ((lane >> 4) * kSub) * m + cc;
   const int step0 = part * g.part_steps;
   const int nsteps = min(g.part_steps, g.steps - step0);
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void slot_down_mfma_kernel(SlotAr
     ChunkRegs regs[NB];
 #pragma unroll
     for (int i = 0; i < NB; ++i) load_step<FMT>(ld, t + i < nsteps ? step0 + t + i : g.steps, chunks, md.cs, regs[i]);
-    mfma_chunk<FMT, NB>(regs, lane_stage + (t * kStepBlocks) * m, m, min(NB, nsteps - t), acc);
+    mfma_chunk<FMT, NB>(ld, regs, lane_stage + (t * kStepBlocks) * m, m, min(NB, nsteps - t), acc);
   }
   if (g.parts > 1) {
     if (part != 0) red[wave * kWave + lane] = acc;
