@@ -52,8 +52,8 @@ def parse():
     ap.add_argument("--eager", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
-    ap.add_argument("--configs", default="c1,c2", help="other BASELINE configurations to time beside the headline, "
-                    "comma separated out of c1,c2,c4,c5 ('' for none; c4 and c5 take a minute of set-up each)")
+    ap.add_argument("--configs", default="c1,c2,c4,c5", help="other BASELINE configurations to time beside the headline, "
+                    "comma separated out of c1,c2,c4,c5 ('' for none)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -283,6 +283,13 @@ def main():
             sec = time_graph(step_mma, args.steps, args.warmup)
             res[f"batch{m}_matrix_core"] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9,
                                             "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+            ws = torch.empty(4 * m * n, dtype=torch.float32, device=dev)
+            def step_split(i):
+                r = i % len(ring)
+                L.launch_mma_gemv_fp4_bf16(act, k, mats[r], out[r], m, n, k, 0, stream, ws, ws.numel() * 4)
+            sec = time_graph(step_split, args.steps, args.warmup)
+            res[f"batch{m}_matrix_core_split_k"] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9,
+                                                    "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
         res["workload"] = "C2 dense NVFP4 GEMV 17408x5120 (gate_up shape), batch 1 and 8 (one weight pass)"
         return res
 

@@ -92,10 +92,14 @@ SIGNATURES = {
     "dgpp_launch_moe_slot_down": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_launch_moe_slot_gate_up_swiglu_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I, _I, _I]),
     "dgpp_launch_moe_slot_down_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _P]),
+    "dgpp_launch_moe_slot_down_accum": (_I, [_P, _Z, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P]),
+    "dgpp_launch_moe_slot_down_accum_fp4": (_I, [_P, _Z, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I]),
     "dgpp_launch_dense_mma_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _Z]),
     "dgpp_launch_dense_mma_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _Z]),
     "dgpp_launch_dense_mma_fp4_bf16": (_I, [_P, _Z, _P, _P, _I, _I, _I, _P]),
     "dgpp_launch_dense_mma_fp4_f32": (_I, [_P, _Z, _P, _P, _I, _I, _I, _P]),
+    "dgpp_launch_mma_gemv_fp4_bf16": (_I, [_P, _Z, _P, _P, _I, _I, _I, _Z, _P, _P, _Z]),
+    "dgpp_launch_mma_gemv_fp4_f32": (_I, [_P, _Z, _P, _P, _I, _I, _I, _Z, _P, _P, _Z]),
     "dgpp_launch_mma_gemv_fp8_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
     "dgpp_launch_mma_gemv_fp8_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
     "dgpp_launch_mma_gemv_fp8e8m0_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),

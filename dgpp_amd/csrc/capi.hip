@@ -103,6 +103,13 @@ hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, 
     default: return launch_grouped_fmt<kFmtMxfp4>(a, n_segs, z_ext, s);
   }
 }
+hipError_t launch_token_down(int fmt, const TokenDownArgs& a, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_token_down_fmt<kFmtFp8F32>(a, s);
+    case kFmtNvfp4: return launch_token_down_fmt<kFmtNvfp4>(a, s);
+    default: return launch_token_down_fmt<kFmtMxfp4>(a, s);
+  }
+}
 hipError_t launch_dense_mma(int fmt, const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t s) {
   switch (fmt) {
     case kFmtFp8F32: return launch_dense_mma_fmt<kFmtFp8F32>(a, ws, ws_bytes, s);
@@ -595,6 +602,52 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
   return finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
 }
 
+// Routed down + ordered accumulation in one launch (no counterpart in the reference, which runs
+// launch_moe_slot_down* and launch_moe_slot_accum_routed_* back to back).
+static int slot_down_accum(int fmt, const uint16_t* act, size_t act_stride, const int32_t* ids,
+                           const DgppMoeExpertView* views, int n, int k, int tokens, int top_k, const float* weights,
+                           uint16_t* out_bf16, float* out_f32, void* stream, const char* who) {
+  if (tokens <= 0) return DGPP_OK;
+  if (!act || !ids || !views || !weights || (!out_bf16 && !out_f32)) return fail_arg(std::string(who) + ": null pointer");
+  if (n <= 0 || k <= 0 || top_k <= 0 || top_k > 16) return fail_arg(std::string(who) + ": degenerate dims (top_k 1..16)");
+  if (tokens > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
+  if (act_stride < static_cast<size_t>(k)) return fail_arg(std::string(who) + ": act_stride below k");
+  if (static_cast<size_t>(top_k) * (stage_bytes(1, k) + 8 * 64 * sizeof(float)) > kMaxLdsBytes)
+    return fail_arg(std::string(who) + ": top_k activation rows of k elements exceed the LDS budget");
+  TokenDownArgs a;
+  a.act = act;
+  a.act_stride = act_stride;
+  a.ids = ids;
+  a.views = views;
+  a.weights = weights;
+  a.out = out_f32 ? static_cast<void*>(out_f32) : static_cast<void*>(out_bf16);
+  a.out_f32 = out_f32 != nullptr;
+  a.n = n;
+  a.k = k;
+  a.tokens = tokens;
+  a.top_k = top_k;
+  return finish(launch_token_down(fmt, a, as_stream(stream)), who);
+}
+int dgpp_launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                    const DgppMoeExpertView* views, int n, int k, int tokens, int top_k,
+                                    const float* weights, uint16_t* out_bf16, float* out_f32, void* stream) {
+  const char* who = "moe_slot_down_accum";
+  if (tokens > 0 && (k % 16 != 0 || stage_bytes(1, k) > kMaxLdsBytes))
+    return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
+  return slot_down_accum(kFmtFp8F32, act, act_stride, ids, views, n, k, tokens, top_k, weights, out_bf16, out_f32, stream, who);
+}
+int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                        const DgppMoeExpertView* views, int n, int k, int tokens, int top_k,
+                                        const float* weights, uint16_t* out_bf16, float* out_f32, void* stream,
+                                        int fp4_group) {
+  const char* who = "moe_slot_down_accum_fp4";
+  if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
+  if (tokens > 0 && (!fp4_k_supported(k) || !fp4_k_compiled(k, fp4_group)))
+    return fail_arg(std::string(who) + ": k must be a multiple of 32 in the fp4 core's compiled set");
+  return slot_down_accum(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, ids, views, n, k, tokens, top_k, weights,
+                         out_bf16, out_f32, stream, who);
+}
+
 // ---- matrix-core launchers (src/kernels/glm_moe_launch.hpp:103-125, :311-345; src/kernels/mma_gemv.hpp:65-85) -----
 static int dense_mma(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,
                      int out_f32, size_t out_stride, int m, int n, int k, void* ws, size_t ws_bytes, void* stream,
@@ -661,7 +714,7 @@ int dgpp_launch_mma_gemv_fp8e8m0_f32(const uint16_t* act, size_t act_stride, con
 }
 
 static int dense_mma_fp4(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, void* out, int out_f32, int m,
-                         int n, int k, void* stream) {
+                         int n, int k, void* stream, size_t out_stride = 0, void* ws = nullptr, size_t ws_bytes = 0) {
   const char* who = "dense_mma_fp4";
   if (m <= 0 || n <= 0) return DGPP_OK;
   if (!w || !act || !w->payload || !w->scales || !out) return fail_arg(std::string(who) + ": null pointer");
@@ -678,7 +731,15 @@ static int dense_mma_fp4(const uint16_t* act, size_t act_stride, const DgppFp4Ma
   mat.rs = 0;
   mat.cs = 0;
   return dense_mma(w->scale_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, mat, w->global_scale, out, out_f32,
-                   static_cast<size_t>(n), m, n, k, nullptr, 0, stream, who);
+                   out_stride, m, n, k, ws, ws_bytes, stream, who);
+}
+int dgpp_launch_mma_gemv_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out, int m,
+                                  int n, int k, size_t out_stride, void* stream, void* ws, size_t ws_bytes) {
+  return dense_mma_fp4(act, act_stride, w, out, 0, m, n, k, stream, out_stride, ws, ws_bytes);
+}
+int dgpp_launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, float* out, int m, int n,
+                                 int k, size_t out_stride, void* stream, void* ws, size_t ws_bytes) {
+  return dense_mma_fp4(act, act_stride, w, out, 1, m, n, k, stream, out_stride, ws, ws_bytes);
 }
 int dgpp_launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out, int m,
                                    int n, int k, void* stream) {

@@ -120,6 +120,16 @@ __device__ __forceinline__ void stage_activations(const uint16_t* __restrict__ x
   }
 }
 
+// Vector v (8 bf16 values) of an activation row.
+__device__ __forceinline__ uint4 load_vec8(const uint16_t* __restrict__ x, int v, bool aligned) {
+  if (aligned) return *reinterpret_cast<const uint4*>(x + static_cast<size_t>(v) * 8);
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    w[i] = static_cast<uint32_t>(x[v * 8 + 2 * i]) | (static_cast<uint32_t>(x[v * 8 + 2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
 // ---- lane butterflies ---------------------------------------------------------------------
 template <int kCtrl>
 __device__ __forceinline__ float dpp_move(float v) {

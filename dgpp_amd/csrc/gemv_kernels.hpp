@@ -286,6 +286,71 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_ker
   }
 }
 
+// ---- decode: routed down projection + ordered accumulation, token-major ----------------------------------
+// One block per (row tile, token), one wavefront per routed slot of the token: wavefront j streams the tile's
+// rows of expert ids[t, j]'s down matrix against the slot's own activation row (the slot kernels' chain per
+// row, bit for bit), the top_k partial rows meet in LDS and the token's accumulation chain
+// (a = 0; a = fma(w_j, y_j, a), j ascending; one rounding) runs right there: no [slots, n] round trip
+// through memory and no second launch. Routed slots only (no shared expert in the chain).
+struct TokenDownArgs {
+  const uint16_t* act;      // [slots, act_stride] slot activation rows, slot = t * (top_k + 1) + j
+  size_t act_stride;
+  const int32_t* ids;       // [tokens, top_k]
+  const DgppMoeExpertView* views;
+  const float* weights;     // [tokens, top_k]
+  void* out;                // [tokens, n] bf16 bits or f32
+  int out_f32;
+  int n, k, tokens, top_k;
+};
+
+template <int FMT, int NB>
+__global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int t = static_cast<int>(blockIdx.y);
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  const int row_vecs = kPieces * chunks;
+  const int rpw = kWave >> g.l2;
+  const int rows_per_block = rpw * steps;
+  const int tile_row0 = static_cast<int>(blockIdx.x) * rows_per_block;
+  uint4* my_x = lds + wave * row_vecs;
+  float* part = reinterpret_cast<float*>(lds + a.top_k * row_vecs);   // [top_k][rows_per_block]
+  const float* gd = nullptr;
+  const MatRef md = mat_of_view<FMT>(a.views[a.ids[static_cast<size_t>(t) * a.top_k + wave] * 3 + 2], &gd);
+  {  // this wavefront's activation row, in the core's [piece][chunk] order
+    const uint16_t* x = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + wave) * a.act_stride;
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    for (int v = lane; v < row_vecs; v += kWave) {
+      const int c = v / kPieces, q = v - c * kPieces;
+      my_x[q * chunks + c] = load_vec8(x, v, aligned);
+    }
+  }
+  __syncthreads();
+  const float dd = load_divisor<FMT>(gd);
+  for (int s = 0; s < steps; ++s) {
+    const int row0 = tile_row0 + s * rpw;
+    if (row0 >= a.n) break;
+    const LaneRow lr = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
+    float acc[1];
+    row_dots<FMT, 1, NB>(lr, g, md.cs, my_x, chunks, 1, acc);
+    if (lr.li == 0) part[wave * rows_per_block + s * rpw + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
+  }
+  __syncthreads();
+  for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
+    const int row = tile_row0 + r;
+    if (row >= a.n) break;
+    float v = 0.f;
+    for (int j = 0; j < a.top_k; ++j)
+      v = fmaf(a.weights[static_cast<size_t>(t) * a.top_k + j], part[j * rows_per_block + r], v);
+    const size_t at = static_cast<size_t>(t) * a.n + row;
+    if (a.out_f32)
+      static_cast<float*>(a.out)[at] = v;
+    else
+      static_cast<uint16_t*>(a.out)[at] = f32_to_bf16(v);
+  }
+}
+
 // ---- grouped (segment-major) twin ------------------------------------------------------------------
 struct GroupedArgs {
   const uint16_t* act;
@@ -367,6 +432,10 @@ hipError_t launch_dense(int fmt, const DenseArgs& a, hipStream_t stream);
 hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t stream);
 hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t stream);
 hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
+
+// Token-major routed down + accumulation (vector core).
+hipError_t launch_token_down(int fmt, const TokenDownArgs& a, hipStream_t stream);
+template <int FMT> hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipStream_t stream);
 
 // The matrix-core launchers proper (the *_mma_* entry points).
 hipError_t launch_dense_mma(int fmt, const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t stream);
@@ -577,6 +646,27 @@ hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
                          steps);
   });
   return hipGetLastError();
+}
+
+template <int FMT>
+hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipStream_t stream) {
+  const RowGeom g = geom_for<FMT>(a.k);
+  const int rpw = kWave >> g.l2;
+  const long long wave_steps = static_cast<long long>((a.n + rpw - 1) / rpw) * a.tokens * a.top_k;
+  int steps = static_cast<int>(wave_steps / 16384);
+  steps = steps < 1 ? 1 : (steps > 8 ? 8 : steps);
+  if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
+  const int rows_per_block = rpw * steps;
+  const dim3 grid(static_cast<unsigned>((a.n + rows_per_block - 1) / rows_per_block), static_cast<unsigned>(a.tokens));
+  const size_t lds = static_cast<size_t>(a.top_k) * (stage_bytes(1, a.k) + static_cast<size_t>(rows_per_block) * sizeof(float));
+  hipError_t err = hipSuccess;
+  dispatch_nb(g.nb, [&](auto nbc) {
+    constexpr int NB = decltype(nbc)::value;
+    auto kern = token_down_accum_kernel<FMT, NB>;
+    err = ensure_lds(kern, lds);
+    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(a.top_k * kWave), lds, stream, a, g, steps);
+  });
+  return err != hipSuccess ? err : hipGetLastError();
 }
 
 template <int FMT>

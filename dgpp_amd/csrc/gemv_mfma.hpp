@@ -223,12 +223,4 @@ __device__ __forceinline__ void mfma_chunk_pair(const GroupLane& gl, ChunkRegs (
   }
 }
 
-// The parts' sums in ascending order (parts is 1, 2 or 4).
-__device__ __forceinline__ f32x4_t fold_parts(const f32x4_t (&acc)[kMaxParts], int parts) {
-  f32x4_t s = acc[0];
-  if (parts >= 2) s = s + acc[1];
-  if (parts >= 4) s = (s + acc[2]) + acc[3];
-  return s;
-}
-
 }  // namespace dgpp_amd

@@ -22,14 +22,15 @@ __host__ __device__ inline int stage_steps_for(int mt, int part_steps) {
 
 // 64 weight rows (one row group per wavefront) against mt <= 16 activation rows, all of K: the
 // block walks K in stages; a stage's activations sit in LDS as [8-element block][row], fetched one
-// stage ahead into registers. acc[p] receives part p's sum. Every thread of the block must call.
+// stage ahead into registers. `sum` receives the parts' sums added in ascending order. Every thread of
+// the block must call.
 // Parts [p_lo, p_hi) only (the others stay zero). `act_rows`, when given, names the activation
 // row of each of the mt rows (a gather folded into the stage load).
 template <int FMT, int NB>
 __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_t* __restrict__ act, size_t act_stride,
                                                 const int32_t* __restrict__ act_rows, int mt, int n, int k, int row0,
                                                 const MGeom& g, int p_lo, int p_hi, uint4* __restrict__ lds,
-                                                f32x4_t (&acc)[kMaxParts]) {
+                                                f32x4_t& sum) {
   constexpr int kSub = MTraits<FMT>::kSub;
   constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
   constexpr int kStepElems = MTraits<FMT>::kStepElems;
@@ -63,15 +64,14 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
       if (idx < units) lds[buf * kStageUnits + idx] = pre[i];
     }
   };
-#pragma unroll
-  for (int p = 0; p < kMaxParts; ++p) acc[p] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   fetch(0);
   put(0);
   __syncthreads();
   int s = 0;
-#pragma unroll
-  for (int p = 0; p < kMaxParts; ++p) {
-    if (p >= p_lo && p < p_hi) {
+  // Each part accumulates from zero and joins the running sum when it ends: ((p0 + p1) + p2) + p3.
+  for (int p = p_lo; p < p_hi; ++p) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    {
       for (int ls = 0; ls < spp; ++ls, ++s) {
         const bool more = s + 1 < total;
         if (more) fetch(s + 1);
@@ -82,12 +82,13 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
           ChunkRegs regs[NB];
 #pragma unroll
           for (int i = 0; i < NB; ++i) load_step<FMT>(gl, t + i < nsteps ? step0 + t + i : g.steps, chunks, mat.cs, regs[i]);
-          mfma_chunk<FMT, NB>(gl, regs, lane_stage + (t * kStepBlocks) * mt, mt, min(NB, nsteps - t), acc[p]);
+          mfma_chunk<FMT, NB>(gl, regs, lane_stage + (t * kStepBlocks) * mt, mt, min(NB, nsteps - t), acc);
         }
         if (more) put((s + 1) & 1);
         __syncthreads();
       }
     }
+    sum = p == p_lo ? acc : sum + acc;
   }
 }
 
@@ -122,21 +123,18 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs 
   const int c0 = static_cast<int>(blockIdx.y) * kTileCols;
   const int mt = min(kTileCols, a.m - c0);
   const int c = lane & 15;
-  f32x4_t acc[kMaxParts];
+  f32x4_t sum;
   if (partials == nullptr) {
     block_rows_mfma<FMT, NB>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k,
-                             row0, g, 0, g.parts, lds, acc);
-    store_tile<FMT>(fold_parts(acc, g.parts), load_divisor<FMT>(a.global), a.out, a.out_f32,
-                    static_cast<size_t>(c0 + c) * a.out_stride, row0, a.n, c < mt);
+                             row0, g, 0, g.parts, lds, sum);
+    store_tile<FMT>(sum, load_divisor<FMT>(a.global), a.out, a.out_f32, static_cast<size_t>(c0 + c) * a.out_stride, row0,
+                    a.n, c < mt);
     return;
   }
   const int part = static_cast<int>(blockIdx.z);
   block_rows_mfma<FMT, NB>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k, row0,
-                           g, part, part + 1, lds, acc);
-  f32x4_t mine = acc[0];
-#pragma unroll
-  for (int p = 1; p < kMaxParts; ++p) mine = part == p ? acc[p] : mine;
-  store_tile<kFmtMxfp4>(mine, 1.0f, partials, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
+                           g, part, part + 1, lds, sum);
+  store_tile<kFmtMxfp4>(sum, 1.0f, partials, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
 }
 
 // out[r][j] = finish(((p0 + p1) + p2) + p3) over partials[part][r][j].
@@ -173,11 +171,11 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
   const int c = lane & 15;
   for (int c0 = z0; c0 < z1; c0 += kTileCols) {
     const int mt = min(kTileCols, z1 - c0);
-    f32x4_t acc[kMaxParts];
+    f32x4_t sum;
     const size_t first = static_cast<size_t>(seg.row0 + c0);
     block_rows_mfma<FMT, NB>(mat, a.act_rows ? a.act : a.act + first * a.act_stride, a.act_stride,
-                             a.act_rows ? a.act_rows + first : nullptr, mt, a.n, a.k, row0, g, 0, g.parts, lds, acc);
-    store_tile<FMT>(fold_parts(acc, g.parts), divisor, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, c < mt);
+                             a.act_rows ? a.act_rows + first : nullptr, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum);
+    store_tile<FMT>(sum, divisor, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, c < mt);
   }
 }
 
@@ -185,7 +183,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
 // A block's four wavefronts are 4 / parts row groups times `parts` K parts. Each wavefront stages
 // ITS part of the run's activation rows ([block][row], m <= MAXM rows) in its own LDS region, streams
 // its 16 rows over that part, and the part sums meet in LDS, added in ascending part order by the
-// part-0 wavefront (fold_parts' order).
+// part-0 wavefront (the block form's order).
 template <int FMT>
 __host__ __device__ inline int slot_wave_units(int maxm, const MGeom& g) {
   return maxm * g.part_steps * MTraits<FMT>::kStepBlocks;

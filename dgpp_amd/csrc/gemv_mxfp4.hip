@@ -9,4 +9,5 @@ template hipError_t launch_slot_down_fmt<kFmtMxfp4>(const SlotArgs&, hipStream_t
 template hipError_t launch_grouped_fmt<kFmtMxfp4>(const GroupedArgs&, int, int, hipStream_t);
 template hipError_t launch_dense_mma_fmt<kFmtMxfp4>(const DenseArgs&, float*, size_t, hipStream_t);
 template hipError_t launch_grouped_mma_fmt<kFmtMxfp4>(const GroupedArgs&, int, int, hipStream_t);
+template hipError_t launch_token_down_fmt<kFmtMxfp4>(const TokenDownArgs&, hipStream_t);
 }  // namespace dgpp_amd

@@ -178,6 +178,11 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
                                    w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
                                    K, cfg_.swiglu_limit, stream, w_.sh_rs, w_.sh_cs);
+    if (!has_shared() && dgpp_tune_get(4) != 1) {   // routed only: down + accumulation in one token-major launch
+      launch_moe_slot_down_accum(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
+                                 out_bf16, out_f32, stream);
+      return;
+    }
     launch_moe_slot_down(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
                          n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, stream, w_.sh_rs, w_.sh_cs);
   } else {
@@ -187,6 +192,11 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
                                        sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
                                        d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, stream, base, fp4_group_,
                                        w_.sh_rs, w_.sh_cs);
+    if (!has_shared() && dgpp_tune_get(4) != 1) {
+      launch_moe_slot_down_accum_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
+                                     out_bf16, out_f32, stream, fp4_group_);
+      return;
+    }
     launch_moe_slot_down_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
                              has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
                              sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, stream, base, fp4_group_,

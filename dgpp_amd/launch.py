@@ -191,6 +191,20 @@ def launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_rou
         _p(tile_counter)))
 
 
+def launch_moe_slot_down_accum(act, act_stride, ids, views, n, k, tokens, top_k, weights, out_bf16, out_f32, stream=None):
+    """Extension: routed down rows + the ordered accumulation in one token-major launch (FP8 experts)."""
+    _check(_lib.load().dgpp_launch_moe_slot_down_accum(_p(act), act_stride, _p(ids), _p(views), n, k, tokens, top_k,
+                                                       _p(weights), _p(out_bf16), _p(out_f32), _stream(stream)))
+
+
+def launch_moe_slot_down_accum_fp4(act, act_stride, ids, views, n, k, tokens, top_k, weights, out_bf16, out_f32,
+                                   stream=None, fp4_group=16):
+    """Extension: routed down rows + the ordered accumulation in one token-major launch (NVFP4 / MXFP4 experts)."""
+    _check(_lib.load().dgpp_launch_moe_slot_down_accum_fp4(_p(act), act_stride, _p(ids), _p(views), n, k, tokens, top_k,
+                                                           _p(weights), _p(out_bf16), _p(out_f32), _stream(stream),
+                                                           fp4_group))
+
+
 # ---- grouped twins ---------------------------------------------------------------------------------------
 def launch_moe_grouped_gemv_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                  out_stride, n, k, stream=None):
@@ -372,3 +386,14 @@ def launch_moe_grouped_mma_fp4_f32(act, act_stride, segs, n_segs, max_rows, rows
     _check(_lib.load().dgpp_launch_moe_grouped_mma_fp4_f32(_p(act), act_stride, _p(segs), n_segs, max_rows, rows_per_block,
                                                            _p(views), which, _p(out), out_stride, n, k, _stream(stream),
                                                            _p(act_rows), fp4_group, tile_rows))
+
+
+def launch_mma_gemv_fp4_bf16(act, act_stride, w: Fp4Matrix, out, m, n, k, out_stride=0, stream=None, ws=None, ws_bytes=0):
+    """Extension: the FP4 dense matrix-core form with an output stride and a split-K workspace."""
+    _check(_lib.load().dgpp_launch_mma_gemv_fp4_bf16(_p(act), act_stride, C.addressof(w), _p(out), m, n, k, out_stride,
+                                                     _stream(stream), _p(ws), ws_bytes))
+
+
+def launch_mma_gemv_fp4_f32(act, act_stride, w: Fp4Matrix, out, m, n, k, out_stride=0, stream=None, ws=None, ws_bytes=0):
+    _check(_lib.load().dgpp_launch_mma_gemv_fp4_f32(_p(act), act_stride, C.addressof(w), _p(out), m, n, k, out_stride,
+                                                    _stream(stream), _p(ws), ws_bytes))

@@ -228,6 +228,20 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
                                   int* tile_counter);
 
 /* ---- grouped (segment-major) GEMV twins ------------------------------------------------------------ */
+/* Extension (no counterpart in the reference, which runs launch_moe_slot_down* and
+ * launch_moe_slot_accum_routed_* back to back): the routed slots' down projection AND the token's ordered
+ * accumulation chain in one launch, token-major (one wavefront per routed slot of a token, the top_k partial
+ * rows meet in LDS). act: the slot activation rows of launch_moe_slot_gate_up_swiglu* (slot = t * (top_k + 1)
+ * + j); out_f32 (when given) or out_bf16: [tokens, n]. Bit-identical to the two-launch form. Routed slots
+ * only: a shared expert is chained separately. */
+int dgpp_launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                    const DgppMoeExpertView* views, int n, int k, int tokens, int top_k,
+                                    const float* weights, uint16_t* out_bf16, float* out_f32, void* stream);
+int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                        const DgppMoeExpertView* views, int n, int k, int tokens, int top_k,
+                                        const float* weights, uint16_t* out_bf16, float* out_f32, void* stream,
+                                        int fp4_group);
+
 /* src/kernels/glm_moe_launch.hpp:77-87 */
 int dgpp_launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride,
                                       const DgppMoeSegment* segs, int n_segs, int max_rows,
@@ -269,6 +283,11 @@ int dgpp_launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const
                                    int n, int k, void* stream);
 int dgpp_launch_dense_mma_fp4_f32(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, float* out, int m, int n,
                                   int k, void* stream);
+/* Extension: the FP4 dense form with the scale-grid launchers' output stride and workspace arguments. */
+int dgpp_launch_mma_gemv_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out, int m,
+                                  int n, int k, size_t out_stride, void* stream, void* ws, size_t ws_bytes);
+int dgpp_launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, float* out, int m, int n,
+                                 int k, size_t out_stride, void* stream, void* ws, size_t ws_bytes);
 int dgpp_launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
                                   uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
                                   void* ws, size_t ws_bytes);

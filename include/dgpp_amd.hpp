@@ -223,6 +223,20 @@ inline void launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, con
                                               k_shared, sh_payload, sh_scales, out, out_stride, slots, top_k, stream,
                                               shared_view_base, fp4_group, sh_rs, sh_cs, tile_counter));
 }
+// Extensions: routed down rows + ordered accumulation in one token-major launch (see dgpp_amd.h).
+inline void launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                       const MoeExpertView* views, int n, int k, int tokens, int top_k,
+                                       const float* weights, uint16_t* out_bf16, float* out_f32, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_slot_down_accum(act, act_stride, ids, views, n, k, tokens, top_k, weights, out_bf16,
+                                                out_f32, stream));
+}
+inline void launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                           const MoeExpertView* views, int n, int k, int tokens, int top_k,
+                                           const float* weights, uint16_t* out_bf16, float* out_f32, hipStream_t stream,
+                                           int fp4_group = kFp4Group) {
+  detail::check(dgpp_launch_moe_slot_down_accum_fp4(act, act_stride, ids, views, n, k, tokens, top_k, weights, out_bf16,
+                                                    out_f32, stream, fp4_group));
+}
 inline void launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
                                          int max_rows, int rows_per_block, const MoeExpertView* views, int which,
                                          uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream) {
@@ -283,6 +297,15 @@ inline void launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, co
 inline void launch_dense_mma_fp4_f32(const uint16_t* act, size_t act_stride, const GlmFp4Matrix& w, float* out, int m, int n,
                                      int k, hipStream_t stream) {
   detail::check(dgpp_launch_dense_mma_fp4_f32(act, act_stride, &w, out, m, n, k, stream));
+}
+inline void launch_mma_gemv_fp4_bf16(const uint16_t* act, size_t act_stride, const GlmFp4Matrix& w, uint16_t* out, int m,
+                                     int n, int k, size_t out_stride, hipStream_t stream, void* ws = nullptr,
+                                     size_t ws_bytes = 0) {
+  detail::check(dgpp_launch_mma_gemv_fp4_bf16(act, act_stride, &w, out, m, n, k, out_stride, stream, ws, ws_bytes));
+}
+inline void launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const GlmFp4Matrix& w, float* out, int m, int n,
+                                    int k, size_t out_stride, hipStream_t stream, void* ws = nullptr, size_t ws_bytes = 0) {
+  detail::check(dgpp_launch_mma_gemv_fp4_f32(act, act_stride, &w, out, m, n, k, out_stride, stream, ws, ws_bytes));
 }
 inline void launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
                                      uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs,

@@ -32,8 +32,12 @@ def test_dense_mma_fp4_matches_oracle_and_rows_are_independent(gpu, group, m, n,
     L.launch_dense_mma_fp4_f32(act_d, k, w, outf, m, n, k, None)
     last = act_d[m - 1:m].contiguous()
     L.launch_dense_mma_fp4_bf16(last, k, w, one, 1, n, k, None)
+    outs = dev_empty((m, n + 8), np.uint16)
+    ws = dev_empty(4 * m * n, np.float32)
+    L.launch_mma_gemv_fp4_bf16(act_d, k, w, outs, m, n, k, n + 8, None, ws, 4 * m * n * 4)
     sync()
     got = host(out, np.uint16)
+    assert np.array_equal(host(outs, np.uint16)[:, :n], got), "the split form's bits are the unsplit form's"
     check(got, raw, f"dense mma fp4 g{group} {m}x{n}x{k}")
     assert np.array_equal(hg.f32_to_bf16(host(outf)), got), "bf16(out_f32) == out_bf16"
     assert np.array_equal(host(one, np.uint16)[0], got[m - 1]), "a row's bits do not depend on the rows beside it"

@@ -248,3 +248,28 @@ def test_slot_launcher_argument_errors(gpu):
     with pytest.raises(L.InvalidArgument):   # fp8: k not a multiple of 16
         L.launch_moe_slot_gate_up_swiglu(*args, 64, 250, 0, 0, None, None, None, None, act, 64, 3, 2, 10.0, None)
     L.launch_moe_slot_gate_up_swiglu_fp4(*args, 64, 256, 0, 0, None, None, None, None, act, 64, 0, 2, 10.0, None, -1, 16)  # slots <= 0
+
+
+@pytest.mark.parametrize("kind,E,H,I,K,T", [("fp8", 12, 384, 96, 3, 7), ("nvfp4", 16, 1024, 256, 8, 2),
+                                            ("mxfp4", 6, 1152, 256, 4, 8), ("mxfp4", 32, 1024, 1024, 8, 1),
+                                            ("nvfp4", 20, 640, 64, 16, 3)])
+def test_token_major_down_accumulate_is_bitwise_the_two_launch_form(gpu, kind, E, H, I, K, T):
+    """The extension launcher (routed down rows + the token's ordered chain in one token-major launch) against
+    launch_moe_slot_down* followed by launch_moe_slot_accum_routed_f32 / round: the same bits."""
+    p = moe_data.make_problem(E, H, I, K, T, kind, 900 + E + T, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    act, down, out = run_slot_path(p, d, ids, w)
+    ids_d, w_d, act_d = dev(ids), dev(w), dev(act)
+    out_b, out_f = dev_empty((T, H), np.uint16), dev_empty((T, H), np.float32)
+    if kind == "fp8":
+        L.launch_moe_slot_down_accum(act_d, I, ids_d, d.views, H, I, T, K, w_d, out_b, None, None)
+        L.launch_moe_slot_down_accum(act_d, I, ids_d, d.views, H, I, T, K, w_d, None, out_f, None)
+    else:
+        L.launch_moe_slot_down_accum_fp4(act_d, I, ids_d, d.views, H, I, T, K, w_d, out_b, None, None, d.fp4_group)
+        L.launch_moe_slot_down_accum_fp4(act_d, I, ids_d, d.views, H, I, T, K, w_d, None, out_f, None, d.fp4_group)
+    sync()
+    assert np.array_equal(host(out_b, np.uint16), out), "fused bf16 output"
+    assert np.array_equal(hg.f32_to_bf16(host(out_f)), out), "fused f32 output"
+    with pytest.raises(L.InvalidArgument):
+        L.launch_moe_slot_down_accum_fp4(act_d, I, ids_d, d.views, H, I, T, 17, w_d, out_b, None, None, 16)
