@@ -67,7 +67,7 @@ struct RowGeom {
 };
 // Bench A/B switches (host side, process-wide; 0 = the default behaviour). Set through
 // dgpp_tune_set; launchers read them when they pick a geometry or a kernel form.
-enum : int { kTunePreferP = 0, kTuneSlotRun = 1, kTuneSlotSteps = 2, kTuneCore = 5, kTuneCount = 8 };
+enum : int { kTunePreferP = 0, kTuneSlotRun = 1, kTuneSlotSteps = 2, kTuneSplitStage = 3, kTuneCore = 5, kTuneCount = 8 };
 int tune_get(int key);
 
 __host__ __device__ inline RowGeom row_geom(int chunks, int prefer_p = 4) {
@@ -360,6 +360,57 @@ __device__ __forceinline__ void row_dots(const LaneRow& lr, const RowGeom& g, in
     if (r < m) acc[r] = group_sum(acc[r], g.l2);
 }
 
+// row_dots with the first pass's loads already issued by the caller. Same chain.
+template <int FMT, int MAXR, int NB>
+__device__ __forceinline__ void row_dots_pre(const LaneRow& lr, const RowGeom& g, int cs,
+                                             const uint4* __restrict__ lds, int chunks, int m,
+                                             const ChunkRegs (&first)[NB], float (&acc)[MAXR]) {
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r) acc[r] = 0.f;
+  consume_pass<FMT, MAXR, NB>(first, lr, 0, g.l2, lds, chunks, m, acc);
+  const int passes = g.P / NB;
+  for (int p = 1; p < passes; ++p) {
+    ChunkRegs cur[NB];
+    issue_pass<FMT, NB>(lr, p, g.l2, cs, cur);
+    consume_pass<FMT, MAXR, NB>(cur, lr, p, g.l2, lds, chunks, m, acc);
+  }
+#pragma unroll
+  for (int r = 0; r < MAXR; ++r)
+    if (r < m) acc[r] = group_sum(acc[r], g.l2);
+}
+
+// Activation staging split in two so that weight loads can be issued in between: the activation loads
+// go out first (memory returns a wavefront's loads in order, so waiting for them does not wait for the
+// younger weight loads), are committed to LDS after the weights are on their way. One row of k <= 8 * XV
+// * threads elements, 16-byte aligned; vector v goes to [(piece) * chunks + chunk] of `dst`.
+template <int XV>
+struct StageRegs {
+  uint4 v[XV];
+};
+template <int FMT, int XV>
+__device__ __forceinline__ void stage_issue(const uint16_t* __restrict__ x, int k, int tid, int threads, StageRegs<XV>& r) {
+  const int vecs = k / 8;
+#pragma unroll
+  for (int i = 0; i < XV; ++i) {
+    const int v = tid + i * threads;
+    r.v[i] = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(v < vecs ? v : 0) * 8);   // always defined
+  }
+}
+template <int FMT, int XV>
+__device__ __forceinline__ void stage_commit(const StageRegs<XV>& r, int k, int tid, int threads, uint4* __restrict__ dst) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+  const int chunks = k / FmtTraits<FMT>::kElemsPerChunk;
+  const int vecs = k / 8;
+#pragma unroll
+  for (int i = 0; i < XV; ++i) {
+    const int v = tid + i * threads;
+    if (v < vecs) {
+      const int c = v / kPieces, q = v - c * kPieces;
+      dst[q * chunks + c] = r.v[i];
+    }
+  }
+}
+
 // One activation row already in registers: acc + dot(chunk, x).
 template <int FMT>
 __device__ __forceinline__ float chunk_dot1(const ChunkRegs& ch, const uint4* xv, float acc) {
@@ -374,11 +425,31 @@ __device__ __forceinline__ float chunk_dot1(const ChunkRegs& ch, const uint4* xv
 // activation rows: both rows' loads are issued together and each chunk column's activation vectors
 // are read from LDS once for the pair. Each (row, activation row) chain is row_dots' chain, bit for
 // bit.
+// One pass of a gate / up row pair against the m staged rows.
+template <int FMT, int NB, int MAXM>
+__device__ __forceinline__ void consume_pass_pair(const ChunkRegs (&ca)[NB], const ChunkRegs (&cb)[NB], int li, int p,
+                                                  int l2, const uint4* __restrict__ lds, int chunks, int m,
+                                                  float (&ra)[MAXM], float (&rb)[MAXM]) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int c = ((p * NB + i) << l2) + li;
+    if constexpr (MAXM == 1) {
+      uint4 xv[kPieces];
+#pragma unroll
+      for (int q = 0; q < kPieces; ++q) xv[q] = lds[q * chunks + c];
+      ra[0] = chunk_dot1<FMT>(ca[i], xv, ra[0]);
+      rb[0] = chunk_dot1<FMT>(cb[i], xv, rb[0]);
+    } else {
+      consume_chunk<FMT, MAXM>(ca[i], XLds<FMT>{lds + c, chunks}, m, ra);
+      consume_chunk<FMT, MAXM>(cb[i], XLds<FMT>{lds + c, chunks}, m, rb);
+    }
+  }
+}
 template <int FMT, int NB, int MAXM>
 __device__ __forceinline__ void row_dots_pair(const LaneRow& la, const LaneRow& lb, const RowGeom& g, int csa,
                                               int csb, const uint4* __restrict__ lds, int chunks, int m,
                                               float (&ra)[MAXM], float (&rb)[MAXM]) {
-  constexpr int kPieces = FmtTraits<FMT>::kPieces;
 #pragma unroll
   for (int r = 0; r < MAXM; ++r) ra[r] = rb[r] = 0.f;
   const int passes = g.P / NB;
@@ -386,20 +457,31 @@ __device__ __forceinline__ void row_dots_pair(const LaneRow& la, const LaneRow& 
     ChunkRegs ca[NB], cb[NB];
     issue_pass<FMT, NB>(la, p, g.l2, csa, ca);
     issue_pass<FMT, NB>(lb, p, g.l2, csb, cb);
+    consume_pass_pair<FMT, NB, MAXM>(ca, cb, la.li, p, g.l2, lds, chunks, m, ra, rb);
+  }
 #pragma unroll
-    for (int i = 0; i < NB; ++i) {
-      const int c = ((p * NB + i) << g.l2) + la.li;
-      if constexpr (MAXM == 1) {
-        uint4 xv[kPieces];
-#pragma unroll
-        for (int q = 0; q < kPieces; ++q) xv[q] = lds[q * chunks + c];
-        ra[0] = chunk_dot1<FMT>(ca[i], xv, ra[0]);
-        rb[0] = chunk_dot1<FMT>(cb[i], xv, rb[0]);
-      } else {
-        consume_chunk<FMT, MAXM>(ca[i], XLds<FMT>{lds + c, chunks}, m, ra);
-        consume_chunk<FMT, MAXM>(cb[i], XLds<FMT>{lds + c, chunks}, m, rb);
-      }
+  for (int r = 0; r < MAXM; ++r) {
+    if (r < m) {
+      ra[r] = group_sum(ra[r], g.l2);
+      rb[r] = group_sum(rb[r], g.l2);
     }
+  }
+}
+// The same with pass 0 of the two rows already issued by the caller (`fa`, `fb`). Same chain.
+template <int FMT, int NB, int MAXM>
+__device__ __forceinline__ void row_dots_pair_pre(const LaneRow& la, const LaneRow& lb, const RowGeom& g, int csa,
+                                                  int csb, const uint4* __restrict__ lds, int chunks, int m,
+                                                  const ChunkRegs (&fa)[NB], const ChunkRegs (&fb)[NB],
+                                                  float (&ra)[MAXM], float (&rb)[MAXM]) {
+#pragma unroll
+  for (int r = 0; r < MAXM; ++r) ra[r] = rb[r] = 0.f;
+  consume_pass_pair<FMT, NB, MAXM>(fa, fb, la.li, 0, g.l2, lds, chunks, m, ra, rb);
+  const int passes = g.P / NB;
+  for (int p = 1; p < passes; ++p) {
+    ChunkRegs ca[NB], cb[NB];
+    issue_pass<FMT, NB>(la, p, g.l2, csa, ca);
+    issue_pass<FMT, NB>(lb, p, g.l2, csb, cb);
+    consume_pass_pair<FMT, NB, MAXM>(ca, cb, la.li, p, g.l2, lds, chunks, m, ra, rb);
   }
 #pragma unroll
   for (int r = 0; r < MAXM; ++r) {

@@ -107,6 +107,9 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_ke
 // ---- MoE decode slots ----------------------------------------------------------------------------
 // Slot layout (src/kernels/glm_moe_launch.hpp:216-226): slot = t * (top_k + 1) + j, j < top_k the
 // token's j-th routed expert (ascending id), j == top_k the shared expert.
+// Activation vectors (16 bytes) a thread holds between the issue and the commit of a split stage.
+constexpr int kSplitStageVecs = 2;
+
 struct SlotArgs {
   const uint16_t* x;        // gate/up: token rows; down: slot activation rows
   size_t x_stride;
@@ -201,7 +204,7 @@ __device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& ru
   return true;
 }
 
-template <int FMT, int NB, int MAXM>
+template <int FMT, int NB, int MAXM, bool SPLIT>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   SlotRun<MAXM> run;
@@ -219,29 +222,60 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_
   }
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
   const int row_vecs = FmtTraits<FMT>::kPieces * chunks;
-#pragma unroll
-  for (int r = 0; r < MAXM; ++r)
-    if (r < run.m)
-      stage_activations<FMT>(a.x + static_cast<size_t>(run.token[r]) * a.x_stride, a.x_stride, 1, a.k, lds + r * row_vecs);
-  __syncthreads();
-  const float dg = load_divisor<FMT>(gg), du = load_divisor<FMT>(gu);
   const int rpw = kWave >> g.l2;
   const int wave = threadIdx.x >> 6;
-  uint16_t* act = static_cast<uint16_t*>(a.out);
   int row0 = blockIdx.x * rows_per_block + wave * rpw;
-  for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
-    if (row0 >= a.n) break;
-    const LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
-    const LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
-    float ag[MAXM], au[MAXM];
-    row_dots_pair<FMT, NB, MAXM>(lg, lu, g, mg.cs, mu.cs, lds, chunks, run.m, ag, au);
-    if (lg.li == 0 && lg.row < a.n) {
+  uint16_t* act = static_cast<uint16_t*>(a.out);
+  // Fast set-up (rows of at most 4096 aligned elements): activation loads, then the first step's weight
+  // loads, then the LDS commit and the barrier — the weights travel while the block sets up.
+  constexpr int XV = kSplitStageVecs;
+  LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
+  LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
+  ChunkRegs fg[NB], fu[NB];
+  if constexpr (SPLIT) {
+    StageRegs<XV> xr[MAXM];
+#pragma unroll
+    for (int r = 0; r < MAXM; ++r)   // every register set is loaded (unused run entries repeat row 0): no partial state
+      stage_issue<FMT, XV>(a.x + static_cast<size_t>(run.token[r]) * a.x_stride, a.k, threadIdx.x, kBlockThreads, xr[r]);
+    issue_pass<FMT, NB>(lg, 0, g.l2, mg.cs, fg);
+    issue_pass<FMT, NB>(lu, 0, g.l2, mu.cs, fu);
+#pragma unroll
+    for (int r = 0; r < MAXM; ++r)
+      if (r < run.m) stage_commit<FMT, XV>(xr[r], a.k, threadIdx.x, kBlockThreads, lds + r * row_vecs);
+  } else {
+#pragma unroll
+    for (int r = 0; r < MAXM; ++r)
+      if (r < run.m)
+        stage_activations<FMT>(a.x + static_cast<size_t>(run.token[r]) * a.x_stride, a.x_stride, 1, a.k, lds + r * row_vecs);
+  }
+  __syncthreads();
+  const float dg = load_divisor<FMT>(gg), du = load_divisor<FMT>(gu);
+  auto finish = [&](const LaneRow& l, const float (&ag)[MAXM], const float (&au)[MAXM]) {
+    if (l.li == 0 && l.row < a.n) {
 #pragma unroll
       for (int r = 0; r < MAXM; ++r)
         if (r < run.m)
-          act[static_cast<size_t>(run.slot[r]) * a.out_stride + lg.row] =
+          act[static_cast<size_t>(run.slot[r]) * a.out_stride + l.row] =
               swiglu_bf16(finish_dot<FMT>(ag[r], dg), finish_dot<FMT>(au[r], du), a.limit);
     }
+  };
+  int s = 0;
+  if constexpr (SPLIT) {
+    if (row0 < a.n) {
+      float ag[MAXM], au[MAXM];
+      row_dots_pair_pre<FMT, NB, MAXM>(lg, lu, g, mg.cs, mu.cs, lds, chunks, run.m, fg, fu, ag, au);
+      finish(lg, ag, au);
+    }
+    s = 1;
+    row0 += kWavesPerBlock * rpw;
+  }
+  for (; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+    if (row0 >= a.n) break;
+    const LaneRow l2g = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
+    const LaneRow l2u = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
+    float ag[MAXM], au[MAXM];
+    row_dots_pair<FMT, NB, MAXM>(l2g, l2u, g, mg.cs, mu.cs, lds, chunks, run.m, ag, au);
+    finish(l2g, ag, au);
   }
 }
 
@@ -303,7 +337,7 @@ struct TokenDownArgs {
   int n, k, tokens, top_k;
 };
 
-template <int FMT, int NB>
+template <int FMT, int NB, bool SPLIT>
 __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   constexpr int kPieces = FmtTraits<FMT>::kPieces;
@@ -318,9 +352,19 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
   float* part = reinterpret_cast<float*>(lds + a.top_k * row_vecs);   // [top_k][rows_per_block]
   const float* gd = nullptr;
   const MatRef md = mat_of_view<FMT>(a.views[a.ids[static_cast<size_t>(t) * a.top_k + wave] * 3 + 2], &gd);
-  {  // this wavefront's activation row, in the core's [piece][chunk] order
-    const uint16_t* x = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + wave) * a.act_stride;
-    const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+  // This wavefront's activation row, in the core's [piece][chunk] order. Fast set-up (a row of at most 1024
+  // aligned elements): activation loads, then the first step's weight loads, then the LDS commit.
+  const uint16_t* x = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + wave) * a.act_stride;
+  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+  constexpr int XV = kSplitStageVecs;
+  LaneRow lr = lane_row<FMT>(md, tile_row0, a.n, a.k, g.l2);
+  ChunkRegs first[NB];
+  if constexpr (SPLIT) {
+    StageRegs<XV> xr;
+    stage_issue<FMT, XV>(x, a.k, lane, kWave, xr);
+    issue_pass<FMT, NB>(lr, 0, g.l2, md.cs, first);
+    stage_commit<FMT, XV>(xr, a.k, lane, kWave, my_x);
+  } else {
     for (int v = lane; v < row_vecs; v += kWave) {
       const int c = v / kPieces, q = v - c * kPieces;
       my_x[q * chunks + c] = load_vec8(x, v, aligned);
@@ -328,13 +372,20 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
   }
   __syncthreads();
   const float dd = load_divisor<FMT>(gd);
-  for (int s = 0; s < steps; ++s) {
+  int s = 0;
+  if constexpr (SPLIT) {
+    float acc[1];
+    row_dots_pre<FMT, 1, NB>(lr, g, md.cs, my_x, chunks, 1, first, acc);   // tile_row0 < n: the grid covers n
+    if (lr.li == 0) part[wave * rows_per_block + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
+    s = 1;
+  }
+  for (; s < steps; ++s) {
     const int row0 = tile_row0 + s * rpw;
     if (row0 >= a.n) break;
-    const LaneRow lr = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
+    const LaneRow l2 = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
     float acc[1];
-    row_dots<FMT, 1, NB>(lr, g, md.cs, my_x, chunks, 1, acc);
-    if (lr.li == 0) part[wave * rows_per_block + s * rpw + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
+    row_dots<FMT, 1, NB>(l2, g, md.cs, my_x, chunks, 1, acc);
+    if (l2.li == 0) part[wave * rows_per_block + s * rpw + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
   }
   __syncthreads();
   for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
@@ -602,12 +653,23 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   const int cap = run_cap_for(a, kGateUpRun);
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
-    if (cap >= kGateUpRun)
-      hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, kGateUpRun>), grid, dim3(kBlockThreads),
-                         stage_bytes(kGateUpRun, a.k), stream, a, g, steps);
-    else
-      hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, 1>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a,
-                         g, steps);
+    const bool split = tune_get(kTuneSplitStage) != 1 && a.k <= 8 * kSplitStageVecs * kBlockThreads &&
+                       (a.x_stride & 7u) == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0;
+    if (cap >= kGateUpRun) {
+      if (split)
+        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, kGateUpRun, true>), grid, dim3(kBlockThreads),
+                           stage_bytes(kGateUpRun, a.k), stream, a, g, steps);
+      else
+        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, kGateUpRun, false>), grid, dim3(kBlockThreads),
+                           stage_bytes(kGateUpRun, a.k), stream, a, g, steps);
+    } else {
+      if (split)
+        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, 1, true>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream,
+                           a, g, steps);
+      else
+        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, 1, false>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream,
+                           a, g, steps);
+    }
   });
   return hipGetLastError();
 }
@@ -662,9 +724,14 @@ hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipStream_t stream) {
   hipError_t err = hipSuccess;
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
-    auto kern = token_down_accum_kernel<FMT, NB>;
-    err = ensure_lds(kern, lds);
-    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(a.top_k * kWave), lds, stream, a, g, steps);
+    const bool split = tune_get(kTuneSplitStage) != 1 && a.k <= 8 * kSplitStageVecs * kWave && (a.act_stride & 7u) == 0 &&
+                       (reinterpret_cast<uintptr_t>(a.act) & 15u) == 0;
+    auto go = [&](auto kern) {
+      err = ensure_lds(kern, lds);
+      if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(a.top_k * kWave), lds, stream, a, g, steps);
+    };
+    if (split) go(token_down_accum_kernel<FMT, NB, true>);
+    else go(token_down_accum_kernel<FMT, NB, false>);
   });
   return err != hipSuccess ? err : hipGetLastError();
 }
