@@ -2,8 +2,8 @@
 """Benchmark of the quantized MoE expert GEMV path on one MI355X.
 
 A "step" is one pass of the hot path over one batch: one MXFP4 MoE decode layer (router top-8
-selection from given logits -> slot order -> fused gate/up + SwiGLU -> down -> ordered
-accumulation) at the BASELINE shape (256 experts, hidden 4096, expert intermediate 1024, top-8,
+selection + slot order from given logits -> fused gate/up + SwiGLU -> down + ordered accumulation:
+three launches) at the BASELINE shape (256 experts, hidden 4096, expert intermediate 1024, top-8,
 no shared expert), T tokens. Consecutive steps walk DIFFERENT layers' weights (a ring of
 `--layers` full layers, as a model's decode step walks its MoE layers), so every step streams its
 experts from HBM, not from the 256 MB Infinity Cache / L2. The steps are captured once in a HIP
@@ -34,7 +34,7 @@ GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
 # HBM-side bytes per launch of the two GEMV kernels at the default workload (T = 8, 256 experts), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the library's plain copy kernel (the summary under
 # profiles/ holds the commands and the raw counters). A counter cannot be read from inside this process.
-MEASURED_TRAFFIC = {"gate_up": 287.3e6, "down": 145.0e6}
+MEASURED_TRAFFIC = {"gate_up": 261.5e6, "down": 138.4e6}
 DOWN_BYTES = H * I // 2 + H * I // 32
 
 
@@ -201,17 +201,14 @@ def main():
             res["gate_up_us"] = sec_k * 1e6
             res["gate_up_bytes"] = kbytes
             res["gate_up_gbps"] = kbytes / sec_k / 1e9
-        downs = torch.empty((nL, slots, H), dtype=torch.float32, device=dev)
-        counter = torch.zeros(2, dtype=torch.int32, device=dev)
-
-        def down(i):
+        def down(i):   # the layer's second GEMV kernel: token-major down projection + ordered accumulation
             l = i % nL
-            L.launch_moe_slot_down_fp4(acts[l], I, layers[l].ids_ptr, orders[l] if T > 1 else None, layers[l]._views_ptr,
-                                       H, I, 0, 0, None, None, downs[l], H, slots, K, stream, -1, 32, 7, 7, counter)
+            L.launch_moe_slot_down_accum_fp4(acts[l], I, layers[l].ids_ptr, layers[l]._views_ptr, H, I, T, K,
+                                             layers[l].weights_ptr, outs[l], None, stream, 32)
 
         if only in ("", "down"):
             sec_d = time_graph(down, steps, warmup)
-            dbytes = u_mean * DOWN_BYTES + T * K * I * 2 + T * K * H * 4
+            dbytes = u_mean * DOWN_BYTES + T * K * I * 2 + T * H * 2
             res["down_us"] = sec_d * 1e6
             res["down_bytes"] = dbytes
             res["down_gbps"] = dbytes / sec_d / 1e9
@@ -519,7 +516,9 @@ def main():
                             "bytes_per_launch": main_res["gate_up_bytes"], "us_per_launch": main_res["gate_up_us"]}
         if "down_us" in main_res:
             line["roofline"]["second_kernel"] = {
-                "kernel": "slot_down_kernel<MXFP4> (down GEMV, f32 out)", "achieved": main_res["down_gbps"],
+                "kernel": "token_down_accum_kernel<MXFP4> (down GEMV + ordered accumulation, bf16 out)",
+                "achieved": main_res["down_gbps"],
+                "traffic": MEASURED_TRAFFIC["down"] if (T == 8 and nE == E and not args.tune) else None,
                 "frac": main_res["down_gbps"] / HBM_PEAK_GBPS, "bytes_per_launch": main_res["down_bytes"],
                 "us_per_launch": main_res["down_us"]}
     print(json.dumps(line))

@@ -171,6 +171,9 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     if (!order_ready) launch_moe_slot_order(ids, d_order_, slots, K, cfg_.n_experts, stream, cfg_.shared_slots_early);
     order = d_order_;
   }
+  // The token-major down kernel fuses the accumulation but reads an expert once per slot; the slot kernel reads
+  // it once per run of slots. Token-major while few slots can share an expert (small batches), runs beyond.
+  const bool token_major = !has_shared() && dgpp_tune_get(4) != 1 && tokens * K * 4 <= cfg_.n_experts;
   const bool sh_args = has_shared() && !w_.shared_in_table;
   const int n_sh = has_shared() ? w_.shared_inter : 0;
   const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
@@ -178,7 +181,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
                                    w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
                                    K, cfg_.swiglu_limit, stream, w_.sh_rs, w_.sh_cs);
-    if (!has_shared() && dgpp_tune_get(4) != 1) {   // routed only: down + accumulation in one token-major launch
+    if (token_major) {   // routed only: down + accumulation in one token-major launch
       launch_moe_slot_down_accum(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                  out_bf16, out_f32, stream);
       return;
@@ -192,7 +195,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
                                        sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
                                        d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, stream, base, fp4_group_,
                                        w_.sh_rs, w_.sh_cs);
-    if (!has_shared() && dgpp_tune_get(4) != 1) {
+    if (token_major) {
       launch_moe_slot_down_accum_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                      out_bf16, out_f32, stream, fp4_group_);
       return;

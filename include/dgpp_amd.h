@@ -40,9 +40,11 @@ const char* dgpp_target_arch(void);
  * keeps such a switch in its launcher header too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90).
  * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: slots of one expert a
  * decode-slot block serves together (0 = default: 2 gate/up, 4 down; 1 = one slot per block);
- * key 2: row steps per block of the slot launches (0 = automatic); key 5: 2 moves the GEMV launchers
- * to the matrix-core form (another fp32 summation order, all launchers alike). Outputs do not depend on
- * keys 1 and 2; key 0 changes the fp32 summation order (every launcher follows it alike). */
+ * key 2: row steps per block of the slot launches (0 = automatic); key 3: 1 stages activations before
+ * any weight load is issued (default: activation loads, first weight pass, LDS commit); key 4: 1 keeps
+ * the layer driver on the two-launch down + accumulate form; key 5: 2 moves the GEMV launchers to the
+ * matrix-core form. Outputs do not depend on keys 1 - 4; keys 0 and 5 change the fp32 summation order
+ * (every GEMV launcher follows them alike, so the launchers stay bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);
 int dgpp_tune_get(int key);
 
