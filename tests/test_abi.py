@@ -60,3 +60,25 @@ def test_host_side_argument_checks_need_no_gpu():
     with pytest.raises(L.InvalidArgument):      # null pointers are refused before any launch
         L.launch_moe_segment(None, 4, 8, 16, None, None, None)
     L.launch_moe_segment(None, 0, 8, 16, None, None, None)      # tokens <= 0 returns silently
+
+
+def test_headers_compile_as_c_and_the_shim_as_cpp(tmp_path):
+    """include/dgpp_amd.h and dgpp_amd_layer.h are plain C; dgpp_amd.hpp (the reference's names) is C++17
+    and links against the library without running anything."""
+    import shutil
+    import subprocess
+    root = Path(__file__).resolve().parent.parent
+    inc = root / "include"
+    c_src = tmp_path / "c_check.c"
+    c_src.write_text('#include "dgpp_amd.h"\n#include "dgpp_amd_layer.h"\nint main(void) { return sizeof(DgppMoeExpertView) == 96 ? 0 : 1; }\n')
+    subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-I", str(inc), "-c", str(c_src), "-o", str(tmp_path / "c.o")],
+                   check=True)
+    rocm_inc = Path("/opt/rocm/include")
+    if not (shutil.which("g++") and rocm_inc.exists()):
+        pytest.skip("no g++ / ROCm headers")
+    cpp_src = tmp_path / "shim_check.cpp"
+    cpp_src.write_text('#include "dgpp_amd.hpp"\n#include "dgpp_amd_layer.h"\n'
+                       "int main() { return dgpp::moe_tile_list_capacity(1, 1, 16) > 0 ? 0 : 1; }\n")
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-I", str(inc), "-I", str(rocm_inc), "-D__HIP_PLATFORM_AMD__",
+                    str(cpp_src), "-L", str(root / "dgpp_amd" / "lib"), "-ldgpp_amd", "-L/opt/rocm/lib", "-lamdhip64",
+                    "-o", str(tmp_path / "shim_check")], check=True)
