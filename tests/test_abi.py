@@ -2,6 +2,7 @@
 import ctypes
 import re
 from pathlib import Path
+import pytest
 
 from dgpp_amd import _lib
 
