@@ -37,6 +37,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
 ]
+HIP_FLAGS += os.environ.get("DGPP_EXTRA_HIP_FLAGS", "").split()   # e.g. -D switches for an experiment
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-ffp-contract=off", "-pthread"]
 
 
