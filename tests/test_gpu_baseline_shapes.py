@@ -45,11 +45,16 @@ def test_c2_dense_nvfp4_17408x5120(gpu):
     got8 = host(out8, np.uint16)
     assert np.array_equal(host(out1, np.uint16)[0], got8[0]), "batch-1 row == batch-8 row 0, every output"
     assert np.array_equal(hg.f32_to_bf16(host(out8f)), got8)
+    out8m = dev_empty((8, n), np.uint16)
+    L.launch_dense_mma_fp4_bf16(a_d, k, wm, out8m, 8, n, k, None)
+    sync()
+    got8m = host(out8m, np.uint16)
     for r0 in (0, 8192, n - 1024):          # row blocks against the oracle (rows are independent)
         sl = slice(r0, r0 + 1024)
         raw = orc.gemv_fp4(act, np.ascontiguousarray(payload[sl]), np.ascontiguousarray(scales[sl]), float(glob[0]),
                            16, 8, 1024, k)
         check(np.ascontiguousarray(got8[:, sl]), raw, f"C2 rows {r0}")
+        check(np.ascontiguousarray(got8m[:, sl]), raw, f"C2 rows {r0}, matrix-core launcher")
 
 
 def _used_experts_table(ids, E, make_views):
@@ -141,6 +146,10 @@ def test_c4_fp8_moe_zipf(gpu):
     orc_experts = [m.orc() for e in range(E) for m in (per[e][1] if e in per else first)]
     raw, _ = orc.moe_forward(x, ids, w, H, I, I, orc_experts, None, float("inf"), threads=8)
     expert_budget(got, raw, "C4")
+    outm = dev_empty((T, H), np.uint16)
+    layer.enqueue_prefill_routed(x_d, H, ids_d, w_d, outm, T)
+    sync()
+    expert_budget(host(outm, np.uint16), raw, "C4, matrix-core grouped path")
     # grouping tables of the same routing, bit-exact against the host counting sort
     rows, slot_row, segs = np.empty(T * K + T, np.int32), np.empty(T * K, np.int32), np.empty((E + 1, 3), np.int32)
     orc.oracle().orc_moe_segment(orc.p(ids), T, K, E, orc.p(rows), orc.p(slot_row), orc.p(segs))
@@ -205,6 +214,19 @@ def test_c5_nvfp4_routed_plus_mxfp8_shared(gpu):
                              np.ascontiguousarray(w[sample]), H, I, SI, orc_experts, [m.orc() for m in sh],
                              float("inf"), threads=8)
     expert_budget(np.ascontiguousarray(got[sample]), raw, "C5 sampled tokens")
+    # the same layer through the matrix-core launchers: routed experts by the grouped form with the gather folded
+    # in, the shared expert by the E8M0-grid form at m = 64 (four 16-row tiles per weight pass)
+    routed_m = dev_empty((T, H), np.float32)
+    layer.enqueue_prefill_routed(x_d, H, dev(ids), dev(w), None, T, out_f32=routed_m)
+    L.launch_mma_gemv_fp8e8m0_bf16(x_d, H, shd[0][0], shd[0][1], g_d, T, SI, H, 0, 0, 5, None)
+    L.launch_mma_gemv_fp8e8m0_bf16(x_d, H, shd[1][0], shd[1][1], u_d, T, SI, H, 0, 0, 5, None)
+    L.launch_moe_swiglu_clamp(g_d, u_d, a_d, T * SI, float("inf"), None)
+    L.launch_mma_gemv_fp8e8m0_f32(a_d, SI, shd[2][0], shd[2][1], shared_down, T, H, SI, 0, 0, 5, None)
+    L.launch_moe_accum(routed_m, shared_down, rows_id, dev(np.ones(T, np.float32)), T, H, None)
+    out_m = dev_empty((T, H), np.uint16)
+    L.launch_moe_round_bf16(out_m, routed_m, T * H, None)
+    sync()
+    expert_budget(np.ascontiguousarray(host(out_m, np.uint16)[sample]), raw, "C5 sampled tokens, matrix-core launchers")
     counts = np.bincount(ids.ravel(), minlength=E)
     print(f"C5 routing: {np.count_nonzero(counts)} distinct experts, busiest {counts.max()} tokens")
     layer.close()
