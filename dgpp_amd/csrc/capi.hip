@@ -149,6 +149,7 @@ int dense_rows(int fmt, const uint16_t* act, size_t act_stride, const MatRef& ma
     a.m = rows;
     a.n = n;
     a.k = k;
+    a.once = m <= max_rows;   // one pass over the weights
     const int rc = finish(launch_dense(fmt, a, stream), who);
     if (rc != DGPP_OK) return rc;
     row0 += rows;
@@ -254,6 +255,7 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
   a.top_k = top_k;
   a.limit = limit;
   a.shared_view_base = -1;
+  a.once = slots <= 8 * (top_k + 1);   // a decode batch of at most 8 tokens: few slots can share an expert
   return a;
 }
 
@@ -278,6 +280,7 @@ int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegmen
   a.rows_per_block = rows_per_block > 0 ? rows_per_block : INT_MAX;
   a.group_rows = max_stage_rows(k);
   a.act_rows = act_rows;
+  a.once = max_rows <= (mma ? kTileCols : a.group_rows);   // every segment in one pass over its expert
   if (mma) return finish(launch_grouped_mma(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
   return finish(launch_grouped(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
 }
@@ -666,6 +669,7 @@ static int dense_mma(int fmt, const uint16_t* act, size_t act_stride, const MatR
   a.m = m;
   a.n = n;
   a.k = k;
+  a.once = m <= kTileCols;   // one activation tile: one pass over the weights
   return finish(launch_dense_mma(fmt, a, static_cast<float*>(ws), ws_bytes, as_stream(stream)), who);
 }
 

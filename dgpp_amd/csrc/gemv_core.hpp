@@ -165,24 +165,32 @@ struct ChunkRegs {
 };
 
 // Issues the loads of chunk index c of the row whose payload / scale rows are given.
-template <int FMT>
+// NT: the launch reads every weight once. Nontemporal loads then keep the stream from displacing the
+// activations and the expert table in the caches (measured: the decode gate/up kernel 9 % faster); where
+// weights are read again (several activation tiles, many slots per expert) the cached form wins. A compile
+// time choice on purpose: a run-time branch between two otherwise identical loads gets merged into one
+// plain load by the optimiser.
+template <int FMT, bool NT>
 __device__ __forceinline__ void load_chunk(const uint8_t* __restrict__ payload_row,
                                            const void* __restrict__ scale_row, int c, int cs,
                                            ChunkRegs& out) {
-  // Weights are read once: nontemporal loads keep them from displacing the activations and the
-  // expert table in the caches (measured: the gate/up kernel 9 % faster).
+  // Weights live in global memory (never LDS or scratch): saying so lets the loads be global_load
+  // instead of flat_load.
   typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(payload_row + static_cast<size_t>(c) * kChunkBytes));
+#define DGPP_AS1 __attribute__((address_space(1)))
+  const DGPP_AS1 u32x4_t* src = (const DGPP_AS1 u32x4_t*)(uintptr_t)(payload_row + static_cast<size_t>(c) * kChunkBytes);
+  const u32x4_t v = NT ? __builtin_nontemporal_load(src) : *src;
   out.w = make_uint4(v.x, v.y, v.z, v.w);
   if constexpr (FMT == kFmtFp8F32) {
-    out.s = reinterpret_cast<const uint32_t*>(scale_row)[((c * 16) >> cs)];
+    out.s = ((const DGPP_AS1 uint32_t*)(uintptr_t)scale_row)[((c * 16) >> cs)];
   } else if constexpr (FMT == kFmtFp8E8M0) {
-    out.s = reinterpret_cast<const uint8_t*>(scale_row)[((c * 16) >> cs)];
+    out.s = ((const DGPP_AS1 uint8_t*)(uintptr_t)scale_row)[((c * 16) >> cs)];
   } else if constexpr (FMT == kFmtNvfp4) {
-    out.s = reinterpret_cast<const uint16_t*>(scale_row)[c];
+    out.s = ((const DGPP_AS1 uint16_t*)(uintptr_t)scale_row)[c];
   } else {
-    out.s = reinterpret_cast<const uint8_t*>(scale_row)[c];
+    out.s = ((const DGPP_AS1 uint8_t*)(uintptr_t)scale_row)[c];
   }
+#undef DGPP_AS1
 }
 
 // Where a chunk's activation vectors come from: LDS (any number of staged rows) ...
@@ -305,10 +313,16 @@ struct LaneRow {
   int li;        // lane index inside the row group
 };
 
-template <int FMT>
-__device__ __forceinline__ LaneRow lane_row(const MatRef& mat, int row0, int n, int k, int l2) {
+// The row with the load policy (load_chunk's NT) as part of its type: functions that issue loads deduce it.
+template <bool NT>
+struct LaneRowT : LaneRow {
+  static constexpr bool kNT = NT;
+};
+
+template <int FMT, bool NT = true>
+__device__ __forceinline__ LaneRowT<NT> lane_row(const MatRef& mat, int row0, int n, int k, int l2) {
   const int lane = threadIdx.x & (kWave - 1);
-  LaneRow lr;
+  LaneRowT<NT> lr;
   lr.li = lane & ((1 << l2) - 1);
   lr.row = row0 + (lane >> l2);
   const int r = lr.row < n ? lr.row : n - 1;
@@ -326,12 +340,12 @@ __device__ __forceinline__ LaneRow lane_row(const MatRef& mat, int row0, int n, 
 }
 
 // Loads one pass (NB chunks) of a row for this lane.
-template <int FMT, int NB>
-__device__ __forceinline__ void issue_pass(const LaneRow& lr, int pass, int l2, int cs,
+template <int FMT, int NB, class LR>
+__device__ __forceinline__ void issue_pass(const LR& lr, int pass, int l2, int cs,
                                            ChunkRegs (&regs)[NB]) {
 #pragma unroll
   for (int i = 0; i < NB; ++i)
-    load_chunk<FMT>(lr.payload_row, lr.scale_row, ((pass * NB + i) << l2) + lr.li, cs, regs[i]);
+    load_chunk<FMT, LR::kNT>(lr.payload_row, lr.scale_row, ((pass * NB + i) << l2) + lr.li, cs, regs[i]);
 }
 
 template <int FMT, int MAXR, int NB>
@@ -347,8 +361,8 @@ __device__ __forceinline__ void consume_pass(const ChunkRegs (&regs)[NB], const 
 
 // Full dot products of this lane's row against m staged activation rows; after the call every
 // lane of the row group holds the finished sums (the NVFP4 division is the caller's epilogue).
-template <int FMT, int MAXR, int NB>
-__device__ __forceinline__ void row_dots(const LaneRow& lr, const RowGeom& g, int cs,
+template <int FMT, int MAXR, int NB, class LR>
+__device__ __forceinline__ void row_dots(const LR& lr, const RowGeom& g, int cs,
                                          const uint4* __restrict__ lds, int chunks, int m,
                                          float (&acc)[MAXR]) {
 #pragma unroll
@@ -365,8 +379,8 @@ __device__ __forceinline__ void row_dots(const LaneRow& lr, const RowGeom& g, in
 }
 
 // row_dots with the first pass's loads already issued by the caller. Same chain.
-template <int FMT, int MAXR, int NB>
-__device__ __forceinline__ void row_dots_pre(const LaneRow& lr, const RowGeom& g, int cs,
+template <int FMT, int MAXR, int NB, class LR>
+__device__ __forceinline__ void row_dots_pre(const LR& lr, const RowGeom& g, int cs,
                                              const uint4* __restrict__ lds, int chunks, int m,
                                              const ChunkRegs (&first)[NB], float (&acc)[MAXR]) {
 #pragma unroll
@@ -450,8 +464,8 @@ __device__ __forceinline__ void consume_pass_pair(const ChunkRegs (&ca)[NB], con
     }
   }
 }
-template <int FMT, int NB, int MAXM>
-__device__ __forceinline__ void row_dots_pair(const LaneRow& la, const LaneRow& lb, const RowGeom& g, int csa,
+template <int FMT, int NB, int MAXM, class LR>
+__device__ __forceinline__ void row_dots_pair(const LR& la, const LR& lb, const RowGeom& g, int csa,
                                               int csb, const uint4* __restrict__ lds, int chunks, int m,
                                               float (&ra)[MAXM], float (&rb)[MAXM]) {
 #pragma unroll
@@ -472,8 +486,8 @@ __device__ __forceinline__ void row_dots_pair(const LaneRow& la, const LaneRow& 
   }
 }
 // The same with pass 0 of the two rows already issued by the caller (`fa`, `fb`). Same chain.
-template <int FMT, int NB, int MAXM>
-__device__ __forceinline__ void row_dots_pair_pre(const LaneRow& la, const LaneRow& lb, const RowGeom& g, int csa,
+template <int FMT, int NB, int MAXM, class LR>
+__device__ __forceinline__ void row_dots_pair_pre(const LR& la, const LR& lb, const RowGeom& g, int csa,
                                                   int csb, const uint4* __restrict__ lds, int chunks, int m,
                                                   const ChunkRegs (&fa)[NB], const ChunkRegs (&fb)[NB],
                                                   float (&ra)[MAXM], float (&rb)[MAXM]) {

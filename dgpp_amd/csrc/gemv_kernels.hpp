@@ -71,9 +71,10 @@ struct DenseArgs {
   size_t out_stride;
   int out_f32;
   int m, n, k;
+  int once;                 // all m rows ride on one pass over the weights (nontemporal loads)
 };
 
-template <int FMT, int MAXR, int NB>
+template <int FMT, int MAXR, int NB, bool NT>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_kernel(DenseArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_ke
   int row0 = blockIdx.x * block_rows(g, steps) + wave * rpw;
   for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
     if (row0 >= a.n) break;
-    const LaneRow lr = lane_row<FMT>(a.mat, row0, a.n, a.k, g.l2);
+    const auto lr = lane_row<FMT, NT>(a.mat, row0, a.n, a.k, g.l2);
     float acc[MAXR];
     row_dots<FMT, MAXR, NB>(lr, g, a.mat.cs, lds, chunks, a.m, acc);
     if (lr.li == 0 && lr.row < a.n) {
@@ -122,6 +123,7 @@ struct SlotArgs {
   int n, k;                 // the dims of the slots this launch computes
   int slots, top_k;
   float limit;
+  int once;                 // few slots can share an expert: the weights stream through once (nontemporal loads)
   int want_shared;          // 0: routed slots, 1: shared slots (others exit)
   int shared_view_base;     // >= 0: shared matrices come from views[base + which]
 };
@@ -204,7 +206,7 @@ __device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& ru
   return true;
 }
 
-template <int FMT, int NB, int MAXM, bool SPLIT>
+template <int FMT, int NB, int MAXM, bool SPLIT, bool NT>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   SlotRun<MAXM> run;
@@ -229,8 +231,8 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_
   // Fast set-up (rows of at most 4096 aligned elements): activation loads, then the first step's weight
   // loads, then the LDS commit and the barrier — the weights travel while the block sets up.
   constexpr int XV = kSplitStageVecs;
-  LaneRow lg = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
-  LaneRow lu = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
+  const auto lg = lane_row<FMT, NT>(mg, row0, a.n, a.k, g.l2);
+  const auto lu = lane_row<FMT, NT>(mu, row0, a.n, a.k, g.l2);
   ChunkRegs fg[NB], fu[NB];
   if constexpr (SPLIT) {
     StageRegs<XV> xr[MAXM];
@@ -271,8 +273,8 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_
   }
   for (; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
     if (row0 >= a.n) break;
-    const LaneRow l2g = lane_row<FMT>(mg, row0, a.n, a.k, g.l2);
-    const LaneRow l2u = lane_row<FMT>(mu, row0, a.n, a.k, g.l2);
+    const auto l2g = lane_row<FMT, NT>(mg, row0, a.n, a.k, g.l2);
+    const auto l2u = lane_row<FMT, NT>(mu, row0, a.n, a.k, g.l2);
     float ag[MAXM], au[MAXM];
     row_dots_pair<FMT, NB, MAXM>(l2g, l2u, g, mg.cs, mu.cs, lds, chunks, run.m, ag, au);
     finish(l2g, ag, au);
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_
 }
 
 // Down rows of a run of slots, unrounded f32.
-template <int FMT, int NB, int MAXM>
+template <int FMT, int NB, int MAXM, bool NT>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   SlotRun<MAXM> run;
@@ -309,7 +311,7 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_ker
   int row0 = tile_row0 + wave * rpw;
   for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
     if (row0 >= a.n) break;
-    const LaneRow lr = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
+    const auto lr = lane_row<FMT, NT>(md, row0, a.n, a.k, g.l2);
     float acc[MAXM];
     row_dots<FMT, MAXM, NB>(lr, g, md.cs, lds, chunks, run.m, acc);
     if (lr.li == 0 && lr.row < a.n) {
@@ -357,7 +359,7 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
   const uint16_t* x = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + wave) * a.act_stride;
   const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
   constexpr int XV = kSplitStageVecs;
-  LaneRow lr = lane_row<FMT>(md, tile_row0, a.n, a.k, g.l2);
+  const auto lr = lane_row<FMT, true>(md, tile_row0, a.n, a.k, g.l2);
   ChunkRegs first[NB];
   if constexpr (SPLIT) {
     StageRegs<XV> xr;
@@ -382,7 +384,7 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
   for (; s < steps; ++s) {
     const int row0 = tile_row0 + s * rpw;
     if (row0 >= a.n) break;
-    const LaneRow l2 = lane_row<FMT>(md, row0, a.n, a.k, g.l2);
+    const auto l2 = lane_row<FMT, true>(md, row0, a.n, a.k, g.l2);
     float acc[1];
     row_dots<FMT, 1, NB>(l2, g, md.cs, my_x, chunks, 1, acc);
     if (l2.li == 0) part[wave * rows_per_block + s * rpw + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
@@ -416,9 +418,10 @@ struct GroupedArgs {
   int rows_per_block;  // segment rows per z block
   int group_rows;      // activation rows staged per pass (<= kMaxActRows)
   const int32_t* act_rows;  // matrix-core form only, nullable: activation row of each segment row
+  int once;                 // every segment fits one pass over its expert (nontemporal loads)
 };
 
-template <int FMT, int NB>
+template <int FMT, int NB, bool NT>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void grouped_gemv_kernel(GroupedArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   const DgppMoeSegment seg = a.segs[blockIdx.y];
@@ -439,7 +442,7 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void grouped_gemv_
     int row0 = blockIdx.x * block_rows(g, steps) + wave * rpw;
     for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
       if (row0 >= a.n) break;
-      const LaneRow lr = lane_row<FMT>(mat, row0, a.n, a.k, g.l2);
+      const auto lr = lane_row<FMT, NT>(mat, row0, a.n, a.k, g.l2);
       float acc[kMaxActRows];
       row_dots<FMT, kMaxActRows, NB>(lr, g, mat.cs, lds, chunks, m, acc);
       if (lr.li == 0 && lr.row < a.n) {
@@ -517,6 +520,12 @@ inline int max_stage_rows(int k) {
 
 // The bodies, included by the per-format translation units.
 #ifdef DGPP_GEMV_IMPL
+template <class F>
+inline void dispatch_bool(bool v, F&& f) {
+  if (v) f(std::true_type{});
+  else f(std::false_type{});
+}
+
 // The GEMV launchers run the vector ALU core (fastest while one or two activation rows ride on a weight
 // pass); the bench switch moves them to the matrix-core form, which the *_mma_* launchers always use.
 inline bool use_mfma_core() { return tune_get(kTuneCore) == 2; }
@@ -530,8 +539,10 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
   const size_t need = static_cast<size_t>(g.parts) * a.m * a.n * sizeof(float);
   const bool split = ws != nullptr && g.parts > 1 && ws_bytes >= need && static_cast<size_t>(gx) * gy < 1024;
   const dim3 grid(gx, gy, split ? g.parts : 1);
-  hipLaunchKernelGGL((mfma_dense_kernel<FMT, kMfmaNB>), grid, dim3(kBlockThreads), 2 * kStageUnits * sizeof(uint4), stream,
-                     a, g, split ? ws : nullptr);
+  dispatch_bool(a.once != 0, [&](auto ntc) {
+    hipLaunchKernelGGL((mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value>), grid, dim3(kBlockThreads),
+                       2 * kStageUnits * sizeof(uint4), stream, a, g, split ? ws : nullptr);
+  });
   if (split) {
     const int64_t total = static_cast<int64_t>(a.m) * a.n;
     hipLaunchKernelGGL(fold_parts_kernel<FMT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream, ws,
@@ -544,8 +555,10 @@ template <int FMT>
 hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {
   const MGeom g = mgeom<FMT>(a.k);
   const dim3 grid(static_cast<unsigned>((a.n + 63) / 64), static_cast<unsigned>(n_segs), static_cast<unsigned>(z_ext));
-  hipLaunchKernelGGL((mfma_grouped_kernel<FMT, kMfmaNB>), grid, dim3(kBlockThreads), 2 * kStageUnits * sizeof(uint4),
-                     stream, a, g);
+  dispatch_bool(a.once != 0, [&](auto ntc) {
+    hipLaunchKernelGGL((mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value>), grid, dim3(kBlockThreads),
+                       2 * kStageUnits * sizeof(uint4), stream, a, g);
+  });
   return hipGetLastError();
 }
 
@@ -615,10 +628,12 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
     constexpr int NB = decltype(nbc)::value;
     auto go = [&](auto rc) {
       constexpr int MAXR = decltype(rc)::value;
-      auto kern = gemv_dense_kernel<FMT, MAXR, NB>;
-      err = ensure_lds(kern, lds);
-      if (err != hipSuccess) return;
-      hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
+      dispatch_bool(a.once != 0, [&](auto ntc) {
+        auto kern = gemv_dense_kernel<FMT, MAXR, NB, decltype(ntc)::value>;
+        err = ensure_lds(kern, lds);
+        if (err != hipSuccess) return;
+        hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
+      });
     };
     if (a.m == 1) go(std::integral_constant<int, 1>{});
     else if (a.m == 2) go(std::integral_constant<int, 2>{});
@@ -655,21 +670,20 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
     constexpr int NB = decltype(nbc)::value;
     const bool split = tune_get(kTuneSplitStage) != 1 && a.k <= 8 * kSplitStageVecs * kBlockThreads &&
                        (a.x_stride & 7u) == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0;
-    if (cap >= kGateUpRun) {
-      if (split)
-        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, kGateUpRun, true>), grid, dim3(kBlockThreads),
-                           stage_bytes(kGateUpRun, a.k), stream, a, g, steps);
-      else
-        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, kGateUpRun, false>), grid, dim3(kBlockThreads),
-                           stage_bytes(kGateUpRun, a.k), stream, a, g, steps);
-    } else {
-      if (split)
-        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, 1, true>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream,
-                           a, g, steps);
-      else
-        hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, 1, false>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream,
-                           a, g, steps);
-    }
+    // Nontemporal loads only with the split set-up (the decode form); shared slots are read by every token.
+    const bool nt = split && a.once && !a.want_shared;
+    auto go = [&](auto mc, auto sc, auto ntc) {
+      constexpr int MAXM = decltype(mc)::value;
+      hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, MAXM, decltype(sc)::value, decltype(ntc)::value>), grid,
+                         dim3(kBlockThreads), stage_bytes(MAXM, a.k), stream, a, g, steps);
+    };
+    auto go_m = [&](auto mc) {
+      if (nt) go(mc, std::true_type{}, std::true_type{});
+      else if (split) go(mc, std::true_type{}, std::false_type{});
+      else go(mc, std::false_type{}, std::false_type{});
+    };
+    if (cap >= kGateUpRun) go_m(std::integral_constant<int, kGateUpRun>{});
+    else go_m(std::integral_constant<int, 1>{});
   });
   return hipGetLastError();
 }
@@ -697,15 +711,18 @@ hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
   const int cap = run_cap_for(a, kDownRun);
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
-    if (cap >= kDownRun)
-      hipLaunchKernelGGL((slot_down_kernel<FMT, NB, kDownRun>), grid, dim3(kBlockThreads), stage_bytes(kDownRun, a.k),
-                         stream, a, g, steps);
-    else if (cap >= 2)
-      hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 2>), grid, dim3(kBlockThreads), stage_bytes(2, a.k), stream, a, g,
-                         steps);
-    else
-      hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 1>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g,
-                         steps);
+    dispatch_bool(a.once && !a.want_shared, [&](auto ntc) {
+      constexpr bool NT = decltype(ntc)::value;
+      if (cap >= kDownRun)
+        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, kDownRun, NT>), grid, dim3(kBlockThreads), stage_bytes(kDownRun, a.k),
+                           stream, a, g, steps);
+      else if (cap >= 2)
+        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 2, NT>), grid, dim3(kBlockThreads), stage_bytes(2, a.k), stream, a, g,
+                           steps);
+      else
+        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 1, NT>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g,
+                           steps);
+    });
   });
   return hipGetLastError();
 }
@@ -758,10 +775,12 @@ hipError_t launch_grouped_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipSt
   hipError_t err = hipSuccess;
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
-    auto kern = grouped_gemv_kernel<FMT, NB>;
-    err = ensure_lds(kern, lds);
-    if (err != hipSuccess) return;
-    hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
+    dispatch_bool(a.once != 0, [&](auto ntc) {
+      auto kern = grouped_gemv_kernel<FMT, NB, decltype(ntc)::value>;
+      err = ensure_lds(kern, lds);
+      if (err != hipSuccess) return;
+      hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
+    });
   });
   return err != hipSuccess ? err : hipGetLastError();
 }

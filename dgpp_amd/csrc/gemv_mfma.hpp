@@ -128,12 +128,16 @@ struct GroupLane {
   int q;          // the piece this lane LOADS
   int from;       // byte address (lane * 4) of the lane whose load this lane consumes
 };
-template <int FMT>
-__device__ __forceinline__ GroupLane group_lane(const MatRef& mat, int row0, int n, int k) {
+template <bool NT>
+struct GroupLaneT : GroupLane {
+  static constexpr bool kNT = NT;   // load_chunk's load policy, part of the type
+};
+template <int FMT, bool NT = true>
+__device__ __forceinline__ GroupLaneT<NT> group_lane(const MatRef& mat, int row0, int n, int k) {
   const int lane = threadIdx.x & (kWave - 1);
   const int row = row0 + (lane >> 2);
   const int r = row < n ? row : n - 1;   // rows past the end redo the last row; their results are dropped
-  GroupLane gl;
+  GroupLaneT<NT> gl;
   gl.q = lane & 3;
   gl.from = (4 * (lane & 15) + (lane >> 4)) * 4;
   if constexpr (FMT == kFmtFp8F32 || FMT == kFmtFp8E8M0) {
@@ -150,11 +154,11 @@ __device__ __forceinline__ GroupLane group_lane(const MatRef& mat, int row0, int
 }
 
 // The lane's 16 bytes of step `step` (chunk index step * 4 + q of the row), or zeros past k.
-template <int FMT>
-__device__ __forceinline__ void load_step(const GroupLane& gl, int step, int chunks, int cs, ChunkRegs& out) {
+template <int FMT, class GL>
+__device__ __forceinline__ void load_step(const GL& gl, int step, int chunks, int cs, ChunkRegs& out) {
   const int c = step * 4 + gl.q;
   if (c < chunks) {
-    load_chunk<FMT>(gl.payload_row, gl.scale_row, c, cs, out);
+    load_chunk<FMT, GL::kNT>(gl.payload_row, gl.scale_row, c, cs, out);
   } else {
     out.w = make_uint4(0u, 0u, 0u, 0u);   // code 0 is +0 in e2m1 and e4m3
     out.s = 0u;

@@ -26,7 +26,7 @@ __host__ __device__ inline int stage_steps_for(int mt, int part_steps) {
 // the block must call.
 // Parts [p_lo, p_hi) only (the others stay zero). `act_rows`, when given, names the activation
 // row of each of the mt rows (a gather folded into the stage load).
-template <int FMT, int NB>
+template <int FMT, int NB, bool NT>
 __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_t* __restrict__ act, size_t act_stride,
                                                 const int32_t* __restrict__ act_rows, int mt, int n, int k, int row0,
                                                 const MGeom& g, int p_lo, int p_hi, uint4* __restrict__ lds,
@@ -35,7 +35,7 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
   constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
   constexpr int kStepElems = MTraits<FMT>::kStepElems;
   const int chunks = k / MTraits<FMT>::kLoadElems;
-  const GroupLane gl = group_lane<FMT>(mat, row0, n, k);
+  const auto gl = group_lane<FMT, NT>(mat, row0, n, k);
   const int lane = threadIdx.x & (kWave - 1);
   const int cc = min(lane & 15, mt - 1);
   const bool aligned = ((reinterpret_cast<uintptr_t>(act) & 15u) == 0) && ((act_stride & 7u) == 0);
@@ -115,7 +115,7 @@ __device__ __forceinline__ void store_tile(const f32x4_t& v, float divisor, void
 // `partials` null: all parts in one block, folded and stored. Otherwise blockIdx.z names the ONE part
 // this block computes and its raw sums go to partials[part][row of out][n] (fp32); fold_parts_kernel
 // then adds the parts in the same ascending order — the split form's bits are the unsplit form's.
-template <int FMT, int NB>
+template <int FMT, int NB, bool NT>
 __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs a, MGeom g, float* partials) {
   extern __shared__ uint4 lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
@@ -125,14 +125,14 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs 
   const int c = lane & 15;
   f32x4_t sum;
   if (partials == nullptr) {
-    block_rows_mfma<FMT, NB>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k,
+    block_rows_mfma<FMT, NB, NT>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k,
                              row0, g, 0, g.parts, lds, sum);
     store_tile<FMT>(sum, load_divisor<FMT>(a.global), a.out, a.out_f32, static_cast<size_t>(c0 + c) * a.out_stride, row0,
                     a.n, c < mt);
     return;
   }
   const int part = static_cast<int>(blockIdx.z);
-  block_rows_mfma<FMT, NB>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k, row0,
+  block_rows_mfma<FMT, NB, NT>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k, row0,
                            g, part, part + 1, lds, sum);
   store_tile<kFmtMxfp4>(sum, 1.0f, partials, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
 }
@@ -156,7 +156,7 @@ __global__ void fold_parts_kernel(const float* __restrict__ partials, int parts,
     static_cast<uint16_t*>(out)[at] = f32_to_bf16(x);
 }
 
-template <int FMT, int NB>
+template <int FMT, int NB, bool NT>
 __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedArgs a, MGeom g) {
   extern __shared__ uint4 lds[];
   const DgppMoeSegment seg = a.segs[blockIdx.y];
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
     const int mt = min(kTileCols, z1 - c0);
     f32x4_t sum;
     const size_t first = static_cast<size_t>(seg.row0 + c0);
-    block_rows_mfma<FMT, NB>(mat, a.act_rows ? a.act : a.act + first * a.act_stride, a.act_stride,
+    block_rows_mfma<FMT, NB, NT>(mat, a.act_rows ? a.act : a.act + first * a.act_stride, a.act_stride,
                              a.act_rows ? a.act_rows + first : nullptr, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum);
     store_tile<FMT>(sum, divisor, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, c < mt);
   }
@@ -241,8 +241,8 @@ __global__ __launch_bounds__(kBlockThreads, 2) void slot_gate_up_mfma_kernel(Slo
   constexpr int kSub = MTraits<FMT>::kSub;
   constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
   const int chunks = a.k / MTraits<FMT>::kLoadElems;
-  const GroupLane lg = group_lane<FMT>(mg, row0, a.n, a.k);
-  const GroupLane lu = group_lane<FMT>(mu, row0, a.n, a.k);
+  const auto lg = group_lane<FMT, true>(mg, row0, a.n, a.k);
+  const auto lu = group_lane<FMT, true>(mu, row0, a.n, a.k);
   const int cc = min(lane & 15, m - 1);
   const uint4* lane_stage = stage + ((lane >> 4) * kSub) * m + cc;
   const int step0 = part * g.part_steps;
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void slot_down_mfma_kernel(SlotAr
   constexpr int kSub = MTraits<FMT>::kSub;
   constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
   const int chunks = a.k / MTraits<FMT>::kLoadElems;
-  const GroupLane ld = group_lane<FMT>(md, row0, a.n, a.k);
+  const auto ld = group_lane<FMT, true>(md, row0, a.n, a.k);
   const int cc = min(lane & 15, m - 1);
   const uint4* lane_stage = stage + ((lane >> 4) * kSub) * m + cc;
   const int step0 = part * g.part_steps;
