@@ -256,6 +256,8 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
   a.limit = limit;
   a.shared_view_base = -1;
   a.once = slots <= 8 * (top_k + 1);   // a decode batch of at most 8 tokens: few slots can share an expert
+  const int tokens = top_k >= 0 ? slots / (top_k + 1) : 0;
+  a.match = order == nullptr && tokens > 1 && tokens * top_k <= 64;
   return a;
 }
 
@@ -362,7 +364,7 @@ int dgpp_launch_moe_router_select_order(const float* scores, const float* biased
   if (!scores || !biased || !ids || !weights) return fail_arg(std::string(who) + ": null pointer");
   const int slots = tokens * (cfg->top_k + 1);
   if (order != nullptr && slots > 1024) return fail_arg(std::string(who) + ": at most 1024 slots");
-  if (tokens <= 16 && cfg->n_experts <= 8 * 64)
+  if (order != nullptr && tokens <= 16 && cfg->n_experts <= 8 * 64)
     return finish(run_router_select_order(cfg->router_mode, scores, biased, ids, weights, order, tokens, cfg->n_experts,
                                           cfg->top_k, cfg->routed_scaling_factor, cfg->norm_topk_prob ? 1 : 0,
                                           shared_early, as_stream(stream)),

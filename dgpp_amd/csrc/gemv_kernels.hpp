@@ -123,6 +123,7 @@ struct SlotArgs {
   int n, k;                 // the dims of the slots this launch computes
   int slots, top_k;
   float limit;
+  int match;                // no order and tokens * top_k <= 64: find the slots that share an expert by ballot
   int once;                 // few slots can share an expert: the weights stream through once (nontemporal loads)
   int want_shared;          // 0: routed slots, 1: shared slots (others exit)
   int shared_view_base;     // >= 0: shared matrices come from views[base + which]
@@ -200,6 +201,44 @@ __device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& ru
         } else {
           alive = false;
         }
+      }
+    } else if (a.match && key0 >= 0) {
+      // No order given, a small decode batch (tokens * top_k <= 64): the slots that use this expert are found
+      // with one ballot over the routed ids (an expert occurs at most once per token, so they sit in
+      // different tokens). The first of every MAXM of them, in (token, j) order, leads the run.
+      const int lane = threadIdx.x & (kWave - 1);
+      const int tk = (a.slots / (a.top_k + 1)) * a.top_k;
+      const int theirs = lane < tk ? a.ids[lane] : -1;
+      const unsigned long long mask = __builtin_amdgcn_ballot_w64(theirs == key0);
+      const int mine = token0 * a.top_k + (slot0 - token0 * (a.top_k + 1));
+      const int before = __builtin_popcountll(mask & ((1ull << mine) - 1ull));
+      if (before % MAXM != 0) return false;
+      unsigned long long rest = mine >= 63 ? 0ull : mask >> (mine + 1);
+      int at = mine;
+#pragma unroll
+      for (int r = 1; r < MAXM; ++r) {
+        run.slot[r] = slot0;
+        run.token[r] = token0;
+        if (rest != 0ull) {
+          const int skip = __builtin_ctzll(rest);
+          at += skip + 1;
+          rest = skip >= 63 ? 0ull : rest >> (skip + 1);
+          const int t = at / a.top_k;
+          run.slot[r] = t * (a.top_k + 1) + (at - t * a.top_k);
+          run.token[r] = t;
+          run.m = r + 1;
+        }
+      }
+    } else if (a.match) {
+      // The shared slots of consecutive tokens use the same (shared) expert.
+      const int tokens = a.slots / (a.top_k + 1);
+      if (token0 % MAXM != 0) return false;
+#pragma unroll
+      for (int r = 1; r < MAXM; ++r) {
+        const bool have = token0 + r < tokens;
+        run.token[r] = have ? token0 + r : token0;
+        run.slot[r] = run.token[r] * (a.top_k + 1) + a.top_k;
+        if (have) run.m = r + 1;
       }
     }
   }
@@ -565,7 +604,7 @@ hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipS
 // Slots per run in the matrix-core slot kernels: bounded by the LDS of the per-wavefront stages.
 template <int FMT>
 inline int mfma_run_cap(const SlotArgs& a, const MGeom& g, int max_run) {
-  if (a.order == nullptr) return 1;
+  if (a.order == nullptr && !a.match) return 1;
   const int tuned = tune_get(kTuneSlotRun);
   int cap = tuned > 0 && tuned < max_run ? tuned : max_run;
   while (cap > 1 && (kWavesPerBlock * slot_wave_units<FMT>(cap, g) + kSlotRedUnits) * sizeof(uint4) > 48 * 1024) --cap;
@@ -649,7 +688,7 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
 constexpr int kGateUpRun = 2;
 constexpr int kDownRun = 4;
 inline int run_cap_for(const SlotArgs& a, int max_run) {
-  if (a.order == nullptr) return 1;            // slots in layout order: no two neighbours share an expert
+  if (a.order == nullptr && !a.match) return 1;   // slots in layout order and no way to find the sharers
   const int tuned = tune_get(kTuneSlotRun);
   int cap = tuned > 0 ? tuned : max_run;
   while (cap > 1 && (cap > max_run || stage_bytes(cap, a.k) > 16 * 1024)) --cap;

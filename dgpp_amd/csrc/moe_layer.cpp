@@ -127,6 +127,15 @@ GlmMoeLayer::~GlmMoeLayer() {
   if (arena_) (void)hipFree(arena_);
 }
 
+// The expert-sorted slot order pays for itself once many slots share experts. A small batch (tokens * top_k <=
+// 64) skips it: the gate/up kernel finds the few sharers by ballot, the token-major down kernel needs no order,
+// and the selection runs as one wavefront per token on separate CUs instead of one block.
+bool GlmMoeLayer::needs_order(int tokens) const {
+  if (tokens <= 1 || tokens * (cfg_.top_k + 1) > 1024) return false;
+  if (dgpp_tune_get(6) == 1) return true;
+  return tokens * cfg_.top_k > 64;
+}
+
 void GlmMoeLayer::check_tokens(int tokens) const {
   if (tokens > max_tokens_) throw std::invalid_argument("GlmMoeLayer: tokens exceed the layer's max_tokens");
 }
@@ -145,7 +154,7 @@ void GlmMoeLayer::enqueue_decode_scores(const uint16_t* x, size_t x_stride, cons
   if (tokens <= 0) return;
   check_tokens(tokens);
   // Selection and slot order in one launch; the chain below then finds its order ready.
-  const bool with_order = tokens > 1 && tokens * (cfg_.top_k + 1) <= 1024;
+  const bool with_order = needs_order(tokens);
   launch_moe_router_select_order(scores, biased, d_ids_, d_weights_, with_order ? d_order_ : nullptr, cfg_, tokens, stream,
                                  cfg_.shared_slots_early);
   expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream, /*order_ready=*/true);
@@ -167,7 +176,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   if (slots > 1024 && tokens > 1)
     throw std::invalid_argument("GlmMoeLayer: the decode-slot path takes at most 1024 slots; use the grouped path");
   const int32_t* order = nullptr;
-  if (tokens > 1) {
+  if (needs_order(tokens)) {
     if (!order_ready) launch_moe_slot_order(ids, d_order_, slots, K, cfg_.n_experts, stream, cfg_.shared_slots_early);
     order = d_order_;
   }

@@ -59,6 +59,7 @@ class GlmMoeLayer {
 
  private:
   void check_tokens(int tokens) const;
+  bool needs_order(int tokens) const;
   void expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                           uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
                           bool order_ready = false);
