@@ -2,8 +2,8 @@
 """Benchmark of the quantized MoE expert GEMV path on one MI355X.
 
 A "step" is one pass of the hot path over one batch: one MXFP4 MoE decode layer (router top-8
-selection + slot order from given logits -> fused gate/up + SwiGLU -> down + ordered accumulation:
-three launches) at the BASELINE shape (256 experts, hidden 4096, expert intermediate 1024, top-8,
+selection from given logits -> fused gate/up + SwiGLU -> down + ordered accumulation: three
+launches) at the BASELINE shape (256 experts, hidden 4096, expert intermediate 1024, top-8,
 no shared expert), T tokens. Consecutive steps walk DIFFERENT layers' weights (a ring of
 `--layers` full layers, as a model's decode step walks its MoE layers), so every step streams its
 experts from HBM, not from the 256 MB Infinity Cache / L2. The steps are captured once in a HIP
@@ -34,7 +34,7 @@ GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
 # HBM-side bytes per launch of the two GEMV kernels at the default workload (T = 8, 256 experts), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the library's plain copy kernel (the summary under
 # profiles/ holds the commands and the raw counters). A counter cannot be read from inside this process.
-MEASURED_TRAFFIC = {"gate_up": 261.5e6, "down": 138.4e6}
+MEASURED_TRAFFIC = {"gate_up": 260.7e6, "down": 138.5e6}
 DOWN_BYTES = H * I // 2 + H * I // 32
 
 
@@ -184,14 +184,15 @@ def main():
         with torch.cuda.stream(stream):
             for l in range(nL):
                 full(l)                                       # leaves ids / weights in the layer's scratch
-                o = torch.empty(slots, dtype=torch.int32, device=dev)
-                if T > 1:
+                o = None
+                if T * K > 64:      # as the layer does: small batches need no slot order (sharers found by ballot)
+                    o = torch.empty(slots, dtype=torch.int32, device=dev)
                     L.launch_moe_slot_order(layers[l].ids_ptr, o, slots, K, nE, stream)
                 orders.append(o)
             stream.synchronize()
         def gate_up(i):
             l = i % nL
-            L.launch_moe_slot_gate_up_swiglu_fp4(xs[l], H, layers[l].ids_ptr, orders[l] if T > 1 else None,
+            L.launch_moe_slot_gate_up_swiglu_fp4(xs[l], H, layers[l].ids_ptr, orders[l],
                                                  layers[l]._views_ptr, I, H, 0, 0, None, None, None, None, acts[l], I,
                                                  slots, K, float("inf"), stream, -1, 32)
 
