@@ -578,10 +578,14 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
   const size_t need = static_cast<size_t>(g.parts) * a.m * a.n * sizeof(float);
   const bool split = ws != nullptr && g.parts > 1 && ws_bytes >= need && static_cast<size_t>(gx) * gy < 1024;
   const dim3 grid(gx, gy, split ? g.parts : 1);
+  hipError_t err = hipSuccess;
   dispatch_bool(a.once != 0, [&](auto ntc) {
-    hipLaunchKernelGGL((mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value>), grid, dim3(kBlockThreads),
-                       2 * kStageUnits * sizeof(uint4), stream, a, g, split ? ws : nullptr);
+    auto kern = mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value>;
+    constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
+    err = ensure_lds(kern, lds);
+    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, split ? ws : nullptr);
   });
+  if (err != hipSuccess) return err;
   if (split) {
     const int64_t total = static_cast<int64_t>(a.m) * a.n;
     hipLaunchKernelGGL(fold_parts_kernel<FMT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream, ws,
@@ -594,11 +598,14 @@ template <int FMT>
 hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {
   const MGeom g = mgeom<FMT>(a.k);
   const dim3 grid(static_cast<unsigned>((a.n + 63) / 64), static_cast<unsigned>(n_segs), static_cast<unsigned>(z_ext));
+  hipError_t err = hipSuccess;
   dispatch_bool(a.once != 0, [&](auto ntc) {
-    hipLaunchKernelGGL((mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value>), grid, dim3(kBlockThreads),
-                       2 * kStageUnits * sizeof(uint4), stream, a, g);
+    auto kern = mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value>;
+    constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
+    err = ensure_lds(kern, lds);
+    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g);
   });
-  return hipGetLastError();
+  return err != hipSuccess ? err : hipGetLastError();
 }
 
 // Slots per run in the matrix-core slot kernels: bounded by the LDS of the per-wavefront stages.

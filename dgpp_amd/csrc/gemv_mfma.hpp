@@ -44,7 +44,7 @@ constexpr int kTileCols = 16;        // activation rows of one MFMA tile
 
 struct MGeom {
   int parts;       // 1, 2 or 4
-  int part_steps;  // steps per part (the last part may be shorter)
+  int part_steps;  // steps per part, a multiple of 4 (trailing parts may be shorter or empty)
   int steps;       // steps covering k
 };
 template <int FMT>
@@ -53,7 +53,7 @@ __host__ __device__ inline MGeom mgeom(int k) {
   MGeom g;
   g.parts = k >= 4096 ? 4 : (k >= 2048 ? 2 : 1);
   g.steps = (k + se - 1) / se;
-  g.part_steps = (g.steps + g.parts - 1) / g.parts;
+  g.part_steps = ((g.steps + g.parts - 1) / g.parts + 3) & ~3;   // whole tiles of four steps
   return g;
 }
 
@@ -171,6 +171,126 @@ __device__ __forceinline__ void to_operand_layout(const GroupLane& gl, ChunkRegs
   r.w.z = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.w.z)));
   r.w.w = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.w.w)));
   r.s = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(gl.from, static_cast<int>(r.s)));
+}
+
+// ---- row-wide tile loads -------------------------------------------------------------------------------
+// The operand layout wants 16 different rows in 16 adjacent lanes; loading that way makes every quarter
+// wavefront touch 4 - 16 rows with 64 or 16 bytes each, which the vector memory pipe serves well below its
+// streaming rate. The block kernels therefore load a TILE — 16 rows x 256 bytes, the four steps of a chunk —
+// row-major (instruction i reads rows 4i .. 4i+3, sixteen lanes per row: 256 contiguous bytes per quarter
+// wavefront), park it in a wavefront-private LDS region and read it back in operand layout. The region is
+// XOR-swizzled by row so that both the row-major writes and the column-major reads are conflict-free.
+constexpr int kTileUnits = 256;   // 16-byte units of one tile (4 KB)
+
+struct WideLane {
+  const uint8_t* base;   // matrix payload
+  uint32_t off[4];       // byte offset of this lane's row for each of the four load instructions
+  uint32_t row_bytes;
+  int piece;             // 16-byte piece of the 256-byte row segment this lane loads
+};
+template <int FMT>
+__device__ __forceinline__ WideLane wide_lane(const MatRef& mat, int row0, int n, int k) {
+  const int lane = threadIdx.x & (kWave - 1);
+  WideLane w;
+  w.base = mat.payload;
+  w.row_bytes = static_cast<uint32_t>(FmtTraits<FMT>::kIsFp4 ? k / 2 : k);
+  w.piece = lane & 15;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = row0 + 4 * i + (lane >> 4);
+    w.off[i] = static_cast<uint32_t>(row < n ? row : n - 1) * w.row_bytes;   // rows past the end redo the last row
+  }
+  return w;
+}
+// The tile that starts at step `step0` (bytes step0 * 64 ... + 255 of each row); zeros past the row's end.
+template <bool NT>
+__device__ __forceinline__ void issue_tile(const WideLane& w, int step0, uint4 (&t)[4]) {
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  const uint32_t in_row = static_cast<uint32_t>(step0) * 64u + static_cast<uint32_t>(w.piece) * 16u;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (in_row < w.row_bytes) {
+      const __attribute__((address_space(1))) u32x4_t* src =
+          (const __attribute__((address_space(1))) u32x4_t*)(uintptr_t)(w.base + w.off[i] + in_row);
+      const u32x4_t v = NT ? __builtin_nontemporal_load(src) : *src;
+      t[i] = make_uint4(v.x, v.y, v.z, v.w);
+    } else {
+      t[i] = make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+}
+__device__ __forceinline__ void commit_tile(uint4* __restrict__ region, const uint4 (&t)[4]) {
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 4 * i + (lane >> 4);
+    region[r * 16 + ((lane & 15) ^ r)] = t[i];
+  }
+}
+// Lane (r = lane % 16, q = lane / 16): its 16 bytes of step t of the tile (piece 4 t + q of row r).
+__device__ __forceinline__ uint4 tile_operand(const uint4* __restrict__ region, int t) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int r = lane & 15;
+  return region[r * 16 + ((4 * t + (lane >> 4)) ^ r)];
+}
+
+// The block scales of a row group in operand layout (lane (r, q): row r, piece q of a step).
+struct ScaleLane {
+  const void* scale_row;
+  int q;
+};
+template <int FMT>
+__device__ __forceinline__ ScaleLane scale_lane(const MatRef& mat, int row0, int n, int k) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int row = row0 + (lane & 15);
+  const int r = row < n ? row : n - 1;
+  ScaleLane sl;
+  sl.q = lane >> 4;
+  if constexpr (FMT == kFmtFp8F32 || FMT == kFmtFp8E8M0) {
+    const size_t scale_cols = (static_cast<size_t>(k) + (1u << mat.cs) - 1) >> mat.cs;
+    const size_t esz = FMT == kFmtFp8F32 ? 4 : 1;
+    sl.scale_row = reinterpret_cast<const uint8_t*>(mat.scales) + (static_cast<size_t>(r >> mat.rs) * scale_cols) * esz;
+  } else {
+    sl.scale_row = reinterpret_cast<const uint8_t*>(mat.scales) + static_cast<size_t>(r) * (k / (FMT == kFmtNvfp4 ? 16 : 32));
+  }
+  return sl;
+}
+// ChunkRegs::s of the lane's piece of step `step` (0 past k).
+template <int FMT>
+__device__ __forceinline__ uint32_t load_scale(const ScaleLane& sl, int step, int chunks, int cs) {
+  const int c = step * 4 + sl.q;
+  if (c >= chunks) return 0u;
+#define DGPP_AS1 __attribute__((address_space(1)))
+  if constexpr (FMT == kFmtFp8F32) {
+    return ((const DGPP_AS1 uint32_t*)(uintptr_t)sl.scale_row)[(c * 16) >> cs];
+  } else if constexpr (FMT == kFmtFp8E8M0) {
+    return ((const DGPP_AS1 uint8_t*)(uintptr_t)sl.scale_row)[(c * 16) >> cs];
+  } else if constexpr (FMT == kFmtNvfp4) {
+    return ((const DGPP_AS1 uint16_t*)(uintptr_t)sl.scale_row)[c];
+  } else {
+    return ((const DGPP_AS1 uint8_t*)(uintptr_t)sl.scale_row)[c];
+  }
+#undef DGPP_AS1
+}
+
+// acc += the chunk whose tile sits in `region` (operand reads) with block scales sc[0 .. 3]; `valid` steps.
+template <int FMT>
+__device__ __forceinline__ void mfma_tile(const uint4* __restrict__ region, const uint32_t (&sc)[4],
+                                          const uint4* __restrict__ lane_stage, int m, int valid, f32x4_t& acc) {
+  constexpr int kSub = MTraits<FMT>::kSub;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (i < valid) {
+      ChunkRegs ch;
+      ch.w = tile_operand(region, i);
+      ch.s = sc[i];
+      Frag f[kSub];
+      decode_frags<FMT>(ch, f);
+#pragma unroll
+      for (int j = 0; j < kSub; ++j) acc = mfma_bf16(f[j], lane_stage[(i * 4 * kSub + j) * m], acc);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
 }
 
 // One 8-element block of an activation row as a 16-byte vector; zeros past k.

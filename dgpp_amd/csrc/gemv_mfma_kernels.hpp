@@ -1,5 +1,5 @@
 // Kernels of the matrix-core GEMV form (gemv_mfma.hpp): dense projection and grouped segments
-// (block-shared, double-buffered activation stages), decode slots (one K part per wavefront).
+// (row-wide tile loads, a block-shared activation stage), decode slots (one K part per wavefront).
 // Included by gemv_kernels.hpp after the argument structs.
 #pragma once
 
@@ -10,85 +10,87 @@ namespace dgpp_amd {
 constexpr int kStageUnits = 1024;   // 16-byte units of one block-shared activation stage (16 KB)
 constexpr int kMfmaNB = 4;          // lane loads in flight per row group and pass
 
-// Steps of one block-shared stage for mt activation rows: a multiple of kMfmaNB within the unit budget.
-template <int FMT>
-__host__ __device__ inline int stage_steps_for(int mt, int part_steps) {
-  int s = kStageUnits / (mt * MTraits<FMT>::kStepBlocks);
-  s -= s % kMfmaNB;
-  if (s < kMfmaNB) s = kMfmaNB;
-  const int cover = (part_steps + kMfmaNB - 1) / kMfmaNB * kMfmaNB;
-  return s < cover ? s : cover;
-}
+// 64 weight rows (one row group per wavefront) against mt <= 16 activation rows, parts [p_lo, p_hi) of K.
+// K is walked in batches of up to kTileBatch tiles (a tile = four steps of a row group, gemv_mfma.hpp):
+// a wavefront puts all of a batch's weight loads in flight, the block then fetches the batch's
+// activations into the LDS stage as [8-element block][row], and the tiles pass one after the other through
+// the wavefront's own LDS region into the matrix core. Nothing of a wavefront is in flight while it
+// computes; the other blocks of the CU cover that, so the kernel is kept small in registers and LDS
+// (several blocks per CU) rather than pipelined inside the wavefront. `sum` receives the parts' sums added
+// in ascending order. `act_rows`, when given, names the activation row of each of the mt rows (a gather
+// folded into the stage load). LDS: the stage, then one tile region per wavefront. Every thread of the
+// block must call.
+constexpr int kTileBatch = 2;   // 8 KB in flight per wavefront; more tiles cost registers, and blocks per CU count for more
+constexpr int kBlockMfmaLdsUnits = kStageUnits + kWavesPerBlock * kTileUnits;
 
-// 64 weight rows (one row group per wavefront) against mt <= 16 activation rows, all of K: the
-// block walks K in stages; a stage's activations sit in LDS as [8-element block][row], fetched one
-// stage ahead into registers. `sum` receives the parts' sums added in ascending order. Every thread of
-// the block must call.
-// Parts [p_lo, p_hi) only (the others stay zero). `act_rows`, when given, names the activation
-// row of each of the mt rows (a gather folded into the stage load).
 template <int FMT, int NB, bool NT>
 __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_t* __restrict__ act, size_t act_stride,
                                                 const int32_t* __restrict__ act_rows, int mt, int n, int k, int row0,
                                                 const MGeom& g, int p_lo, int p_hi, uint4* __restrict__ lds,
                                                 f32x4_t& sum) {
+  static_assert(NB == 4, "a tile is four steps");
   constexpr int kSub = MTraits<FMT>::kSub;
   constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
   constexpr int kStepElems = MTraits<FMT>::kStepElems;
+  constexpr int kStageRegs = kStageUnits / kBlockThreads;
   const int chunks = k / MTraits<FMT>::kLoadElems;
-  const auto gl = group_lane<FMT, NT>(mat, row0, n, k);
-  const int lane = threadIdx.x & (kWave - 1);
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  const WideLane wl = wide_lane<FMT>(mat, row0, n, k);
+  const ScaleLane sl = scale_lane<FMT>(mat, row0, n, k);
+  uint4* region = lds + kStageUnits + wave * kTileUnits;
   const int cc = min(lane & 15, mt - 1);
   const bool aligned = ((reinterpret_cast<uintptr_t>(act) & 15u) == 0) && ((act_stride & 7u) == 0);
-  const int stage_steps = stage_steps_for<FMT>(mt, g.part_steps);
-  const int spp = (g.part_steps + stage_steps - 1) / stage_steps;
-  const int total = (p_hi - p_lo) * spp;
-  const int units = stage_steps * kStepBlocks * mt;
-  uint4 pre[4];
-  auto fetch = [&](int s) {
-    const int p = p_lo + s / spp, ls = s - (p - p_lo) * spp;
-    const int k_base = (p * g.part_steps + ls * stage_steps) * kStepElems;
+  const int cpp = g.part_steps / NB;   // tiles per part: part_steps is a multiple of four
+  const int batch = max(1, min(kTileBatch, kStageUnits / (mt * kStepBlocks * NB)));
+  const int t_hi = p_hi * cpp;
+  // this thread's pieces of a batch's activations: 8-element block kb of row c for each of its units
+  int unit_kb[kStageRegs];
+  const uint16_t* unit_row[kStageRegs];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = threadIdx.x + i * kBlockThreads;
-      if (idx < units) {
-        const int kb = idx / mt, c = idx - kb * mt;
-        const size_t arow = act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(c);
-        pre[i] = load_act_block(act + arow * act_stride, k_base + kb * 8, k, aligned);
-      }
+  for (int i = 0; i < kStageRegs; ++i) {
+    const int idx = threadIdx.x + i * kBlockThreads;
+    const int kb = idx / mt, c = idx - kb * mt;
+    unit_kb[i] = kb;
+    unit_row[i] = act + (act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(c)) * act_stride;
+  }
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = p_lo * cpp; t0 < t_hi; t0 += batch) {
+    const int tiles = min(batch, t_hi - t0);
+    uint4 tile[kTileBatch][4];
+    uint32_t sc[kTileBatch][4];
+    int valid[kTileBatch];
+#pragma unroll
+    for (int d = 0; d < kTileBatch; ++d) {
+      const int step0 = (t0 + d) * NB;
+      valid[d] = d < tiles ? max(0, min(NB, g.steps - step0)) : 0;
+      issue_tile<NT>(wl, valid[d] > 0 ? step0 : g.steps, tile[d]);   // nothing to read: zeros, no loads
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sc[d][i] = load_scale<FMT>(sl, i < valid[d] ? step0 + i : g.steps, chunks, mat.cs);
     }
-  };
-  auto put = [&](int buf) {
+    const int units = tiles * NB * kStepBlocks * mt;
+    const int k_base = t0 * NB * kStepElems;
+    uint4 pre[kStageRegs];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int idx = threadIdx.x + i * kBlockThreads;
-      if (idx < units) lds[buf * kStageUnits + idx] = pre[i];
+    for (int i = 0; i < kStageRegs; ++i) {
+      pre[i] = make_uint4(0u, 0u, 0u, 0u);
+      if (threadIdx.x + i * kBlockThreads < units) pre[i] = load_act_block(unit_row[i], k_base + unit_kb[i] * 8, k, aligned);
     }
-  };
-  fetch(0);
-  put(0);
-  __syncthreads();
-  int s = 0;
-  // Each part accumulates from zero and joins the running sum when it ends: ((p0 + p1) + p2) + p3.
-  for (int p = p_lo; p < p_hi; ++p) {
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-    {
-      for (int ls = 0; ls < spp; ++ls, ++s) {
-        const bool more = s + 1 < total;
-        if (more) fetch(s + 1);
-        const uint4* lane_stage = lds + (s & 1) * kStageUnits + ((lane >> 4) * kSub) * mt + cc;
-        const int step0 = p * g.part_steps + ls * stage_steps;
-        const int nsteps = min(stage_steps, g.part_steps - ls * stage_steps);
-        for (int t = 0; t < nsteps; t += NB) {
-          ChunkRegs regs[NB];
+    __syncthreads();   // the stage's readers of the batch before are through
 #pragma unroll
-          for (int i = 0; i < NB; ++i) load_step<FMT>(gl, t + i < nsteps ? step0 + t + i : g.steps, chunks, mat.cs, regs[i]);
-          mfma_chunk<FMT, NB>(gl, regs, lane_stage + (t * kStepBlocks) * mt, mt, min(NB, nsteps - t), acc);
+    for (int i = 0; i < kStageRegs; ++i)
+      if (threadIdx.x + i * kBlockThreads < units) lds[threadIdx.x + i * kBlockThreads] = pre[i];
+    __syncthreads();
+#pragma unroll
+    for (int d = 0; d < kTileBatch; ++d) {
+      if (d < tiles) {
+        commit_tile(region, tile[d]);   // the region's earlier reads were issued before: LDS keeps a wavefront's order
+        mfma_tile<FMT>(region, sc[d], lds + (d * NB * kStepBlocks + (lane >> 4) * kSub) * mt + cc, mt, valid[d], acc);
+        if ((t0 + d + 1) % cpp == 0) {   // a part ends: it joins the running sum, ((p0 + p1) + p2) + p3
+          sum = (t0 + d + 1 == (p_lo + 1) * cpp) ? acc : sum + acc;
+          acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
-        if (more) put((s + 1) & 1);
-        __syncthreads();
       }
     }
-    sum = p == p_lo ? acc : sum + acc;
   }
 }
 
