@@ -411,7 +411,10 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
       my_x[q * chunks + c] = load_vec8(x, v, aligned);
     }
   }
-  __syncthreads();
+  // The staged row is this wavefront's own: LDS keeps a wavefront's writes and reads in order, no block barrier.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   const float dd = load_divisor<FMT>(gd);
   int s = 0;
   if constexpr (SPLIT) {
