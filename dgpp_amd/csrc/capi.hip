@@ -89,6 +89,13 @@ hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t s) {
     default: return launch_slot_gate_up_fmt<kFmtMxfp4>(a, s);
   }
 }
+hipError_t launch_select_gate_up(int fmt, const SlotArgs& a, const SelectArgs& sel, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_select_gate_up_fmt<kFmtFp8F32>(a, sel, s);
+    case kFmtNvfp4: return launch_select_gate_up_fmt<kFmtNvfp4>(a, sel, s);
+    default: return launch_select_gate_up_fmt<kFmtMxfp4>(a, sel, s);
+  }
+}
 hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t s) {
   switch (fmt) {
     case kFmtFp8F32: return launch_slot_down_fmt<kFmtFp8F32>(a, s);
@@ -511,6 +518,77 @@ int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, cons
   a.sh[0] = fp8_mat(sh_gate_payload, sh_gate_scales, sh_rs, sh_cs);
   a.sh[1] = fp8_mat(sh_up_payload, sh_up_scales, sh_rs, sh_cs);
   return finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who);
+}
+
+namespace {
+// The limits of select_gate_up_kernel: one token, its score row fits a wavefront's registers, and the
+// decode form of the gate/up kernel (fast set-up) applies.
+bool select_gate_up_fits(const SlotArgs& a, int tokens, int n_experts) {
+  return tokens == 1 && a.top_k <= kWave && n_experts <= 8 * kWave && tune_get(kTuneCore) != 2 &&
+         tune_get(kTuneSplitStage) != 1 && tune_get(kTuneSelectAlone) != 1 && a.k <= 8 * kSplitStageVecs * kBlockThreads &&
+         (a.x_stride & 7u) == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0;
+}
+
+int select_gate_up(int fmt, const float* scores, const float* biased, int32_t* ids, float* weights, const DgppMoeConfig* cfg,
+                   int tokens, const uint16_t* x, size_t x_stride, const DgppMoeExpertView* views, int n_routed,
+                   int k_routed, uint16_t* act, int act_stride, float limit, void* stream, int fp4_group, const char* who) {
+  int rc = dgpp_moe_config_validate(cfg);
+  if (rc != DGPP_OK) return rc;
+  if (tokens <= 0) return DGPP_OK;
+  if (!scores || !biased || !ids || !weights) return fail_arg(std::string(who) + ": null pointer");
+  if (tokens > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
+  const int slots = tokens * (cfg->top_k + 1);
+  SlotArgs a = slot_args(x, x_stride, ids, nullptr, views, act, act_stride, slots, cfg->top_k, limit);
+  a.n = n_routed;
+  a.k = k_routed;
+  a.want_shared = 0;
+  if (!x || !views || !act || n_routed <= 0 || k_routed <= 0 || act_stride < n_routed || !select_gate_up_fits(a, tokens, cfg->n_experts)) {
+    // outside the one-launch form (or invalid: the two launchers say why)
+    rc = dgpp_launch_moe_router_select(scores, biased, ids, weights, cfg, tokens, stream);
+    if (rc != DGPP_OK) return rc;
+    if (fmt == kFmtFp8F32)
+      return dgpp_launch_moe_slot_gate_up_swiglu(x, x_stride, ids, nullptr, views, n_routed, k_routed, 0, 0, nullptr, nullptr,
+                                                 nullptr, nullptr, act, act_stride, slots, cfg->top_k, limit, stream, 7, 7);
+    return dgpp_launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, nullptr, views, n_routed, k_routed, 0, 0, nullptr, nullptr,
+                                                   nullptr, nullptr, act, act_stride, slots, cfg->top_k, limit, stream, -1,
+                                                   fp4_group, 7, 7);
+  }
+  if (fmt == kFmtFp8F32) {
+    rc = check_slot_common(x, ids, views, act, n_routed, k_routed, 0, 0, who);
+    if (rc != DGPP_OK) return rc;
+    if (k_routed % 16 != 0 || stage_bytes(1, k_routed) > kMaxLdsBytes)
+      return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
+  } else {
+    rc = check_fp4_slot(x, ids, views, act, n_routed, k_routed, 0, 0, -1, fp4_group, who);
+    if (rc != DGPP_OK) return rc;
+  }
+  SelectArgs sel;
+  sel.scores = scores;
+  sel.biased = biased;
+  sel.ids = ids;
+  sel.weights = weights;
+  sel.mode = cfg->router_mode;
+  sel.n_experts = cfg->n_experts;
+  sel.scaling = cfg->routed_scaling_factor;
+  sel.norm_topk = cfg->norm_topk_prob ? 1 : 0;
+  return finish(launch_select_gate_up(fmt, a, sel, as_stream(stream)), who);
+}
+}  // namespace
+
+int dgpp_launch_moe_select_gate_up_swiglu(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                          const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                          const DgppMoeExpertView* views, int n_routed, int k_routed, uint16_t* act,
+                                          int act_stride, float limit, void* stream) {
+  return select_gate_up(kFmtFp8F32, scores, biased, ids, weights, cfg, tokens, x, x_stride, views, n_routed, k_routed, act,
+                        act_stride, limit, stream, 0, "moe_select_gate_up");
+}
+int dgpp_launch_moe_select_gate_up_swiglu_fp4(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                              const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                              const DgppMoeExpertView* views, int n_routed, int k_routed, uint16_t* act,
+                                              int act_stride, float limit, void* stream, int fp4_group) {
+  if (fp4_group != 16 && fp4_group != 32) return fail_arg("moe_select_gate_up_fp4: fp4_group must be 16 or 32");
+  return select_gate_up(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, scores, biased, ids, weights, cfg, tokens, x, x_stride, views,
+                        n_routed, k_routed, act, act_stride, limit, stream, fp4_group, "moe_select_gate_up_fp4");
 }
 
 int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,

@@ -11,6 +11,7 @@
 
 #include "../../include/dgpp_amd.h"
 #include "gemv_core.hpp"
+#include "router_select.hpp"
 
 namespace dgpp_amd {
 
@@ -127,6 +128,18 @@ struct SlotArgs {
   int once;                 // few slots can share an expert: the weights stream through once (nontemporal loads)
   int want_shared;          // 0: routed slots, 1: shared slots (others exit)
   int shared_view_base;     // >= 0: shared matrices come from views[base + which]
+};
+
+// The router selection a gate/up launch can repeat in every block instead of reading `ids` (select_gate_up_kernel).
+struct SelectArgs {
+  const float* scores;      // [tokens, n_experts]
+  const float* biased;      // [tokens, n_experts]
+  int32_t* ids;             // out [tokens, top_k], stored by block (0, 0)
+  float* weights;           // out [tokens, top_k]
+  int mode;                 // DGPP_ROUTER_*
+  int n_experts;
+  float scaling;
+  int norm_topk;
 };
 
 template <int FMT>
@@ -246,8 +259,7 @@ __device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& ru
 }
 
 template <int FMT, int NB, int MAXM, bool SPLIT, bool NT>
-__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
-  extern __shared__ uint4 lds[];
+__device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGeom& g, int steps, uint4* __restrict__ lds) {
   SlotRun<MAXM> run;
   if (!resolve_run<MAXM>(a, run)) return;
   const int rows_per_block = block_rows(g, steps);
@@ -318,6 +330,53 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_
     row_dots_pair<FMT, NB, MAXM>(l2g, l2u, g, mg.cs, mu.cs, lds, chunks, run.m, ag, au);
     finish(l2g, ag, au);
   }
+}
+
+template <int FMT, int NB, int MAXM, bool SPLIT, bool NT>
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  slot_gate_up_body<FMT, NB, MAXM, SPLIT, NT>(a, g, steps, lds);
+}
+
+// The router's selection and the routed gate/up pass of a ONE-token decode step in one launch: the first
+// wavefront of every block repeats the selection (whole score row in registers: the selection kernel's own
+// code), the ids go to LDS behind the activation stage and the block goes on as slot_gate_up_kernel does.
+// Block (0, 0) stores ids and weights for the launches that follow. One token only: the repeated selection
+// costs every SIMD a few microseconds per token, which a launch of its own undercuts from two tokens on.
+// n_experts <= 512, routed slots only; the fast set-up, nontemporal weight loads.
+template <int FMT, int NB>
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void select_gate_up_kernel(SlotArgs a, SelectArgs sel, RowGeom g,
+                                                                                        int steps) {
+  extern __shared__ uint4 lds[];
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  int32_t* ids = reinterpret_cast<int32_t*>(lds + FmtTraits<FMT>::kPieces * chunks);
+  const int lane = threadIdx.x & (kWave - 1);
+  if (threadIdx.x < kWave) {
+    int id;
+    float w;
+    if (sel.n_experts <= 4 * kWave) {
+      if (sel.mode == DGPP_ROUTER_SOFTMAX_TOPK)
+        rsel::select_token<DGPP_ROUTER_SOFTMAX_TOPK, 4>(sel.scores, sel.biased, sel.n_experts, a.top_k, sel.scaling, sel.norm_topk, lane, id, w);
+      else
+        rsel::select_token<DGPP_ROUTER_SIGMOID_BIAS, 4>(sel.scores, sel.biased, sel.n_experts, a.top_k, sel.scaling, sel.norm_topk, lane, id, w);
+    } else {
+      if (sel.mode == DGPP_ROUTER_SOFTMAX_TOPK)
+        rsel::select_token<DGPP_ROUTER_SOFTMAX_TOPK, 8>(sel.scores, sel.biased, sel.n_experts, a.top_k, sel.scaling, sel.norm_topk, lane, id, w);
+      else
+        rsel::select_token<DGPP_ROUTER_SIGMOID_BIAS, 8>(sel.scores, sel.biased, sel.n_experts, a.top_k, sel.scaling, sel.norm_topk, lane, id, w);
+    }
+    if (lane < a.top_k) {
+      ids[lane] = id;
+      if (blockIdx.x == 0 && blockIdx.y == 0) {
+        sel.ids[lane] = id;
+        sel.weights[lane] = w;
+      }
+    }
+  }
+  __syncthreads();
+  SlotArgs b = a;
+  b.ids = ids;
+  slot_gate_up_body<FMT, NB, 1, true, true>(b, g, steps, lds);
 }
 
 // Down rows of a run of slots, unrounded f32.
@@ -526,6 +585,7 @@ inline int pick_steps(long long block_steps_total) {
 
 hipError_t launch_dense(int fmt, const DenseArgs& a, hipStream_t stream);
 hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t stream);
+hipError_t launch_select_gate_up(int fmt, const SlotArgs& a, const SelectArgs& sel, hipStream_t stream);
 hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t stream);
 hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
 
@@ -542,6 +602,7 @@ template <int FMT> hipError_t launch_grouped_mma_fmt(const GroupedArgs& a, int n
 // Per-format implementations.
 template <int FMT> hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream);
 template <int FMT> hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream);
+template <int FMT> hipError_t launch_select_gate_up_fmt(const SlotArgs& a, const SelectArgs& sel, hipStream_t stream);
 template <int FMT> hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream);
 template <int FMT> hipError_t launch_grouped_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
 
@@ -733,6 +794,23 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
     };
     if (cap >= kGateUpRun) go_m(std::integral_constant<int, kGateUpRun>{});
     else go_m(std::integral_constant<int, 1>{});
+  });
+  return hipGetLastError();
+}
+
+// The fused selection + gate/up launch; the caller has checked its limits (capi.hip, select_gate_up_fits).
+template <int FMT>
+hipError_t launch_select_gate_up_fmt(const SlotArgs& a, const SelectArgs& sel, hipStream_t stream) {
+  const RowGeom g = geom_for<FMT>(a.k);
+  const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
+  const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
+  int steps = pick_steps(per_slot * a.slots);
+  if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
+  const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
+  dispatch_nb(g.nb, [&](auto nbc) {
+    constexpr int NB = decltype(nbc)::value;
+    hipLaunchKernelGGL((select_gate_up_kernel<FMT, NB>), grid, dim3(kBlockThreads),
+                       stage_bytes(1, a.k) + kWave * sizeof(int32_t), stream, a, sel, g, steps);
   });
   return hipGetLastError();
 }

@@ -5,6 +5,7 @@
 namespace dgpp_amd {
 template hipError_t launch_dense_fmt<kFmtMxfp4>(const DenseArgs&, hipStream_t);
 template hipError_t launch_slot_gate_up_fmt<kFmtMxfp4>(const SlotArgs&, hipStream_t);
+template hipError_t launch_select_gate_up_fmt<kFmtMxfp4>(const SlotArgs&, const SelectArgs&, hipStream_t);
 template hipError_t launch_slot_down_fmt<kFmtMxfp4>(const SlotArgs&, hipStream_t);
 template hipError_t launch_grouped_fmt<kFmtMxfp4>(const GroupedArgs&, int, int, hipStream_t);
 template hipError_t launch_dense_mma_fmt<kFmtMxfp4>(const DenseArgs&, float*, size_t, hipStream_t);

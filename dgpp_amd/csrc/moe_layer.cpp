@@ -153,11 +153,15 @@ void GlmMoeLayer::enqueue_decode_scores(const uint16_t* x, size_t x_stride, cons
                                         uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
   if (tokens <= 0) return;
   check_tokens(tokens);
-  // Selection and slot order in one launch; the chain below then finds its order ready.
+  // One routed-only token: the gate/up launch repeats the selection in its blocks (no launch of its own).
+  // Otherwise selection and slot order in one launch; the chain below then finds its order ready.
   const bool with_order = needs_order(tokens);
-  launch_moe_router_select_order(scores, biased, d_ids_, d_weights_, with_order ? d_order_ : nullptr, cfg_, tokens, stream,
-                                 cfg_.shared_slots_early);
-  expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream, /*order_ready=*/true);
+  const bool fused = tokens == 1 && !has_shared() && dgpp_tune_get(7) != 1;
+  if (!fused)
+    launch_moe_router_select_order(scores, biased, d_ids_, d_weights_, with_order ? d_order_ : nullptr, cfg_, tokens, stream,
+                                   cfg_.shared_slots_early);
+  expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream, /*order_ready=*/true,
+                     fused ? scores : nullptr, fused ? biased : nullptr);
 }
 
 void GlmMoeLayer::enqueue_decode_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
@@ -170,7 +174,7 @@ void GlmMoeLayer::enqueue_decode_routed(const uint16_t* x, size_t x_stride, cons
 // Steps 4-7 of the reference's decode call order (src/models/glm/moe_layer.cpp:1555-1677).
 void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                                      uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
-                                     bool order_ready) {
+                                     bool order_ready, const float* sel_scores, const float* sel_biased) {
   const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter;
   const int slots = tokens * (K + 1);
   if (slots > 1024 && tokens > 1)
@@ -186,10 +190,17 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   const bool sh_args = has_shared() && !w_.shared_in_table;
   const int n_sh = has_shared() ? w_.shared_inter : 0;
   const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
+  // With scores given, ids / weights are this layer's own buffers and the gate/up launch fills them.
+  const bool fused = sel_scores != nullptr && ids == d_ids_ && weights == d_weights_ && order == nullptr && !has_shared();
+  if (sel_scores != nullptr && !fused) throw std::logic_error("GlmMoeLayer: fused selection outside its form");
   if (w_.format == GlmExpertFormat::Fp8) {
-    launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
-                                   w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
-                                   K, cfg_.swiglu_limit, stream, w_.sh_rs, w_.sh_cs);
+    if (fused)
+      launch_moe_select_gate_up_swiglu(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
+                                       d_slot_act_, max_inter_, cfg_.swiglu_limit, stream);
+    else
+      launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
+                                     w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
+                                     K, cfg_.swiglu_limit, stream, w_.sh_rs, w_.sh_cs);
     if (token_major) {   // routed only: down + accumulation in one token-major launch
       launch_moe_slot_down_accum(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                  out_bf16, out_f32, stream);
@@ -199,11 +210,15 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
                          n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, stream, w_.sh_rs, w_.sh_cs);
   } else {
     const int base = w_.shared_in_table ? cfg_.n_experts * 3 : -1;
-    launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
-                                       sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
-                                       sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
-                                       d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, stream, base, fp4_group_,
-                                       w_.sh_rs, w_.sh_cs);
+    if (fused)
+      launch_moe_select_gate_up_swiglu_fp4(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I,
+                                           H, d_slot_act_, max_inter_, cfg_.swiglu_limit, stream, fp4_group_);
+    else
+      launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
+                                         sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
+                                         sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
+                                         d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, stream, base, fp4_group_,
+                                         w_.sh_rs, w_.sh_cs);
     if (token_major) {
       launch_moe_slot_down_accum_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                      out_bf16, out_f32, stream, fp4_group_);

@@ -62,7 +62,7 @@ class GlmMoeLayer {
   bool needs_order(int tokens) const;
   void expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                           uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
-                          bool order_ready = false);
+                          bool order_ready = false, const float* sel_scores = nullptr, const float* sel_biased = nullptr);
 
   GlmMoeConfig cfg_;
   GlmMoeLayerWeights w_;

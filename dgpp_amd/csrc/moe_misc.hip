@@ -13,12 +13,14 @@
 #include "../../include/dgpp_amd.h"
 #include "moe_misc.hpp"
 #include "numerics.hpp"
+#include "router_select.hpp"
 
 namespace dgpp_amd {
 namespace {
 
 constexpr int kElemThreads = 256;
-constexpr int kWaveSize = 64;
+using rsel::kWaveSize;
+using rsel::select_token;
 
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -183,136 +185,6 @@ __global__ __launch_bounds__(kWaveSize) void router_select_kernel(
     ids[static_cast<size_t>(t) * top_k + i] = sel[i];
     weights[static_cast<size_t>(t) * top_k + i] = w;
   }
-}
-
-// The same selection for up to 64 * PER_LANE experts with the whole row in registers (expert e
-// lives in lane e % 64, slot e / 64): no LDS, no barriers, DPP reductions inside 16-lane rows and
-// four lane reads across them. A value's ordering key is a monotone unsigned image of the float
-// (-0 folded into +0 first: they compare equal as floats; NaN maps to 0 and never wins); among
-// equal keys the LOWEST id is taken — the strict '>' scan's outcome.
-template <int kCtrl>
-__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
-  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), kCtrl, 0xF, 0xF, true));
-}
-template <int kCtrl>
-__device__ __forceinline__ float dpp_f32(float v) {
-  return bits_f32(dpp_u32<kCtrl>(f32_bits(v)));
-}
-__device__ __forceinline__ float row_lane(float v, int lane) {
-  return bits_f32(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(f32_bits(v)), lane)));
-}
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-  v += dpp_f32<0xB1>(v);
-  v += dpp_f32<0x4E>(v);
-  v += dpp_f32<0x141>(v);
-  v += dpp_f32<0x140>(v);
-  return (row_lane(v, 0) + row_lane(v, 16)) + (row_lane(v, 32) + row_lane(v, 48));
-}
-__device__ __forceinline__ float wave_max_dpp(float v) {
-  v = fmaxf(v, dpp_f32<0xB1>(v));
-  v = fmaxf(v, dpp_f32<0x4E>(v));
-  v = fmaxf(v, dpp_f32<0x141>(v));
-  v = fmaxf(v, dpp_f32<0x140>(v));
-  return fmaxf(fmaxf(row_lane(v, 0), row_lane(v, 16)), fmaxf(row_lane(v, 32), row_lane(v, 48)));
-}
-__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
-__device__ __forceinline__ uint32_t lane_u32(uint32_t v, int lane) {
-  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane));
-}
-__device__ __forceinline__ uint32_t order_key(float v) {
-  if (v != v) return 0u;                       // NaN: below every real key
-  const uint32_t u = f32_bits(v + 0.0f);       // -0 -> +0
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
-
-// One wavefront selects for one token. On return lane p < top_k holds the token's p-th expert in
-// ascending id order and its final weight; no private arrays, no LDS.
-template <int kMode, int PER_LANE>
-__device__ __forceinline__ void select_token(const float* __restrict__ scores, const float* __restrict__ biased,
-                                             int n_experts, int top_k, float scaling, int norm_topk, int lane,
-                                             int& out_id, float& out_w) {
-  float sc[PER_LANE];
-  uint32_t key[PER_LANE];
-#pragma unroll
-  for (int j = 0; j < PER_LANE; ++j) {
-    const int e = lane + j * kWaveSize;
-    const bool live = e < n_experts;
-    sc[j] = live ? scores[e] : -INFINITY;
-    key[j] = live ? order_key(biased[e]) : 0u;
-  }
-  if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
-    float m = -INFINITY;
-#pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) m = fmaxf(m, sc[j]);
-    m = wave_max_dpp(m);
-    float sum = 0.f;
-#pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) {
-      sc[j] = lane + j * kWaveSize < n_experts ? expf(sc[j] - m) : 0.f;
-      sum += sc[j];
-    }
-    sum = wave_sum_dpp(sum);
-#pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) sc[j] = sc[j] / sum;
-  }
-  // Pick r lands in lane r. A round takes the wave-wide maximum key (one DPP max per step), then the
-  // LOWEST expert id among the lanes and slots that hold it: slot-major ids (e = lane + 64 * slot),
-  // so the first slot with a match wins and, inside it, the lowest matching lane.
-  int my_id = INT_MAX;
-  float my_w = 0.f;
-  for (int r = 0; r < top_k; ++r) {
-    uint32_t m = key[0];
-#pragma unroll
-    for (int j = 1; j < PER_LANE; ++j) m = m > key[j] ? m : key[j];
-    m = umax(m, dpp_u32<0xB1>(m));
-    m = umax(m, dpp_u32<0x4E>(m));
-    m = umax(m, dpp_u32<0x141>(m));
-    m = umax(m, dpp_u32<0x140>(m));
-    const uint32_t top = umax(umax(lane_u32(m, 0), lane_u32(m, 16)), umax(lane_u32(m, 32), lane_u32(m, 48)));
-    int best = 0;
-    bool found = false;
-#pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) {
-      const uint64_t hit = __builtin_amdgcn_ballot_w64(key[j] == top);
-      if (!found && hit != 0) {
-        best = j * kWaveSize + __builtin_ctzll(hit);
-        found = true;
-      }
-    }
-    if (top == 0u || best >= n_experts) best = 0;   // a row of NaN keys: stay in bounds
-    const int owner = best & (kWaveSize - 1), slot = best >> 6;
-    float mine = 0.f;
-#pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) {
-      if (j == slot) {
-        mine = sc[j];
-        if (lane == owner) key[j] = 0u;          // taken: below every real key
-      }
-    }
-    const float w = row_lane(mine, owner);
-    if (lane == r) {
-      my_id = best;
-      my_w = w;
-    }
-  }
-  // Ascending expert id, stable in pick order: rank of lane's pick, then the inverse permutation.
-  int rank = 0;
-  for (int i = 0; i < top_k; ++i) {
-    const int oid = __builtin_amdgcn_readlane(my_id, i);
-    rank += (oid < my_id) || (oid == my_id && i < lane);
-  }
-  int src = 0;
-  for (int i = 0; i < top_k; ++i)
-    if (__builtin_amdgcn_readlane(rank, i) == lane) src = i;
-  const int sid = __shfl(my_id, src);
-  const float sw = __shfl(my_w, src);
-  float denom = 0.f;
-  for (int i = 0; i < top_k; ++i) denom += row_lane(sw, i);   // fp32 adds in id order
-  denom += 1e-20f;
-  float w = norm_topk ? (sw / denom) * scaling : sw * scaling;
-  if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) w = bf16_to_f32(f32_to_bf16(w));
-  out_id = sid;
-  out_w = w;
 }
 
 template <int kMode, int PER_LANE>

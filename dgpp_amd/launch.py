@@ -81,6 +81,23 @@ def launch_moe_router_select_order(scores, biased, ids, weights, order, cfg: Moe
                                                            _stream(stream)))
 
 
+def launch_moe_select_gate_up_swiglu(scores, biased, ids, weights, cfg: MoeConfig, tokens, x, x_stride, views, n_routed,
+                                     k_routed, act, act_stride, limit, stream=None):
+    """Extension: selection + routed FP8 gate/up in one launch (ids and weights are outputs)."""
+    _check(_lib.load().dgpp_launch_moe_select_gate_up_swiglu(_p(scores), _p(biased), _p(ids), _p(weights), C.addressof(cfg),
+                                                             tokens, _p(x), x_stride, _p(views), n_routed, k_routed, _p(act),
+                                                             act_stride, limit, _stream(stream)))
+
+
+def launch_moe_select_gate_up_swiglu_fp4(scores, biased, ids, weights, cfg: MoeConfig, tokens, x, x_stride, views, n_routed,
+                                         k_routed, act, act_stride, limit, stream=None, fp4_group=16):
+    """Extension: selection + routed NVFP4 / MXFP4 gate/up in one launch (ids and weights are outputs)."""
+    _check(_lib.load().dgpp_launch_moe_select_gate_up_swiglu_fp4(_p(scores), _p(biased), _p(ids), _p(weights),
+                                                                 C.addressof(cfg), tokens, _p(x), x_stride, _p(views),
+                                                                 n_routed, k_routed, _p(act), act_stride, limit,
+                                                                 _stream(stream), fp4_group))
+
+
 # ---- elementwise --------------------------------------------------------------------------------
 def launch_moe_swiglu_clamp(gate, up, out, n, limit, stream=None):
     _check(_lib.load().dgpp_launch_moe_swiglu_clamp(_p(gate), _p(up), _p(out), n, limit, _stream(stream)))

@@ -43,8 +43,12 @@ const char* dgpp_target_arch(void);
  * key 2: row steps per block of the slot launches (0 = automatic); key 3: 1 stages activations before
  * any weight load is issued (default: activation loads, first weight pass, LDS commit); key 4: 1 keeps
  * the layer driver on the two-launch down + accumulate form; key 5: 2 moves the GEMV launchers to the
- * matrix-core form. Outputs do not depend on keys 1 - 4; keys 0 and 5 change the fp32 summation order
- * (every GEMV launcher follows them alike, so the launchers stay bitwise twins of each other). */
+ * matrix-core form; key 6: 1 makes the layer driver compute the slot order for small decode batches too
+ * (default: batches of at most 64 routed slots find the sharers of an expert by ballot, no order);
+ * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
+ * blocks, dgpp_launch_moe_select_gate_up_swiglu). Outputs do not depend on keys 1 - 4, 6 and 7; keys 0 and
+ * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
+ * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);
 int dgpp_tune_get(int key);
 
@@ -206,6 +210,21 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
                               int k_routed, int n_shared, int k_shared, const uint8_t* sh_payload,
                               const float* sh_scales, float* out, int out_stride, int slots,
                               int top_k, void* stream, int sh_rs, int sh_cs);
+
+/* Extension (no counterpart in the reference): dgpp_launch_moe_router_select followed by the routed pass of
+ * dgpp_launch_moe_slot_gate_up_swiglu / _fp4 (order == NULL, no shared expert; slots = tokens * (top_k + 1)),
+ * same outputs bit for bit. For ONE token (n_experts <= 512, k <= 4096, 16-byte-aligned row) this is one launch:
+ * the first wavefront of every gate/up block repeats the selection in registers, block (0, 0) stores `ids` and
+ * `weights` for the launches that follow. Any other call runs the two launchers. */
+int dgpp_launch_moe_select_gate_up_swiglu(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                          const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                          const DgppMoeExpertView* views, int n_routed, int k_routed,
+                                          uint16_t* act, int act_stride, float limit, void* stream);
+int dgpp_launch_moe_select_gate_up_swiglu_fp4(const float* scores, const float* biased, int32_t* ids,
+                                              float* weights, const DgppMoeConfig* cfg, int tokens,
+                                              const uint16_t* x, size_t x_stride, const DgppMoeExpertView* views,
+                                              int n_routed, int k_routed, uint16_t* act, int act_stride,
+                                              float limit, void* stream, int fp4_group);
 
 /* ---- NVFP4 / MXFP4 decode-slot kernels ----------------------------------------------------------- */
 /* src/kernels/glm_moe_launch.hpp:392-399 */

@@ -126,6 +126,23 @@ inline void launch_moe_router_select_order(const float* scores, const float* bia
   detail::check(dgpp_launch_moe_router_select_order(scores, biased, ids, weights, order, &c, tokens,
                                                     shared_early ? 1 : 0, stream));
 }
+// Extension: selection + routed gate/up in one launch (see dgpp_amd.h).
+inline void launch_moe_select_gate_up_swiglu(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                             const GlmMoeConfig& cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                             const MoeExpertView* views, int n_routed, int k_routed, uint16_t* act,
+                                             int act_stride, float limit, hipStream_t stream) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_select_gate_up_swiglu(scores, biased, ids, weights, &c, tokens, x, x_stride, views, n_routed,
+                                                      k_routed, act, act_stride, limit, stream));
+}
+inline void launch_moe_select_gate_up_swiglu_fp4(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                                 const GlmMoeConfig& cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                                 const MoeExpertView* views, int n_routed, int k_routed, uint16_t* act,
+                                                 int act_stride, float limit, hipStream_t stream, int fp4_group = 16) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_select_gate_up_swiglu_fp4(scores, biased, ids, weights, &c, tokens, x, x_stride, views,
+                                                          n_routed, k_routed, act, act_stride, limit, stream, fp4_group));
+}
 inline void launch_moe_swiglu_clamp(const uint16_t* gate, const uint16_t* up, uint16_t* out, int64_t n, float limit,
                                     hipStream_t stream) {
   detail::check(dgpp_launch_moe_swiglu_clamp(gate, up, out, n, limit, stream));

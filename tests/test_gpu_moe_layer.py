@@ -103,4 +103,15 @@ def test_layer_from_given_scores_softmax(gpu):
     orc.oracle().orc_router_select(orc.p(l64), orc.p(l64), 1, T, E, K, 1.0, 1, orc.p(ids), orc.p(w))
     raw, _ = moe_data.orc_forward(p, ids, w)
     expert_budget(host(out, np.uint16), raw, "scores-driven layer")
+    # the selection as a launch of its own (bench switch 7) gives the same bits as the selection repeated in the
+    # gate/up blocks
+    out2 = dev_empty((T, H), np.uint16)
+    from dgpp_amd import _lib
+    _lib.load().dgpp_tune_set(7, 1)
+    try:
+        layer.enqueue_decode_scores(d.x, H, lg, lg, out2, T)
+        sync()
+    finally:
+        _lib.load().dgpp_tune_set(7, 0)
+    assert np.array_equal(host(out2, np.uint16), host(out, np.uint16))
     layer.close()

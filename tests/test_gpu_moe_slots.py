@@ -273,3 +273,47 @@ def test_token_major_down_accumulate_is_bitwise_the_two_launch_form(gpu, kind, E
     assert np.array_equal(hg.f32_to_bf16(host(out_f)), out), "fused f32 output"
     with pytest.raises(L.InvalidArgument):
         L.launch_moe_slot_down_accum_fp4(act_d, I, ids_d, d.views, H, I, T, 17, w_d, out_b, None, None, 16)
+
+
+@pytest.mark.parametrize("kind,mode,E,H,I,K,T", [("mxfp4", 1, 256, 1024, 256, 8, 1), ("mxfp4", 0, 64, 1152, 128, 8, 1),
+                                                 ("nvfp4", 0, 40, 640, 64, 4, 1), ("fp8", 1, 300, 384, 96, 8, 1),
+                                                 ("fp8", 0, 16, 512, 80, 2, 1), ("nvfp4", 1, 600, 1024, 64, 8, 1),
+                                                 ("nvfp4", 1, 512, 1024, 64, 16, 1), ("mxfp4", 0, 32, 1024, 64, 8, 4)])
+def test_select_gate_up_is_bitwise_select_then_gate_up(gpu, kind, mode, E, H, I, K, T):
+    """The one-launch extension (one token: the router selection repeated in every gate/up block) against
+    launch_moe_router_select followed by the routed gate/up launcher: the same ids, weights and activation rows,
+    including the calls it hands back to the two launchers (more than 512 experts, more than one token)."""
+    p = moe_data.make_problem(E, H, I, K, T, kind, 1300 + E + T, shared_kind=None, limit=7.0, std=0.05)
+    d = DeviceMoe(p)
+    rng = np.random.default_rng(11 * E + T)
+    scores = rng.uniform(0.05, 0.95, (T, E)).astype(np.float32) if mode == 0 else hg.bf16_to_f32(hg.normal_bf16(E + T, (T, E)))
+    biased = (scores + rng.normal(0, 0.05, (T, E))).astype(np.float32) if mode == 0 else scores
+    scores[0, : E // 2] = scores[0, 0]          # a row with many exact ties: lower id wins
+    if mode == 0:
+        biased[0] = scores[0]
+    cfg = L.make_config(H, I, E, K, router_mode=mode, routed_scaling_factor=1.0 if mode else 2.5, n_shared_experts=0)
+    slots = T * (K + 1)
+    s_d, b_d = dev(scores), dev(biased)
+    ids1, w1 = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32)
+    ids2, w2 = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32)
+    act1, act2 = dev_empty((slots, I), np.uint16), dev_empty((slots, I), np.uint16)
+    act1.zero_()
+    act2.zero_()
+    L.launch_moe_router_select(s_d, b_d, ids1, w1, cfg, T, None)
+    if kind == "fp8":
+        L.launch_moe_slot_gate_up_swiglu(d.x, H, ids1, None, d.views, I, H, 0, 0, None, None, None, None, act1, I, slots, K,
+                                         p.limit, None)
+        L.launch_moe_select_gate_up_swiglu(s_d, b_d, ids2, w2, cfg, T, d.x, H, d.views, I, H, act2, I, p.limit, None)
+    else:
+        L.launch_moe_slot_gate_up_swiglu_fp4(d.x, H, ids1, None, d.views, I, H, 0, 0, None, None, None, None, act1, I, slots,
+                                             K, p.limit, None, -1, d.fp4_group)
+        L.launch_moe_select_gate_up_swiglu_fp4(s_d, b_d, ids2, w2, cfg, T, d.x, H, d.views, I, H, act2, I, p.limit, None,
+                                               d.fp4_group)
+    sync()
+    assert np.array_equal(host(ids1), host(ids2)), "ids"
+    assert np.array_equal(host(w1).view(np.uint32), host(w2).view(np.uint32)), "weights"
+    assert np.array_equal(host(act1, np.uint16), host(act2, np.uint16)), "activation rows"
+    with pytest.raises(L.InvalidArgument):
+        L.launch_moe_select_gate_up_swiglu_fp4(s_d, b_d, ids2, w2, cfg, T, d.x, H, d.views, I, H, act2, I, p.limit, None, 8)
+    with pytest.raises(L.InvalidArgument):
+        L.launch_moe_select_gate_up_swiglu(s_d, None, ids2, w2, cfg, T, d.x, H, d.views, I, H, act2, I, p.limit, None)
