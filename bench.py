@@ -52,8 +52,8 @@ def parse():
     ap.add_argument("--eager", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
-    ap.add_argument("--configs", default="c1,c2,c4,c5", help="other BASELINE configurations to time beside the headline, "
-                    "comma separated out of c1,c2,c4,c5 ('' for none)")
+    ap.add_argument("--configs", default=None, help="other BASELINE configurations to time beside the headline, comma "
+                    "separated out of c1,c2,c4,c5 ('' for none; default: all four, none under --tune)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -425,8 +425,9 @@ def main():
         return res
 
     other_configs = {}
-    if not args.only and not args.tune:
-        for name in filter(None, args.configs.split(",")):
+    configs = args.configs if args.configs is not None else ("" if args.tune else "c1,c2,c4,c5")
+    if not args.only:
+        for name in filter(None, configs.split(",")):
             t0 = time.time()
             other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0

@@ -270,7 +270,8 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
 
 int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
             int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32, size_t out_stride,
-            int n, int k, void* stream, const char* who, bool mma = false, const int32_t* act_rows = nullptr) {
+            int n, int k, void* stream, const char* who, bool mma = false, const int32_t* act_rows = nullptr,
+            const float* gate_up_limit = nullptr) {
   if (max_rows <= 0) return fail_arg(std::string(who) + ": max_rows must be positive");
   if (which < 0 || which > 2) return fail_arg(std::string(who) + ": which must be 0, 1 or 2");
   const unsigned z_ext = rows_per_block > 0 ? static_cast<unsigned>((max_rows + rows_per_block - 1) / rows_per_block) : 1u;
@@ -289,6 +290,8 @@ int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegmen
   a.rows_per_block = rows_per_block > 0 ? rows_per_block : INT_MAX;
   a.group_rows = max_stage_rows(k);
   a.act_rows = act_rows;
+  a.gate_up = gate_up_limit != nullptr;
+  a.limit = gate_up_limit ? *gate_up_limit : 0.f;
   a.once = max_rows <= (mma ? kTileCols : a.group_rows);   // every segment in one pass over its expert
   if (mma) return finish(launch_grouped_mma(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
   return finish(launch_grouped(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
@@ -836,13 +839,14 @@ int dgpp_launch_dense_mma_fp4_f32(const uint16_t* act, size_t act_stride, const 
 
 static int grouped_mma_fp8(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
                            int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
-                           size_t out_stride, int n, int k, void* stream, const int32_t* act_rows) {
+                           size_t out_stride, int n, int k, void* stream, const int32_t* act_rows,
+                           const float* gate_up_limit = nullptr) {
   const char* who = "moe grouped mma";
   if (n_segs <= 0 || n <= 0) return DGPP_OK;
   if (!act || !segs || !views || !out) return fail_arg(std::string(who) + ": null pointer");
   if (k <= 0 || k % 16 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 16");
   return grouped(kFmtFp8F32, act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_f32,
-                 out_stride, n, k, stream, who, true, act_rows);
+                 out_stride, n, k, stream, who, true, act_rows, gate_up_limit);
 }
 int dgpp_launch_moe_grouped_mma_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
                                      int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
@@ -859,14 +863,30 @@ int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, cons
 }
 static int grouped_mma_fp4(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
                            int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
-                           size_t out_stride, int n, int k, void* stream, const int32_t* act_rows, int fp4_group) {
+                           size_t out_stride, int n, int k, void* stream, const int32_t* act_rows, int fp4_group,
+                           const float* gate_up_limit = nullptr) {
   const char* who = "moe grouped mma fp4";
   if (n_segs <= 0 || n <= 0) return DGPP_OK;
   if (!act || !segs || !views || !out) return fail_arg(std::string(who) + ": null pointer");
   if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
   if (k <= 0 || k % 32 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 32");
   return grouped(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
-                 which, out, out_f32, out_stride, n, k, stream, who, true, act_rows);
+                 which, out, out_f32, out_stride, n, k, stream, who, true, act_rows, gate_up_limit);
+}
+int dgpp_launch_moe_grouped_mma_gate_up_swiglu(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs,
+                                               int n_segs, int max_rows, int rows_per_block, const DgppMoeExpertView* views,
+                                               uint16_t* out, size_t out_stride, int n, int k, float limit, void* stream,
+                                               const int32_t* act_rows) {
+  return grouped_mma_fp8(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, 0, out, 0, out_stride, n, k, stream,
+                         act_rows, &limit);
+}
+int dgpp_launch_moe_grouped_mma_gate_up_swiglu_fp4(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs,
+                                                   int n_segs, int max_rows, int rows_per_block,
+                                                   const DgppMoeExpertView* views, uint16_t* out, size_t out_stride, int n,
+                                                   int k, float limit, void* stream, const int32_t* act_rows,
+                                                   int fp4_group) {
+  return grouped_mma_fp4(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, 0, out, 0, out_stride, n, k, stream,
+                         act_rows, fp4_group, &limit);
 }
 int dgpp_launch_moe_grouped_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
                                          int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,

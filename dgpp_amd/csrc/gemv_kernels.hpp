@@ -520,6 +520,8 @@ struct GroupedArgs {
   int group_rows;      // activation rows staged per pass (<= kMaxActRows)
   const int32_t* act_rows;  // matrix-core form only, nullable: activation row of each segment row
   int once;                 // every segment fits one pass over its expert (nontemporal loads)
+  int gate_up;              // matrix-core form only: gate and up rows + SwiGLU in one launch (`which` unused, bf16 out)
+  float limit;              // the SwiGLU clamp of that form
 };
 
 template <int FMT, int NB, bool NT>
@@ -664,10 +666,12 @@ hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipS
   const dim3 grid(static_cast<unsigned>((a.n + 63) / 64), static_cast<unsigned>(n_segs), static_cast<unsigned>(z_ext));
   hipError_t err = hipSuccess;
   dispatch_bool(a.once != 0, [&](auto ntc) {
-    auto kern = mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value>;
-    constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
-    err = ensure_lds(kern, lds);
-    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g);
+    dispatch_bool(a.gate_up != 0, [&](auto guc) {
+      auto kern = mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value, decltype(guc)::value>;
+      constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
+      err = ensure_lds(kern, lds);
+      if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g);
+    });
   });
   return err != hipSuccess ? err : hipGetLastError();
 }
@@ -762,7 +766,8 @@ inline int run_cap_for(const SlotArgs& a, int max_run) {
   if (a.order == nullptr && !a.match) return 1;   // slots in layout order and no way to find the sharers
   const int tuned = tune_get(kTuneSlotRun);
   int cap = tuned > 0 ? tuned : max_run;
-  while (cap > 1 && (cap > max_run || stage_bytes(cap, a.k) > 16 * 1024)) --cap;
+  // 32 KB of staged rows keeps five blocks on a CU; two slots per weight pass also halve the decode work per slot
+  while (cap > 1 && (cap > max_run || stage_bytes(cap, a.k) > 32 * 1024)) --cap;
   return cap;
 }
 

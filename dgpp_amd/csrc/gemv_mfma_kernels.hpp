@@ -158,15 +158,17 @@ __global__ void fold_parts_kernel(const float* __restrict__ partials, int parts,
     static_cast<uint16_t*>(out)[at] = f32_to_bf16(x);
 }
 
-template <int FMT, int NB, bool NT>
+// GU: the block computes its rows of the segment's gate AND up matrices (two walks over K, the same
+// activations) and stores SwiGLU(bf16(gate), bf16(up)) — the bits of two launches and the elementwise kernel.
+template <int FMT, int NB, bool NT, bool GU>
 __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedArgs a, MGeom g) {
   extern __shared__ uint4 lds[];
   const DgppMoeSegment seg = a.segs[blockIdx.y];
   const int z0 = static_cast<int>(blockIdx.z) * a.rows_per_block;
   if (z0 >= seg.rows) return;
   const int z1 = min(seg.rows, z0 + a.rows_per_block);
-  const float* gp = nullptr;
-  const MatRef mat = mat_of_view<FMT>(a.views[seg.expert * 3 + a.which], &gp);
+  const float *gp = nullptr, *gp2 = nullptr;
+  const MatRef mat = mat_of_view<FMT>(a.views[seg.expert * 3 + (GU ? 0 : a.which)], &gp);
   const float divisor = load_divisor<FMT>(gp);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
   const int row0 = (static_cast<int>(blockIdx.x) * kWavesPerBlock + wave) * kGroupRows;
@@ -175,9 +177,25 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
     const int mt = min(kTileCols, z1 - c0);
     f32x4_t sum;
     const size_t first = static_cast<size_t>(seg.row0 + c0);
-    block_rows_mfma<FMT, NB, NT>(mat, a.act_rows ? a.act : a.act + first * a.act_stride, a.act_stride,
-                             a.act_rows ? a.act_rows + first : nullptr, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum);
-    store_tile<FMT>(sum, divisor, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, c < mt);
+    const uint16_t* act = a.act_rows ? a.act : a.act + first * a.act_stride;
+    const int32_t* rows = a.act_rows ? a.act_rows + first : nullptr;
+    block_rows_mfma<FMT, NB, NT>(mat, act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum);
+    if constexpr (GU) {
+      const MatRef mat_up = mat_of_view<FMT>(a.views[seg.expert * 3 + 1], &gp2);
+      const float divisor_up = load_divisor<FMT>(gp2);
+      f32x4_t sum_up;
+      block_rows_mfma<FMT, NB, NT>(mat_up, act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum_up);
+      if (c < mt) {
+        uint16_t* out = static_cast<uint16_t*>(a.out) + (first + c) * a.out_stride;
+        const int r = row0 + (lane >> 4) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (r + i < a.n)
+            out[r + i] = swiglu_bf16(finish_dot<FMT>(sum[i], divisor), finish_dot<FMT>(sum_up[i], divisor_up), a.limit);
+      }
+    } else {
+      store_tile<FMT>(sum, divisor, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, c < mt);
+    }
   }
 }
 

@@ -290,16 +290,13 @@ void GlmMoeLayer::enqueue_prefill_routed(const uint16_t* x, size_t x_stride, con
   const int tk = tokens * K;
   launch_moe_segment(ids, tokens, K, E, d_rows_, d_slot_row_, d_segs_, stream);
   const int max_rows = tokens;
-  if (w_.format == GlmExpertFormat::Fp8) {
-    launch_moe_grouped_mma_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 0, d_gate_, I, I, H, stream, d_rows_);
-    launch_moe_grouped_mma_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 1, d_up_, I, I, H, stream, d_rows_);
-  } else {
-    launch_moe_grouped_mma_fp4_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 0, d_gate_, I, I, H, stream, d_rows_,
-                                    fp4_group_);
-    launch_moe_grouped_mma_fp4_bf16(x, x_stride, d_segs_, E, max_rows, 0, d_views_, 1, d_up_, I, I, H, stream, d_rows_,
-                                    fp4_group_);
-  }
-  launch_moe_swiglu_clamp(d_gate_, d_up_, d_slot_act_, static_cast<int64_t>(tk) * I, cfg_.swiglu_limit, stream);
+  // gate + up + SwiGLU in one launch (the bits of the two grouped launches and the elementwise kernel)
+  if (w_.format == GlmExpertFormat::Fp8)
+    launch_moe_grouped_mma_gate_up_swiglu(x, x_stride, d_segs_, E, max_rows, 0, d_views_, d_slot_act_, I, I, H,
+                                          cfg_.swiglu_limit, stream, d_rows_);
+  else
+    launch_moe_grouped_mma_gate_up_swiglu_fp4(x, x_stride, d_segs_, E, max_rows, 0, d_views_, d_slot_act_, I, I, H,
+                                              cfg_.swiglu_limit, stream, d_rows_, fp4_group_);
   if (w_.format == GlmExpertFormat::Fp8)
     launch_moe_grouped_mma_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream);
   else

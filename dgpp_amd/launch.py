@@ -391,6 +391,22 @@ def launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per
                                                        _p(act_rows)))
 
 
+def launch_moe_grouped_mma_gate_up_swiglu(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, out, out_stride,
+                                          n, k, limit, stream=None, act_rows=None):
+    """Extension: grouped FP8 gate + up + SwiGLU in one matrix-core launch."""
+    _check(_lib.load().dgpp_launch_moe_grouped_mma_gate_up_swiglu(_p(act), act_stride, _p(segs), n_segs, max_rows,
+                                                                  rows_per_block, _p(views), _p(out), out_stride, n, k,
+                                                                  limit, _stream(stream), _p(act_rows)))
+
+
+def launch_moe_grouped_mma_gate_up_swiglu_fp4(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, out,
+                                              out_stride, n, k, limit, stream=None, act_rows=None, fp4_group=16):
+    """Extension: grouped NVFP4 / MXFP4 gate + up + SwiGLU in one matrix-core launch."""
+    _check(_lib.load().dgpp_launch_moe_grouped_mma_gate_up_swiglu_fp4(_p(act), act_stride, _p(segs), n_segs, max_rows,
+                                                                      rows_per_block, _p(views), _p(out), out_stride, n,
+                                                                      k, limit, _stream(stream), _p(act_rows), fp4_group))
+
+
 def launch_moe_grouped_mma_fp4_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out, out_stride,
                                     n, k, stream=None, act_rows=None, fp4_group=16, tile_rows=64):
     _check(_lib.load().dgpp_launch_moe_grouped_mma_fp4_bf16(_p(act), act_stride, _p(segs), n_segs, max_rows, rows_per_block,

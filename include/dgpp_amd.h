@@ -328,6 +328,19 @@ int dgpp_launch_moe_grouped_mma_bf16(const uint16_t* act, size_t act_stride, con
 int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
                                     int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which, float* out,
                                     size_t out_stride, int n, int k, void* stream, const int32_t* act_rows);
+/* Extension (no counterpart in the reference): dgpp_launch_moe_grouped_mma{,_fp4}_bf16 for which = 0 and which = 1
+ * followed by dgpp_launch_moe_swiglu_clamp, in one launch: a block walks its rows of the segment's gate matrix, then
+ * of its up matrix, against the same activation rows and stores SwiGLU(bf16(gate), bf16(up)). Same bits as the
+ * three launches. out: [sum of segment rows, out_stride] bf16 activation rows. */
+int dgpp_launch_moe_grouped_mma_gate_up_swiglu(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs,
+                                               int n_segs, int max_rows, int rows_per_block,
+                                               const DgppMoeExpertView* views, uint16_t* out, size_t out_stride,
+                                               int n, int k, float limit, void* stream, const int32_t* act_rows);
+int dgpp_launch_moe_grouped_mma_gate_up_swiglu_fp4(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs,
+                                                   int n_segs, int max_rows, int rows_per_block,
+                                                   const DgppMoeExpertView* views, uint16_t* out, size_t out_stride,
+                                                   int n, int k, float limit, void* stream, const int32_t* act_rows,
+                                                   int fp4_group);
 int dgpp_launch_moe_grouped_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
                                          int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which,
                                          uint16_t* out, size_t out_stride, int n, int k, void* stream,

@@ -360,6 +360,22 @@ inline void launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, c
   detail::check(dgpp_launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                                 out_stride, n, k, stream, act_rows));
 }
+// Extension: grouped gate + up + SwiGLU in one matrix-core launch (see dgpp_amd.h).
+inline void launch_moe_grouped_mma_gate_up_swiglu(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
+                                                  int max_rows, int rows_per_block, const MoeExpertView* views,
+                                                  uint16_t* out, size_t out_stride, int n, int k, float limit,
+                                                  hipStream_t stream, const int32_t* act_rows = nullptr) {
+  detail::check(dgpp_launch_moe_grouped_mma_gate_up_swiglu(act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
+                                                           out, out_stride, n, k, limit, stream, act_rows));
+}
+inline void launch_moe_grouped_mma_gate_up_swiglu_fp4(const uint16_t* act, size_t act_stride, const MoeSegment* segs,
+                                                      int n_segs, int max_rows, int rows_per_block,
+                                                      const MoeExpertView* views, uint16_t* out, size_t out_stride, int n,
+                                                      int k, float limit, hipStream_t stream,
+                                                      const int32_t* act_rows = nullptr, int fp4_group = kFp4Group) {
+  detail::check(dgpp_launch_moe_grouped_mma_gate_up_swiglu_fp4(act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
+                                                               out, out_stride, n, k, limit, stream, act_rows, fp4_group));
+}
 inline void launch_moe_grouped_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
                                             int max_rows, int rows_per_block, const MoeExpertView* views, int which,
                                             uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream,

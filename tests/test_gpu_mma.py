@@ -132,6 +132,38 @@ def test_grouped_mma_is_bitwise_the_dense_mma_per_segment_with_and_without_the_g
         check(np.ascontiguousarray(a[r0:r0 + cnt]), raw, f"grouped mma {kind} segment {e}")
 
 
+@pytest.mark.parametrize("kind,limit", [("fp8", 7.0), ("nvfp4", float("inf")), ("mxfp4", 0.75)])
+def test_grouped_mma_gate_up_swiglu_is_bitwise_the_three_launches(gpu, kind, limit):
+    """The one-launch extension (gate rows, up rows, SwiGLU in the matrix-core grouped kernel) against the two grouped
+    launches and launch_moe_swiglu_clamp, with the folded gather and with a z split."""
+    E, H, I, K, T = 5, 640, 160 if kind != "fp8" else 144, 2, 21
+    p = moe_data.make_problem(E, H, I, K, T, kind, 77, shared_kind=None, limit=limit, std=0.05)
+    d = DeviceMoe(p)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    ids_d = dev(ids)
+    rows_d, sr_d, segs_d = dev_empty(T * K + T, np.int32), dev_empty(T * K, np.int32), dev_empty((E + 1, 3), np.int32)
+    L.launch_moe_segment(ids_d, T, K, E, rows_d, sr_d, segs_d, None)
+    gate, up, want, got, got_z = (dev_empty((T * K, I), np.uint16) for _ in range(5))
+    if kind == "fp8":
+        L.launch_moe_grouped_mma_bf16(d.x, H, segs_d, E, T, 0, d.views, 0, gate, I, I, H, None, rows_d)
+        L.launch_moe_grouped_mma_bf16(d.x, H, segs_d, E, T, 0, d.views, 1, up, I, I, H, None, rows_d)
+        L.launch_moe_grouped_mma_gate_up_swiglu(d.x, H, segs_d, E, T, 0, d.views, got, I, I, H, limit, None, rows_d)
+        L.launch_moe_grouped_mma_gate_up_swiglu(d.x, H, segs_d, E, T, 16, d.views, got_z, I, I, H, limit, None, rows_d)
+    else:
+        L.launch_moe_grouped_mma_fp4_bf16(d.x, H, segs_d, E, T, 0, d.views, 0, gate, I, I, H, None, rows_d, d.fp4_group)
+        L.launch_moe_grouped_mma_fp4_bf16(d.x, H, segs_d, E, T, 0, d.views, 1, up, I, I, H, None, rows_d, d.fp4_group)
+        L.launch_moe_grouped_mma_gate_up_swiglu_fp4(d.x, H, segs_d, E, T, 0, d.views, got, I, I, H, limit, None, rows_d,
+                                                    d.fp4_group)
+        L.launch_moe_grouped_mma_gate_up_swiglu_fp4(d.x, H, segs_d, E, T, 16, d.views, got_z, I, I, H, limit, None, rows_d,
+                                                    d.fp4_group)
+    L.launch_moe_swiglu_clamp(gate, up, want, T * K * I, limit, None)
+    sync()
+    assert np.array_equal(host(got, np.uint16), host(want, np.uint16))
+    assert np.array_equal(host(got_z, np.uint16), host(want, np.uint16)), "the z split does not change a row"
+    with pytest.raises(L.InvalidArgument):
+        L.launch_moe_grouped_mma_gate_up_swiglu(d.x, H, segs_d, E, 0, 0, d.views, got, I, I, H, limit, None, rows_d)
+
+
 @pytest.mark.parametrize("kind", ["fp8", "nvfp4", "mxfp4"])
 def test_prefill_path_matches_oracle_and_gemv_launchers_on_the_matrix_core_are_its_twins(gpu, kind):
     """The layer's matrix-core grouped path against the oracle's layer budget; then, with the bench switch that
