@@ -3,7 +3,7 @@
 
 A "step" is one pass of the hot path over one batch: one MXFP4 MoE decode layer (router top-8
 selection from given logits -> fused gate/up + SwiGLU -> down + ordered accumulation: three
-launches) at the BASELINE shape (256 experts, hidden 4096, expert intermediate 1024, top-8,
+launches) at the headline shape (256 experts, hidden 4096, expert intermediate 1024, top-8,
 no shared expert), T tokens. Consecutive steps walk DIFFERENT layers' weights (a ring of
 `--layers` full layers, as a model's decode step walks its MoE layers), so every step streams its
 experts from HBM, not from the 256 MB Infinity Cache / L2. The steps are captured once in a HIP
@@ -28,7 +28,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0
-E, H, I, K = 256, 4096, 1024, 8          # BASELINE config 3 (MXFP4 MoE decode layer)
+E, H, I, K = 256, 4096, 1024, 8          # the headline configuration (MXFP4 MoE decode layer)
 EXPERT_BYTES = 3 * I * H // 2 + 3 * I * H // 32          # payload + e8m0 scales of gate, up, down
 GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
 # HBM-side bytes per launch of the two GEMV kernels at the default workload (T = 8, 256 experts), from
@@ -45,14 +45,14 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--tokens", type=int, default=8, help="decode batch of the headline number (1..8)")
     ap.add_argument("--layers", type=int, default=16, help="ring of distinct layers' weights (cold-cache rotation)")
-    ap.add_argument("--experts", type=int, default=E, help="experts per layer (256 = the BASELINE shape)")
+    ap.add_argument("--experts", type=int, default=E, help="experts per layer (256 = the headline shape)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="'layer', 'gate_up' or 'down': run only that timed graph (for profiling)")
     ap.add_argument("--no-others", action="store_true", help="skip the T=1/4/8 side measurements")
     ap.add_argument("--eager", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
-    ap.add_argument("--configs", default=None, help="other BASELINE configurations to time beside the headline, comma "
+    ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
                     "separated out of c1,c2,c4,c5 ('' for none; default: all four, none under --tune)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
@@ -237,7 +237,7 @@ def main():
             if t != T:
                 others[f"T{t}"] = measure(t, args.steps, args.warmup)
 
-    # ---- the other BASELINE configurations (reported beside the headline, never part of `value`) ------------
+    # ---- the other benchmark configurations (reported beside the headline, never part of `value`) -----------
     def ring_copies(tensors, nbytes, want=2 * 256 * 2**20 + 64 * 2**20):
         """Device copies of a weight set so that consecutive timed launches never find it in the caches."""
         n = max(2, -(-want // nbytes))

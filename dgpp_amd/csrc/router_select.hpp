@@ -63,12 +63,21 @@ __device__ __forceinline__ void select_token(const float* __restrict__ scores, c
                                              int& out_id, float& out_w) {
   float sc[PER_LANE];
   uint32_t key[PER_LANE];
+  {
+    // every load is issued before the first is waited for (dead slots re-read the last expert): one trip to memory
+    float raw_s[PER_LANE], raw_b[PER_LANE];
 #pragma unroll
-  for (int j = 0; j < PER_LANE; ++j) {
-    const int e = lane + j * kWaveSize;
-    const bool live = e < n_experts;
-    sc[j] = live ? scores[e] : -INFINITY;
-    key[j] = live ? order_key(biased[e]) : 0u;
+    for (int j = 0; j < PER_LANE; ++j) {
+      const int e = min(lane + j * kWaveSize, n_experts - 1);
+      raw_s[j] = scores[e];
+      raw_b[j] = biased[e];
+    }
+#pragma unroll
+    for (int j = 0; j < PER_LANE; ++j) {
+      const bool live = lane + j * kWaveSize < n_experts;
+      sc[j] = live ? raw_s[j] : -INFINITY;
+      key[j] = live ? order_key(raw_b[j]) : 0u;
+    }
   }
   if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
     float m = -INFINITY;

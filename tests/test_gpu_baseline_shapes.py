@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their FULL shapes on the GPU: oracle checks where the CPU
+"""The five benchmark configurations at their FULL shapes on the GPU: oracle checks where the CPU
 finishes in seconds (whole outputs for C1 / C3 / C4, row and token samples for C2 / C5) plus
 size-independent properties (rows independent of the batch, slot path == grouped path, bf16(f32) ==
 bf16 epilogue). Only experts that the seeded routing selects are materialised; the remaining table

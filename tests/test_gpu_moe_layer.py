@@ -1,6 +1,6 @@
 """The C++ host layer driver (the reference's GlmMoeLayer counterpart) end to end against the oracle,
 at small shapes with every path (router from hidden rows, from given scores, given routes; decode
-slots and grouped), plus the BASELINE layer shapes through size-independent properties."""
+slots and grouped), plus the benchmark's layer shapes through size-independent properties."""
 import ctypes as C
 
 import numpy as np
