@@ -186,6 +186,12 @@ def load() -> C.CDLL:
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `python -m dgpp_amd.build` "
             "(there is no CPU fallback for the HIP path)")
+    # One HIP runtime per process: PyTorch ships its own copy, and a process that uses both (tests, the bench)
+    # must let PyTorch load it first; this library then binds to the copy already in the process.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(str(LIB_PATH))
     for name, (res, args) in {**SIGNATURES, **LAYER_SIGNATURES}.items():
         fn = getattr(lib, name)
