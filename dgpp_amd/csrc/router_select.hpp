@@ -49,6 +49,23 @@ __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b 
 __device__ __forceinline__ uint32_t lane_u32(uint32_t v, int lane) {
   return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), lane));
 }
+// Wave-wide max / min of one value per lane, the same in every lane on return: a butterfly inside each row of
+// 16 lanes, then row 0 -> 1 and 2 -> 3, then row 1 -> 2, 3 (row broadcasts), and lane 63 read back.
+template <bool kMax>
+__device__ __forceinline__ uint32_t wave_reduce_u32(uint32_t v) {
+  auto op = [](uint32_t a, uint32_t b) { return kMax ? (a > b ? a : b) : (a < b ? a : b); };
+  v = op(v, dpp_u32<0xB1>(v));
+  v = op(v, dpp_u32<0x4E>(v));
+  v = op(v, dpp_u32<0x141>(v));
+  v = op(v, dpp_u32<0x140>(v));
+  const int i = static_cast<int>(v);
+  v = op(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(i, i, 0x142, 0xA, 0xF, false)));   // row_bcast:15 into rows 1, 3
+  const int k = static_cast<int>(v);
+  v = op(v, static_cast<uint32_t>(__builtin_amdgcn_update_dpp(k, k, 0x143, 0xC, 0xF, false)));   // row_bcast:31 into rows 2, 3
+  return lane_u32(v, 63);
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) { return wave_reduce_u32<true>(v); }
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) { return wave_reduce_u32<false>(v); }
 __device__ __forceinline__ uint32_t order_key(float v) {
   if (v != v) return 0u;                       // NaN: below every real key
   const uint32_t u = f32_bits(v + 0.0f);       // -0 -> +0
@@ -94,41 +111,28 @@ __device__ __forceinline__ void select_token(const float* __restrict__ scores, c
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) sc[j] = sc[j] / sum;
   }
-  // Pick r lands in lane r. A round takes the wave-wide maximum key (one DPP max per step), then the
-  // LOWEST expert id among the lanes and slots that hold it: slot-major ids (e = lane + 64 * slot),
-  // so the first slot with a match wins and, inside it, the lowest matching lane.
+  // Pick r lands in lane r. A round is two wave-wide reductions on the vector side: the maximum key, then the
+  // LOWEST expert id among the lanes and slots that hold it (ids are slot-major, e = lane + 64 * slot).
   int my_id = INT_MAX;
   float my_w = 0.f;
   for (int r = 0; r < top_k; ++r) {
     uint32_t m = key[0];
 #pragma unroll
     for (int j = 1; j < PER_LANE; ++j) m = m > key[j] ? m : key[j];
-    m = umax(m, dpp_u32<0xB1>(m));
-    m = umax(m, dpp_u32<0x4E>(m));
-    m = umax(m, dpp_u32<0x141>(m));
-    m = umax(m, dpp_u32<0x140>(m));
-    const uint32_t top = umax(umax(lane_u32(m, 0), lane_u32(m, 16)), umax(lane_u32(m, 32), lane_u32(m, 48)));
-    int best = 0;
-    bool found = false;
+    const uint32_t top = wave_max_u32(m);
+    uint32_t cand = 0xFFFFFFFFu;
 #pragma unroll
-    for (int j = 0; j < PER_LANE; ++j) {
-      const uint64_t hit = __builtin_amdgcn_ballot_w64(key[j] == top);
-      if (!found && hit != 0) {
-        best = j * kWaveSize + __builtin_ctzll(hit);
-        found = true;
-      }
-    }
+    for (int j = PER_LANE - 1; j >= 0; --j) cand = key[j] == top ? static_cast<uint32_t>(lane + j * kWaveSize) : cand;
+    int best = static_cast<int>(wave_min_u32(cand));
     if (top == 0u || best >= n_experts) best = 0;   // a row of NaN keys: stay in bounds
-    const int owner = best & (kWaveSize - 1), slot = best >> 6;
     float mine = 0.f;
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) {
-      if (j == slot) {
-        mine = sc[j];
-        if (lane == owner) key[j] = 0u;          // taken: below every real key
-      }
+      const bool hit = lane + j * kWaveSize == best;
+      mine = hit ? sc[j] : mine;
+      key[j] = hit ? 0u : key[j];                   // taken: below every real key
     }
-    const float w = row_lane(mine, owner);
+    const float w = row_lane(mine, best & (kWaveSize - 1));
     if (lane == r) {
       my_id = best;
       my_w = w;
