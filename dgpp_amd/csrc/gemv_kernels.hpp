@@ -778,6 +778,7 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
   int steps = pick_steps(per_slot * a.slots);
+  if (a.once && a.slots > a.top_k + 1) steps = 2;   // a decode batch of 2 - 8 tokens: measured best (one token: 1)
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
   const int cap = run_cap_for(a, kGateUpRun);
@@ -865,7 +866,7 @@ hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipStream_t stream) {
   const int rpw = kWave >> g.l2;
   const long long wave_steps = static_cast<long long>((a.n + rpw - 1) / rpw) * a.tokens * a.top_k;
   int steps = static_cast<int>(wave_steps / 16384);
-  steps = steps < 1 ? 1 : (steps > 8 ? 8 : steps);
+  steps = steps < 2 ? 2 : (steps > 8 ? 8 : steps);   // two row groups per wavefront measured best from one token on
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const int rows_per_block = rpw * steps;
   const dim3 grid(static_cast<unsigned>((a.n + rows_per_block - 1) / rows_per_block), static_cast<unsigned>(a.tokens));
