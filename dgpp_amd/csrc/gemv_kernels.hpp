@@ -734,7 +734,8 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
   const RowGeom g = geom_for<FMT>(a.k);
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long block_steps = (a.n + rows_per_step - 1) / rows_per_step;
-  const int steps = pick_steps(block_steps);
+  int steps = pick_steps(block_steps);
+  if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((block_steps + steps - 1) / steps));
   const size_t lds = stage_bytes(a.m, a.k);
   hipError_t err = hipSuccess;
