@@ -271,7 +271,7 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
 int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
             int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32, size_t out_stride,
             int n, int k, void* stream, const char* who, bool mma = false, const int32_t* act_rows = nullptr,
-            const float* gate_up_limit = nullptr) {
+            const float* gate_up_limit = nullptr, void* out_up = nullptr) {
   if (max_rows <= 0) return fail_arg(std::string(who) + ": max_rows must be positive");
   if (which < 0 || which > 2) return fail_arg(std::string(who) + ": which must be 0, 1 or 2");
   const unsigned z_ext = rows_per_block > 0 ? static_cast<unsigned>((max_rows + rows_per_block - 1) / rows_per_block) : 1u;
@@ -290,8 +290,9 @@ int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegmen
   a.rows_per_block = rows_per_block > 0 ? rows_per_block : INT_MAX;
   a.group_rows = max_stage_rows(k);
   a.act_rows = act_rows;
-  a.gate_up = gate_up_limit != nullptr;
+  a.gate_up = out_up ? 2 : (gate_up_limit != nullptr ? 1 : 0);
   a.limit = gate_up_limit ? *gate_up_limit : 0.f;
+  a.out_up = out_up;
   a.once = max_rows <= (mma ? kTileCols : a.group_rows);   // every segment in one pass over its expert
   if (mma) return finish(launch_grouped_mma(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
   return finish(launch_grouped(fmt, a, n_segs, static_cast<int>(z_ext), as_stream(stream)), who);
@@ -737,7 +738,7 @@ int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, 
 // ---- matrix-core launchers (src/kernels/glm_moe_launch.hpp:103-125, :311-345; src/kernels/mma_gemv.hpp:65-85) -----
 static int dense_mma(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,
                      int out_f32, size_t out_stride, int m, int n, int k, void* ws, size_t ws_bytes, void* stream,
-                     const char* who) {
+                     const char* who, const uint16_t* act_up = nullptr, float limit = 0.f) {
   if (out_stride == 0) out_stride = static_cast<size_t>(n);
   if (out_stride < static_cast<size_t>(n)) return fail_arg(std::string(who) + ": output row stride narrower than n");
   if ((m + kTileCols - 1) / kTileCols > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
@@ -753,12 +754,15 @@ static int dense_mma(int fmt, const uint16_t* act, size_t act_stride, const MatR
   a.n = n;
   a.k = k;
   a.once = m <= kTileCols;   // one activation tile: one pass over the weights
+  a.act_up = act_up;
+  a.limit = limit;
   return finish(launch_dense_mma(fmt, a, static_cast<float*>(ws), ws_bytes, as_stream(stream)), who);
 }
 
 static int dense_mma_fp8(const uint16_t* act, size_t act_stride, const uint8_t* payload, const void* scales, int e8m0,
                          void* out, int out_f32, int m, int n, int k, size_t out_stride, int rs, int cs, void* ws,
-                         size_t ws_bytes, void* stream, const char* who) {
+                         size_t ws_bytes, void* stream, const char* who, const uint16_t* act_up = nullptr,
+                         float limit = 0.f) {
   if (m <= 0 || n <= 0) return DGPP_OK;
   if (!act || !payload || !scales || !out) return fail_arg(std::string(who) + ": null pointer");
   const bool row_grid = rs == 0 && cs >= 4;
@@ -767,7 +771,18 @@ static int dense_mma_fp8(const uint16_t* act, size_t act_stride, const uint8_t* 
   if (k <= 0 || !fp8_shape_ok(payload, k))
     return fail_arg(std::string(who) + ": k must be a positive multiple of 16 with a 16-byte aligned payload");
   return dense_mma(e8m0 ? kFmtFp8E8M0 : kFmtFp8F32, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, out,
-                   out_f32, out_stride, m, n, k, ws, ws_bytes, stream, who);
+                   out_f32, out_stride, m, n, k, ws, ws_bytes, stream, who, act_up, limit);
+}
+int dgpp_launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t* up, float limit, size_t act_stride,
+                                        const uint8_t* w, const float* scales, float* out, int m, int n, int k,
+                                        size_t out_stride, int rs, int cs, void* stream) {
+  const char* who = "mma_gemv_fp8_swiglu";
+  if (m > 0 && n > 0) {
+    if (!gate || !up) return fail_arg(std::string(who) + ": null pointer");
+    if (((reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up)) & 15u) != 0 || (act_stride & 7u) != 0)
+      return fail_arg(std::string(who) + ": gate and up rows must be 16-byte aligned");
+  }
+  return dense_mma_fp8(gate, act_stride, w, scales, 0, out, 1, m, n, k, out_stride, rs, cs, nullptr, 0, stream, who, up, limit);
 }
 int dgpp_launch_dense_mma_bf16(const uint16_t* act, size_t act_stride, const uint8_t* payload, const float* scales,
                                uint16_t* out, int m, int n, int k, void* stream, size_t out_stride) {
@@ -864,14 +879,31 @@ int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, cons
 static int grouped_mma_fp4(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs, int max_rows,
                            int rows_per_block, const DgppMoeExpertView* views, int which, void* out, int out_f32,
                            size_t out_stride, int n, int k, void* stream, const int32_t* act_rows, int fp4_group,
-                           const float* gate_up_limit = nullptr) {
+                           const float* gate_up_limit = nullptr, void* out_up = nullptr) {
   const char* who = "moe grouped mma fp4";
   if (n_segs <= 0 || n <= 0) return DGPP_OK;
   if (!act || !segs || !views || !out) return fail_arg(std::string(who) + ": null pointer");
   if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
   if (k <= 0 || k % 32 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 32");
   return grouped(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, segs, n_segs, max_rows, rows_per_block, views,
-                 which, out, out_f32, out_stride, n, k, stream, who, true, act_rows, gate_up_limit);
+                 which, out, out_f32, out_stride, n, k, stream, who, true, act_rows, gate_up_limit, out_up);
+}
+/* src/kernels/glm_moe.cu:4809-4823: one segment read from the device, the grouped kernel's chain. */
+int dgpp_launch_dense_mma_fp4_prod_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
+                                        const DgppMoeExpertView* views, int which, uint16_t* out, int m, int n, int k,
+                                        void* stream, int fp4_group) {
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  return grouped_mma_fp4(act, act_stride, seg, 1, m, 0, views, which, out, 0, static_cast<size_t>(n), n, k, stream, nullptr,
+                         fp4_group);
+}
+/* src/kernels/dense_fp4_decode.cu:310-319: gate and up of one segment; one launch here, the bits of two prod launches. */
+int dgpp_launch_dense_mma_fp4_gate_up_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
+                                           const DgppMoeExpertView* views, uint16_t* gate, uint16_t* up, int m, int n,
+                                           int k, void* stream, int fp4_group) {
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  if (!up) return fail_arg("dense mma fp4 gate_up: null pointer");
+  return grouped_mma_fp4(act, act_stride, seg, 1, m, 0, views, 0, gate, 0, static_cast<size_t>(n), n, k, stream, nullptr,
+                         fp4_group, nullptr, up);
 }
 int dgpp_launch_moe_grouped_mma_gate_up_swiglu(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs,
                                                int n_segs, int max_rows, int rows_per_block, const DgppMoeExpertView* views,

@@ -73,6 +73,9 @@ struct DenseArgs {
   int out_f32;
   int m, n, k;
   int once;                 // all m rows ride on one pass over the weights (nontemporal loads)
+  // matrix-core form only: the activation is SwiGLU(act, act_up) with this clamp, computed as the rows are staged
+  const uint16_t* act_up = nullptr;
+  float limit = 0.f;
 };
 
 template <int FMT, int MAXR, int NB, bool NT>
@@ -520,8 +523,10 @@ struct GroupedArgs {
   int group_rows;      // activation rows staged per pass (<= kMaxActRows)
   const int32_t* act_rows;  // matrix-core form only, nullable: activation row of each segment row
   int once;                 // every segment fits one pass over its expert (nontemporal loads)
-  int gate_up;              // matrix-core form only: gate and up rows + SwiGLU in one launch (`which` unused, bf16 out)
-  float limit;              // the SwiGLU clamp of that form
+  int gate_up;              // matrix-core form only, `which` unused, bf16 out: 1 = gate and up rows + SwiGLU in one
+                            // launch; 2 = gate rows to `out`, up rows to `out_up`
+  float limit;              // the SwiGLU clamp of form 1
+  void* out_up;             // form 2
 };
 
 template <int FMT, int NB, bool NT>
@@ -646,10 +651,15 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
   const dim3 grid(gx, gy, split ? g.parts : 1);
   hipError_t err = hipSuccess;
   dispatch_bool(a.once != 0, [&](auto ntc) {
-    auto kern = mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value>;
-    constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
-    err = ensure_lds(kern, lds);
-    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, split ? ws : nullptr);
+    auto go = [&](auto kern) {
+      constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
+      err = ensure_lds(kern, lds);
+      if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, split ? ws : nullptr);
+    };
+    if constexpr (FMT == kFmtFp8F32) {   // the SwiGLU-staging form exists for the reference's one launcher of it
+      if (a.act_up) return go(mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value, true>);
+    }
+    go(mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value, false>);
   });
   if (err != hipSuccess) return err;
   if (split) {

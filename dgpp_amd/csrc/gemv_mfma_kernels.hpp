@@ -10,6 +10,19 @@ namespace dgpp_amd {
 constexpr int kStageUnits = 1024;   // 16-byte units of one block-shared activation stage (16 KB)
 constexpr int kMfmaNB = 4;          // lane loads in flight per row group and pass
 
+// SwiGLU of eight bf16 gate / up pairs (the elementwise kernel's arithmetic; zeros stay zeros).
+__device__ __forceinline__ uint4 swiglu_block(const uint4& gate, const uint4& up, float limit) {
+  const uint32_t g[4] = {gate.x, gate.y, gate.z, gate.w}, u[4] = {up.x, up.y, up.z, up.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint16_t lo = swiglu_bf16(bf16_to_f32(static_cast<uint16_t>(g[i] & 0xFFFFu)), bf16_to_f32(static_cast<uint16_t>(u[i] & 0xFFFFu)), limit);
+    const uint16_t hi = swiglu_bf16(bf16_to_f32(static_cast<uint16_t>(g[i] >> 16)), bf16_to_f32(static_cast<uint16_t>(u[i] >> 16)), limit);
+    o[i] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 // 64 weight rows (one row group per wavefront) against mt <= 16 activation rows, parts [p_lo, p_hi) of K.
 // K is walked in batches of up to kTileBatch tiles (a tile = four steps of a row group, gemv_mfma.hpp):
 // a wavefront puts all of a batch's weight loads in flight, the block then fetches the batch's
@@ -23,11 +36,12 @@ constexpr int kMfmaNB = 4;          // lane loads in flight per row group and pa
 constexpr int kTileBatch = 2;   // 8 KB in flight per wavefront; more tiles cost registers, and blocks per CU count for more
 constexpr int kBlockMfmaLdsUnits = kStageUnits + kWavesPerBlock * kTileUnits;
 
-template <int FMT, int NB, bool NT>
+template <int FMT, int NB, bool NT, bool SW = false>
 __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_t* __restrict__ act, size_t act_stride,
                                                 const int32_t* __restrict__ act_rows, int mt, int n, int k, int row0,
                                                 const MGeom& g, int p_lo, int p_hi, uint4* __restrict__ lds,
-                                                f32x4_t& sum) {
+                                                f32x4_t& sum, const uint16_t* __restrict__ act_up = nullptr,
+                                                float limit = 0.f) {
   static_assert(NB == 4, "a tile is four steps");
   constexpr int kSub = MTraits<FMT>::kSub;
   constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
@@ -39,19 +53,20 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
   const ScaleLane sl = scale_lane<FMT>(mat, row0, n, k);
   uint4* region = lds + kStageUnits + wave * kTileUnits;
   const int cc = min(lane & 15, mt - 1);
-  const bool aligned = ((reinterpret_cast<uintptr_t>(act) & 15u) == 0) && ((act_stride & 7u) == 0);
+  const bool aligned = (((reinterpret_cast<uintptr_t>(act) | reinterpret_cast<uintptr_t>(act_up)) & 15u) == 0) &&
+                       ((act_stride & 7u) == 0);
   const int cpp = g.part_steps / NB;   // tiles per part: part_steps is a multiple of four
   const int batch = max(1, min(kTileBatch, kStageUnits / (mt * kStepBlocks * NB)));
   const int t_hi = p_hi * cpp;
   // this thread's pieces of a batch's activations: 8-element block kb of row c for each of its units
   int unit_kb[kStageRegs];
-  const uint16_t* unit_row[kStageRegs];
+  size_t unit_row[kStageRegs];   // element offset of the unit's activation row
 #pragma unroll
   for (int i = 0; i < kStageRegs; ++i) {
     const int idx = threadIdx.x + i * kBlockThreads;
     const int kb = idx / mt, c = idx - kb * mt;
     unit_kb[i] = kb;
-    unit_row[i] = act + (act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(c)) * act_stride;
+    unit_row[i] = (act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(c)) * act_stride;
   }
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
   for (int t0 = p_lo * cpp; t0 < t_hi; t0 += batch) {
@@ -73,7 +88,11 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
 #pragma unroll
     for (int i = 0; i < kStageRegs; ++i) {
       pre[i] = make_uint4(0u, 0u, 0u, 0u);
-      if (threadIdx.x + i * kBlockThreads < units) pre[i] = load_act_block(unit_row[i], k_base + unit_kb[i] * 8, k, aligned);
+      if (threadIdx.x + i * kBlockThreads < units) {
+        pre[i] = load_act_block(act + unit_row[i], k_base + unit_kb[i] * 8, k, aligned);
+        if constexpr (SW)   // the activation is SwiGLU(act, act_up), computed on its way into the stage
+          pre[i] = swiglu_block(pre[i], load_act_block(act_up + unit_row[i], k_base + unit_kb[i] * 8, k, aligned), limit);
+      }
     }
     __syncthreads();   // the stage's readers of the batch before are through
 #pragma unroll
@@ -117,7 +136,7 @@ __device__ __forceinline__ void store_tile(const f32x4_t& v, float divisor, void
 // `partials` null: all parts in one block, folded and stored. Otherwise blockIdx.z names the ONE part
 // this block computes and its raw sums go to partials[part][row of out][n] (fp32); fold_parts_kernel
 // then adds the parts in the same ascending order — the split form's bits are the unsplit form's.
-template <int FMT, int NB, bool NT>
+template <int FMT, int NB, bool NT, bool SW>
 __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs a, MGeom g, float* partials) {
   extern __shared__ uint4 lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
@@ -127,15 +146,17 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs 
   const int c = lane & 15;
   f32x4_t sum;
   if (partials == nullptr) {
-    block_rows_mfma<FMT, NB, NT>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k,
-                             row0, g, 0, g.parts, lds, sum);
+    block_rows_mfma<FMT, NB, NT, SW>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n,
+                                 a.k, row0, g, 0, g.parts, lds, sum,
+                                 SW ? a.act_up + static_cast<size_t>(c0) * a.act_stride : nullptr, a.limit);
     store_tile<FMT>(sum, load_divisor<FMT>(a.global), a.out, a.out_f32, static_cast<size_t>(c0 + c) * a.out_stride, row0,
                     a.n, c < mt);
     return;
   }
   const int part = static_cast<int>(blockIdx.z);
-  block_rows_mfma<FMT, NB, NT>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k, row0,
-                           g, part, part + 1, lds, sum);
+  block_rows_mfma<FMT, NB, NT, SW>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k,
+                               row0, g, part, part + 1, lds, sum,
+                               SW ? a.act_up + static_cast<size_t>(c0) * a.act_stride : nullptr, a.limit);
   store_tile<kFmtMxfp4>(sum, 1.0f, partials, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
 }
 
@@ -179,13 +200,27 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
     const size_t first = static_cast<size_t>(seg.row0 + c0);
     const uint16_t* act = a.act_rows ? a.act : a.act + first * a.act_stride;
     const int32_t* rows = a.act_rows ? a.act_rows + first : nullptr;
-    block_rows_mfma<FMT, NB, NT>(mat, act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum);
     if constexpr (GU) {
-      const MatRef mat_up = mat_of_view<FMT>(a.views[seg.expert * 3 + 1], &gp2);
-      const float divisor_up = load_divisor<FMT>(gp2);
-      f32x4_t sum_up;
-      block_rows_mfma<FMT, NB, NT>(mat_up, act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum_up);
-      if (c < mt) {
+      // one compiled walk, run for the gate matrix and again for the up matrix (kept a loop: register budget)
+      f32x4_t sum_up = {0.f, 0.f, 0.f, 0.f};
+      float divisor_up = 1.f;
+#pragma unroll 1
+      for (int w = 0; w < 2; ++w) {
+        const MatRef mw = mat_of_view<FMT>(a.views[seg.expert * 3 + w], &gp2);
+        f32x4_t t;
+        block_rows_mfma<FMT, NB, NT>(mw, act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, t);
+        const float dw = load_divisor<FMT>(gp2);
+        if (w == 0) {
+          sum = t;
+        } else {
+          sum_up = t;
+          divisor_up = dw;
+        }
+      }
+      if (a.gate_up == 2) {
+        store_tile<FMT>(sum, divisor, a.out, 0, (first + c) * a.out_stride, row0, a.n, c < mt);
+        store_tile<FMT>(sum_up, divisor_up, a.out_up, 0, (first + c) * a.out_stride, row0, a.n, c < mt);
+      } else if (c < mt) {
         uint16_t* out = static_cast<uint16_t*>(a.out) + (first + c) * a.out_stride;
         const int r = row0 + (lane >> 4) * 4;
 #pragma unroll
@@ -194,6 +229,7 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
             out[r + i] = swiglu_bf16(finish_dot<FMT>(sum[i], divisor), finish_dot<FMT>(sum_up[i], divisor_up), a.limit);
       }
     } else {
+      block_rows_mfma<FMT, NB, NT>(mat, act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum);
       store_tile<FMT>(sum, divisor, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, c < mt);
     }
   }

@@ -391,6 +391,22 @@ def launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per
                                                        _p(act_rows)))
 
 
+def launch_mma_gemv_fp8_swiglu_f32(gate, up, limit, act_stride, w, scales, out, m, n, k, out_stride=0, rs=7, cs=7,
+                                   stream=None):
+    _check(_lib.load().dgpp_launch_mma_gemv_fp8_swiglu_f32(_p(gate), _p(up), limit, act_stride, _p(w), _p(scales), _p(out),
+                                                           m, n, k, out_stride, rs, cs, _stream(stream)))
+
+
+def launch_dense_mma_fp4_prod_bf16(act, act_stride, seg, views, which, out, m, n, k, stream=None, fp4_group=16):
+    _check(_lib.load().dgpp_launch_dense_mma_fp4_prod_bf16(_p(act), act_stride, _p(seg), _p(views), which, _p(out), m, n, k,
+                                                           _stream(stream), fp4_group))
+
+
+def launch_dense_mma_fp4_gate_up_bf16(act, act_stride, seg, views, gate, up, m, n, k, stream=None, fp4_group=16):
+    _check(_lib.load().dgpp_launch_dense_mma_fp4_gate_up_bf16(_p(act), act_stride, _p(seg), _p(views), _p(gate), _p(up), m, n,
+                                                              k, _stream(stream), fp4_group))
+
+
 def launch_moe_grouped_mma_gate_up_swiglu(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, out, out_stride,
                                           n, k, limit, stream=None, act_rows=None):
     """Extension: grouped FP8 gate + up + SwiGLU in one matrix-core launch."""

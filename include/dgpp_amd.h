@@ -328,6 +328,22 @@ int dgpp_launch_moe_grouped_mma_bf16(const uint16_t* act, size_t act_stride, con
 int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
                                     int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which, float* out,
                                     size_t out_stride, int n, int k, void* stream, const int32_t* act_rows);
+/* src/kernels/mma_gemv.hpp:86-95 (launch_mma_gemv_fp8_swiglu_f32): out = swiglu(gate, up) x W^T with the activation
+ * computed as the rows are staged; bitwise dgpp_launch_moe_swiglu_clamp followed by dgpp_launch_mma_gemv_fp8_f32
+ * (unsplit). gate / up: bf16 [m, act_stride], 16-byte aligned rows. */
+int dgpp_launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t* up, float limit, size_t act_stride,
+                                        const uint8_t* w, const float* scales, float* out, int m, int n, int k,
+                                        size_t out_stride, int rs, int cs, void* stream);
+/* src/kernels/glm_moe_launch.hpp:354-357 (launch_dense_mma_fp4_prod_bf16): the rows of ONE device-resident segment
+ * against views[seg->expert * 3 + which]; out [m, n]. The grouped matrix-core kernel's chain. */
+int dgpp_launch_dense_mma_fp4_prod_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
+                                        const DgppMoeExpertView* views, int which, uint16_t* out, int m, int n, int k,
+                                        void* stream, int fp4_group);
+/* src/kernels/glm_moe_launch.hpp:366-369 (launch_dense_mma_fp4_gate_up_bf16): gate and up of that segment in one
+ * launch; the bits of two dgpp_launch_dense_mma_fp4_prod_bf16 calls. */
+int dgpp_launch_dense_mma_fp4_gate_up_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
+                                           const DgppMoeExpertView* views, uint16_t* gate, uint16_t* up, int m, int n,
+                                           int k, void* stream, int fp4_group);
 /* Extension (no counterpart in the reference): dgpp_launch_moe_grouped_mma{,_fp4}_bf16 for which = 0 and which = 1
  * followed by dgpp_launch_moe_swiglu_clamp, in one launch: a block walks its rows of the segment's gate matrix, then
  * of its up matrix, against the same activation rows and stores SwiGLU(bf16(gate), bf16(up)). Same bits as the

@@ -360,6 +360,22 @@ inline void launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, c
   detail::check(dgpp_launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                                 out_stride, n, k, stream, act_rows));
 }
+inline void launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t* up, float limit, size_t act_stride,
+                                           const uint8_t* w, const float* scales, float* out, int m, int n, int k,
+                                           size_t out_stride, int rs, int cs, hipStream_t stream) {
+  detail::check(dgpp_launch_mma_gemv_fp8_swiglu_f32(gate, up, limit, act_stride, w, scales, out, m, n, k, out_stride, rs, cs,
+                                                    stream));
+}
+inline void launch_dense_mma_fp4_prod_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* seg,
+                                           const MoeExpertView* views, int which, uint16_t* out, int m, int n, int k,
+                                           hipStream_t stream, int fp4_group = kFp4Group) {
+  detail::check(dgpp_launch_dense_mma_fp4_prod_bf16(act, act_stride, seg, views, which, out, m, n, k, stream, fp4_group));
+}
+inline void launch_dense_mma_fp4_gate_up_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* seg,
+                                              const MoeExpertView* views, uint16_t* gate, uint16_t* up, int m, int n, int k,
+                                              hipStream_t stream, int fp4_group = kFp4Group) {
+  detail::check(dgpp_launch_dense_mma_fp4_gate_up_bf16(act, act_stride, seg, views, gate, up, m, n, k, stream, fp4_group));
+}
 // Extension: grouped gate + up + SwiGLU in one matrix-core launch (see dgpp_amd.h).
 inline void launch_moe_grouped_mma_gate_up_swiglu(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
                                                   int max_rows, int rows_per_block, const MoeExpertView* views,

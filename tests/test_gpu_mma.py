@@ -132,6 +132,46 @@ def test_grouped_mma_is_bitwise_the_dense_mma_per_segment_with_and_without_the_g
         check(np.ascontiguousarray(a[r0:r0 + cnt]), raw, f"grouped mma {kind} segment {e}")
 
 
+@pytest.mark.parametrize("m,n,k,limit", [(3, 200, 1024, 7.0), (20, 96, 2048, float("inf")), (16, 130, 304, 0.5)])
+def test_mma_gemv_fp8_swiglu_is_bitwise_swiglu_then_mma_gemv(gpu, m, n, k, limit):
+    """src/kernels/mma_gemv.hpp:86-95: the activation computed as the rows are staged gives the bits of
+    launch_moe_swiglu_clamp followed by launch_mma_gemv_fp8_f32 (unsplit)."""
+    w = hg.f32_to_bf16(hg.normal_f32(0x9A0 + n + k, (n, k), 0.02))
+    payload, scales = hg.encode_fp8_blocks(w, 128, 128)
+    gate, up = hg.normal_bf16(0x9A1 + n, (m, k), 2.0), hg.normal_bf16(0x9A2 + n, (m, k))
+    g_d, u_d, p_d, s_d = dev(gate), dev(up), dev(payload), dev(scales)
+    act, want, got = dev_empty((m, k), np.uint16), dev_empty((m, n), np.float32), dev_empty((m, n), np.float32)
+    L.launch_moe_swiglu_clamp(g_d, u_d, act, m * k, limit, None)
+    L.launch_mma_gemv_fp8_f32(act, k, p_d, s_d, want, m, n, k, 0, 7, 7, None)
+    L.launch_mma_gemv_fp8_swiglu_f32(g_d, u_d, limit, k, p_d, s_d, got, m, n, k, 0, 7, 7, None)
+    sync()
+    assert np.array_equal(host(got).view(np.uint32), host(want).view(np.uint32))
+    with pytest.raises(L.InvalidArgument):
+        L.launch_mma_gemv_fp8_swiglu_f32(g_d, None, limit, k, p_d, s_d, got, m, n, k, 0, 7, 7, None)
+
+
+@pytest.mark.parametrize("kind", ["nvfp4", "mxfp4"])
+def test_dense_mma_fp4_prod_and_gate_up_are_the_grouped_kernel_on_one_segment(gpu, kind):
+    """src/kernels/glm_moe.cu:4809-4823 and src/kernels/dense_fp4_decode.cu:310-319: one device-resident segment
+    through the grouped matrix-core kernel; the paired launcher gives the bits of two prod launches."""
+    E, H, I, K, T = 4, 512, 96, 2, 19
+    p = moe_data.make_problem(E, H, I, K, T, kind, 55, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    expert, m = 2, 19
+    seg = dev(np.array([[0, m, expert]], np.int32))
+    g1, u1, g2, u2, gg = (dev_empty((m, I), np.uint16) for _ in range(5))
+    L.launch_dense_mma_fp4_prod_bf16(d.x, H, seg, d.views, 0, g1, m, I, H, None, d.fp4_group)
+    L.launch_dense_mma_fp4_prod_bf16(d.x, H, seg, d.views, 1, u1, m, I, H, None, d.fp4_group)
+    L.launch_dense_mma_fp4_gate_up_bf16(d.x, H, seg, d.views, g2, u2, m, I, H, None, d.fp4_group)
+    L.launch_moe_grouped_mma_fp4_bf16(d.x, H, seg, 1, m, 0, d.views, 0, gg, I, I, H, None, None, d.fp4_group)
+    sync()
+    assert np.array_equal(host(g1, np.uint16), host(gg, np.uint16))
+    assert np.array_equal(host(g1, np.uint16), host(g2, np.uint16)) and np.array_equal(host(u1, np.uint16), host(u2, np.uint16))
+    mat = p.experts[expert][1]
+    raw = orc.gemv_fp4(p.x, mat.payload, mat.scales, float(mat.glob[0]) if mat.glob is not None else 1.0, d.fp4_group, m, I, H)
+    check(host(u2, np.uint16), raw, f"dense mma fp4 gate_up {kind}: up rows")
+
+
 @pytest.mark.parametrize("kind,limit", [("fp8", 7.0), ("nvfp4", float("inf")), ("mxfp4", 0.75)])
 def test_grouped_mma_gate_up_swiglu_is_bitwise_the_three_launches(gpu, kind, limit):
     """The one-launch extension (gate rows, up rows, SwiGLU in the matrix-core grouped kernel) against the two grouped
