@@ -26,7 +26,7 @@ HIP_SOURCES = [
     "moe_misc.hip",
     "capi.hip",
 ]
-HOST_SOURCES = ["host_codec.cpp"]
+HOST_SOURCES = ["host_codec.cpp", "loader.cpp"]
 # Host C++ that needs the HIP runtime headers (compiled by hipcc as plain host code).
 HIP_HOST_SOURCES = ["moe_layer.cpp"]
 

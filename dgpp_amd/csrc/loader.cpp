@@ -1,0 +1,576 @@
+// Host side of the loader C ABI (include/dgpp_amd_loader.h): a memory-mapped safetensors reader and the
+// pointer views over quantized matrices. No GPU calls.
+//
+// The header is scanned by a small strict JSON reader written for this one document shape: an object of
+// tensor descriptors ({"dtype": string, "shape": [ints], "data_offsets": [begin, end]}) plus an optional
+// "__metadata__" member that is kept as raw text. Everything the reference's reader rejects is rejected
+// here with a message that names the same cause (src/loaders/safetensors.hpp:198-252; its unit tests
+// tests/unit/safetensors_test.cpp:140-175 list the cases).
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <cerrno>
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <stdexcept>
+#include <string>
+#include <string_view>
+#include <vector>
+
+#include "../../include/dgpp_amd_loader.h"
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const std::string& msg) {
+  g_error = msg;
+  return code;
+}
+
+struct Tensor {
+  std::string name;
+  DgppTensorInfo info;
+};
+
+// ---- the JSON scanner -----------------------------------------------------------------------------------
+struct Number {
+  bool integer = false;   // an integer literal that fits int64
+  int64_t value = 0;
+};
+
+class Scanner {
+ public:
+  explicit Scanner(std::string_view text) : s_(text) {}
+
+  void ws() {
+    while (p_ < s_.size() && (s_[p_] == ' ' || s_[p_] == '\t' || s_[p_] == '\n' || s_[p_] == '\r')) ++p_;
+  }
+  bool at_end() {
+    ws();
+    return p_ >= s_.size();
+  }
+  char peek() {
+    ws();
+    if (p_ >= s_.size()) throw std::runtime_error("unexpected end of header JSON");
+    return s_[p_];
+  }
+  void expect(char c) {
+    if (peek() != c) throw std::runtime_error(std::string("header JSON: expected '") + c + "'");
+    ++p_;
+  }
+  bool take(char c) {
+    if (peek() != c) return false;
+    ++p_;
+    return true;
+  }
+
+  std::string string() {
+    expect('"');
+    std::string out;
+    while (true) {
+      if (p_ >= s_.size()) throw std::runtime_error("header JSON: unterminated string");
+      const unsigned char c = static_cast<unsigned char>(s_[p_++]);
+      if (c == '"') return out;
+      if (c < 0x20) throw std::runtime_error("header JSON: control character in string");
+      if (c != '\\') {
+        out.push_back(static_cast<char>(c));
+        continue;
+      }
+      if (p_ >= s_.size()) throw std::runtime_error("header JSON: unterminated escape");
+      const char e = s_[p_++];
+      switch (e) {
+        case '"': out.push_back('"'); break;
+        case '\\': out.push_back('\\'); break;
+        case '/': out.push_back('/'); break;
+        case 'b': out.push_back('\b'); break;
+        case 'f': out.push_back('\f'); break;
+        case 'n': out.push_back('\n'); break;
+        case 'r': out.push_back('\r'); break;
+        case 't': out.push_back('\t'); break;
+        case 'u': {
+          unsigned cp = hex4();
+          if (cp >= 0xD800 && cp <= 0xDBFF && p_ + 1 < s_.size() && s_[p_] == '\\' && s_[p_ + 1] == 'u') {
+            p_ += 2;
+            const unsigned lo = hex4();
+            if (lo >= 0xDC00 && lo <= 0xDFFF) cp = 0x10000 + ((cp - 0xD800) << 10) + (lo - 0xDC00);
+          }
+          utf8(cp, out);
+          break;
+        }
+        default: throw std::runtime_error("header JSON: bad escape");
+      }
+    }
+  }
+
+  // -?(0|[1-9][0-9]*)(.[0-9]+)?([eE][+-]?[0-9]+)?  — a leading zero before another digit is malformed.
+  Number number() {
+    ws();
+    const size_t start = p_;
+    bool neg = false;
+    if (p_ < s_.size() && s_[p_] == '-') {
+      neg = true;
+      ++p_;
+    }
+    if (p_ >= s_.size() || s_[p_] < '0' || s_[p_] > '9') throw std::runtime_error("header JSON: malformed number");
+    if (s_[p_] == '0' && p_ + 1 < s_.size() && s_[p_ + 1] >= '0' && s_[p_ + 1] <= '9')
+      throw std::runtime_error("header JSON: malformed number (leading zero)");
+    bool fits = true;
+    uint64_t mag = 0;
+    while (p_ < s_.size() && s_[p_] >= '0' && s_[p_] <= '9') {
+      const uint64_t d = static_cast<uint64_t>(s_[p_] - '0');
+      if (mag > (std::numeric_limits<uint64_t>::max() - d) / 10) fits = false;
+      else mag = mag * 10 + d;
+      ++p_;
+    }
+    bool integral = true;
+    if (p_ < s_.size() && s_[p_] == '.') {
+      integral = false;
+      ++p_;
+      if (p_ >= s_.size() || s_[p_] < '0' || s_[p_] > '9') throw std::runtime_error("header JSON: malformed number");
+      while (p_ < s_.size() && s_[p_] >= '0' && s_[p_] <= '9') ++p_;
+    }
+    if (p_ < s_.size() && (s_[p_] == 'e' || s_[p_] == 'E')) {
+      integral = false;
+      ++p_;
+      if (p_ < s_.size() && (s_[p_] == '+' || s_[p_] == '-')) ++p_;
+      if (p_ >= s_.size() || s_[p_] < '0' || s_[p_] > '9') throw std::runtime_error("header JSON: malformed number");
+      while (p_ < s_.size() && s_[p_] >= '0' && s_[p_] <= '9') ++p_;
+    }
+    (void)start;
+    Number n;
+    const uint64_t limit = neg ? (1ull << 63) : static_cast<uint64_t>(std::numeric_limits<int64_t>::max());
+    if (integral && fits && mag <= limit) {
+      n.integer = true;
+      n.value = neg ? static_cast<int64_t>(0 - mag) : static_cast<int64_t>(mag);
+    }
+    return n;
+  }
+
+  void literal(const char* word) {
+    ws();
+    const size_t n = std::strlen(word);
+    if (s_.compare(p_, n, word) != 0) throw std::runtime_error("header JSON: bad literal");
+    p_ += n;
+  }
+
+  // Skips any value; returns its raw text.
+  std::string_view skip_value() {
+    ws();
+    const size_t start = p_;
+    skip();
+    return s_.substr(start, p_ - start);
+  }
+
+ private:
+  void skip() {
+    const char c = peek();
+    if (c == '{') {
+      ++p_;
+      if (take('}')) return;
+      do {
+        string();
+        expect(':');
+        skip();
+      } while (take(','));
+      expect('}');
+    } else if (c == '[') {
+      ++p_;
+      if (take(']')) return;
+      do skip();
+      while (take(','));
+      expect(']');
+    } else if (c == '"') {
+      string();
+    } else if (c == 't') {
+      literal("true");
+    } else if (c == 'f') {
+      literal("false");
+    } else if (c == 'n') {
+      literal("null");
+    } else {
+      number();
+    }
+  }
+  unsigned hex4() {
+    if (p_ + 4 > s_.size()) throw std::runtime_error("header JSON: bad \\u escape");
+    unsigned v = 0;
+    for (int i = 0; i < 4; ++i) {
+      const char c = s_[p_++];
+      v <<= 4;
+      if (c >= '0' && c <= '9') v |= static_cast<unsigned>(c - '0');
+      else if (c >= 'a' && c <= 'f') v |= static_cast<unsigned>(c - 'a' + 10);
+      else if (c >= 'A' && c <= 'F') v |= static_cast<unsigned>(c - 'A' + 10);
+      else throw std::runtime_error("header JSON: bad \\u escape");
+    }
+    return v;
+  }
+  static void utf8(unsigned cp, std::string& out) {
+    if (cp < 0x80) {
+      out.push_back(static_cast<char>(cp));
+    } else if (cp < 0x800) {
+      out.push_back(static_cast<char>(0xC0 | (cp >> 6)));
+      out.push_back(static_cast<char>(0x80 | (cp & 0x3F)));
+    } else if (cp < 0x10000) {
+      out.push_back(static_cast<char>(0xE0 | (cp >> 12)));
+      out.push_back(static_cast<char>(0x80 | ((cp >> 6) & 0x3F)));
+      out.push_back(static_cast<char>(0x80 | (cp & 0x3F)));
+    } else {
+      out.push_back(static_cast<char>(0xF0 | (cp >> 18)));
+      out.push_back(static_cast<char>(0x80 | ((cp >> 12) & 0x3F)));
+      out.push_back(static_cast<char>(0x80 | ((cp >> 6) & 0x3F)));
+      out.push_back(static_cast<char>(0x80 | (cp & 0x3F)));
+    }
+  }
+
+  std::string_view s_;
+  size_t p_ = 0;
+};
+
+int dtype_of(std::string_view s) {
+  if (s == "F32") return DGPP_DT_F32;
+  if (s == "F16") return DGPP_DT_F16;
+  if (s == "BF16") return DGPP_DT_BF16;
+  if (s == "F8_E4M3" || s == "F8" || s == "FP8") return DGPP_DT_F8_E4M3;
+  if (s == "I64") return DGPP_DT_I64;
+  if (s == "I32") return DGPP_DT_I32;
+  if (s == "U8" || s == "BOOL") return DGPP_DT_U8;
+  if (s == "I8") return DGPP_DT_I8;
+  if (s == "F8_E8M0") return DGPP_DT_F8_E8M0;
+  if (s == "U32") return DGPP_DT_U32;
+  if (s == "I16") return DGPP_DT_I16;
+  return -1;
+}
+
+}  // namespace
+
+struct DgppSafetensors {
+  std::string path;
+  int fd = -1;
+  uint8_t* map = nullptr;
+  size_t map_len = 0;
+  uint64_t header_fold = 0;
+  std::string metadata;
+  std::vector<Tensor> tensors;   // sorted by name
+
+  ~DgppSafetensors() { unmap(false); }
+
+  void unmap(bool drop_page_cache) {
+    if (map != nullptr) {
+      munmap(map, map_len ? map_len : 1);
+      map = nullptr;
+    }
+    if (fd >= 0) {
+      if (drop_page_cache) posix_fadvise(fd, 0, 0, POSIX_FADV_DONTNEED);   // only effective after the munmap
+      ::close(fd);
+      fd = -1;
+    }
+    tensors.clear();
+  }
+
+  // One tensor descriptor; `s` stands on its '{'.
+  void descriptor(Scanner& s, const std::string& name, uint64_t data_start) {
+    bool have_dtype = false, have_shape = false, have_offsets = false;
+    Tensor t;
+    t.name = name;
+    std::memset(&t.info, 0, sizeof(t.info));
+    uint64_t begin = 0, end = 0;
+    uint64_t numel = 1;
+    s.expect('{');
+    if (!s.take('}')) {
+      do {
+        const std::string key = s.string();
+        s.expect(':');
+        if (key == "dtype") {
+          if (s.peek() != '"') throw std::runtime_error(path + ": tensor " + name + " dtype is not a string");
+          const std::string d = s.string();
+          const int dt = dtype_of(d);
+          if (dt < 0) throw std::runtime_error(path + ": unknown dtype " + d);
+          t.info.dtype = dt;
+          have_dtype = true;
+        } else if (key == "shape") {
+          if (s.peek() != '[') throw std::runtime_error(path + ": tensor " + name + " shape is not an array");
+          s.expect('[');
+          int rank = 0;
+          numel = 1;
+          if (!s.take(']')) {
+            do {
+              const char c = s.peek();
+              if (c != '-' && (c < '0' || c > '9'))
+                throw std::runtime_error(path + ": tensor " + name + " shape must contain nonnegative integers");
+              const Number n = s.number();
+              if (!n.integer || n.value < 0)
+                throw std::runtime_error(path + ": tensor " + name + " shape must contain nonnegative integers");
+              if (rank >= DGPP_MAX_TENSOR_RANK)
+                throw std::runtime_error(path + ": tensor " + name + " shape has more dimensions than this reader takes");
+              t.info.shape[rank++] = n.value;
+              // the ordered checked product: a zero met before an overflowing factor keeps the tensor empty,
+              // a later zero does not undo an overflow
+              const uint64_t d = static_cast<uint64_t>(n.value);
+              if (numel != 0 && d > std::numeric_limits<size_t>::max() / numel)
+                throw std::runtime_error(path + ": tensor " + name + " shape element count overflows");
+              numel *= d;
+            } while (s.take(','));
+            s.expect(']');
+          }
+          t.info.rank = rank;
+          have_shape = true;
+        } else if (key == "data_offsets") {
+          const std::string bad = path + ": tensor " + name + " data_offsets must contain two nonnegative integers";
+          if (s.peek() != '[') throw std::runtime_error(bad);
+          s.expect('[');
+          uint64_t v[2] = {0, 0};
+          int count = 0;
+          if (!s.take(']')) {
+            do {
+              const char c = s.peek();
+              if (c != '-' && (c < '0' || c > '9')) throw std::runtime_error(bad);
+              const Number n = s.number();
+              if (!n.integer || n.value < 0 || count >= 2) throw std::runtime_error(bad);
+              v[count++] = static_cast<uint64_t>(n.value);
+            } while (s.take(','));
+            s.expect(']');
+          }
+          if (count != 2) throw std::runtime_error(bad);
+          begin = v[0];
+          end = v[1];
+          have_offsets = true;
+        } else {
+          s.skip_value();
+        }
+      } while (s.take(','));
+      s.expect('}');
+    }
+    if (!have_dtype) throw std::runtime_error(path + ": tensor " + name + " has no dtype");
+    if (!have_shape) throw std::runtime_error(path + ": tensor " + name + " has no shape");
+    if (!have_offsets) throw std::runtime_error(path + ": tensor " + name + " has no data_offsets");
+    if (begin > end || end > map_len - data_start)
+      throw std::runtime_error(path + ": tensor " + name + " has invalid data_offsets");
+    const uint64_t width = dgpp_dtype_size(t.info.dtype);
+    if (numel > std::numeric_limits<size_t>::max() / width || numel * width != end - begin)
+      throw std::runtime_error(path + ": tensor " + name + " shape/dtype byte count mismatch");
+    t.info.numel = numel;
+    t.info.nbytes = end - begin;
+    t.info.file_offset = data_start + begin;
+    t.info.data = map + t.info.file_offset;
+    // a name given twice: the later descriptor stands
+    auto it = std::find_if(tensors.begin(), tensors.end(), [&](const Tensor& o) { return o.name == name; });
+    if (it != tensors.end()) *it = std::move(t);
+    else tensors.push_back(std::move(t));
+  }
+
+  void parse() {
+    if (map_len < 8) throw std::runtime_error(path + ": too small for safetensors");
+    uint64_t hlen;
+    std::memcpy(&hlen, map, 8);
+    if (hlen > map_len - 8) throw std::runtime_error(path + ": header length overruns file");
+    const std::string_view json(reinterpret_cast<const char*>(map + 8), static_cast<size_t>(hlen));
+    header_fold = 1469598103934665603ull;
+    for (const char c : json) header_fold = (header_fold ^ static_cast<uint8_t>(c)) * 1099511628211ull;
+    const uint64_t data_start = 8 + hlen;
+    Scanner s(json);
+    if (s.at_end() || s.peek() != '{') throw std::runtime_error(path + ": safetensors header not an object");
+    s.expect('{');
+    if (!s.take('}')) {
+      do {
+        const std::string key = s.string();
+        s.expect(':');
+        if (key == "__metadata__") {
+          metadata = std::string(s.skip_value());
+          continue;
+        }
+        if (s.peek() != '{') throw std::runtime_error(path + ": tensor " + key + " descriptor is not an object");
+        descriptor(s, key, data_start);
+      } while (s.take(','));
+      s.expect('}');
+    }
+    if (!s.at_end()) throw std::runtime_error(path + ": trailing characters after the header object");
+    std::sort(tensors.begin(), tensors.end(), [](const Tensor& a, const Tensor& b) { return a.name < b.name; });
+  }
+
+  void page_span(const DgppTensorInfo& t, size_t& begin, size_t& len) const {
+    static const size_t page = static_cast<size_t>(sysconf(_SC_PAGESIZE));
+    begin = static_cast<size_t>(t.file_offset / page) * page;
+    size_t end = static_cast<size_t>((t.file_offset + t.nbytes + page - 1) / page) * page;
+    if (end > map_len) end = map_len;
+    len = end > begin ? end - begin : 0;
+  }
+};
+
+extern "C" {
+
+const char* dgpp_loader_last_error(void) { return g_error.c_str(); }
+
+size_t dgpp_dtype_size(int dtype) {
+  switch (dtype) {
+    case DGPP_DT_F32: case DGPP_DT_I32: case DGPP_DT_U32: return 4;
+    case DGPP_DT_F16: case DGPP_DT_BF16: case DGPP_DT_I16: return 2;
+    case DGPP_DT_I64: return 8;
+    case DGPP_DT_F8_E4M3: case DGPP_DT_U8: case DGPP_DT_I8: case DGPP_DT_F8_E8M0: return 1;
+    default: return 0;
+  }
+}
+
+int dgpp_safetensors_open(const char* path, DgppSafetensors** out) {
+  if (!path || !out) return fail(DGPP_INVALID_ARGUMENT, "safetensors_open: null argument");
+  *out = nullptr;
+  DgppSafetensors* f = nullptr;
+  try {
+    f = new DgppSafetensors();
+    f->path = path;
+    f->fd = ::open(path, O_RDONLY | O_CLOEXEC);
+    if (f->fd < 0) throw std::runtime_error(std::string("cannot open ") + path + ": " + std::strerror(errno));
+    struct stat st {};
+    if (fstat(f->fd, &st) != 0) throw std::runtime_error(std::string("fstat failed for ") + path);
+    f->map_len = static_cast<size_t>(st.st_size);
+    void* m = mmap(nullptr, f->map_len ? f->map_len : 1, PROT_READ, MAP_PRIVATE, f->fd, 0);
+    if (m == MAP_FAILED) throw std::runtime_error(std::string("mmap failed for ") + path);
+    f->map = static_cast<uint8_t*>(m);
+    f->parse();
+  } catch (const std::exception& e) {
+    g_error = e.what();
+    delete f;
+    return DGPP_RUNTIME_ERROR;
+  }
+  *out = f;
+  return DGPP_OK;
+}
+
+void dgpp_safetensors_close(DgppSafetensors* f, int drop_page_cache) {
+  if (!f) return;
+  f->unmap(drop_page_cache != 0);
+  delete f;
+}
+
+int dgpp_safetensors_count(const DgppSafetensors* f) { return f ? static_cast<int>(f->tensors.size()) : 0; }
+
+const char* dgpp_safetensors_name(const DgppSafetensors* f, int index) {
+  if (!f || index < 0 || index >= static_cast<int>(f->tensors.size())) return nullptr;
+  return f->tensors[static_cast<size_t>(index)].name.c_str();
+}
+
+int dgpp_safetensors_find(const DgppSafetensors* f, const char* name, DgppTensorInfo* out) {
+  if (!f || !name || !out) return fail(DGPP_INVALID_ARGUMENT, "safetensors_find: null argument");
+  const std::string_view key(name);
+  auto it = std::lower_bound(f->tensors.begin(), f->tensors.end(), key,
+                             [](const Tensor& t, std::string_view k) { return std::string_view(t.name) < k; });
+  if (it == f->tensors.end() || it->name != key)
+    return fail(DGPP_INVALID_ARGUMENT, "tensor not found: " + std::string(name) + " in " + f->path);
+  *out = it->info;
+  return DGPP_OK;
+}
+
+uint64_t dgpp_safetensors_header_fold(const DgppSafetensors* f) { return f ? f->header_fold : 0; }
+
+const char* dgpp_safetensors_metadata_json(const DgppSafetensors* f) { return f ? f->metadata.c_str() : ""; }
+
+void dgpp_safetensors_prefetch(const DgppSafetensors* f, const DgppTensorInfo* t) {
+  if (!f || !t || f->map == nullptr || t->nbytes == 0) return;
+  size_t begin, len;
+  f->page_span(*t, begin, len);
+  if (len) madvise(f->map + begin, len, MADV_WILLNEED);
+}
+
+void dgpp_safetensors_discard(const DgppSafetensors* f, const DgppTensorInfo* t) {
+  if (!f || !t || f->map == nullptr || t->nbytes == 0) return;
+  size_t begin, len;
+  f->page_span(*t, begin, len);
+  if (!len) return;
+  madvise(f->map + begin, len, MADV_DONTNEED);
+  posix_fadvise(f->fd, static_cast<off_t>(begin), static_cast<off_t>(len), POSIX_FADV_DONTNEED);
+}
+
+// ---- matrix views -----------------------------------------------------------------------------------------
+int dgpp_quant_scale_shifts(const DgppQuantMatrix* m, int* rs, int* cs) {
+  if (!m || !rs || !cs) return 0;
+  auto log2_exact = [](int64_t v) {
+    if (v <= 0 || (v & (v - 1)) != 0) return -1;
+    int s = 0;
+    while ((1LL << s) < v) ++s;
+    return s;
+  };
+  *rs = log2_exact(m->scale_block_rows);
+  *cs = log2_exact(m->scale_block_cols);
+  return *rs >= 0 && *cs >= 4;
+}
+
+int dgpp_quant_rows_view(const DgppQuantMatrix* m, int64_t row_start, int64_t rows, DgppQuantMatrix* out) {
+  if (!m || !out) return fail(DGPP_INVALID_ARGUMENT, "quant_rows_view: null argument");
+  if (m->scale_block_rows <= 0 || m->scale_block_cols <= 0)
+    return fail(DGPP_INVALID_ARGUMENT, "quant_rows_view: the scale block sizes must be positive");
+  if (row_start < 0 || rows < 0 || rows > m->rows || row_start > m->rows - rows)
+    return fail(DGPP_INVALID_ARGUMENT, "quant_rows_view: range out of bounds");
+  if (row_start % m->scale_block_rows != 0)
+    return fail(DGPP_INVALID_ARGUMENT,
+                "quant_rows_view: row_start must be aligned to the scale block (a slice that starts inside a block "
+                "cannot re-anchor the block scales)");
+  const int64_t scale_cols = (m->cols + m->scale_block_cols - 1) / m->scale_block_cols;
+  const int64_t first_block = row_start / m->scale_block_rows;
+  DgppQuantMatrix v = *m;
+  v.payload = m->payload + row_start * m->cols;
+  v.scales = m->scales ? m->scales + first_block * scale_cols : nullptr;
+  v.scales_e8m0 = m->scales_e8m0 ? m->scales_e8m0 + first_block * scale_cols : nullptr;
+  v.rows = rows;
+  *out = v;
+  return DGPP_OK;
+}
+
+int dgpp_fp4_check_cols(int64_t cols, int scale_group) {
+  if (scale_group != 16 && scale_group != 32) return fail(DGPP_INVALID_ARGUMENT, "fp4: the scale group must be 16 or 32");
+  if (cols <= 0 || cols % scale_group != 0)
+    return fail(DGPP_INVALID_ARGUMENT, "fp4: K must be a positive multiple of " + std::to_string(scale_group));
+  return DGPP_OK;
+}
+
+int dgpp_fp4_rows_view(const DgppFp4Matrix* m, int64_t row_start, int64_t rows, DgppFp4Matrix* out) {
+  if (!m || !out) return fail(DGPP_INVALID_ARGUMENT, "fp4_rows_view: null argument");
+  const int rc = dgpp_fp4_check_cols(m->cols, m->scale_group);
+  if (rc != DGPP_OK) return rc;
+  if (row_start < 0 || rows < 0 || rows > m->rows || row_start > m->rows - rows)
+    return fail(DGPP_INVALID_ARGUMENT, "fp4_rows_view: range out of bounds");
+  DgppFp4Matrix v = *m;
+  v.payload = m->payload + row_start * (m->cols / 2);
+  v.scales = m->scales + row_start * (m->cols / m->scale_group);
+  v.rows = rows;
+  *out = v;
+  return DGPP_OK;
+}
+
+int dgpp_expert_view_from_quant(const DgppQuantMatrix* m, DgppMoeExpertView* out) {
+  if (!m || !out) return fail(DGPP_INVALID_ARGUMENT, "expert_view_from_quant: null argument");
+  int rs = 0, cs = 0;
+  if (!m->payload || !m->scales)
+    return fail(DGPP_INVALID_ARGUMENT, "expert_view_from_quant: the table takes E4M3 payloads with an F32 scale grid");
+  if (!dgpp_quant_scale_shifts(m, &rs, &cs))
+    return fail(DGPP_INVALID_ARGUMENT, "expert_view_from_quant: the scale blocks must be powers of two, columns >= 16");
+  std::memset(out, 0, sizeof(*out));
+  out->payload = m->payload;
+  out->scales = m->scales;
+  out->scale_shift_rows = rs;
+  out->scale_shift_cols = cs;
+  out->fp4_group = 16;
+  return DGPP_OK;
+}
+
+int dgpp_expert_view_from_fp4(const DgppFp4Matrix* m, DgppMoeExpertView* out) {
+  if (!m || !out) return fail(DGPP_INVALID_ARGUMENT, "expert_view_from_fp4: null argument");
+  const int rc = dgpp_fp4_check_cols(m->cols, m->scale_group);
+  if (rc != DGPP_OK) return rc;
+  if (!m->payload || !m->scales) return fail(DGPP_INVALID_ARGUMENT, "expert_view_from_fp4: null payload or scales");
+  if (m->scale_group == 16 && !m->global_scale)
+    return fail(DGPP_INVALID_ARGUMENT, "expert_view_from_fp4: an NVFP4 matrix carries a device global scale");
+  std::memset(out, 0, sizeof(*out));
+  out->payload = m->payload;
+  out->fp4_scales = m->scales;
+  out->fp4_global = m->scale_group == 16 ? m->global_scale : nullptr;
+  out->scale_shift_rows = 7;
+  out->scale_shift_cols = 7;
+  out->fp4_group = m->scale_group;
+  return DGPP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,164 @@
+"""ctypes mirror of include/dgpp_amd_loader.h: the memory-mapped safetensors reader and the quantized
+matrix views (reference: src/loaders/safetensors.hpp, src/models/quant_matrix.hpp). Host side only."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+
+MAX_RANK = 8
+DT_F32, DT_F16, DT_BF16, DT_F8_E4M3, DT_I64, DT_I32, DT_U8, DT_I8, DT_F8_E8M0, DT_U32, DT_I16 = range(11)
+_NUMPY = {DT_F32: np.float32, DT_F16: np.float16, DT_BF16: np.uint16, DT_F8_E4M3: np.uint8, DT_I64: np.int64,
+          DT_I32: np.int32, DT_U8: np.uint8, DT_I8: np.int8, DT_F8_E8M0: np.uint8, DT_U32: np.uint32, DT_I16: np.int16}
+
+
+class LoaderError(RuntimeError):
+    pass
+
+
+class TensorInfo(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("rank", C.c_int32), ("shape", C.c_int64 * MAX_RANK), ("numel", C.c_uint64),
+                ("nbytes", C.c_uint64), ("file_offset", C.c_uint64), ("data", C.c_void_p)]
+
+    def dims(self):
+        return tuple(self.shape[i] for i in range(self.rank))
+
+
+class QuantMatrix(C.Structure):
+    """src/models/quant_matrix.hpp:16-52 (GlmQuantMatrix)."""
+    _fields_ = [("payload", C.c_void_p), ("scales", C.c_void_p), ("scales_e8m0", C.c_void_p), ("rows", C.c_int64),
+                ("cols", C.c_int64), ("scale_block_rows", C.c_int32), ("scale_block_cols", C.c_int32)]
+
+
+_P, _I = C.c_void_p, C.c_int
+SIGNATURES = {
+    "dgpp_loader_last_error": (C.c_char_p, []),
+    "dgpp_dtype_size": (C.c_size_t, [_I]),
+    "dgpp_safetensors_open": (_I, [C.c_char_p, C.POINTER(_P)]),
+    "dgpp_safetensors_close": (None, [_P, _I]),
+    "dgpp_safetensors_count": (_I, [_P]),
+    "dgpp_safetensors_name": (C.c_char_p, [_P, _I]),
+    "dgpp_safetensors_find": (_I, [_P, C.c_char_p, C.POINTER(TensorInfo)]),
+    "dgpp_safetensors_header_fold": (C.c_uint64, [_P]),
+    "dgpp_safetensors_metadata_json": (C.c_char_p, [_P]),
+    "dgpp_safetensors_prefetch": (None, [_P, C.POINTER(TensorInfo)]),
+    "dgpp_safetensors_discard": (None, [_P, C.POINTER(TensorInfo)]),
+    "dgpp_quant_scale_shifts": (_I, [C.POINTER(QuantMatrix), C.POINTER(_I), C.POINTER(_I)]),
+    "dgpp_quant_rows_view": (_I, [C.POINTER(QuantMatrix), C.c_int64, C.c_int64, C.POINTER(QuantMatrix)]),
+    "dgpp_fp4_check_cols": (_I, [C.c_int64, _I]),
+    "dgpp_fp4_rows_view": (_I, [C.POINTER(_lib.Fp4Matrix), C.c_int64, C.c_int64, C.POINTER(_lib.Fp4Matrix)]),
+    "dgpp_expert_view_from_quant": (_I, [C.POINTER(QuantMatrix), C.POINTER(_lib.MoeExpertView)]),
+    "dgpp_expert_view_from_fp4": (_I, [C.POINTER(_lib.Fp4Matrix), C.POINTER(_lib.MoeExpertView)]),
+}
+_typed = False
+
+
+def lib() -> C.CDLL:
+    global _typed
+    handle = _lib.load()
+    if not _typed:
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _typed = True
+    return handle
+
+
+def _check(rc: int) -> None:
+    if rc == _lib.OK:
+        return
+    msg = lib().dgpp_loader_last_error().decode()
+    if rc == _lib.INVALID_ARGUMENT:
+        raise ValueError(msg)
+    raise LoaderError(msg)
+
+
+class SafetensorsFile:
+    """A mapped checkpoint shard. Arrays returned by `array` alias the mapping: drop them before `close`."""
+
+    def __init__(self, path: str):
+        self._h = _P()
+        _check(lib().dgpp_safetensors_open(str(path).encode(), C.byref(self._h)))
+
+    def close(self, drop_page_cache: bool = False) -> None:
+        if self._h:
+            lib().dgpp_safetensors_close(self._h, 1 if drop_page_cache else 0)
+            self._h = _P()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __len__(self) -> int:
+        return lib().dgpp_safetensors_count(self._h)
+
+    def names(self):
+        return [lib().dgpp_safetensors_name(self._h, i).decode() for i in range(len(self))]
+
+    def find(self, name: str) -> TensorInfo:
+        info = TensorInfo()
+        _check(lib().dgpp_safetensors_find(self._h, name.encode(), C.byref(info)))
+        return info
+
+    def __contains__(self, name: str) -> bool:
+        info = TensorInfo()
+        return lib().dgpp_safetensors_find(self._h, name.encode(), C.byref(info)) == _lib.OK
+
+    def header_fold(self) -> int:
+        return lib().dgpp_safetensors_header_fold(self._h)
+
+    def metadata_json(self) -> str:
+        return lib().dgpp_safetensors_metadata_json(self._h).decode()
+
+    def prefetch(self, info: TensorInfo) -> None:
+        lib().dgpp_safetensors_prefetch(self._h, C.byref(info))
+
+    def discard(self, info: TensorInfo) -> None:
+        lib().dgpp_safetensors_discard(self._h, C.byref(info))
+
+    def array(self, name: str) -> np.ndarray:
+        """The tensor's bytes as a read-only numpy view of the mapping (bf16 as uint16 bit patterns,
+        fp8 / e8m0 as uint8)."""
+        info = self.find(name)
+        dt = np.dtype(_NUMPY[info.dtype])
+        if info.nbytes == 0:
+            return np.empty(info.dims(), dtype=dt)
+        buf = (C.c_uint8 * info.nbytes).from_address(info.data)
+        a = np.frombuffer(buf, dtype=dt).reshape(info.dims())
+        a.flags.writeable = False
+        return a
+
+
+def quant_scale_shifts(m: QuantMatrix):
+    rs, cs = _I(), _I()
+    ok = lib().dgpp_quant_scale_shifts(C.byref(m), C.byref(rs), C.byref(cs))
+    return bool(ok), rs.value, cs.value
+
+
+def quant_rows_view(m: QuantMatrix, row_start: int, rows: int) -> QuantMatrix:
+    out = QuantMatrix()
+    _check(lib().dgpp_quant_rows_view(C.byref(m), row_start, rows, C.byref(out)))
+    return out
+
+
+def fp4_rows_view(m, row_start: int, rows: int):
+    out = _lib.Fp4Matrix()
+    _check(lib().dgpp_fp4_rows_view(C.byref(m), row_start, rows, C.byref(out)))
+    return out
+
+
+def expert_view_from_quant(m: QuantMatrix):
+    out = _lib.MoeExpertView()
+    _check(lib().dgpp_expert_view_from_quant(C.byref(m), C.byref(out)))
+    return out
+
+
+def expert_view_from_fp4(m):
+    out = _lib.MoeExpertView()
+    _check(lib().dgpp_expert_view_from_fp4(C.byref(m), C.byref(out)))
+    return out

@@ -1,0 +1,116 @@
+/* Loader side of the quantized MoE path: a memory-mapped safetensors reader and the matrix views the
+ * launchers consume, so that a checkpoint's bytes reach the kernels untouched (no re-encoding, no copies
+ * on the host beyond the upload).
+ *
+ * Host code only: nothing here touches the GPU. Errors return DGPP_INVALID_ARGUMENT / DGPP_RUNTIME_ERROR
+ * (dgpp_amd.h) with the message in dgpp_loader_last_error() (thread-local).
+ *
+ * Reference counterparts: src/loaders/safetensors.hpp (SafetensorsFile, TensorInfo),
+ * src/common/dtypes.hpp:66-79 (dtype names), src/models/quant_matrix.hpp:16-96 (GlmQuantMatrix,
+ * quant_scale_shifts, quant_rows_view), :117-164 (GlmFp4Matrix, fp4_rows_view). */
+#ifndef DGPP_AMD_LOADER_H_
+#define DGPP_AMD_LOADER_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "dgpp_amd.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* dgpp_loader_last_error(void);
+
+/* Element types a header may name (src/common/dtypes.hpp:66-79; "F8" and "FP8" are aliases of F8_E4M3,
+ * "BOOL" of U8). Any other name fails the open. */
+enum {
+  DGPP_DT_F32 = 0,
+  DGPP_DT_F16 = 1,
+  DGPP_DT_BF16 = 2,
+  DGPP_DT_F8_E4M3 = 3,
+  DGPP_DT_I64 = 4,
+  DGPP_DT_I32 = 5,
+  DGPP_DT_U8 = 6,
+  DGPP_DT_I8 = 7,
+  DGPP_DT_F8_E8M0 = 8,
+  DGPP_DT_U32 = 9,
+  DGPP_DT_I16 = 10
+};
+/* Bytes of one element of `dtype`, 0 for an unknown code. */
+size_t dgpp_dtype_size(int dtype);
+
+#define DGPP_MAX_TENSOR_RANK 8
+
+/* One tensor of an open file (src/loaders/safetensors.hpp:22-49, TensorInfo). `data` points into the
+ * file's mapping and lives until the file is closed; an empty tensor's `data` is where its (empty) byte
+ * range starts, possibly the end of the mapping. */
+typedef struct DgppTensorInfo {
+  int32_t dtype;
+  int32_t rank;
+  int64_t shape[DGPP_MAX_TENSOR_RANK];
+  uint64_t numel;
+  uint64_t nbytes;
+  uint64_t file_offset; /* of the first byte, from the start of the file */
+  const void* data;
+} DgppTensorInfo;
+
+typedef struct DgppSafetensors DgppSafetensors;
+
+/* src/loaders/safetensors.hpp:103-127, :198-252: maps the file read-only and parses its header. The open
+ * fails (DGPP_RUNTIME_ERROR, nothing left mapped) on a header length outside the file, malformed JSON
+ * (numbers with leading zeros included), an unknown dtype, a shape or data_offsets entry that is not a
+ * non-negative integer, offsets outside the payload or out of order, an element count that overflows, or
+ * a byte range that is not numel * element size; more than DGPP_MAX_TENSOR_RANK dimensions likewise. */
+int dgpp_safetensors_open(const char* path, DgppSafetensors** out);
+/* src/loaders/safetensors.hpp:54-78 (close_mapping): unmaps; with drop_page_cache the file's pages are
+ * also dropped from the page cache (advisory). Every DgppTensorInfo::data of this file dangles afterwards. */
+void dgpp_safetensors_close(DgppSafetensors* f, int drop_page_cache);
+int dgpp_safetensors_count(const DgppSafetensors* f);
+/* Tensor names in ascending byte order of the name; NULL past the end. */
+const char* dgpp_safetensors_name(const DgppSafetensors* f, int index);
+/* DGPP_INVALID_ARGUMENT when the file has no tensor of that name (`out` untouched). */
+int dgpp_safetensors_find(const DgppSafetensors* f, const char* name, DgppTensorInfo* out);
+/* FNV-1a of the raw header JSON (src/loaders/safetensors.hpp:151-153): the shard's identity for caches. */
+uint64_t dgpp_safetensors_header_fold(const DgppSafetensors* f);
+/* The "__metadata__" object of the header as raw JSON text ("" when absent); lives until the close. */
+const char* dgpp_safetensors_metadata_json(const DgppSafetensors* f);
+/* src/loaders/safetensors.hpp:90-101: read-ahead before a one-pass copy of the tensor, and release of its
+ * pages (mapping and page cache) after it. Both advisory, page-rounded. */
+void dgpp_safetensors_prefetch(const DgppSafetensors* f, const DgppTensorInfo* t);
+void dgpp_safetensors_discard(const DgppSafetensors* f, const DgppTensorInfo* t);
+
+/* src/models/quant_matrix.hpp:16-52 (GlmQuantMatrix): an FP8-E4M3 matrix with an F32 block-scale grid, or
+ * (scales_e8m0) the MXFP8 byte grid. Pointers may be host or device addresses: the views below only do
+ * pointer arithmetic. */
+typedef struct DgppQuantMatrix {
+  const uint8_t* payload;     /* E4M3 [rows, cols] */
+  const float* scales;        /* F32 [ceil(rows / scale_block_rows), ceil(cols / scale_block_cols)] */
+  const uint8_t* scales_e8m0; /* the same grid as e8m0 bytes; exactly one of the two is set */
+  int64_t rows;
+  int64_t cols;
+  int32_t scale_block_rows;   /* 128 in the checkpoints; 1 with scale_block_cols >= cols is the channel grid */
+  int32_t scale_block_cols;
+} DgppQuantMatrix;
+
+/* src/models/quant_matrix.hpp:55-66: the grid as the launchers' log2 block sizes. Returns 1 and writes
+ * rs / cs when both block sizes are powers of two and the column block is at least 16, else 0. */
+int dgpp_quant_scale_shifts(const DgppQuantMatrix* m, int* rs, int* cs);
+/* src/models/quant_matrix.hpp:78-96: rows [row_start, row_start + rows) as a pointer view. A start that is
+ * not a multiple of the scale block's rows cannot re-anchor the grid and is rejected. */
+int dgpp_quant_rows_view(const DgppQuantMatrix* m, int64_t row_start, int64_t rows, DgppQuantMatrix* out);
+/* src/models/quant_matrix.hpp:144-164: K must be a positive multiple of the scale group (16 or 32); any row
+ * range is a pointer view (every row carries its own scales). */
+int dgpp_fp4_check_cols(int64_t cols, int scale_group);
+int dgpp_fp4_rows_view(const DgppFp4Matrix* m, int64_t row_start, int64_t rows, DgppFp4Matrix* out);
+
+/* One entry of the device expert table (DgppMoeExpertView, three per expert: gate, up, down) from a
+ * resident matrix. The FP8 form needs a grid dgpp_quant_scale_shifts accepts and F32 scales. */
+int dgpp_expert_view_from_quant(const DgppQuantMatrix* m, DgppMoeExpertView* out);
+int dgpp_expert_view_from_fp4(const DgppFp4Matrix* m, DgppMoeExpertView* out);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* DGPP_AMD_LOADER_H_ */

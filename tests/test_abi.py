@@ -27,6 +27,11 @@ def test_library_exports_every_declared_symbol():
     assert set(layer) == set(_lib.LAYER_SIGNATURES)
     for n in layer:
         assert hasattr(lib, n), f"{n} is declared in include/dgpp_amd_layer.h but not exported"
+    from dgpp_amd import loader
+    loader_names = declared_symbols("dgpp_amd_loader.h")
+    assert set(loader_names) == set(loader.SIGNATURES)
+    for n in loader_names:
+        assert hasattr(lib, n), f"{n} is declared in include/dgpp_amd_loader.h but not exported"
     assert lib.dgpp_target_arch() == b"gfx950"
 
 
@@ -71,7 +76,8 @@ def test_headers_compile_as_c_and_the_shim_as_cpp(tmp_path):
     root = Path(__file__).resolve().parent.parent
     inc = root / "include"
     c_src = tmp_path / "c_check.c"
-    c_src.write_text('#include "dgpp_amd.h"\n#include "dgpp_amd_layer.h"\nint main(void) { return sizeof(DgppMoeExpertView) == 96 ? 0 : 1; }\n')
+    c_src.write_text('#include "dgpp_amd.h"\n#include "dgpp_amd_layer.h"\n#include "dgpp_amd_loader.h"\n'
+                     "int main(void) { return sizeof(DgppMoeExpertView) == 96 && sizeof(DgppTensorInfo) == 104 ? 0 : 1; }\n")
     subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-I", str(inc), "-c", str(c_src), "-o", str(tmp_path / "c.o")],
                    check=True)
     rocm_inc = Path("/opt/rocm/include")

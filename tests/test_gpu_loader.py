@@ -1,0 +1,130 @@
+"""A checkpoint on disk drives the layer: per-expert tensors are written as a safetensors file (the names a
+compressed-tensors MoE export uses), read back through the memory-mapped reader, uploaded as they are, turned
+into expert-table entries by the loader's view helpers, and the layer's output equals — bit for bit — the
+output of the same weights handed over directly. Row slices of a resident matrix (the tensor-parallel split of
+gate / up) give the rows of the unsliced launch."""
+import struct
+
+import numpy as np
+import pytest
+
+import moe_data
+from dgpp_amd import _lib, launch as L, loader as LD, moe_layer as ML
+from gpu_util import DeviceMoe, dev, dev_empty, host, sync, view_table
+from test_gpu_moe_layer import make_layer
+
+pytestmark = pytest.mark.gpu
+
+_DT = {np.dtype(np.uint8): "U8", np.dtype(np.float32): "F32", np.dtype(np.uint16): "BF16"}
+PROJ = ("gate_proj", "up_proj", "down_proj")
+
+
+def write_checkpoint(path, tensors, dtypes=None):
+    """A safetensors file from numpy arrays (header JSON + payload, 8-byte padded header)."""
+    header, payload, at = {}, [], 0
+    for name, a in tensors.items():
+        a = np.ascontiguousarray(a)
+        dt = (dtypes or {}).get(name, _DT[a.dtype])
+        header[name] = {"dtype": dt, "shape": list(a.shape), "data_offsets": [at, at + a.nbytes]}
+        payload.append(a.tobytes())
+        at += a.nbytes
+    import json
+    h = json.dumps(header, separators=(",", ":"))
+    while (8 + len(h)) % 8:
+        h += " "
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(h)))
+        f.write(h.encode())
+        for b in payload:
+            f.write(b)
+
+
+@pytest.mark.parametrize("kind", ["fp8", "nvfp4", "mxfp4"])
+def test_layer_from_a_checkpoint_file_is_bitwise_the_layer_from_the_arrays(gpu, tmp_path, kind):
+    E, H, I, K, T = 6, 512, 128, 3, 5
+    p = moe_data.make_problem(E, H, I, K, T, kind, 8800, shared_kind=None, limit=float("inf"), std=0.05)
+    tensors, dtypes = {}, {}
+    for e, mats in enumerate(p.experts):
+        for m, proj in zip(mats, PROJ):
+            base = f"model.layers.3.mlp.experts.{e}.{proj}"
+            tensors[base + ".weight"] = m.payload
+            tensors[base + ".weight_scale"] = m.scales
+            if kind == "fp8":
+                dtypes[base + ".weight"] = "F8_E4M3"
+            elif kind == "nvfp4":
+                dtypes[base + ".weight_scale"] = "F8_E4M3"
+                tensors[base + ".weight_global"] = m.glob          # the device-side divisor, F32 [1]
+            else:
+                dtypes[base + ".weight_scale"] = "F8_E8M0"
+    path = str(tmp_path / "layer3.safetensors")
+    write_checkpoint(path, tensors, dtypes)
+
+    keep, entries = [], []
+    with LD.SafetensorsFile(path) as f:
+        assert len(f) == len(tensors)
+        for e in range(E):
+            for proj in PROJ:
+                base = f"model.layers.3.mlp.experts.{e}.{proj}"
+                w, s = f.find(base + ".weight"), f.find(base + ".weight_scale")
+                f.prefetch(w)
+                wd, sd = dev(np.array(f.array(base + ".weight"))), dev(np.array(f.array(base + ".weight_scale")))
+                f.discard(w)
+                keep += [wd, sd]
+                rows = w.dims()[0]
+                if kind == "fp8":
+                    assert w.dtype == LD.DT_F8_E4M3 and s.dtype == LD.DT_F32
+                    m = LD.QuantMatrix(wd.data_ptr(), sd.data_ptr(), None, rows, w.dims()[1], 128, 128)
+                    entries.append(LD.expert_view_from_quant(m))
+                else:
+                    group = 16 if kind == "nvfp4" else 32
+                    assert s.dtype == (LD.DT_F8_E4M3 if kind == "nvfp4" else LD.DT_F8_E8M0)
+                    gd = None
+                    if kind == "nvfp4":
+                        gd = dev(np.array(f.array(base + ".weight_global")))
+                        keep.append(gd)
+                    m = _lib.Fp4Matrix(wd.data_ptr(), sd.data_ptr(), gd.data_ptr() if gd is not None else None, rows,
+                                       w.dims()[1] * 2, group, 0, None)
+                    entries.append(LD.expert_view_from_fp4(m))
+    # the mapping is gone; the layer runs from the uploaded bytes alone
+    d = DeviceMoe(p)
+    ref_layer = make_layer(p, d, 1, 1.0, T)
+    d2 = DeviceMoe.__new__(DeviceMoe)
+    d2.p, d2.keep, d2.views, d2.x, d2.shared_view_base, d2.sh = p, keep, view_table(entries), d.x, -1, None
+    d2.fp4_group = d.fp4_group
+    got_layer = make_layer(p, d2, 1, 1.0, T)
+    want, got = dev_empty((T, H), np.uint16), dev_empty((T, H), np.uint16)
+    ref_layer.enqueue_decode(d.x, H, want, T)
+    got_layer.enqueue_decode(d.x, H, got, T)
+    sync()
+    assert np.array_equal(host(got, np.uint16), host(want, np.uint16))
+    assert host(want, np.uint16).any()
+    ref_layer.close()
+    got_layer.close()
+
+
+def test_row_slices_of_resident_matrices_give_the_rows_of_the_whole(gpu):
+    """The tensor-parallel split of gate / up is a row range of the resident matrix: a pointer view
+    (src/models/quant_matrix.hpp:78-96, :152-164) whose GEMV equals the rows of the unsliced launch."""
+    n, k, m = 512, 1024, 3
+    fp8 = moe_data.make_mat("fp8", n, k, 9100, 0.05)
+    nv = moe_data.make_mat("nvfp4", n, k, 9101, 0.05)
+    act = dev(moe_data.hg.normal_bf16(9102, (m, k)))
+    pd, sd = dev(fp8.payload), dev(fp8.scales)
+    whole = LD.QuantMatrix(pd.data_ptr(), sd.data_ptr(), None, n, k, 128, 128)
+    full, part = dev_empty((m, n), np.uint16), dev_empty((m, 256), np.uint16)
+    L.launch_scale_gemm_bf16(act, k, pd, sd, full, m, n, k, None)
+    v = LD.quant_rows_view(whole, 256, 256)
+    ok, rs, cs = LD.quant_scale_shifts(v)
+    assert ok and (rs, cs) == (7, 7)
+    L.launch_scale_gemm_bf16(act, k, v.payload, v.scales, part, m, 256, k, None)
+    sync()
+    assert np.array_equal(host(part, np.uint16), host(full, np.uint16)[:, 256:512])
+
+    p4, s4, g4 = dev(nv.payload), dev(nv.scales), dev(nv.glob)
+    whole4 = _lib.Fp4Matrix(p4.data_ptr(), s4.data_ptr(), g4.data_ptr(), n, k, 16, 0, None)
+    full4, part4 = dev_empty((m, n), np.uint16), dev_empty((m, 100), np.uint16)
+    L.launch_fp4_gemv_bf16(act, k, whole4, full4, m, n, k, None)
+    v4 = LD.fp4_rows_view(whole4, 37, 100)
+    L.launch_fp4_gemv_bf16(act, k, v4, part4, m, 100, k, None)
+    sync()
+    assert np.array_equal(host(part4, np.uint16), host(full4, np.uint16)[:, 37:137])

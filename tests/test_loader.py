@@ -1,0 +1,234 @@
+"""The loader side on the CPU: the memory-mapped safetensors reader against files written by the `safetensors`
+package and against the cases the reference's reader is tested with (tests/unit/safetensors_test.cpp:47-234:
+the round trip fixture, header lengths outside the file, numbers with leading zeros, invalid data_offsets and
+shapes, byte-count mismatches and overflows, scalar / empty tensors, dtype aliases with a padded header), and
+the matrix views' contracts (src/models/quant_matrix.hpp:55-96, :144-164)."""
+import ctypes as C
+import json
+import struct
+
+import numpy as np
+import pytest
+
+from dgpp_amd import _lib, loader as LD
+
+
+def write_raw(path, header: str, payload: bytes = b"", length=None):
+    h = header.encode()
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(h) if length is None else length))
+        f.write(h)
+        f.write(payload)
+    return str(path)
+
+
+def tensor_header(shape: str, offsets: str, dtype: str = "U8") -> str:
+    return '{"x":{"dtype":"%s","shape":%s,"data_offsets":%s}}' % (dtype, shape, offsets)
+
+
+def expect_rejected(tmp_path, header, payload_bytes, diagnostic, length=None):
+    p = write_raw(tmp_path / "bad.safetensors", header, bytes(i % 251 for i in range(payload_bytes)), length)
+    with pytest.raises(LD.LoaderError) as e:
+        LD.SafetensorsFile(p)
+    assert diagnostic in str(e.value), str(e.value)
+
+
+def test_reference_fixture_round_trip(tmp_path):
+    header = ('{"a_f32":{"dtype":"F32","shape":[2,3],"data_offsets":[0,24]},'
+              '"b_bf16":{"dtype":"BF16","shape":[4],"data_offsets":[24,32]},'
+              '"c_fp8":{"dtype":"F8_E4M3","shape":[2,2],"data_offsets":[32,36]}}')
+    f32 = np.array([1.0, -2.5, 3.25, 4.0, -5.0, 0.125], np.float32)
+    bf16 = (np.array([0.0, 0.5, 1.0, 1.5], np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    fp8 = np.array([0x38, 0x40, 0x7E, 0x00], np.uint8)
+    p = write_raw(tmp_path / "fixture.safetensors", header, f32.tobytes() + bf16.tobytes() + fp8.tobytes())
+    with LD.SafetensorsFile(p) as f:
+        assert len(f) == 3 and f.names() == ["a_f32", "b_bf16", "c_fp8"]
+        a = f.find("a_f32")
+        assert (a.dtype, a.dims(), a.numel, a.nbytes) == (LD.DT_F32, (2, 3), 6, 24)
+        assert a.file_offset == 8 + len(header)
+        assert np.array_equal(f.array("a_f32"), f32.reshape(2, 3))
+        assert np.array_equal(f.array("b_bf16"), bf16)
+        assert np.array_equal(f.array("c_fp8"), fp8.reshape(2, 2))
+        assert "missing" not in f
+        with pytest.raises(ValueError):
+            f.find("missing")
+        fold = 1469598103934665603
+        for c in header.encode():
+            fold = ((fold ^ c) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+        assert f.header_fold() == fold
+        assert f.metadata_json() == ""
+        f.prefetch(a)
+        f.discard(a)
+        assert np.array_equal(f.array("a_f32"), f32.reshape(2, 3)), "discarded pages are read again from the file"
+
+
+def test_files_written_by_the_safetensors_package(tmp_path):
+    st = pytest.importorskip("safetensors.numpy")
+    rng = np.random.default_rng(5)
+    tensors = {
+        "model.layers.0.mlp.experts.3.gate_proj.weight": rng.integers(0, 256, (64, 48), dtype=np.uint8),
+        "model.layers.0.mlp.experts.3.gate_proj.weight_scale": rng.random((1, 1), dtype=np.float32),
+        "ids": rng.integers(-5, 5, (7,), dtype=np.int64),
+        "half": rng.random((3, 5)).astype(np.float16),
+        "i32": rng.integers(-9, 9, (2, 2, 2), dtype=np.int32),
+        "i8": rng.integers(-9, 9, (5,), dtype=np.int8),
+        "scalar": np.array(3.5, dtype=np.float32),
+    }
+    path = str(tmp_path / "pkg.safetensors")
+    st.save_file(tensors, path, metadata={"format": "pt", "note": 'a "quoted" value'})
+    with LD.SafetensorsFile(path) as f:
+        assert sorted(tensors) == f.names()
+        for name, want in tensors.items():
+            got = f.array(name)
+            assert got.dtype == want.dtype and got.shape == want.shape and np.array_equal(got, want), name
+        meta = json.loads(f.metadata_json())
+        assert meta == {"format": "pt", "note": 'a "quoted" value'}
+
+
+def test_rejects_header_lengths_outside_file(tmp_path):
+    expect_rejected(tmp_path, "", 0, "header length", 2**64 - 1)
+    expect_rejected(tmp_path, "{}", 0, "header length", 3)
+    p = tmp_path / "tiny.safetensors"
+    p.write_bytes(b"\x00\x00")
+    with pytest.raises(LD.LoaderError, match="too small"):
+        LD.SafetensorsFile(str(p))
+    with pytest.raises(LD.LoaderError, match="cannot open"):
+        LD.SafetensorsFile(str(tmp_path / "absent.safetensors"))
+
+
+def test_rejects_leading_zero_numbers(tmp_path):
+    expect_rejected(tmp_path, tensor_header("[01]", "[0,1]"), 1, "malformed number")
+    expect_rejected(tmp_path, tensor_header("[1]", "[00,1]"), 1, "malformed number")
+
+
+@pytest.mark.parametrize("offsets", ["[-1,0]", "[-8,-4]", "[0,-1]", "[1,0]", "[1048576,0]", "[0,2]",
+                                     "[9223372036854775807,0]", "[18446744073709551615,0]", "[0.5,1]", '["0",1]',
+                                     "[false,1]", "[0,1,2]", "[0]", "[]", "{}"])
+def test_rejects_invalid_data_offsets(tmp_path, offsets):
+    expect_rejected(tmp_path, tensor_header("[1]", offsets), 1, "data_offsets")
+
+
+@pytest.mark.parametrize("shape", ["{}", "[-1]", "[0,-1]", "[1.5]", '["1"]', "[true]", "[18446744073709551615]"])
+def test_rejects_invalid_shapes(tmp_path, shape):
+    expect_rejected(tmp_path, tensor_header(shape, "[0,0]"), 0, "shape")
+
+
+def test_rejects_size_mismatch_and_overflow(tmp_path):
+    expect_rejected(tmp_path, tensor_header("[2]", "[0,4]", "F32"), 4, "shape/dtype")
+    expect_rejected(tmp_path, tensor_header("[1]", "[0,8]", "F32"), 8, "shape/dtype")
+    expect_rejected(tmp_path, tensor_header("[4294967296,4294967296]", "[0,0]"), 0, "element count")
+    wide = str((2**64 - 1) // 4 + 1)
+    expect_rejected(tmp_path, tensor_header("[" + wide + "]", "[0,0]", "F32"), 0, "shape/dtype")
+    # the ordered checked product: a later zero does not undo an earlier overflowing multiply
+    expect_rejected(tmp_path, tensor_header("[9223372036854775807,9223372036854775807,0]", "[0,0]"), 0, "element count")
+    expect_rejected(tmp_path, tensor_header("[1]", "[0,1]", "F4"), 1, "unknown dtype")
+    expect_rejected(tmp_path, "[1,2]", 0, "not an object")
+    expect_rejected(tmp_path, '{"x":{"dtype":"U8","shape":[1]}}', 1, "data_offsets")
+    expect_rejected(tmp_path, tensor_header("[1,1,1,1,1,1,1,1,1]", "[0,1]"), 1, "dimensions")
+
+
+def test_scalar_empty_and_payload_end_views(tmp_path):
+    header = ('{"scalar":{"dtype":"F32","shape":[],"data_offsets":[0,4]},'
+              '"empty":{"dtype":"BF16","shape":[2,0,3],"data_offsets":[4,4]},'
+              '"zero_first":{"dtype":"U8","shape":[0,5],"data_offsets":[4,4]}}')
+    p = write_raw(tmp_path / "s.safetensors", header, bytes([0, 1, 2, 3]))
+    with LD.SafetensorsFile(p) as f:
+        assert len(f) == 3
+        s = f.find("scalar")
+        assert (s.rank, s.numel, s.nbytes) == (0, 1, 4)
+        assert bytes((C.c_uint8 * 4).from_address(s.data)) == bytes([0, 1, 2, 3])
+        for name in ("empty", "zero_first"):
+            t = f.find(name)
+            assert t.numel == 0 and t.nbytes == 0 and t.file_offset == 8 + len(header) + 4   # the end of the file
+            assert f.array(name).size == 0
+    # a zero reached before any overflowing product remains a valid empty tensor
+    large = str((2**64 - 1) // 2)
+    p = write_raw(tmp_path / "e.safetensors", tensor_header("[0," + large + "," + large + "]", "[0,0]"))
+    with LD.SafetensorsFile(p) as f:
+        assert f.find("x").numel == 0
+
+
+@pytest.mark.parametrize("name,code,width", [("F32", LD.DT_F32, 4), ("F16", LD.DT_F16, 2), ("BF16", LD.DT_BF16, 2),
+                                             ("F8_E4M3", LD.DT_F8_E4M3, 1), ("F8", LD.DT_F8_E4M3, 1),
+                                             ("FP8", LD.DT_F8_E4M3, 1), ("I64", LD.DT_I64, 8), ("I32", LD.DT_I32, 4),
+                                             ("U8", LD.DT_U8, 1), ("I8", LD.DT_I8, 1), ("F8_E8M0", LD.DT_F8_E8M0, 1),
+                                             ("BOOL", LD.DT_U8, 1), ("U32", LD.DT_U32, 4), ("I16", LD.DT_I16, 2)])
+def test_dtype_aliases_and_padded_header(tmp_path, name, code, width):
+    header = tensor_header("[3]", "[0,%d]" % (3 * width), name)
+    while (8 + len(header)) % 8:
+        header += " "
+    payload = bytes(i % 251 for i in range(3 * width))
+    p = write_raw(tmp_path / "d.safetensors", header, payload)
+    with LD.SafetensorsFile(p) as f:
+        t = f.find("x")
+        assert (t.dtype, t.numel, t.nbytes) == (code, 3, 3 * width)
+        assert LD.lib().dgpp_dtype_size(code) == width
+        assert bytes((C.c_uint8 * t.nbytes).from_address(t.data)) == payload
+
+
+def test_duplicate_names_nested_metadata_and_escapes(tmp_path):
+    header = ('{"__metadata__":{"a":{"b":[1,2.5e3,null,true]},"k":"v"},'
+              '"t\\u0065nsor\\n":{"dtype":"U8","shape":[2],"data_offsets":[0,2],"extra":[{"x":1}]},'
+              '"dup":{"dtype":"U8","shape":[1],"data_offsets":[0,1]},'
+              '"dup":{"dtype":"U8","shape":[2],"data_offsets":[0,2]}}')
+    p = write_raw(tmp_path / "m.safetensors", header, b"\x07\x09")
+    with LD.SafetensorsFile(p) as f:
+        assert f.names() == ["dup", "tensor\n"]
+        assert f.find("dup").numel == 2, "the later descriptor of a repeated name stands"
+        assert list(f.array("tensor\n")) == [7, 9]
+        assert json.loads(f.metadata_json()) == {"a": {"b": [1, 2500.0, None, True]}, "k": "v"}
+    expect_rejected(tmp_path, '{"x":{"dtype":"U8","shape":[1],"data_offsets":[0,1]}} trailing', 1, "trailing")
+
+
+def test_quant_matrix_views_follow_the_scale_grid_contract():
+    rows, cols = 512, 384
+    payload = np.arange(rows * cols, dtype=np.uint32).astype(np.uint8)
+    scales = np.arange(4 * 3, dtype=np.float32)
+    m = LD.QuantMatrix(payload.ctypes.data, scales.ctypes.data, None, rows, cols, 128, 128)
+    assert LD.quant_scale_shifts(m) == (True, 7, 7)
+    v = LD.quant_rows_view(m, 256, 128)
+    assert v.payload == payload.ctypes.data + 256 * cols and v.scales == scales.ctypes.data + 2 * 3 * 4
+    assert (v.rows, v.cols, v.scale_block_rows, v.scale_block_cols) == (128, cols, 128, 128)
+    assert LD.quant_rows_view(m, 0, rows).payload == payload.ctypes.data
+    assert LD.quant_rows_view(m, 512, 0).rows == 0
+    for start, n in ((200, 100), (64, 64), (-128, 128), (384, 256), (0, 513), (0, -1)):
+        with pytest.raises(ValueError):
+            LD.quant_rows_view(m, start, n)
+    # the byte grid moves with the view too
+    e8 = np.zeros(rows * (cols // 32), np.uint8)
+    mx = LD.QuantMatrix(payload.ctypes.data, None, e8.ctypes.data, rows, cols, 1, 32)
+    assert LD.quant_scale_shifts(mx) == (True, 0, 5)
+    assert LD.quant_rows_view(mx, 7, 5).scales_e8m0 == e8.ctypes.data + 7 * (cols // 32)
+    # a channel grid and grids no launcher takes
+    assert LD.quant_scale_shifts(LD.QuantMatrix(None, None, None, 8, 4096, 1, 4096)) == (True, 0, 12)
+    assert LD.quant_scale_shifts(LD.QuantMatrix(None, None, None, 8, 64, 96, 128))[0] is False
+    assert LD.quant_scale_shifts(LD.QuantMatrix(None, None, None, 8, 64, 128, 8))[0] is False
+    view = LD.expert_view_from_quant(m)
+    assert (view.payload, view.scales, view.scale_shift_rows, view.scale_shift_cols) == (m.payload, m.scales, 7, 7)
+    with pytest.raises(ValueError):
+        LD.expert_view_from_quant(mx)
+
+
+def test_fp4_matrix_views():
+    rows, cols = 96, 256
+    payload, scales = np.zeros(rows * cols // 2, np.uint8), np.zeros(rows * cols // 16, np.uint8)
+    glob = np.ones(1, np.float32)
+    m = _lib.Fp4Matrix(payload.ctypes.data, scales.ctypes.data, glob.ctypes.data, rows, cols, 16, 0, None)
+    v = LD.fp4_rows_view(m, 33, 20)
+    assert v.payload == payload.ctypes.data + 33 * cols // 2 and v.scales == scales.ctypes.data + 33 * cols // 16
+    assert (v.rows, v.cols, v.scale_group, v.global_scale) == (20, cols, 16, glob.ctypes.data)
+    mx = _lib.Fp4Matrix(payload.ctypes.data, scales.ctypes.data, None, rows, cols, 32, 0, None)
+    assert LD.fp4_rows_view(mx, 95, 1).scales == scales.ctypes.data + 95 * cols // 32
+    for start, n in ((90, 7), (-1, 1), (0, 97)):
+        with pytest.raises(ValueError):
+            LD.fp4_rows_view(m, start, n)
+    with pytest.raises(ValueError):
+        LD.fp4_rows_view(_lib.Fp4Matrix(payload.ctypes.data, scales.ctypes.data, None, rows, 250, 16, 0, None), 0, 1)
+    with pytest.raises(ValueError):
+        LD.fp4_rows_view(_lib.Fp4Matrix(payload.ctypes.data, scales.ctypes.data, None, rows, cols, 64, 0, None), 0, 1)
+    e = LD.expert_view_from_fp4(m)
+    assert (e.payload, e.fp4_scales, e.fp4_global, e.fp4_group) == (m.payload, m.scales, glob.ctypes.data, 16)
+    e = LD.expert_view_from_fp4(mx)
+    assert (e.fp4_global, e.fp4_group) == (None, 32)
+    with pytest.raises(ValueError):
+        LD.expert_view_from_fp4(_lib.Fp4Matrix(payload.ctypes.data, scales.ctypes.data, None, rows, cols, 16, 0, None))
