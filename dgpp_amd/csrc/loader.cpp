@@ -540,6 +540,99 @@ int dgpp_fp4_rows_view(const DgppFp4Matrix* m, int64_t row_start, int64_t rows, 
   return DGPP_OK;
 }
 
+namespace {
+int64_t gcd64(int64_t a, int64_t b) {
+  while (b != 0) {
+    const int64_t t = a % b;
+    a = b;
+    b = t;
+  }
+  return a < 0 ? -a : a;
+}
+// The sliced axis' new block size, or 0 when the slice is not one this library takes.
+int64_t slice_block(const DgppQuantMatrix* m, int axis, int64_t start, int64_t count) {
+  if (!m || (axis != 0 && axis != 1) || m->scale_block_rows <= 0 || m->scale_block_cols <= 0) return 0;
+  const int64_t extent = axis == 0 ? m->rows : m->cols;
+  if (start < 0 || count <= 0 || count > extent || start > extent - count) return 0;
+  const int64_t block = axis == 0 ? m->scale_block_rows : m->scale_block_cols;
+  const int64_t g = gcd64(block, gcd64(start, count));
+  if ((g & (g - 1)) != 0) return 0;
+  if (g < 32 && g != block) return 0;   // the grid launchers take blocks of 32, 64 and 128 (or the parent's own)
+  return g;
+}
+}  // namespace
+
+int64_t dgpp_quant_slice_scale_count(const DgppQuantMatrix* m, int axis, int64_t start, int64_t count) {
+  const int64_t g = slice_block(m, axis, start, count);
+  if (g == 0) return -1;
+  if (axis == 0) return ((count + g - 1) / g) * ((m->cols + m->scale_block_cols - 1) / m->scale_block_cols);
+  return ((m->rows + m->scale_block_rows - 1) / m->scale_block_rows) * ((count + g - 1) / g);
+}
+
+int dgpp_quant_slice(const DgppQuantMatrix* m, int axis, int64_t start, int64_t count, uint8_t* payload_out,
+                     float* scales_out, DgppQuantMatrix* out) {
+  if (!m || !payload_out || !scales_out || !out) return fail(DGPP_INVALID_ARGUMENT, "quant_slice: null argument");
+  if (!m->payload || !m->scales)
+    return fail(DGPP_INVALID_ARGUMENT, "quant_slice: takes an E4M3 payload with an F32 scale grid (host addresses)");
+  const int64_t g = slice_block(m, axis, start, count);
+  if (g == 0)
+    return fail(DGPP_INVALID_ARGUMENT,
+                "quant_slice: the range must lie inside the matrix and re-block to a grid the launchers take "
+                "(gcd(block, start, count) a power of two, at least 32 unless it is the parent's block)");
+  const int64_t parent_cols = (m->cols + m->scale_block_cols - 1) / m->scale_block_cols;
+  DgppQuantMatrix v = *m;
+  v.payload = payload_out;
+  v.scales = scales_out;
+  v.scales_e8m0 = nullptr;
+  if (axis == 0) {
+    std::memcpy(payload_out, m->payload + start * m->cols, static_cast<size_t>(count * m->cols));
+    const int64_t blocks = (count + g - 1) / g;
+    for (int64_t i = 0; i < blocks; ++i) {
+      const int64_t parent = (start + i * g) / m->scale_block_rows;
+      std::memcpy(scales_out + i * parent_cols, m->scales + parent * parent_cols, static_cast<size_t>(parent_cols) * sizeof(float));
+    }
+    v.rows = count;
+    v.scale_block_rows = static_cast<int32_t>(g);
+  } else {
+    for (int64_t r = 0; r < m->rows; ++r)
+      std::memcpy(payload_out + r * count, m->payload + r * m->cols + start, static_cast<size_t>(count));
+    const int64_t blocks = (count + g - 1) / g;
+    const int64_t grid_rows = (m->rows + m->scale_block_rows - 1) / m->scale_block_rows;
+    for (int64_t br = 0; br < grid_rows; ++br)
+      for (int64_t j = 0; j < blocks; ++j)
+        scales_out[br * blocks + j] = m->scales[br * parent_cols + (start + j * g) / m->scale_block_cols];
+    v.cols = count;
+    v.scale_block_cols = static_cast<int32_t>(g);
+  }
+  *out = v;
+  return DGPP_OK;
+}
+
+int dgpp_fp4_cols_slice(const DgppFp4Matrix* m, int64_t col_start, int64_t cols, uint8_t* payload_out,
+                        uint8_t* scales_out, DgppFp4Matrix* out) {
+  if (!m || !payload_out || !scales_out || !out) return fail(DGPP_INVALID_ARGUMENT, "fp4_cols_slice: null argument");
+  int rc = dgpp_fp4_check_cols(m->cols, m->scale_group);
+  if (rc != DGPP_OK) return rc;
+  rc = dgpp_fp4_check_cols(cols, m->scale_group);
+  if (rc != DGPP_OK) return rc;
+  if (!m->payload || !m->scales) return fail(DGPP_INVALID_ARGUMENT, "fp4_cols_slice: null payload or scales");
+  if (col_start < 0 || col_start % m->scale_group != 0 || cols > m->cols || col_start > m->cols - cols)
+    return fail(DGPP_INVALID_ARGUMENT, "fp4_cols_slice: the range must start on a scale-group boundary inside the matrix");
+  const int64_t src_bytes = m->cols / 2, dst_bytes = cols / 2;
+  const int64_t src_scales = m->cols / m->scale_group, dst_scales = cols / m->scale_group;
+  for (int64_t r = 0; r < m->rows; ++r) {
+    std::memcpy(payload_out + r * dst_bytes, m->payload + r * src_bytes + col_start / 2, static_cast<size_t>(dst_bytes));
+    std::memcpy(scales_out + r * dst_scales, m->scales + r * src_scales + col_start / m->scale_group,
+                static_cast<size_t>(dst_scales));
+  }
+  DgppFp4Matrix v = *m;
+  v.payload = payload_out;
+  v.scales = scales_out;
+  v.cols = cols;
+  *out = v;
+  return DGPP_OK;
+}
+
 int dgpp_expert_view_from_quant(const DgppQuantMatrix* m, DgppMoeExpertView* out) {
   if (!m || !out) return fail(DGPP_INVALID_ARGUMENT, "expert_view_from_quant: null argument");
   int rs = 0, cs = 0;

@@ -49,6 +49,9 @@ SIGNATURES = {
     "dgpp_quant_rows_view": (_I, [C.POINTER(QuantMatrix), C.c_int64, C.c_int64, C.POINTER(QuantMatrix)]),
     "dgpp_fp4_check_cols": (_I, [C.c_int64, _I]),
     "dgpp_fp4_rows_view": (_I, [C.POINTER(_lib.Fp4Matrix), C.c_int64, C.c_int64, C.POINTER(_lib.Fp4Matrix)]),
+    "dgpp_quant_slice_scale_count": (C.c_int64, [C.POINTER(QuantMatrix), _I, C.c_int64, C.c_int64]),
+    "dgpp_quant_slice": (_I, [C.POINTER(QuantMatrix), _I, C.c_int64, C.c_int64, _P, _P, C.POINTER(QuantMatrix)]),
+    "dgpp_fp4_cols_slice": (_I, [C.POINTER(_lib.Fp4Matrix), C.c_int64, C.c_int64, _P, _P, C.POINTER(_lib.Fp4Matrix)]),
     "dgpp_expert_view_from_quant": (_I, [C.POINTER(QuantMatrix), C.POINTER(_lib.MoeExpertView)]),
     "dgpp_expert_view_from_fp4": (_I, [C.POINTER(_lib.Fp4Matrix), C.POINTER(_lib.MoeExpertView)]),
 }
@@ -162,3 +165,28 @@ def expert_view_from_fp4(m):
     out = _lib.MoeExpertView()
     _check(lib().dgpp_expert_view_from_fp4(C.byref(m), C.byref(out)))
     return out
+
+
+def quant_slice(m: QuantMatrix, axis: int, start: int, count: int):
+    """A host copy of a row (axis 0) or column (axis 1) range with the sliced axis' grid re-blocked.
+    Returns (payload uint8 [rows, cols], scales float32 [grid], QuantMatrix over them)."""
+    n = lib().dgpp_quant_slice_scale_count(C.byref(m), axis, start, count)
+    if n < 0:
+        n = 0
+    rows, cols = (count, m.cols) if axis == 0 else (m.rows, count)
+    payload = np.empty((rows, cols) if n else (0, 0), dtype=np.uint8)
+    scales = np.empty(n, dtype=np.float32)
+    out = QuantMatrix()
+    _check(lib().dgpp_quant_slice(C.byref(m), axis, start, count, payload.ctypes.data, scales.ctypes.data, C.byref(out)))
+    grid_rows = -(-out.rows // out.scale_block_rows)
+    return payload, scales.reshape(grid_rows, -1), out
+
+
+def fp4_cols_slice(m, col_start: int, cols: int):
+    """A host copy of a column range of an NVFP4 / MXFP4 matrix (whole scale groups)."""
+    ok = cols > 0 and m.scale_group in (16, 32) and cols % m.scale_group == 0
+    payload = np.empty((m.rows, cols // 2) if ok else (0, 0), dtype=np.uint8)
+    scales = np.empty((m.rows, cols // m.scale_group) if ok else (0, 0), dtype=np.uint8)
+    out = _lib.Fp4Matrix()
+    _check(lib().dgpp_fp4_cols_slice(C.byref(m), col_start, cols, payload.ctypes.data, scales.ctypes.data, C.byref(out)))
+    return payload, scales, out

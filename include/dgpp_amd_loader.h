@@ -104,6 +104,24 @@ int dgpp_quant_rows_view(const DgppQuantMatrix* m, int64_t row_start, int64_t ro
 int dgpp_fp4_check_cols(int64_t cols, int scale_group);
 int dgpp_fp4_rows_view(const DgppFp4Matrix* m, int64_t row_start, int64_t rows, DgppFp4Matrix* out);
 
+/* Slices that are NOT pointer views: a copy of a HOST-resident matrix's range along rows (axis 0) or columns
+ * (axis 1) into caller buffers — the tensor-parallel split of the down projection (columns), or a row split
+ * that starts inside a scale block. The sliced axis of an F32 grid is re-blocked at
+ * g = gcd(block, start, count): every new block lies inside one parent block and takes that block's scale
+ * (src/models/quant_matrix.hpp:28-34; the reference's model loaders slice at gcd(128, I / world)), so each
+ * element dequantizes to exactly the value it had in the parent. The result must still be a grid the launchers
+ * take (g a power of two and at least 32, or the parent's own block), else DGPP_INVALID_ARGUMENT.
+ * payload_out: count * cols (axis 0) or rows * count (axis 1) bytes; scales_out:
+ * dgpp_quant_slice_scale_count floats. `out` describes the copy (its pointers are the two buffers). */
+int64_t dgpp_quant_slice_scale_count(const DgppQuantMatrix* m, int axis, int64_t start, int64_t count);
+int dgpp_quant_slice(const DgppQuantMatrix* m, int axis, int64_t start, int64_t count, uint8_t* payload_out,
+                     float* scales_out, DgppQuantMatrix* out);
+/* Column range of a HOST-resident NVFP4 / MXFP4 matrix (src/models/quant_matrix.hpp:140-150: it starts on a
+ * scale-group boundary and spans whole groups). payload_out: rows * cols / 2 bytes; scales_out:
+ * rows * cols / scale_group bytes. The global scale pointer is carried over. */
+int dgpp_fp4_cols_slice(const DgppFp4Matrix* m, int64_t col_start, int64_t cols, uint8_t* payload_out,
+                        uint8_t* scales_out, DgppFp4Matrix* out);
+
 /* One entry of the device expert table (DgppMoeExpertView, three per expert: gate, up, down) from a
  * resident matrix. The FP8 form needs a grid dgpp_quant_scale_shifts accepts and F32 scales. */
 int dgpp_expert_view_from_quant(const DgppQuantMatrix* m, DgppMoeExpertView* out);

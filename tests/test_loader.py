@@ -232,3 +232,55 @@ def test_fp4_matrix_views():
     assert (e.fp4_global, e.fp4_group) == (None, 32)
     with pytest.raises(ValueError):
         LD.expert_view_from_fp4(_lib.Fp4Matrix(payload.ctypes.data, scales.ctypes.data, None, rows, cols, 16, 0, None))
+
+
+@pytest.mark.parametrize("axis,start,count", [(0, 96, 96), (0, 64, 192), (0, 32, 32), (0, 128, 256), (1, 96, 96),
+                                              (1, 192, 192), (1, 32, 160), (1, 0, 384), (0, 0, 512)])
+def test_quant_slices_reblock_the_grid_and_keep_every_dequantized_value(axis, start, count):
+    """A slice that starts inside a scale block is re-blocked at gcd(block, start, count) with the parent block's
+    scale replicated (src/models/quant_matrix.hpp:28-34): each element dequantizes to exactly its parent value."""
+    import np_ref
+    from dgpp_amd import hostgen as hg
+    rows, cols = 512, 384
+    w = hg.f32_to_bf16(hg.normal_f32(0x5EED + axis, (rows, cols), 0.05))
+    payload, scales = hg.encode_fp8_blocks(w, 128, 128)
+    m = LD.QuantMatrix(payload.ctypes.data, scales.ctypes.data, None, rows, cols, 128, 128)
+    sp, ss, v = LD.quant_slice(m, axis, start, count)
+    g = int(np.gcd(128, np.gcd(start, count)))
+    want_blocks = (g, 128) if axis == 0 else (128, g)
+    assert (v.scale_block_rows, v.scale_block_cols) == want_blocks
+    assert (v.rows, v.cols) == ((count, cols) if axis == 0 else (rows, count))
+    ok, rs, cs = LD.quant_scale_shifts(v)
+    assert ok and (1 << rs, 1 << cs) == want_blocks
+    parent = np_ref.dequant_fp8(payload, scales, 7, 7)
+    part = np_ref.dequant_fp8(sp, ss, rs, cs)
+    sl = (slice(start, start + count), slice(None)) if axis == 0 else (slice(None), slice(start, start + count))
+    assert np.array_equal(part, parent[sl])
+
+
+def test_quant_slice_and_fp4_cols_slice_contracts():
+    import np_ref
+    from dgpp_amd import hostgen as hg
+    rows, cols = 256, 256
+    payload, scales = hg.encode_fp8_blocks(hg.f32_to_bf16(hg.normal_f32(77, (rows, cols), 0.05)), 128, 128)
+    m = LD.QuantMatrix(payload.ctypes.data, scales.ctypes.data, None, rows, cols, 128, 128)
+    for axis, start, count in ((1, 16, 16), (1, 24, 24), (0, 100, 60), (0, 48, 48), (0, -1, 4), (1, 200, 100), (2, 0, 32),
+                               (0, 0, 0)):
+        with pytest.raises(ValueError):
+            LD.quant_slice(m, axis, start, count)   # blocks under 32 or not a power of two / outside the matrix
+    assert LD.lib().dgpp_quant_slice_scale_count(C.byref(m), 1, 64, 64) == 2 * 1
+    e8 = np.zeros((rows, cols // 32), np.uint8)
+    with pytest.raises(ValueError):
+        LD.quant_slice(LD.QuantMatrix(payload.ctypes.data, None, e8.ctypes.data, rows, cols, 1, 32), 1, 0, 64)
+
+    for group, enc in ((16, hg.encode_nvfp4), (32, hg.encode_mxfp4)):
+        res = enc(hg.normal_f32(78 + group, (rows, cols), 0.05))
+        p4, s4 = res[0], res[1]
+        glob = np.ones(1, np.float32)
+        m4 = _lib.Fp4Matrix(p4.ctypes.data, s4.ctypes.data, glob.ctypes.data if group == 16 else None, rows, cols, group, 0, None)
+        sp, ss, v = LD.fp4_cols_slice(m4, 64, 96)
+        assert (v.rows, v.cols, v.scale_group, v.global_scale) == (rows, 96, group, m4.global_scale)
+        assert np.array_equal(np_ref.dequant_fp4(sp, ss, group), np_ref.dequant_fp4(p4, s4, group)[:, 64:160])
+        for start, n in ((8, 32), (0, 40), (224, 64), (-32, 32), (0, 0)):
+            with pytest.raises(ValueError):
+                LD.fp4_cols_slice(m4, start, n)
