@@ -203,6 +203,21 @@ __global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
   }
 }
 
+// Ranks by (key, slot) as one integer: key << 10 | slot (slots < 1024, keys <= n_experts < 2^16), unique per slot.
+__device__ __forceinline__ int32_t slot_sort_key(int key, int slot) { return (key << 10) | slot; }
+// Rank of a slot among `padded` such integers (a multiple of 4; pad entries hold INT_MAX): how many are below
+// `mine`. Four per LDS read, one compare and one add each: the ranking is bound by the vector ALU.
+__device__ __forceinline__ int slot_rank(const int32_t* __restrict__ sort_keys, int padded, int32_t mine) {
+  const int4* k4 = reinterpret_cast<const int4*>(sort_keys);
+  int pos = 0;
+#pragma unroll 4
+  for (int o = 0; o < padded / 4; ++o) {
+    const int4 v = k4[o];
+    pos += (v.x < mine) + (v.y < mine) + (v.z < mine) + (v.w < mine);
+  }
+  return pos;
+}
+
 // Selection and slot order in ONE launch for a decode batch: one wavefront per token selects, the
 // block then ranks the slots by (expert, slot) exactly as slot_order_kernel does (key = expert id,
 // or n_experts for the token's shared slot). tokens * 64 threads, tokens <= 16.
@@ -211,7 +226,7 @@ __global__ __launch_bounds__(1024) void router_select_order_kernel(
     const float* __restrict__ scores, const float* __restrict__ biased, int32_t* __restrict__ ids,
     float* __restrict__ weights, int32_t* __restrict__ order, int tokens, int n_experts, int top_k, float scaling,
     int norm_topk, int shared_early) {
-  __shared__ int32_t keys[16 * 17];
+  __shared__ __align__(16) int32_t keys[16 * 17 + 4];
   const int t = threadIdx.x >> 6, lane = threadIdx.x & (kWaveSize - 1);
   const size_t row = static_cast<size_t>(t) * n_experts;
   int id;
@@ -220,21 +235,18 @@ __global__ __launch_bounds__(1024) void router_select_order_kernel(
   if (lane < top_k) {
     ids[static_cast<size_t>(t) * top_k + lane] = id;
     weights[static_cast<size_t>(t) * top_k + lane] = w;
-    keys[t * (top_k + 1) + lane] = id;
+    keys[t * (top_k + 1) + lane] = slot_sort_key(id, t * (top_k + 1) + lane);
   } else if (lane == top_k) {
-    keys[t * (top_k + 1) + lane] = n_experts;
+    keys[t * (top_k + 1) + lane] = slot_sort_key(n_experts, t * (top_k + 1) + lane);
   }
   if (order == nullptr) return;
-  __syncthreads();
   const int slots = tokens * (top_k + 1);
+  const int padded = (slots + 3) & ~3;
+  if (threadIdx.x < padded - slots) keys[slots + threadIdx.x] = INT_MAX;
+  __syncthreads();
   const int s = threadIdx.x;
   if (s >= slots) return;
-  const int mine = keys[s];
-  int pos = 0;
-  for (int o = 0; o < slots; ++o) {
-    const int k = keys[o];
-    pos += (k < mine) || (k == mine && o < s);
-  }
+  int pos = slot_rank(keys, padded, keys[s]);
   if (shared_early) {
     const int routed = tokens * top_k;
     pos = pos < routed ? pos + (pos < tokens ? pos : tokens) : 2 * (pos - routed) + 1;
@@ -396,23 +408,22 @@ __global__ __launch_bounds__(kSegThreads) void segment_kernel(const int32_t* __r
 __global__ void slot_order_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ order,
                                   int32_t* __restrict__ runs, int slots, int top_k, int n_experts,
                                   int shared_early) {
-  extern __shared__ int32_t so_lds[];  // keys [slots]; with runs: sorted [slots], groups [slots]
+  extern __shared__ __align__(16) int32_t so_lds[];  // keys [slots padded to 4]; with runs: sorted [slots], groups [slots]
+  const int padded = (slots + 3) & ~3;
   int32_t* keys = so_lds;
-  int32_t* sorted = keys + slots;
+  int32_t* sorted = keys + padded;
   int32_t* groups = sorted + slots;
   const int s = threadIdx.x;
   if (s < slots) {
     const int t = s / (top_k + 1), j = s - t * (top_k + 1);
-    keys[s] = j < top_k ? ids[static_cast<size_t>(t) * top_k + j] : n_experts;
+    keys[s] = slot_sort_key(j < top_k ? ids[static_cast<size_t>(t) * top_k + j] : n_experts, s);
+  } else if (s < padded) {
+    keys[s] = INT_MAX;
   }
   __syncthreads();
   if (s < slots) {
-    const int mine = keys[s];
-    int pos = 0;
-    for (int o = 0; o < slots; ++o) {
-      const int k = keys[o];
-      pos += (k < mine) || (k == mine && o < s);
-    }
+    const int mine = keys[s] >> 10;
+    int pos = slot_rank(keys, padded, keys[s]);
     if (shared_early) {
       const int tokens = slots / (top_k + 1), routed = tokens * top_k;
       pos = pos < routed ? pos + (pos < tokens ? pos : tokens) : 2 * (pos - routed) + 1;
@@ -444,6 +455,52 @@ __global__ void slot_order_kernel(const int32_t* __restrict__ ids, int32_t* __re
     if (s == slots - 1)
       for (int i = base + groups[s]; i < slots / (kTileRows + 1) + 1; ++i) list[i] = -1;
   }
+}
+
+// The same order from several blocks (no run list): every block builds all sort keys in its LDS and ranks its own
+// 32 slots with four lanes each, so the ranking's vector work spreads over CUs instead of queueing on one.
+constexpr int kOrderThreads = 128;
+__global__ __launch_bounds__(kOrderThreads) void slot_order_wide_kernel(const int32_t* __restrict__ ids,
+                                                                        int32_t* __restrict__ order, int slots, int top_k,
+                                                                        int n_experts, int shared_early) {
+  extern __shared__ __align__(16) int32_t sw_lds[];   // sort keys [slots padded to 4]
+  const int padded = (slots + 3) & ~3;
+  // at most 1024 slots: eight per thread, every id load issued before the first is used
+  int32_t v[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int i = threadIdx.x + u * kOrderThreads;
+    const int c = i < slots ? i : 0;
+    const int t = c / (top_k + 1), j = c - t * (top_k + 1);
+    v[u] = ids[static_cast<size_t>(t) * top_k + (j < top_k ? j : 0)];
+    v[u] = i < slots ? slot_sort_key(j < top_k ? v[u] : n_experts, i) : INT_MAX;
+  }
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int i = threadIdx.x + u * kOrderThreads;
+    if (i < padded) sw_lds[i] = v[u];
+  }
+  __syncthreads();
+  // four lanes per slot, each over a quarter of the keys (16-byte reads, interleaved), then a quad sum
+  const int gid = blockIdx.x * kOrderThreads + threadIdx.x;
+  const int s = gid >> 2, q = gid & 3;
+  const int sc = s < slots ? s : slots - 1;
+  const int32_t mine = sw_lds[sc];
+  const int4* k4 = reinterpret_cast<const int4*>(sw_lds);
+  int pos = 0;
+#pragma unroll 4
+  for (int o = q; o < padded / 4; o += 4) {
+    const int4 v = k4[o];
+    pos += (v.x < mine) + (v.y < mine) + (v.z < mine) + (v.w < mine);
+  }
+  pos += __shfl_xor(pos, 1);
+  pos += __shfl_xor(pos, 2);
+  if (s >= slots || q != 0) return;
+  if (shared_early) {
+    const int tokens = slots / (top_k + 1), routed = tokens * top_k;
+    pos = pos < routed ? pos + (pos < tokens ? pos : tokens) : 2 * (pos - routed) + 1;
+  }
+  order[pos] = s;
 }
 
 constexpr int kTileThreads = 256;
@@ -653,8 +710,14 @@ hipError_t run_segment(const int32_t* ids, int tokens, int top_k, int n_experts,
 
 hipError_t run_slot_order(const int32_t* ids, int32_t* order, int32_t* runs, int slots, int top_k, int n_experts,
                           int shared_early, hipStream_t stream) {
+  if (runs == nullptr && slots > kOrderThreads) {
+    const size_t wide_lds = static_cast<size_t>((slots + 3) & ~3) * sizeof(int32_t);
+    hipLaunchKernelGGL(slot_order_wide_kernel, dim3((4 * slots + kOrderThreads - 1) / kOrderThreads), dim3(kOrderThreads), wide_lds,
+                       stream, ids, order, slots, top_k, n_experts, shared_early);
+    return hipGetLastError();
+  }
   const int threads = (slots + kWaveSize - 1) / kWaveSize * kWaveSize;
-  const size_t lds = static_cast<size_t>(slots) * sizeof(int32_t) * (runs ? 3 : 1);
+  const size_t lds = (static_cast<size_t>((slots + 3) & ~3) + (runs ? 2 * static_cast<size_t>(slots) : 0)) * sizeof(int32_t);
   hipLaunchKernelGGL(slot_order_kernel, dim3(1), dim3(threads), lds, stream, ids, order, runs, slots, top_k, n_experts,
                      shared_early);
   return hipGetLastError();
