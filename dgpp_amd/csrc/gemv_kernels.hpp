@@ -772,6 +772,7 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
 // LDS a block may take without giving up residency (16 KB of staged activations) and by the
 // accumulators a lane holds.
 constexpr int kGateUpRun = 2;
+constexpr int kGateUpRunBatch = 4;
 constexpr int kDownRun = 4;
 inline int run_cap_for(const SlotArgs& a, int max_run) {
   if (a.order == nullptr && !a.match) return 1;   // slots in layout order and no way to find the sharers
@@ -792,7 +793,8 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   if (a.once && a.slots > a.top_k + 1) steps = 2;   // a decode batch of 2 - 8 tokens: measured best (one token: 1)
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
-  const int cap = run_cap_for(a, kGateUpRun);
+  // Larger batches (many slots per expert, an order given): runs of four where the rows fit the stage.
+  const int cap = run_cap_for(a, (!a.once && a.order != nullptr) ? kGateUpRunBatch : kGateUpRun);
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
     const bool split = tune_get(kTuneSplitStage) != 1 && a.k <= 8 * kSplitStageVecs * kBlockThreads &&
@@ -809,6 +811,9 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
       else if (split) go(mc, std::true_type{}, std::false_type{});
       else go(mc, std::false_type{}, std::false_type{});
     };
+    if constexpr (NB <= 4) {   // two accumulators per slot and matrix: four slots fit the registers up to four loads per pass
+      if (cap >= kGateUpRunBatch) return go(std::integral_constant<int, kGateUpRunBatch>{}, std::false_type{}, std::false_type{});
+    }
     if (cap >= kGateUpRun) go_m(std::integral_constant<int, kGateUpRun>{});
     else go_m(std::integral_constant<int, 1>{});
   });
