@@ -96,7 +96,7 @@ def main():
     layers, keep = [], []
     cfg = L.make_config(H, I, nE, K, n_shared_experts=0, routed_scaling_factor=1.0, swiglu_limit=float("inf"),
                         router_mode=L.ROUTER_SOFTMAX_TOPK)
-    max_t = 8
+    max_t = max(8, args.tokens)
     d0 = [t.to(dev) for t in host_layer0]
     for l in range(nL):
         if l == 0:

@@ -262,7 +262,7 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
   a.top_k = top_k;
   a.limit = limit;
   a.shared_view_base = -1;
-  a.once = slots <= 8 * (top_k + 1);   // a decode batch of at most 8 tokens: few slots can share an expert
+  a.once = slots <= 16 * (top_k + 1);   // a decode batch of at most 16 tokens: few slots share an expert (measured up to there)
   const int tokens = top_k >= 0 ? slots / (top_k + 1) : 0;
   a.match = order == nullptr && tokens > 1 && tokens * top_k <= 64;
   return a;

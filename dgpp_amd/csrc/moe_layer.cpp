@@ -186,7 +186,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   }
   // The token-major down kernel fuses the accumulation but reads an expert once per slot; the slot kernel reads
   // it once per run of slots. Token-major while few slots can share an expert (small batches), runs beyond.
-  const bool token_major = !has_shared() && dgpp_tune_get(4) != 1 && tokens * K * 4 <= cfg_.n_experts;
+  const bool token_major = !has_shared() && dgpp_tune_get(4) != 1 && tokens * K * 2 <= cfg_.n_experts;
   const bool sh_args = has_shared() && !w_.shared_in_table;
   const int n_sh = has_shared() ? w_.shared_inter : 0;
   const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
