@@ -185,7 +185,7 @@ def main():
             for l in range(nL):
                 full(l)                                       # leaves ids / weights in the layer's scratch
                 o = None
-                if T * K > 64:      # as the layer does: small batches need no slot order (sharers found by ballot)
+                if T * K > 128:     # as the layer does: small batches need no slot order (sharers found by ballot)
                     o = torch.empty(slots, dtype=torch.int32, device=dev)
                     L.launch_moe_slot_order(layers[l].ids_ptr, o, slots, K, nE, stream)
                 orders.append(o)

@@ -264,7 +264,7 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
   a.shared_view_base = -1;
   a.once = slots <= 16 * (top_k + 1);   // a decode batch of at most 16 tokens: few slots share an expert (measured up to there)
   const int tokens = top_k >= 0 ? slots / (top_k + 1) : 0;
-  a.match = order == nullptr && tokens > 1 && tokens * top_k <= 64;
+  a.match = order == nullptr && tokens > 1 && tokens * top_k <= 128;
   return a;
 }
 

@@ -219,30 +219,48 @@ __device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& ru
         }
       }
     } else if (a.match && key0 >= 0) {
-      // No order given, a small decode batch (tokens * top_k <= 64): the slots that use this expert are found
-      // with one ballot over the routed ids (an expert occurs at most once per token, so they sit in
+      // No order given, a small decode batch (tokens * top_k <= 128): the slots that use this expert are found
+      // with two ballots over the routed ids (an expert occurs at most once per token, so they sit in
       // different tokens). The first of every MAXM of them, in (token, j) order, leads the run.
       const int lane = threadIdx.x & (kWave - 1);
       const int tk = (a.slots / (a.top_k + 1)) * a.top_k;
-      const int theirs = lane < tk ? a.ids[lane] : -1;
-      const unsigned long long mask = __builtin_amdgcn_ballot_w64(theirs == key0);
+      const int lo = lane < tk ? a.ids[lane] : -1;
+      const int hi = lane + kWave < tk ? a.ids[lane + kWave] : -1;
+      const unsigned long long m0 = __builtin_amdgcn_ballot_w64(lo == key0);
+      const unsigned long long m1 = __builtin_amdgcn_ballot_w64(hi == key0);
       const int mine = token0 * a.top_k + (slot0 - token0 * (a.top_k + 1));
-      const int before = __builtin_popcountll(mask & ((1ull << mine) - 1ull));
+      auto below = [](unsigned long long m, int n) {   // set bits of m at positions < n, n in 0 .. 64
+        return n <= 0 ? 0 : __builtin_popcountll(n >= 64 ? m : m & ((1ull << n) - 1ull));
+      };
+      const int before = below(m0, mine) + below(m1, mine - kWave);
       if (before % MAXM != 0) return false;
-      unsigned long long rest = mine >= 63 ? 0ull : mask >> (mine + 1);
+      auto next_after = [&](int at) {                  // the next sharer's index above `at`, or -1
+        if (at < kWave - 1) {
+          const unsigned long long r = m0 >> (at + 1);
+          if (r != 0ull) return at + 1 + __builtin_ctzll(r);
+        }
+        const int from = at < kWave ? 0 : at - kWave + 1;
+        if (from < kWave) {
+          const unsigned long long r = m1 >> from;
+          if (r != 0ull) return kWave + from + __builtin_ctzll(r);
+        }
+        return -1;
+      };
       int at = mine;
+      bool alive = true;
 #pragma unroll
       for (int r = 1; r < MAXM; ++r) {
         run.slot[r] = slot0;
         run.token[r] = token0;
-        if (rest != 0ull) {
-          const int skip = __builtin_ctzll(rest);
-          at += skip + 1;
-          rest = skip >= 63 ? 0ull : rest >> (skip + 1);
+        const int nxt = alive ? next_after(at) : -1;
+        if (nxt >= 0) {
+          at = nxt;
           const int t = at / a.top_k;
           run.slot[r] = t * (a.top_k + 1) + (at - t * a.top_k);
           run.token[r] = t;
           run.m = r + 1;
+        } else {
+          alive = false;
         }
       }
     } else if (a.match) {

@@ -133,7 +133,7 @@ GlmMoeLayer::~GlmMoeLayer() {
 bool GlmMoeLayer::needs_order(int tokens) const {
   if (tokens <= 1 || tokens * (cfg_.top_k + 1) > 1024) return false;
   if (dgpp_tune_get(6) == 1) return true;
-  return tokens * cfg_.top_k > 64;
+  return tokens * cfg_.top_k > 128;   // up to 128 routed slots the gate/up kernel finds the sharers of an expert by ballot
 }
 
 void GlmMoeLayer::check_tokens(int tokens) const {

@@ -44,7 +44,7 @@ const char* dgpp_target_arch(void);
  * any weight load is issued (default: activation loads, first weight pass, LDS commit); key 4: 1 keeps
  * the layer driver on the two-launch down + accumulate form; key 5: 2 moves the GEMV launchers to the
  * matrix-core form; key 6: 1 makes the layer driver compute the slot order for small decode batches too
- * (default: batches of at most 64 routed slots find the sharers of an expert by ballot, no order);
+ * (default: batches of at most 128 routed slots find the sharers of an expert by ballot, no order);
  * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
  * blocks, dgpp_launch_moe_select_gate_up_swiglu). Outputs do not depend on keys 1 - 4, 6 and 7; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
