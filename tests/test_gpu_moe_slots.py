@@ -121,6 +121,10 @@ CASES = [
     (32, 1024, 256, 8, 4, "mxfp4", None, None, float("inf")),
     (8, 512, 128, 2, 6, "mxfp4", "fp8", 384, 7.0),
     (9, 256, 64, 3, 2, "mxfp4", "mxfp4", 64, 10.0),
+    # more than 64 routed slots without an order: the sharers of an expert sit in both ballot words
+    (12, 256, 64, 8, 12, "mxfp4", None, None, float("inf")),
+    (24, 384, 96, 8, 16, "fp8", None, None, float("inf")),
+    (10, 512, 64, 8, 9, "nvfp4", "fp8", 128, 10.0),
 ]
 
 
