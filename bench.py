@@ -34,7 +34,7 @@ GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
 # HBM-side bytes per launch of the two GEMV kernels at the default workload (T = 8, 256 experts), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the library's plain copy kernel (the summary under
 # profiles/ holds the commands and the raw counters). A counter cannot be read from inside this process.
-MEASURED_TRAFFIC = {"gate_up": 260.7e6, "down": 138.5e6}
+MEASURED_TRAFFIC = {"gate_up": 260.3e6, "down": 138.5e6}
 DOWN_BYTES = H * I // 2 + H * I // 32
 
 
@@ -96,7 +96,7 @@ def main():
     layers, keep = [], []
     cfg = L.make_config(H, I, nE, K, n_shared_experts=0, routed_scaling_factor=1.0, swiglu_limit=float("inf"),
                         router_mode=L.ROUTER_SOFTMAX_TOPK)
-    max_t = max(8, args.tokens)
+    max_t = max(16, args.tokens)
     d0 = [t.to(dev) for t in host_layer0]
     for l in range(nL):
         if l == 0:
@@ -233,7 +233,7 @@ def main():
     main_res = measure(T, args.steps, args.warmup, args.only)
     others = {}
     if not args.only and not args.tune and not args.no_others:
-        for t in (1, 4, 8):
+        for t in (1, 4, 8, 16):
             if t != T:
                 others[f"T{t}"] = measure(t, args.steps, args.warmup)
 
