@@ -8,6 +8,7 @@
 #include <unordered_map>
 
 #include "../../include/dgpp_amd.h"
+#include "capi_errors.hpp"
 #include "gemv_kernels.hpp"
 #include "moe_misc.hpp"
 
@@ -303,6 +304,12 @@ int grouped(int fmt, const uint16_t* act, size_t act_stride, const DgppMoeSegmen
 extern "C" {
 
 const char* dgpp_last_error(void) { return g_last_error.c_str(); }
+}  // extern "C"
+namespace dgpp_amd {
+int report_invalid(const std::string& what) { return fail_arg(what); }
+int report_hip(hipError_t err, const char* who) { return finish(err, who); }
+}  // namespace dgpp_amd
+extern "C" {
 const char* dgpp_target_arch(void) { return "gfx950"; }
 int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
   const char* who = "probe copy";

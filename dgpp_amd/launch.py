@@ -397,6 +397,25 @@ def launch_mma_gemv_fp8_swiglu_f32(gate, up, limit, act_stride, w, scales, out, 
                                                            m, n, k, out_stride, rs, cs, _stream(stream)))
 
 
+def launch_mxfp8_quantize_rows(x, x_stride, rows, k, codes, scales, stream=None):
+    _check(_lib.load().dgpp_launch_mxfp8_quantize_rows(_p(x), x_stride, rows, k, _p(codes), _p(scales), _stream(stream)))
+
+
+def launch_minimax_swiglu_mxfp8_rows(gate, up, stride, rows, k, alpha, limit, codes, scales, stream=None):
+    _check(_lib.load().dgpp_launch_minimax_swiglu_mxfp8_rows(_p(gate), _p(up), stride, rows, k, alpha, limit, _p(codes),
+                                                             _p(scales), _stream(stream)))
+
+
+def launch_mxfp8_gemm_bf16(a, a_scales, w, w_scales, out, m, n, k, stream=None, out_stride=0, output_tile=0):
+    _check(_lib.load().dgpp_launch_mxfp8_gemm_bf16(_p(a), _p(a_scales), _p(w), _p(w_scales), _p(out), m, n, k,
+                                                   _stream(stream), out_stride, output_tile))
+
+
+def launch_mxfp8_gemm_f32(a, a_scales, w, w_scales, out, m, n, k, stream=None, out_stride=0, output_tile=0):
+    _check(_lib.load().dgpp_launch_mxfp8_gemm_f32(_p(a), _p(a_scales), _p(w), _p(w_scales), _p(out), m, n, k,
+                                                  _stream(stream), out_stride, output_tile))
+
+
 def launch_dense_mma_fp4_prod_bf16(act, act_stride, seg, views, which, out, m, n, k, stream=None, fp4_group=16):
     _check(_lib.load().dgpp_launch_dense_mma_fp4_prod_bf16(_p(act), act_stride, _p(seg), _p(views), which, _p(out), m, n, k,
                                                            _stream(stream), fp4_group))

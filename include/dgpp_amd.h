@@ -436,6 +436,36 @@ int dgpp_launch_fp8_dequant_blocks_e8m0(const uint8_t* payload, const uint8_t* s
                                         uint16_t* out_bf16, int64_t rows, int64_t cols,
                                         void* stream, int rs, int cs);
 
+/* ---- activation-quantized MXFP8 (W8A8) form ---------------------------------------------------------------------
+ * The weights' MXFP8 payload meets activations quantized to MXFP8 on the fly; the products run on the
+ * block-scaled matrix-core instruction (V_MFMA_SCALE_F32_16X16X128_F8F6F4, e8m0 scale per 32 values of
+ * either operand), FP32 accumulation. Its numerics are those of src/kernels/mxfp8_gemm.cu, not of the
+ * BF16-activation launchers above: the activations carry MXFP8 rounding.
+ *
+ * src/kernels/mxfp8_gemm.hpp:8-12, src/kernels/mxfp8_gemm.cu:246-256: BF16 x [rows, k] (row stride
+ * x_stride elements) -> E4M3 codes [rows, k] and e8m0 scales [rows, k / 32]. A group's scale is
+ * 2^ceil(log2(amax / 448)) (at least 2^-127; a zero group stores byte 0 and zero codes), its codes
+ * e4m3_rne(x / scale). DGPP_INVALID_ARGUMENT unless k is a positive multiple of 32 and x_stride is at
+ * least k and a multiple of 4; x must be 8-byte and codes 4-byte aligned; at most 65535 rows. */
+int dgpp_launch_mxfp8_quantize_rows(const uint16_t* x, size_t x_stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                    void* stream);
+/* src/kernels/mxfp8_gemm.hpp:14-18, src/kernels/mxfp8_gemm.cu:258-268: the same quantizer behind the clamped
+ * SwiGLU of the MiniMax dense/shared MLP, v = bf16(g' * sigmoid(alpha * g') * (u' + 1)) with g' = min(g, limit),
+ * u' = clamp(u, -limit, limit); sigmoid = 1 / (1 + 2^(-alpha * g' * log2 e)) through the hardware's
+ * exponential and reciprocal. gate and up share `stride`. */
+int dgpp_launch_minimax_swiglu_mxfp8_rows(const uint16_t* gate, const uint16_t* up, size_t stride, int rows, int k, float alpha,
+                                          float limit, uint8_t* codes, uint8_t* scales, void* stream);
+/* src/kernels/mxfp8_gemm.hpp:20-31, src/kernels/mxfp8_gemm.cu:217-243, :270-279: out[m, n] = A[m, k] * W[n, k]^T,
+ * both operands row-major E4M3 with e8m0 scales [rows, k / 32]; out_stride in output elements (0 -> n).
+ * DGPP_INVALID_ARGUMENT unless k is a positive multiple of 64, out_stride >= n and output_tile is one of
+ * 0, 8, 16, 32, 64 (a diagnostic of the reference's kernel: accepted, and without effect here); both payloads
+ * 16-byte aligned. An output element's value depends on its own two rows and k only, never on m, n or
+ * the rows sharing the launch; the bf16 form is the f32 form rounded to nearest even. */
+int dgpp_launch_mxfp8_gemm_bf16(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales,
+                                uint16_t* out, int m, int n, int k, void* stream, size_t out_stride, int output_tile);
+int dgpp_launch_mxfp8_gemm_f32(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales, float* out,
+                               int m, int n, int k, void* stream, size_t out_stride, int output_tile);
+
 /* ---- host-side weight encoders and synthetic data (no GPU involved) ------------------------------------------ */
 /* Scalar codecs, src/common/dtypes.hpp:83-190, src/kernels/latent_format.hpp:117-162. */
 float dgpp_bf16_to_f32(uint16_t bits);

@@ -366,6 +366,25 @@ inline void launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t*
   detail::check(dgpp_launch_mma_gemv_fp8_swiglu_f32(gate, up, limit, act_stride, w, scales, out, m, n, k, out_stride, rs, cs,
                                                     stream));
 }
+// src/kernels/mxfp8_gemm.hpp:11-31.
+inline void launch_mxfp8_quantize_rows(const uint16_t* x, size_t x_stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                       hipStream_t stream) {
+  detail::check(dgpp_launch_mxfp8_quantize_rows(x, x_stride, rows, k, codes, scales, stream));
+}
+inline void launch_minimax_swiglu_mxfp8_rows(const uint16_t* gate, const uint16_t* up, size_t stride, int rows, int k,
+                                             float alpha, float limit, uint8_t* codes, uint8_t* scales, hipStream_t stream) {
+  detail::check(dgpp_launch_minimax_swiglu_mxfp8_rows(gate, up, stride, rows, k, alpha, limit, codes, scales, stream));
+}
+inline void launch_mxfp8_gemm_bf16(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales,
+                                   uint16_t* out, int m, int n, int k, hipStream_t stream, size_t out_stride = 0,
+                                   int output_tile = 0) {
+  detail::check(dgpp_launch_mxfp8_gemm_bf16(a, a_scales, w, w_scales, out, m, n, k, stream, out_stride, output_tile));
+}
+inline void launch_mxfp8_gemm_f32(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales,
+                                  float* out, int m, int n, int k, hipStream_t stream, size_t out_stride = 0,
+                                  int output_tile = 0) {
+  detail::check(dgpp_launch_mxfp8_gemm_f32(a, a_scales, w, w_scales, out, m, n, k, stream, out_stride, output_tile));
+}
 inline void launch_dense_mma_fp4_prod_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* seg,
                                            const MoeExpertView* views, int which, uint16_t* out, int m, int n, int k,
                                            hipStream_t stream, int fp4_group = kFp4Group) {

@@ -494,6 +494,68 @@ void orc_moe_forward(const uint16_t* x, int64_t x_stride, const int32_t* ids, co
   }
 }
 
+// ---- activation-quantized MXFP8 form ---------------------------------------------------------
+
+void orc_mxfp8_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, uint8_t* codes, uint8_t* scales) {
+  const int groups = k / 32;
+  for (int r = 0; r < rows; ++r)
+    for (int g = 0; g < groups; ++g) {
+      const uint16_t* src = x + static_cast<size_t>(r) * stride + static_cast<size_t>(g) * 32;
+      float maximum = 0.f;
+      for (int i = 0; i < 32; ++i) maximum = std::max(maximum, std::fabs(orc_bf16_to_f32(src[i])));
+      // ceil(log2(maximum / 448)) off the float's fields: 448 = 1.75 * 2^8, so the ceiling is the
+      // exponent less 8, plus one when the significand exceeds 1.75.
+      const uint32_t u = f2u(maximum);
+      const int field = static_cast<int>((u >> 23) & 0xFF);
+      const int exponent = std::max(-127, field - 127 - 8 + ((u & 0x7FFFFFu) > 0x600000u ? 1 : 0));
+      // 2^-exponent is a float for every exponent the rule can produce (-127 .. 120).
+      const float inverse = static_cast<float>(std::ldexp(1.0, -exponent));
+      for (int i = 0; i < 32; ++i)
+        codes[static_cast<size_t>(r) * k + static_cast<size_t>(g) * 32 + i] = orc_f32_to_e4m3(orc_bf16_to_f32(src[i]) * inverse);
+      scales[static_cast<size_t>(r) * groups + g] = static_cast<uint8_t>(exponent + 127);
+    }
+}
+
+void orc_swiglu_oai(const uint16_t* gate, const uint16_t* up, int64_t stride, int rows, int k, float alpha, float limit,
+                    double* exact, uint16_t* rounded) {
+  for (int r = 0; r < rows; ++r)
+    for (int c = 0; c < k; ++c) {
+      const size_t at = static_cast<size_t>(r) * stride + c, to = static_cast<size_t>(r) * k + c;
+      const double g = std::min(bf16d(gate[at]), static_cast<double>(limit));
+      const double u = std::min(std::max(bf16d(up[at]), -static_cast<double>(limit)), static_cast<double>(limit));
+      const double v = g / (1.0 + std::exp(-static_cast<double>(alpha) * g)) * (u + 1.0);
+      if (exact) exact[to] = v;
+      if (rounded) rounded[to] = d2bf16(v);
+    }
+}
+
+void orc_mxfp8_gemm(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales, int m, int n, int k,
+                    double* out, double* out_abs) {
+  const int groups = k / 32;
+  std::vector<double> ad(static_cast<size_t>(m) * k), wd(static_cast<size_t>(n) * k);
+  for (int r = 0; r < m; ++r)
+    for (int c = 0; c < k; ++c)
+      ad[static_cast<size_t>(r) * k + c] = std::ldexp(static_cast<double>(orc_e4m3_to_f32(a[static_cast<size_t>(r) * k + c])),
+                                                       static_cast<int>(a_scales[static_cast<size_t>(r) * groups + c / 32]) - 127);
+  for (int r = 0; r < n; ++r)
+    for (int c = 0; c < k; ++c)
+      wd[static_cast<size_t>(r) * k + c] = std::ldexp(static_cast<double>(orc_e4m3_to_f32(w[static_cast<size_t>(r) * k + c])),
+                                                       static_cast<int>(w_scales[static_cast<size_t>(r) * groups + c / 32]) - 127);
+  for (int r = 0; r < m; ++r)
+    for (int c = 0; c < n; ++c) {
+      double sum = 0, abs_sum = 0;
+      const double* ar = &ad[static_cast<size_t>(r) * k];
+      const double* wr = &wd[static_cast<size_t>(c) * k];
+      for (int i = 0; i < k; ++i) {
+        const double prod = ar[i] * wr[i];
+        sum += prod;
+        abs_sum += std::fabs(prod);
+      }
+      out[static_cast<size_t>(r) * n + c] = sum;
+      if (out_abs) out_abs[static_cast<size_t>(r) * n + c] = abs_sum;
+    }
+}
+
 void orc_compare_bf16(const uint16_t* got, const double* oracle, int64_t n, double ulp_budget,
                       double floor_frac, OrcCompare* rep) {
   compare_impl<uint16_t>(got, oracle, n, ulp_budget, floor_frac, rep, [](uint16_t b) { return bf16d(b); });

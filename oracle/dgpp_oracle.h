@@ -19,6 +19,8 @@
  *   swiglu            compiled reference forward (I = 1 degenerate chain) + edge KATs
  *   accumulation      numpy float32 fma emulation through float64 (exact for one fma)
  *   moe forward       compiled reference glm_moe_ref_forward, FP8 / NVFP4 / MXFP4
+ *   mxfp8 quantizer   the closed form of the reference's own kernel test in numpy float64, all finite BF16
+ *   mxfp8 gemm        numpy float64 brute force; swiglu-oai: closed-form points + numpy
  */
 #ifndef DGPP_ORACLE_H
 #define DGPP_ORACLE_H
@@ -136,6 +138,26 @@ void orc_moe_forward(const uint16_t* x, int64_t x_stride, const int32_t* ids, co
                      int tokens, int top_k, int hidden, int inter, int shared_inter,
                      const OrcMatrix* experts, const OrcMatrix* shared, float swiglu_limit,
                      int threads, double* out_raw, uint16_t* out_bf16);
+
+/* ---- activation-quantized MXFP8 form (its own numerics contract: the activations carry MXFP8 rounding) ---- */
+/* BF16 x [rows, k] (row stride in elements) -> E4M3 codes [rows, k], e8m0 scales [rows, k / 32]: per
+ * 32-group the exponent is max(-127, ceil(log2(amax / 448))) (a zero group: -127, byte 0), codes are
+ * e4m3_rne_sat(x * 2^-exponent). src/kernels/mxfp8_gemm.cu:58-79.
+ * Pinned by the closed form the reference's own test checks its kernel with, evaluated in numpy float64
+ * (ceil(log2(amax / 448)), tests/cuda/mxfp8_gemm_test.cu:77-92) over every finite BF16 pattern and the
+ * 446 / 448 / 450 * 2^e boundary rows of that test (:96-123); the code conversion is orc_f32_to_e4m3. */
+void orc_mxfp8_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, uint8_t* codes, uint8_t* scales);
+/* The clamped SwiGLU the fused quantizer applies first, in double:
+ * min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + 1); `exact` (nullable) unrounded,
+ * `rounded` (nullable) as BF16, both [rows, k] dense. src/kernels/mxfp8_gemm.cu:37-56 states the formula,
+ * tests/cuda/mxfp8_gemm_test.cu:155-170 the double form used here. Pinned by closed-form points
+ * (g = 0, u = -1, saturated clamps) and numpy. */
+void orc_swiglu_oai(const uint16_t* gate, const uint16_t* up, int64_t stride, int rows, int k, float alpha, float limit,
+                    double* exact, uint16_t* rounded);
+/* out[m, n] = sum_k e4m3(a) 2^(sa - 127) * e4m3(w) 2^(sw - 127) in double, and (nullable) the same sum of
+ * magnitudes for the forward-error bound. tests/cuda/mxfp8_gemm_test.cu:222-236. Pinned by numpy brute force. */
+void orc_mxfp8_gemm(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales, int m, int n, int k,
+                    double* out, double* out_abs);
 
 /* ---- comparators ---------------------------------------------------------------- */
 typedef struct {
