@@ -403,9 +403,28 @@ def main():
             L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
             L.launch_moe_round_bf16(out, routed, cT * cH, stream)
 
+        # The shared expert in the activation-quantized form: x and the SwiGLU output go through the MXFP8 row
+        # quantizers and the three projections run on the block-scaled matrix-core instruction (different
+        # numerics from the legs above: the activations carry MXFP8 rounding; SwiGLU-OAI with alpha 1.702, limit 7).
+        xq, aq = (torch.empty((cT, d), dtype=torch.uint8, device=dev) for d in (cH, cSI))
+        xq_s, aq_s = (torch.empty((cT, d // 32), dtype=torch.uint8, device=dev) for d in (cH, cSI))
+
+        def shared_w8a8(i):
+            L.launch_mxfp8_quantize_rows(x, cH, cT, cH, xq, xq_s, stream)
+            L.launch_mxfp8_gemm_bf16(xq, xq_s, sh[0][0], sh[0][1], g_d, cT, cSI, cH, stream)
+            L.launch_mxfp8_gemm_bf16(xq, xq_s, sh[1][0], sh[1][1], u_d, cT, cSI, cH, stream)
+            L.launch_minimax_swiglu_mxfp8_rows(g_d, u_d, cSI, cT, cSI, 1.702, 7.0, aq, aq_s, stream)
+            L.launch_mxfp8_gemm_f32(aq, aq_s, sh[2][0], sh[2][1], shared_down, cT, cH, cSI, stream)
+            L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
+            L.launch_moe_round_bf16(out, routed, cT * cH, stream)
+
         def full(i):
             routed_part(i)
             shared_mc(i)
+
+        def full_w8a8(i):
+            routed_part(i)
+            shared_w8a8(i)
 
         n_steps = max(args.steps // 10, 5)
         per_expert = 3 * cI * cH // 2 + 3 * cI * cH // 16 + 12
@@ -417,7 +436,9 @@ def main():
         for name, fn, nb in (("layer", full, nbytes), ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
                              ("routed_only_matrix_core", routed_mc, uniq * per_expert + cT * cH * 6),
                              ("shared_only_gemv_launchers", shared_part, shared_bytes + cT * cH * 4),
-                             ("shared_only", shared_mc, shared_bytes + cT * cH * 4)):
+                             ("shared_only", shared_mc, shared_bytes + cT * cH * 4),
+                             ("shared_only_w8a8_scaled_matrix_core", shared_w8a8, shared_bytes + cT * cH * 4),
+                             ("layer_with_w8a8_shared", full_w8a8, nbytes)):
             sec = time_graph(fn, n_steps, 2)
             res[name] = {"us": sec * 1e6, "algorithmic_bytes": nb, "gbps": nb / sec / 1e9,
                          "frac_of_peak": nb / sec / 1e9 / HBM_PEAK_GBPS}

@@ -21,8 +21,6 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kQuantThreads = 256;
-constexpr int kGemmWaves = 4;
-constexpr int kGemmThreads = kGemmWaves * 64;
 
 // ---- quantizers ----------------------------------------------------------------------------------
 
@@ -116,116 +114,153 @@ __device__ __forceinline__ void put<uint16_t>(uint16_t* p, float v) { *p = f32_t
 
 // out[m, n] = A[m, k] * W[n, k]^T. A block owns 16 rows of W over all of k and MT * 16 rows of A.
 //
-// One matrix-core step covers 128 of k. Lane (r, g) = (lane % 16, lane / 16) hands over, for row r of
-// its 16, the 16 bytes at k = 16 g of the step in the operand's registers 0-3 and the 16 bytes at
-// k = 64 + 16 g in registers 4-7 (so one load instruction of the wave reads 64 contiguous bytes of each
-// of the 16 rows), and the scale byte of the row's k-block g of the step, which the hardware applies to
-// that block wherever its bytes sit (block b of a row is held by lanes 2 (b % 2) and 2 (b % 2) + 1, in
-// registers 4 (b / 2) .. 4 (b / 2) + 3). W is the first operand, a 16-row tile of A the second; the lane
-// receives out[a row r][w rows 4 g .. 4 g + 3].
-// The block's four waves take the steps in pairs, wave w the pairs w, w + 4, ...; their partial sums
-// are added in wave order by wave 0. The chain of every output element is therefore fixed by k alone,
-// whatever m, n and the rows that share a launch (src/kernels/mxfp8_gemm.hpp:23 asks the same of the
-// reference's row geometries).
+// One matrix-core step covers 128 of k. Its operand layout: lane (r, g) = (lane % 16, lane / 16) holds,
+// for row r of its 16, the 16 bytes at k = 16 g of the step in registers 0-3 and the 16 bytes at
+// k = 64 + 16 g in registers 4-7, and supplies the scale byte of the row's k-block g of the step, which
+// the hardware applies to that block wherever its bytes sit. W is the first operand, a 16-row tile of A
+// the second; the lane receives out[a row r][w rows 4 g .. 4 g + 3].
+//
+// Loading in that layout would ask the memory pipe for 64 bytes of 16 different rows per instruction,
+// which it serves at about half its streaming rate. A step's 16 x 128 bytes of either operand are
+// therefore loaded row-major (two instructions of 8 rows x 128 contiguous bytes), parked in a
+// wavefront-private LDS region and read back in operand layout; the region is XOR-swizzled so that the
+// writes and the reads both touch every bank once.
+//
+// The block's WAVES waves split k: wave w takes the steps w, w + WAVES, ..., and the partial sums are
+// added in wave order (tile t by wave t). The chain of every output element is therefore fixed by k alone
+// (WAVES is chosen from k), whatever m, n and the rows that share a launch
+// (src/kernels/mxfp8_gemm.hpp:23 asks the same of the reference's row geometries).
 // Rows past n or m are clamped to the last one and never stored; bytes past k contribute zeros.
-template <typename Out, int MT>
-__global__ __launch_bounds__(kGemmThreads) void mxfp8_gemm_kernel(
+constexpr int kStepUnits = 128;   // 16-byte units of one step of one operand tile: 16 rows x 128 bytes
+
+// The swizzled place of 16-byte piece `piece` (0-7) of row `row` (0-15) in a region.
+__device__ __forceinline__ int region_unit(int row, int piece) { return row * 8 + (piece ^ ((row >> 1) & 7)); }
+
+// This lane's two row-major loads of a step: rows (lane / 8) and 8 + (lane / 8) of the 16 that start at
+// row0 (clamped to the last row), piece lane % 8 of the step's 128 bytes; zeros past k.
+template <bool NT>
+__device__ __forceinline__ void issue_step(const uint8_t* __restrict__ base, int row0, int rows, int k, int step,
+                                           u32x4 (&t)[2]) {
+  const int lane = threadIdx.x & 63;
+  const int at = step * 128 + (lane & 7) * 16;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = min(row0 + 8 * i + (lane >> 3), rows - 1);
+    const u32x4* src = reinterpret_cast<const u32x4*>(base + static_cast<size_t>(row) * k + (at < k ? at : 0));
+    const u32x4 v = NT ? __builtin_nontemporal_load(src) : *src;
+    t[i] = at < k ? v : u32x4{0u, 0u, 0u, 0u};
+  }
+}
+__device__ __forceinline__ void commit_step(u32x4* __restrict__ region, const u32x4 (&t)[2]) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) region[region_unit(8 * i + (lane >> 3), lane & 7)] = t[i];
+}
+__device__ __forceinline__ v8i step_operand(const u32x4* __restrict__ region) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  return as_operand(region[region_unit(r, g)], region[region_unit(r, 4 + g)]);
+}
+
+template <typename Out, int MT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void mxfp8_gemm_kernel(
     const uint8_t* __restrict__ a, const uint8_t* __restrict__ a_scales, const uint8_t* __restrict__ w,
     const uint8_t* __restrict__ w_scales, Out* __restrict__ out, int m, int n, int k, size_t out_stride) {
-  __shared__ float4 fold[kGemmWaves - 1][MT][64];
+  static_assert(WAVES >= MT, "one folding wave per tile");
+  // Two regions per wave while the steps run, the partial sums of every wave afterwards.
+  constexpr int kStageUnits = WAVES * 2 * kStepUnits, kFoldUnits = WAVES * MT * 64;
+  __shared__ u32x4 lds[kStageUnits > kFoldUnits ? kStageUnits : kFoldUnits];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16, m0 = blockIdx.y * (16 * MT);
   const int kblocks = k >> 5;
   const int steps = (kblocks + 3) >> 2;
+  u32x4* region = lds + wave * 2 * kStepUnits;
 
-  const int w_row = min(n0 + r, n - 1);
-  const uint8_t* wp = w + static_cast<size_t>(w_row) * k;
-  const uint8_t* wsp = w_scales + static_cast<size_t>(w_row) * kblocks;
-  const uint8_t* ap[MT];
+  const uint8_t* wsp = w_scales + static_cast<size_t>(min(n0 + r, n - 1)) * kblocks;
   const uint8_t* asp[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int a_row = min(m0 + t * 16 + r, m - 1);
-    ap[t] = a + static_cast<size_t>(a_row) * k;
-    asp[t] = a_scales + static_cast<size_t>(a_row) * kblocks;
-  }
+  for (int t = 0; t < MT; ++t) asp[t] = a_scales + static_cast<size_t>(min(m0 + t * 16 + r, m - 1)) * kblocks;
 
   v4f acc[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  for (int s = wave * 2; s < steps; s += kGemmWaves * 2) {
-    u32x4 wq[2][2], aq[2][MT][2];
-    int ws[2], as[2][MT];
-    bool valid[2][2];
-    // Every load of the pair is issued before the first use.
+  // Steps interleave over the waves, so that at any time the block reads a few KB of each row in one piece.
+  // DEPTH steps of a wave are in flight together: every load of them is issued before the first use.
+  constexpr int DEPTH = MT == 1 ? 4 : MT == 2 ? 2 : 1;
+  for (int s0 = wave; s0 < steps; s0 += WAVES * DEPTH) {
+    u32x4 wq[DEPTH][2], aq[DEPTH][MT][2];
+    int ws[DEPTH], as[DEPTH][MT];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int kb = (s + j) * 4 + g;
-      const int kc = kb < kblocks ? kb : kblocks - 1;
-      ws[j] = wsp[kc];
+    for (int d = 0; d < DEPTH; ++d) {
+      const int s = s0 + d * WAVES;
+      if (s >= steps) break;   // the same for the whole wave
+      issue_step<true>(w, n0, n, k, s, wq[d]);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) as[j][t] = asp[t][kc];
+      for (int t = 0; t < MT; ++t) issue_step<false>(a, m0 + t * 16, m, k, s, aq[d][t]);
+      const int kb = s * 4 + g;
+      const int kc = kb < kblocks ? kb : kblocks - 1;   // a block past k holds zeros: any scale does
+      ws[d] = wsp[kc];
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int at = (s + j) * 128 + h * 64 + g * 16;
-        valid[j][h] = at < k;
-        const int off = valid[j][h] ? at : 0;
-        wq[j][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(wp + off));
+      for (int t = 0; t < MT; ++t) as[d][t] = asp[t][kc];
+    }
 #pragma unroll
-        for (int t = 0; t < MT; ++t) aq[j][t][h] = *reinterpret_cast<const u32x4*>(ap[t] + off);
+    for (int d = 0; d < DEPTH; ++d) {
+      if (s0 + d * WAVES >= steps) break;
+      commit_step(region, wq[d]);
+      __builtin_amdgcn_wave_barrier();
+      const v8i wv = step_operand(region);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        u32x4* mine = region + ((t + 1) & 1) * kStepUnits;   // the other region than the tile before
+        commit_step(mine, aq[d][t]);
+        __builtin_amdgcn_wave_barrier();
+        acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, step_operand(mine), acc[t], 0, 0, 0, ws[d], 0, as[d][t]);
       }
     }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-        if (!valid[j][h]) {
-          wq[j][h] = u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-          for (int t = 0; t < MT; ++t) aq[j][t][h] = u32x4{0u, 0u, 0u, 0u};
-        }
-      const v8i wv = as_operand(wq[j][0], wq[j][1]);
-#pragma unroll
-      for (int t = 0; t < MT; ++t)
-        acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, as_operand(aq[j][t][0], aq[j][t][1]), acc[t],
-                                                                  0, 0, 0, ws[j], 0, as[j][t]);
-    }
   }
 
-  if (wave != 0) {
+  __syncthreads();   // every wave is done with its regions
+  float4* fold = reinterpret_cast<float4*>(lds);
 #pragma unroll
-    for (int t = 0; t < MT; ++t) fold[wave - 1][t][lane] = float4{acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
-  }
+  for (int t = 0; t < MT; ++t) fold[(wave * MT + t) * 64 + lane] = float4{acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
   __syncthreads();
-  if (wave != 0) return;
+  if (wave >= MT) return;
+  const int t = wave;
+  float4 sum = fold[t * 64 + lane];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    float sum[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
-#pragma unroll
-    for (int p = 0; p < kGemmWaves - 1; ++p) {
-      const float4 part = fold[p][t][lane];
-      sum[0] += part.x;
-      sum[1] += part.y;
-      sum[2] += part.z;
-      sum[3] += part.w;
-    }
-    const int a_row = m0 + t * 16 + r;
-    if (a_row >= m) continue;
-    Out* dst = out + static_cast<size_t>(a_row) * out_stride + n0 + g * 4;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (n0 + g * 4 + i < n) put<Out>(dst + i, sum[i]);
+  for (int p = 1; p < WAVES; ++p) {
+    const float4 part = fold[(p * MT + t) * 64 + lane];
+    sum.x += part.x;
+    sum.y += part.y;
+    sum.z += part.z;
+    sum.w += part.w;
   }
+  const int a_row = m0 + t * 16 + r;
+  if (a_row >= m) return;
+  Out* dst = out + static_cast<size_t>(a_row) * out_stride + n0 + g * 4;
+  const float v[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (n0 + g * 4 + i < n) put<Out>(dst + i, v[i]);
 }
 
-template <typename Out, int MT>
+template <typename Out, int MT, int WAVES>
 hipError_t launch_gemm_mt(const uint8_t* a, const uint8_t* as, const uint8_t* w, const uint8_t* ws, Out* out, int m, int n,
                           int k, size_t stride, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>((n + 15) / 16), static_cast<unsigned>((m + 16 * MT - 1) / (16 * MT)));
-  hipLaunchKernelGGL((mxfp8_gemm_kernel<Out, MT>), grid, dim3(kGemmThreads), 0, stream, a, as, w, ws, out, m, n, k, stride);
+  hipLaunchKernelGGL((mxfp8_gemm_kernel<Out, MT, WAVES>), grid, dim3(WAVES * 64), 0, stream, a, as, w, ws, out, m, n, k, stride);
   return hipGetLastError();
+}
+
+template <typename Out, int WAVES>
+hipError_t launch_gemm_waves(const uint8_t* a, const uint8_t* as, const uint8_t* w, const uint8_t* ws, Out* out, int m, int n,
+                             int k, size_t stride, hipStream_t s) {
+  if (m <= 16) return launch_gemm_mt<Out, 1, WAVES>(a, as, w, ws, out, m, n, k, stride, s);
+  if (m <= 32) return launch_gemm_mt<Out, 2, WAVES>(a, as, w, ws, out, m, n, k, stride, s);
+  if (m <= 48) return launch_gemm_mt<Out, 3, WAVES>(a, as, w, ws, out, m, n, k, stride, s);
+  return launch_gemm_mt<Out, 4, WAVES>(a, as, w, ws, out, m, n, k, stride, s);
 }
 
 // src/kernels/mxfp8_gemm.cu:217-243.
@@ -243,16 +278,11 @@ int gemm(const uint8_t* a, const uint8_t* as, const uint8_t* w, const uint8_t* w
   if (((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) & 15u) != 0)
     return report_invalid(std::string(who) + ": payloads must be 16-byte aligned");
   // The tile override is a diagnostic of the reference's kernel; every value gives the same chain here.
+  // Waves per block from k alone (an output element's chain must not depend on m or n): sixteen once every
+  // wave has a step of its own.
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipError_t err;
-  if (m <= 16)
-    err = launch_gemm_mt<Out, 1>(a, as, w, ws, out, m, n, k, stride, s);
-  else if (m <= 32)
-    err = launch_gemm_mt<Out, 2>(a, as, w, ws, out, m, n, k, stride, s);
-  else if (m <= 48)
-    err = launch_gemm_mt<Out, 3>(a, as, w, ws, out, m, n, k, stride, s);
-  else
-    err = launch_gemm_mt<Out, 4>(a, as, w, ws, out, m, n, k, stride, s);
+  const hipError_t err = k >= 16 * 128 ? launch_gemm_waves<Out, 16>(a, as, w, ws, out, m, n, k, stride, s)
+                                       : launch_gemm_waves<Out, 4>(a, as, w, ws, out, m, n, k, stride, s);
   return report_hip(err, who);
 }
 
