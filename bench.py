@@ -53,7 +53,7 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5 ('' for none; default: all four, none under --tune)")
+                    "separated out of c1,c2,c4,c5,w8a8 ('' for none; default: c1,c2,c4,c5, none under --tune)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -445,12 +445,42 @@ def main():
         lay.close()
         return res
 
+    def bench_w8a8():
+        """The activation-quantized MXFP8 GEMM at the C5 shared expert's projection shapes, swept over the row count
+        (not a BASELINE configuration: run with --configs w8a8). Weights rotate so that no launch finds them cached."""
+        res = {"workload": "MXFP8 x MXFP8 block-scaled GEMM (scaled matrix-core instruction), rotating weights"}
+        for n, k in ((4096, 6144), (6144, 4096)):
+            pw, sw = hg.encode_mxfp8(hg.normal_f32(0xD6996000 + n, (n, k), 0.02))
+            ring = ring_copies([torch.from_numpy(pw).to(dev), torch.from_numpy(sw).to(dev)], pw.nbytes)
+            for m in (1, 16, 64, 256):
+                x = torch.from_numpy(hg.normal_bf16(0xD6996100 + m, (m, k)).view(np.int16)).to(dev)
+                xq = torch.empty((m, k), dtype=torch.uint8, device=dev)
+                xs = torch.empty((m, k // 32), dtype=torch.uint8, device=dev)
+                out = torch.empty((m, n), dtype=torch.int16, device=dev)
+                L.launch_mxfp8_quantize_rows(x, k, m, k, xq, xs, stream)
+
+                def step(i):
+                    r = i % len(ring)
+                    L.launch_mxfp8_gemm_bf16(xq, xs, ring[r][0], ring[r][1], out, m, n, k, stream)
+
+                def quant(i):
+                    L.launch_mxfp8_quantize_rows(x, k, m, k, xq, xs, stream)
+
+                sec = time_graph(step, args.steps, args.warmup)
+                nbytes = (n + m) * k * 33 // 32 + m * n * 2
+                res[f"gemm_m{m}_n{n}_k{k}"] = {"us": sec * 1e6, "algorithmic_bytes": nbytes, "gbps": nbytes / sec / 1e9,
+                                              "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                              "tflops": 2.0 * m * n * k / sec / 1e12}
+                qsec = time_graph(quant, args.steps, args.warmup)
+                res[f"quantize_rows{m}_k{k}"] = {"us": qsec * 1e6}
+        return res
+
     other_configs = {}
     configs = args.configs if args.configs is not None else ("" if args.tune else "c1,c2,c4,c5")
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
-            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5}[name]()
+            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
 
