@@ -190,3 +190,79 @@ def test_quantize_then_gemm_on_normal_data(gpu):
     assert np.abs(err).max() <= 2e-4 * np.abs(want).max()
     full = bf16_bits_to_f64(x) @ bf16_bits_to_f64(wt).T
     assert np.sqrt(((host(out) - full) ** 2).sum() / (full ** 2).sum()) < 0.06
+
+
+def mlp_chain(x_d, w_d, rows, hidden, inter, alpha, limit, stream, bufs):
+    """The MiniMax MLP's native call order (src/models/minimax/layers.cpp:222-238) on `stream`."""
+    xq, xs, gate, up, aq, a_s, out = bufs
+    (wg, wgs), (wu, wus), (wd, wds) = w_d
+    L.launch_mxfp8_quantize_rows(x_d, hidden, rows, hidden, xq, xs, stream)
+    L.launch_mxfp8_gemm_bf16(xq, xs, wg, wgs, gate, rows, inter, hidden, stream)
+    L.launch_mxfp8_gemm_bf16(xq, xs, wu, wus, up, rows, inter, hidden, stream)
+    L.launch_minimax_swiglu_mxfp8_rows(gate, up, inter, rows, inter, alpha, limit, aq, a_s, stream)
+    L.launch_mxfp8_gemm_bf16(aq, a_s, wd, wds, out, rows, hidden, inter, stream)
+
+
+def test_mlp_chain_against_the_oracle_chain_and_under_graph_replay(gpu):
+    import torch
+    from dgpp_amd import hostgen as hg
+
+    rows, hidden, inter, alpha, limit = 20, 1024, 512, 1.702, 7.0
+    x = hg.normal_bf16(0x3F80, (rows, hidden), 1.0)
+    w = [hg.encode_mxfp8(hg.normal_f32(0x3F81 + i, shape, 0.05)) for i, shape in
+         enumerate(((inter, hidden), (inter, hidden), (hidden, inter)))]
+    x_d = dev(x)
+    w_d = [(dev(p), dev(s)) for p, s in w]
+    bufs = (dev_empty((rows, hidden), np.uint8), dev_empty((rows, hidden // 32), np.uint8),
+            dev_empty((rows, inter), np.uint16), dev_empty((rows, inter), np.uint16),
+            dev_empty((rows, inter), np.uint8), dev_empty((rows, inter // 32), np.uint8),
+            dev_empty((rows, hidden), np.uint16))
+    mlp_chain(x_d, w_d, rows, hidden, inter, alpha, limit, None, bufs)
+    sync()
+    eager = [host(b).copy() for b in bufs]
+
+    # The oracle's chain: every stage from the oracle's own previous stage, float64 products rounded to BF16.
+    o = orc.oracle()
+
+    def gemm64(a, a_s, wp, wsc, m, n, k):
+        res = np.empty((m, n))
+        o.orc_mxfp8_gemm(orc.p(a), orc.p(a_s), orc.p(wp), orc.p(wsc), m, n, k, orc.p(res), None)
+        return res
+
+    xq, xs = oracle_quantize(x, rows, hidden)
+    assert np.array_equal(eager[0], xq) and np.array_equal(eager[1], xs)
+    gate64 = gemm64(xq, xs, w[0][0], w[0][1], rows, inter, hidden)
+    up64 = gemm64(xq, xs, w[1][0], w[1][1], rows, inter, hidden)
+    gate, up = md.f32_to_bf16_bits(gate64.astype(np.float32)), md.f32_to_bf16_bits(up64.astype(np.float32))
+    # one stage, the reference's comparator for a GEMV stage: within 2 BF16 ulps or under 1e-3 of the largest output
+    for got, want64, want in ((eager[2].view(np.uint16), gate64, gate), (eager[3].view(np.uint16), up64, up)):
+        got = np.ascontiguousarray(got)
+        rep = orc.compare_bf16(got, bf16_bits_to_f64(want), 2.0, 1e-3)
+        assert rep.mismatches == 0 and rep.nan_pattern_errors == 0 and rep.l2_rel <= 1e-3
+        assert (got != want).mean() < 0.03
+    act = np.empty((rows, inter), dtype=np.uint16)
+    o.orc_swiglu_oai(orc.p(gate), orc.p(up), inter, rows, inter, alpha, limit, None, orc.p(act))
+    aq, a_s = oracle_quantize(act, rows, inter)
+    want = gemm64(aq, a_s, w[2][0], w[2][1], rows, hidden, inter)
+    got = bf16_bits_to_f64(eager[6].view(np.uint16))
+    # Whole chain: a flipped BF16 step upstream moves an MXFP8 code of the activation now and then; the outputs stay
+    # within a few percent of MXFP8's own step of the oracle chain, and are mostly its very bits.
+    assert np.sqrt(((got - want) ** 2).sum() / (want ** 2).sum()) < 5e-3
+    assert np.abs(got - want).max() <= 0.02 * np.abs(want).max()
+
+    # Captured once, replayed twice over scribbled outputs: the same bits as the eager run every time.
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        mlp_chain(x_d, w_d, rows, hidden, inter, alpha, limit, stream, bufs)     # warm-up on the capture stream
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            mlp_chain(x_d, w_d, rows, hidden, inter, alpha, limit, stream, bufs)
+        for replay in range(2):
+            for b in bufs:
+                b.fill_(0x55 if b.dtype == torch.uint8 else 0x3F01)
+            stream.synchronize()
+            g.replay()
+            stream.synchronize()
+            for b, want_b in zip(bufs, eager):
+                assert np.array_equal(host(b), want_b), f"replay {replay}"
