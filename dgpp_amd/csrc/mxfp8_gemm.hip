@@ -208,6 +208,8 @@ __global__ __launch_bounds__(WAVES * 64) void mxfp8_gemm_kernel(
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (s0 + d * WAVES >= steps) break;
+      // The LDS serves a wavefront's accesses in order: a region is rewritten as soon as the read of its
+      // previous content has been issued. The barriers only keep the compiler from moving accesses across.
       commit_step(region, wq[d]);
       __builtin_amdgcn_wave_barrier();
       const v8i wv = step_operand(region);
