@@ -53,7 +53,7 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5,w8a8 ('' for none; default: c1,c2,c4,c5, none under --tune)")
+                    "separated out of c1,c2,c4,c5,w8a8,qwen_tail ('' for none; default: c1,c2,c4,c5, none under --tune)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -475,12 +475,55 @@ def main():
                 res[f"quantize_rows{m}_k{k}"] = {"us": qsec * 1e6}
         return res
 
+    def bench_qwen_tail():
+        """The gated shared expert's decode tail (block-FP8 weights, hidden 2048, shared inter 512) in its two launches
+        against the seven-launch chain it is bitwise equal to (not a BASELINE configuration: --configs qwen_tail)."""
+        H, S, K = 2048, 512, 10
+        res = {"workload": f"gated shared expert decode tail, FP8 block-128, hidden {H}, inter {S}: two launches vs the unfused chain"}
+        mats = [hg.encode_fp8_blocks(hg.f32_to_bf16(hg.normal_f32(0xD6997000 + i, shape, 0.03)), 128, 128)
+                for i, shape in enumerate(((S, H), (S, H), (H, S)))]
+        ring = ring_copies([torch.from_numpy(a).to(dev) for pair in mats for a in pair], sum(p.nbytes for p, _ in mats))
+        gvec = torch.from_numpy(hg.normal_bf16(0xD6997010, (H,), 0.03).view(np.int16)).to(dev)
+        for T in (1, 8):
+            x = torch.from_numpy(hg.normal_bf16(0xD6997020 + T, (T, H)).view(np.int16)).to(dev)
+            contrib = torch.from_numpy(hg.normal_f32(0xD6997030 + T, (T * (K + 1), H), 0.3)).to(dev)
+            wts = torch.from_numpy(np.abs(hg.normal_f32(0xD6997040 + T, (T, K), 0.2)).astype(np.float32)).to(dev)
+            act, g_o, u_o = (torch.empty((T, S), dtype=torch.int16, device=dev) for _ in range(3))
+            sw = torch.empty((T,), dtype=torch.float32, device=dev)
+            down = torch.empty((T, H), dtype=torch.float32, device=dev)
+            routed = torch.empty((T, H), dtype=torch.float32, device=dev)
+            out = torch.empty((T, H), dtype=torch.int16, device=dev)
+            rows_id = torch.arange(T, dtype=torch.int32, device=dev)
+
+            def fused(i):
+                gp, gs, up, us, dp, ds = ring[i % len(ring)]
+                L.qwen_moe_shared_tail_decode_routed_fp8(x, H, gp, gs, up, us, dp, ds, gvec, act, sw, contrib, wts, K, out, T, H, S,
+                                                         stream)
+
+            def chain(i):
+                gp, gs, up, us, dp, ds = ring[i % len(ring)]
+                L.launch_scale_gemm_grid_bf16(x, H, gp, gs, g_o, T, S, H, stream, 0, 7, 7)
+                L.launch_scale_gemm_grid_bf16(x, H, up, us, u_o, T, S, H, stream, 0, 7, 7)
+                L.launch_moe_swiglu_clamp(g_o, u_o, act, T * S, float("inf"), stream)
+                L.launch_scale_gemm_grid_f32(act, S, dp, ds, down, T, H, S, stream, 0, 7, 7)
+                L.qwen_moe_shared_gate_bf16(x, gvec, sw, T, H, stream)
+                L.launch_moe_slot_accum_routed_f32(routed, contrib, wts, T, H, K, stream)
+                L.launch_moe_accum(routed, down, rows_id, sw, T, H, stream)
+                L.launch_moe_round_bf16(out, routed, T * H, stream)
+
+            nbytes = 3 * S * H + 3 * (S // 128) * (H // 128) * 4 + T * H * 2 + T * (K + 1) * H * 4 + T * H * 2
+            for name, fn in (("two_launches", fused), ("unfused_chain", chain)):
+                sec = time_graph(fn, args.steps, args.warmup)
+                res[f"T{T}_{name}"] = {"us": sec * 1e6, "algorithmic_bytes": nbytes, "gbps": nbytes / sec / 1e9,
+                                       "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+        return res
+
     other_configs = {}
     configs = args.configs if args.configs is not None else ("" if args.tune else "c1,c2,c4,c5")
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
-            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8}[name]()
+            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
 

@@ -109,6 +109,13 @@ SIGNATURES = {
     "dgpp_launch_moe_grouped_mma_bf16": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _P]),
     "dgpp_launch_moe_grouped_mma_f32": (_I, [_P, _Z, _P, _I, _I, _I, _P, _I, _P, _Z, _I, _I, _P, _P]),
     "dgpp_launch_mma_gemv_fp8_swiglu_f32": (_I, [_P, _P, _F, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P]),
+    "dgpp_qwen_moe_shared_gate_bf16": (_I, [_P, _P, _P, _I, _I, _P]),
+    "dgpp_qwen_moe_shared_gate_up_decode_fp8": (_I, [_P, _Z, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
+    "dgpp_qwen_moe_shared_down_decode_fp8": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
+    "dgpp_qwen_moe_shared_down_decode_routed_fp8": (_I, [_P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _P, _I, _I]),
+    "dgpp_qwen_moe_shared_tail_decode_fp8": (_I, [_P, _Z, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
+    "dgpp_qwen_moe_shared_tail_decode_routed_fp8": (_I, [_P, _Z, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I,
+                                                         _I, _P, _I, _I]),
     "dgpp_launch_mxfp8_quantize_rows": (_I, [_P, _Z, _I, _I, _P, _P, _P]),
     "dgpp_launch_minimax_swiglu_mxfp8_rows": (_I, [_P, _P, _Z, _I, _I, _F, _F, _P, _P, _P]),
     "dgpp_launch_mxfp8_gemm_bf16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _I]),

@@ -25,6 +25,7 @@ HIP_SOURCES = [
     "gemv_fp8e8m0.hip",
     "moe_misc.hip",
     "mxfp8_gemm.hip",
+    "qwen_tail.hip",
     "capi.hip",
 ]
 HOST_SOURCES = ["host_codec.cpp", "loader.cpp"]

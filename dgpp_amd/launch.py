@@ -397,6 +397,43 @@ def launch_mma_gemv_fp8_swiglu_f32(gate, up, limit, act_stride, w, scales, out, 
                                                            m, n, k, out_stride, rs, cs, _stream(stream)))
 
 
+def qwen_moe_shared_gate_bf16(x, g, w, tokens, hidden, stream=None):
+    _check(_lib.load().dgpp_qwen_moe_shared_gate_bf16(_p(x), _p(g), _p(w), tokens, hidden, _stream(stream)))
+
+
+def qwen_moe_shared_gate_up_decode_fp8(x, x_stride, gate_p, gate_s, up_p, up_s, g, act, sw, tokens, H, S, stream=None, rs=7,
+                                       cs=7):
+    _check(_lib.load().dgpp_qwen_moe_shared_gate_up_decode_fp8(_p(x), x_stride, _p(gate_p), _p(gate_s), _p(up_p), _p(up_s),
+                                                               _p(g), _p(act), _p(sw), tokens, H, S, _stream(stream), rs, cs))
+
+
+def qwen_moe_shared_down_decode_fp8(act, down_p, down_s, sw, acc, out, tokens, H, S, stream=None, rs=7, cs=7):
+    _check(_lib.load().dgpp_qwen_moe_shared_down_decode_fp8(_p(act), _p(down_p), _p(down_s), _p(sw), _p(acc), _p(out), tokens,
+                                                            H, S, _stream(stream), rs, cs))
+
+
+def qwen_moe_shared_down_decode_routed_fp8(act, down_p, down_s, sw, contrib, weights, top_k, out, tokens, H, S, stream=None,
+                                           rs=7, cs=7):
+    _check(_lib.load().dgpp_qwen_moe_shared_down_decode_routed_fp8(_p(act), _p(down_p), _p(down_s), _p(sw), _p(contrib),
+                                                                   _p(weights), top_k, _p(out), tokens, H, S,
+                                                                   _stream(stream), rs, cs))
+
+
+def qwen_moe_shared_tail_decode_fp8(x, x_stride, gate_p, gate_s, up_p, up_s, down_p, down_s, g, act, sw, acc, out, tokens, H, S,
+                                    stream=None, rs=7, cs=7):
+    _check(_lib.load().dgpp_qwen_moe_shared_tail_decode_fp8(_p(x), x_stride, _p(gate_p), _p(gate_s), _p(up_p), _p(up_s),
+                                                            _p(down_p), _p(down_s), _p(g), _p(act), _p(sw), _p(acc), _p(out),
+                                                            tokens, H, S, _stream(stream), rs, cs))
+
+
+def qwen_moe_shared_tail_decode_routed_fp8(x, x_stride, gate_p, gate_s, up_p, up_s, down_p, down_s, g, act, sw, contrib, weights,
+                                           top_k, out, tokens, H, S, stream=None, rs=7, cs=7):
+    _check(_lib.load().dgpp_qwen_moe_shared_tail_decode_routed_fp8(_p(x), x_stride, _p(gate_p), _p(gate_s), _p(up_p), _p(up_s),
+                                                                   _p(down_p), _p(down_s), _p(g), _p(act), _p(sw), _p(contrib),
+                                                                   _p(weights), top_k, _p(out), tokens, H, S,
+                                                                   _stream(stream), rs, cs))
+
+
 def launch_mxfp8_quantize_rows(x, x_stride, rows, k, codes, scales, stream=None):
     _check(_lib.load().dgpp_launch_mxfp8_quantize_rows(_p(x), x_stride, rows, k, _p(codes), _p(scales), _stream(stream)))
 

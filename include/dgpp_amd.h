@@ -466,6 +466,43 @@ int dgpp_launch_mxfp8_gemm_bf16(const uint8_t* a, const uint8_t* a_scales, const
 int dgpp_launch_mxfp8_gemm_f32(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales, float* out,
                                int m, int n, int k, void* stream, size_t out_stride, int output_tile);
 
+/* ---- the gated shared expert's decode tail, block-FP8 weights -------------------------------------------------
+ * src/kernels/qwen_moe.hpp:12-19, src/kernels/qwen_moe.cu:312-326: w[t] = bf16(sigmoid(bf16(x[t] . g))) as an F32
+ * value; x BF16 [tokens, hidden] (dense rows), g BF16 [hidden] or NULL (then w[t] = 1). The dot runs in the
+ * reference's order: 32 strided partial sums over 16-byte vectors and the xor tree 16, 8, 4, 2, 1.
+ * DGPP_INVALID_ARGUMENT unless hidden is a positive multiple of 8 and x, g are 16-byte aligned. */
+int dgpp_qwen_moe_shared_gate_bf16(const uint16_t* x, const uint16_t* g, float* w, int tokens, int hidden, void* stream);
+/* src/kernels/qwen_moe.hpp:34-87, the FP8 forms (src/kernels/qwen_moe.cu:377-413, :443-482). The tail in two launches:
+ *   gate_up:  act[t, s] = swiglu(bf16(x[t] . gate[s]), bf16(x[t] . up[s])) without clamps, BF16 [tokens, S];
+ *             sw[t] as dgpp_qwen_moe_shared_gate_bf16 (x rows at x_stride);
+ *   down:     out[t, h] = bf16(fma(sw[t], act[t] . down[h], a)), a = acc[t, h] (F32 [tokens, H]), or, in the
+ *             routed form, the fma chain over j < top_k of weights[t, j] * contrib[(t * (top_k + 1) + j), h]
+ *             from zero (the routed accumulate kernel's order), top_k <= 16.
+ * gate / up: E4M3 [S, H], down: E4M3 [H, S], F32 scales on the (rs, cs) grid (log2 block rows / columns, cs >= 4).
+ * tokens <= 8 (one pass over the weights for all of them), H and S multiples of 16, operands 16-byte aligned.
+ * Each launch is bitwise the unfused launchers it stands for (dgpp_launch_scale_gemm_grid_bf16 twice,
+ * dgpp_launch_moe_swiglu_clamp with an infinite limit, dgpp_launch_scale_gemm_grid_f32, the gate, the accumulate,
+ * dgpp_launch_moe_round_bf16). The halves are entries of their own so that gate_up can run beside the routed
+ * experts on another stream; the BF16-weight forms of the reference's tail are not provided. */
+int dgpp_qwen_moe_shared_gate_up_decode_fp8(const uint16_t* x, size_t x_stride, const uint8_t* gate_p, const float* gate_s,
+                                            const uint8_t* up_p, const float* up_s, const uint16_t* g, uint16_t* act, float* sw,
+                                            int tokens, int H, int S, void* stream, int rs, int cs);
+int dgpp_qwen_moe_shared_down_decode_fp8(const uint16_t* act, const uint8_t* down_p, const float* down_s, const float* sw,
+                                         const float* acc, uint16_t* out, int tokens, int H, int S, void* stream, int rs,
+                                         int cs);
+int dgpp_qwen_moe_shared_down_decode_routed_fp8(const uint16_t* act, const uint8_t* down_p, const float* down_s, const float* sw,
+                                                const float* contrib, const float* weights, int top_k, uint16_t* out,
+                                                int tokens, int H, int S, void* stream, int rs, int cs);
+int dgpp_qwen_moe_shared_tail_decode_fp8(const uint16_t* x, size_t x_stride, const uint8_t* gate_p, const float* gate_s,
+                                         const uint8_t* up_p, const float* up_s, const uint8_t* down_p, const float* down_s,
+                                         const uint16_t* g, uint16_t* act, float* sw, const float* acc, uint16_t* out,
+                                         int tokens, int H, int S, void* stream, int rs, int cs);
+int dgpp_qwen_moe_shared_tail_decode_routed_fp8(const uint16_t* x, size_t x_stride, const uint8_t* gate_p, const float* gate_s,
+                                                const uint8_t* up_p, const float* up_s, const uint8_t* down_p,
+                                                const float* down_s, const uint16_t* g, uint16_t* act, float* sw,
+                                                const float* contrib, const float* weights, int top_k, uint16_t* out,
+                                                int tokens, int H, int S, void* stream, int rs, int cs);
+
 /* ---- host-side weight encoders and synthetic data (no GPU involved) ------------------------------------------ */
 /* Scalar codecs, src/common/dtypes.hpp:83-190, src/kernels/latent_format.hpp:117-162. */
 float dgpp_bf16_to_f32(uint16_t bits);

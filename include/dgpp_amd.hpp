@@ -366,6 +366,43 @@ inline void launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t*
   detail::check(dgpp_launch_mma_gemv_fp8_swiglu_f32(gate, up, limit, act_stride, w, scales, out, m, n, k, out_stride, rs, cs,
                                                     stream));
 }
+// src/kernels/qwen_moe.hpp:18-87 (the shared gate and the FP8 forms of the shared expert's decode tail).
+inline void qwen_moe_shared_gate_bf16(const uint16_t* x, const uint16_t* g, float* w, int tokens, int hidden, hipStream_t stream) {
+  detail::check(dgpp_qwen_moe_shared_gate_bf16(x, g, w, tokens, hidden, stream));
+}
+inline void qwen_moe_shared_gate_up_decode_fp8(const uint16_t* x, size_t x_stride, const uint8_t* gate_p, const float* gate_s,
+                                               const uint8_t* up_p, const float* up_s, const uint16_t* g, uint16_t* act,
+                                               float* sw, int tokens, int H, int S, hipStream_t stream, int rs = 7, int cs = 7) {
+  detail::check(dgpp_qwen_moe_shared_gate_up_decode_fp8(x, x_stride, gate_p, gate_s, up_p, up_s, g, act, sw, tokens, H, S, stream,
+                                                        rs, cs));
+}
+inline void qwen_moe_shared_down_decode_fp8(const uint16_t* act, const uint8_t* down_p, const float* down_s, const float* sw,
+                                            const float* acc, uint16_t* out, int tokens, int H, int S, hipStream_t stream,
+                                            int rs = 7, int cs = 7) {
+  detail::check(dgpp_qwen_moe_shared_down_decode_fp8(act, down_p, down_s, sw, acc, out, tokens, H, S, stream, rs, cs));
+}
+inline void qwen_moe_shared_down_decode_routed_fp8(const uint16_t* act, const uint8_t* down_p, const float* down_s,
+                                                   const float* sw, const float* contrib, const float* weights, int top_k,
+                                                   uint16_t* out, int tokens, int H, int S, hipStream_t stream, int rs = 7,
+                                                   int cs = 7) {
+  detail::check(dgpp_qwen_moe_shared_down_decode_routed_fp8(act, down_p, down_s, sw, contrib, weights, top_k, out, tokens, H, S,
+                                                            stream, rs, cs));
+}
+inline void qwen_moe_shared_tail_decode_fp8(const uint16_t* x, size_t x_stride, const uint8_t* gate_p, const float* gate_s,
+                                            const uint8_t* up_p, const float* up_s, const uint8_t* down_p, const float* down_s,
+                                            const uint16_t* g, uint16_t* act, float* sw, const float* acc, uint16_t* out,
+                                            int tokens, int H, int S, hipStream_t stream, int rs = 7, int cs = 7) {
+  detail::check(dgpp_qwen_moe_shared_tail_decode_fp8(x, x_stride, gate_p, gate_s, up_p, up_s, down_p, down_s, g, act, sw, acc, out,
+                                                     tokens, H, S, stream, rs, cs));
+}
+inline void qwen_moe_shared_tail_decode_routed_fp8(const uint16_t* x, size_t x_stride, const uint8_t* gate_p, const float* gate_s,
+                                                   const uint8_t* up_p, const float* up_s, const uint8_t* down_p,
+                                                   const float* down_s, const uint16_t* g, uint16_t* act, float* sw,
+                                                   const float* contrib, const float* weights, int top_k, uint16_t* out,
+                                                   int tokens, int H, int S, hipStream_t stream, int rs = 7, int cs = 7) {
+  detail::check(dgpp_qwen_moe_shared_tail_decode_routed_fp8(x, x_stride, gate_p, gate_s, up_p, up_s, down_p, down_s, g, act, sw,
+                                                            contrib, weights, top_k, out, tokens, H, S, stream, rs, cs));
+}
 // src/kernels/mxfp8_gemm.hpp:11-31.
 inline void launch_mxfp8_quantize_rows(const uint16_t* x, size_t x_stride, int rows, int k, uint8_t* codes, uint8_t* scales,
                                        hipStream_t stream) {

@@ -494,6 +494,19 @@ void orc_moe_forward(const uint16_t* x, int64_t x_stride, const int32_t* ids, co
   }
 }
 
+void orc_shared_gate(const uint16_t* x, int64_t x_stride, const uint16_t* g, int tokens, int hidden, float* w) {
+  for (int t = 0; t < tokens; ++t) {
+    if (!g) {
+      w[t] = 1.0f;
+      continue;
+    }
+    double logit = 0.0;
+    for (int k = 0; k < hidden; ++k) logit += bf16d(x[static_cast<size_t>(t) * x_stride + k]) * bf16d(g[k]);
+    logit = bf16d(d2bf16(logit));
+    w[t] = static_cast<float>(bf16d(d2bf16(1.0 / (1.0 + std::exp(-logit)))));
+  }
+}
+
 // ---- activation-quantized MXFP8 form ---------------------------------------------------------
 
 void orc_mxfp8_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, uint8_t* codes, uint8_t* scales) {

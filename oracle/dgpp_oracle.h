@@ -139,6 +139,11 @@ void orc_moe_forward(const uint16_t* x, int64_t x_stride, const int32_t* ids, co
                      const OrcMatrix* experts, const OrcMatrix* shared, float swiglu_limit,
                      int threads, double* out_raw, uint16_t* out_bf16);
 
+/* The gated shared expert's weight: w[t] = bf16(sigmoid(bf16(x[t] . g))) with the dot and the sigmoid in double
+ * (g null: 1). src/models/qwen/moe_reference.cpp:153-157. Pinned by numpy float64 and closed-form points
+ * (x = 0 -> 0.5; a large logit -> 1). */
+void orc_shared_gate(const uint16_t* x, int64_t x_stride, const uint16_t* g, int tokens, int hidden, float* w);
+
 /* ---- activation-quantized MXFP8 form (its own numerics contract: the activations carry MXFP8 rounding) ---- */
 /* BF16 x [rows, k] (row stride in elements) -> E4M3 codes [rows, k], e8m0 scales [rows, k / 32]: per
  * 32-group the exponent is max(-127, ceil(log2(amax / 448))) (a zero group: -127, byte 0), codes are

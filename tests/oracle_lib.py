@@ -45,6 +45,7 @@ _SIG = {
     "orc_slot_accum": (None, [_P, _P, _I, _I, _I, _I, _P, _P]),
     "orc_accum_ordered": (None, [_P, _L, _P, _P, _P, _I, _I, _I, _I, _P, _P]),
     "orc_moe_forward": (None, [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P, _P, _F, _I, _P, _P]),
+    "orc_shared_gate": (None, [_P, _L, _P, _I, _I, _P]),
     "orc_mxfp8_quantize_rows": (None, [_P, _L, _I, _I, _P, _P]),
     "orc_swiglu_oai": (None, [_P, _P, _L, _I, _I, _F, _F, _P, _P]),
     "orc_mxfp8_gemm": (None, [_P, _P, _P, _P, _I, _I, _I, _P, _P]),
