@@ -447,7 +447,7 @@ def main():
 
     def bench_w8a8():
         """The activation-quantized MXFP8 GEMM at the C5 shared expert's projection shapes, swept over the row count
-        (not a BASELINE configuration: run with --configs w8a8). Weights rotate so that no launch finds them cached."""
+        (not one of the headline benchmark's configurations: run with --configs w8a8). Weights rotate so that no launch finds them cached."""
         res = {"workload": "MXFP8 x MXFP8 block-scaled GEMM (scaled matrix-core instruction), rotating weights"}
         for n, k in ((4096, 6144), (6144, 4096)):
             pw, sw = hg.encode_mxfp8(hg.normal_f32(0xD6996000 + n, (n, k), 0.02))
@@ -477,7 +477,7 @@ def main():
 
     def bench_qwen_tail():
         """The gated shared expert's decode tail (block-FP8 weights, hidden 2048, shared inter 512) in its two launches
-        against the seven-launch chain it is bitwise equal to (not a BASELINE configuration: --configs qwen_tail)."""
+        against the seven-launch chain it is bitwise equal to (not one of the headline benchmark's configurations: --configs qwen_tail)."""
         H, S, K = 2048, 512, 10
         res = {"workload": f"gated shared expert decode tail, FP8 block-128, hidden {H}, inter {S}: two launches vs the unfused chain"}
         mats = [hg.encode_fp8_blocks(hg.f32_to_bf16(hg.normal_f32(0xD6997000 + i, shape, 0.03)), 128, 128)
