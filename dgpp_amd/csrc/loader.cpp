@@ -667,3 +667,103 @@ int dgpp_expert_view_from_fp4(const DgppFp4Matrix* m, DgppMoeExpertView* out) {
 }
 
 }  // extern "C"
+
+// ---- tensor names of a GLM-family MoE layer ------------------------------------------------------------------
+
+namespace {
+
+// The first of the shards that holds `name`, its description in `out`.
+int find_in(const DgppSafetensors* const* files, int n_files, const std::string& name, DgppTensorInfo* out, int* file_index) {
+  for (int i = 0; i < n_files; ++i) {
+    if (!files[i]) continue;
+    const std::string_view key(name);
+    const auto& ts = files[i]->tensors;
+    auto it = std::lower_bound(ts.begin(), ts.end(), key,
+                               [](const Tensor& t, std::string_view k) { return std::string_view(t.name) < k; });
+    if (it != ts.end() && it->name == key) {
+      *out = it->info;
+      if (file_index) *file_index = i;
+      return DGPP_OK;
+    }
+  }
+  return fail(DGPP_INVALID_ARGUMENT, "missing tensor '" + name + "'");
+}
+
+std::string shape_text(const DgppTensorInfo& t) {
+  std::string s = "[";
+  for (int i = 0; i < t.rank; ++i) s += (i ? ", " : "") + std::to_string(t.shape[i]);
+  return s + "]";
+}
+
+int expect(const DgppTensorInfo& t, const std::string& name, int dtype, std::initializer_list<int64_t> shape) {
+  bool ok = t.dtype == dtype && t.rank == static_cast<int>(shape.size());
+  int i = 0;
+  for (int64_t d : shape) ok = ok && t.shape[i++] == d;
+  if (ok) return DGPP_OK;
+  std::string want = "[";
+  i = 0;
+  for (int64_t d : shape) want += (i++ ? ", " : "") + std::to_string(d);
+  return fail(DGPP_INVALID_ARGUMENT, "tensor '" + name + "' is dtype " + std::to_string(t.dtype) + " " + shape_text(t) +
+                                         ", expected dtype " + std::to_string(dtype) + " " + want + "]");
+}
+
+// One logical [rows, cols] matrix named `base` ("...proj.weight"): the FP8 pair or the NVFP4 triple.
+int bind_matrix(const DgppSafetensors* const* files, int n_files, const std::string& base, int64_t rows, int64_t cols, int format,
+                DgppMoeMatrixTensors* out) {
+  std::memset(out, 0, sizeof(*out));
+  out->format = format;
+  int rc;
+  if (format == DGPP_BIND_NVFP4) {
+    if (cols % 16 != 0) return fail(DGPP_INVALID_ARGUMENT, "NVFP4 needs K % 16 == 0: '" + base + "'");
+    if ((rc = find_in(files, n_files, base + "_packed", &out->payload, &out->file_index)) != DGPP_OK) return rc;
+    if ((rc = expect(out->payload, base + "_packed", DGPP_DT_U8, {rows, cols / 2})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, base + "_scale", &out->scales, nullptr)) != DGPP_OK) return rc;
+    if ((rc = expect(out->scales, base + "_scale", DGPP_DT_F8_E4M3, {rows, cols / 16})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, base + "_global_scale", &out->global, nullptr)) != DGPP_OK) return rc;
+    return expect(out->global, base + "_global_scale", DGPP_DT_F32, {1});
+  }
+  if (format != DGPP_BIND_FP8) return fail(DGPP_INVALID_ARGUMENT, "unknown expert format " + std::to_string(format));
+  if ((rc = find_in(files, n_files, base, &out->payload, &out->file_index)) != DGPP_OK) return rc;
+  if ((rc = expect(out->payload, base, DGPP_DT_F8_E4M3, {rows, cols})) != DGPP_OK) return rc;
+  if ((rc = find_in(files, n_files, base + "_scale_inv", &out->scales, nullptr)) != DGPP_OK) return rc;
+  return expect(out->scales, base + "_scale_inv", DGPP_DT_F32, {(rows + 127) / 128, (cols + 127) / 128});
+}
+
+}  // namespace
+
+extern "C" int dgpp_glm_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* layer_prefix, int n_experts,
+                                       int64_t hidden, int64_t inter, int routed_format, int64_t shared_inter, int with_bias,
+                                       DgppTensorInfo* router_weight, DgppTensorInfo* router_bias, DgppMoeMatrixTensors* shared,
+                                       DgppMoeMatrixTensors* routed) {
+  if (!files || n_files <= 0 || !layer_prefix || !router_weight || !routed || (shared_inter > 0 && !shared) || (with_bias && !router_bias))
+    return fail(DGPP_INVALID_ARGUMENT, "glm_moe_bind_layer: null argument");
+  if (n_experts <= 0 || hidden <= 0 || inter <= 0 || shared_inter < 0) return fail(DGPP_INVALID_ARGUMENT, "glm_moe_bind_layer: geometry must be positive");
+  const std::string p(layer_prefix);
+  static const char* const kProj[3] = {"gate_proj.weight", "up_proj.weight", "down_proj.weight"};
+  int rc;
+  if ((rc = find_in(files, n_files, p + "mlp.gate.weight", router_weight, nullptr)) != DGPP_OK) return rc;
+  if ((rc = expect(*router_weight, p + "mlp.gate.weight", DGPP_DT_BF16, {n_experts, hidden})) != DGPP_OK) return rc;
+  if (with_bias) {
+    const std::string name = p + "mlp.gate.e_score_correction_bias";
+    if ((rc = find_in(files, n_files, name, router_bias, nullptr)) != DGPP_OK) return rc;
+    if ((rc = expect(*router_bias, name, DGPP_DT_F32, {n_experts})) != DGPP_OK) return rc;
+  }
+  if (shared_inter > 0) {
+    // One shared expert under the un-indexed name, always block FP8.
+    for (int m = 0; m < 3; ++m) {
+      const int64_t rows = m == 2 ? hidden : shared_inter, cols = m == 2 ? shared_inter : hidden;
+      if ((rc = bind_matrix(files, n_files, p + "mlp.shared_experts." + kProj[m], rows, cols, DGPP_BIND_FP8, shared + m)) != DGPP_OK)
+        return rc;
+    }
+  }
+  for (int e = 0; e < n_experts; ++e) {
+    const std::string ep = p + "mlp.experts." + std::to_string(e) + ".";
+    for (int m = 0; m < 3; ++m) {
+      const int64_t rows = m == 2 ? hidden : inter, cols = m == 2 ? inter : hidden;
+      if ((rc = bind_matrix(files, n_files, ep + kProj[m], rows, cols, routed_format, routed + static_cast<size_t>(e) * 3 + m)) !=
+          DGPP_OK)
+        return rc;
+    }
+  }
+  return DGPP_OK;
+}

@@ -190,3 +190,32 @@ def fp4_cols_slice(m, col_start: int, cols: int):
     out = _lib.Fp4Matrix()
     _check(lib().dgpp_fp4_cols_slice(C.byref(m), col_start, cols, payload.ctypes.data, scales.ctypes.data, C.byref(out)))
     return payload, scales, out
+
+
+BIND_FP8, BIND_NVFP4 = 0, 1
+
+
+class MoeMatrixTensors(C.Structure):
+    """DgppMoeMatrixTensors: where one expert matrix's tensors sit in the shards."""
+    _fields_ = [("payload", TensorInfo), ("scales", TensorInfo), ("global_", TensorInfo), ("format", C.c_int32),
+                ("file_index", C.c_int32)]
+
+
+SIGNATURES["dgpp_glm_moe_bind_layer"] = (_I, [C.POINTER(_P), _I, C.c_char_p, _I, C.c_int64, C.c_int64, _I, C.c_int64, _I,
+                                               C.POINTER(TensorInfo), C.POINTER(TensorInfo), C.POINTER(MoeMatrixTensors),
+                                               C.POINTER(MoeMatrixTensors)])
+
+
+def glm_moe_bind_layer(files, layer_prefix: str, n_experts: int, hidden: int, inter: int, routed_format: int, shared_inter: int = 0,
+                       with_bias: bool = True):
+    """The tensors of one GLM-family MoE layer looked up by name across `files` (SafetensorsFile objects) and checked
+    against the geometry. Returns (router_weight, router_bias or None, shared [3] or None, routed [n_experts][3])."""
+    handles = (_P * len(files))(*[f._h for f in files])
+    rw, rb = TensorInfo(), TensorInfo()
+    shared = (MoeMatrixTensors * 3)()
+    routed = (MoeMatrixTensors * (3 * n_experts))()
+    _check(lib().dgpp_glm_moe_bind_layer(handles, len(files), layer_prefix.encode(), n_experts, hidden, inter, routed_format,
+                                         shared_inter, 1 if with_bias else 0, C.byref(rw), C.byref(rb) if with_bias else None,
+                                         shared if shared_inter > 0 else None, routed))
+    return (rw, rb if with_bias else None, list(shared) if shared_inter > 0 else None,
+            [[routed[3 * e + m] for m in range(3)] for e in range(n_experts)])

@@ -127,6 +127,31 @@ int dgpp_fp4_cols_slice(const DgppFp4Matrix* m, int64_t col_start, int64_t cols,
 int dgpp_expert_view_from_quant(const DgppQuantMatrix* m, DgppMoeExpertView* out);
 int dgpp_expert_view_from_fp4(const DgppFp4Matrix* m, DgppMoeExpertView* out);
 
+/* The tensors of one MoE layer of a GLM-family checkpoint under the names its exports carry
+ * (src/models/glm/binding.cpp:32-54, :163-206), looked up across the given shards and checked against the
+ * geometry: router `<p>mlp.gate.weight` BF16 [E, H] (and `<p>mlp.gate.e_score_correction_bias` F32 [E]); the shared
+ * expert `<p>mlp.shared_experts.{gate,up,down}_proj.weight` as block FP8; routed expert e
+ * `<p>mlp.experts.<e>.{gate,up,down}_proj.weight` as block FP8 (`<name>` F8_E4M3 [rows, cols] with
+ * `<name>_scale_inv` F32 [ceil(rows / 128), ceil(cols / 128)]) or as NVFP4 (`<name>_packed` U8 [rows, cols / 2],
+ * `<name>_scale` F8_E4M3 [rows, cols / 16], `<name>_global_scale` F32 [1]: the divisor the kernels take).
+ * gate / up are [inter, hidden], down is [hidden, inter]. */
+enum { DGPP_BIND_FP8 = 0, DGPP_BIND_NVFP4 = 1 };
+typedef struct DgppMoeMatrixTensors {
+  DgppTensorInfo payload;
+  DgppTensorInfo scales;
+  DgppTensorInfo global;   /* NVFP4 only; zeroed otherwise */
+  int32_t format;          /* DGPP_BIND_* */
+  int32_t file_index;      /* the shard (index into `files`) that holds the payload */
+} DgppMoeMatrixTensors;
+/* `p` = layer_prefix, e.g. "model.layers.3.". routed: [n_experts * 3] (gate, up, down per expert); shared: [3]
+ * when shared_inter > 0 (its width; the exports use the routed experts' own); router_bias when with_bias. A missing tensor, or one whose dtype or shape differs from what
+ * the geometry fixes, fails with DGPP_INVALID_ARGUMENT and a message that names it; nothing is copied: the
+ * descriptions point into the shards' mappings. */
+int dgpp_glm_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* layer_prefix, int n_experts,
+                            int64_t hidden, int64_t inter, int routed_format, int64_t shared_inter, int with_bias,
+                            DgppTensorInfo* router_weight, DgppTensorInfo* router_bias, DgppMoeMatrixTensors* shared,
+                            DgppMoeMatrixTensors* routed);
+
 #ifdef __cplusplus
 }
 #endif

@@ -161,3 +161,72 @@ def test_column_slices_feed_the_grid_launchers(gpu):
     sync()
     ref = host(full).astype(np.float64)
     assert np.max(np.abs(total - ref)) <= 1e-4 * max(1.0, np.max(np.abs(ref)))
+
+
+@pytest.mark.parametrize("kind", ["fp8", "nvfp4"])
+def test_layer_bound_by_the_glm_tensor_names_is_bitwise_the_layer_from_the_arrays(gpu, tmp_path, kind):
+    """The checkpoint spells its tensors as a GLM-family export does (src/models/glm/binding.cpp:32-54, :163-206);
+    the loader's binding finds and checks them across two shards, and the layer built from what it found gives the
+    bits of the layer built from the arrays."""
+    import ctypes as C
+
+    E, H, I, K, T = 6, 512, 128, 3, 5
+    p = moe_data.make_problem(E, H, I, K, T, kind, 8900, shared_kind=None, limit=float("inf"), std=0.05)
+    prefix = "model.layers.7."
+    tensors, dtypes = {prefix + "mlp.gate.weight": p.router_gate,
+                       prefix + "mlp.gate.e_score_correction_bias": p.router_bias}, {}
+    for e, mats in enumerate(p.experts):
+        for m, proj in zip(mats, PROJ):
+            base = f"{prefix}mlp.experts.{e}.{proj}.weight"
+            if kind == "fp8":
+                tensors[base], dtypes[base] = m.payload, "F8_E4M3"
+                tensors[base + "_scale_inv"] = m.scales
+            else:
+                tensors[base + "_packed"] = m.payload
+                tensors[base + "_scale"], dtypes[base + "_scale"] = m.scales, "F8_E4M3"
+                tensors[base + "_global_scale"] = m.glob
+    names = sorted(tensors)
+    paths = []
+    for i in range(2):
+        paths.append(str(tmp_path / f"model-0000{i + 1}-of-00002.safetensors"))
+        write_checkpoint(paths[-1], {n: tensors[n] for n in names[i::2]}, dtypes)
+
+    def upload(info):
+        a = np.frombuffer((C.c_uint8 * info.nbytes).from_address(info.data), dtype=np.uint8)
+        return dev(np.array(a))
+
+    files = [LD.SafetensorsFile(q) for q in paths]
+    keep, entries = [], []
+    try:
+        rw, rb, shared, routed = LD.glm_moe_bind_layer(files, prefix, E, H, I, LD.BIND_FP8 if kind == "fp8" else LD.BIND_NVFP4)
+        assert shared is None and rw.dims() == (E, H) and rb.dims() == (E,)
+        for e in range(E):
+            for m in routed[e]:
+                wd, sd = upload(m.payload), upload(m.scales)
+                keep += [wd, sd]
+                rows = m.payload.dims()[0]
+                if kind == "fp8":
+                    q = LD.QuantMatrix(wd.data_ptr(), sd.data_ptr(), None, rows, m.payload.dims()[1], 128, 128)
+                    entries.append(LD.expert_view_from_quant(q))
+                else:
+                    gd = upload(m.global_)
+                    keep.append(gd)
+                    q = _lib.Fp4Matrix(wd.data_ptr(), sd.data_ptr(), gd.data_ptr(), rows, m.payload.dims()[1] * 2, 16, 0, None)
+                    entries.append(LD.expert_view_from_fp4(q))
+    finally:
+        for f in files:
+            f.close()
+    d = DeviceMoe(p)
+    ref_layer = make_layer(p, d, 1, 1.0, T)
+    d2 = DeviceMoe.__new__(DeviceMoe)
+    d2.p, d2.keep, d2.views, d2.x, d2.shared_view_base, d2.sh = p, keep, view_table(entries), d.x, -1, None
+    d2.fp4_group = d.fp4_group
+    got_layer = make_layer(p, d2, 1, 1.0, T)
+    want, got = dev_empty((T, H), np.uint16), dev_empty((T, H), np.uint16)
+    ref_layer.enqueue_decode(d.x, H, want, T)
+    got_layer.enqueue_decode(d.x, H, got, T)
+    sync()
+    assert np.array_equal(host(got, np.uint16), host(want, np.uint16))
+    assert host(want, np.uint16).any()
+    ref_layer.close()
+    got_layer.close()

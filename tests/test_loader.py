@@ -284,3 +284,119 @@ def test_quant_slice_and_fp4_cols_slice_contracts():
         for start, n in ((8, 32), (0, 40), (224, 64), (-32, 32), (0, 0)):
             with pytest.raises(ValueError):
                 LD.fp4_cols_slice(m4, start, n)
+
+
+# ---- tensor names of a GLM-family MoE layer (src/models/glm/binding.cpp:32-54, :163-206) ---------------------------
+
+def _glm_layer_tensors(prefix, E, H, I, fmt, shared_inter, rng):
+    tensors, dtypes = {}, {}
+
+    def fp8(name, rows, cols):
+        tensors[name] = rng.integers(0, 120, size=(rows, cols), dtype=np.uint8)
+        dtypes[name] = "F8_E4M3"
+        tensors[name + "_scale_inv"] = rng.random((-(-rows // 128), -(-cols // 128)), dtype=np.float32)
+
+    def nvfp4(name, rows, cols):
+        tensors[name + "_packed"] = rng.integers(0, 256, size=(rows, cols // 2), dtype=np.uint8)
+        tensors[name + "_scale"] = rng.integers(0, 120, size=(rows, cols // 16), dtype=np.uint8)
+        dtypes[name + "_scale"] = "F8_E4M3"
+        tensors[name + "_global_scale"] = np.array([2688.0], dtype=np.float32)
+
+    tensors[prefix + "mlp.gate.weight"] = rng.integers(0, 2 ** 15, size=(E, H), dtype=np.uint16)
+    dtypes[prefix + "mlp.gate.weight"] = "BF16"
+    tensors[prefix + "mlp.gate.e_score_correction_bias"] = rng.random(E, dtype=np.float32)
+    for proj, (r, c) in (("gate_proj", (shared_inter, H)), ("up_proj", (shared_inter, H)), ("down_proj", (H, shared_inter))):
+        if shared_inter:
+            fp8(f"{prefix}mlp.shared_experts.{proj}.weight", r, c)
+    for e in range(E):
+        for proj, (r, c) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            (nvfp4 if fmt == LD.BIND_NVFP4 else fp8)(f"{prefix}mlp.experts.{e}.{proj}.weight", r, c)
+    return tensors, dtypes
+
+
+def _write_named(path, tensors, dtypes):
+    names = {np.dtype(np.uint8): "U8", np.dtype(np.float32): "F32", np.dtype(np.uint16): "BF16"}
+    header, blobs, at = {}, [], 0
+    for name, a in tensors.items():
+        a = np.ascontiguousarray(a)
+        header[name] = {"dtype": dtypes.get(name, names[a.dtype]), "shape": list(a.shape), "data_offsets": [at, at + a.nbytes]}
+        blobs.append(a.tobytes())
+        at += a.nbytes
+    text = json.dumps(header, separators=(",", ":"))
+    text += " " * (-(8 + len(text)) % 8)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(text)) + text.encode() + b"".join(blobs))
+
+
+@pytest.mark.parametrize("fmt", [LD.BIND_FP8, LD.BIND_NVFP4])
+def test_glm_moe_layer_binding_finds_every_tensor_across_shards(tmp_path, fmt):
+    rng = np.random.default_rng(17)
+    E, H, I, S = 5, 256, 160, 160
+    prefix = "model.layers.3."
+    tensors, dtypes = _glm_layer_tensors(prefix, E, H, I, fmt, S, rng)
+    names = list(tensors)
+    shards = [dict((n, tensors[n]) for n in names[i::2]) for i in range(2)]      # spread over two shards
+    paths = []
+    for i, sh in enumerate(shards):
+        paths.append(str(tmp_path / f"model-{i}.safetensors"))
+        _write_named(paths[-1], sh, dtypes)
+    files = [LD.SafetensorsFile(p) for p in paths]
+    try:
+        rw, rb, shared, routed = LD.glm_moe_bind_layer(files, prefix, E, H, I, fmt, S)
+        assert rw.dims() == (E, H) and rw.dtype == LD.DT_BF16 and rb.dims() == (E,)
+        assert np.array_equal(files[0].array(prefix + "mlp.gate.weight") if (prefix + "mlp.gate.weight") in files[0]
+                              else files[1].array(prefix + "mlp.gate.weight"), tensors[prefix + "mlp.gate.weight"])
+        assert [m.payload.dims() for m in shared] == [(S, H), (S, H), (H, S)] and all(m.format == LD.BIND_FP8 for m in shared)
+        for e in range(E):
+            for m, proj, (r, c) in zip(routed[e], ("gate_proj", "up_proj", "down_proj"), ((I, H), (I, H), (H, I))):
+                base = f"{prefix}mlp.experts.{e}.{proj}.weight"
+                pay_name = base + ("_packed" if fmt == LD.BIND_NVFP4 else "")
+                assert m.format == fmt and pay_name in files[m.file_index]
+                want = tensors[pay_name]
+                got = np.frombuffer((C.c_uint8 * m.payload.nbytes).from_address(m.payload.data), dtype=np.uint8)
+                assert np.array_equal(got.reshape(want.shape), want)
+                if fmt == LD.BIND_NVFP4:
+                    assert m.payload.dims() == (r, c // 2) and m.scales.dims() == (r, c // 16) and m.global_.dims() == (1,)
+                    assert m.scales.dtype == LD.DT_F8_E4M3 and m.global_.dtype == LD.DT_F32
+                else:
+                    assert m.payload.dims() == (r, c) and m.scales.dims() == (-(-r // 128), -(-c // 128))
+                    assert m.payload.dtype == LD.DT_F8_E4M3 and m.scales.dtype == LD.DT_F32
+        # no shared expert, no bias: nothing of them is looked up
+        rw2, rb2, sh2, routed2 = LD.glm_moe_bind_layer(files, prefix, E, H, I, fmt, 0, with_bias=False)
+        assert rb2 is None and sh2 is None and len(routed2) == E
+    finally:
+        for f in files:
+            f.close()
+
+
+def test_glm_moe_layer_binding_names_what_is_wrong(tmp_path):
+    rng = np.random.default_rng(18)
+    E, H, I = 3, 128, 64
+    prefix = "model.layers.0."
+    tensors, dtypes = _glm_layer_tensors(prefix, E, H, I, LD.BIND_FP8, 0, rng)
+
+    def bind(t, d, **kw):
+        path = str(tmp_path / f"m{len(list(tmp_path.iterdir()))}.safetensors")
+        _write_named(path, t, d)
+        with LD.SafetensorsFile(path) as f:
+            return LD.glm_moe_bind_layer([f], prefix, kw.get("E", E), H, I, kw.get("fmt", LD.BIND_FP8), kw.get("S", 0))
+
+    bind(tensors, dtypes)
+    missing = dict(tensors)
+    del missing[prefix + "mlp.experts.2.up_proj.weight_scale_inv"]
+    with pytest.raises(ValueError, match=r"missing tensor 'model\.layers\.0\.mlp\.experts\.2\.up_proj\.weight_scale_inv'"):
+        bind(missing, dtypes)
+    wrong_dtype = dict(dtypes)
+    wrong_dtype[prefix + "mlp.experts.1.down_proj.weight"] = "U8"
+    with pytest.raises(ValueError, match=r"experts\.1\.down_proj\.weight' is dtype"):
+        bind(tensors, wrong_dtype)
+    wrong_shape = dict(tensors)
+    wrong_shape[prefix + "mlp.experts.0.gate_proj.weight_scale_inv"] = np.zeros((2, 1), dtype=np.float32)
+    with pytest.raises(ValueError, match=r"gate_proj\.weight_scale_inv' is dtype .* expected"):
+        bind(wrong_shape, dtypes)
+    with pytest.raises(ValueError, match=r"mlp\.gate\.weight' is dtype .*\[3, 128\], expected .*\[4, 128\]"):
+        bind(tensors, dtypes, E=4)                       # the router of this file serves three experts
+    with pytest.raises(ValueError, match="missing tensor"):
+        bind(tensors, dtypes, fmt=LD.BIND_NVFP4)         # the NVFP4 spelling is not there
+    with pytest.raises(ValueError, match="shared_experts"):
+        bind(tensors, dtypes, S=64)
