@@ -722,11 +722,30 @@ int bind_matrix(const DgppSafetensors* const* files, int n_files, const std::str
     if ((rc = find_in(files, n_files, base + "_global_scale", &out->global, nullptr)) != DGPP_OK) return rc;
     return expect(out->global, base + "_global_scale", DGPP_DT_F32, {1});
   }
-  if (format != DGPP_BIND_FP8) return fail(DGPP_INVALID_ARGUMENT, "unknown expert format " + std::to_string(format));
+  const std::string stem = base.size() > 7 && base.compare(base.size() - 7, 7, ".weight") == 0 ? base.substr(0, base.size() - 7) : base;
+  if (format == DGPP_BIND_NVFP4_MODELOPT) {
+    if (cols % 16 != 0) return fail(DGPP_INVALID_ARGUMENT, "NVFP4 needs K % 16 == 0: '" + base + "'");
+    if ((rc = find_in(files, n_files, base, &out->payload, &out->file_index)) != DGPP_OK) return rc;
+    if ((rc = expect(out->payload, base, DGPP_DT_U8, {rows, cols / 2})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, stem + ".weight_scale", &out->scales, nullptr)) != DGPP_OK) return rc;
+    if ((rc = expect(out->scales, stem + ".weight_scale", DGPP_DT_F8_E4M3, {rows, cols / 16})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, stem + ".weight_scale_2", &out->global, nullptr)) != DGPP_OK) return rc;
+    return expect(out->global, stem + ".weight_scale_2", DGPP_DT_F32, {});
+  }
+  if (format == DGPP_BIND_MXFP8) {
+    if (cols % 32 != 0) return fail(DGPP_INVALID_ARGUMENT, "MXFP8 needs K % 32 == 0: '" + base + "'");
+    if ((rc = find_in(files, n_files, base, &out->payload, &out->file_index)) != DGPP_OK) return rc;
+    if ((rc = expect(out->payload, base, DGPP_DT_F8_E4M3, {rows, cols})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, stem + ".weight_scale", &out->scales, nullptr)) != DGPP_OK) return rc;
+    return expect(out->scales, stem + ".weight_scale", DGPP_DT_U8, {rows, cols / 32});
+  }
+  if (format != DGPP_BIND_FP8 && format != DGPP_BIND_FP8_BF16_SCALES)
+    return fail(DGPP_INVALID_ARGUMENT, "unknown expert format " + std::to_string(format));
   if ((rc = find_in(files, n_files, base, &out->payload, &out->file_index)) != DGPP_OK) return rc;
   if ((rc = expect(out->payload, base, DGPP_DT_F8_E4M3, {rows, cols})) != DGPP_OK) return rc;
   if ((rc = find_in(files, n_files, base + "_scale_inv", &out->scales, nullptr)) != DGPP_OK) return rc;
-  return expect(out->scales, base + "_scale_inv", DGPP_DT_F32, {(rows + 127) / 128, (cols + 127) / 128});
+  return expect(out->scales, base + "_scale_inv", format == DGPP_BIND_FP8 ? DGPP_DT_F32 : DGPP_DT_BF16,
+                {(rows + 127) / 128, (cols + 127) / 128});
 }
 
 }  // namespace
@@ -758,6 +777,40 @@ extern "C" int dgpp_glm_moe_bind_layer(const DgppSafetensors* const* files, int 
   }
   for (int e = 0; e < n_experts; ++e) {
     const std::string ep = p + "mlp.experts." + std::to_string(e) + ".";
+    for (int m = 0; m < 3; ++m) {
+      const int64_t rows = m == 2 ? hidden : inter, cols = m == 2 ? inter : hidden;
+      if ((rc = bind_matrix(files, n_files, ep + kProj[m], rows, cols, routed_format, routed + static_cast<size_t>(e) * 3 + m)) !=
+          DGPP_OK)
+        return rc;
+    }
+  }
+  return DGPP_OK;
+}
+
+extern "C" int dgpp_qwen_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* mlp_prefix, int n_experts,
+                                        int64_t hidden, int64_t inter, int routed_format, int64_t shared_inter, int shared_format,
+                                        DgppTensorInfo* router_weight, DgppTensorInfo* shared_gate, DgppMoeMatrixTensors* shared,
+                                        DgppMoeMatrixTensors* routed) {
+  if (!files || n_files <= 0 || !mlp_prefix || !router_weight || !routed || (shared_inter > 0 && (!shared || !shared_gate)))
+    return fail(DGPP_INVALID_ARGUMENT, "qwen_moe_bind_layer: null argument");
+  if (n_experts <= 0 || hidden <= 0 || inter <= 0 || shared_inter < 0)
+    return fail(DGPP_INVALID_ARGUMENT, "qwen_moe_bind_layer: geometry must be positive");
+  const std::string p(mlp_prefix);
+  static const char* const kProj[3] = {"gate_proj.weight", "up_proj.weight", "down_proj.weight"};
+  int rc;
+  if ((rc = find_in(files, n_files, p + "gate.weight", router_weight, nullptr)) != DGPP_OK) return rc;
+  if ((rc = expect(*router_weight, p + "gate.weight", DGPP_DT_BF16, {n_experts, hidden})) != DGPP_OK) return rc;
+  if (shared_inter > 0) {
+    if ((rc = find_in(files, n_files, p + "shared_expert_gate.weight", shared_gate, nullptr)) != DGPP_OK) return rc;
+    if ((rc = expect(*shared_gate, p + "shared_expert_gate.weight", DGPP_DT_BF16, {1, hidden})) != DGPP_OK) return rc;
+    for (int m = 0; m < 3; ++m) {
+      const int64_t rows = m == 2 ? hidden : shared_inter, cols = m == 2 ? shared_inter : hidden;
+      if ((rc = bind_matrix(files, n_files, p + "shared_expert." + kProj[m], rows, cols, shared_format, shared + m)) != DGPP_OK)
+        return rc;
+    }
+  }
+  for (int e = 0; e < n_experts; ++e) {
+    const std::string ep = p + "experts." + std::to_string(e) + ".";
     for (int m = 0; m < 3; ++m) {
       const int64_t rows = m == 2 ? hidden : inter, cols = m == 2 ? inter : hidden;
       if ((rc = bind_matrix(files, n_files, ep + kProj[m], rows, cols, routed_format, routed + static_cast<size_t>(e) * 3 + m)) !=

@@ -192,7 +192,7 @@ def fp4_cols_slice(m, col_start: int, cols: int):
     return payload, scales, out
 
 
-BIND_FP8, BIND_NVFP4 = 0, 1
+BIND_FP8, BIND_NVFP4, BIND_FP8_BF16_SCALES, BIND_NVFP4_MODELOPT, BIND_MXFP8 = 0, 1, 2, 3, 4
 
 
 class MoeMatrixTensors(C.Structure):
@@ -218,4 +218,24 @@ def glm_moe_bind_layer(files, layer_prefix: str, n_experts: int, hidden: int, in
                                          shared_inter, 1 if with_bias else 0, C.byref(rw), C.byref(rb) if with_bias else None,
                                          shared if shared_inter > 0 else None, routed))
     return (rw, rb if with_bias else None, list(shared) if shared_inter > 0 else None,
+            [[routed[3 * e + m] for m in range(3)] for e in range(n_experts)])
+
+
+SIGNATURES["dgpp_qwen_moe_bind_layer"] = (_I, [C.POINTER(_P), _I, C.c_char_p, _I, C.c_int64, C.c_int64, _I, C.c_int64, _I,
+                                                C.POINTER(TensorInfo), C.POINTER(TensorInfo), C.POINTER(MoeMatrixTensors),
+                                                C.POINTER(MoeMatrixTensors)])
+
+
+def qwen_moe_bind_layer(files, mlp_prefix: str, n_experts: int, hidden: int, inter: int, routed_format: int, shared_inter: int = 0,
+                        shared_format: int = BIND_FP8):
+    """The tensors of one Qwen-family MoE block. Returns (router_weight, shared_gate or None, shared [3] or None,
+    routed [n_experts][3])."""
+    handles = (_P * len(files))(*[f._h for f in files])
+    rw, sg = TensorInfo(), TensorInfo()
+    shared = (MoeMatrixTensors * 3)()
+    routed = (MoeMatrixTensors * (3 * n_experts))()
+    _check(lib().dgpp_qwen_moe_bind_layer(handles, len(files), mlp_prefix.encode(), n_experts, hidden, inter, routed_format,
+                                          shared_inter, shared_format, C.byref(rw), C.byref(sg) if shared_inter > 0 else None,
+                                          shared if shared_inter > 0 else None, routed))
+    return (rw, sg if shared_inter > 0 else None, list(shared) if shared_inter > 0 else None,
             [[routed[3 * e + m] for m in range(3)] for e in range(n_experts)])

@@ -135,7 +135,14 @@ int dgpp_expert_view_from_fp4(const DgppFp4Matrix* m, DgppMoeExpertView* out);
  * `<name>_scale_inv` F32 [ceil(rows / 128), ceil(cols / 128)]) or as NVFP4 (`<name>_packed` U8 [rows, cols / 2],
  * `<name>_scale` F8_E4M3 [rows, cols / 16], `<name>_global_scale` F32 [1]: the divisor the kernels take).
  * gate / up are [inter, hidden], down is [hidden, inter]. */
-enum { DGPP_BIND_FP8 = 0, DGPP_BIND_NVFP4 = 1 };
+enum {
+  DGPP_BIND_FP8 = 0,              /* `<name>` F8_E4M3 + `<name>_scale_inv` F32 grid */
+  DGPP_BIND_NVFP4 = 1,            /* `<name>_packed`, `<name>_scale`, `<name>_global_scale` (the divisor itself) */
+  DGPP_BIND_FP8_BF16_SCALES = 2,  /* as FP8 with a BF16 grid: widen it to F32 at load (exact) before the launchers see it */
+  DGPP_BIND_NVFP4_MODELOPT = 3,   /* `<base>.weight` U8 [rows, cols / 2], `<base>.weight_scale` F8_E4M3 [rows, cols / 16],
+                                     `<base>.weight_scale_2` F32 scalar: the kernels' divisor is 1 / weight_scale_2 */
+  DGPP_BIND_MXFP8 = 4             /* `<base>.weight` F8_E4M3, `<base>.weight_scale` U8 (e8m0) [rows, cols / 32] */
+};
 typedef struct DgppMoeMatrixTensors {
   DgppTensorInfo payload;
   DgppTensorInfo scales;
@@ -151,6 +158,17 @@ int dgpp_glm_moe_bind_layer(const DgppSafetensors* const* files, int n_files, co
                             int64_t hidden, int64_t inter, int routed_format, int64_t shared_inter, int with_bias,
                             DgppTensorInfo* router_weight, DgppTensorInfo* router_bias, DgppMoeMatrixTensors* shared,
                             DgppMoeMatrixTensors* routed);
+
+/* The same for a Qwen-family MoE block (src/models/qwen/binding.cpp:26-66, :158-215); `p` = mlp_prefix, e.g.
+ * "model.layers.3.mlp.": router `<p>gate.weight` BF16 [E, H]; with shared_inter > 0 the shared expert's scalar gate
+ * `<p>shared_expert_gate.weight` BF16 [1, H] and `<p>shared_expert.{gate,up,down}_proj.weight` in shared_format
+ * (DGPP_BIND_FP8 or DGPP_BIND_MXFP8); routed expert e `<p>experts.<e>.{gate,up,down}_proj.weight` in routed_format
+ * (DGPP_BIND_FP8_BF16_SCALES, DGPP_BIND_FP8 or DGPP_BIND_NVFP4_MODELOPT; the export's `input_scale` is not looked up:
+ * this path keeps BF16 activations). BF16-weight and int4 forms of these exports are not bound. */
+int dgpp_qwen_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* mlp_prefix, int n_experts,
+                             int64_t hidden, int64_t inter, int routed_format, int64_t shared_inter, int shared_format,
+                             DgppTensorInfo* router_weight, DgppTensorInfo* shared_gate, DgppMoeMatrixTensors* shared,
+                             DgppMoeMatrixTensors* routed);
 
 #ifdef __cplusplus
 }

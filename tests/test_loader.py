@@ -318,7 +318,7 @@ def _write_named(path, tensors, dtypes):
     names = {np.dtype(np.uint8): "U8", np.dtype(np.float32): "F32", np.dtype(np.uint16): "BF16"}
     header, blobs, at = {}, [], 0
     for name, a in tensors.items():
-        a = np.ascontiguousarray(a)
+        a = np.asarray(a, order="C")                       # keeps a scalar's empty shape
         header[name] = {"dtype": dtypes.get(name, names[a.dtype]), "shape": list(a.shape), "data_offsets": [at, at + a.nbytes]}
         blobs.append(a.tobytes())
         at += a.nbytes
@@ -400,3 +400,80 @@ def test_glm_moe_layer_binding_names_what_is_wrong(tmp_path):
         bind(tensors, dtypes, fmt=LD.BIND_NVFP4)         # the NVFP4 spelling is not there
     with pytest.raises(ValueError, match="shared_experts"):
         bind(tensors, dtypes, S=64)
+
+
+# ---- tensor names of a Qwen-family MoE block (src/models/qwen/binding.cpp:26-66, :158-215) -------------------------
+
+def _qwen_block_tensors(p, E, H, I, S, routed_fmt, shared_fmt, rng):
+    tensors, dtypes = {}, {}
+
+    def put(name, rows, cols, fmt):
+        stem = name[:-len(".weight")]
+        if fmt == LD.BIND_NVFP4_MODELOPT:
+            tensors[name] = rng.integers(0, 256, size=(rows, cols // 2), dtype=np.uint8)
+            tensors[stem + ".weight_scale"] = rng.integers(0, 120, size=(rows, cols // 16), dtype=np.uint8)
+            dtypes[stem + ".weight_scale"] = "F8_E4M3"
+            tensors[stem + ".weight_scale_2"] = np.array(3.5e-4, dtype=np.float32)
+            tensors[stem + ".input_scale"] = np.array(1.0, dtype=np.float32)       # shipped, never looked up
+        elif fmt == LD.BIND_MXFP8:
+            tensors[name] = rng.integers(0, 120, size=(rows, cols), dtype=np.uint8)
+            dtypes[name] = "F8_E4M3"
+            tensors[stem + ".weight_scale"] = rng.integers(110, 130, size=(rows, cols // 32), dtype=np.uint8)
+        else:
+            tensors[name] = rng.integers(0, 120, size=(rows, cols), dtype=np.uint8)
+            dtypes[name] = "F8_E4M3"
+            grid = (-(-rows // 128), -(-cols // 128))
+            if fmt == LD.BIND_FP8_BF16_SCALES:
+                tensors[name + "_scale_inv"] = rng.integers(0x3000, 0x3F00, size=grid, dtype=np.uint16)
+                dtypes[name + "_scale_inv"] = "BF16"
+            else:
+                tensors[name + "_scale_inv"] = rng.random(grid, dtype=np.float32)
+
+    tensors[p + "gate.weight"] = rng.integers(0, 2 ** 15, size=(E, H), dtype=np.uint16)
+    dtypes[p + "gate.weight"] = "BF16"
+    if S:
+        tensors[p + "shared_expert_gate.weight"] = rng.integers(0, 2 ** 15, size=(1, H), dtype=np.uint16)
+        dtypes[p + "shared_expert_gate.weight"] = "BF16"
+        for proj, (r, c) in (("gate_proj", (S, H)), ("up_proj", (S, H)), ("down_proj", (H, S))):
+            put(f"{p}shared_expert.{proj}.weight", r, c, shared_fmt)
+    for e in range(E):
+        for proj, (r, c) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            put(f"{p}experts.{e}.{proj}.weight", r, c, routed_fmt)
+    return tensors, dtypes
+
+
+@pytest.mark.parametrize("routed_fmt,shared_fmt", [(LD.BIND_FP8_BF16_SCALES, LD.BIND_FP8), (LD.BIND_NVFP4_MODELOPT, LD.BIND_MXFP8),
+                                                   (LD.BIND_FP8, LD.BIND_FP8)])
+def test_qwen_moe_block_binding(tmp_path, routed_fmt, shared_fmt):
+    rng = np.random.default_rng(23)
+    E, H, I, S = 4, 256, 128, 192
+    p = "model.layers.5.mlp."
+    tensors, dtypes = _qwen_block_tensors(p, E, H, I, S, routed_fmt, shared_fmt, rng)
+    path = str(tmp_path / "qwen.safetensors")
+    _write_named(path, tensors, dtypes)
+    with LD.SafetensorsFile(path) as f:
+        rw, sg, shared, routed = LD.qwen_moe_bind_layer([f], p, E, H, I, routed_fmt, S, shared_fmt)
+        assert rw.dims() == (E, H) and sg.dims() == (1, H) and sg.dtype == LD.DT_BF16
+        assert [m.format for m in shared] == [shared_fmt] * 3
+        assert shared[2].payload.dims() == (H, S)
+        if shared_fmt == LD.BIND_MXFP8:
+            assert shared[0].scales.dims() == (S, H // 32) and shared[0].scales.dtype == LD.DT_U8
+        for e in range(E):
+            g, u, d = routed[e]
+            if routed_fmt == LD.BIND_NVFP4_MODELOPT:
+                assert g.payload.dims() == (I, H // 2) and g.scales.dims() == (I, H // 16) and g.global_.dims() == ()
+                assert d.payload.dims() == (H, I // 2)
+                got = np.frombuffer((C.c_uint8 * 4).from_address(g.global_.data), dtype=np.float32)[0]
+                assert got == np.float32(3.5e-4)
+            else:
+                want_dt = LD.DT_BF16 if routed_fmt == LD.BIND_FP8_BF16_SCALES else LD.DT_F32
+                assert g.payload.dims() == (I, H) and g.scales.dims() == (1, 2) and g.scales.dtype == want_dt
+                assert d.scales.dims() == (2, 1)
+        rw2, sg2, sh2, routed2 = LD.qwen_moe_bind_layer([f], p, E, H, I, routed_fmt)
+        assert sg2 is None and sh2 is None and len(routed2) == E
+        with pytest.raises(ValueError, match="missing tensor|is dtype"):
+            LD.qwen_moe_bind_layer([f], p, E, H, I, LD.BIND_MXFP8 if routed_fmt != LD.BIND_MXFP8 else LD.BIND_FP8)
+        with pytest.raises(ValueError, match=r"shared_expert\.gate_proj\.weight' is dtype"):
+            LD.qwen_moe_bind_layer([f], p, E, H, I, routed_fmt, S + 64, shared_fmt)
+        with pytest.raises(ValueError, match="unknown expert format"):
+            LD.qwen_moe_bind_layer([f], p, E, H, I, 9)
