@@ -13,6 +13,11 @@
 
 #include <algorithm>
 #include <cerrno>
+#include <filesystem>
+#include <fstream>
+#include <iterator>
+#include <map>
+#include <set>
 #include <cstdint>
 #include <cstring>
 #include <limits>
@@ -819,4 +824,112 @@ extern "C" int dgpp_qwen_moe_bind_layer(const DgppSafetensors* const* files, int
     }
   }
   return DGPP_OK;
+}
+
+// ---- a checkpoint directory: the shard set and one name -> shard map ----------------------------------
+struct DgppCheckpoint {
+  std::vector<DgppSafetensors*> shards;            // in ascending path order
+  std::map<std::string, int, std::less<>> where;   // tensor name -> index into shards
+  ~DgppCheckpoint() {
+    for (DgppSafetensors* f : shards) dgpp_safetensors_close(f, 0);
+  }
+};
+
+int dgpp_checkpoint_open(const char* dir, DgppCheckpoint** out) {
+  namespace fs = std::filesystem;
+  if (!dir || !out) return fail(DGPP_INVALID_ARGUMENT, "checkpoint_open: null argument");
+  *out = nullptr;
+  DgppCheckpoint* ck = nullptr;
+  try {
+    const fs::path root(dir);
+    if (!fs::is_directory(root)) throw std::runtime_error(std::string("checkpoint_open: not a directory: ") + dir);
+    std::vector<fs::path> paths;
+    const fs::path index_path = root / "model.safetensors.index.json";
+    if (fs::exists(index_path)) {
+      // The index's weight_map names the shard set, sub-directories included; a .safetensors file it does not
+      // name is ignored (src/loaders/resident_stream.hpp:259-283).
+      std::ifstream in(index_path, std::ios::binary);
+      if (!in) throw std::runtime_error("checkpoint_open: cannot read shard index " + index_path.string());
+      const std::string text((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+      std::set<std::string> named;
+      bool have_map = false;
+      Scanner s(text);
+      s.expect('{');
+      if (!s.take('}')) {
+        do {
+          const std::string key = s.string();
+          s.expect(':');
+          if (key != "weight_map") {
+            s.skip_value();
+            continue;
+          }
+          have_map = true;
+          s.expect('{');
+          if (!s.take('}')) {
+            do {
+              s.string();
+              s.expect(':');
+              if (s.peek() != '"') throw std::runtime_error("checkpoint_open: a weight_map entry is not a string");
+              named.insert(s.string());
+            } while (s.take(','));
+            s.expect('}');
+          }
+        } while (s.take(','));
+        s.expect('}');
+      }
+      if (!s.at_end()) throw std::runtime_error("checkpoint_open: trailing text after the shard index");
+      if (!have_map) throw std::runtime_error("checkpoint_open: the shard index has no weight_map");
+      for (const std::string& name : named) {
+        const fs::path f = root / name;
+        if (!fs::exists(f))
+          throw std::runtime_error("checkpoint_open: shard '" + name + "' named by the index is missing from " + dir);
+        paths.push_back(f);
+      }
+    } else {
+      for (const auto& entry : fs::directory_iterator(root))
+        if (entry.path().extension() == ".safetensors") paths.push_back(entry.path());
+    }
+    if (paths.empty()) throw std::runtime_error(std::string("checkpoint_open: no .safetensors shards in ") + dir);
+    std::sort(paths.begin(), paths.end());
+    ck = new DgppCheckpoint();
+    for (const fs::path& f : paths) {
+      DgppSafetensors* h = nullptr;
+      if (dgpp_safetensors_open(f.string().c_str(), &h) != DGPP_OK) throw std::runtime_error(g_error);
+      ck->shards.push_back(h);
+      const int at = static_cast<int>(ck->shards.size()) - 1;
+      for (const Tensor& t : h->tensors)
+        if (!ck->where.emplace(t.name, at).second)
+          throw std::runtime_error("checkpoint_open: duplicate tensor '" + t.name + "' in " + f.string());
+    }
+  } catch (const std::exception& e) {
+    const std::string msg = e.what();   // the shards' closes below do not touch it, but keep it safe
+    delete ck;
+    g_error = msg;
+    return DGPP_RUNTIME_ERROR;
+  }
+  *out = ck;
+  return DGPP_OK;
+}
+
+void dgpp_checkpoint_close(DgppCheckpoint* ck) { delete ck; }
+
+int dgpp_checkpoint_shard_count(const DgppCheckpoint* ck) { return ck ? static_cast<int>(ck->shards.size()) : 0; }
+
+const DgppSafetensors* const* dgpp_checkpoint_shards(const DgppCheckpoint* ck) {
+  return ck && !ck->shards.empty() ? ck->shards.data() : nullptr;
+}
+
+const char* dgpp_checkpoint_shard_path(const DgppCheckpoint* ck, int index) {
+  if (!ck || index < 0 || index >= static_cast<int>(ck->shards.size())) return nullptr;
+  return ck->shards[static_cast<size_t>(index)]->path.c_str();
+}
+
+uint64_t dgpp_checkpoint_tensor_count(const DgppCheckpoint* ck) { return ck ? ck->where.size() : 0; }
+
+int dgpp_checkpoint_find(const DgppCheckpoint* ck, const char* name, DgppTensorInfo* out, int* shard_index) {
+  if (!ck || !name || !out) return fail(DGPP_INVALID_ARGUMENT, "checkpoint_find: null argument");
+  const auto it = ck->where.find(std::string_view(name));
+  if (it == ck->where.end()) return fail(DGPP_INVALID_ARGUMENT, std::string("missing tensor '") + name + "'");
+  if (shard_index) *shard_index = it->second;
+  return dgpp_safetensors_find(ck->shards[static_cast<size_t>(it->second)], name, out);
 }

@@ -54,6 +54,13 @@ SIGNATURES = {
     "dgpp_fp4_cols_slice": (_I, [C.POINTER(_lib.Fp4Matrix), C.c_int64, C.c_int64, _P, _P, C.POINTER(_lib.Fp4Matrix)]),
     "dgpp_expert_view_from_quant": (_I, [C.POINTER(QuantMatrix), C.POINTER(_lib.MoeExpertView)]),
     "dgpp_expert_view_from_fp4": (_I, [C.POINTER(_lib.Fp4Matrix), C.POINTER(_lib.MoeExpertView)]),
+    "dgpp_checkpoint_open": (_I, [C.c_char_p, C.POINTER(_P)]),
+    "dgpp_checkpoint_close": (None, [_P]),
+    "dgpp_checkpoint_shard_count": (_I, [_P]),
+    "dgpp_checkpoint_shards": (C.POINTER(_P), [_P]),
+    "dgpp_checkpoint_shard_path": (C.c_char_p, [_P, _I]),
+    "dgpp_checkpoint_tensor_count": (C.c_uint64, [_P]),
+    "dgpp_checkpoint_find": (_I, [_P, C.c_char_p, C.POINTER(TensorInfo), C.POINTER(_I)]),
 }
 _typed = False
 
@@ -135,6 +142,57 @@ class SafetensorsFile:
         a = np.frombuffer(buf, dtype=dt).reshape(info.dims())
         a.flags.writeable = False
         return a
+
+
+class _Shard(SafetensorsFile):
+    """A shard a Checkpoint owns: the same accessors, closed with the checkpoint."""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    def close(self, drop_page_cache: bool = False) -> None:   # the checkpoint closes it
+        self._h = _P()
+
+
+class Checkpoint:
+    """A checkpoint directory as one shard set: the index's weight_map names the shards when there is an index, else
+    every *.safetensors file of the directory. `files` is what the bind functions take."""
+
+    def __init__(self, directory: str):
+        self._h = _P()
+        _check(lib().dgpp_checkpoint_open(str(directory).encode(), C.byref(self._h)))
+        n = lib().dgpp_checkpoint_shard_count(self._h)
+        arr = lib().dgpp_checkpoint_shards(self._h)
+        self.files = [_Shard(_P(arr[i])) for i in range(n)]
+
+    def close(self) -> None:
+        if self._h:
+            for f in self.files:
+                f.close()
+            lib().dgpp_checkpoint_close(self._h)
+            self._h = _P()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def shard_paths(self):
+        return [lib().dgpp_checkpoint_shard_path(self._h, i).decode() for i in range(len(self.files))]
+
+    def tensor_count(self) -> int:
+        return int(lib().dgpp_checkpoint_tensor_count(self._h))
+
+    def find(self, name: str):
+        """(TensorInfo, shard index); ValueError when no shard has the tensor."""
+        info, at = TensorInfo(), _I()
+        _check(lib().dgpp_checkpoint_find(self._h, name.encode(), C.byref(info), C.byref(at)))
+        return info, at.value
+
+    def array(self, name: str) -> np.ndarray:
+        _, at = self.find(name)
+        return self.files[at].array(name)
 
 
 def quant_scale_shifts(m: QuantMatrix):

@@ -170,6 +170,23 @@ int dgpp_qwen_moe_bind_layer(const DgppSafetensors* const* files, int n_files, c
                              DgppTensorInfo* router_weight, DgppTensorInfo* shared_gate, DgppMoeMatrixTensors* shared,
                              DgppMoeMatrixTensors* routed);
 
+/* A checkpoint directory as one set of shards (src/loaders/resident_stream.hpp:257-296). With a
+ * `model.safetensors.index.json` the distinct file names of its "weight_map" are the shard set (relative to the
+ * directory, sub-directories included; a .safetensors file the map does not name is ignored, a named one that is
+ * missing fails the open); without it every *.safetensors file of the directory itself. Shards open in ascending
+ * path order; no shard at all, or a tensor name that two shards carry, fails the open (DGPP_RUNTIME_ERROR, nothing
+ * left mapped). dgpp_checkpoint_shards is the array the bind functions above take; it and every DgppTensorInfo::data
+ * live until the close. */
+typedef struct DgppCheckpoint DgppCheckpoint;
+int dgpp_checkpoint_open(const char* dir, DgppCheckpoint** out);
+void dgpp_checkpoint_close(DgppCheckpoint* ck);
+int dgpp_checkpoint_shard_count(const DgppCheckpoint* ck);
+const DgppSafetensors* const* dgpp_checkpoint_shards(const DgppCheckpoint* ck);
+const char* dgpp_checkpoint_shard_path(const DgppCheckpoint* ck, int index);
+uint64_t dgpp_checkpoint_tensor_count(const DgppCheckpoint* ck);
+/* DGPP_INVALID_ARGUMENT when no shard has the tensor; shard_index (nullable) receives the shard's position. */
+int dgpp_checkpoint_find(const DgppCheckpoint* ck, const char* name, DgppTensorInfo* out, int* shard_index);
+
 #ifdef __cplusplus
 }
 #endif

@@ -5,6 +5,7 @@ shapes, byte-count mismatches and overflows, scalar / empty tensors, dtype alias
 the matrix views' contracts (src/models/quant_matrix.hpp:55-96, :144-164)."""
 import ctypes as C
 import json
+import os
 import struct
 
 import numpy as np
@@ -477,3 +478,70 @@ def test_qwen_moe_block_binding(tmp_path, routed_fmt, shared_fmt):
             LD.qwen_moe_bind_layer([f], p, E, H, I, routed_fmt, S + 64, shared_fmt)
         with pytest.raises(ValueError, match="unknown expert format"):
             LD.qwen_moe_bind_layer([f], p, E, H, I, 9)
+
+
+def test_checkpoint_directory_follows_the_index_when_there_is_one(tmp_path):
+    """The shard set of a checkpoint directory (reference: src/loaders/resident_stream.hpp:257-296): the index's
+    weight_map is authoritative (sub-directories included, files it does not name ignored), else every shard of the
+    directory; a layer binds across the set by name."""
+    rng = np.random.default_rng(23)
+    E, H, I = 3, 256, 128
+    prefix = "model.layers.0."
+    tensors, dtypes = _glm_layer_tensors(prefix, E, H, I, LD.BIND_FP8, 0, rng)
+    names = list(tensors)
+    (tmp_path / "tensors").mkdir()
+    rel = ["model-00002-of-00002.safetensors", "tensors/model-00001-of-00002.safetensors"]
+    for i, r in enumerate(rel):
+        _write_named(str(tmp_path / r), dict((n, tensors[n]) for n in names[i::2]), dtypes)
+    # a stray shard that repeats a tensor: ignored under an index, a duplicate without one
+    _write_named(str(tmp_path / "stray.safetensors"), {names[0]: tensors[names[0]]}, dtypes)
+    index = {"metadata": {"total_size": 1, "nested": {"a": [1, 2, {"b": None}]}},
+             "weight_map": {n: rel[i % 2] for i, n in enumerate(names)}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    with LD.Checkpoint(str(tmp_path)) as ck:
+        assert [os.path.relpath(p, tmp_path) for p in ck.shard_paths()] == sorted(rel)     # ascending path order
+        assert ck.tensor_count() == len(names)
+        for n in names[:7]:
+            info, at = ck.find(n)
+            assert rel[names.index(n) % 2] == os.path.relpath(ck.shard_paths()[at], tmp_path)
+            assert np.array_equal(ck.array(n), np.asarray(tensors[n]))
+        with pytest.raises(ValueError, match="missing tensor 'nope'"):
+            ck.find("nope")
+        rw, rb, shared, routed = LD.glm_moe_bind_layer(ck.files, prefix, E, H, I, LD.BIND_FP8, 0)
+        assert len(routed) == E and shared is None
+        assert routed[2][1].payload.dims() == (I, H)
+    # a shard the index names but the directory lacks
+    index["weight_map"]["extra.weight"] = "model-00003-of-00003.safetensors"
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(LD.LoaderError, match="named by the index is missing"):
+        LD.Checkpoint(str(tmp_path))
+    # an index without a weight_map, and one that is not JSON
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"metadata": {}}))
+    with pytest.raises(LD.LoaderError, match="no weight_map"):
+        LD.Checkpoint(str(tmp_path))
+    (tmp_path / "model.safetensors.index.json").write_text('{"weight_map": {"a": 3}}')
+    with pytest.raises(LD.LoaderError):
+        LD.Checkpoint(str(tmp_path))
+
+
+def test_checkpoint_directory_without_an_index(tmp_path):
+    rng = np.random.default_rng(29)
+    a = rng.integers(0, 255, size=(4, 32), dtype=np.uint8)
+    b = rng.random((3,), dtype=np.float32)
+    with pytest.raises(LD.LoaderError, match="no .safetensors shards"):
+        LD.Checkpoint(str(tmp_path))
+    with pytest.raises(LD.LoaderError, match="not a directory"):
+        LD.Checkpoint(str(tmp_path / "absent"))
+    _write_named(str(tmp_path / "b.safetensors"), {"w.b": b}, {})
+    _write_named(str(tmp_path / "a.safetensors"), {"w.a": a}, {})
+    (tmp_path / "notes.txt").write_text("not a shard")
+    (tmp_path / "sub").mkdir()
+    _write_named(str(tmp_path / "sub" / "c.safetensors"), {"w.a": a}, {})          # only the directory itself is scanned
+    with LD.Checkpoint(str(tmp_path)) as ck:
+        assert [os.path.basename(p) for p in ck.shard_paths()] == ["a.safetensors", "b.safetensors"]
+        assert ck.find("w.a")[1] == 0 and ck.find("w.b")[1] == 1
+        assert np.array_equal(ck.array("w.b"), b)
+    _write_named(str(tmp_path / "c.safetensors"), {"w.a": a}, {})                  # the same name in two shards
+    with pytest.raises(LD.LoaderError, match="duplicate tensor 'w.a'"):
+        LD.Checkpoint(str(tmp_path))
+
