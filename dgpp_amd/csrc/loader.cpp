@@ -737,6 +737,29 @@ int bind_matrix(const DgppSafetensors* const* files, int n_files, const std::str
     if ((rc = find_in(files, n_files, stem + ".weight_scale_2", &out->global, nullptr)) != DGPP_OK) return rc;
     return expect(out->global, stem + ".weight_scale_2", DGPP_DT_F32, {});
   }
+  if (format == DGPP_BIND_NVFP4_COMPRESSED) {
+    if (cols % 16 != 0) return fail(DGPP_INVALID_ARGUMENT, "NVFP4 needs K % 16 == 0: '" + base + "'");
+    if ((rc = find_in(files, n_files, stem + ".weight_packed", &out->payload, &out->file_index)) != DGPP_OK) return rc;
+    if ((rc = expect(out->payload, stem + ".weight_packed", DGPP_DT_U8, {rows, cols / 2})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, stem + ".weight_scale", &out->scales, nullptr)) != DGPP_OK) return rc;
+    if ((rc = expect(out->scales, stem + ".weight_scale", DGPP_DT_F8_E4M3, {rows, cols / 16})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, stem + ".weight_global_scale", &out->global, nullptr)) != DGPP_OK) return rc;
+    return expect(out->global, stem + ".weight_global_scale", DGPP_DT_F32, {});
+  }
+  if (format == DGPP_BIND_MXFP4) {
+    if (cols % 32 != 0) return fail(DGPP_INVALID_ARGUMENT, "MXFP4 needs K % 32 == 0: '" + base + "'");
+    if ((rc = find_in(files, n_files, base, &out->payload, &out->file_index)) != DGPP_OK) return rc;
+    if ((rc = expect(out->payload, base, DGPP_DT_U8, {rows, cols / 2})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, stem + ".weight_scale", &out->scales, nullptr)) != DGPP_OK) return rc;
+    return expect(out->scales, stem + ".weight_scale", DGPP_DT_U8, {rows, cols / 32});
+  }
+  if (format == DGPP_BIND_MXFP8_SCALE_INV) {
+    if (cols % 32 != 0) return fail(DGPP_INVALID_ARGUMENT, "MXFP8 needs K % 32 == 0: '" + base + "'");
+    if ((rc = find_in(files, n_files, base, &out->payload, &out->file_index)) != DGPP_OK) return rc;
+    if ((rc = expect(out->payload, base, DGPP_DT_F8_E4M3, {rows, cols})) != DGPP_OK) return rc;
+    if ((rc = find_in(files, n_files, stem + ".weight_scale_inv", &out->scales, nullptr)) != DGPP_OK) return rc;
+    return expect(out->scales, stem + ".weight_scale_inv", DGPP_DT_U8, {rows, cols / 32});
+  }
   if (format == DGPP_BIND_MXFP8) {
     if (cols % 32 != 0) return fail(DGPP_INVALID_ARGUMENT, "MXFP8 needs K % 32 == 0: '" + base + "'");
     if ((rc = find_in(files, n_files, base, &out->payload, &out->file_index)) != DGPP_OK) return rc;
@@ -819,6 +842,66 @@ extern "C" int dgpp_qwen_moe_bind_layer(const DgppSafetensors* const* files, int
     for (int m = 0; m < 3; ++m) {
       const int64_t rows = m == 2 ? hidden : inter, cols = m == 2 ? inter : hidden;
       if ((rc = bind_matrix(files, n_files, ep + kProj[m], rows, cols, routed_format, routed + static_cast<size_t>(e) * 3 + m)) !=
+          DGPP_OK)
+        return rc;
+    }
+  }
+  return DGPP_OK;
+}
+
+// src/models/mimo/binding.cpp:58-71: router BF16 + F32 bias, routed experts MXFP4, no shared expert.
+extern "C" int dgpp_mimo_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* mlp_prefix, int n_experts,
+                                        int64_t hidden, int64_t inter, DgppTensorInfo* router_weight, DgppTensorInfo* router_bias,
+                                        DgppMoeMatrixTensors* routed) {
+  if (!files || n_files <= 0 || !mlp_prefix || !router_weight || !router_bias || !routed)
+    return fail(DGPP_INVALID_ARGUMENT, "mimo_moe_bind_layer: null argument");
+  if (n_experts <= 0 || hidden <= 0 || inter <= 0) return fail(DGPP_INVALID_ARGUMENT, "mimo_moe_bind_layer: geometry must be positive");
+  const std::string p(mlp_prefix);
+  static const char* const kProj[3] = {"gate_proj.weight", "up_proj.weight", "down_proj.weight"};
+  int rc;
+  if ((rc = find_in(files, n_files, p + "gate.weight", router_weight, nullptr)) != DGPP_OK) return rc;
+  if ((rc = expect(*router_weight, p + "gate.weight", DGPP_DT_BF16, {n_experts, hidden})) != DGPP_OK) return rc;
+  if ((rc = find_in(files, n_files, p + "gate.e_score_correction_bias", router_bias, nullptr)) != DGPP_OK) return rc;
+  if ((rc = expect(*router_bias, p + "gate.e_score_correction_bias", DGPP_DT_F32, {n_experts})) != DGPP_OK) return rc;
+  for (int e = 0; e < n_experts; ++e) {
+    const std::string ep = p + "experts." + std::to_string(e) + ".";
+    for (int m = 0; m < 3; ++m) {
+      const int64_t rows = m == 2 ? hidden : inter, cols = m == 2 ? inter : hidden;
+      if ((rc = bind_matrix(files, n_files, ep + kProj[m], rows, cols, DGPP_BIND_MXFP4, routed + static_cast<size_t>(e) * 3 + m)) !=
+          DGPP_OK)
+        return rc;
+    }
+  }
+  return DGPP_OK;
+}
+
+// src/models/minimax/binding.cpp:15-35, :60-71: F32 router and bias, the shared expert MXFP8 (`weight_scale_inv` bytes),
+// routed experts NVFP4 under w1 (gate), w3 (up), w2 (down).
+extern "C" int dgpp_minimax_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* moe_prefix, int n_experts,
+                                           int64_t hidden, int64_t inter, int64_t shared_inter, DgppTensorInfo* router_weight,
+                                           DgppTensorInfo* router_bias, DgppMoeMatrixTensors* shared, DgppMoeMatrixTensors* routed) {
+  if (!files || n_files <= 0 || !moe_prefix || !router_weight || !router_bias || !routed || (shared_inter > 0 && !shared))
+    return fail(DGPP_INVALID_ARGUMENT, "minimax_moe_bind_layer: null argument");
+  if (n_experts <= 0 || hidden <= 0 || inter <= 0 || shared_inter < 0)
+    return fail(DGPP_INVALID_ARGUMENT, "minimax_moe_bind_layer: geometry must be positive");
+  const std::string p(moe_prefix);
+  static const char* const kProj[3] = {"gate_proj.weight", "up_proj.weight", "down_proj.weight"};
+  static const char* const kW[3] = {"w1.weight", "w3.weight", "w2.weight"};
+  int rc;
+  if ((rc = find_in(files, n_files, p + "gate.weight", router_weight, nullptr)) != DGPP_OK) return rc;
+  if ((rc = expect(*router_weight, p + "gate.weight", DGPP_DT_F32, {n_experts, hidden})) != DGPP_OK) return rc;
+  if ((rc = find_in(files, n_files, p + "e_score_correction_bias", router_bias, nullptr)) != DGPP_OK) return rc;
+  if ((rc = expect(*router_bias, p + "e_score_correction_bias", DGPP_DT_F32, {n_experts})) != DGPP_OK) return rc;
+  for (int m = 0; m < 3 && shared_inter > 0; ++m) {
+    const int64_t rows = m == 2 ? hidden : shared_inter, cols = m == 2 ? shared_inter : hidden;
+    if ((rc = bind_matrix(files, n_files, p + "shared_experts." + kProj[m], rows, cols, DGPP_BIND_MXFP8_SCALE_INV, shared + m)) != DGPP_OK)
+      return rc;
+  }
+  for (int e = 0; e < n_experts; ++e) {
+    const std::string ep = p + "experts." + std::to_string(e) + ".";
+    for (int m = 0; m < 3; ++m) {
+      const int64_t rows = m == 2 ? hidden : inter, cols = m == 2 ? inter : hidden;
+      if ((rc = bind_matrix(files, n_files, ep + kW[m], rows, cols, DGPP_BIND_NVFP4_COMPRESSED, routed + static_cast<size_t>(e) * 3 + m)) !=
           DGPP_OK)
         return rc;
     }

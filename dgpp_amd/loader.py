@@ -251,6 +251,7 @@ def fp4_cols_slice(m, col_start: int, cols: int):
 
 
 BIND_FP8, BIND_NVFP4, BIND_FP8_BF16_SCALES, BIND_NVFP4_MODELOPT, BIND_MXFP8 = 0, 1, 2, 3, 4
+BIND_NVFP4_COMPRESSED, BIND_MXFP4, BIND_MXFP8_SCALE_INV = 5, 6, 7
 
 
 class MoeMatrixTensors(C.Structure):
@@ -297,3 +298,34 @@ def qwen_moe_bind_layer(files, mlp_prefix: str, n_experts: int, hidden: int, int
                                           shared if shared_inter > 0 else None, routed))
     return (rw, sg if shared_inter > 0 else None, list(shared) if shared_inter > 0 else None,
             [[routed[3 * e + m] for m in range(3)] for e in range(n_experts)])
+
+
+SIGNATURES["dgpp_mimo_moe_bind_layer"] = (_I, [C.POINTER(_P), _I, C.c_char_p, _I, C.c_int64, C.c_int64, C.POINTER(TensorInfo),
+                                                C.POINTER(TensorInfo), C.POINTER(MoeMatrixTensors)])
+SIGNATURES["dgpp_minimax_moe_bind_layer"] = (_I, [C.POINTER(_P), _I, C.c_char_p, _I, C.c_int64, C.c_int64, C.c_int64,
+                                                   C.POINTER(TensorInfo), C.POINTER(TensorInfo), C.POINTER(MoeMatrixTensors),
+                                                   C.POINTER(MoeMatrixTensors)])
+
+
+def mimo_moe_bind_layer(files, mlp_prefix: str, n_experts: int, hidden: int, inter: int):
+    """The tensors of one MiMo-family MXFP4 MoE block. Returns (router_weight, router_bias, routed [n_experts][3])."""
+    handles = (_P * len(files))(*[f._h for f in files])
+    rw, rb = TensorInfo(), TensorInfo()
+    routed = (MoeMatrixTensors * (3 * n_experts))()
+    _check(lib().dgpp_mimo_moe_bind_layer(handles, len(files), mlp_prefix.encode(), n_experts, hidden, inter, C.byref(rw),
+                                          C.byref(rb), routed))
+    return rw, rb, [[routed[3 * e + m] for m in range(3)] for e in range(n_experts)]
+
+
+def minimax_moe_bind_layer(files, moe_prefix: str, n_experts: int, hidden: int, inter: int, shared_inter: int = 0):
+    """The tensors of one MiniMax-family MoE block (NVFP4 routed w1 / w3 / w2 as gate / up / down, MXFP8 shared).
+    Returns (router_weight, router_bias, shared [3] or None, routed [n_experts][3])."""
+    handles = (_P * len(files))(*[f._h for f in files])
+    rw, rb = TensorInfo(), TensorInfo()
+    shared = (MoeMatrixTensors * 3)()
+    routed = (MoeMatrixTensors * (3 * n_experts))()
+    _check(lib().dgpp_minimax_moe_bind_layer(handles, len(files), moe_prefix.encode(), n_experts, hidden, inter, shared_inter,
+                                             C.byref(rw), C.byref(rb), shared if shared_inter > 0 else None, routed))
+    return (rw, rb, list(shared) if shared_inter > 0 else None,
+            [[routed[3 * e + m] for m in range(3)] for e in range(n_experts)])
+

@@ -141,7 +141,11 @@ enum {
   DGPP_BIND_FP8_BF16_SCALES = 2,  /* as FP8 with a BF16 grid: widen it to F32 at load (exact) before the launchers see it */
   DGPP_BIND_NVFP4_MODELOPT = 3,   /* `<base>.weight` U8 [rows, cols / 2], `<base>.weight_scale` F8_E4M3 [rows, cols / 16],
                                      `<base>.weight_scale_2` F32 scalar: the kernels' divisor is 1 / weight_scale_2 */
-  DGPP_BIND_MXFP8 = 4             /* `<base>.weight` F8_E4M3, `<base>.weight_scale` U8 (e8m0) [rows, cols / 32] */
+  DGPP_BIND_MXFP8 = 4,            /* `<base>.weight` F8_E4M3, `<base>.weight_scale` U8 (e8m0) [rows, cols / 32] */
+  DGPP_BIND_NVFP4_COMPRESSED = 5, /* `<base>.weight_packed` U8 [rows, cols / 2], `<base>.weight_scale` F8_E4M3 [rows, cols / 16],
+                                     `<base>.weight_global_scale` F32 scalar (the divisor itself) */
+  DGPP_BIND_MXFP4 = 6,            /* `<base>.weight` U8 [rows, cols / 2], `<base>.weight_scale` U8 (e8m0) [rows, cols / 32] */
+  DGPP_BIND_MXFP8_SCALE_INV = 7   /* as MXFP8 with the bytes under `<base>.weight_scale_inv` */
 };
 typedef struct DgppMoeMatrixTensors {
   DgppTensorInfo payload;
@@ -169,6 +173,21 @@ int dgpp_qwen_moe_bind_layer(const DgppSafetensors* const* files, int n_files, c
                              int64_t hidden, int64_t inter, int routed_format, int64_t shared_inter, int shared_format,
                              DgppTensorInfo* router_weight, DgppTensorInfo* shared_gate, DgppMoeMatrixTensors* shared,
                              DgppMoeMatrixTensors* routed);
+
+/* The MXFP4 MoE block of a MiMo-family export (src/models/mimo/binding.cpp:38-42, :58-71); `p` = mlp_prefix:
+ * router `<p>gate.weight` BF16 [E, H] and `<p>gate.e_score_correction_bias` F32 [E]; routed expert e
+ * `<p>experts.<e>.{gate,up,down}_proj` as DGPP_BIND_MXFP4. No shared expert. */
+int dgpp_mimo_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* mlp_prefix, int n_experts,
+                             int64_t hidden, int64_t inter, DgppTensorInfo* router_weight, DgppTensorInfo* router_bias,
+                             DgppMoeMatrixTensors* routed);
+/* The MoE block of a MiniMax-family export (src/models/minimax/binding.cpp:15-35, :60-71); `p` = moe_prefix, e.g.
+ * "language_model.model.layers.3.block_sparse_moe.": router `<p>gate.weight` F32 [E, H] and
+ * `<p>e_score_correction_bias` F32 [E]; with shared_inter > 0 `<p>shared_experts.{gate,up,down}_proj` as
+ * DGPP_BIND_MXFP8_SCALE_INV; routed expert e `<p>experts.<e>.{w1,w3,w2}` (gate, up, down in that order) as
+ * DGPP_BIND_NVFP4_COMPRESSED (the export's `input_global_scale` is not looked up: this path keeps BF16 activations). */
+int dgpp_minimax_moe_bind_layer(const DgppSafetensors* const* files, int n_files, const char* moe_prefix, int n_experts,
+                                int64_t hidden, int64_t inter, int64_t shared_inter, DgppTensorInfo* router_weight,
+                                DgppTensorInfo* router_bias, DgppMoeMatrixTensors* shared, DgppMoeMatrixTensors* routed);
 
 /* A checkpoint directory as one set of shards (src/loaders/resident_stream.hpp:257-296). With a
  * `model.safetensors.index.json` the distinct file names of its "weight_map" are the shard set (relative to the

@@ -545,3 +545,72 @@ def test_checkpoint_directory_without_an_index(tmp_path):
     with pytest.raises(LD.LoaderError, match="duplicate tensor 'w.a'"):
         LD.Checkpoint(str(tmp_path))
 
+
+def test_mimo_and_minimax_moe_block_bindings(tmp_path):
+    """The MXFP4 block of a MiMo-family export (reference: src/models/mimo/binding.cpp:38-71) and the NVFP4 + MXFP8
+    block of a MiniMax-family export (src/models/minimax/binding.cpp:15-71: w1 / w3 / w2 are gate / up / down)."""
+    rng = np.random.default_rng(31)
+    E, H, I, S = 3, 256, 128, 192
+    tensors, dtypes = {}, {}
+
+    def u8(name, shape, dt=None):
+        tensors[name] = rng.integers(0, 120, size=shape, dtype=np.uint8)
+        if dt:
+            dtypes[name] = dt
+
+    p = "model.layers.2.mlp."
+    tensors[p + "gate.weight"] = rng.integers(0, 2 ** 15, size=(E, H), dtype=np.uint16)
+    dtypes[p + "gate.weight"] = "BF16"
+    tensors[p + "gate.e_score_correction_bias"] = rng.random(E, dtype=np.float32)
+    q = "language_model.model.layers.4.block_sparse_moe."
+    tensors[q + "gate.weight"] = rng.random((E, H), dtype=np.float32)
+    tensors[q + "e_score_correction_bias"] = rng.random(E, dtype=np.float32)
+    for proj, (r, c) in (("gate_proj", (S, H)), ("up_proj", (S, H)), ("down_proj", (H, S))):
+        u8(f"{q}shared_experts.{proj}.weight", (r, c), "F8_E4M3")
+        u8(f"{q}shared_experts.{proj}.weight_scale_inv", (r, c // 32))
+    for e in range(E):
+        for proj, (r, c) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            u8(f"{p}experts.{e}.{proj}.weight", (r, c // 2))
+            u8(f"{p}experts.{e}.{proj}.weight_scale", (r, c // 32))
+        for w, (r, c) in (("w1", (I, H)), ("w3", (I, H)), ("w2", (H, I))):
+            u8(f"{q}experts.{e}.{w}.weight_packed", (r, c // 2))
+            u8(f"{q}experts.{e}.{w}.weight_scale", (r, c // 16), "F8_E4M3")
+            tensors[f"{q}experts.{e}.{w}.weight_global_scale"] = np.float32(2688.0 + e)
+            tensors[f"{q}experts.{e}.{w}.input_global_scale"] = np.float32(1.0)
+    path = str(tmp_path / "blocks.safetensors")
+    _write_named(path, tensors, dtypes)
+    with LD.SafetensorsFile(path) as f:
+        rw, rb, routed = LD.mimo_moe_bind_layer([f], p, E, H, I)
+        assert rw.dims() == (E, H) and rw.dtype == LD.DT_BF16 and rb.dims() == (E,)
+        for e in range(E):
+            g, u, d = routed[e]
+            assert [m.format for m in (g, u, d)] == [LD.BIND_MXFP4] * 3
+            assert g.payload.dims() == (I, H // 2) and g.scales.dims() == (I, H // 32) and g.scales.dtype == LD.DT_U8
+            assert d.payload.dims() == (H, I // 2) and d.scales.dims() == (H, I // 32)
+            assert np.array_equal(np.frombuffer((C.c_uint8 * u.payload.nbytes).from_address(u.payload.data), dtype=np.uint8),
+                                  tensors[f"{p}experts.{e}.up_proj.weight"].ravel())
+        with pytest.raises(ValueError, match=r"experts\.0\.gate_proj\.weight' is dtype"):
+            LD.mimo_moe_bind_layer([f], p, E, H, I * 2)
+        with pytest.raises(ValueError, match=r"gate\.weight' is dtype 2 \[3, 256\], expected dtype 2 \[4, 256\]"):
+            LD.mimo_moe_bind_layer([f], p, E + 1, H, I)
+        with pytest.raises(ValueError, match="missing tensor 'model.layers.9"):
+            LD.mimo_moe_bind_layer([f], "model.layers.9.mlp.", E, H, I)
+
+        rw, rb, shared, routed = LD.minimax_moe_bind_layer([f], q, E, H, I, S)
+        assert rw.dims() == (E, H) and rw.dtype == LD.DT_F32 and rb.dims() == (E,)
+        assert [m.format for m in shared] == [LD.BIND_MXFP8_SCALE_INV] * 3
+        assert shared[0].scales.dims() == (S, H // 32) and shared[2].payload.dims() == (H, S)
+        for e in range(E):
+            g, u, d = routed[e]
+            assert g.payload.dims() == (I, H // 2) and g.scales.dims() == (I, H // 16) and g.global_.dims() == ()
+            assert d.payload.dims() == (H, I // 2) and d.scales.dims() == (H, I // 16)
+            # w3 is the up projection, w2 the down projection
+            assert np.array_equal(np.frombuffer((C.c_uint8 * u.payload.nbytes).from_address(u.payload.data), dtype=np.uint8),
+                                  tensors[f"{q}experts.{e}.w3.weight_packed"].ravel())
+            assert np.array_equal(np.frombuffer((C.c_uint8 * d.payload.nbytes).from_address(d.payload.data), dtype=np.uint8),
+                                  tensors[f"{q}experts.{e}.w2.weight_packed"].ravel())
+            assert np.frombuffer((C.c_uint8 * 4).from_address(g.global_.data), dtype=np.float32)[0] == np.float32(2688.0 + e)
+        assert LD.minimax_moe_bind_layer([f], q, E, H, I)[2] is None
+        with pytest.raises(ValueError, match=r"shared_experts\.gate_proj\.weight' is dtype"):
+            LD.minimax_moe_bind_layer([f], q, E, H, I, S + 32)
+
