@@ -195,7 +195,14 @@ def test_layer_bound_by_the_glm_tensor_names_is_bitwise_the_layer_from_the_array
         a = np.frombuffer((C.c_uint8 * info.nbytes).from_address(info.data), dtype=np.uint8)
         return dev(np.array(a))
 
-    files = [LD.SafetensorsFile(q) for q in paths]
+    # the directory opens as one shard set through its index
+    import json
+    import os
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(
+        {"metadata": {}, "weight_map": {n: os.path.basename(paths[i % 2]) for i, n in enumerate(names)}}))
+    ck = LD.Checkpoint(str(tmp_path))
+    files = ck.files
+    assert ck.tensor_count() == len(names) and len(files) == 2
     keep, entries = [], []
     try:
         rw, rb, shared, routed = LD.glm_moe_bind_layer(files, prefix, E, H, I, LD.BIND_FP8 if kind == "fp8" else LD.BIND_NVFP4)
@@ -214,8 +221,7 @@ def test_layer_bound_by_the_glm_tensor_names_is_bitwise_the_layer_from_the_array
                     q = _lib.Fp4Matrix(wd.data_ptr(), sd.data_ptr(), gd.data_ptr(), rows, m.payload.dims()[1] * 2, 16, 0, None)
                     entries.append(LD.expert_view_from_fp4(q))
     finally:
-        for f in files:
-            f.close()
+        ck.close()
     d = DeviceMoe(p)
     ref_layer = make_layer(p, d, 1, 1.0, T)
     d2 = DeviceMoe.__new__(DeviceMoe)
