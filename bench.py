@@ -574,10 +574,75 @@ def main():
         out1 = torch.empty((1, H), dtype=torch.int16, device=dev)
         layers[0].enqueue_decode_scores(xs[0], H, lg_d[0], lg_d[0], out1, 1, None)
         torch.cuda.synchronize()
-        got = hg.bf16_to_f32(out1.cpu().numpy().view(np.uint16)).astype(np.float64)[0]
+        got_bits = out1.cpu().numpy().view(np.uint16)
+        got = hg.bf16_to_f32(got_bits).astype(np.float64)[0]
         ref = raw1[0]
         floor = 0.02 * float(np.sqrt(np.mean(ref ** 2)))
+        # against the unrounded fp64 oracle: the raw figure carries the bf16 output's own rounding (up to 2^-8 = 3.9e-3),
+        # the second one is the error beyond that rounding (the parity tests' measure, bound 2e-3)
         cpu["gpu_vs_cpu_max_rel"] = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+        cpu["gpu_vs_cpu_beyond_bf16_rounding"] = orc.north_star_rel(got_bits[0], ref)
+
+        # ---- the reference's OWN CPU oracle (compiled from its sources into oracle/_ref), where that was built ----
+        # glm_moe_ref_forward at the same layer shape: router GEMV over the hidden row, 8 routed experts and the
+        # shared expert it always runs (here: expert 0's matrices once more), single-threaded, weights dequantised
+        # to double per use. Timed on a few token rows; its output must equal the port's bit for bit.
+        ref_lib = orc.ref()
+        if ref_lib is not None and hasattr(ref_lib, "ref_moe_layer_create"):
+            mat_pay = [3 * I * H // 2 // 3] * 3                      # gate, up, down payload bytes (equal sizes)
+            mat_sc = [I * H // 32] * 3
+            pay = np.empty((nE + 1) * sum(mat_pay), np.uint8)
+            sc = np.empty((nE + 1) * sum(mat_sc), np.uint8)
+            for e in range(nE + 1):
+                src = e % nE                                          # the shared triple = expert 0's matrices
+                po, so = e * sum(mat_pay), e * sum(mat_sc)
+                for m in range(3):
+                    pm = (gu_p[src, m] if m < 2 else dn_p[src]).numpy().ravel()
+                    sm = (gu_s[src, m] if m < 2 else dn_s[src]).numpy().ravel()
+                    pay[po + m * mat_pay[0]: po + (m + 1) * mat_pay[0]] = pm
+                    sc[so + m * mat_sc[0]: so + (m + 1) * mat_sc[0]] = sm
+            gate = hg.normal_bf16(0xD6990200, (nE, H), std=1.0 / 64.0)   # logits = x . gate ~ N(0, 1)
+            ref_layer = ref_lib.ref_moe_layer_create(H, I, nE, K, 1, 1.0, 1, float("inf"), orc.p(gate), None, 32, orc.p(pay),
+                                                     pay.size, orc.p(sc), sc.size, None, 0)
+            if ref_layer:
+                n_ref = 8
+                ref_out = np.empty((1, H), np.uint16)
+                row0 = np.ascontiguousarray(xl[0])
+                t0 = time.time()
+                for r in range(n_ref):
+                    row = np.ascontiguousarray(xl[r % nL])
+                    rc = ref_lib.ref_moe_layer_forward(ref_layer, orc.p(row), 1, orc.p(ref_out))
+                    assert rc == 0, "the reference oracle threw"
+                t_ref = (time.time() - t0) / n_ref
+                # the port on the reference's own routing of row 0 (its router is the reference's, bit for bit: tests)
+                rc = ref_lib.ref_moe_layer_forward(ref_layer, orc.p(row0), 1, orc.p(ref_out))
+                rid, rw, rb = np.empty((1, K), np.int32), np.empty((1, K), np.float32), np.empty((1, nE), np.float64)
+                ref_lib.ref_router(orc.p(row0), orc.p(gate), None, 1, 1, nE, H, K, 1.0, 1, orc.p(rid), orc.p(rw), orc.p(rb))
+                used_r = set(int(v) for v in rid.ravel()) | {0}
+                mats_r, hold_r = [], []
+                for e in range(nE):
+                    for m in range(3):
+                        if e in used_r:
+                            pa = (gu_p[e, m] if m < 2 else dn_p[e]).numpy()
+                            sa = (gu_s[e, m] if m < 2 else dn_s[e]).numpy()
+                            hold_r += [pa, sa]
+                            mats_r.append(orc.make_matrix(1, pa, sa, group=32))
+                        else:
+                            mats_r.append(orc.make_matrix(1, zero8, zero8, group=32))
+                _, port_bits = orc.moe_forward(row0, rid, rw, H, I, I, mats_r, mats_r[0:3], float("inf"), threads=cores)
+                ref_lib.ref_moe_layer_destroy(ref_layer)
+                bytes_ref = (K + 1) * EXPERT_BYTES + nE * H * 2 + 2 * H * 2
+                port = dict(cpu)
+                cpu = {"value": bytes_ref / t_ref / 1e9, "unit": "GB/s", "cores": 1, "kind": "reference",
+                       "sample": f"{n_ref} T=1 passes of the reference's own glm_moe_ref_forward (compiled from its sources: router "
+                                 f"GEMV + 8 routed MXFP4 experts + the shared expert it always runs = {bytes_ref / 1e6:.1f} MB per "
+                                 "pass), one thread as the reference runs it",
+                       "us_per_layer": t_ref * 1e6,
+                       "port_equals_reference_bits": bool(np.array_equal(port_bits, ref_out)),
+                       "gpu_vs_cpu_max_rel": port.pop("gpu_vs_cpu_max_rel"),
+                       "gpu_vs_cpu_beyond_bf16_rounding": port.pop("gpu_vs_cpu_beyond_bf16_rounding"),
+                       "port": port}
+                del pay, sc
 
     sec = main_res.get("us_per_layer", float("nan")) * 1e-6
     line = {

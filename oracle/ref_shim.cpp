@@ -103,4 +103,47 @@ int ref_moe_forward(const uint16_t* hidden, int tokens, int hidden_dim, int inte
   }
 }
 
+// The same oracle with the layer's weights kept between calls (an FP4 layer: the routed matrices then the
+// shared triple), so that a timed pass is the reference's forward alone and not the copy of its weights.
+struct RefLayer {
+  GlmMoeConfig cfg;
+  GlmMoeHostWeights w;
+};
+
+void* ref_moe_layer_create(int hidden_dim, int inter, int experts, int top_k, int mode, float scaling, int norm,
+                           float limit, const uint16_t* router_gate, const float* router_bias, int fp4_group,
+                           const uint8_t* fp4_payloads, int64_t n_fp4_payloads, const uint8_t* fp4_scales,
+                           int64_t n_fp4_scales, const float* fp4_globals, int64_t n_fp4_globals) {
+  try {
+    auto* l = new RefLayer();
+    l->cfg = make_cfg(hidden_dim, inter, experts, top_k, mode, scaling, norm, limit);
+    l->w.router_gate.assign(router_gate, router_gate + static_cast<size_t>(experts) * hidden_dim);
+    if (router_bias) l->w.router_bias.assign(router_bias, router_bias + experts);
+    else l->w.router_bias.assign(static_cast<size_t>(experts), 0.f);
+    l->w.nvfp4 = true;
+    l->w.shared_nvfp4 = true;
+    l->w.fp4_group = fp4_group;
+    l->w.fp4_payloads.assign(fp4_payloads, fp4_payloads + n_fp4_payloads);
+    l->w.fp4_scales.assign(fp4_scales, fp4_scales + n_fp4_scales);
+    if (fp4_globals) l->w.fp4_globals.assign(fp4_globals, fp4_globals + n_fp4_globals);
+    return l;
+  } catch (const std::exception&) {
+    return nullptr;
+  }
+}
+
+int ref_moe_layer_forward(const void* layer, const uint16_t* hidden, int tokens, uint16_t* out) {
+  try {
+    const auto* l = static_cast<const RefLayer*>(layer);
+    std::vector<uint16_t> o;
+    glm_moe_ref_forward(hidden, l->w, l->cfg, tokens, o);
+    std::memcpy(out, o.data(), o.size() * sizeof(uint16_t));
+    return 0;
+  } catch (const std::exception&) {
+    return 1;
+  }
+}
+
+void ref_moe_layer_destroy(void* layer) { delete static_cast<RefLayer*>(layer); }
+
 }  // extern "C"

@@ -64,6 +64,9 @@ _REF_SIG = {
     "ref_router": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P]),
     "ref_moe_forward": (_I, [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _P, _P, _P, _L, _P, _L, _I, _I, _I, _P, _L, _P,
                              _L, _P, _L, _P]),
+    "ref_moe_layer_create": (_P, [_I, _I, _I, _I, _I, _F, _I, _F, _P, _P, _I, _P, _L, _P, _L, _P, _L]),
+    "ref_moe_layer_forward": (_I, [_P, _P, _I, _P]),
+    "ref_moe_layer_destroy": (None, [_P]),
 }
 
 _orc = None
