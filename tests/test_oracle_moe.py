@@ -61,6 +61,30 @@ def test_live_reference_router_and_forward(E, H, I, K, T, kind, shared, mode, sc
     assert np.array_equal(bits, want)
 
 
+def test_live_reference_layer_handle_matches_the_one_shot_call():
+    """The benchmark's CPU baseline keeps the reference oracle's weights between passes (ref_moe_layer_*): same
+    output as the one-shot ref_moe_forward on an FP4 layer with an FP4 shared expert, repeated passes included."""
+    r = orc.ref()
+    if r is None or not hasattr(r, "ref_moe_layer_create"):
+        pytest.skip("oracle/_ref not built (no reference checkout)")
+    E, H, I, K, T = 6, 128, 64, 3, 4
+    p = moe_data.make_problem(E, H, I, K, T, "mxfp4", 555, shared_kind="mxfp4", limit=float("inf"), std=0.05)
+    want = moe_data.ref_forward(p, 1, 1.0, True)
+    mats = [m for e in p.experts for m in e] + p.shared
+    pay = np.ascontiguousarray(np.concatenate([m.payload.ravel() for m in mats]))
+    sc = np.ascontiguousarray(np.concatenate([m.scales.ravel() for m in mats]))
+    layer = r.ref_moe_layer_create(H, I, E, K, 1, 1.0, 1, p.limit, orc.p(p.router_gate), orc.p(p.router_bias), 32, orc.p(pay),
+                                   pay.size, orc.p(sc), sc.size, None, 0)
+    assert layer
+    try:
+        for _ in range(2):
+            out = np.zeros((T, H), np.uint16)
+            assert r.ref_moe_layer_forward(layer, orc.p(p.x), T, orc.p(out)) == 0
+            assert np.array_equal(out, want)
+    finally:
+        r.ref_moe_layer_destroy(layer)
+
+
 def test_router_tie_rule_all_equal_scores():
     """tests/cuda/glm_moe_test.cu:1498-1545: all-equal scores pick ids 0..K-1, weight s/(K*s)*scale."""
     E, K, T = 40, 8, 3
