@@ -261,3 +261,112 @@ def test_fp8_dequant_bridge_is_bit_exact(gpu):
     assert np.array_equal(np.isnan(got), np.isnan(want))
     ok = ~np.isnan(want)
     assert np.array_equal(got[ok], want[ok])
+
+
+def test_fp8_gemv_multi_is_bitwise_the_single_launches(gpu):
+    """launch_scale_gemv_multi_bf16 (reference: src/kernels/scale_gemm.hpp:88-107, its test
+    scale_gemm_gemv_multi_is_bitwise_the_single_launches): up to four [n_i, k] matrices against the same rows, every
+    out_i bitwise the single launcher's for its problem, for every row count the form takes (1 .. 8)."""
+    from dgpp_amd import _lib
+    k = 1024
+    geo = [(264, 7, 7, 0), (100, 5, 5, 128), (520, 6, 7, 0), (48, 0, 5, 64)]     # n, rs, cs, out_stride (0: n)
+    mats = []
+    for i, (n, rs, cs, _) in enumerate(geo):
+        w = hg.f32_to_bf16(hg.normal_f32(0x3A00 + i, (n, k), 0.02))
+        payload, scales = hg.encode_fp8_blocks(w, 1 << rs, 1 << cs)
+        mats.append((dev(payload), dev(scales)))
+    assert L.fp8_gemv_can_stage(mats[0][0], k) and not L.fp8_gemv_can_stage(mats[0][0], k + 8)
+    for rows in (1, 3, 4, 5, 8):
+        act = dev(hg.normal_bf16(0x3B00 + rows, (rows, k + 16)))                 # rows strided by k + 16 elements
+        outs, singles, problems = [], [], []
+        for (n, rs, cs, stride), (p_d, s_d) in zip(geo, mats):
+            o = dev_empty((rows, stride or n), np.uint16)
+            o.zero_()
+            outs.append(o)
+            problems.append(_lib.Fp8GemvProblem(p_d.data_ptr(), s_d.data_ptr(), o.data_ptr(), n, 0, stride, rs, cs, None))
+            one = dev_empty((rows, n), np.uint16)
+            L.launch_scale_gemm_grid_bf16(act, k + 16, p_d, s_d, one, rows, n, k, None, 0, rs, cs)
+            singles.append(one)
+        L.launch_scale_gemv_multi_bf16(problems, act, k + 16, rows, k)
+        sync()
+        for (n, _, _, stride), o, one in zip(geo, outs, singles):
+            got = host(o, np.uint16)
+            assert np.array_equal(got[:, :n], host(one, np.uint16)), f"rows {rows}, n {n}"
+            assert not got[:, n:].any(), "columns past n stay untouched"
+    with pytest.raises(L.InvalidArgument):
+        L.launch_scale_gemv_multi_bf16(problems + problems[:1], act, k + 16, 8, k)        # five problems
+    with pytest.raises(L.InvalidArgument):
+        L.launch_scale_gemv_multi_bf16(problems, act, k + 16, 9, k)                       # nine rows
+    bad = _lib.Fp8GemvProblem(mats[0][0].data_ptr(), mats[0][1].data_ptr(), outs[0].data_ptr(), 264, 0, 0, 7, 7,
+                              mats[0][0].data_ptr())
+    with pytest.raises(L.InvalidArgument):
+        L.launch_scale_gemv_multi_bf16([bad], act, k + 16, 1, k)                          # a bf16-weight problem
+
+
+def test_fp8_saturation_extremes(gpu):
+    """The reference's scale_gemm_saturation_extremes (tests/cuda/scale_gemm_test.cu:501-532): all-maximum payloads
+    (0x7E = 448) with scales of 1e30 (products near 1e35 stay finite in bf16 and fp32), and the minimum subnormal
+    (0x01 = 2^-9) with scales of 2^-20: both ends of the exponent range against both oracles."""
+    m, n, k = 8, 256, 256
+    for code, scale, seed, label in ((0x7E, 1e30, 0xD4, "448 x 1e30"), (0x01, 2.0 ** -20, 0xD5, "subnormal minimum")):
+        payload = np.full((n, k), code, np.uint8)
+        scales = np.full((2, 2), scale, np.float32)
+        act = hg.normal_bf16(seed, (m, k))
+        out = dev_empty((m, n), np.uint16)
+        L.launch_scale_gemm_bf16(dev(act), k, dev(payload), dev(scales), out, m, n, k, None)
+        sync()
+        got = host(out, np.uint16)
+        assert np.isfinite(hg.bf16_to_f32(got)).all(), label
+        check(got, orc.gemv_fp8(act, payload, scales, m, n, k, 7, 7, strict=True), label)
+        sem = orc.gemv_fp8(act, payload, scales, m, n, k, 7, 7, strict=False)
+        assert orc.compare_bf16(got, sem, 8.0, 2e-2).mismatches == 0, label
+
+
+def test_fp8_gemv_decodes_every_code_as_the_bridge_does(gpu):
+    """The reference's fp8_gemv_hardware_conversion_matches_bridge_on_every_code: a one-hot activation reads single
+    weights back through the GEMV; for every e4m3 code and a spread of block scales the value is the dequant
+    bridge's bf16(decode * scale), bit for bit (NaN codes give NaN)."""
+    n, k = 256, 256
+    payload = np.tile(np.arange(256, dtype=np.uint8)[:, None], (1, k))          # row r holds code r everywhere
+    rng = np.random.default_rng(5)
+    scales = np.exp2(rng.uniform(-18, 8, (2, 2))).astype(np.float32)
+    bridge = dev_empty((n, k), np.uint16)
+    L.launch_fp8_dequant_blocks(dev(payload), dev(scales), bridge, n, k, None)
+    cols = [3, 200]                                                             # one column in each scale block
+    act = np.zeros((len(cols), k), np.uint16)
+    for i, c in enumerate(cols):
+        act[i, c] = 0x3F80                                                      # 1.0
+    out = dev_empty((len(cols), n), np.float32)
+    L.launch_scale_gemm_f32(dev(act), k, dev(payload), dev(scales), out, len(cols), n, k, None)
+    sync()
+    got, want = host(out), hg.bf16_to_f32(host(bridge, np.uint16))
+    for i, c in enumerate(cols):
+        # a NaN weight times the zeros of the other columns poisons its whole row either way: rows 0x7F and 0xFF are NaN
+        nan = np.isnan(want[:, c])
+        assert np.array_equal(np.isnan(got[i]), nan) and nan.sum() == 2
+        # values, not bit patterns: code 0x80 (-0) leaves the dot's accumulator at +0 (0 + -0 * 1), as fmaf does
+        assert np.array_equal(got[i][~nan], want[:, c][~nan]), f"column {c}"
+        assert np.count_nonzero(got[i][~nan]) == 252                              # every code but the two zeros
+
+
+def test_e8m0_grid_is_bitwise_the_f32_grid_of_the_same_powers_of_two(gpu):
+    """The reference's mma_gemv_fp8_e8m0_grid_is_bitwise_the_f32_grid, for the GEMV launchers and the matrix-core
+    launchers: an E8M0 byte grid and the F32 grid holding 2^(b - 127) describe the same weights, and every product
+    e4m3 * 2^e is exact in bf16, so the two launchers give the same bits."""
+    m, n, k = 5, 200, 1024
+    w = hg.normal_f32(0xE80, (n, k), 0.02)
+    payload, bytes_ = hg.encode_mxfp8(w)
+    bytes_ = np.ascontiguousarray(bytes_)
+    f32 = np.exp2(bytes_.astype(np.float64) - 127.0).astype(np.float32)
+    act = dev(hg.normal_bf16(0xE81, (m, k)))
+    p_d, b_d, f_d = dev(payload), dev(bytes_), dev(f32)
+    a, b = dev_empty((m, n), np.uint16), dev_empty((m, n), np.uint16)
+    L.launch_scale_gemm_grid_e8m0_bf16(act, k, p_d, b_d, a, m, n, k, None, 0, 0, 5)
+    L.launch_scale_gemm_grid_bf16(act, k, p_d, f_d, b, m, n, k, None, 0, 0, 5)
+    sync()
+    assert np.array_equal(host(a, np.uint16), host(b, np.uint16)), "GEMV launchers"
+    a2, b2 = dev_empty((m, n), np.float32), dev_empty((m, n), np.float32)
+    L.launch_mma_gemv_fp8e8m0_f32(act, k, p_d, b_d, a2, m, n, k, 0, 0, 5, None)
+    L.launch_mma_gemv_fp8_f32(act, k, p_d, f_d, b2, m, n, k, 0, 0, 5, None)
+    sync()
+    assert np.array_equal(host(a2).view(np.uint32), host(b2).view(np.uint32)), "matrix-core launchers"
