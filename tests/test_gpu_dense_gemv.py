@@ -370,3 +370,25 @@ def test_e8m0_grid_is_bitwise_the_f32_grid_of_the_same_powers_of_two(gpu):
     L.launch_mma_gemv_fp8_f32(act, k, p_d, f_d, b2, m, n, k, 0, 0, 5, None)
     sync()
     assert np.array_equal(host(a2).view(np.uint32), host(b2).view(np.uint32)), "matrix-core launchers"
+
+
+def test_fp8_dequant_bridge_e8m0_is_bit_exact(gpu):
+    """The bridge over an E8M0 byte grid (reference: src/kernels/fp8_dequant.cu:28-31, :79-83): every e4m3 code under
+    block bytes across the range that keeps the products inside bf16's normal range, plus bytes 0 and 255:
+    bf16(decode * 2^(b - 127)) bit for bit, NaN where the code or the byte says so."""
+    rows, cols = 64, 256
+    payload = np.tile(np.arange(256, dtype=np.uint8), (rows, 1))
+    rng = np.random.default_rng(9)
+    scales = rng.integers(20, 240, (rows, cols // 32), dtype=np.uint8)
+    scales[0, 0], scales[1, 1], scales[2, 2] = 0, 255, 254
+    want = np.empty((rows, cols), np.float64)
+    orc.oracle().orc_dequant_fp8(orc.p(payload), None, orc.p(scales), rows, cols, 0, 5, 1, orc.p(want))
+    out = dev_empty((rows, cols), np.uint16)
+    L.launch_fp8_dequant_blocks_e8m0(dev(payload), dev(scales), out, rows, cols, None, 0, 5)
+    sync()
+    got = hg.bf16_to_f32(host(out, np.uint16)).astype(np.float64)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok], want[ok])
+    with pytest.raises(L.InvalidArgument):
+        L.launch_fp8_dequant_blocks_e8m0(dev(payload), dev(scales), out, rows, cols, None, 0, 3)

@@ -35,9 +35,12 @@ def test_dense_mma_fp4_matches_oracle_and_rows_are_independent(gpu, group, m, n,
     outs = dev_empty((m, n + 8), np.uint16)
     ws = dev_empty(4 * m * n, np.float32)
     L.launch_mma_gemv_fp4_bf16(act_d, k, w, outs, m, n, k, n + 8, None, ws, 4 * m * n * 4)
+    outsf = dev_empty((m, n + 8), np.float32)
+    L.launch_mma_gemv_fp4_f32(act_d, k, w, outsf, m, n, k, n + 8, None, ws, 4 * m * n * 4)
     sync()
     got = host(out, np.uint16)
     assert np.array_equal(host(outs, np.uint16)[:, :n], got), "the split form's bits are the unsplit form's"
+    assert np.array_equal(hg.f32_to_bf16(host(outsf)[:, :n]), got), "the split form's unrounded output rounds to the same bits"
     check(got, raw, f"dense mma fp4 g{group} {m}x{n}x{k}")
     assert np.array_equal(hg.f32_to_bf16(host(outf)), got), "bf16(out_f32) == out_bf16"
     assert np.array_equal(host(one, np.uint16)[0], got[m - 1]), "a row's bits do not depend on the rows beside it"
@@ -76,10 +79,12 @@ def test_mma_gemv_fp8_matches_oracle_split_and_unsplit(gpu, e8m0, rs, cs, m, n, 
     assert np.array_equal(hg.f32_to_bf16(host(outf)), got)
     assert np.array_equal(host(outs, np.uint16), got), "the split form's bits are the unsplit form's"
     if not e8m0 and rs == 7 and cs == 7:
-        outd = dev_empty((m, n), np.uint16)
+        outd, outdf = dev_empty((m, n), np.uint16), dev_empty((m, n), np.float32)
         L.launch_dense_mma_bf16(a_d, k, p_d, s_d, outd, m, n, k, None)
+        L.launch_dense_mma_f32(a_d, k, p_d, s_d, outdf, m, n, k, None)
         sync()
         assert np.array_equal(host(outd, np.uint16), got)
+        assert np.array_equal(hg.f32_to_bf16(host(outdf)), got)
 
 
 @pytest.mark.parametrize("kind", ["fp8", "nvfp4", "mxfp4"])
