@@ -89,3 +89,19 @@ def test_headers_compile_as_c_and_the_shim_as_cpp(tmp_path):
     subprocess.run(["g++", "-std=c++17", "-Wall", "-I", str(inc), "-I", str(rocm_inc), "-D__HIP_PLATFORM_AMD__",
                     str(cpp_src), "-L", str(root / "dgpp_amd" / "lib"), "-ldgpp_amd", "-L/opt/rocm/lib", "-lamdhip64",
                     "-o", str(tmp_path / "shim_check")], check=True)
+
+
+def test_layer_scratch_bytes_covers_what_the_layer_stages():
+    """dgpp_moe_layer_scratch_bytes (reference: GlmMoeLayer::scratch_bytes, src/models/glm/moe_layer.cpp:72-129) is a
+    host computation: at least the expert table, the slot activations and the unrounded slot outputs, and it grows
+    with the token count and with a shared expert."""
+    from dgpp_amd import launch as L, moe_layer as ML
+    E, H, I, K = 256, 4096, 1024, 8
+    cfg = L.make_config(H, I, E, K, n_shared_experts=0, router_mode=L.ROUTER_SOFTMAX_TOPK)
+    sizes = [ML.scratch_bytes(cfg, t) for t in (1, 8, 64)]
+    assert sizes[0] < sizes[1] < sizes[2]
+    for t, s in zip((1, 8, 64), sizes):
+        floor = E * 3 * 96 + t * (K + 1) * I * 2 + t * (K + 1) * H * 4 + t * K * 8
+        assert floor <= s < 64 * floor
+    cfg_sh = L.make_config(H, I, E, K, n_shared_experts=1, router_mode=L.ROUTER_SOFTMAX_TOPK)
+    assert ML.scratch_bytes(cfg_sh, 8, 2048) > ML.scratch_bytes(cfg_sh, 8, 1024) >= sizes[1]
