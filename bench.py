@@ -53,7 +53,7 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5,w8a8,qwen_tail ('' for none; default: c1,c2,c4,c5, none under --tune)")
+                    "separated out of c1,c2,c4,c5,w8a8,qwen_tail,slotbench ('' for none; default: c1,c2,c4,c5, none under --tune)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -445,6 +445,90 @@ def main():
         lay.close()
         return res
 
+    def bench_slotbench():
+        """The reference's own micro-benchmark of this path (benchmarks/micro/moe_slot_bench.cu: the whole decode chain
+        - router dots, selection, gate/up + SwiGLU, down, accumulation - at its per-rank production geometry: 288
+        experts, top-8 sigmoid-bias routing, hidden 4096, expert slice 512, one block-FP8 shared expert; 1, 2 and 8
+        rows; routed experts NVFP4 or block FP8), timed here on the MI355X beside the figures it publishes for a
+        GB10 (docs/nvfp4_plan.md:299-300, docs/measurements.md:485-488). Not one of BASELINE's configurations: run with
+        --configs slotbench. Cold: 16 input row sets route to different experts, two copies of the routed weights
+        alternate and every step has its own copy of the shared expert."""
+        bE, bH, bI, bK, G, NX = 288, 4096, 512, 8, 8, 16
+        published = {"nvfp4": {1: 209.0, 2: 334.0, 8: 929.0}, "fp8": {1: 273.0, 2: 469.0, 8: 1420.0}}
+        gate = torch.from_numpy(hg.normal_bf16(0xD6996000, (bE, bH), 1.0 / 64.0).view(np.int16)).to(dev)
+        bias = torch.from_numpy(hg.normal_f32(0xD6996001, (bE,), 0.05)).to(dev)
+        shared = []
+        for c in range(NX):
+            tri = []
+            for mi, (r, cc) in enumerate(((bI, bH), (bI, bH), (bH, bI))):
+                if c == 0:
+                    pw, sw = hg.encode_fp8_blocks(hg.f32_to_bf16(hg.normal_f32(0xD6996100 + mi, (r, cc), 0.02)), 128, 128)
+                    tri.append((torch.from_numpy(pw).to(dev), torch.from_numpy(sw).to(dev)))
+                else:
+                    tri.append((shared[0][mi][0].clone(), shared[0][mi][1].clone()))
+            shared.append(tri)
+        cfgb = L.make_config(bH, bI, bE, bK, n_shared_experts=1, routed_scaling_factor=2.5, swiglu_limit=float("inf"),
+                             router_mode=L.ROUTER_SIGMOID_BIAS)
+        res = {"workload": "the reference's moe_slot_bench geometry: 288 experts, top-8 sigmoid-bias router from the hidden rows, "
+                           "hidden 4096, expert slice 512, one block-FP8 shared expert; whole decode chain (enqueue_decode), cold"}
+        for fmt in ("nvfp4", "fp8"):
+            gen = []
+            for g in range(G):
+                mats = []
+                for mi, (r, cc) in enumerate(((bI, bH), (bI, bH), (bH, bI))):
+                    wf = hg.normal_f32(0xD6996200 + g * 3 + mi, (r, cc), 0.02)
+                    if fmt == "nvfp4":
+                        pw, sw, ws2 = hg.encode_nvfp4(wf)
+                        mats.append((torch.from_numpy(pw).to(dev), torch.from_numpy(sw).to(dev),
+                                     torch.tensor([1.0 / np.float32(ws2)], dtype=torch.float32, device=dev)))
+                    else:
+                        pw, sw = hg.encode_fp8_blocks(hg.f32_to_bf16(wf), 128, 128)
+                        mats.append((torch.from_numpy(pw).to(dev), torch.from_numpy(sw).to(dev), None))
+                gen.append(mats)
+            keep, tables = [], []
+            for copy in range(2):
+                views = []
+                for e in range(bE):
+                    for pw, sw, gl in gen[e % G]:
+                        pc, sc_ = pw.clone(), sw.clone()
+                        keep += [pc, sc_]
+                        v = L.MoeExpertView()
+                        v.payload = pc.data_ptr()
+                        if fmt == "nvfp4":
+                            v.fp4_scales, v.fp4_global = sc_.data_ptr(), gl.data_ptr()
+                        else:
+                            v.scales = sc_.data_ptr()
+                        v.scale_shift_rows = v.scale_shift_cols = 7
+                        v.fp4_group = 16
+                        views.append(v)
+                tables.append(views)
+            per_expert = (3 * bI * bH // 2 + 3 * bI * bH // 16 + 12) if fmt == "nvfp4" else (3 * bI * bH + 3 * (bI // 128) * (bH // 128) * 4)
+            shared_bytes = 3 * bI * bH + 3 * (bI // 128) * (bH // 128) * 4
+            for rows in (1, 2, 8):
+                lay = [ML.MoeLayer(cfgb, ML.EXPERTS_NVFP4 if fmt == "nvfp4" else ML.EXPERTS_FP8, tables[c % 2], rows,
+                                   shared_inter=bI, sh_payload=[t[0] for t in shared[c]], sh_scales=[t[1] for t in shared[c]],
+                                   router_gate=gate, router_bias=bias) for c in range(NX)]
+                x = torch.from_numpy(hg.normal_bf16(0xD6996300 + rows, (NX, rows, bH)).view(np.int16)).to(dev)
+                out = torch.empty((NX, rows, bH), dtype=torch.int16, device=dev)
+
+                def step(i):
+                    c = i % NX
+                    lay[c].enqueue_decode(x[c], bH, out[c], rows, stream)
+                sec = time_graph(step, args.steps, args.warmup)
+                # the reference's accounting: rows * (top_k experts + the shared one), no expert sharing
+                slot_bytes = rows * (bK * per_expert + shared_bytes)
+                res[f"{fmt}_rows{rows}"] = {
+                    "us": sec * 1e6,
+                    "reference_published_us_on_gb10": published[fmt][rows],
+                    "slot_bytes_no_expert_sharing": slot_bytes,
+                    "slot_gbps": slot_bytes / sec / 1e9,
+                    "frac_of_peak": slot_bytes / sec / 1e9 / HBM_PEAK_GBPS}
+                for l_ in lay:
+                    l_.close()
+            del keep, tables, gen
+            torch.cuda.empty_cache()
+        return res
+
     def bench_w8a8():
         """The activation-quantized MXFP8 GEMM at the C5 shared expert's projection shapes, swept over the row count
         (not one of the headline benchmark's configurations: run with --configs w8a8). Weights rotate so that no launch finds them cached."""
@@ -523,7 +607,8 @@ def main():
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
-            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail}[name]()
+            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail,
+                                   "slotbench": bench_slotbench}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
 
