@@ -501,6 +501,19 @@ int dgpp_launch_moe_slot_accum_routed_bf16(uint16_t* out, const float* contrib, 
                 "moe_slot_accum_routed_bf16");
 }
 
+namespace {
+// Which passes the next decode-slot launcher call of this thread runs (dgpp_moe_slot_passes): bit 0 the routed
+// slots, bit 1 the shared slots. One call consumes the setting.
+thread_local int g_slot_passes = 3;
+int take_slot_passes() {
+  const int p = g_slot_passes;
+  g_slot_passes = 3;
+  return p;
+}
+}  // namespace
+
+void dgpp_moe_slot_passes(int passes) { g_slot_passes = (passes & 3) ? (passes & 3) : 3; }
+
 int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
                                         const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
                                         int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
@@ -508,6 +521,7 @@ int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, cons
                                         int act_stride, int slots, int top_k, float limit, void* stream, int sh_rs,
                                         int sh_cs) {
   const char* who = "moe_slot_gate_up";
+  const int passes = take_slot_passes();
   if (slots <= 0) return DGPP_OK;
   int rc = check_slot_common(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, who);
   if (rc != DGPP_OK) return rc;
@@ -521,8 +535,8 @@ int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, cons
   a.n = n_routed;
   a.k = k_routed;
   a.want_shared = 0;
-  rc = finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who);
-  if (rc != DGPP_OK || n_shared == 0) return rc;
+  rc = (passes & 1) ? finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who) : DGPP_OK;
+  if (rc != DGPP_OK || n_shared == 0 || !(passes & 2)) return rc;
   a.n = n_shared;
   a.k = k_shared;
   a.want_shared = 1;
@@ -607,6 +621,7 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
                               const uint8_t* sh_payload, const float* sh_scales, float* out, int out_stride, int slots,
                               int top_k, void* stream, int sh_rs, int sh_cs) {
   const char* who = "moe_slot_down";
+  const int passes = take_slot_passes();
   if (slots <= 0) return DGPP_OK;
   int rc = check_slot_common(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, who);
   if (rc != DGPP_OK) return rc;
@@ -619,8 +634,8 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
   a.n = n_routed;
   a.k = k_routed;
   a.want_shared = 0;
-  rc = finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
-  if (rc != DGPP_OK || n_shared == 0) return rc;
+  rc = (passes & 1) ? finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who) : DGPP_OK;
+  if (rc != DGPP_OK || n_shared == 0 || !(passes & 2)) return rc;
   a.n = n_shared;
   a.k = k_shared;
   a.want_shared = 1;
@@ -636,6 +651,7 @@ int dgpp_launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_stride, 
                                             int top_k, float limit, void* stream, int shared_view_base, int fp4_group,
                                             int sh_rs, int sh_cs) {
   const char* who = "moe_slot_gate_up_fp4";
+  const int passes = take_slot_passes();
   if (slots <= 0) return DGPP_OK;
   int rc = check_fp4_slot(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
   if (rc != DGPP_OK) return rc;
@@ -650,8 +666,8 @@ int dgpp_launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_stride, 
   a.n = n_routed;
   a.k = k_routed;
   a.want_shared = 0;
-  rc = finish(launch_slot_gate_up(fmt, a, as_stream(stream)), who);
-  if (rc != DGPP_OK || n_shared == 0) return rc;
+  rc = (passes & 1) ? finish(launch_slot_gate_up(fmt, a, as_stream(stream)), who) : DGPP_OK;
+  if (rc != DGPP_OK || n_shared == 0 || !(passes & 2)) return rc;
   a.n = n_shared;
   a.k = k_shared;
   a.want_shared = 1;
@@ -670,6 +686,7 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
                                   int out_stride, int slots, int top_k, void* stream, int shared_view_base,
                                   int fp4_group, int sh_rs, int sh_cs, int* tile_counter) {
   const char* who = "moe_slot_down_fp4";
+  const int passes = take_slot_passes();
   if (slots <= 0) return DGPP_OK;
   if (tile_counter == nullptr) return fail_arg(std::string(who) + ": the stealing counter pair is required");
   int rc = check_fp4_slot(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
@@ -683,8 +700,8 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
   a.n = n_routed;
   a.k = k_routed;
   a.want_shared = 0;
-  rc = finish(launch_slot_down(fmt, a, as_stream(stream)), who);
-  if (rc != DGPP_OK || n_shared == 0) return rc;
+  rc = (passes & 1) ? finish(launch_slot_down(fmt, a, as_stream(stream)), who) : DGPP_OK;
+  if (rc != DGPP_OK || n_shared == 0 || !(passes & 2)) return rc;
   a.n = n_shared;
   a.k = k_shared;
   a.want_shared = 1;

@@ -121,9 +121,17 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   hip_ok(hipMemcpy(d_views_, w.views.data(), w.views.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
          "GlmMoeLayer: table upload");
   hip_ok(hipMemset(d_tile_counter_, 0, 2 * sizeof(int)), "GlmMoeLayer: counter");
+  if (has_shared()) {
+    hip_ok(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking), "GlmMoeLayer: side stream");
+    hip_ok(hipEventCreateWithFlags(&fork_, hipEventDisableTiming), "GlmMoeLayer: event");
+    hip_ok(hipEventCreateWithFlags(&join_, hipEventDisableTiming), "GlmMoeLayer: event");
+  }
 }
 
 GlmMoeLayer::~GlmMoeLayer() {
+  if (join_) (void)hipEventDestroy(join_);
+  if (fork_) (void)hipEventDestroy(fork_);
+  if (side_) (void)hipStreamDestroy(side_);
   if (arena_) (void)hipFree(arena_);
 }
 
@@ -193,41 +201,69 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   // With scores given, ids / weights are this layer's own buffers and the gate/up launch fills them.
   const bool fused = sel_scores != nullptr && ids == d_ids_ && weights == d_weights_ && order == nullptr && !has_shared();
   if (sel_scores != nullptr && !fused) throw std::logic_error("GlmMoeLayer: fused selection outside its form");
+  // The shared expert's gate/up and down passes read nothing the routed passes write (disjoint slot rows): they run
+  // on the side stream beside them, forked here and joined before the accumulation. One launcher call per pass.
+  // From a few tokens on: the two cross-stream dependencies cost more than the two hand-overs they take off the
+  // chain while a pass is only a few microseconds long (measured: slower at one token, level at two).
+  const bool split = has_shared() && side_ != nullptr && dgpp_tune_get(9) != 1 && (tokens >= 3 || dgpp_tune_get(9) == 2);
+  if (split) {
+    hip_ok(hipEventRecord(fork_, stream), "GlmMoeLayer: fork");
+    hip_ok(hipStreamWaitEvent(side_, fork_, 0), "GlmMoeLayer: fork");
+  }
+  auto for_passes = [&](auto&& call) {
+    if (!split) return call(stream);
+    moe_slot_passes(1);
+    call(stream);
+    moe_slot_passes(2);
+    call(side_);
+  };
   if (w_.format == GlmExpertFormat::Fp8) {
     if (fused)
       launch_moe_select_gate_up_swiglu(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
                                        d_slot_act_, max_inter_, cfg_.swiglu_limit, stream);
     else
-      launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
-                                     w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
-                                     K, cfg_.swiglu_limit, stream, w_.sh_rs, w_.sh_cs);
+      for_passes([&](hipStream_t st) {
+        launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
+                                       w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
+                                       K, cfg_.swiglu_limit, st, w_.sh_rs, w_.sh_cs);
+      });
     if (token_major) {   // routed only: down + accumulation in one token-major launch
       launch_moe_slot_down_accum(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                  out_bf16, out_f32, stream);
       return;
     }
-    launch_moe_slot_down(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
-                         n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, stream, w_.sh_rs, w_.sh_cs);
+    for_passes([&](hipStream_t st) {
+      launch_moe_slot_down(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
+                           n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, st, w_.sh_rs, w_.sh_cs);
+    });
   } else {
     const int base = w_.shared_in_table ? cfg_.n_experts * 3 : -1;
     if (fused)
       launch_moe_select_gate_up_swiglu_fp4(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I,
                                            H, d_slot_act_, max_inter_, cfg_.swiglu_limit, stream, fp4_group_);
     else
-      launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
-                                         sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
-                                         sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
-                                         d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, stream, base, fp4_group_,
-                                         w_.sh_rs, w_.sh_cs);
+      for_passes([&](hipStream_t st) {
+        launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
+                                           sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
+                                           sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
+                                           d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, st, base, fp4_group_,
+                                           w_.sh_rs, w_.sh_cs);
+      });
     if (token_major) {
       launch_moe_slot_down_accum_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                      out_bf16, out_f32, stream, fp4_group_);
       return;
     }
-    launch_moe_slot_down_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
-                             has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
-                             sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, stream, base, fp4_group_,
-                             w_.sh_rs, w_.sh_cs, d_tile_counter_);
+    for_passes([&](hipStream_t st) {
+      launch_moe_slot_down_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
+                               has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
+                               sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, st, base, fp4_group_,
+                               w_.sh_rs, w_.sh_cs, d_tile_counter_);
+    });
+  }
+  if (split) {
+    hip_ok(hipEventRecord(join_, side_), "GlmMoeLayer: join");
+    hip_ok(hipStreamWaitEvent(stream, join_, 0), "GlmMoeLayer: join");
   }
   if (has_shared()) {
     if (out_f32) {

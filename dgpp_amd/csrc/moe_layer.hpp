@@ -81,6 +81,10 @@ class GlmMoeLayer {
   float* d_slot_down_ = nullptr;     // [slots, hidden]
   float* d_acc_ = nullptr;           // [tokens, hidden]
   int* d_tile_counter_ = nullptr;    // [2]
+  // The shared expert's passes run beside the routed ones: a second stream of the default priority, forked from
+  // and joined to the caller's stream with two events (created only for a layer with a shared expert).
+  hipStream_t side_ = nullptr;
+  hipEvent_t fork_ = nullptr, join_ = nullptr;
   int32_t* d_rows_ = nullptr;        // grouped path
   int32_t* d_slot_row_ = nullptr;
   MoeSegment* d_segs_ = nullptr;

@@ -46,7 +46,10 @@ const char* dgpp_target_arch(void);
  * matrix-core form; key 6: 1 makes the layer driver compute the slot order for small decode batches too
  * (default: batches of at most 128 routed slots find the sharers of an expert by ballot, no order);
  * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
- * blocks, dgpp_launch_moe_select_gate_up_swiglu). Outputs do not depend on keys 1 - 4, 6 and 7; keys 0 and
+ * blocks, dgpp_launch_moe_select_gate_up_swiglu); key 9: 1 keeps the shared expert's passes of the layer driver
+ * on the caller's stream, 2 moves them to a second stream beside the routed passes at every batch size (default:
+ * from three tokens on). Outputs do not depend on keys
+ * 1 - 4, 6, 7 and 9; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
  * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);
@@ -210,6 +213,13 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
                               int k_routed, int n_shared, int k_shared, const uint8_t* sh_payload,
                               const float* sh_scales, float* out, int out_stride, int slots,
                               int top_k, void* stream, int sh_rs, int sh_cs);
+
+/* Extension (no counterpart in the reference): the four decode-slot launchers above and below (gate/up and down,
+ * FP8 and FP4) run a routed pass and, with n_shared > 0, a shared pass: two launches that touch disjoint slot rows.
+ * This call selects which of them the NEXT such launcher call of the calling thread runs - 1 the routed pass, 2 the
+ * shared pass, 3 both (the default, restored after that one call) - so that a host can put the shared expert's
+ * passes on a second stream beside the routed ones. Same arguments, same checks, same bits per pass. */
+void dgpp_moe_slot_passes(int passes);
 
 /* Extension (no counterpart in the reference): dgpp_launch_moe_router_select followed by the routed pass of
  * dgpp_launch_moe_slot_gate_up_swiglu / _fp4 (order == NULL, no shared expert; slots = tokens * (top_k + 1)),

@@ -126,6 +126,8 @@ inline void launch_moe_router_select_order(const float* scores, const float* bia
   detail::check(dgpp_launch_moe_router_select_order(scores, biased, ids, weights, order, &c, tokens,
                                                     shared_early ? 1 : 0, stream));
 }
+// Extension: which passes the next decode-slot launcher call of this thread runs (see dgpp_amd.h).
+inline void moe_slot_passes(int passes) { dgpp_moe_slot_passes(passes); }
 // Extension: selection + routed gate/up in one launch (see dgpp_amd.h).
 inline void launch_moe_select_gate_up_swiglu(const float* scores, const float* biased, int32_t* ids, float* weights,
                                              const GlmMoeConfig& cfg, int tokens, const uint16_t* x, size_t x_stride,

@@ -115,3 +115,53 @@ def test_layer_from_given_scores_softmax(gpu):
         _lib.load().dgpp_tune_set(7, 0)
     assert np.array_equal(host(out2, np.uint16), host(out, np.uint16))
     layer.close()
+
+
+@pytest.mark.parametrize("E,H,I,K,T,kind,shared,sI", [(16, 512, 128, 4, 4, "nvfp4", "fp8", 256), (16, 256, 128, 4, 3, "fp8", "fp8", 128),
+                                                      (10, 512, 64, 2, 2, "nvfp4", "nvfp4", 64), (12, 512, 128, 8, 24, "mxfp4", "fp8", 128)])
+def test_shared_expert_passes_beside_the_routed_ones_give_the_same_bits(gpu, E, H, I, K, T, kind, shared, sI):
+    """The layer driver runs the shared expert's gate/up and down passes on a second stream beside the routed passes
+    (forked and joined with events). Same bits as with everything on the caller's stream (bench switch 9), eagerly on
+    a side stream of the caller and as a captured graph replayed several times with eager work in between."""
+    from dgpp_amd import _lib
+    p = moe_data.make_problem(E, H, I, K, T, kind, 700 + E + T, shared_kind=shared, shared_I=sI, limit=10.0, std=0.05)
+    d = DeviceMoe(p)
+    layer = make_layer(p, d, 0, 2.5, T)
+    want = dev_empty((T, H), np.uint16)
+    _lib.load().dgpp_tune_set(9, 1)
+    try:
+        layer.enqueue_decode(d.x, H, want, T)
+        sync()
+    finally:
+        _lib.load().dgpp_tune_set(9, 0)
+    want_h = host(want, np.uint16).copy()
+    ids, w, _, _ = moe_data.orc_router(p, 0, 2.5, True)
+    raw, _ = moe_data.orc_forward(p, ids, w)
+    expert_budget(want_h, raw, "shared-expert layer on one stream")
+    s = torch.cuda.Stream()
+    got = dev_empty((T, H), np.uint16)
+    _lib.load().dgpp_tune_set(9, 2)           # the two-stream form at every batch size (default: from three tokens on)
+    try:
+        _two_stream_runs(layer, d, got, want_h, T, H, s)
+    finally:
+        _lib.load().dgpp_tune_set(9, 0)
+    layer.close()
+
+
+def _two_stream_runs(layer, d, got, want_h, T, H, s):
+    with torch.cuda.stream(s):
+        for _ in range(3):
+            got.zero_()
+            layer.enqueue_decode(d.x, H, got, T, s)
+            s.synchronize()
+            assert np.array_equal(host(got, np.uint16), want_h), "eager, passes on two streams"
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            layer.enqueue_decode(d.x, H, got, T, s)
+            layer.enqueue_decode(d.x, H, got, T, s)
+        for _ in range(3):
+            got.zero_()                       # eager work between the replays
+            s.synchronize()
+            g.replay()
+            s.synchronize()
+            assert np.array_equal(host(got, np.uint16), want_h), "graph replay"
