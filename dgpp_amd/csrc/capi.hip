@@ -360,6 +360,20 @@ int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const f
                 "moe_router");
 }
 
+int dgpp_launch_moe_router_dots(const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
+                                float* biased, const DgppMoeConfig* cfg, int tokens, void* stream) {
+  const int rc = dgpp_moe_config_validate(cfg);
+  if (rc != DGPP_OK) return rc;
+  if (tokens <= 0) return DGPP_OK;
+  const bool softmax = cfg->router_mode == DGPP_ROUTER_SOFTMAX_TOPK;
+  if (!hidden || !gate || (!softmax && !bias) || !scores || !biased) return fail_arg("moe_router_dots: null pointer");
+  if (scores == biased) return fail_arg("moe_router_dots: scores and biased must not alias");
+  if (cfg->n_experts > 65535 || tokens > 65535) return fail_arg("moe_router_dots: grid dimension overflow");
+  return finish(run_router_dots(cfg->router_mode, hidden, gate, bias, scores, biased, tokens, cfg->hidden, cfg->n_experts,
+                                as_stream(stream)),
+                "moe_router_dots");
+}
+
 int dgpp_launch_moe_router_select(const float* scores, const float* biased, int32_t* ids, float* weights,
                                   const DgppMoeConfig* cfg, int tokens, void* stream) {
   const int rc = dgpp_moe_config_validate(cfg);

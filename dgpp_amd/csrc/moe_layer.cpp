@@ -153,8 +153,10 @@ void GlmMoeLayer::enqueue_decode(const uint16_t* x, size_t x_stride, uint16_t* o
   if (tokens <= 0) return;
   check_tokens(tokens);
   if (!w_.router_gate) throw std::invalid_argument("GlmMoeLayer: the router gate is not bound");
-  launch_moe_router(x, w_.router_gate, w_.router_bias, d_ids_, d_weights_, d_scores_, d_biased_, cfg_, tokens, stream);
-  expert_chain_slots(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream);
+  // The score rows, then the chain from given scores: the selection rides a later launch where one takes it
+  // (with the slot order, or inside the gate/up launch of a one-token step).
+  launch_moe_router_dots(x, w_.router_gate, w_.router_bias, d_scores_, d_biased_, cfg_, tokens, stream);
+  enqueue_decode_scores(x, x_stride, d_scores_, d_biased_, out_bf16, out_f32, tokens, stream);
 }
 
 void GlmMoeLayer::enqueue_decode_scores(const uint16_t* x, size_t x_stride, const float* scores, const float* biased,
@@ -164,7 +166,7 @@ void GlmMoeLayer::enqueue_decode_scores(const uint16_t* x, size_t x_stride, cons
   // One routed-only token: the gate/up launch repeats the selection in its blocks (no launch of its own).
   // Otherwise selection and slot order in one launch; the chain below then finds its order ready.
   const bool with_order = needs_order(tokens);
-  const bool fused = tokens == 1 && !has_shared() && dgpp_tune_get(7) != 1;
+  const bool fused = tokens == 1 && dgpp_tune_get(7) != 1;
   if (!fused)
     launch_moe_router_select_order(scores, biased, d_ids_, d_weights_, with_order ? d_order_ : nullptr, cfg_, tokens, stream,
                                    cfg_.shared_slots_early);
@@ -199,7 +201,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   const int n_sh = has_shared() ? w_.shared_inter : 0;
   const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
   // With scores given, ids / weights are this layer's own buffers and the gate/up launch fills them.
-  const bool fused = sel_scores != nullptr && ids == d_ids_ && weights == d_weights_ && order == nullptr && !has_shared();
+  const bool fused = sel_scores != nullptr && ids == d_ids_ && weights == d_weights_ && order == nullptr;
   if (sel_scores != nullptr && !fused) throw std::logic_error("GlmMoeLayer: fused selection outside its form");
   // The shared expert's gate/up and down passes read nothing the routed passes write (disjoint slot rows): they run
   // on the side stream beside them, forked here and joined before the accumulation. One launcher call per pass.
@@ -218,10 +220,16 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     call(side_);
   };
   if (w_.format == GlmExpertFormat::Fp8) {
-    if (fused)
+    if (fused) {
       launch_moe_select_gate_up_swiglu(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
                                        d_slot_act_, max_inter_, cfg_.swiglu_limit, stream);
-    else
+      if (has_shared()) {   // the shared slot's pass: the launcher's own, the routed pass already done above
+        moe_slot_passes(2);
+        launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
+                                       w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
+                                       K, cfg_.swiglu_limit, split ? side_ : stream, w_.sh_rs, w_.sh_cs);
+      }
+    } else
       for_passes([&](hipStream_t st) {
         launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
                                        w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
@@ -238,10 +246,18 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     });
   } else {
     const int base = w_.shared_in_table ? cfg_.n_experts * 3 : -1;
-    if (fused)
+    if (fused) {
       launch_moe_select_gate_up_swiglu_fp4(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I,
                                            H, d_slot_act_, max_inter_, cfg_.swiglu_limit, stream, fp4_group_);
-    else
+      if (has_shared()) {
+        moe_slot_passes(2);
+        launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
+                                           sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
+                                           sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
+                                           d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, split ? side_ : stream, base,
+                                           fp4_group_, w_.sh_rs, w_.sh_cs);
+      }
+    } else
       for_passes([&](hipStream_t st) {
         launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
                                            sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,

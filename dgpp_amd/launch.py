@@ -68,6 +68,12 @@ def launch_moe_router(hidden, gate, bias, ids, weights, scores, biased, cfg: Moe
                                               1 if allow_tiled else 0))
 
 
+def launch_moe_router_dots(hidden, gate, bias, scores, biased, cfg: MoeConfig, tokens, stream=None):
+    """Extension: the router's score rows without the selection."""
+    _check(_lib.load().dgpp_launch_moe_router_dots(_p(hidden), _p(gate), _p(bias), _p(scores), _p(biased), C.addressof(cfg),
+                                                   tokens, _stream(stream)))
+
+
 def launch_moe_router_select(scores, biased, ids, weights, cfg: MoeConfig, tokens, stream=None):
     _check(_lib.load().dgpp_launch_moe_router_select(_p(scores), _p(biased), _p(ids), _p(weights), C.addressof(cfg),
                                                      tokens, _stream(stream)))

@@ -132,6 +132,12 @@ int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const f
                            int32_t* ids, float* weights, float* scores, float* biased,
                            const DgppMoeConfig* cfg, int tokens, void* stream, int* counters,
                            int allow_tiled);
+/* Extension (no counterpart in the reference): step 1 of dgpp_launch_moe_router alone - the score rows (`scores`,
+ * and `biased` = scores + bias, or the same values in softmax mode) without the selection, for hosts that run the
+ * selection inside a later launch (dgpp_launch_moe_router_select_order, dgpp_launch_moe_select_gate_up_swiglu). */
+int dgpp_launch_moe_router_dots(const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
+                                float* biased, const DgppMoeConfig* cfg, int tokens, void* stream);
+
 /* The selection half of launch_moe_router alone (src/kernels/glm_moe.cu:314-329,
  * moe_router_select_kernel): scores / biased f32 [tokens, n_experts] already on the device
  * (softmax mode: the bf16-rounded logits in both) -> ids ascending, weights. */

@@ -126,6 +126,12 @@ inline void launch_moe_router_select_order(const float* scores, const float* bia
   detail::check(dgpp_launch_moe_router_select_order(scores, biased, ids, weights, order, &c, tokens,
                                                     shared_early ? 1 : 0, stream));
 }
+// Extension: the router's score rows without the selection (see dgpp_amd.h).
+inline void launch_moe_router_dots(const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
+                                   float* biased, const GlmMoeConfig& cfg, int tokens, hipStream_t stream) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_router_dots(hidden, gate, bias, scores, biased, &c, tokens, stream));
+}
 // Extension: which passes the next decode-slot launcher call of this thread runs (see dgpp_amd.h).
 inline void moe_slot_passes(int passes) { dgpp_moe_slot_passes(passes); }
 // Extension: selection + routed gate/up in one launch (see dgpp_amd.h).

@@ -155,6 +155,17 @@ def test_router_tie_rule_and_full_router(gpu):
                 assert np.all(np.abs(host(w_d)[t] - want_w[t]) <= np.abs(want_w[t]) * (2.0 ** -7 if mode == 1 else 1e-4))
         with pytest.raises(L.InvalidArgument):
             L.launch_moe_router(dev(x), dev(gate), None, ids_d, w_d, sc_d, sc_d, cfg, T, None)  # aliasing
+        # the dots alone, then the selection from them: the router's own bits
+        sc2, bi2 = dev_empty((T, E), np.float32), dev_empty((T, E), np.float32)
+        ids2, w2 = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32)
+        L.launch_moe_router_dots(dev(x), dev(gate), None if mode == 1 else dev(bias), sc2, bi2, cfg, T, None)
+        L.launch_moe_router_select(sc2, bi2, ids2, w2, cfg, T, None)
+        sync()
+        assert np.array_equal(host(sc2).view(np.uint32), host(sc_d).view(np.uint32))
+        assert np.array_equal(host(bi2).view(np.uint32), host(bi_d).view(np.uint32))
+        assert np.array_equal(host(ids2), got_ids) and np.array_equal(host(w2).view(np.uint32), host(w_d).view(np.uint32))
+        with pytest.raises(L.InvalidArgument):
+            L.launch_moe_router_dots(dev(x), dev(gate), None, sc2, sc2, cfg, T, None)           # aliasing
 
 
 def test_swiglu_clamp(gpu):
