@@ -809,6 +809,7 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
   int steps = pick_steps(per_slot * a.slots);
   if (a.once && a.slots > a.top_k + 1) steps = 2;   // a decode batch of 2 - 8 tokens: measured best (one token: 1)
+  if (a.want_shared && a.once) steps = 1;           // one expert's rows over few runs: as many blocks as there are row groups
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
   // Larger batches (many slots per expert, an order given): runs of four where the rows fit the stage.
@@ -863,6 +864,7 @@ inline void slot_down_grid(const SlotArgs& a, RowGeom& g, int& steps, unsigned& 
   const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
   const long long per_slot = (a.n + rows_per_step - 1) / rows_per_step;
   steps = pick_steps(per_slot * a.slots);
+  if (a.want_shared && a.once) steps = 1;
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   tiles = static_cast<unsigned>((per_slot + steps - 1) / steps);
 }
