@@ -74,6 +74,7 @@ SIGNATURES = {
     "dgpp_launch_moe_router_select": (_I, [_P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_router_select_order": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P]),
     "dgpp_moe_slot_passes": (None, [_I]),
+    "dgpp_moe_slot_down_accum_into": (None, [_P, _P]),
     "dgpp_launch_moe_router_dots": (_I, [_P, _P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu_fp4": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P, _I]),

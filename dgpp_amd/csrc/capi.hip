@@ -263,6 +263,8 @@ SlotArgs slot_args(const uint16_t* x, size_t x_stride, const int32_t* ids, const
   a.top_k = top_k;
   a.limit = limit;
   a.shared_view_base = -1;
+  a.acc_weights = nullptr;
+  a.acc_out = nullptr;
   a.once = slots <= 16 * (top_k + 1);   // a decode batch of at most 16 tokens: few slots share an expert (measured up to there)
   const int tokens = top_k >= 0 ? slots / (top_k + 1) : 0;
   a.match = order == nullptr && tokens > 1 && tokens * top_k <= 128;
@@ -528,6 +530,24 @@ int take_slot_passes() {
 
 void dgpp_moe_slot_passes(int passes) { g_slot_passes = (passes & 3) ? (passes & 3) : 3; }
 
+namespace {
+// The accumulation the next slot-down launcher call of this thread folds into its shared pass
+// (dgpp_moe_slot_down_accum_into). One call consumes the setting.
+thread_local const float* g_down_acc_weights = nullptr;
+thread_local uint16_t* g_down_acc_out = nullptr;
+void take_down_accum(const float** w, uint16_t** out) {
+  *w = g_down_acc_weights;
+  *out = g_down_acc_out;
+  g_down_acc_weights = nullptr;
+  g_down_acc_out = nullptr;
+}
+}  // namespace
+
+void dgpp_moe_slot_down_accum_into(const float* weights, uint16_t* out_bf16) {
+  g_down_acc_weights = weights;
+  g_down_acc_out = out_bf16;
+}
+
 int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
                                         const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
                                         int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
@@ -636,6 +656,9 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
                               int top_k, void* stream, int sh_rs, int sh_cs) {
   const char* who = "moe_slot_down";
   const int passes = take_slot_passes();
+  const float* acc_w = nullptr;
+  uint16_t* acc_o = nullptr;
+  take_down_accum(&acc_w, &acc_o);
   if (slots <= 0) return DGPP_OK;
   int rc = check_slot_common(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, who);
   if (rc != DGPP_OK) return rc;
@@ -653,6 +676,7 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
   a.n = n_shared;
   a.k = k_shared;
   a.want_shared = 1;
+  if (acc_w && acc_o) a.acc_weights = acc_w, a.acc_out = acc_o;
   a.sh[0] = fp8_mat(sh_payload, sh_scales, sh_rs, sh_cs);
   return finish(launch_slot_down(kFmtFp8F32, a, as_stream(stream)), who);
 }
@@ -701,6 +725,9 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
                                   int fp4_group, int sh_rs, int sh_cs, int* tile_counter) {
   const char* who = "moe_slot_down_fp4";
   const int passes = take_slot_passes();
+  const float* acc_w = nullptr;
+  uint16_t* acc_o = nullptr;
+  take_down_accum(&acc_w, &acc_o);
   if (slots <= 0) return DGPP_OK;
   if (tile_counter == nullptr) return fail_arg(std::string(who) + ": the stealing counter pair is required");
   int rc = check_fp4_slot(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
@@ -719,6 +746,7 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
   a.n = n_shared;
   a.k = k_shared;
   a.want_shared = 1;
+  if (acc_w && acc_o) a.acc_weights = acc_w, a.acc_out = acc_o;
   if (shared_fp4) {
     a.shared_view_base = shared_view_base;
     return finish(launch_slot_down(fmt, a, as_stream(stream)), who);

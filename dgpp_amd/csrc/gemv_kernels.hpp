@@ -131,6 +131,11 @@ struct SlotArgs {
   int once;                 // few slots can share an expert: the weights stream through once (nontemporal loads)
   int want_shared;          // 0: routed slots, 1: shared slots (others exit)
   int shared_view_base;     // >= 0: shared matrices come from views[base + which]
+  // Down launches of the shared slots only, nullable: the token's accumulation as the epilogue. `out` then holds the
+  // routed slots' finished rows; the shared row is not stored, the token's row goes to acc_out as bf16:
+  // a = 0; a = fma(w_j, out[slot j], a) for j ascending; a = fma(1, shared dot, a); one rounding.
+  const float* acc_weights; // [tokens, top_k]
+  uint16_t* acc_out;        // [tokens, n]
 };
 
 // The router selection a gate/up launch can repeat in every block instead of reading `ids` (select_gate_up_kernel).
@@ -401,7 +406,7 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void select_gate_u
 }
 
 // Down rows of a run of slots, unrounded f32.
-template <int FMT, int NB, int MAXM, bool NT>
+template <int FMT, int NB, int MAXM, bool NT, bool ACC = false>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   SlotRun<MAXM> run;
@@ -434,9 +439,23 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_down_ker
     float acc[MAXM];
     row_dots<FMT, MAXM, NB>(lr, g, md.cs, lds, chunks, run.m, acc);
     if (lr.li == 0 && lr.row < a.n) {
+      if constexpr (ACC) {
 #pragma unroll
-      for (int r = 0; r < MAXM; ++r)
-        if (r < run.m) out[static_cast<size_t>(run.slot[r]) * a.out_stride + lr.row] = finish_dot<FMT>(acc[r], dd);
+        for (int r = 0; r < MAXM; ++r)
+          if (r < run.m) {
+            const int t = run.token[r];
+            const size_t base = static_cast<size_t>(t) * (a.top_k + 1);
+            float v = 0.f;
+            for (int j = 0; j < a.top_k; ++j)
+              v = fmaf(a.acc_weights[static_cast<size_t>(t) * a.top_k + j], out[(base + j) * a.out_stride + lr.row], v);
+            v = fmaf(1.0f, finish_dot<FMT>(acc[r], dd), v);
+            a.acc_out[static_cast<size_t>(t) * a.n + lr.row] = f32_to_bf16(v);
+          }
+      } else {
+#pragma unroll
+        for (int r = 0; r < MAXM; ++r)
+          if (r < run.m) out[static_cast<size_t>(run.slot[r]) * a.out_stride + lr.row] = finish_dot<FMT>(acc[r], dd);
+      }
     }
   }
 }
@@ -878,6 +897,21 @@ hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
   slot_down_grid<FMT>(a, g, steps, tiles);
   const dim3 grid(tiles, static_cast<unsigned>(a.slots));
   const int cap = run_cap_for(a, kDownRun);
+  if (a.acc_out != nullptr) {   // a shared pass that ends with the token's accumulation: cached loads, every run length
+    dispatch_nb(g.nb, [&](auto nbc) {
+      constexpr int NB = decltype(nbc)::value;
+      if (cap >= kDownRun)
+        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, kDownRun, false, true>), grid, dim3(kBlockThreads),
+                           stage_bytes(kDownRun, a.k), stream, a, g, steps);
+      else if (cap >= 2)
+        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 2, false, true>), grid, dim3(kBlockThreads), stage_bytes(2, a.k), stream,
+                           a, g, steps);
+      else
+        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 1, false, true>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream,
+                           a, g, steps);
+    });
+    return hipGetLastError();
+  }
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
     dispatch_bool(a.once && !a.want_shared, [&](auto ntc) {

@@ -212,6 +212,11 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     hip_ok(hipEventRecord(fork_, stream), "GlmMoeLayer: fork");
     hip_ok(hipStreamWaitEvent(side_, fork_, 0), "GlmMoeLayer: fork");
   }
+  // On one stream the shared down pass ends with the token's accumulation (no launch of its own).
+  // (One token, where a launch is a fifth of the step; measured level at two tokens. Bench switch 9 = 4 folds at any
+  // batch size, 3 never.)
+  const bool fold_accum = has_shared() && !split && out_bf16 != nullptr && out_f32 == nullptr && dgpp_tune_get(9) != 3 &&
+                          (tokens == 1 || dgpp_tune_get(9) == 4);
   auto for_passes = [&](auto&& call) {
     if (!split) return call(stream);
     moe_slot_passes(1);
@@ -240,6 +245,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
                                  out_bf16, out_f32, stream);
       return;
     }
+    if (fold_accum) moe_slot_down_accum_into(weights, out_bf16);
     for_passes([&](hipStream_t st) {
       launch_moe_slot_down(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
                            n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, st, w_.sh_rs, w_.sh_cs);
@@ -270,6 +276,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
                                      out_bf16, out_f32, stream, fp4_group_);
       return;
     }
+    if (fold_accum) moe_slot_down_accum_into(weights, out_bf16);
     for_passes([&](hipStream_t st) {
       launch_moe_slot_down_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
                                has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
@@ -281,6 +288,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     hip_ok(hipEventRecord(join_, side_), "GlmMoeLayer: join");
     hip_ok(hipStreamWaitEvent(stream, join_, 0), "GlmMoeLayer: join");
   }
+  if (fold_accum) return;
   if (has_shared()) {
     if (out_f32) {
       // The shared chain, unrounded: the ordered form over the slot layout's rows.

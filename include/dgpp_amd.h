@@ -48,7 +48,8 @@ const char* dgpp_target_arch(void);
  * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
  * blocks, dgpp_launch_moe_select_gate_up_swiglu); key 9: 1 keeps the shared expert's passes of the layer driver
  * on the caller's stream, 2 moves them to a second stream beside the routed passes at every batch size (default:
- * from three tokens on). Outputs do not depend on keys
+ * from three tokens on); 3 and 4 keep one stream and never / always fold the accumulation into the shared down pass
+ * (default: at one token). Outputs do not depend on keys
  * 1 - 4, 6, 7 and 9; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
  * bitwise twins of each other). */
@@ -226,6 +227,13 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
  * shared pass, 3 both (the default, restored after that one call) - so that a host can put the shared expert's
  * passes on a second stream beside the routed ones. Same arguments, same checks, same bits per pass. */
 void dgpp_moe_slot_passes(int passes);
+/* Extension (no counterpart in the reference): the NEXT dgpp_launch_moe_slot_down / _fp4 call of the calling thread
+ * folds dgpp_launch_moe_slot_accum into its shared pass. `out` of that call must hold the routed slots' finished rows
+ * by the time the shared pass runs (the same call's routed pass, or an earlier one on the stream); the shared pass then
+ * stores no slot row but the token's accumulated row - a = 0; a = fma(weights[t, j], out[slot j], a) for j ascending;
+ * a = fma(1, shared dot, a); one rounding - to out_bf16 [tokens, n_shared]. Same bits as the two launches. One call
+ * consumes the setting; a null argument clears it. */
+void dgpp_moe_slot_down_accum_into(const float* weights, uint16_t* out_bf16);
 
 /* Extension (no counterpart in the reference): dgpp_launch_moe_router_select followed by the routed pass of
  * dgpp_launch_moe_slot_gate_up_swiglu / _fp4 (order == NULL, no shared expert; slots = tokens * (top_k + 1)),

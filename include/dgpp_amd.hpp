@@ -134,6 +134,10 @@ inline void launch_moe_router_dots(const uint16_t* hidden, const uint16_t* gate,
 }
 // Extension: which passes the next decode-slot launcher call of this thread runs (see dgpp_amd.h).
 inline void moe_slot_passes(int passes) { dgpp_moe_slot_passes(passes); }
+// Extension: the next slot-down call's shared pass ends with the token's accumulation (see dgpp_amd.h).
+inline void moe_slot_down_accum_into(const float* weights, uint16_t* out_bf16) {
+  dgpp_moe_slot_down_accum_into(weights, out_bf16);
+}
 // Extension: selection + routed gate/up in one launch (see dgpp_amd.h).
 inline void launch_moe_select_gate_up_swiglu(const float* scores, const float* biased, int32_t* ids, float* weights,
                                              const GlmMoeConfig& cfg, int tokens, const uint16_t* x, size_t x_stride,

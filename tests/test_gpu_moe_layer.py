@@ -128,13 +128,18 @@ def test_shared_expert_passes_beside_the_routed_ones_give_the_same_bits(gpu, E, 
     d = DeviceMoe(p)
     layer = make_layer(p, d, 0, 2.5, T)
     want = dev_empty((T, H), np.uint16)
-    _lib.load().dgpp_tune_set(9, 1)
+    _lib.load().dgpp_tune_set(9, 3)           # one stream, the accumulation a launch of its own
     try:
         layer.enqueue_decode(d.x, H, want, T)
         sync()
+        want_h = host(want, np.uint16).copy()
+        _lib.load().dgpp_tune_set(9, 4)       # one stream, the accumulation folded into the shared down pass
+        want.zero_()
+        layer.enqueue_decode(d.x, H, want, T)
+        sync()
+        assert np.array_equal(host(want, np.uint16), want_h), "folded accumulation"
     finally:
         _lib.load().dgpp_tune_set(9, 0)
-    want_h = host(want, np.uint16).copy()
     ids, w, _, _ = moe_data.orc_router(p, 0, 2.5, True)
     raw, _ = moe_data.orc_forward(p, ids, w)
     expert_budget(want_h, raw, "shared-expert layer on one stream")
