@@ -31,10 +31,28 @@ HBM_PEAK_GBPS = 8000.0
 E, H, I, K = 256, 4096, 1024, 8          # the headline configuration (MXFP4 MoE decode layer)
 EXPERT_BYTES = 3 * I * H // 2 + 3 * I * H // 32          # payload + e8m0 scales of gate, up, down
 GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
-# HBM-side bytes per launch of the two GEMV kernels at the default workload (T = 8, 256 experts), from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the library's plain copy kernel (the summary under
-# profiles/ holds the commands and the raw counters). A counter cannot be read from inside this process.
-MEASURED_TRAFFIC = {"gate_up": 260.3e6, "down": 138.5e6}
+# HBM-side bytes per launch of the two GEMV kernels at the default workload (T = 8, 256 experts) come from rocprofv3
+# --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the library's plain copy kernel: a counter cannot be read from inside
+# this process, so the figures are read out of the committed summary of those runs (its `traffic_bytes_per_launch`
+# lines, which also name the kernels they were taken from) and dropped from the line when the workload differs.
+TRAFFIC_PROFILE = "profiles/moe_gemv_kernels_mxfp4_c3_t8_hbm_counters.txt"
+
+
+def measured_traffic():
+    """{"gate_up": bytes, "down": bytes, "gate_up_kernel": name, "down_kernel": name} from the counter summary, or {}."""
+    out = {}
+    try:
+        text = (ROOT / TRAFFIC_PROFILE).read_text()
+    except OSError:
+        return out
+    for line in text.splitlines():
+        part = line.split()
+        if len(part) >= 4 and part[0] == "traffic_bytes_per_launch":
+            out[part[1]] = float(part[2])
+            out[part[1] + "_kernel"] = " ".join(part[3:])
+    return out
+
+
 DOWN_BYTES = H * I // 2 + H * I // 32
 
 
@@ -126,36 +144,49 @@ def main():
 
     stream = torch.cuda.Stream()
 
-    def time_graph(enqueue, steps, warmup):
-        """Captures `steps` calls of enqueue(i) in one graph, replays it once untimed (plus `warmup` eager
-        steps before capture) and once timed with events on the launch stream. Returns seconds per step."""
+    def time_graph(enqueue, steps, warmup, stats=None):
+        """Captures `steps` calls of enqueue(i) in one HIP graph and replays it back to back at least 50 times (and until
+        at least 1000 steps have run), with an event on the launch stream between consecutive replays. A replay's time
+        is the span between its two events; the figure returned is the MEDIAN replay divided by `steps`, in seconds per
+        step, so it does not depend on how many steps one graph holds (the replays queue behind each other: a graph's
+        launch set-up overlaps its predecessor's run). `stats`, when given, receives median / min / max per step in
+        microseconds and the replay count. `warmup` eager steps run before the capture and one untimed replay after it."""
+        replays = max(50, -(-1000 // max(steps, 1)))
         with torch.cuda.stream(stream):
             for i in range(max(warmup, 1)):
                 enqueue(i)
             stream.synchronize()
             if args.eager:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record(stream)
-                for i in range(steps):
-                    enqueue(i)
-                e1.record(stream)
+                evs = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+                evs[0].record(stream)
+                for r in range(replays):
+                    for i in range(steps):
+                        enqueue(i)
+                    evs[r + 1].record(stream)
+            else:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    for i in range(steps):
+                        enqueue(i)
+                g.replay()
+                stream.synchronize()
+                evs = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
                 torch.cuda.synchronize()
-                return e0.elapsed_time(e1) * 1e-3 / steps
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=stream):
-                for i in range(steps):
-                    enqueue(i)
-            g.replay()
-            stream.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                evs[0].record(stream)
+                for r in range(replays):
+                    g.replay()
+                    evs[r + 1].record(stream)
             torch.cuda.synchronize()
-            e0.record(stream)
-            g.replay()
-            e1.record(stream)
-            torch.cuda.synchronize()
-            return e0.elapsed_time(e1) * 1e-3 / steps
+        per = np.array([evs[r].elapsed_time(evs[r + 1]) for r in range(replays)], dtype=np.float64) * 1e-3 / steps
+        if stats is not None:
+            stats.update({"us_median": float(np.median(per)) * 1e6, "us_min": float(per.min()) * 1e6,
+                          "us_max": float(per.max()) * 1e6, "replays": replays, "steps_per_replay": steps})
+        return float(np.median(per))
 
     def measure(T, steps, warmup, only=""):
+        # a graph holds whole walks of the ring (at least four), so that a replay never meets a layer its predecessor has
+        # just left and the few microseconds between two replays stay below one percent of a replay
+        steps = max(4, -(-steps // nL)) * nL
         xs, lg_d, lg = inputs(T)
         outs = torch.empty((nL, T, H), dtype=torch.int16, device=dev)
         # distinct experts per layer-step (the algorithmic bytes count each distinct expert once)
@@ -173,8 +204,10 @@ def main():
             layers[l].enqueue_decode_scores(xs[l], H, lg_d[l], lg_d[l], outs[l], T, stream)
 
         if only in ("", "layer"):
-            sec = time_graph(full, steps, warmup)
+            st = {}
+            sec = time_graph(full, steps, warmup, st)
             res["us_per_layer"] = sec * 1e6
+            res["timing"] = st
             res["gbps"] = layer_bytes / sec / 1e9
             res["frac_of_peak"] = res["gbps"] / HBM_PEAK_GBPS
         # the dominant kernel alone: the fused gate/up + SwiGLU slot kernel on the routes the layers hold
@@ -197,7 +230,9 @@ def main():
                                                  slots, K, float("inf"), stream, -1, 32)
 
         if only in ("", "gate_up"):
-            sec_k = time_graph(gate_up, steps, warmup)
+            st_k = {}
+            sec_k = time_graph(gate_up, steps, warmup, st_k)
+            res["gate_up_timing"] = st_k
             kbytes = u_mean * GATE_UP_BYTES + T * H * 2 + T * K * I * 2
             res["gate_up_us"] = sec_k * 1e6
             res["gate_up_bytes"] = kbytes
@@ -208,7 +243,9 @@ def main():
                                              layers[l].weights_ptr, outs[l], None, stream, 32)
 
         if only in ("", "down"):
-            sec_d = time_graph(down, steps, warmup)
+            st_d = {}
+            sec_d = time_graph(down, steps, warmup, st_d)
+            res["down_timing"] = st_d
             dbytes = u_mean * DOWN_BYTES + T * K * I * 2 + T * H * 2
             res["down_us"] = sec_d * 1e6
             res["down_bytes"] = dbytes
@@ -751,8 +788,10 @@ def main():
                 "router logits ~ N(0,1)",
         "config": {"workload": f"BASELINE config 3: MXFP4 MoE decode layer, {nE} experts, hidden {H}, inter {I}, "
                                f"top-{K} softmax-renormalised, no shared expert, T={T} tokens",
-                   "tokens": T, "ring_layers": nL, "timing": "HIP graph of `steps` layer passes, events on the "
-                   "launch stream, weights cold (ring >= 2x the 256 MB cache)",
+                   "tokens": T, "ring_layers": nL, "timing": "median over back-to-back replays (>= 50, >= 1000 layer passes) of one HIP graph of "
+                   "`steps` layer passes rounded up to whole walks of the layer ring (at least four), an event on the launch stream between "
+                   "replays; weights cold (ring >= 2x the 256 MB cache)",
+                   "timing_stats": main_res.get("timing"),
                    "distinct_experts_mean": main_res["distinct_experts_mean"],
                    "algorithmic_bytes_per_layer": main_res["algorithmic_bytes"]},
         "roofline": None,
@@ -761,17 +800,20 @@ def main():
         "other_configs": other_configs,
         "build_seconds": build_s,
     }
+    traffic = measured_traffic()
+    same_workload = T == 8 and nE == E and not args.tune
     if "gate_up_us" in main_res:
         line["roofline"] = {"kernel": "slot_gate_up_kernel<MXFP4> (fused gate/up GEMV + SwiGLU)", "bound": "hbm",
                             "achieved": main_res["gate_up_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                             "frac": main_res["gate_up_gbps"] / HBM_PEAK_GBPS,
-                            "traffic": MEASURED_TRAFFIC["gate_up"] if (T == 8 and nE == E and not args.tune) else None,
+                            "traffic": traffic.get("gate_up") if same_workload else None,
+                            "traffic_source": (TRAFFIC_PROFILE + ": " + traffic.get("gate_up_kernel", "")) if same_workload else None,
                             "bytes_per_launch": main_res["gate_up_bytes"], "us_per_launch": main_res["gate_up_us"]}
         if "down_us" in main_res:
             line["roofline"]["second_kernel"] = {
                 "kernel": "token_down_accum_kernel<MXFP4> (down GEMV + ordered accumulation, bf16 out)",
                 "achieved": main_res["down_gbps"],
-                "traffic": MEASURED_TRAFFIC["down"] if (T == 8 and nE == E and not args.tune) else None,
+                "traffic": traffic.get("down") if same_workload else None,
                 "frac": main_res["down_gbps"] / HBM_PEAK_GBPS, "bytes_per_launch": main_res["down_bytes"],
                 "us_per_launch": main_res["down_us"]}
     print(json.dumps(line))

@@ -12,6 +12,7 @@
 #include "../../include/dgpp_amd.h"
 #include "gemv_core.hpp"
 #include "router_select.hpp"
+#include "swiglu.hpp"
 
 namespace dgpp_amd {
 
@@ -23,20 +24,7 @@ namespace dgpp_amd {
 #endif
 constexpr int kMinWavesPerSimd = DGPP_MIN_WAVES_PER_SIMD;
 
-// ---- epilogues ------------------------------------------------------------------------------
-__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
-
-// SwiGLU on the bf16-rounded dots with the reference's rounding points
-// (src/kernels/glm_moe.cu:659-666): gate clamped above only, up on both sides.
-__device__ __forceinline__ uint16_t swiglu_bf16(float gate_dot, float up_dot, float limit) {
-  float g = bf16_to_f32(f32_to_bf16(gate_dot));
-  float u = bf16_to_f32(f32_to_bf16(up_dot));
-  if (g > limit) g = limit;
-  u = fminf(fmaxf(u, -limit), limit);
-  const uint16_t t = f32_to_bf16(g * sigmoid_f32(g));
-  return f32_to_bf16(bf16_to_f32(t) * u);
-}
-
+// ---- epilogues (SwiGLU: swiglu.hpp) -------------------------------------------------------------
 template <int FMT>
 __device__ __forceinline__ float finish_dot(float acc, float divisor) {
   if constexpr (FMT == kFmtNvfp4) return acc / divisor;  // one correctly rounded division

@@ -10,19 +10,6 @@ namespace dgpp_amd {
 constexpr int kStageUnits = 1024;   // 16-byte units of one block-shared activation stage (16 KB)
 constexpr int kMfmaNB = 4;          // lane loads in flight per row group and pass
 
-// SwiGLU of eight bf16 gate / up pairs (the elementwise kernel's arithmetic; zeros stay zeros).
-__device__ __forceinline__ uint4 swiglu_block(const uint4& gate, const uint4& up, float limit) {
-  const uint32_t g[4] = {gate.x, gate.y, gate.z, gate.w}, u[4] = {up.x, up.y, up.z, up.w};
-  uint32_t o[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint16_t lo = swiglu_bf16(bf16_to_f32(static_cast<uint16_t>(g[i] & 0xFFFFu)), bf16_to_f32(static_cast<uint16_t>(u[i] & 0xFFFFu)), limit);
-    const uint16_t hi = swiglu_bf16(bf16_to_f32(static_cast<uint16_t>(g[i] >> 16)), bf16_to_f32(static_cast<uint16_t>(u[i] >> 16)), limit);
-    o[i] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
-  }
-  return make_uint4(o[0], o[1], o[2], o[3]);
-}
-
 // 64 weight rows (one row group per wavefront) against mt <= 16 activation rows, parts [p_lo, p_hi) of K.
 // K is walked in batches of up to kTileBatch tiles (a tile = four steps of a row group, gemv_mfma.hpp):
 // a wavefront puts all of a batch's weight loads in flight, the block then fetches the batch's
@@ -91,7 +78,7 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
       if (threadIdx.x + i * kBlockThreads < units) {
         pre[i] = load_act_block(act + unit_row[i], k_base + unit_kb[i] * 8, k, aligned);
         if constexpr (SW)   // the activation is SwiGLU(act, act_up), computed on its way into the stage
-          pre[i] = swiglu_block(pre[i], load_act_block(act_up + unit_row[i], k_base + unit_kb[i] * 8, k, aligned), limit);
+          pre[i] = swiglu_bf16x8(pre[i], load_act_block(act_up + unit_row[i], k_base + unit_kb[i] * 8, k, aligned), limit);
       }
     }
     __syncthreads();   // the stage's readers of the batch before are through
