@@ -312,6 +312,12 @@ def main():
             nbytes = n * k // 2 + n * k // 16 + 4 + m * (k * 2 + n * 2)
             res[f"batch{m}"] = {"us": sec * 1e6, "algorithmic_bytes": nbytes, "gbps": nbytes / sec / 1e9,
                                 "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+            if m > 4:   # the same launcher pinned to the vector core (what it ran before the row-count dispatch)
+                lib.dgpp_tune_set(5, 1)
+                sec = time_graph(step, args.steps, args.warmup)
+                lib.dgpp_tune_set(5, 0)
+                res[f"batch{m}_vector_core"] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9,
+                                                "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
             def step_mma(i):
                 r = i % len(ring)
                 L.launch_dense_mma_fp4_bf16(act, k, mats[r], out[r], m, n, k, stream)
@@ -455,9 +461,9 @@ def main():
             L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
             L.launch_moe_round_bf16(out, routed, cT * cH, stream)
 
-        def full(i):
+        def full(i):            # the shared expert through the GEMV-named launchers (they take the matrix core at 64 rows)
             routed_part(i)
-            shared_mc(i)
+            shared_part(i)
 
         def full_w8a8(i):
             routed_part(i)
@@ -468,7 +474,7 @@ def main():
         shared_bytes = 3 * cSI * cH + 3 * cSI * cH // 32
         nbytes = uniq * per_expert + shared_bytes + cT * cH * 4
         res = {"workload": f"C5 NVFP4 routed MoE (256 experts, hidden 6144, inter 2048, top-8, {uniq} distinct; decode slots) "
-                           f"+ MXFP8 shared expert (inter 4096; matrix-core launchers), T=64; routed expert weights = device copies of {G} generated experts",
+                           f"+ MXFP8 shared expert (inter 4096; launch_scale_gemm_grid_e8m0_*, which run the matrix-core form at 64 rows), T=64; routed expert weights = device copies of {G} generated experts",
                "algorithmic_bytes": nbytes}
         for name, fn, nb in (("layer", full, nbytes), ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
                              ("routed_only_matrix_core", routed_mc, uniq * per_expert + cT * cH * 6),

@@ -66,15 +66,10 @@ _P, _I, _F, _Z, _L = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_int64
 SIGNATURES = {
     "dgpp_last_error": (C.c_char_p, []),
     "dgpp_target_arch": (C.c_char_p, []),
-    "dgpp_tune_set": (None, [_I, _I]),
-    "dgpp_tune_get": (_I, [_I]),
-    "dgpp_probe_copy": (_I, [_P, _P, C.c_size_t, _P]),
     "dgpp_moe_config_validate": (_I, [_P]),
     "dgpp_launch_moe_router": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_launch_moe_router_select": (_I, [_P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_router_select_order": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P]),
-    "dgpp_moe_slot_passes": (None, [_I]),
-    "dgpp_moe_slot_down_accum_into": (None, [_P, _P]),
     "dgpp_launch_moe_router_dots": (_I, [_P, _P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu_fp4": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P, _I]),
@@ -97,6 +92,10 @@ SIGNATURES = {
     "dgpp_launch_moe_slot_down": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_launch_moe_slot_gate_up_swiglu_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I, _I, _I]),
     "dgpp_launch_moe_slot_down_fp4": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _P]),
+    "dgpp_launch_moe_slot_gate_up_swiglu_ex": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I, _I]),
+    "dgpp_launch_moe_slot_down_ex": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _P, _P]),
+    "dgpp_launch_moe_slot_gate_up_swiglu_fp4_ex": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _P, _I, _I, _I, _I, _I]),
+    "dgpp_launch_moe_slot_down_fp4_ex": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _P, _I, _P, _P]),
     "dgpp_launch_moe_slot_down_accum": (_I, [_P, _Z, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P]),
     "dgpp_launch_moe_slot_down_accum_fp4": (_I, [_P, _Z, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I]),
     "dgpp_launch_dense_mma_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _Z]),
@@ -191,6 +190,14 @@ LAYER_SIGNATURES = {
     "dgpp_moe_layer_weights": (_P, [_P]),
 }
 
+# include/dgpp_amd_bench.h (measurement aids; not part of the launcher surface)
+BENCH_SIGNATURES = {
+    "dgpp_tune_set": (None, [_I, _I]),
+    "dgpp_tune_get": (_I, [_I]),
+    "dgpp_probe_copy": (_I, [_P, _P, C.c_size_t, _P]),
+    "dgpp_probe_read": (_I, [_P, C.c_size_t, _P, _I, _P]),
+}
+
 _lib = None
 
 
@@ -210,7 +217,7 @@ def load() -> C.CDLL:
     except ImportError:
         pass
     lib = C.CDLL(str(LIB_PATH))
-    for name, (res, args) in {**SIGNATURES, **LAYER_SIGNATURES}.items():
+    for name, (res, args) in {**SIGNATURES, **LAYER_SIGNATURES, **BENCH_SIGNATURES}.items():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args

@@ -23,7 +23,9 @@ HIP_SOURCES = [
     "gemv_nvfp4.hip",
     "gemv_fp8f32.hip",
     "gemv_fp8e8m0.hip",
-    "moe_misc.hip",
+    "moe_router.hip",
+    "moe_grouping.hip",
+    "moe_elementwise.hip",
     "mxfp8_gemm.hip",
     "qwen_tail.hip",
     "capi.hip",

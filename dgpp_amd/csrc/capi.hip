@@ -8,6 +8,7 @@
 #include <unordered_map>
 
 #include "../../include/dgpp_amd.h"
+#include "../../include/dgpp_amd_bench.h"
 #include "capi_errors.hpp"
 #include "gemv_kernels.hpp"
 #include "moe_misc.hpp"
@@ -137,12 +138,35 @@ hipError_t launch_grouped_mma(int fmt, const GroupedArgs& a, int n_segs, int z_e
 
 namespace {
 
-// Dense GEMV over m rows in chunks the LDS can stage (each row's chain is the same whatever
-// the chunking). k == 0 zero-fills. `out_elem` is 2 (bf16) or 4 (f32).
+// Dense projection over m rows. Few rows take the vector-core GEMV in chunks the LDS can stage (each row's chain is
+// the same whatever the chunking); from `mma_from` rows on the call goes to the matrix-core form, which carries 16
+// rows per weight pass (the reference's launchers move to their tensor-core forms as m grows in the same way:
+// src/kernels/scale_gemm.cu:296-339, src/kernels/glm_moe_launch.hpp:363). The two forms differ in fp32 summation
+// order, so a row's bits depend on which side of the boundary the call's m lies - both are held to the same oracle
+// tolerance. `ws` (nullable) is the split-K workspace of the matrix-core form. `out_elem` is 2 (bf16) or 4 (f32).
+constexpr int kFp4MmaFromRows = 5;   // vector core: 8 dot chains per weight beyond 4 rows cost more than the matrix core's decode
+constexpr int kFp8MmaFromRows = 9;   // the vector core's one-pass limit (kMaxActRows)
 int dense_rows(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,
-               size_t out_stride, int out_f32, int m, int n, int k, hipStream_t stream, const char* who) {
-  // The matrix-core form takes every row in one launch (16 per weight pass); the vector form what LDS can stage.
-  const int max_rows = tune_get(kTuneCore) == 2 ? m : max_stage_rows(k);
+               size_t out_stride, int out_f32, int m, int n, int k, hipStream_t stream, const char* who, int mma_from,
+               void* ws = nullptr, size_t ws_bytes = 0) {
+  const int core = tune_get(kTuneCore);   // bench switch: 1 pins the vector core, 2 the matrix core
+  if (core != 1 && (core == 2 || m >= mma_from)) {
+    if ((m + kTileCols - 1) / kTileCols > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
+    DenseArgs a;
+    a.act = act;
+    a.act_stride = act_stride;
+    a.mat = mat;
+    a.global = global;
+    a.out = out;
+    a.out_stride = out_stride;
+    a.out_f32 = out_f32;
+    a.m = m;
+    a.n = n;
+    a.k = k;
+    a.once = m <= kTileCols;
+    return finish(launch_dense_mma(fmt, a, static_cast<float*>(ws), ws_bytes, stream), who);
+  }
+  const int max_rows = max_stage_rows(k);
   const size_t esz = out_f32 ? 4 : 2;
   for (int row0 = 0; row0 < m;) {
     const int rows = std::min(max_rows, m - row0);
@@ -184,14 +208,15 @@ int fp4_gemv(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, voi
   mat.rs = 0;
   mat.cs = 0;
   return dense_rows(w->scale_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, mat, w->global_scale, out,
-                    static_cast<size_t>(n), out_f32, m, n, k, as_stream(stream), "fp4_gemv");
+                    static_cast<size_t>(n), out_f32, m, n, k, as_stream(stream), "fp4_gemv", kFp4MmaFromRows);
 }
 
 // src/kernels/scale_gemm.cu:280-365 (launch_scale_gemm) and :406-462 (launch_scale_gemm_grid):
 // every m takes the row-independent GEMV form here.
 int scale_gemm(const uint16_t* act, size_t act_stride, const uint8_t* payload, const void* scales, int e8m0, void* out,
                int out_f32, int m, int n, int k, void* stream, size_t out_stride, int rs, int cs, int last_row_only,
-               int compact_row, bool grid_form, const char* who) {
+               int compact_row, bool grid_form, const char* who, int mma_from_rows = 0, void* ws = nullptr,
+               size_t ws_bytes = 0) {
   if (m <= 0 || n <= 0) return DGPP_OK;
   if (!act || !payload || !scales || !out) return fail_arg(std::string(who) + ": null pointer");
   if (grid_form) {
@@ -220,8 +245,10 @@ int scale_gemm(const uint16_t* act, size_t act_stride, const uint8_t* payload, c
   }
   if (!fp8_shape_ok(payload, k))
     return fail_arg(std::string(who) + ": k must be a multiple of 16 with a 16-byte aligned payload");
+  // the caller's own threshold (the reference's mma_from_rows) can only lower the boundary
+  const int mma_from = mma_from_rows > 0 && mma_from_rows < kFp8MmaFromRows ? mma_from_rows : kFp8MmaFromRows;
   return dense_rows(e8m0 ? kFmtFp8E8M0 : kFmtFp8F32, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, o,
-                    out_stride, out_f32, m, n, k, as_stream(stream), who);
+                    out_stride, out_f32, m, n, k, as_stream(stream), who, mma_from, ws, ws_bytes);
 }
 
 // src/kernels/glm_moe.cu:1683-1703 (check_slot_args) and :2197-2228 (check_fp4_slot_args).
@@ -320,6 +347,14 @@ int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
   if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(dst) % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0)
     return fail_arg(std::string(who) + ": bytes and both pointers must be multiples of 16");
   return finish(run_probe_copy(dst, src, bytes, as_stream(stream)), who);
+}
+int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, void* stream) {
+  const char* who = "probe read";
+  if (bytes == 0) return DGPP_OK;
+  if (!src || !sink) return fail_arg(std::string(who) + ": null pointer");
+  if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0)
+    return fail_arg(std::string(who) + ": bytes and the pointer must be multiples of 16");
+  return finish(run_probe_read(src, bytes, sink, nontemporal, as_stream(stream)), who);
 }
 void dgpp_tune_set(int key, int value) {
   if (key >= 0 && key < kTuneCount) g_tune[key] = value;
@@ -518,35 +553,19 @@ int dgpp_launch_moe_slot_accum_routed_bf16(uint16_t* out, const float* contrib, 
 }
 
 namespace {
-// Which passes the next decode-slot launcher call of this thread runs (dgpp_moe_slot_passes): bit 0 the routed
-// slots, bit 1 the shared slots. One call consumes the setting.
-thread_local int g_slot_passes = 3;
-int take_slot_passes() {
-  const int p = g_slot_passes;
-  g_slot_passes = 3;
-  return p;
+// The pass selector of the *_ex decode-slot launchers: bit 0 the routed slots, bit 1 the shared slots.
+// A request that cannot be carried out is an error, never dropped: a pass selector outside 1..3, a shared pass
+// without a shared expert, an accumulation target without the shared pass that would write it.
+int check_passes(int passes, int n_shared, const float* acc_w, const uint16_t* acc_o, const char* who) {
+  if (passes < 1 || passes > 3) return fail_arg(std::string(who) + ": passes must be 1 (routed), 2 (shared) or 3 (both)");
+  if (passes == 2 && n_shared == 0) return fail_arg(std::string(who) + ": the shared pass was asked for and there is no shared expert");
+  if ((acc_w == nullptr) != (acc_o == nullptr))
+    return fail_arg(std::string(who) + ": the accumulation needs both its weights and its output row");
+  if (acc_o != nullptr && (n_shared == 0 || !(passes & 2)))
+    return fail_arg(std::string(who) + ": the accumulation rides the shared pass, which this call does not run");
+  return DGPP_OK;
 }
 }  // namespace
-
-void dgpp_moe_slot_passes(int passes) { g_slot_passes = (passes & 3) ? (passes & 3) : 3; }
-
-namespace {
-// The accumulation the next slot-down launcher call of this thread folds into its shared pass
-// (dgpp_moe_slot_down_accum_into). One call consumes the setting.
-thread_local const float* g_down_acc_weights = nullptr;
-thread_local uint16_t* g_down_acc_out = nullptr;
-void take_down_accum(const float** w, uint16_t** out) {
-  *w = g_down_acc_weights;
-  *out = g_down_acc_out;
-  g_down_acc_weights = nullptr;
-  g_down_acc_out = nullptr;
-}
-}  // namespace
-
-void dgpp_moe_slot_down_accum_into(const float* weights, uint16_t* out_bf16) {
-  g_down_acc_weights = weights;
-  g_down_acc_out = out_bf16;
-}
 
 int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
                                         const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
@@ -554,10 +573,22 @@ int dgpp_launch_moe_slot_gate_up_swiglu(const uint16_t* x, size_t x_stride, cons
                                         const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
                                         int act_stride, int slots, int top_k, float limit, void* stream, int sh_rs,
                                         int sh_cs) {
+  return dgpp_launch_moe_slot_gate_up_swiglu_ex(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                                sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride,
+                                                slots, top_k, limit, stream, sh_rs, sh_cs, 3);
+}
+
+int dgpp_launch_moe_slot_gate_up_swiglu_ex(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                                           const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                           int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                           const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                           int act_stride, int slots, int top_k, float limit, void* stream, int sh_rs,
+                                           int sh_cs, int passes) {
   const char* who = "moe_slot_gate_up";
-  const int passes = take_slot_passes();
   if (slots <= 0) return DGPP_OK;
-  int rc = check_slot_common(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, who);
+  int rc = check_passes(passes, n_shared, nullptr, nullptr, who);
+  if (rc != DGPP_OK) return rc;
+  rc = check_slot_common(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, who);
   if (rc != DGPP_OK) return rc;
   if (k_routed % 16 != 0 || stage_bytes(1, k_routed) > kMaxLdsBytes)
     return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
@@ -654,13 +685,20 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
                               const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared, int k_shared,
                               const uint8_t* sh_payload, const float* sh_scales, float* out, int out_stride, int slots,
                               int top_k, void* stream, int sh_rs, int sh_cs) {
+  return dgpp_launch_moe_slot_down_ex(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared, sh_payload,
+                                      sh_scales, out, out_stride, slots, top_k, stream, sh_rs, sh_cs, 3, nullptr, nullptr);
+}
+
+int dgpp_launch_moe_slot_down_ex(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                 const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared, int k_shared,
+                                 const uint8_t* sh_payload, const float* sh_scales, float* out, int out_stride, int slots,
+                                 int top_k, void* stream, int sh_rs, int sh_cs, int passes, const float* acc_w,
+                                 uint16_t* acc_o) {
   const char* who = "moe_slot_down";
-  const int passes = take_slot_passes();
-  const float* acc_w = nullptr;
-  uint16_t* acc_o = nullptr;
-  take_down_accum(&acc_w, &acc_o);
   if (slots <= 0) return DGPP_OK;
-  int rc = check_slot_common(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, who);
+  int rc = check_passes(passes, n_shared, acc_w, acc_o, who);
+  if (rc != DGPP_OK) return rc;
+  rc = check_slot_common(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, who);
   if (rc != DGPP_OK) return rc;
   if (k_routed % 16 != 0 || stage_bytes(1, k_routed) > kMaxLdsBytes)
     return fail_arg(std::string(who) + ": k must be a multiple of 16 (16B-aligned payloads)");
@@ -688,10 +726,24 @@ int dgpp_launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_stride, 
                                             const float* sh_up_scales, uint16_t* act, int act_stride, int slots,
                                             int top_k, float limit, void* stream, int shared_view_base, int fp4_group,
                                             int sh_rs, int sh_cs) {
+  return dgpp_launch_moe_slot_gate_up_swiglu_fp4_ex(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                                    sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act,
+                                                    act_stride, slots, top_k, limit, stream, shared_view_base, fp4_group,
+                                                    sh_rs, sh_cs, 3);
+}
+
+int dgpp_launch_moe_slot_gate_up_swiglu_fp4_ex(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                               const int32_t* order, const DgppMoeExpertView* views, int n_routed,
+                                               int k_routed, int n_shared, int k_shared, const uint8_t* sh_gate_payload,
+                                               const float* sh_gate_scales, const uint8_t* sh_up_payload,
+                                               const float* sh_up_scales, uint16_t* act, int act_stride, int slots,
+                                               int top_k, float limit, void* stream, int shared_view_base, int fp4_group,
+                                               int sh_rs, int sh_cs, int passes) {
   const char* who = "moe_slot_gate_up_fp4";
-  const int passes = take_slot_passes();
   if (slots <= 0) return DGPP_OK;
-  int rc = check_fp4_slot(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
+  int rc = check_passes(passes, n_shared, nullptr, nullptr, who);
+  if (rc != DGPP_OK) return rc;
+  rc = check_fp4_slot(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
   if (rc != DGPP_OK) return rc;
   const bool shared_fp4 = shared_view_base >= 0;
   if (n_shared > 0 && !shared_fp4 &&
@@ -723,14 +775,23 @@ int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const 
                                   int k_shared, const uint8_t* sh_payload, const float* sh_scales, float* out,
                                   int out_stride, int slots, int top_k, void* stream, int shared_view_base,
                                   int fp4_group, int sh_rs, int sh_cs, int* tile_counter) {
+  return dgpp_launch_moe_slot_down_fp4_ex(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                          sh_payload, sh_scales, out, out_stride, slots, top_k, stream, shared_view_base,
+                                          fp4_group, sh_rs, sh_cs, tile_counter, 3, nullptr, nullptr);
+}
+
+int dgpp_launch_moe_slot_down_fp4_ex(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                     const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                     int k_shared, const uint8_t* sh_payload, const float* sh_scales, float* out,
+                                     int out_stride, int slots, int top_k, void* stream, int shared_view_base,
+                                     int fp4_group, int sh_rs, int sh_cs, int* tile_counter, int passes,
+                                     const float* acc_w, uint16_t* acc_o) {
   const char* who = "moe_slot_down_fp4";
-  const int passes = take_slot_passes();
-  const float* acc_w = nullptr;
-  uint16_t* acc_o = nullptr;
-  take_down_accum(&acc_w, &acc_o);
   if (slots <= 0) return DGPP_OK;
   if (tile_counter == nullptr) return fail_arg(std::string(who) + ": the stealing counter pair is required");
-  int rc = check_fp4_slot(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
+  int rc = check_passes(passes, n_shared, acc_w, acc_o, who);
+  if (rc != DGPP_OK) return rc;
+  rc = check_fp4_slot(act, ids, views, out, n_routed, k_routed, n_shared, k_shared, shared_view_base, fp4_group, who);
   if (rc != DGPP_OK) return rc;
   const bool shared_fp4 = shared_view_base >= 0;
   if (n_shared > 0 && !shared_fp4 && (!sh_payload || !sh_scales || !fp8_shape_ok(sh_payload, k_shared)))
@@ -1074,49 +1135,47 @@ int dgpp_fp4_gemv_accepts(const DgppFp4Matrix* w) {
 int dgpp_launch_scale_gemm_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
                                 const float* w_scales, uint16_t* out, int m, int n, int k, void* stream,
                                 size_t out_row_stride_elems, int mma_from_rows, void* ws, size_t ws_bytes) {
-  (void)mma_from_rows; (void)ws; (void)ws_bytes;
   return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 0, m, n, k, stream, out_row_stride_elems, 7,
-                    7, 0, -1, false, "scale_gemm");
+                    7, 0, -1, false, "scale_gemm", mma_from_rows, ws, ws_bytes);
 }
 int dgpp_launch_scale_gemm_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
                                const float* w_scales, float* out, int m, int n, int k, void* stream,
                                size_t out_row_stride_elems, int mma_from_rows, int last_row_only, void* ws,
                                size_t ws_bytes, int compact_row) {
-  (void)mma_from_rows; (void)ws; (void)ws_bytes;
   return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 1, m, n, k, stream, out_row_stride_elems, 7,
-                    7, last_row_only, compact_row, false, "scale_gemm");
+                    7, last_row_only, compact_row, false, "scale_gemm", mma_from_rows, ws, ws_bytes);
 }
 int dgpp_launch_scale_gemm_grid_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
                                      const float* w_scales, uint16_t* out, int m, int n, int k, void* stream,
                                      size_t out_row_stride_elems, int rs, int cs, int decode_mma, void* ws,
                                      size_t ws_bytes, int prefill_tile) {
-  (void)decode_mma; (void)ws; (void)ws_bytes; (void)prefill_tile;
+  (void)decode_mma; (void)prefill_tile;
   return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 0, m, n, k, stream, out_row_stride_elems, rs,
-                    cs, 0, -1, true, "scale_gemm_grid");
+                    cs, 0, -1, true, "scale_gemm_grid", 0, ws, ws_bytes);
 }
 int dgpp_launch_scale_gemm_grid_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
                                     const float* w_scales, float* out, int m, int n, int k, void* stream,
                                     size_t out_row_stride_elems, int rs, int cs, int decode_mma, void* ws,
                                     size_t ws_bytes, int prefill_tile) {
-  (void)decode_mma; (void)ws; (void)ws_bytes; (void)prefill_tile;
+  (void)decode_mma; (void)prefill_tile;
   return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 0, out, 1, m, n, k, stream, out_row_stride_elems, rs,
-                    cs, 0, -1, true, "scale_gemm_grid");
+                    cs, 0, -1, true, "scale_gemm_grid", 0, ws, ws_bytes);
 }
 int dgpp_launch_scale_gemm_grid_e8m0_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
                                           const uint8_t* w_scales, uint16_t* out, int m, int n, int k, void* stream,
                                           size_t out_row_stride_elems, int rs, int cs, void* ws, size_t ws_bytes,
                                           int prefill_tile) {
-  (void)ws; (void)ws_bytes; (void)prefill_tile;
+  (void)prefill_tile;
   return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 1, out, 0, m, n, k, stream, out_row_stride_elems, rs,
-                    cs, 0, -1, true, "scale_gemm_grid_e8m0");
+                    cs, 0, -1, true, "scale_gemm_grid_e8m0", 0, ws, ws_bytes);
 }
 int dgpp_launch_scale_gemm_grid_e8m0_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
                                          const uint8_t* w_scales, float* out, int m, int n, int k, void* stream,
                                          size_t out_row_stride_elems, int rs, int cs, void* ws, size_t ws_bytes,
                                          int prefill_tile) {
-  (void)ws; (void)ws_bytes; (void)prefill_tile;
+  (void)prefill_tile;
   return scale_gemm(act, act_row_stride_elems, w_payload, w_scales, 1, out, 1, m, n, k, stream, out_row_stride_elems, rs,
-                    cs, 0, -1, true, "scale_gemm_grid_e8m0");
+                    cs, 0, -1, true, "scale_gemm_grid_e8m0", 0, ws, ws_bytes);
 }
 
 int dgpp_launch_scale_gemv_multi_bf16(const DgppFp8GemvProblem* problems, int n_problems, const uint16_t* act,

@@ -6,6 +6,7 @@
 #include <stdexcept>
 #include <string>
 
+#include "../../include/dgpp_amd_bench.h"
 #include "../../include/dgpp_amd_layer.h"
 
 namespace dgpp {
@@ -94,6 +95,7 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
 
   const Layout l = layout_of(cfg, max_tokens, w.shared_inter, w.views.size());
   hip_ok(hipMalloc(&arena_, l.total), "GlmMoeLayer: hipMalloc");
+  try {
   uint8_t* p = static_cast<uint8_t*>(arena_);
   auto carve = [&p](size_t bytes) {
     uint8_t* q = p;
@@ -126,14 +128,23 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
     hip_ok(hipEventCreateWithFlags(&fork_, hipEventDisableTiming), "GlmMoeLayer: event");
     hip_ok(hipEventCreateWithFlags(&join_, hipEventDisableTiming), "GlmMoeLayer: event");
   }
+  } catch (...) {   // a throwing constructor runs no destructor: give back what was taken so far
+    release();
+    throw;
+  }
 }
 
-GlmMoeLayer::~GlmMoeLayer() {
+void GlmMoeLayer::release() {
   if (join_) (void)hipEventDestroy(join_);
   if (fork_) (void)hipEventDestroy(fork_);
   if (side_) (void)hipStreamDestroy(side_);
   if (arena_) (void)hipFree(arena_);
+  join_ = fork_ = nullptr;
+  side_ = nullptr;
+  arena_ = nullptr;
 }
+
+GlmMoeLayer::~GlmMoeLayer() { release(); }
 
 // The expert-sorted slot order pays for itself once many slots share experts. A small batch (tokens * top_k <=
 // 64) skips it: the gate/up kernel finds the few sharers by ballot, the token-major down kernel needs no order,
@@ -208,92 +219,103 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   // From a few tokens on: the two cross-stream dependencies cost more than the two hand-overs they take off the
   // chain while a pass is only a few microseconds long (measured: slower at one token, level at two).
   const bool split = has_shared() && side_ != nullptr && dgpp_tune_get(9) != 1 && (tokens >= 3 || dgpp_tune_get(9) == 2);
-  if (split) {
-    hip_ok(hipEventRecord(fork_, stream), "GlmMoeLayer: fork");
-    hip_ok(hipStreamWaitEvent(side_, fork_, 0), "GlmMoeLayer: fork");
-  }
   // On one stream the shared down pass ends with the token's accumulation (no launch of its own).
   // (One token, where a launch is a fifth of the step; measured level at two tokens. Bench switch 9 = 4 folds at any
   // batch size, 3 never.)
   const bool fold_accum = has_shared() && !split && out_bf16 != nullptr && out_f32 == nullptr && dgpp_tune_get(9) != 3 &&
                           (tokens == 1 || dgpp_tune_get(9) == 4);
+  // Everything that can be refused is refused before the first enqueue.
+  if (has_shared() && out_f32 != nullptr)
+    throw std::invalid_argument("GlmMoeLayer: an unrounded output with a shared expert is not a decode form");
+  if (out_bf16 == nullptr && out_f32 == nullptr) throw std::invalid_argument("GlmMoeLayer: no output buffer");
+  // The side stream joins the caller's stream again on EVERY way out of this function (a launcher that throws
+  // between fork and join must not leave a captured graph with an unjoined branch).
+  struct Fork {
+    hipStream_t main, side;
+    hipEvent_t join;
+    bool open = false;
+    void close_quietly() {
+      if (!open) return;
+      open = false;
+      if (hipEventRecord(join, side) == hipSuccess) (void)hipStreamWaitEvent(main, join, 0);
+    }
+    ~Fork() { close_quietly(); }
+  } fork{stream, side_, join_};
+  if (split) {
+    hip_ok(hipEventRecord(fork_, stream), "GlmMoeLayer: fork");
+    hip_ok(hipStreamWaitEvent(side_, fork_, 0), "GlmMoeLayer: fork");
+    fork.open = true;
+  }
+  // One launcher call per pass and stream: the routed pass on the caller's stream, the shared pass beside it.
   auto for_passes = [&](auto&& call) {
-    if (!split) return call(stream);
-    moe_slot_passes(1);
-    call(stream);
-    moe_slot_passes(2);
-    call(side_);
+    if (!split) return call(stream, 3);
+    call(stream, 1);
+    call(side_, 2);
   };
+  const float* fold_w = fold_accum ? weights : nullptr;
+  uint16_t* fold_o = fold_accum ? out_bf16 : nullptr;
   if (w_.format == GlmExpertFormat::Fp8) {
     if (fused) {
       launch_moe_select_gate_up_swiglu(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
                                        d_slot_act_, max_inter_, cfg_.swiglu_limit, stream);
-      if (has_shared()) {   // the shared slot's pass: the launcher's own, the routed pass already done above
-        moe_slot_passes(2);
-        launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
-                                       w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
-                                       K, cfg_.swiglu_limit, split ? side_ : stream, w_.sh_rs, w_.sh_cs);
-      }
+      if (has_shared())   // the shared slot's pass: the routed pass already ran above
+        launch_moe_slot_gate_up_swiglu_ex(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
+                                          w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
+                                          K, cfg_.swiglu_limit, split ? side_ : stream, w_.sh_rs, w_.sh_cs, 2);
     } else
-      for_passes([&](hipStream_t st) {
-        launch_moe_slot_gate_up_swiglu(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
-                                       w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
-                                       K, cfg_.swiglu_limit, st, w_.sh_rs, w_.sh_cs);
+      for_passes([&](hipStream_t st, int passes) {
+        launch_moe_slot_gate_up_swiglu_ex(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
+                                          w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
+                                          K, cfg_.swiglu_limit, st, w_.sh_rs, w_.sh_cs, passes);
       });
     if (token_major) {   // routed only: down + accumulation in one token-major launch
       launch_moe_slot_down_accum(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                  out_bf16, out_f32, stream);
       return;
     }
-    if (fold_accum) moe_slot_down_accum_into(weights, out_bf16);
-    for_passes([&](hipStream_t st) {
-      launch_moe_slot_down(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
-                           n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, st, w_.sh_rs, w_.sh_cs);
+    for_passes([&](hipStream_t st, int passes) {
+      launch_moe_slot_down_ex(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
+                              n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, st, w_.sh_rs, w_.sh_cs,
+                              passes, fold_w, fold_o);
     });
   } else {
     const int base = w_.shared_in_table ? cfg_.n_experts * 3 : -1;
     if (fused) {
       launch_moe_select_gate_up_swiglu_fp4(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I,
                                            H, d_slot_act_, max_inter_, cfg_.swiglu_limit, stream, fp4_group_);
-      if (has_shared()) {
-        moe_slot_passes(2);
-        launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
-                                           sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
-                                           sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
-                                           d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, split ? side_ : stream, base,
-                                           fp4_group_, w_.sh_rs, w_.sh_cs);
-      }
+      if (has_shared())
+        launch_moe_slot_gate_up_swiglu_fp4_ex(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
+                                              sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
+                                              sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
+                                              d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, split ? side_ : stream,
+                                              base, fp4_group_, w_.sh_rs, w_.sh_cs, 2);
     } else
-      for_passes([&](hipStream_t st) {
-        launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
-                                           sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
-                                           sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
-                                           d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, st, base, fp4_group_,
-                                           w_.sh_rs, w_.sh_cs);
+      for_passes([&](hipStream_t st, int passes) {
+        launch_moe_slot_gate_up_swiglu_fp4_ex(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
+                                              sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
+                                              sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
+                                              d_slot_act_, max_inter_, slots, K, cfg_.swiglu_limit, st, base, fp4_group_,
+                                              w_.sh_rs, w_.sh_cs, passes);
       });
     if (token_major) {
       launch_moe_slot_down_accum_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, d_views_, H, I, tokens, K, weights,
                                      out_bf16, out_f32, stream, fp4_group_);
       return;
     }
-    if (fold_accum) moe_slot_down_accum_into(weights, out_bf16);
-    for_passes([&](hipStream_t st) {
-      launch_moe_slot_down_fp4(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
-                               has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
-                               sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, st, base, fp4_group_,
-                               w_.sh_rs, w_.sh_cs, d_tile_counter_);
+    for_passes([&](hipStream_t st, int passes) {
+      launch_moe_slot_down_fp4_ex(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
+                                  has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
+                                  sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, st, base, fp4_group_,
+                                  w_.sh_rs, w_.sh_cs, d_tile_counter_, passes, fold_w, fold_o);
     });
   }
-  if (split) {
+  if (fork.open) {
+    fork.open = false;
     hip_ok(hipEventRecord(join_, side_), "GlmMoeLayer: join");
     hip_ok(hipStreamWaitEvent(stream, join_, 0), "GlmMoeLayer: join");
   }
   if (fold_accum) return;
   if (has_shared()) {
-    if (out_f32) {
-      // The shared chain, unrounded: the ordered form over the slot layout's rows.
-      throw std::invalid_argument("GlmMoeLayer: an unrounded output with a shared expert is not a decode form");
-    }
     launch_moe_slot_accum(out_bf16, d_slot_down_, weights, tokens, H, K, stream);
   } else if (out_f32) {
     launch_moe_slot_accum_routed_f32(out_f32, d_slot_down_, weights, tokens, H, K, stream);

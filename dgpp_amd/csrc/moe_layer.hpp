@@ -58,6 +58,7 @@ class GlmMoeLayer {
   bool has_shared() const { return w_.shared_inter > 0; }
 
  private:
+  void release();
   void check_tokens(int tokens) const;
   bool needs_order(int tokens) const;
   void expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,

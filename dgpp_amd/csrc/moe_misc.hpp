@@ -1,4 +1,5 @@
-// Host entry points of the router / grouping / elementwise kernels (moe_misc.hip). Arguments are
+// Host entry points of the router (moe_router.hip), grouping (moe_grouping.hip) and elementwise / accumulation
+// (moe_elementwise.hip) kernels. Arguments are
 // validated by the C ABI layer; these only pick grids and launch.
 #pragma once
 
@@ -38,6 +39,8 @@ hipError_t run_tile_list(const DgppMoeSegment* segs, int n_segs, int tile_rows, 
 hipError_t run_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* output, int experts, int capacity,
                                 hipStream_t stream);
 hipError_t run_probe_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
+// sink: at least 8192 words, never written in practice (keeps the loads alive)
+hipError_t run_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, hipStream_t stream);
 hipError_t run_fp8_dequant(const uint8_t* payload, const void* scales, int e8m0, uint16_t* out, int64_t rows,
                            int64_t cols, int rs, int cs, hipStream_t stream);
 

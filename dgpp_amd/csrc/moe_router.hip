@@ -1,0 +1,202 @@
+// The MoE router: score rows (one dot product per expert and token) and the top-k selection, alone or
+// together with the decode slots' expert order.
+//
+// Reference counterparts in src/kernels/glm_moe.cu: router dots :86-196, selection :211-329, slot order :465-517.
+// Ids given the scores are a bit-exact contract; the weights are fp32 chains in a defined order.
+#include <hip/hip_runtime.h>
+#include <limits.h>
+#include <stdint.h>
+
+#include "../../include/dgpp_amd.h"
+#include "moe_misc.hpp"
+#include "moe_rank.hpp"
+#include "numerics.hpp"
+#include "router_select.hpp"
+
+namespace dgpp_amd {
+namespace {
+
+using rsel::kWaveSize;
+using rsel::select_token;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+// ---- router ---------------------------------------------------------------------------------
+// One wavefront per (expert, token): lanes stride the hidden vector in 16-byte vectors, each
+// lane an fp32 fma chain in k order, then the butterfly.
+constexpr int kRouterWaves = 4;
+
+template <int kMode>
+__global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_kernel(
+    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ gate, const float* __restrict__ bias,
+    float* __restrict__ scores, float* __restrict__ biased, int tokens, int hidden_dim, int n_experts,
+    int vector_loads) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int e = blockIdx.x * kRouterWaves + wave;
+  const int t = blockIdx.y;
+  if (e >= n_experts || t >= tokens) return;
+  const uint16_t* x = hidden + static_cast<size_t>(t) * hidden_dim;
+  const uint16_t* w = gate + static_cast<size_t>(e) * hidden_dim;
+  float dot = 0.f;
+  if (vector_loads) {
+    const int vecs = hidden_dim / 8;
+    for (int v = lane; v < vecs; v += kWaveSize) {
+      const uint4 xv = reinterpret_cast<const uint4*>(x)[v];
+      const uint4 wv = reinterpret_cast<const uint4*>(w)[v];
+      const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, ww[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        dot = fmaf(bits_f32(xw[q] << 16), bits_f32(ww[q] << 16), dot);
+        dot = fmaf(bits_f32(xw[q] & 0xFFFF0000u), bits_f32(ww[q] & 0xFFFF0000u), dot);
+      }
+    }
+  } else {
+    for (int k = lane; k < hidden_dim; k += kWaveSize) dot = fmaf(bf16_to_f32(x[k]), bf16_to_f32(w[k]), dot);
+  }
+  dot = wave_sum(dot);
+  if (lane != 0) return;
+  const size_t at = static_cast<size_t>(t) * n_experts + e;
+  if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
+    const float l = bf16_to_f32(f32_to_bf16(dot));
+    scores[at] = l;
+    biased[at] = l;
+  } else {
+    float sc;
+    if (kMode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS)
+      sc = sqrtf(dot > 20.f ? dot : log1pf(expf(dot)));
+    else
+      sc = 1.0f / (1.0f + expf(-dot));
+    scores[at] = sc;
+    biased[at] = sc + bias[e];
+  }
+}
+
+// One wavefront per token, the whole score row in registers (router_select.hpp): 64 * PER_LANE experts.
+template <int kMode, int PER_LANE>
+__global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
+    const float* __restrict__ scores, const float* __restrict__ biased, int32_t* __restrict__ ids,
+    float* __restrict__ weights, int tokens, int n_experts, int top_k, float scaling, int norm_topk) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  if (t >= tokens) return;
+  const size_t row = static_cast<size_t>(t) * n_experts;
+  int id;
+  float w;
+  select_token<kMode, PER_LANE>(scores + row, biased + row, n_experts, top_k, scaling, norm_topk, lane, id, w);
+  if (lane < top_k) {
+    ids[static_cast<size_t>(t) * top_k + lane] = id;
+    weights[static_cast<size_t>(t) * top_k + lane] = w;
+  }
+}
+
+// Selection and slot order in ONE launch for a decode batch: one wavefront per token selects, the
+// block then ranks the slots by (expert, slot) exactly as slot_order_kernel does (key = expert id,
+// or n_experts for the token's shared slot). tokens * 64 threads, tokens <= 16.
+template <int kMode, int PER_LANE>
+__global__ __launch_bounds__(1024) void router_select_order_kernel(
+    const float* __restrict__ scores, const float* __restrict__ biased, int32_t* __restrict__ ids,
+    float* __restrict__ weights, int32_t* __restrict__ order, int tokens, int n_experts, int top_k, float scaling,
+    int norm_topk, int shared_early) {
+  __shared__ __align__(16) int32_t keys[16 * 17 + 4];
+  const int t = threadIdx.x >> 6, lane = threadIdx.x & (kWaveSize - 1);
+  const size_t row = static_cast<size_t>(t) * n_experts;
+  int id;
+  float w;
+  select_token<kMode, PER_LANE>(scores + row, biased + row, n_experts, top_k, scaling, norm_topk, lane, id, w);
+  if (lane < top_k) {
+    ids[static_cast<size_t>(t) * top_k + lane] = id;
+    weights[static_cast<size_t>(t) * top_k + lane] = w;
+    keys[t * (top_k + 1) + lane] = slot_sort_key(id, t * (top_k + 1) + lane);
+  } else if (lane == top_k) {
+    keys[t * (top_k + 1) + lane] = slot_sort_key(n_experts, t * (top_k + 1) + lane);
+  }
+  if (order == nullptr) return;
+  const int slots = tokens * (top_k + 1);
+  const int padded = (slots + 3) & ~3;
+  if (threadIdx.x < padded - slots) keys[slots + threadIdx.x] = INT_MAX;
+  __syncthreads();
+  const int s = threadIdx.x;
+  if (s >= slots) return;
+  int pos = slot_rank(keys, padded, keys[s]);
+  if (shared_early) {
+    const int routed = tokens * top_k;
+    pos = pos < routed ? pos + (pos < tokens ? pos : tokens) : 2 * (pos - routed) + 1;
+  }
+  order[pos] = s;
+}
+
+}  // namespace
+
+hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
+                           float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream) {
+  const int vec = (hidden_dim % 8 == 0) && ((reinterpret_cast<uintptr_t>(hidden) & 15u) == 0) &&
+                  ((reinterpret_cast<uintptr_t>(gate) & 15u) == 0);
+  const dim3 grid((n_experts + kRouterWaves - 1) / kRouterWaves, tokens);
+  const dim3 block(kRouterWaves * kWaveSize);
+  if (mode == DGPP_ROUTER_SOFTMAX_TOPK)
+    hipLaunchKernelGGL(router_dots_kernel<DGPP_ROUTER_SOFTMAX_TOPK>, grid, block, 0, stream, hidden, gate, bias, scores,
+                       biased, tokens, hidden_dim, n_experts, vec);
+  else if (mode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS)
+    hipLaunchKernelGGL(router_dots_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS>, grid, block, 0, stream, hidden, gate, bias,
+                       scores, biased, tokens, hidden_dim, n_experts, vec);
+  else
+    hipLaunchKernelGGL(router_dots_kernel<DGPP_ROUTER_SIGMOID_BIAS>, grid, block, 0, stream, hidden, gate, bias, scores,
+                       biased, tokens, hidden_dim, n_experts, vec);
+  return hipGetLastError();
+}
+
+// PER_LANE for a row of n_experts (<= 4096, the configuration's limit): the smallest power of two that holds it.
+template <int kMode, int PER_LANE>
+static void launch_select_reg(const float* scores, const float* biased, int32_t* ids, float* weights, int tokens,
+                              int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream) {
+  hipLaunchKernelGGL((router_select_reg_kernel<kMode, PER_LANE>), dim3(tokens), dim3(kWaveSize), 0, stream, scores, biased,
+                     ids, weights, tokens, n_experts, top_k, scaling, norm_topk);
+}
+template <int kMode>
+static void launch_select_mode(const float* scores, const float* biased, int32_t* ids, float* weights, int tokens,
+                               int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream) {
+  const int per_lane = (n_experts + kWaveSize - 1) / kWaveSize;
+  if (per_lane <= 4) launch_select_reg<kMode, 4>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+  else if (per_lane <= 8) launch_select_reg<kMode, 8>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+  else if (per_lane <= 16) launch_select_reg<kMode, 16>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+  else if (per_lane <= 32) launch_select_reg<kMode, 32>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+  else launch_select_reg<kMode, 64>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+}
+
+hipError_t run_router_select(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
+                             int tokens, int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream) {
+  if (n_experts > 64 * kWaveSize) return hipErrorInvalidValue;   // the configuration check stops at 4096 experts
+  if (mode == DGPP_ROUTER_SOFTMAX_TOPK)
+    launch_select_mode<DGPP_ROUTER_SOFTMAX_TOPK>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+  else
+    launch_select_mode<DGPP_ROUTER_SIGMOID_BIAS>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+  return hipGetLastError();
+}
+
+hipError_t run_router_select_order(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
+                                   int32_t* order, int tokens, int n_experts, int top_k, float scaling, int norm_topk,
+                                   int shared_early, hipStream_t stream) {
+  const bool softmax = mode == DGPP_ROUTER_SOFTMAX_TOPK;
+  const dim3 grid(1), block(tokens * kWaveSize);
+  if (n_experts <= 4 * kWaveSize) {
+    if (softmax)
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 4>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
+    else
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SIGMOID_BIAS, 4>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
+  } else {
+    if (softmax)
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 8>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
+    else
+      hipLaunchKernelGGL((router_select_order_kernel<DGPP_ROUTER_SIGMOID_BIAS, 8>), grid, block, 0, stream, scores,
+                         biased, ids, weights, order, tokens, n_experts, top_k, scaling, norm_topk, shared_early);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace dgpp_amd

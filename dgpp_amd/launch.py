@@ -214,6 +214,45 @@ def launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_rou
         _p(tile_counter)))
 
 
+def launch_moe_slot_gate_up_swiglu_ex(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                      sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride,
+                                      slots, top_k, limit, stream=None, sh_rs=7, sh_cs=7, passes=3):
+    """Extension: the launcher above with the pass selector as an argument (1 routed, 2 shared, 3 both)."""
+    _check(_lib.load().dgpp_launch_moe_slot_gate_up_swiglu_ex(
+        _p(x), x_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_gate_payload),
+        _p(sh_gate_scales), _p(sh_up_payload), _p(sh_up_scales), _p(act), act_stride, slots, top_k, limit,
+        _stream(stream), sh_rs, sh_cs, passes))
+
+
+def launch_moe_slot_down_ex(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared, sh_payload,
+                            sh_scales, out, out_stride, slots, top_k, stream=None, sh_rs=7, sh_cs=7, passes=3,
+                            acc_weights=None, acc_out=None):
+    """Extension: pass selector, and the accumulation the shared pass ends with (both or neither of acc_*)."""
+    _check(_lib.load().dgpp_launch_moe_slot_down_ex(
+        _p(act), act_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_payload),
+        _p(sh_scales), _p(out), out_stride, slots, top_k, _stream(stream), sh_rs, sh_cs, passes, _p(acc_weights),
+        _p(acc_out)))
+
+
+def launch_moe_slot_gate_up_swiglu_fp4_ex(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                          sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride,
+                                          slots, top_k, limit, stream=None, shared_view_base=-1, fp4_group=16, sh_rs=7,
+                                          sh_cs=7, passes=3):
+    _check(_lib.load().dgpp_launch_moe_slot_gate_up_swiglu_fp4_ex(
+        _p(x), x_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_gate_payload),
+        _p(sh_gate_scales), _p(sh_up_payload), _p(sh_up_scales), _p(act), act_stride, slots, top_k, limit,
+        _stream(stream), shared_view_base, fp4_group, sh_rs, sh_cs, passes))
+
+
+def launch_moe_slot_down_fp4_ex(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared, sh_payload,
+                                sh_scales, out, out_stride, slots, top_k, stream=None, shared_view_base=-1, fp4_group=16,
+                                sh_rs=7, sh_cs=7, tile_counter=None, passes=3, acc_weights=None, acc_out=None):
+    _check(_lib.load().dgpp_launch_moe_slot_down_fp4_ex(
+        _p(act), act_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_payload),
+        _p(sh_scales), _p(out), out_stride, slots, top_k, _stream(stream), shared_view_base, fp4_group, sh_rs, sh_cs,
+        _p(tile_counter), passes, _p(acc_weights), _p(acc_out)))
+
+
 def launch_moe_slot_down_accum(act, act_stride, ids, views, n, k, tokens, top_k, weights, out_bf16, out_f32, stream=None):
     """Extension: routed down rows + the ordered accumulation in one token-major launch (FP8 experts)."""
     _check(_lib.load().dgpp_launch_moe_slot_down_accum(_p(act), act_stride, _p(ids), _p(views), n, k, tokens, top_k,

@@ -36,31 +36,6 @@ const char* dgpp_last_error(void);
 /* "gfx950" — the only architecture the library carries code for. */
 const char* dgpp_target_arch(void);
 
-/* Bench A/B switches, process-wide, not thread-safe against concurrent launches (the reference
- * keeps such a switch in its launcher header too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90).
- * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: slots of one expert a
- * decode-slot block serves together (0 = default: 2 gate/up, 4 down; 1 = one slot per block);
- * key 2: row steps per block of the slot launches (0 = automatic); key 3: 1 stages activations before
- * any weight load is issued (default: activation loads, first weight pass, LDS commit); key 4: 1 keeps
- * the layer driver on the two-launch down + accumulate form; key 5: 2 moves the GEMV launchers to the
- * matrix-core form; key 6: 1 makes the layer driver compute the slot order for small decode batches too
- * (default: batches of at most 128 routed slots find the sharers of an expert by ballot, no order);
- * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
- * blocks, dgpp_launch_moe_select_gate_up_swiglu); key 9: 1 keeps the shared expert's passes of the layer driver
- * on the caller's stream, 2 moves them to a second stream beside the routed passes at every batch size (default:
- * from three tokens on); 3 and 4 keep one stream and never / always fold the accumulation into the shared down pass
- * (default: at one token). Outputs do not depend on keys
- * 1 - 4, 6, 7 and 9; keys 0 and
- * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
- * bitwise twins of each other). */
-void dgpp_tune_set(int key, int value);
-int dgpp_tune_get(int key);
-
-/* Measurement aid with no counterpart in the reference: a plain streaming copy of `bytes`
- * (a multiple of 16; both pointers 16-byte aligned) on `stream`. A profiler's HBM byte counters
- * are calibrated against it: it reads `bytes` and writes `bytes`, nothing else. */
-int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
-
 /* ---- POD types shared with device code -------------------------------------------------- */
 
 /* Device-side expert table entry, read by the slot and grouped kernels.
@@ -221,19 +196,47 @@ int dgpp_launch_moe_slot_down(const uint16_t* act, size_t act_stride, const int3
                               const float* sh_scales, float* out, int out_stride, int slots,
                               int top_k, void* stream, int sh_rs, int sh_cs);
 
-/* Extension (no counterpart in the reference): the four decode-slot launchers above and below (gate/up and down,
+/* Extensions (no counterpart in the reference): the four decode-slot launchers above and below (gate/up and down,
  * FP8 and FP4) run a routed pass and, with n_shared > 0, a shared pass: two launches that touch disjoint slot rows.
- * This call selects which of them the NEXT such launcher call of the calling thread runs - 1 the routed pass, 2 the
- * shared pass, 3 both (the default, restored after that one call) - so that a host can put the shared expert's
- * passes on a second stream beside the routed ones. Same arguments, same checks, same bits per pass. */
-void dgpp_moe_slot_passes(int passes);
-/* Extension (no counterpart in the reference): the NEXT dgpp_launch_moe_slot_down / _fp4 call of the calling thread
- * folds dgpp_launch_moe_slot_accum into its shared pass. `out` of that call must hold the routed slots' finished rows
- * by the time the shared pass runs (the same call's routed pass, or an earlier one on the stream); the shared pass then
- * stores no slot row but the token's accumulated row - a = 0; a = fma(weights[t, j], out[slot j], a) for j ascending;
- * a = fma(1, shared dot, a); one rounding - to out_bf16 [tokens, n_shared]. Same bits as the two launches. One call
- * consumes the setting; a null argument clears it. */
-void dgpp_moe_slot_down_accum_into(const float* weights, uint16_t* out_bf16);
+ * The *_ex forms take the reference launcher's arguments unchanged and then
+ *   passes       1 the routed pass, 2 the shared pass, 3 both (what the plain launcher runs), so that a host can put
+ *                the shared expert's passes on a second stream beside the routed ones; same checks, same bits per pass;
+ *   acc_weights, acc_out (down launchers only, both or neither): the shared pass ends with the token's accumulation
+ *                instead of a dgpp_launch_moe_slot_accum launch. `out` must hold the routed slots' finished rows by the
+ *                time the shared pass runs (the same call's routed pass, or an earlier one on the stream); the shared
+ *                pass then stores no slot row but the token's row - a = 0; a = fma(acc_weights[t, j], out[slot j], a)
+ *                for j ascending; a = fma(1, shared dot, a); one rounding - to acc_out [tokens, n_shared] (bf16).
+ *                Same bits as the two launches.
+ * A request that cannot be honoured is DGPP_INVALID_ARGUMENT and nothing is launched: passes outside 1..3, the shared
+ * pass alone without a shared expert, an accumulation without the shared pass that would write it. */
+int dgpp_launch_moe_slot_gate_up_swiglu_ex(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                           const int32_t* order, const DgppMoeExpertView* views,
+                                           int n_routed, int k_routed, int n_shared, int k_shared,
+                                           const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                           const uint8_t* sh_up_payload, const float* sh_up_scales,
+                                           uint16_t* act, int act_stride, int slots, int top_k,
+                                           float limit, void* stream, int sh_rs, int sh_cs, int passes);
+int dgpp_launch_moe_slot_down_ex(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                 const int32_t* order, const DgppMoeExpertView* views, int n_routed,
+                                 int k_routed, int n_shared, int k_shared, const uint8_t* sh_payload,
+                                 const float* sh_scales, float* out, int out_stride, int slots,
+                                 int top_k, void* stream, int sh_rs, int sh_cs, int passes,
+                                 const float* acc_weights, uint16_t* acc_out);
+int dgpp_launch_moe_slot_gate_up_swiglu_fp4_ex(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                               const int32_t* order, const DgppMoeExpertView* views,
+                                               int n_routed, int k_routed, int n_shared, int k_shared,
+                                               const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                               const uint8_t* sh_up_payload, const float* sh_up_scales,
+                                               uint16_t* act, int act_stride, int slots, int top_k,
+                                               float limit, void* stream, int shared_view_base,
+                                               int fp4_group, int sh_rs, int sh_cs, int passes);
+int dgpp_launch_moe_slot_down_fp4_ex(const uint16_t* act, size_t act_stride, const int32_t* ids,
+                                     const int32_t* order, const DgppMoeExpertView* views, int n_routed,
+                                     int k_routed, int n_shared, int k_shared, const uint8_t* sh_payload,
+                                     const float* sh_scales, float* out, int out_stride, int slots,
+                                     int top_k, void* stream, int shared_view_base, int fp4_group,
+                                     int sh_rs, int sh_cs, int* tile_counter, int passes,
+                                     const float* acc_weights, uint16_t* acc_out);
 
 /* Extension (no counterpart in the reference): dgpp_launch_moe_router_select followed by the routed pass of
  * dgpp_launch_moe_slot_gate_up_swiglu / _fp4 (order == NULL, no shared expert; slots = tokens * (top_k + 1)),
@@ -390,7 +393,11 @@ int dgpp_launch_moe_grouped_mma_fp4_f32(const uint16_t* act, size_t act_stride, 
                                         float* out, size_t out_stride, int n, int k, void* stream, const int32_t* act_rows,
                                         int fp4_group, int tile_rows);
 
-/* src/kernels/fp4_gemv.hpp:23-32. `w` is a HOST struct holding device pointers. */
+/* src/kernels/fp4_gemv.hpp:23-32. `w` is a HOST struct holding device pointers.
+ * Row-count dispatch: up to 4 rows ride the vector-core GEMV (one weight pass); from 5 rows on the call runs the
+ * matrix-core form (16 rows per weight pass), as the reference moves to its tensor-core form as m grows
+ * (src/kernels/glm_moe_launch.hpp:363). The two forms sum in different fp32 orders: a row's bits depend on which side
+ * of the boundary the call's m lies (never on m otherwise); both are held to the same oracle tolerance. */
 int dgpp_launch_fp4_gemv_bf16(const uint16_t* act, size_t act_row_stride_elems,
                               const DgppFp4Matrix* w, uint16_t* out, int m, int n, int k,
                               void* stream);
@@ -400,8 +407,13 @@ int dgpp_launch_fp4_gemv_f32(const uint16_t* act, size_t act_row_stride_elems,
 int dgpp_fp4_gemv_accepts(const DgppFp4Matrix* w);
 
 /* ---- dense FP8 block-scaled projection GEMV ------------------------------------------------------------ */
-/* src/kernels/scale_gemm.hpp:57-79. mma_from_rows, ws and ws_bytes are accepted for signature
- * parity; every m takes the row-independent GEMV form here. */
+/* src/kernels/scale_gemm.hpp:57-79. Row-count dispatch (reference: src/kernels/scale_gemm.cu:296-339): up to 8 rows
+ * ride the vector-core GEMV in one weight pass; from 9 rows on - or from mma_from_rows on when the caller gives a
+ * smaller positive bound - the call runs the matrix-core form (16 rows per weight pass), which uses `ws` / `ws_bytes`
+ * (nullable; parts(k) * m * n floats) to split K over blocks when the unsplit grid would leave the chip under-filled.
+ * Split and unsplit give the same bits; the two cores sum in different fp32 orders (both held to the same oracle
+ * tolerance), so a row's bits depend on which side of the boundary the call's m lies, never on m otherwise.
+ * last_row_only / compact_row compute one row and stay on the vector core. */
 int dgpp_launch_scale_gemm_bf16(const uint16_t* act, size_t act_row_stride_elems,
                                 const uint8_t* w_payload, const float* w_scales, uint16_t* out,
                                 int m, int n, int k, void* stream, size_t out_row_stride_elems,
@@ -411,7 +423,8 @@ int dgpp_launch_scale_gemm_f32(const uint16_t* act, size_t act_row_stride_elems,
                                int n, int k, void* stream, size_t out_row_stride_elems,
                                int mma_from_rows, int last_row_only, void* ws, size_t ws_bytes,
                                int compact_row);
-/* src/kernels/scale_gemm.hpp:140-149 (decode_mma / ws / prefill_tile accepted, GEMV form). */
+/* src/kernels/scale_gemm.hpp:140-149: the same on a stated scale grid; the matrix-core form from 9 rows on (ws as
+ * above; decode_mma and prefill_tile are the reference's tuning hints and are accepted unused). */
 int dgpp_launch_scale_gemm_grid_bf16(const uint16_t* act, size_t act_row_stride_elems,
                                      const uint8_t* w_payload, const float* w_scales, uint16_t* out,
                                      int m, int n, int k, void* stream,

@@ -132,12 +132,6 @@ inline void launch_moe_router_dots(const uint16_t* hidden, const uint16_t* gate,
   const DgppMoeConfig c = cfg.c_config();
   detail::check(dgpp_launch_moe_router_dots(hidden, gate, bias, scores, biased, &c, tokens, stream));
 }
-// Extension: which passes the next decode-slot launcher call of this thread runs (see dgpp_amd.h).
-inline void moe_slot_passes(int passes) { dgpp_moe_slot_passes(passes); }
-// Extension: the next slot-down call's shared pass ends with the token's accumulation (see dgpp_amd.h).
-inline void moe_slot_down_accum_into(const float* weights, uint16_t* out_bf16) {
-  dgpp_moe_slot_down_accum_into(weights, out_bf16);
-}
 // Extension: selection + routed gate/up in one launch (see dgpp_amd.h).
 inline void launch_moe_select_gate_up_swiglu(const float* scores, const float* biased, int32_t* ids, float* weights,
                                              const GlmMoeConfig& cfg, int tokens, const uint16_t* x, size_t x_stride,
@@ -251,6 +245,50 @@ inline void launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, con
   detail::check(dgpp_launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_routed, n_shared,
                                               k_shared, sh_payload, sh_scales, out, out_stride, slots, top_k, stream,
                                               shared_view_base, fp4_group, sh_rs, sh_cs, tile_counter));
+}
+// Extensions: the four decode-slot launchers with the pass selector (1 routed, 2 shared, 3 both) and, for the down
+// launchers, the accumulation the shared pass ends with, as trailing arguments (see dgpp_amd.h).
+inline void launch_moe_slot_gate_up_swiglu_ex(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                                              const MoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                              int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                              const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                              int act_stride, int slots, int top_k, float limit, hipStream_t stream,
+                                              int sh_rs, int sh_cs, int passes) {
+  detail::check(dgpp_launch_moe_slot_gate_up_swiglu_ex(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                                       sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act,
+                                                       act_stride, slots, top_k, limit, stream, sh_rs, sh_cs, passes));
+}
+inline void launch_moe_slot_down_ex(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                    const MoeExpertView* views, int n_routed, int k_routed, int n_shared, int k_shared,
+                                    const uint8_t* sh_payload, const float* sh_scales, float* out, int out_stride,
+                                    int slots, int top_k, hipStream_t stream, int sh_rs, int sh_cs, int passes,
+                                    const float* acc_weights, uint16_t* acc_out) {
+  detail::check(dgpp_launch_moe_slot_down_ex(act, act_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                             sh_payload, sh_scales, out, out_stride, slots, top_k, stream, sh_rs, sh_cs,
+                                             passes, acc_weights, acc_out));
+}
+inline void launch_moe_slot_gate_up_swiglu_fp4_ex(const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                                  const int32_t* order, const MoeExpertView* views, int n_routed,
+                                                  int k_routed, int n_shared, int k_shared,
+                                                  const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                                  const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                                  int act_stride, int slots, int top_k, float limit, hipStream_t stream,
+                                                  int shared_view_base, int fp4_group, int sh_rs, int sh_cs, int passes) {
+  detail::check(dgpp_launch_moe_slot_gate_up_swiglu_fp4_ex(x, x_stride, ids, order, views, n_routed, k_routed, n_shared,
+                                                           k_shared, sh_gate_payload, sh_gate_scales, sh_up_payload,
+                                                           sh_up_scales, act, act_stride, slots, top_k, limit, stream,
+                                                           shared_view_base, fp4_group, sh_rs, sh_cs, passes));
+}
+inline void launch_moe_slot_down_fp4_ex(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
+                                        const MoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                        int k_shared, const uint8_t* sh_payload, const float* sh_scales, float* out,
+                                        int out_stride, int slots, int top_k, hipStream_t stream, int shared_view_base,
+                                        int fp4_group, int sh_rs, int sh_cs, int* tile_counter, int passes,
+                                        const float* acc_weights, uint16_t* acc_out) {
+  detail::check(dgpp_launch_moe_slot_down_fp4_ex(act, act_stride, ids, order, views, n_routed, k_routed, n_shared,
+                                                 k_shared, sh_payload, sh_scales, out, out_stride, slots, top_k, stream,
+                                                 shared_view_base, fp4_group, sh_rs, sh_cs, tile_counter, passes,
+                                                 acc_weights, acc_out));
 }
 // Extensions: routed down rows + ordered accumulation in one token-major launch (see dgpp_amd.h).
 inline void launch_moe_slot_down_accum(const uint16_t* act, size_t act_stride, const int32_t* ids,

@@ -1,0 +1,49 @@
+/* Measurement aids of libdgpp_amd.so: A/B switches and streaming probes used by the benchmark and by the tests that
+ * compare kernel forms. Nothing here is part of the drop-in launcher surface (dgpp_amd.h does not include this
+ * file) and no product caller needs it. */
+#ifndef DGPP_AMD_BENCH_H
+#define DGPP_AMD_BENCH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Bench A/B switches, process-wide, not thread-safe against concurrent launches (the reference
+ * keeps such a switch in its launcher header too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90).
+ * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: slots of one expert a
+ * decode-slot block serves together (0 = default: 2 gate/up, 4 down; 1 = one slot per block);
+ * key 2: row steps per block of the slot launches (0 = automatic); key 3: 1 stages activations before
+ * any weight load is issued (default: activation loads, first weight pass, LDS commit); key 4: 1 keeps
+ * the layer driver on the two-launch down + accumulate form; key 5: 2 moves every GEMV launcher to the
+ * matrix-core form, 1 keeps the dense launchers on the vector core at every row count (default: the dense launchers
+ * move to the matrix core from 5 rows (FP4) / 9 rows (FP8) on); key 6: 1 makes the layer driver compute the slot order for small decode batches too
+ * (default: batches of at most 128 routed slots find the sharers of an expert by ballot, no order);
+ * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
+ * blocks, dgpp_launch_moe_select_gate_up_swiglu); key 9: 1 keeps the shared expert's passes of the layer driver
+ * on the caller's stream, 2 moves them to a second stream beside the routed passes at every batch size (default:
+ * from three tokens on); 3 and 4 keep one stream and never / always fold the accumulation into the shared down pass
+ * (default: at one token). Outputs do not depend on keys
+ * 1 - 4, 6, 7 and 9; keys 0 and
+ * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
+ * bitwise twins of each other). */
+void dgpp_tune_set(int key, int value);
+int dgpp_tune_get(int key);
+
+/* Measurement aid with no counterpart in the reference: a plain streaming copy of `bytes`
+ * (a multiple of 16; both pointers 16-byte aligned) on `stream`. A profiler's HBM byte counters
+ * are calibrated against it: it reads `bytes` and writes `bytes`, nothing else. */
+int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
+
+/* A plain streaming READ of `bytes` (a multiple of 16, 16-byte aligned) on `stream`: 16-byte loads, four in flight
+ * per lane, nothing stored (`sink`, at least 8192 words, is written only for a checksum no input produces). The rate
+ * it reaches is the ceiling of a weight stream on this chip; nontemporal != 0 uses the nontemporal load form the
+ * GEMV kernels use where a launch reads its weights once. */
+int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -23,6 +23,10 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} is declared in include/dgpp_amd.h but not exported"
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert set(_lib.SIGNATURES) == set(names)
+    bench = declared_symbols("dgpp_amd_bench.h")
+    assert set(bench) == set(_lib.BENCH_SIGNATURES) and not set(bench) & set(names)
+    for n in bench:
+        assert hasattr(lib, n), f"{n} is declared in include/dgpp_amd_bench.h but not exported"
     layer = declared_symbols("dgpp_amd_layer.h")
     assert set(layer) == set(_lib.LAYER_SIGNATURES)
     for n in layer:
@@ -76,7 +80,7 @@ def test_headers_compile_as_c_and_the_shim_as_cpp(tmp_path):
     root = Path(__file__).resolve().parent.parent
     inc = root / "include"
     c_src = tmp_path / "c_check.c"
-    c_src.write_text('#include "dgpp_amd.h"\n#include "dgpp_amd_layer.h"\n#include "dgpp_amd_loader.h"\n'
+    c_src.write_text('#include "dgpp_amd.h"\n#include "dgpp_amd_layer.h"\n#include "dgpp_amd_loader.h"\n#include "dgpp_amd_bench.h"\n'
                      "int main(void) { return sizeof(DgppMoeExpertView) == 96 && sizeof(DgppTensorInfo) == 104 ? 0 : 1; }\n")
     subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-I", str(inc), "-c", str(c_src), "-o", str(tmp_path / "c.o")],
                    check=True)
@@ -105,3 +109,44 @@ def test_layer_scratch_bytes_covers_what_the_layer_stages():
         assert floor <= s < 64 * floor
     cfg_sh = L.make_config(H, I, E, K, n_shared_experts=1, router_mode=L.ROUTER_SOFTMAX_TOPK)
     assert ML.scratch_bytes(cfg_sh, 8, 2048) > ML.scratch_bytes(cfg_sh, 8, 1024) >= sizes[1]
+
+
+def test_slot_ex_launchers_refuse_what_they_cannot_honour():
+    """The *_ex decode-slot launchers never drop a request silently: a pass selector outside 1..3, the shared pass
+    alone without a shared expert, an accumulation target without both of its arguments or without the shared pass
+    that would write it are all invalid arguments, raised before anything is launched (no GPU needed)."""
+    from dgpp_amd import launch as L
+    fake = 0x10000      # non-null, 16-byte aligned; never dereferenced: every call below is refused on the host
+    base = dict(n_routed=128, k_routed=256, slots=9, top_k=8)
+
+    def gate_up(n_shared, passes):
+        L.launch_moe_slot_gate_up_swiglu_ex(fake, 256, fake, None, fake, base["n_routed"], base["k_routed"], n_shared,
+                                            256 if n_shared else 0, fake, fake, fake, fake, fake, 128, base["slots"],
+                                            base["top_k"], 10.0, None, 7, 7, passes)
+
+    def down(n_shared, passes, acc_w, acc_o, fp4=False):
+        if fp4:
+            L.launch_moe_slot_down_fp4_ex(fake, 128, fake, None, fake, 256, 128, n_shared, 128 if n_shared else 0, fake, fake,
+                                          fake, 256, base["slots"], base["top_k"], None, -1, 32, 7, 7, fake, passes, acc_w, acc_o)
+        else:
+            L.launch_moe_slot_down_ex(fake, 128, fake, None, fake, 256, 128, n_shared, 128 if n_shared else 0, fake, fake, fake,
+                                      256, base["slots"], base["top_k"], None, 7, 7, passes, acc_w, acc_o)
+
+    for bad in (0, 4, -1):
+        with pytest.raises(L.InvalidArgument):
+            gate_up(128, bad)
+        with pytest.raises(L.InvalidArgument):
+            down(256, bad, None, None)
+    with pytest.raises(L.InvalidArgument):
+        gate_up(0, 2)                                # the shared pass alone, no shared expert
+    for fp4 in (False, True):
+        with pytest.raises(L.InvalidArgument):
+            down(0, 2, None, None, fp4)
+        with pytest.raises(L.InvalidArgument):
+            down(256, 3, fake, None, fp4)            # weights without an output row
+        with pytest.raises(L.InvalidArgument):
+            down(256, 3, None, fake, fp4)
+        with pytest.raises(L.InvalidArgument):
+            down(256, 1, fake, fake, fp4)            # the accumulation rides the shared pass, which is not run
+        with pytest.raises(L.InvalidArgument):
+            down(0, 3, fake, fake, fp4)              # ... or does not exist

@@ -89,8 +89,13 @@ def test_tile_list_and_compaction_bit_exact(gpu):
 
 
 @pytest.mark.parametrize("mode,E,K,T", [(1, 256, 8, 8), (1, 128, 8, 32), (0, 288, 8, 4), (2, 64, 6, 5), (1, 5, 2, 3),
-                                        (0, 1000, 16, 2)])
+                                        (0, 1000, 16, 2), (1, 1000, 8, 3), (0, 2048, 8, 2), (1, 4096, 16, 2)])
 def test_router_select_ids_exact_weights_close(gpu, mode, E, K, T):
+    """Ids are bit-exact given the scores. The weights are NOT a bit-exact contract: the device computes the softmax and
+    the renormalisation in fp32 (as the reference's kernel does) while the oracle (as the reference's CPU oracle) works
+    in double, so a softmax-mode weight - a bf16 value - may land on the neighbouring bf16 code when the exact value
+    sits next to a rounding boundary. The test bounds every weight by one bf16 ulp, counts such flips and holds them
+    to a small share; the other modes' unrounded fp32 weights stay within 2e-6 relative."""
     rng = np.random.default_rng(E + K)
     if mode == 1:   # softmax: bf16-rounded logits in both rows
         scores = hg.bf16_to_f32(hg.normal_bf16(E * 3 + T, (T, E)))
@@ -112,6 +117,9 @@ def test_router_select_ids_exact_weights_close(gpu, mode, E, K, T):
         assert np.array_equal(hg.bf16_to_f32(hg.f32_to_bf16(got_w)), got_w)
         assert np.all(np.abs(got_w - want_w) <= np.abs(want_w) * 2.0 ** -7)
         assert np.all(np.abs(got_w.sum(axis=1) - 1) < 0.02)
+        flips = int(np.count_nonzero(got_w != want_w))
+        print(f"softmax router weights E={E} K={K} T={T}: {flips} of {got_w.size} differ from the double oracle by one bf16 code")
+        assert flips <= max(1, got_w.size // 16)
     else:
         assert np.allclose(got_w, want_w, rtol=2e-6, atol=0)
 

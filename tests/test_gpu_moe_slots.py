@@ -321,3 +321,53 @@ def test_select_gate_up_is_bitwise_select_then_gate_up(gpu, kind, mode, E, H, I,
         L.launch_moe_select_gate_up_swiglu_fp4(s_d, b_d, ids2, w2, cfg, T, d.x, H, d.views, I, H, act2, I, p.limit, None, 8)
     with pytest.raises(L.InvalidArgument):
         L.launch_moe_select_gate_up_swiglu(s_d, None, ids2, w2, cfg, T, d.x, H, d.views, I, H, act2, I, p.limit, None)
+
+
+@pytest.mark.parametrize("kind,shared,sI", [("fp8", "fp8", 256), ("nvfp4", "fp8", 128), ("mxfp4", "mxfp4", 64)])
+def test_slot_ex_passes_and_folded_accumulation_are_bitwise_the_plain_launchers(gpu, kind, shared, sI):
+    """The *_ex launchers (pass selector, accumulation as the shared down pass's epilogue): routed pass and shared pass in
+    two calls give the plain launcher's rows bit for bit, and the folded accumulation gives dgpp_launch_moe_slot_accum's
+    token rows bit for bit."""
+    E, H, I, K, T = 12, 256, 64 if kind == "mxfp4" else 128, 4, 3
+    p = moe_data.make_problem(E, H, I, K, T, kind, 911, shared_kind=shared, shared_I=sI, limit=10.0, std=0.05)
+    d = DeviceMoe(p)
+    ids, weights, _, _ = moe_data.orc_router(p, 0, 2.5, True)
+    act_ref, down_ref, out_ref = run_slot_path(p, d, ids, weights, use_order=True)
+    slots, maxI = T * (K + 1), max(p.I, sI)
+    ids_d, w_d = dev(ids), dev(weights)
+    order_d = dev_empty(slots, np.int32)
+    L.launch_moe_slot_order(ids_d, order_d, slots, K, p.E, None, False)
+    act_d = dev_empty((slots, maxI), np.uint16)
+    act_d.zero_()
+    down_d = dev_empty((slots, p.H), np.float32)
+    down_d.zero_()
+    out_d = dev_empty((T, p.H), np.uint16)
+    sh = d.sh
+    shp = lambda i, j: sh[i][j] if sh else None
+    for passes in (2, 1):          # the shared pass first: the two passes touch disjoint rows
+        if kind == "fp8":
+            L.launch_moe_slot_gate_up_swiglu_ex(d.x, p.H, ids_d, order_d, d.views, p.I, p.H, sI, p.H, shp(0, 0), shp(0, 1),
+                                                shp(1, 0), shp(1, 1), act_d, maxI, slots, K, p.limit, None, 7, 7, passes)
+        else:
+            L.launch_moe_slot_gate_up_swiglu_fp4_ex(d.x, p.H, ids_d, order_d, d.views, p.I, p.H, sI, p.H, shp(0, 0),
+                                                    shp(0, 1), shp(1, 0), shp(1, 1), act_d, maxI, slots, K, p.limit, None,
+                                                    d.shared_view_base, d.fp4_group, 7, 7, passes)
+    sync()
+    assert np.array_equal(host(act_d, np.uint16), act_ref)
+    counter = dev(np.zeros(2, np.int32))
+    # routed pass alone, then the shared pass with the accumulation folded in
+    if kind == "fp8":
+        L.launch_moe_slot_down_ex(act_d, maxI, ids_d, order_d, d.views, p.H, p.I, p.H, sI, shp(2, 0), shp(2, 1), down_d, p.H,
+                                  slots, K, None, 7, 7, 1)
+        L.launch_moe_slot_down_ex(act_d, maxI, ids_d, order_d, d.views, p.H, p.I, p.H, sI, shp(2, 0), shp(2, 1), down_d, p.H,
+                                  slots, K, None, 7, 7, 2, w_d, out_d)
+    else:
+        L.launch_moe_slot_down_fp4_ex(act_d, maxI, ids_d, order_d, d.views, p.H, p.I, p.H, sI, shp(2, 0), shp(2, 1), down_d,
+                                      p.H, slots, K, None, d.shared_view_base, d.fp4_group, 7, 7, counter, 1)
+        L.launch_moe_slot_down_fp4_ex(act_d, maxI, ids_d, order_d, d.views, p.H, p.I, p.H, sI, shp(2, 0), shp(2, 1), down_d,
+                                      p.H, slots, K, None, d.shared_view_base, d.fp4_group, 7, 7, counter, 2, w_d, out_d)
+    sync()
+    got_down = host(down_d)
+    routed = np.array([s for s in range(slots) if s % (K + 1) != K])
+    assert np.array_equal(got_down[routed].view(np.uint32), down_ref[routed].view(np.uint32))
+    assert np.array_equal(host(out_d, np.uint16), out_ref)
