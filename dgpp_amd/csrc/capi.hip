@@ -970,6 +970,56 @@ int dgpp_launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const D
                                  int k, size_t out_stride, void* stream, void* ws, size_t ws_bytes) {
   return dense_mma_fp4(act, act_stride, w, out, 1, m, n, k, stream, out_stride, ws, ws_bytes);
 }
+// ---- the entry point that allocates nothing ------------------------------------------------------------------------
+// dgpp_launch_mma_gemv_fp4_bf16 with the split-K workspace taken from a file-scope device array instead of a caller's
+// buffer, for callers that cannot allocate one (code under graph capture, tight serving loops). Each GPU holds its own
+// copy of the array at its own address; the address is looked up once per device and handed to the kernels as an
+// ordinary argument (the array's name is only a host-side handle). The partial sums of a call are all written before the
+// folding launch reads them, so nothing has to start at zero; calls that overlap on one GPU share the array and race.
+}  // extern "C"
+namespace {
+constexpr size_t kStaticScratchBytes = DGPP_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+namespace {
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+// The device address of `scratch` on the current device (looked up on the first call there).
+int static_scratch(void** ptr, const char* who) {
+  int device = -1;
+  hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return finish(err, who);
+  if (device < 0 || device >= kMaxDevices) return fail_arg(std::string(who) + ": device ordinal beyond the per-device table");
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[device] == nullptr) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return finish(err, who);
+    if (p == nullptr) return fail_arg(std::string(who) + ": the scratch array has no address on this device");
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  return DGPP_OK;
+}
+}  // namespace
+extern "C" {
+int dgpp_launch_mma_gemv_fp4_bf16_static(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out,
+                                         int m, int n, int k, size_t out_stride, void* stream) {
+  const char* who = "mma_gemv_fp4_static";
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  if (k <= 0 || k % 32 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 32");
+  const size_t parts = static_cast<size_t>(w && w->scale_group == 32 ? mgeom<kFmtMxfp4>(k).parts : mgeom<kFmtNvfp4>(k).parts);
+  const size_t need = parts * static_cast<size_t>(m) * static_cast<size_t>(n) * sizeof(float);
+  if (need > kStaticScratchBytes)
+    return fail_arg(std::string(who) + ": parts(k) * m * n floats (" + std::to_string(need) + " bytes) exceed the " +
+                    std::to_string(kStaticScratchBytes) + "-byte static workspace; pass a workspace of your own to "
+                    "dgpp_launch_mma_gemv_fp4_bf16");
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws, who);
+  if (rc != DGPP_OK) return rc;
+  return dense_mma_fp4(act, act_stride, w, out, 0, m, n, k, stream, out_stride, ws, kStaticScratchBytes);
+}
 int dgpp_launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out, int m,
                                    int n, int k, void* stream) {
   return dense_mma_fp4(act, act_stride, w, out, 0, m, n, k, stream);

@@ -544,6 +544,12 @@ def launch_mma_gemv_fp4_bf16(act, act_stride, w: Fp4Matrix, out, m, n, k, out_st
                                                      _stream(stream), _p(ws), ws_bytes))
 
 
+def launch_mma_gemv_fp4_bf16_static(act, act_stride, w: Fp4Matrix, out, m, n, k, out_stride=0, stream=None):
+    """Extension: launch_mma_gemv_fp4_bf16 on the library's own static workspace (allocates nothing)."""
+    _check(_lib.load().dgpp_launch_mma_gemv_fp4_bf16_static(_p(act), act_stride, C.addressof(w), _p(out), m, n, k,
+                                                            out_stride, _stream(stream)))
+
+
 def launch_mma_gemv_fp4_f32(act, act_stride, w: Fp4Matrix, out, m, n, k, out_stride=0, stream=None, ws=None, ws_bytes=0):
     _check(_lib.load().dgpp_launch_mma_gemv_fp4_f32(_p(act), act_stride, C.addressof(w), _p(out), m, n, k, out_stride,
                                                     _stream(stream), _p(ws), ws_bytes))

@@ -336,6 +336,16 @@ int dgpp_launch_mma_gemv_fp4_bf16(const uint16_t* act, size_t act_stride, const 
                                   int n, int k, size_t out_stride, void* stream, void* ws, size_t ws_bytes);
 int dgpp_launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, float* out, int m, int n,
                                  int k, size_t out_stride, void* stream, void* ws, size_t ws_bytes);
+/* No counterpart in the reference. dgpp_launch_mma_gemv_fp4_bf16 for callers that cannot allocate a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid allocation): the split-K partial sums go to a
+ * workspace of DGPP_STATIC_SCRATCH_BYTES that the library holds in a file-scope device array (each GPU the library runs
+ * on keeps its own copy until the process ends). The call allocates nothing and gives dgpp_launch_mma_gemv_fp4_bf16's
+ * bits. parts(k) * m * n floats (parts = 4 from k = 4096, 2 from k = 2048, else 1) beyond the static workspace are
+ * refused with DGPP_INVALID_ARGUMENT. Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream do not. The first call on a device looks the array's address up. */
+#define DGPP_STATIC_SCRATCH_BYTES (8u << 20)
+int dgpp_launch_mma_gemv_fp4_bf16_static(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out,
+                                         int m, int n, int k, size_t out_stride, void* stream);
 int dgpp_launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
                                   uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
                                   void* ws, size_t ws_bytes);
