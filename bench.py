@@ -71,7 +71,7 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5,w8a8,qwen_tail,slotbench ('' for none; default: c1,c2,c4,c5, none under --tune)")
+                    "separated out of c1,c2,c4,c5,w8a8,qwen_tail,slotbench,readprobe ('' for none; default: c1,c2,c4,c5, none under --tune)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -645,12 +645,40 @@ def main():
                                        "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
         return res
 
+    def bench_readprobe():
+        """The plain-read ceiling of this chip (not one of the headline benchmark's configurations: --configs readprobe):
+        the library's streaming read kernel (16-byte loads, eight in flight per lane, nothing stored) over a 1 GiB buffer
+        (every launch cold: four times the 256 MB Infinity Cache) and over a 128 MiB buffer read again and again (served
+        by the Infinity Cache), by grid size, access pattern (one contiguous span per block / the grid striding together)
+        and load form (plain / nontemporal). A weight-streaming kernel cannot beat the best of these rates."""
+        res = {"workload": "plain streaming read, 16 bytes per lane, blocks of 256 threads"}
+        sink = torch.zeros(8192, dtype=torch.int32, device=dev)
+        best = {}
+        for label, mib in (("cold_1GiB", 1024), ("cache_resident_128MiB", 128)):
+            buf = torch.zeros(mib << 20, dtype=torch.uint8, device=dev)
+            for blocks in (512, 1024, 2048, 4096, 8192):
+                for span in (1, 0):
+                    for nt in (0, 1):
+                        def step(i):
+                            if lib.dgpp_probe_read(buf.data_ptr(), buf.numel(), sink.data_ptr(), nt, blocks, span,
+                                                   stream.cuda_stream) != 0:
+                                raise RuntimeError(lib.dgpp_last_error().decode())
+                        st = {}
+                        sec = time_graph(step, 8, 2, st)
+                        key = f"{label}_blocks{blocks}_{'span' if span else 'stride'}_{'nontemporal' if nt else 'plain'}"
+                        res[key] = {"us": sec * 1e6, "gbps": buf.numel() / sec / 1e9, "us_min": st["us_min"], "us_max": st["us_max"]}
+                        if label not in best or res[key]["gbps"] > best[label][1]:
+                            best[label] = (key, res[key]["gbps"])
+            del buf
+        res["best"] = {k: {"form": v[0], "gbps": v[1], "frac_of_peak": v[1] / HBM_PEAK_GBPS} for k, v in best.items()}
+        return res
+
     other_configs = {}
     configs = args.configs if args.configs is not None else ("" if args.tune else "c1,c2,c4,c5")
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
-            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail,
+            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail, "readprobe": bench_readprobe,
                                    "slotbench": bench_slotbench}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
@@ -802,6 +830,7 @@ def main():
                    "algorithmic_bytes_per_layer": main_res["algorithmic_bytes"]},
         "roofline": None,
         "cpu_baseline": cpu,
+        "headline_legs": {k: v for k, v in main_res.items() if k.startswith(("gate_up_", "down_"))},
         "other_batches": others,
         "other_configs": other_configs,
         "build_seconds": build_s,

@@ -348,13 +348,13 @@ int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
     return fail_arg(std::string(who) + ": bytes and both pointers must be multiples of 16");
   return finish(run_probe_copy(dst, src, bytes, as_stream(stream)), who);
 }
-int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, void* stream) {
+int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, int blocks, int span, void* stream) {
   const char* who = "probe read";
   if (bytes == 0) return DGPP_OK;
   if (!src || !sink) return fail_arg(std::string(who) + ": null pointer");
   if (bytes % 16 != 0 || reinterpret_cast<uintptr_t>(src) % 16 != 0)
     return fail_arg(std::string(who) + ": bytes and the pointer must be multiples of 16");
-  return finish(run_probe_read(src, bytes, sink, nontemporal, as_stream(stream)), who);
+  return finish(run_probe_read(src, bytes, sink, nontemporal, blocks, span, as_stream(stream)), who);
 }
 void dgpp_tune_set(int key, int value) {
   if (key >= 0 && key < kTuneCount) g_tune[key] = value;

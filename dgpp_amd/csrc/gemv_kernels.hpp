@@ -463,6 +463,8 @@ struct TokenDownArgs {
   void* out;                // [tokens, n] bf16 bits or f32
   int out_f32;
   int n, k, tokens, top_k;
+  int tiles;                // row tiles per token; the grid is tiles * tokens blocks
+  int xcd_group;            // row tiles an XCD takes for one token before it turns to the next token (see the kernel)
 };
 
 template <int FMT, int NB, bool SPLIT>
@@ -470,12 +472,31 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
   extern __shared__ uint4 lds[];
   constexpr int kPieces = FmtTraits<FMT>::kPieces;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
-  const int t = static_cast<int>(blockIdx.y);
+  // Block -> (row tile, token). Consecutive blocks go to the chip's eight XCDs in turn (block b runs on XCD b % 8 as
+  // the b / 8-th block there) and each XCD has an L2 of its own. An XCD therefore takes `xcd_group` of its row tiles
+  // for one token, then the SAME tiles for the next token, and so on through the batch before it moves on: tokens that
+  // routed to the same expert find its rows in that L2 instead of fetching them again over the fabric. A large group
+  // (all of an XCD's tiles) is plain token-major order: the longest sequential walk through each expert's rows, the
+  // better order while few tokens share experts.
+  int t, tile;
+  {
+    const int b = static_cast<int>(blockIdx.x);
+    const int G = a.xcd_group;
+    if (G > 0) {     // tiles is a multiple of 8 * G
+      const int seq = b >> 3;
+      const int gi = seq % G, rest = seq / G;
+      t = rest % a.tokens;
+      tile = ((rest / a.tokens) * G + gi) * 8 + (b & 7);
+    } else {
+      t = b / a.tiles;
+      tile = b - t * a.tiles;
+    }
+  }
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
   const int row_vecs = kPieces * chunks;
   const int rpw = kWave >> g.l2;
   const int rows_per_block = rpw * steps;
-  const int tile_row0 = static_cast<int>(blockIdx.x) * rows_per_block;
+  const int tile_row0 = tile * rows_per_block;
   uint4* my_x = lds + wave * row_vecs;
   float* part = reinterpret_cast<float*>(lds + a.top_k * row_vecs);   // [top_k][rows_per_block]
   const float* gd = nullptr;
@@ -927,7 +948,16 @@ hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipStream_t stream) {
   steps = steps < 2 ? 2 : (steps > 8 ? 8 : steps);   // two row groups per wavefront measured best from one token on
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const int rows_per_block = rpw * steps;
-  const dim3 grid(static_cast<unsigned>((a.n + rows_per_block - 1) / rows_per_block), static_cast<unsigned>(a.tokens));
+  TokenDownArgs b = a;
+  b.tiles = (a.n + rows_per_block - 1) / rows_per_block;
+  // Tokens share experts often enough to pay for the XCD-local order from about a quarter of the experts in use.
+  b.xcd_group = 0;
+  {
+    int want = tune_get(kTuneXcdGroup) > 0 ? tune_get(kTuneXcdGroup) : (a.tokens * a.top_k * 4 >= 256 ? 1 : 0);
+    if (a.tokens > 1 && want > 0 && b.tiles % (8 * want) == 0) b.xcd_group = want;
+  }
+  if (static_cast<long long>(b.tiles) * a.tokens > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  const dim3 grid(static_cast<unsigned>(b.tiles) * static_cast<unsigned>(a.tokens));
   const size_t lds = static_cast<size_t>(a.top_k) * (stage_bytes(1, a.k) + static_cast<size_t>(rows_per_block) * sizeof(float));
   hipError_t err = hipSuccess;
   dispatch_nb(g.nb, [&](auto nbc) {
@@ -936,7 +966,7 @@ hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipStream_t stream) {
                        (reinterpret_cast<uintptr_t>(a.act) & 15u) == 0;
     auto go = [&](auto kern) {
       err = ensure_lds(kern, lds);
-      if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(a.top_k * kWave), lds, stream, a, g, steps);
+      if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(a.top_k * kWave), lds, stream, b, g, steps);
     };
     if (split) go(token_down_accum_kernel<FMT, NB, true>);
     else go(token_down_accum_kernel<FMT, NB, false>);

@@ -270,23 +270,35 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(uint4* __restrict__ dst
   for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n16; i += stride)
     dst[i] = src[i];
 }
-// Plain read: every lane streams 16-byte vectors (four in flight), xors them together and stores one word per block
-// only if the result is a value no input produces — the rate a weight stream could reach with no arithmetic at all.
+// Plain read: a block owns a contiguous span and walks it with 16-byte loads, eight 4 KB lines in flight per block
+// step (`span` != 0), or all lanes of the grid stride through the buffer together (`span` == 0); the loads are xor-ed
+// together and one word per block is stored only if the result is a value no input produces — the rate a weight stream
+// could reach with no arithmetic at all.
 __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict__ src, size_t n16, uint32_t* __restrict__ sink,
-                                                         int nontemporal) {
+                                                         int nontemporal, int span) {
   typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
   const __attribute__((address_space(1))) u32x4_t* p = (const __attribute__((address_space(1))) u32x4_t*)(uintptr_t)src;
-  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  constexpr int U = 8;
   u32x4_t acc = {0u, 0u, 0u, 0u};
-  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    u32x4_t v[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = nontemporal ? __builtin_nontemporal_load(p + i + u * stride) : p[i + u * stride];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) acc ^= v[u];
+  size_t i, end, step;
+  if (span) {
+    const size_t per_block = (n16 + gridDim.x - 1) / gridDim.x;
+    i = per_block * blockIdx.x + threadIdx.x;
+    end = min(n16, per_block * (blockIdx.x + 1));
+    step = blockDim.x;
+  } else {
+    i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    end = n16;
+    step = static_cast<size_t>(gridDim.x) * blockDim.x;
   }
-  for (; i < n16; i += stride) acc ^= p[i];
+  for (; i + (U - 1) * step < end; i += U * step) {
+    u32x4_t v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = nontemporal ? __builtin_nontemporal_load(p + i + u * step) : p[i + u * step];
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc ^= v[u];
+  }
+  for (; i < end; i += step) acc ^= p[i];
   const uint32_t x = acc.x ^ acc.y ^ acc.z ^ acc.w;
   if (x == 0x9E3779B9u && sink != nullptr) sink[blockIdx.x] = x;
 }
@@ -380,12 +392,12 @@ hipError_t run_probe_copy(void* dst, const void* src, size_t bytes, hipStream_t 
   return hipGetLastError();
 }
 
-hipError_t run_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, hipStream_t stream) {
+hipError_t run_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, int blocks, int span, hipStream_t stream) {
   const size_t n16 = bytes / 16;
-  const size_t want = (n16 + 1023) / 1024;
-  const unsigned blocks = static_cast<unsigned>(want < 1 ? 1 : (want > 8192 ? 8192 : want));
-  hipLaunchKernelGGL(probe_read_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<const uint4*>(src), n16,
-                     static_cast<uint32_t*>(sink), nontemporal);
+  if (blocks <= 0) blocks = 2048;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(probe_read_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                     static_cast<const uint4*>(src), n16, static_cast<uint32_t*>(sink), nontemporal, span);
   return hipGetLastError();
 }
 

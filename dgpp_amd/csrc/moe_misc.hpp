@@ -40,7 +40,7 @@ hipError_t run_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* out
                                 hipStream_t stream);
 hipError_t run_probe_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 // sink: at least 8192 words, never written in practice (keeps the loads alive)
-hipError_t run_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, hipStream_t stream);
+hipError_t run_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, int blocks, int span, hipStream_t stream);
 hipError_t run_fp8_dequant(const uint8_t* payload, const void* scales, int e8m0, uint16_t* out, int64_t rows,
                            int64_t cols, int rs, int cs, hipStream_t stream);
 

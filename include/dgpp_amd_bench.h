@@ -22,11 +22,13 @@ extern "C" {
  * move to the matrix core from 5 rows (FP4) / 9 rows (FP8) on); key 6: 1 makes the layer driver compute the slot order for small decode batches too
  * (default: batches of at most 128 routed slots find the sharers of an expert by ballot, no order);
  * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
- * blocks, dgpp_launch_moe_select_gate_up_swiglu); key 9: 1 keeps the shared expert's passes of the layer driver
+ * blocks, dgpp_launch_moe_select_gate_up_swiglu); key 8: row tiles an XCD takes for one token before it turns to the next token in the token-major
+ * down + accumulate launch (0 = automatic: 1 from 64 routed slots on, else plain token-major order);
+ * key 9: 1 keeps the shared expert's passes of the layer driver
  * on the caller's stream, 2 moves them to a second stream beside the routed passes at every batch size (default:
  * from three tokens on); 3 and 4 keep one stream and never / always fold the accumulation into the shared down pass
  * (default: at one token). Outputs do not depend on keys
- * 1 - 4, 6, 7 and 9; keys 0 and
+ * 1 - 4 and 6 - 9; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
  * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);
@@ -37,11 +39,12 @@ int dgpp_tune_get(int key);
  * are calibrated against it: it reads `bytes` and writes `bytes`, nothing else. */
 int dgpp_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
 
-/* A plain streaming READ of `bytes` (a multiple of 16, 16-byte aligned) on `stream`: 16-byte loads, four in flight
- * per lane, nothing stored (`sink`, at least 8192 words, is written only for a checksum no input produces). The rate
- * it reaches is the ceiling of a weight stream on this chip; nontemporal != 0 uses the nontemporal load form the
- * GEMV kernels use where a launch reads its weights once. */
-int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, void* stream);
+/* A plain streaming READ of `bytes` (a multiple of 16, 16-byte aligned) on `stream`: 16-byte loads, eight in flight
+ * per lane, nothing stored (`sink`, at least 8192 words, is written only for a checksum no input produces). `blocks`
+ * blocks of 256 threads (0 = 2048, at most 8192); span != 0 gives every block one contiguous span of the buffer, span == 0
+ * lets the whole grid stride through it together. The rate it reaches is the ceiling of a weight stream on this chip;
+ * nontemporal != 0 uses the nontemporal load form the GEMV kernels use where a launch reads its weights once. */
+int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, int blocks, int span, void* stream);
 
 #ifdef __cplusplus
 }
