@@ -461,9 +461,19 @@ def main():
             L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
             L.launch_moe_round_bf16(out, routed, cT * cH, stream)
 
-        def full(i):            # the shared expert through the GEMV-named launchers (they take the matrix core at 64 rows)
+        def stitched(i):        # the shared expert through the GEMV-named launchers (they take the matrix core at 64 rows)
             routed_part(i)
             shared_part(i)
+
+        # the whole layer as ONE call of the layer driver: the MXFP8 shared expert of its own width runs as dense
+        # projections on a second stream beside the routed passes, then the chain's last step and the rounding
+        cfg5s = L.make_config(cH, cI, cE, cK, n_shared_experts=1, routed_scaling_factor=1.0, swiglu_limit=float("inf"),
+                              router_mode=L.ROUTER_SOFTMAX_TOPK)
+        lay1 = ML.MoeLayer(cfg5s, ML.EXPERTS_NVFP4, views, cT, shared_inter=cSI, sh_payload=[t[0] for t in sh],
+                           sh_scales_e8m0=[t[1] for t in sh])
+
+        def full(i):
+            lay1.enqueue_decode_scores(x, cH, lg5, lg5, out, cT, stream)
 
         def full_w8a8(i):
             routed_part(i)
@@ -474,9 +484,10 @@ def main():
         shared_bytes = 3 * cSI * cH + 3 * cSI * cH // 32
         nbytes = uniq * per_expert + shared_bytes + cT * cH * 4
         res = {"workload": f"C5 NVFP4 routed MoE (256 experts, hidden 6144, inter 2048, top-8, {uniq} distinct; decode slots) "
-                           f"+ MXFP8 shared expert (inter 4096; launch_scale_gemm_grid_e8m0_*, which run the matrix-core form at 64 rows), T=64; routed expert weights = device copies of {G} generated experts",
+                           f"+ MXFP8 shared expert (inter 4096, dense projections: launch_scale_gemm_grid_e8m0_*, the matrix-core form at 64 rows) as ONE layer-driver call, T=64; routed expert weights = device copies of {G} generated experts",
                "algorithmic_bytes": nbytes}
-        for name, fn, nb in (("layer", full, nbytes), ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
+        for name, fn, nb in (("layer", full, nbytes), ("layer_stitched_from_launchers", stitched, nbytes),
+                             ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
                              ("routed_only_matrix_core", routed_mc, uniq * per_expert + cT * cH * 6),
                              ("shared_only_gemv_launchers", shared_part, shared_bytes + cT * cH * 4),
                              ("shared_only", shared_mc, shared_bytes + cT * cH * 4),
@@ -486,6 +497,7 @@ def main():
             res[name] = {"us": sec * 1e6, "algorithmic_bytes": nb, "gbps": nb / sec / 1e9,
                          "frac_of_peak": nb / sec / 1e9 / HBM_PEAK_GBPS}
         lay.close()
+        lay1.close()
         return res
 
     def bench_slotbench():

@@ -171,7 +171,7 @@ class MoeLayerDesc(C.Structure):
         ("cfg", MoeConfig), ("expert_format", C.c_int32), ("max_tokens", C.c_int32), ("views", C.c_void_p),
         ("shared_in_table", C.c_int32), ("shared_inter", C.c_int32), ("sh_payload", C.c_void_p * 3),
         ("sh_scales", C.c_void_p * 3), ("sh_rs", C.c_int32), ("sh_cs", C.c_int32), ("router_gate", C.c_void_p),
-        ("router_bias", C.c_void_p),
+        ("router_bias", C.c_void_p), ("sh_scales_e8m0", C.c_void_p * 3),
     ]
 
 
@@ -179,6 +179,7 @@ class MoeLayerDesc(C.Structure):
 LAYER_SIGNATURES = {
     "dgpp_moe_layer_last_error": (C.c_char_p, []),
     "dgpp_moe_layer_scratch_bytes": (C.c_size_t, [_P, _I, _I]),
+    "dgpp_moe_layer_scratch_bytes_dense_shared": (C.c_size_t, [_P, _I, _I]),
     "dgpp_moe_layer_create": (_I, [_P, _P]),
     "dgpp_moe_layer_destroy": (None, [_P]),
     "dgpp_moe_layer_enqueue_decode": (_I, [_P, _P, _Z, _P, _P, _I, _P]),

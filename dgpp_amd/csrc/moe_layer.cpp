@@ -20,9 +20,9 @@ size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 // Buffer sizes in bytes, in the order they are carved (each rounded to 256).
 struct Layout {
   size_t views, ids, weights, scores, biased, order, slot_act, slot_down, acc, counter, rows, slot_row, segs, gather,
-      gate, up, total;
+      gate, up, sh_gate, sh_up, sh_act, sh_down, sh_ws, rows_id, ones, total;
 };
-Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t n_views) {
+Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t n_views, bool dense_shared) {
   const size_t M = static_cast<size_t>(std::max(max_tokens, 0)), H = c.hidden, K = c.top_k, E = c.n_experts;
   const size_t I = static_cast<size_t>(std::max(c.inter, shared_inter));
   const size_t slots = M * (K + 1);
@@ -43,15 +43,48 @@ Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t
   l.gather = align_up(slots * H * 2);
   l.gate = align_up(slots * I * 2);
   l.up = align_up(slots * I * 2);
+  if (dense_shared) {
+    const size_t SI = static_cast<size_t>(std::max(shared_inter, 0));
+    l.sh_gate = l.sh_up = l.sh_act = align_up(M * SI * 2);
+    l.sh_down = align_up(M * H * 4);
+    l.sh_ws = align_up(4 * M * std::max(SI, H) * 4);   // up to four K parts of [tokens, n] partial sums
+    l.rows_id = align_up(M * 4);
+    l.ones = align_up(M * 4);
+  }
   l.total = l.views + l.ids + l.weights + l.scores + l.biased + l.order + l.slot_act + l.slot_down + l.acc + l.counter +
-            l.rows + l.slot_row + l.segs + l.gather + l.gate + l.up;
+            l.rows + l.slot_row + l.segs + l.gather + l.gate + l.up + l.sh_gate + l.sh_up + l.sh_act + l.sh_down + l.sh_ws +
+            l.rows_id + l.ones;
   return l;
 }
 
+// A branch of work on the side stream: forked from the caller's stream and joined to it again on EVERY way out of the
+// scope that opened it (a launcher that throws between fork and join must not leave a captured graph with an
+// unjoined branch).
+struct StreamFork {
+  hipStream_t main, side;
+  hipEvent_t fork_ev, join_ev;
+  bool open = false;
+  void begin() {
+    hip_ok(hipEventRecord(fork_ev, main), "GlmMoeLayer: fork");
+    hip_ok(hipStreamWaitEvent(side, fork_ev, 0), "GlmMoeLayer: fork");
+    open = true;
+  }
+  void end() {
+    if (!open) return;
+    open = false;
+    hip_ok(hipEventRecord(join_ev, side), "GlmMoeLayer: join");
+    hip_ok(hipStreamWaitEvent(main, join_ev, 0), "GlmMoeLayer: join");
+  }
+  ~StreamFork() {
+    if (!open) return;
+    if (hipEventRecord(join_ev, side) == hipSuccess) (void)hipStreamWaitEvent(main, join_ev, 0);
+  }
+};
+
 }  // namespace
 
-size_t GlmMoeLayer::scratch_bytes(const GlmMoeConfig& cfg, int max_tokens, int shared_inter) {
-  return layout_of(cfg, max_tokens, shared_inter, static_cast<size_t>(cfg.n_experts + 1) * 3).total;
+size_t GlmMoeLayer::scratch_bytes(const GlmMoeConfig& cfg, int max_tokens, int shared_inter, bool dense_shared) {
+  return layout_of(cfg, max_tokens, shared_inter, static_cast<size_t>(cfg.n_experts + 1) * 3, dense_shared).total;
 }
 
 GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, int max_tokens)
@@ -80,7 +113,15 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
                                  std::to_string(i) + ")");
     }
   }
-  if (w.shared_in_table) {
+  const bool e8m0_shared = w.sh_scales_e8m0[0] || w.sh_scales_e8m0[1] || w.sh_scales_e8m0[2];
+  if (e8m0_shared) {
+    if (w.shared_in_table || w.shared_inter <= 0)
+      throw std::runtime_error("GlmMoeLayer: an MXFP8 shared expert is given by payloads and scale bytes and needs its width");
+    for (int i = 0; i < 3; ++i)
+      if (!w.sh_payload[i] || !w.sh_scales_e8m0[i]) throw std::runtime_error("GlmMoeLayer: inconsistent MXFP8 shared matrices");
+    if (cfg.hidden % 32 != 0 || w.shared_inter % 32 != 0)
+      throw std::runtime_error("GlmMoeLayer: an MXFP8 shared expert needs hidden and its width in multiples of 32");
+  } else if (w.shared_in_table) {
     if (!fp4) throw std::runtime_error("GlmMoeLayer: a table-resident shared expert needs an fp4 table");
     if (w.shared_inter != cfg.inter)
       throw std::runtime_error(
@@ -91,9 +132,9 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   }
   if ((cfg.n_shared_experts != 0) != (w.shared_inter > 0))
     throw std::runtime_error("GlmMoeLayer: n_shared_experts does not match the shared weights");
-  max_inter_ = std::max(cfg.inter, w.shared_inter);
+  max_inter_ = e8m0_shared ? cfg.inter : std::max(cfg.inter, w.shared_inter);   // a dense shared expert takes no slot rows
 
-  const Layout l = layout_of(cfg, max_tokens, w.shared_inter, w.views.size());
+  const Layout l = layout_of(cfg, max_tokens, w.shared_inter, w.views.size(), e8m0_shared);
   hip_ok(hipMalloc(&arena_, l.total), "GlmMoeLayer: hipMalloc");
   try {
   uint8_t* p = static_cast<uint8_t*>(arena_);
@@ -118,6 +159,21 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   d_gather_ = reinterpret_cast<uint16_t*>(carve(l.gather));
   d_gate_ = reinterpret_cast<uint16_t*>(carve(l.gate));
   d_up_ = reinterpret_cast<uint16_t*>(carve(l.up));
+  if (e8m0_shared) {
+    d_sh_gate_ = reinterpret_cast<uint16_t*>(carve(l.sh_gate));
+    d_sh_up_ = reinterpret_cast<uint16_t*>(carve(l.sh_up));
+    d_sh_act_ = reinterpret_cast<uint16_t*>(carve(l.sh_act));
+    d_sh_down_ = reinterpret_cast<float*>(carve(l.sh_down));
+    d_sh_ws_ = carve(l.sh_ws);
+    sh_ws_bytes_ = l.sh_ws;
+    d_rows_id_ = reinterpret_cast<int32_t*>(carve(l.rows_id));
+    d_ones_ = reinterpret_cast<float*>(carve(l.ones));
+    std::vector<int32_t> idv(static_cast<size_t>(max_tokens));
+    std::vector<float> onev(static_cast<size_t>(max_tokens), 1.0f);
+    for (int i = 0; i < max_tokens; ++i) idv[static_cast<size_t>(i)] = i;
+    hip_ok(hipMemcpy(d_rows_id_, idv.data(), idv.size() * 4, hipMemcpyHostToDevice), "GlmMoeLayer: row list upload");
+    hip_ok(hipMemcpy(d_ones_, onev.data(), onev.size() * 4, hipMemcpyHostToDevice), "GlmMoeLayer: unit weights upload");
+  }
   // The device expert table is uploaded once (the reference's capture form prepares a per-binding
   // device table once too, src/models/glm/moe_layer.cpp:364-396); the counter pair is zero at rest.
   hip_ok(hipMemcpy(d_views_, w.views.data(), w.views.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
@@ -192,11 +248,44 @@ void GlmMoeLayer::enqueue_decode_routed(const uint16_t* x, size_t x_stride, cons
   expert_chain_slots(x, x_stride, ids, weights, out_bf16, out_f32, tokens, stream);
 }
 
+// The dense shared expert: gate and up projections of every token row, SwiGLU, the down projection (unrounded).
+void GlmMoeLayer::dense_shared_chain(const uint16_t* x, size_t x_stride, int tokens, hipStream_t st) {
+  const int H = cfg_.hidden, SI = w_.shared_inter;
+  launch_scale_gemm_grid_e8m0_bf16(x, x_stride, w_.sh_payload[0], w_.sh_scales_e8m0[0], d_sh_gate_, tokens, SI, H, st,
+                                   static_cast<size_t>(SI), 0, 5, d_sh_ws_, sh_ws_bytes_);
+  launch_scale_gemm_grid_e8m0_bf16(x, x_stride, w_.sh_payload[1], w_.sh_scales_e8m0[1], d_sh_up_, tokens, SI, H, st,
+                                   static_cast<size_t>(SI), 0, 5, d_sh_ws_, sh_ws_bytes_);
+  launch_moe_swiglu_clamp(d_sh_gate_, d_sh_up_, d_sh_act_, static_cast<int64_t>(tokens) * SI, cfg_.swiglu_limit, st);
+  launch_scale_gemm_grid_e8m0_f32(d_sh_act_, static_cast<size_t>(SI), w_.sh_payload[2], w_.sh_scales_e8m0[2], d_sh_down_,
+                                  tokens, H, SI, st, static_cast<size_t>(H), 0, 5, d_sh_ws_, sh_ws_bytes_);
+}
+
 // Steps 4-7 of the reference's decode call order (src/models/glm/moe_layer.cpp:1555-1677).
 void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                                      uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
-                                     bool order_ready, const float* sel_scores, const float* sel_biased) {
+                                     bool order_ready, const float* sel_scores, const float* sel_biased,
+                                     bool routed_only) {
   const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter;
+  if (out_bf16 == nullptr && out_f32 == nullptr) throw std::invalid_argument("GlmMoeLayer: no output buffer");
+  if (dense_shared() && !routed_only) {
+    // The routed chain, unrounded, with the shared expert's dense projections beside it on the side stream (they
+    // depend on nothing but x); then the chain's last step a = fma(1, shared, a) and the one rounding.
+    float* acc = out_f32 ? out_f32 : d_acc_;
+    StreamFork fork{stream, side_, fork_, join_};
+    const bool beside = side_ != nullptr && dgpp_tune_get(9) != 1;
+    if (beside) {
+      fork.begin();
+      dense_shared_chain(x, x_stride, tokens, side_);
+    }
+    expert_chain_slots(x, x_stride, ids, weights, nullptr, acc, tokens, stream, order_ready, sel_scores, sel_biased,
+                       /*routed_only=*/true);
+    if (beside) fork.end();
+    else dense_shared_chain(x, x_stride, tokens, stream);
+    launch_moe_accum(acc, d_sh_down_, d_rows_id_, d_ones_, tokens, H, stream);
+    if (!out_f32) launch_moe_round_bf16(out_bf16, acc, static_cast<int64_t>(tokens) * H, stream);
+    return;
+  }
+  const bool slot_shared = has_shared() && !dense_shared();   // the shared expert as slot top_k of every token
   const int slots = tokens * (K + 1);
   if (slots > 1024 && tokens > 1)
     throw std::invalid_argument("GlmMoeLayer: the decode-slot path takes at most 1024 slots; use the grouped path");
@@ -207,10 +296,10 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   }
   // The token-major down kernel fuses the accumulation but reads an expert once per slot; the slot kernel reads
   // it once per run of slots. Token-major while few slots can share an expert (small batches), runs beyond.
-  const bool token_major = !has_shared() && dgpp_tune_get(4) != 1 && tokens * K * 2 <= cfg_.n_experts;
-  const bool sh_args = has_shared() && !w_.shared_in_table;
-  const int n_sh = has_shared() ? w_.shared_inter : 0;
-  const int k_sh_up = has_shared() ? H : 0;     // the shared gate/up contract over hidden
+  const bool token_major = !slot_shared && dgpp_tune_get(4) != 1 && tokens * K * 2 <= cfg_.n_experts;
+  const bool sh_args = slot_shared && !w_.shared_in_table;
+  const int n_sh = slot_shared ? w_.shared_inter : 0;
+  const int k_sh_up = slot_shared ? H : 0;     // the shared gate/up contract over hidden
   // With scores given, ids / weights are this layer's own buffers and the gate/up launch fills them.
   const bool fused = sel_scores != nullptr && ids == d_ids_ && weights == d_weights_ && order == nullptr;
   if (sel_scores != nullptr && !fused) throw std::logic_error("GlmMoeLayer: fused selection outside its form");
@@ -218,34 +307,18 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   // on the side stream beside them, forked here and joined before the accumulation. One launcher call per pass.
   // From a few tokens on: the two cross-stream dependencies cost more than the two hand-overs they take off the
   // chain while a pass is only a few microseconds long (measured: slower at one token, level at two).
-  const bool split = has_shared() && side_ != nullptr && dgpp_tune_get(9) != 1 && (tokens >= 3 || dgpp_tune_get(9) == 2);
+  const bool split = slot_shared && side_ != nullptr && dgpp_tune_get(9) != 1 && (tokens >= 3 || dgpp_tune_get(9) == 2);
   // On one stream the shared down pass ends with the token's accumulation (no launch of its own).
   // (One token, where a launch is a fifth of the step; measured level at two tokens. Bench switch 9 = 4 folds at any
   // batch size, 3 never.)
-  const bool fold_accum = has_shared() && !split && out_bf16 != nullptr && out_f32 == nullptr && dgpp_tune_get(9) != 3 &&
+  const bool fold_accum = slot_shared && !split && out_bf16 != nullptr && out_f32 == nullptr && dgpp_tune_get(9) != 3 &&
                           (tokens == 1 || dgpp_tune_get(9) == 4);
   // Everything that can be refused is refused before the first enqueue.
-  if (has_shared() && out_f32 != nullptr)
+  if (slot_shared && out_f32 != nullptr)
     throw std::invalid_argument("GlmMoeLayer: an unrounded output with a shared expert is not a decode form");
   if (out_bf16 == nullptr && out_f32 == nullptr) throw std::invalid_argument("GlmMoeLayer: no output buffer");
-  // The side stream joins the caller's stream again on EVERY way out of this function (a launcher that throws
-  // between fork and join must not leave a captured graph with an unjoined branch).
-  struct Fork {
-    hipStream_t main, side;
-    hipEvent_t join;
-    bool open = false;
-    void close_quietly() {
-      if (!open) return;
-      open = false;
-      if (hipEventRecord(join, side) == hipSuccess) (void)hipStreamWaitEvent(main, join, 0);
-    }
-    ~Fork() { close_quietly(); }
-  } fork{stream, side_, join_};
-  if (split) {
-    hip_ok(hipEventRecord(fork_, stream), "GlmMoeLayer: fork");
-    hip_ok(hipStreamWaitEvent(side_, fork_, 0), "GlmMoeLayer: fork");
-    fork.open = true;
-  }
+  StreamFork fork{stream, side_, fork_, join_};
+  if (split) fork.begin();
   // One launcher call per pass and stream: the routed pass on the caller's stream, the shared pass beside it.
   auto for_passes = [&](auto&& call) {
     if (!split) return call(stream, 3);
@@ -258,7 +331,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     if (fused) {
       launch_moe_select_gate_up_swiglu(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
                                        d_slot_act_, max_inter_, cfg_.swiglu_limit, stream);
-      if (has_shared())   // the shared slot's pass: the routed pass already ran above
+      if (slot_shared)   // the shared slot's pass: the routed pass already ran above
         launch_moe_slot_gate_up_swiglu_ex(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up, w_.sh_payload[0],
                                           w_.sh_scales[0], w_.sh_payload[1], w_.sh_scales[1], d_slot_act_, max_inter_, slots,
                                           K, cfg_.swiglu_limit, split ? side_ : stream, w_.sh_rs, w_.sh_cs, 2);
@@ -274,7 +347,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
       return;
     }
     for_passes([&](hipStream_t st, int passes) {
-      launch_moe_slot_down_ex(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, has_shared() ? H : 0,
+      launch_moe_slot_down_ex(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I, slot_shared ? H : 0,
                               n_sh, w_.sh_payload[2], w_.sh_scales[2], d_slot_down_, H, slots, K, st, w_.sh_rs, w_.sh_cs,
                               passes, fold_w, fold_o);
     });
@@ -283,7 +356,7 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     if (fused) {
       launch_moe_select_gate_up_swiglu_fp4(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I,
                                            H, d_slot_act_, max_inter_, cfg_.swiglu_limit, stream, fp4_group_);
-      if (has_shared())
+      if (slot_shared)
         launch_moe_slot_gate_up_swiglu_fp4_ex(x, x_stride, ids, order, d_views_, I, H, n_sh, k_sh_up,
                                               sh_args ? w_.sh_payload[0] : nullptr, sh_args ? w_.sh_scales[0] : nullptr,
                                               sh_args ? w_.sh_payload[1] : nullptr, sh_args ? w_.sh_scales[1] : nullptr,
@@ -304,18 +377,14 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     }
     for_passes([&](hipStream_t st, int passes) {
       launch_moe_slot_down_fp4_ex(d_slot_act_, static_cast<size_t>(max_inter_), ids, order, d_views_, H, I,
-                                  has_shared() ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
+                                  slot_shared ? H : 0, n_sh, sh_args ? w_.sh_payload[2] : nullptr,
                                   sh_args ? w_.sh_scales[2] : nullptr, d_slot_down_, H, slots, K, st, base, fp4_group_,
                                   w_.sh_rs, w_.sh_cs, d_tile_counter_, passes, fold_w, fold_o);
     });
   }
-  if (fork.open) {
-    fork.open = false;
-    hip_ok(hipEventRecord(join_, side_), "GlmMoeLayer: join");
-    hip_ok(hipStreamWaitEvent(stream, join_, 0), "GlmMoeLayer: join");
-  }
+  fork.end();
   if (fold_accum) return;
-  if (has_shared()) {
+  if (slot_shared) {
     launch_moe_slot_accum(out_bf16, d_slot_down_, weights, tokens, H, K, stream);
   } else if (out_f32) {
     launch_moe_slot_accum_routed_f32(out_f32, d_slot_down_, weights, tokens, H, K, stream);
@@ -436,6 +505,10 @@ size_t dgpp_moe_layer_scratch_bytes(const DgppMoeConfig* cfg, int max_tokens, in
   return dgpp::GlmMoeLayer::scratch_bytes(cpp_config(*cfg), max_tokens, shared_inter);
 }
 
+size_t dgpp_moe_layer_scratch_bytes_dense_shared(const DgppMoeConfig* cfg, int max_tokens, int shared_inter) {
+  return dgpp::GlmMoeLayer::scratch_bytes(cpp_config(*cfg), max_tokens, shared_inter, true);
+}
+
 int dgpp_moe_layer_create(const DgppMoeLayerDesc* d, DgppMoeLayer** out) {
   return guarded([&] {
     if (!d || !out || !d->views) throw std::invalid_argument("moe_layer_create: null pointer");
@@ -451,6 +524,7 @@ int dgpp_moe_layer_create(const DgppMoeLayerDesc* d, DgppMoeLayer** out) {
     }
     w.sh_rs = d->sh_rs;
     w.sh_cs = d->sh_cs;
+    for (int i = 0; i < 3; ++i) w.sh_scales_e8m0[i] = d->sh_scales_e8m0[i];
     w.router_gate = d->router_gate;
     w.router_bias = d->router_bias;
     *out = new DgppMoeLayer(cpp_config(d->cfg), w, d->max_tokens);

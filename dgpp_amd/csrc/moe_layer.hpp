@@ -26,6 +26,8 @@ struct GlmMoeLayerWeights {
   const uint8_t* sh_payload[3] = {nullptr, nullptr, nullptr};
   const float* sh_scales[3] = {nullptr, nullptr, nullptr};
   int sh_rs = 7, sh_cs = 7;
+  // All three non-null: an MXFP8 shared expert (E8M0 byte per 32 columns) of its own width, run as dense projections.
+  const uint8_t* sh_scales_e8m0[3] = {nullptr, nullptr, nullptr};
   const uint16_t* router_gate = nullptr;
   const float* router_bias = nullptr;
 };
@@ -37,7 +39,7 @@ class GlmMoeLayer {
   GlmMoeLayer(const GlmMoeLayer&) = delete;
   GlmMoeLayer& operator=(const GlmMoeLayer&) = delete;
 
-  static size_t scratch_bytes(const GlmMoeConfig& cfg, int max_tokens, int shared_inter);
+  static size_t scratch_bytes(const GlmMoeConfig& cfg, int max_tokens, int shared_inter, bool dense_shared = false);
 
   // out_f32 non-null: the unrounded chain goes there and out_bf16 is not written.
   void enqueue_decode(const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32, int tokens,
@@ -56,14 +58,18 @@ class GlmMoeLayer {
   const int32_t* ids() const { return d_ids_; }
   const float* weights() const { return d_weights_; }
   bool has_shared() const { return w_.shared_inter > 0; }
+  // The shared expert runs as dense projections over the token rows (MXFP8), not as slot top_k of every token.
+  bool dense_shared() const { return has_shared() && w_.sh_scales_e8m0[0] != nullptr; }
 
  private:
   void release();
   void check_tokens(int tokens) const;
   bool needs_order(int tokens) const;
+  void dense_shared_chain(const uint16_t* x, size_t x_stride, int tokens, hipStream_t stream);
   void expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                           uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
-                          bool order_ready = false, const float* sel_scores = nullptr, const float* sel_biased = nullptr);
+                          bool order_ready = false, const float* sel_scores = nullptr, const float* sel_biased = nullptr,
+                          bool routed_only = false);
 
   GlmMoeConfig cfg_;
   GlmMoeLayerWeights w_;
@@ -92,6 +98,16 @@ class GlmMoeLayer {
   uint16_t* d_gather_ = nullptr;     // [rows_total, hidden]
   uint16_t* d_gate_ = nullptr;       // [rows_total, max_inter]
   uint16_t* d_up_ = nullptr;
+  // dense shared expert: gate / up / SwiGLU rows [tokens, shared_inter], unrounded down rows [tokens, hidden], the
+  // split-K workspace of its projections, and the identity row list / unit weights of the last chain step
+  uint16_t* d_sh_gate_ = nullptr;
+  uint16_t* d_sh_up_ = nullptr;
+  uint16_t* d_sh_act_ = nullptr;
+  float* d_sh_down_ = nullptr;
+  void* d_sh_ws_ = nullptr;
+  size_t sh_ws_bytes_ = 0;
+  int32_t* d_rows_id_ = nullptr;
+  float* d_ones_ = nullptr;
 };
 
 }  // namespace dgpp

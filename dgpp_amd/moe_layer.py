@@ -21,7 +21,9 @@ def _check(rc: int) -> None:
     raise RuntimeError(msg)
 
 
-def scratch_bytes(cfg: MoeConfig, max_tokens: int, shared_inter: int = 0) -> int:
+def scratch_bytes(cfg: MoeConfig, max_tokens: int, shared_inter: int = 0, dense_shared: bool = False) -> int:
+    if dense_shared:
+        return _lib.load().dgpp_moe_layer_scratch_bytes_dense_shared(C.addressof(cfg), max_tokens, shared_inter)
     return _lib.load().dgpp_moe_layer_scratch_bytes(C.addressof(cfg), max_tokens, shared_inter)
 
 
@@ -30,7 +32,8 @@ class MoeLayer:
 
     def __init__(self, cfg: MoeConfig, expert_format: int, views: list[MoeExpertView], max_tokens: int, *,
                  shared_in_table: bool = False, shared_inter: int = 0, sh_payload=(None, None, None),
-                 sh_scales=(None, None, None), sh_rs: int = 7, sh_cs: int = 7, router_gate=None, router_bias=None):
+                 sh_scales=(None, None, None), sh_rs: int = 7, sh_cs: int = 7, router_gate=None, router_bias=None,
+                 sh_scales_e8m0=(None, None, None)):
         self._lib = _lib.load()
         arr = (MoeExpertView * len(views))(*views)
         d = MoeLayerDesc()
@@ -43,11 +46,12 @@ class MoeLayer:
         for i in range(3):
             d.sh_payload[i] = _p(sh_payload[i])
             d.sh_scales[i] = _p(sh_scales[i])
+            d.sh_scales_e8m0[i] = _p(sh_scales_e8m0[i])    # all three given: an MXFP8 shared expert run as dense projections
         d.sh_rs, d.sh_cs = sh_rs, sh_cs
         d.router_gate = _p(router_gate)
         d.router_bias = _p(router_bias)
         self.cfg = cfg
-        self._keep = (sh_payload, sh_scales, router_gate, router_bias)
+        self._keep = (sh_payload, sh_scales, router_gate, router_bias, sh_scales_e8m0)
         handle = C.c_void_p()
         _check(self._lib.dgpp_moe_layer_create(C.addressof(d), C.addressof(handle)))
         self._h = handle

@@ -37,11 +37,19 @@ typedef struct DgppMoeLayerDesc {
   const uint16_t* router_gate;        /* bf16 [n_experts, hidden] (may be null when only
                                          enqueue_decode_scores is used) */
   const float* router_bias;           /* f32 [n_experts] (null in softmax mode) */
+  const uint8_t* sh_scales_e8m0[3];   /* all three non-null: the shared expert is an MXFP8 expert (E4M3 payload in
+                                         sh_payload, one E8M0 scale byte per 32 columns here; sh_scales, sh_rs and sh_cs
+                                         unused) of its OWN width shared_inter, run as dense projections over the
+                                         batch's token rows beside the routed passes (reference:
+                                         src/models/minimax/layers.cpp:34-45, 222-238) and added last to each token's
+                                         chain with weight 1, one rounding. hidden and shared_inter multiples of 32. */
 } DgppMoeLayerDesc;
 
 /* Device bytes the layer's scratch takes for max_tokens (reference: GlmMoeLayer::scratch_bytes,
  * src/models/glm/moe_layer.cpp:72-129, decode-slot and grouped buffers). */
 size_t dgpp_moe_layer_scratch_bytes(const DgppMoeConfig* cfg, int max_tokens, int shared_inter);
+/* The same for a layer whose shared expert is the dense MXFP8 form (sh_scales_e8m0 given). */
+size_t dgpp_moe_layer_scratch_bytes_dense_shared(const DgppMoeConfig* cfg, int max_tokens, int shared_inter);
 int dgpp_moe_layer_create(const DgppMoeLayerDesc* desc, DgppMoeLayer** out);
 void dgpp_moe_layer_destroy(DgppMoeLayer* layer);
 

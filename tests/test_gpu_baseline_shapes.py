@@ -167,17 +167,27 @@ def test_c4_fp8_moe_zipf(gpu):
 
 
 def test_c5_nvfp4_routed_plus_mxfp8_shared(gpu):
+    """C5 at full size. The whole layer is ONE call of the layer driver (NVFP4 routed experts in decode slots, the MXFP8
+    shared expert of its own width as dense projections beside them, combined last with weight 1): bitwise the chain
+    stitched from the loose launchers, and held to the oracle on twelve tokens spread over the batch whose routes reach
+    at least 32 distinct generated experts."""
     E, H, I, K, T, SI = 256, 6144, 2048, 8, 64, 4096
-    G = 12                                   # distinct routed experts materialised; expert e uses e % G
+    BASE, G = 10, 40                         # BASE generated experts; expert e uses variant e % G of them (variant g is
+                                             # base expert g % BASE with its rows rotated by 64 * (g // BASE): other weights)
     x = hg.normal_bf16(0xD6990050, (T, H))
     logits = hg.bf16_to_f32(hg.normal_bf16(0xD6990051, (T, E)))
     l64 = logits.astype(np.float64)
     ids, w = np.empty((T, K), np.int32), np.empty((T, K), np.float32)
     orc.oracle().orc_router_select(orc.p(l64), orc.p(l64), 1, T, E, K, 1.0, 1, orc.p(ids), orc.p(w))
-    keep, gen = [], []
+    keep, gen, base = [], [], []
+    for b in range(BASE):
+        base.append([moe_data.make_mat("nvfp4", I, H, 0xD6995000 + b * 3), moe_data.make_mat("nvfp4", I, H, 0xD6995001 + b * 3),
+                     moe_data.make_mat("nvfp4", H, I, 0xD6995002 + b * 3)])
     for g in range(G):
-        mats = [moe_data.make_mat("nvfp4", I, H, 0xD6995000 + g * 3), moe_data.make_mat("nvfp4", I, H, 0xD6995001 + g * 3),
-                moe_data.make_mat("nvfp4", H, I, 0xD6995002 + g * 3)]
+        shift = 64 * (g // BASE)
+        mats = [moe_data.Mat(m.kind, m.rows, m.cols, np.ascontiguousarray(np.roll(m.payload, shift, axis=0)),
+                             np.ascontiguousarray(np.roll(m.scales, shift, axis=0)), m.glob) if shift else m
+                for m in base[g % BASE]]
         vs = []
         for m in mats:
             pd, sd, gd = dev(m.payload), dev(m.scales), dev(m.glob)
@@ -213,8 +223,23 @@ def test_c5_nvfp4_routed_plus_mxfp8_shared(gpu):
     sync()
     got = host(out, np.uint16)
     assert np.array_equal(hg.f32_to_bf16(host(routed_g) + host(shared_down)), got), "fma(1, shared, acc) == acc + shared"
-    # two tokens against the oracle (routed NVFP4 chain + MXFP8 shared expert)
-    sample = [0, 37]
+    # the same layer as ONE driver call: a layer whose shared expert is the dense MXFP8 form
+    cfg1 = L.make_config(H, I, E, K, n_shared_experts=1, routed_scaling_factor=1.0, swiglu_limit=float("inf"),
+                         router_mode=L.ROUTER_SOFTMAX_TOPK)
+    layer1 = ML.MoeLayer(cfg1, ML.EXPERTS_NVFP4, views, T, shared_inter=SI, sh_payload=[t[0] for t in shd],
+                         sh_scales_e8m0=[t[1] for t in shd])
+    out1 = dev_empty((T, H), np.uint16)
+    layer1.enqueue_decode_scores(x_d, H, lg_d, lg_d, out1, T)
+    sync()
+    assert np.array_equal(host(out1, np.uint16), got), "one driver call == the chain stitched from the launchers, bitwise"
+    out1b = dev_empty((13, H), np.uint16)       # a smaller batch through the same layer, given routes
+    layer1.enqueue_decode_routed(x_d, H, dev(ids[:13]), dev(w[:13]), out1b, 13)
+    sync()
+    assert np.array_equal(host(out1b, np.uint16), got[:13]), "rows do not depend on the batch they ride in"
+    layer1.close()
+    # twelve tokens against the oracle (routed NVFP4 chain + MXFP8 shared expert)
+    sample = [0, 5, 11, 17, 23, 29, 34, 40, 46, 52, 58, 63]
+    assert len({int(e) % G for e in ids[sample].ravel()}) >= 32, "the sampled tokens must reach >= 32 distinct generated experts"
     orc_experts = [m.orc() for e in range(E) for m in gen[e % G][1]]
     raw, _ = orc.moe_forward(np.ascontiguousarray(x[sample]), np.ascontiguousarray(ids[sample]),
                              np.ascontiguousarray(w[sample]), H, I, SI, orc_experts, [m.orc() for m in sh],
