@@ -71,7 +71,9 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5,w8a8,qwen_tail,slotbench,readprobe ('' for none; default: c1,c2,c4,c5, none under --tune)")
+                    "separated out of c1,c2,c4,c5,c5skew,w8a8,qwen_tail,slotbench,readprobe ('' for none; default: c1,c2,c4,c5, none under --tune)")
+    ap.add_argument("--replays", type=int, default=0, help="timed graph replays per measurement (0 = at least 50 and at "
+                    "least 1000 steps; a small number keeps a run under a profiler's counters short)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
     return ap.parse_args()
 
@@ -151,7 +153,7 @@ def main():
         step, so it does not depend on how many steps one graph holds (the replays queue behind each other: a graph's
         launch set-up overlaps its predecessor's run). `stats`, when given, receives median / min / max per step in
         microseconds and the replay count. `warmup` eager steps run before the capture and one untimed replay after it."""
-        replays = max(50, -(-1000 // max(steps, 1)))
+        replays = args.replays if args.replays > 0 else max(50, -(-1000 // max(steps, 1)))
         with torch.cuda.stream(stream):
             for i in range(max(warmup, 1)):
                 enqueue(i)
@@ -382,7 +384,7 @@ def main():
             l_.close()
         return res
 
-    def bench_c5():
+    def bench_c5(skew=False):
         cE, cH, cI, cK, cT, cSI, G = 256, 6144, 2048, 8, 64, 4096, 8
         keep5, gen = [], []
         for g in range(G):    # G generated experts; the 256 table entries are device COPIES of them (own addresses)
@@ -434,6 +436,30 @@ def main():
         ids5 = torch.empty((cT, cK), dtype=torch.int32, device=dev)
         w5 = torch.empty((cT, cK), dtype=torch.float32, device=dev)
         L.launch_moe_router_select(lg5, lg5, ids5, w5, cfg5, cT, stream)
+        if skew:
+            # The same layer under Zipf(1.1) expert popularity: few experts take most tokens, so routed segments reach
+            # 16 and more rows - the shape the matrix-core grouped form is for. Routes are given (ids drawn from the
+            # popularity law, weights the renormalised softmax of N(0,1) draws); routed experts only.
+            ids_h = hg.zipf_routes(0xD6990058, 1.1, cT, cK, cE)
+            lw = hg.bf16_to_f32(hg.normal_bf16(0xD6990059, (cT, cK))).astype(np.float64)
+            wz = np.exp(lw - lw.max(1, keepdims=True))
+            wz = (wz / wz.sum(1, keepdims=True)).astype(np.float32)
+            ids_z, w_z = torch.from_numpy(ids_h).to(dev), torch.from_numpy(wz).to(dev)
+            counts = np.bincount(ids_h.ravel(), minlength=cE)
+            uz = int(np.count_nonzero(counts))
+            per_expert = 3 * cI * cH // 2 + 3 * cI * cH // 16 + 12
+            nb = uz * per_expert + cT * cH * 6
+            res = {"workload": f"C5's routed NVFP4 experts under Zipf(1.1) routing, T=64: {uz} distinct experts, busiest "
+                               f"{int(counts.max())} tokens, {int(np.count_nonzero(counts >= 16))} experts with >= 16 tokens",
+                   "algorithmic_bytes": nb, "flops": 2.0 * cT * cK * 3 * cI * cH}
+            legs = (("decode_slots", lambda i: lay.enqueue_decode_routed(x, cH, ids_z, w_z, None, cT, stream, out_f32=routed)),
+                    ("grouped_matrix_core", lambda i: lay.enqueue_prefill_routed(x, cH, ids_z, w_z, None, cT, stream, out_f32=routed)))
+            for name, fn in legs:
+                sec = time_graph(fn, max(args.steps // 10, 5), 2)
+                res[name] = {"us": sec * 1e6, "gbps": nb / sec / 1e9, "frac_of_peak": nb / sec / 1e9 / HBM_PEAK_GBPS,
+                             "tflops": res["flops"] / sec / 1e12}
+            lay.close()
+            return res
 
         def routed_mc(i):
             lay.enqueue_prefill_routed(x, cH, ids5, w5, None, cT, stream, out_f32=routed)
@@ -690,7 +716,7 @@ def main():
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
-            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail, "readprobe": bench_readprobe,
+            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "c5skew": lambda: bench_c5(True), "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail, "readprobe": bench_readprobe,
                                    "slotbench": bench_slotbench}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
