@@ -842,6 +842,7 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
   // Larger batches (many slots per expert, an order given): runs of four where the rows fit the stage.
   const int cap = run_cap_for(a, (!a.once && a.order != nullptr) ? kGateUpRunBatch : kGateUpRun);
+  hipError_t err = hipSuccess;
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
     const bool split = tune_get(kTuneSplitStage) != 1 && a.k <= 8 * kSplitStageVecs * kBlockThreads &&
@@ -850,8 +851,9 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
     const bool nt = split && a.once && !a.want_shared;
     auto go = [&](auto mc, auto sc, auto ntc) {
       constexpr int MAXM = decltype(mc)::value;
-      hipLaunchKernelGGL((slot_gate_up_kernel<FMT, NB, MAXM, decltype(sc)::value, decltype(ntc)::value>), grid,
-                         dim3(kBlockThreads), stage_bytes(MAXM, a.k), stream, a, g, steps);
+      auto kern = slot_gate_up_kernel<FMT, NB, MAXM, decltype(sc)::value, decltype(ntc)::value>;
+      err = ensure_lds(kern, stage_bytes(MAXM, a.k));   // one staged row of a wide k can exceed the default LDS ceiling
+      if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), stage_bytes(MAXM, a.k), stream, a, g, steps);
     };
     auto go_m = [&](auto mc) {
       if (nt) go(mc, std::true_type{}, std::true_type{});
@@ -864,7 +866,7 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
     if (cap >= kGateUpRun) go_m(std::integral_constant<int, kGateUpRun>{});
     else go_m(std::integral_constant<int, 1>{});
   });
-  return hipGetLastError();
+  return err != hipSuccess ? err : hipGetLastError();
 }
 
 // The fused selection + gate/up launch; the caller has checked its limits (capi.hip, select_gate_up_fits).
@@ -876,12 +878,15 @@ hipError_t launch_select_gate_up_fmt(const SlotArgs& a, const SelectArgs& sel, h
   int steps = pick_steps(per_slot * a.slots);
   if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
   const dim3 grid(static_cast<unsigned>((per_slot + steps - 1) / steps), static_cast<unsigned>(a.slots));
+  hipError_t err = hipSuccess;
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
-    hipLaunchKernelGGL((select_gate_up_kernel<FMT, NB>), grid, dim3(kBlockThreads),
-                       stage_bytes(1, a.k) + kWave * sizeof(int32_t), stream, a, sel, g, steps);
+    auto kern = select_gate_up_kernel<FMT, NB>;
+    const size_t lds = stage_bytes(1, a.k) + kWave * sizeof(int32_t);
+    err = ensure_lds(kern, lds);
+    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, sel, g, steps);
   });
-  return hipGetLastError();
+  return err != hipSuccess ? err : hipGetLastError();
 }
 
 // Row tiles (grid x) and steps of a vector-form down launch.
@@ -906,37 +911,30 @@ hipError_t launch_slot_down_fmt(const SlotArgs& a, hipStream_t stream) {
   slot_down_grid<FMT>(a, g, steps, tiles);
   const dim3 grid(tiles, static_cast<unsigned>(a.slots));
   const int cap = run_cap_for(a, kDownRun);
+  hipError_t err = hipSuccess;
+  auto launch = [&](auto kern, int rows) {
+    err = ensure_lds(kern, stage_bytes(rows, a.k));   // one staged row of a wide k can exceed the default LDS ceiling
+    if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), stage_bytes(rows, a.k), stream, a, g, steps);
+  };
   if (a.acc_out != nullptr) {   // a shared pass that ends with the token's accumulation: cached loads, every run length
     dispatch_nb(g.nb, [&](auto nbc) {
       constexpr int NB = decltype(nbc)::value;
-      if (cap >= kDownRun)
-        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, kDownRun, false, true>), grid, dim3(kBlockThreads),
-                           stage_bytes(kDownRun, a.k), stream, a, g, steps);
-      else if (cap >= 2)
-        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 2, false, true>), grid, dim3(kBlockThreads), stage_bytes(2, a.k), stream,
-                           a, g, steps);
-      else
-        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 1, false, true>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream,
-                           a, g, steps);
+      if (cap >= kDownRun) launch(slot_down_kernel<FMT, NB, kDownRun, false, true>, kDownRun);
+      else if (cap >= 2) launch(slot_down_kernel<FMT, NB, 2, false, true>, 2);
+      else launch(slot_down_kernel<FMT, NB, 1, false, true>, 1);
     });
-    return hipGetLastError();
+    return err != hipSuccess ? err : hipGetLastError();
   }
   dispatch_nb(g.nb, [&](auto nbc) {
     constexpr int NB = decltype(nbc)::value;
     dispatch_bool(a.once && !a.want_shared, [&](auto ntc) {
       constexpr bool NT = decltype(ntc)::value;
-      if (cap >= kDownRun)
-        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, kDownRun, NT>), grid, dim3(kBlockThreads), stage_bytes(kDownRun, a.k),
-                           stream, a, g, steps);
-      else if (cap >= 2)
-        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 2, NT>), grid, dim3(kBlockThreads), stage_bytes(2, a.k), stream, a, g,
-                           steps);
-      else
-        hipLaunchKernelGGL((slot_down_kernel<FMT, NB, 1, NT>), grid, dim3(kBlockThreads), stage_bytes(1, a.k), stream, a, g,
-                           steps);
+      if (cap >= kDownRun) launch(slot_down_kernel<FMT, NB, kDownRun, NT>, kDownRun);
+      else if (cap >= 2) launch(slot_down_kernel<FMT, NB, 2, NT>, 2);
+      else launch(slot_down_kernel<FMT, NB, 1, NT>, 1);
     });
   });
-  return hipGetLastError();
+  return err != hipSuccess ? err : hipGetLastError();
 }
 
 template <int FMT>

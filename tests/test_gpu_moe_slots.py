@@ -371,3 +371,15 @@ def test_slot_ex_passes_and_folded_accumulation_are_bitwise_the_plain_launchers(
     routed = np.array([s for s in range(slots) if s % (K + 1) != K])
     assert np.array_equal(got_down[routed].view(np.uint32), down_ref[routed].view(np.uint32))
     assert np.array_equal(host(out_d, np.uint16), out_ref)
+
+
+def test_fp8_slot_kernels_stage_a_row_wider_than_the_default_lds_ceiling(gpu):
+    """An FP8 slot launch whose hidden row (k = 40960: 80 KB staged) needs more dynamic LDS than a block gets without
+    opting in: the launchers raise the kernel's ceiling themselves (a CU has 160 KB) instead of failing at launch."""
+    E, H, I, K, T = 2, 40960, 32, 1, 2
+    p = moe_data.make_problem(E, H, I, K, T, "fp8", 4711, shared_kind=None, limit=float("inf"), std=0.02)
+    d = DeviceMoe(p)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    act, down, out = run_slot_path(p, d, ids, w)
+    raw, _ = moe_data.orc_forward(p, ids, w)
+    expert_budget(out, raw, "k = 40960 FP8 slots")
