@@ -119,6 +119,11 @@ SIGNATURES = {
     "dgpp_qwen_moe_shared_tail_decode_fp8": (_I, [_P, _Z, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_qwen_moe_shared_tail_decode_routed_fp8": (_I, [_P, _Z, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I,
                                                          _I, _P, _I, _I]),
+    "dgpp_nvfp4_act_scale_stride": (C.c_size_t, [_I]),
+    "dgpp_launch_quantize_rows_nvfp4": (_I, [_P, _Z, _I, _I, _P, _P, _P, _P, _F, _P]),
+    "dgpp_launch_swiglu_quantize_rows_nvfp4": (_I, [_P, _P, _Z, _I, _I, _F, _P, _P, _P, _P, _F, _P, _I]),
+    "dgpp_launch_moe_grouped_w4a4_bf16": (_I, [_P, _P, _P, _P, _P, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
+    "dgpp_launch_moe_grouped_w4a4_f32": (_I, [_P, _P, _P, _P, _P, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
     "dgpp_launch_mxfp8_quantize_rows": (_I, [_P, _Z, _I, _I, _P, _P, _P]),
     "dgpp_launch_minimax_swiglu_mxfp8_rows": (_I, [_P, _P, _Z, _I, _I, _F, _F, _P, _P, _P]),
     "dgpp_launch_mxfp8_gemm_bf16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _I]),

@@ -27,6 +27,7 @@ HIP_SOURCES = [
     "moe_grouping.hip",
     "moe_elementwise.hip",
     "mxfp8_gemm.hip",
+    "nvfp4_act.hip",
     "qwen_tail.hip",
     "capi.hip",
 ]

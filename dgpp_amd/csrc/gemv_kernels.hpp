@@ -573,6 +573,10 @@ struct GroupedArgs {
                             // launch; 2 = gate rows to `out`, up rows to `out_up`
   float limit;              // the SwiGLU clamp of form 1
   void* out_up;             // form 2
+  // matrix-core form, NVFP4 experts: the activations are NVFP4 rows (act = codes, act_stride = bytes per row)
+  const uint8_t* a4_scales = nullptr;   // e4m3 [rows, a4_scale_stride]
+  size_t a4_scale_stride = 0;
+  const float* a4_gs = nullptr;         // [rows]
 };
 
 template <int FMT, int NB, bool NT>
@@ -721,6 +725,17 @@ hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipS
   const MGeom g = mgeom<FMT>(a.k);
   const dim3 grid(static_cast<unsigned>((a.n + 63) / 64), static_cast<unsigned>(n_segs), static_cast<unsigned>(z_ext));
   hipError_t err = hipSuccess;
+  if constexpr (FMT == kFmtNvfp4) {
+    if (a.a4_scales != nullptr) {   // the activation-quantized form
+      dispatch_bool(a.once != 0, [&](auto ntc) {
+        auto kern = mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value, false, true>;
+        constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
+        err = ensure_lds(kern, lds);
+        if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g);
+      });
+      return err != hipSuccess ? err : hipGetLastError();
+    }
+  }
   dispatch_bool(a.once != 0, [&](auto ntc) {
     dispatch_bool(a.gate_up != 0, [&](auto guc) {
       auto kern = mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value, decltype(guc)::value>;

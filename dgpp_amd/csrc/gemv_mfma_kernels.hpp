@@ -20,15 +20,44 @@ constexpr int kMfmaNB = 4;          // lane loads in flight per row group and pa
 // in ascending order. `act_rows`, when given, names the activation row of each of the mt rows (a gather
 // folded into the stage load). LDS: the stage, then one tile region per wavefront. Every thread of the
 // block must call.
+// Activation rows that arrive already quantized to NVFP4 (the W4A4 form): e2m1 codes [rows, k / 2], one e4m3 scale per
+// 16 elements [rows, scale_stride]; the row's fp32 global is applied by the caller's epilogue. A row's eight-element
+// block decodes to eight BF16 values exactly (e2m1 x e4m3 needs six significant bits), so the matrix core multiplies
+// the same numbers a block-scaled FP4 x FP4 instruction would.
+struct A4Src {
+  const uint8_t* scales = nullptr;
+  size_t scale_stride = 0;
+  int row_base = 0;   // row of activation 0 when no row list is given
+};
+__device__ __forceinline__ uint4 load_act_block_nvfp4(const uint8_t* __restrict__ codes_row, const uint8_t* __restrict__ scale_row,
+                                                      int k0, int k) {
+  if (k0 >= k) return make_uint4(0u, 0u, 0u, 0u);
+  const uint32_t codes = *reinterpret_cast<const uint32_t*>(codes_row + (k0 >> 1));
+  const float s = __builtin_amdgcn_cvt_f32_fp8(static_cast<uint32_t>(scale_row[k0 >> 4]), 0);
+  uint32_t o[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    f32x2_t v;
+    if (q == 0) v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 0);
+    else if (q == 1) v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 1);
+    else if (q == 2) v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 2);
+    else v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 3);
+    o[q] = __builtin_bit_cast(uint32_t, pack_bf16(v.x * s, v.y * s));
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 constexpr int kTileBatch = 2;   // 8 KB in flight per wavefront; more tiles cost registers, and blocks per CU count for more
 constexpr int kBlockMfmaLdsUnits = kStageUnits + kWavesPerBlock * kTileUnits;
 
-template <int FMT, int NB, bool NT, bool SW = false>
+// A4: `act` holds NVFP4 codes (act_stride in BYTES) described by `a4`; the rows are then named by act_rows or start at
+// a4.row_base.
+template <int FMT, int NB, bool NT, bool SW = false, bool A4 = false>
 __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_t* __restrict__ act, size_t act_stride,
                                                 const int32_t* __restrict__ act_rows, int mt, int n, int k, int row0,
                                                 const MGeom& g, int p_lo, int p_hi, uint4* __restrict__ lds,
                                                 f32x4_t& sum, const uint16_t* __restrict__ act_up = nullptr,
-                                                float limit = 0.f) {
+                                                float limit = 0.f, const A4Src a4 = A4Src()) {
   static_assert(NB == 4, "a tile is four steps");
   constexpr int kSub = MTraits<FMT>::kSub;
   constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
@@ -53,7 +82,10 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
     const int idx = threadIdx.x + i * kBlockThreads;
     const int kb = idx / mt, c = idx - kb * mt;
     unit_kb[i] = kb;
-    unit_row[i] = (act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(c)) * act_stride;
+    if constexpr (A4)   // the row itself: codes and scales have different strides
+      unit_row[i] = act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(a4.row_base + c);
+    else
+      unit_row[i] = (act_rows ? static_cast<size_t>(act_rows[c]) : static_cast<size_t>(c)) * act_stride;
   }
   f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
   for (int t0 = p_lo * cpp; t0 < t_hi; t0 += batch) {
@@ -76,7 +108,11 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
     for (int i = 0; i < kStageRegs; ++i) {
       pre[i] = make_uint4(0u, 0u, 0u, 0u);
       if (threadIdx.x + i * kBlockThreads < units) {
-        pre[i] = load_act_block(act + unit_row[i], k_base + unit_kb[i] * 8, k, aligned);
+        if constexpr (A4)
+          pre[i] = load_act_block_nvfp4(reinterpret_cast<const uint8_t*>(act) + unit_row[i] * act_stride,
+                                        a4.scales + unit_row[i] * a4.scale_stride, k_base + unit_kb[i] * 8, k);
+        else
+          pre[i] = load_act_block(act + unit_row[i], k_base + unit_kb[i] * 8, k, aligned);
         if constexpr (SW)   // the activation is SwiGLU(act, act_up), computed on its way into the stage
           pre[i] = swiglu_bf16x8(pre[i], load_act_block(act_up + unit_row[i], k_base + unit_kb[i] * 8, k, aligned), limit);
       }
@@ -168,7 +204,9 @@ __global__ void fold_parts_kernel(const float* __restrict__ partials, int parts,
 
 // GU: the block computes its rows of the segment's gate AND up matrices (two walks over K, the same
 // activations) and stores SwiGLU(bf16(gate), bf16(up)) — the bits of two launches and the elementwise kernel.
-template <int FMT, int NB, bool NT, bool GU>
+// A4 (NVFP4 experts only, GU false): the activations are NVFP4 rows (a.act the codes, a.act_stride bytes per row,
+// a.a4_scales / a.a4_gs); out = acc * (gs[row] * (1 / global)), the reference's epilogue (src/kernels/moe_w4a4.cu:424).
+template <int FMT, int NB, bool NT, bool GU, bool A4 = false>
 __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedArgs a, MGeom g) {
   extern __shared__ uint4 lds[];
   const DgppMoeSegment seg = a.segs[blockIdx.y];
@@ -214,6 +252,19 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
         for (int i = 0; i < 4; ++i)
           if (r + i < a.n)
             out[r + i] = swiglu_bf16(finish_dot<FMT>(sum[i], divisor), finish_dot<FMT>(sum_up[i], divisor_up), a.limit);
+      }
+    } else if constexpr (A4) {
+      A4Src src;
+      src.scales = a.a4_scales;
+      src.scale_stride = a.a4_scale_stride;
+      src.row_base = static_cast<int>(first);
+      block_rows_mfma<FMT, NB, NT, false, true>(mat, a.act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum,
+                                                nullptr, 0.f, src);
+      if (c < mt) {
+        const size_t arow = rows ? static_cast<size_t>(rows[c]) : first + c;
+        const float mul = a.a4_gs[arow] * (1.0f / divisor);
+        const f32x4_t scaled = {sum[0] * mul, sum[1] * mul, sum[2] * mul, sum[3] * mul};
+        store_tile<kFmtMxfp4>(scaled, 1.0f, a.out, a.out_f32, (first + c) * a.out_stride, row0, a.n, true);
       }
     } else {
       block_rows_mfma<FMT, NB, NT>(mat, act, a.act_stride, rows, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum);

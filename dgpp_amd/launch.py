@@ -553,3 +553,32 @@ def launch_mma_gemv_fp4_bf16_static(act, act_stride, w: Fp4Matrix, out, m, n, k,
 def launch_mma_gemv_fp4_f32(act, act_stride, w: Fp4Matrix, out, m, n, k, out_stride=0, stream=None, ws=None, ws_bytes=0):
     _check(_lib.load().dgpp_launch_mma_gemv_fp4_f32(_p(act), act_stride, C.addressof(w), _p(out), m, n, k, out_stride,
                                                     _stream(stream), _p(ws), ws_bytes))
+
+
+# ---- activation-quantized NVFP4 (W4A4) form: src/kernels/moe_w4a4.hpp ------------------------------------------------
+def nvfp4_act_scale_stride(k: int) -> int:
+    return _lib.load().dgpp_nvfp4_act_scale_stride(k)
+
+
+def launch_quantize_rows_nvfp4(x, x_stride, rows, k, codes, scales, gs, stream=None, static_gs=0.0, static_gs_dev=None):
+    _check(_lib.load().dgpp_launch_quantize_rows_nvfp4(_p(x), x_stride, rows, k, _p(codes), _p(scales), _p(gs), _stream(stream),
+                                                       static_gs, _p(static_gs_dev)))
+
+
+def launch_swiglu_quantize_rows_nvfp4(gate, up, stride, rows, k, limit, codes, scales, gs, stream=None, static_gs=0.0,
+                                      static_gs_dev=None, qwen_rounding=False):
+    _check(_lib.load().dgpp_launch_swiglu_quantize_rows_nvfp4(_p(gate), _p(up), stride, rows, k, limit, _p(codes), _p(scales),
+                                                              _p(gs), _stream(stream), static_gs, _p(static_gs_dev),
+                                                              1 if qwen_rounding else 0))
+
+
+def launch_moe_grouped_w4a4_bf16(codes, scales, gs, act_rows, segs, n_segs, max_rows, views, which, out, out_stride, n, k,
+                                 stream=None):
+    _check(_lib.load().dgpp_launch_moe_grouped_w4a4_bf16(_p(codes), _p(scales), _p(gs), _p(act_rows), _p(segs), n_segs, max_rows,
+                                                         _p(views), which, _p(out), out_stride, n, k, _stream(stream)))
+
+
+def launch_moe_grouped_w4a4_f32(codes, scales, gs, act_rows, segs, n_segs, max_rows, views, which, out, out_stride, n, k,
+                                stream=None):
+    _check(_lib.load().dgpp_launch_moe_grouped_w4a4_f32(_p(codes), _p(scales), _p(gs), _p(act_rows), _p(segs), n_segs, max_rows,
+                                                        _p(views), which, _p(out), out_stride, n, k, _stream(stream)))

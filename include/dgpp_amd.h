@@ -483,6 +483,40 @@ int dgpp_launch_fp8_dequant_blocks_e8m0(const uint8_t* payload, const uint8_t* s
                                         uint16_t* out_bf16, int64_t rows, int64_t cols,
                                         void* stream, int rs, int cs);
 
+/* ---- activation-quantized NVFP4 (W4A4) form ---------------------------------------------------------------------
+ * The NVFP4 experts meet activations quantized to NVFP4 on the fly (per row a fp32 global gs, per 16 elements an e4m3
+ * scale, e2m1 codes: x ~= e2m1 * scale * gs). Its numerics are those of src/kernels/moe_w4a4.cu, not of the
+ * BF16-activation launchers above: the activations carry NVFP4 rounding. The quantizers reproduce the reference's
+ * recipe bit for bit (a chain of single IEEE fp32 operations). The GEMM multiplies the exactly decoded operands on the
+ * BF16 matrix core with FP32 accumulation (this chip's block-scaled FP4 instruction takes one power-of-two scale per 32
+ * elements; NVFP4 carries an e4m3 per 16) and is held, like the reference's kernel, to the fp64 dot of the same
+ * quantized operands: |got - dot| < 1e-5 * sum |terms| (tests/cuda/moe_w4a4_test.cu:193-216). */
+/* src/kernels/moe_w4a4.hpp:15, moe_w4a4.cu:596: the activation scale buffer's row stride in bytes: k / 16 rounded up to 8. */
+size_t dgpp_nvfp4_act_scale_stride(int k);
+/* src/kernels/moe_w4a4.hpp:17-26, moe_w4a4.cu:598-611: BF16 rows [rows, k] (stride x_stride elements, a multiple of 8;
+ * 16-byte aligned) -> codes [rows, k / 2] (low nibble = even element; 8-byte aligned), scales [rows,
+ * dgpp_nvfp4_act_scale_stride(k)], gs [rows]. The global is *static_gs_dev when that DEVICE pointer is given, else
+ * static_gs; a global <= 0 means amax / (6 * 448) per row (1 for a zero row); what exceeds 6 * 448 * gs saturates.
+ * k a multiple of 64, <= 32768. */
+int dgpp_launch_quantize_rows_nvfp4(const uint16_t* x, size_t x_stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                    float* gs, void* stream, float static_gs, const float* static_gs_dev);
+/* src/kernels/moe_w4a4.hpp:27-35, moe_w4a4.cu:613-634: the same with the activation computed on the way - the MoE's
+ * SwiGLU of (gate, up) with its clamp and two BF16 roundings (dgpp_launch_moe_swiglu_clamp's arithmetic), or with
+ * qwen_rounding != 0 the dense MLP's of the Qwen family (silu as g / (1 + exp(-g)), one rounding of the product, no
+ * clamp) - bitwise the activation kernel followed by the quantizer. */
+int dgpp_launch_swiglu_quantize_rows_nvfp4(const uint16_t* gate, const uint16_t* up, size_t stride, int rows, int k,
+                                           float limit, uint8_t* codes, uint8_t* scales, float* gs, void* stream,
+                                           float static_gs, const float* static_gs_dev, int qwen_rounding);
+/* src/kernels/moe_w4a4.hpp:37-49, moe_w4a4.cu:636-715: out[seg.row0 + m, :n] = act(row) . W(expert, which)^T for every
+ * segment, act(row) the quantized row act_rows[seg.row0 + m] (or seg.row0 + m when act_rows is null); out = acc *
+ * (gs[row] * (1 / global)). Segment / view / out conventions of dgpp_launch_moe_grouped_mma_fp4_*; k a multiple of 64. */
+int dgpp_launch_moe_grouped_w4a4_bf16(const uint8_t* codes, const uint8_t* scales, const float* gs, const int32_t* act_rows,
+                                      const DgppMoeSegment* segs, int n_segs, int max_rows, const DgppMoeExpertView* views,
+                                      int which, uint16_t* out, size_t out_stride, int n, int k, void* stream);
+int dgpp_launch_moe_grouped_w4a4_f32(const uint8_t* codes, const uint8_t* scales, const float* gs, const int32_t* act_rows,
+                                     const DgppMoeSegment* segs, int n_segs, int max_rows, const DgppMoeExpertView* views,
+                                     int which, float* out, size_t out_stride, int n, int k, void* stream);
+
 /* ---- activation-quantized MXFP8 (W8A8) form ---------------------------------------------------------------------
  * The weights' MXFP8 payload meets activations quantized to MXFP8 on the fly; the products run on the
  * block-scaled matrix-core instruction (V_MFMA_SCALE_F32_16X16X128_F8F6F4, e8m0 scale per 32 values of

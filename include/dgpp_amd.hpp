@@ -453,6 +453,33 @@ inline void qwen_moe_shared_tail_decode_routed_fp8(const uint16_t* x, size_t x_s
   detail::check(dgpp_qwen_moe_shared_tail_decode_routed_fp8(x, x_stride, gate_p, gate_s, up_p, up_s, down_p, down_s, g, act, sw,
                                                             contrib, weights, top_k, out, tokens, H, S, stream, rs, cs));
 }
+// ---- activation-quantized NVFP4 (W4A4) form: src/kernels/moe_w4a4.hpp ----
+inline size_t nvfp4_act_scale_stride(int k) { return dgpp_nvfp4_act_scale_stride(k); }
+inline void launch_quantize_rows_nvfp4(const uint16_t* x, size_t x_stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                       float* gs, hipStream_t stream, float static_gs = 0.f,
+                                       const float* static_gs_dev = nullptr) {
+  detail::check(dgpp_launch_quantize_rows_nvfp4(x, x_stride, rows, k, codes, scales, gs, stream, static_gs, static_gs_dev));
+}
+inline void launch_swiglu_quantize_rows_nvfp4(const uint16_t* gate, const uint16_t* up, size_t stride, int rows, int k,
+                                              float limit, uint8_t* codes, uint8_t* scales, float* gs, hipStream_t stream,
+                                              float static_gs, const float* static_gs_dev = nullptr,
+                                              bool qwen_rounding = false) {
+  detail::check(dgpp_launch_swiglu_quantize_rows_nvfp4(gate, up, stride, rows, k, limit, codes, scales, gs, stream, static_gs,
+                                                       static_gs_dev, qwen_rounding ? 1 : 0));
+}
+inline void launch_moe_grouped_w4a4_bf16(const uint8_t* codes, const uint8_t* scales, const float* gs, const int32_t* act_rows,
+                                         const MoeSegment* segs, int n_segs, int max_rows, const MoeExpertView* views,
+                                         int which, uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_grouped_w4a4_bf16(codes, scales, gs, act_rows, segs, n_segs, max_rows, views, which, out,
+                                                  out_stride, n, k, stream));
+}
+inline void launch_moe_grouped_w4a4_f32(const uint8_t* codes, const uint8_t* scales, const float* gs, const int32_t* act_rows,
+                                        const MoeSegment* segs, int n_segs, int max_rows, const MoeExpertView* views,
+                                        int which, float* out, size_t out_stride, int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_grouped_w4a4_f32(codes, scales, gs, act_rows, segs, n_segs, max_rows, views, which, out,
+                                                 out_stride, n, k, stream));
+}
+
 // src/kernels/mxfp8_gemm.hpp:11-31.
 inline void launch_mxfp8_quantize_rows(const uint16_t* x, size_t x_stride, int rows, int k, uint8_t* codes, uint8_t* scales,
                                        hipStream_t stream) {

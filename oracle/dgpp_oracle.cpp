@@ -507,6 +507,71 @@ void orc_shared_gate(const uint16_t* x, int64_t x_stride, const uint16_t* g, int
   }
 }
 
+// ---- activation-quantized NVFP4 form -----------------------------------------------------------
+// src/kernels/moe_w4a4.cu:139-236: per row a global, per 16 elements an e4m3 scale, e2m1 codes. Plain fp32 operations
+// in the reference's order (this file is compiled with -ffp-contract=off).
+void orc_nvfp4_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, float static_gs, uint8_t* codes,
+                             uint8_t* scales, int64_t scale_stride, float* gs) {
+  const int groups = k / 16;
+  for (int r = 0; r < rows; ++r) {
+    const uint16_t* src = x + static_cast<size_t>(r) * stride;
+    float row_amax = 0.f;
+    for (int c = 0; c < k; ++c) row_amax = std::max(row_amax, std::fabs(orc_bf16_to_f32(src[c])));
+    const float global = static_gs > 0.f ? static_gs : (row_amax > 0.f ? row_amax / (6.f * 448.f) : 1.f);
+    gs[r] = global;
+    for (int g = 0; g < groups; ++g) {
+      float gmax = 0.f;
+      for (int i = 0; i < 16; ++i) gmax = std::max(gmax, std::fabs(orc_bf16_to_f32(src[g * 16 + i])));
+      uint8_t* code = codes + static_cast<size_t>(r) * (k / 2) + static_cast<size_t>(g) * 8;
+      const uint8_t sb = orc_f32_to_e4m3(gmax / (6.f * global));
+      const float bs = orc_e4m3_to_f32(sb);
+      if (gmax == 0.f || bs == 0.f) {
+        scales[static_cast<size_t>(r) * scale_stride + g] = 0;
+        for (int i = 0; i < 8; ++i) code[i] = 0;
+        continue;
+      }
+      scales[static_cast<size_t>(r) * scale_stride + g] = sb;
+      const float q = 1.f / (bs * global);
+      for (int i = 0; i < 8; ++i) {
+        const uint8_t lo = orc_f32_to_e2m1(orc_bf16_to_f32(src[g * 16 + 2 * i]) * q);
+        const uint8_t hi = orc_f32_to_e2m1(orc_bf16_to_f32(src[g * 16 + 2 * i + 1]) * q);
+        code[i] = static_cast<uint8_t>(lo | (hi << 4));
+      }
+    }
+  }
+}
+
+void orc_w4a4_gemm(const uint8_t* a_codes, const uint8_t* a_scales, int64_t a_scale_stride, const float* a_gs,
+                   const uint8_t* w_codes, const uint8_t* w_scales, double w_global, int m, int n, int k, double* out,
+                   double* out_abs) {
+  std::vector<double> a(static_cast<size_t>(m) * k), w(static_cast<size_t>(n) * k);
+  for (int r = 0; r < m; ++r)
+    for (int c = 0; c < k; ++c) {
+      const uint8_t b = a_codes[static_cast<size_t>(r) * (k / 2) + c / 2];
+      a[static_cast<size_t>(r) * k + c] = static_cast<double>(orc_e2m1_to_f32(c % 2 ? b >> 4 : b & 15)) *
+                                          static_cast<double>(orc_e4m3_to_f32(a_scales[static_cast<size_t>(r) * a_scale_stride + c / 16])) *
+                                          static_cast<double>(a_gs[r]);
+    }
+  for (int r = 0; r < n; ++r)
+    for (int c = 0; c < k; ++c) {
+      const uint8_t b = w_codes[static_cast<size_t>(r) * (k / 2) + c / 2];
+      w[static_cast<size_t>(r) * k + c] = static_cast<double>(orc_e2m1_to_f32(c % 2 ? b >> 4 : b & 15)) *
+                                          static_cast<double>(orc_e4m3_to_f32(w_scales[static_cast<size_t>(r) * (k / 16) + c / 16])) /
+                                          w_global;
+    }
+  for (int r = 0; r < m; ++r)
+    for (int c = 0; c < n; ++c) {
+      double dot = 0.0, mag = 0.0;
+      for (int kk = 0; kk < k; ++kk) {
+        const double t = a[static_cast<size_t>(r) * k + kk] * w[static_cast<size_t>(c) * k + kk];
+        dot += t;
+        mag += std::fabs(t);
+      }
+      out[static_cast<size_t>(r) * n + c] = dot;
+      if (out_abs) out_abs[static_cast<size_t>(r) * n + c] = mag;
+    }
+}
+
 // ---- activation-quantized MXFP8 form ---------------------------------------------------------
 
 void orc_mxfp8_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, uint8_t* codes, uint8_t* scales) {

@@ -164,6 +164,25 @@ void orc_swiglu_oai(const uint16_t* gate, const uint16_t* up, int64_t stride, in
 void orc_mxfp8_gemm(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w, const uint8_t* w_scales, int m, int n, int k,
                     double* out, double* out_abs);
 
+/* ---- activation-quantized NVFP4 form (W4A4: the activations carry NVFP4 rounding) ---- */
+/* BF16 x [rows, k] (row stride in elements) -> e2m1 codes [rows, k / 2] (low nibble = even element), e4m3 block scales
+ * [rows, scale_stride] (one per 16 elements), gs[rows]: x ~= e2m1 * scale * gs. The row's global is static_gs when > 0
+ * (what exceeds 6 * 448 * gs saturates), else amax / (6 * 448) (1 for a zero row); a block's scale is
+ * e4m3_rne_sat(amax16 / (6 * gs)); codes are e2m1_rne_sat(x * (1 / (scale * gs))); a zero block or a zero scale
+ * gives scale byte 0 and codes 0. Every operation is a single IEEE fp32 operation in the reference
+ * (src/kernels/moe_w4a4.cu:139-236), so the restatement is bit-exact by construction.
+ * Pinned by the reference test's known-answer rows (values representable under scale 0.25 and a static global of 1 come
+ * back bit for bit, tests/cuda/moe_w4a4_test.cu:291-326), closed-form points (zero rows, saturation at 6 * 448 * gs)
+ * and an independent numpy float32 evaluation of the same recipe; the conversions are orc_f32_to_e4m3 / orc_f32_to_e2m1. */
+void orc_nvfp4_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, float static_gs, uint8_t* codes,
+                             uint8_t* scales, int64_t scale_stride, float* gs);
+/* out[m, n] = (sum_k e2m1(a) e4m3(sa) * e2m1(w) e4m3(sw)) * gs[m] / w_global in double, and (nullable) the same sum of
+ * magnitudes: the fp64 dot of the SAME quantized operands the reference's kernel test compares against
+ * (tests/cuda/moe_w4a4_test.cu:193-216, bound |got - dot| < 1e-5 * sum|terms|). Pinned by numpy brute force. */
+void orc_w4a4_gemm(const uint8_t* a_codes, const uint8_t* a_scales, int64_t a_scale_stride, const float* a_gs,
+                   const uint8_t* w_codes, const uint8_t* w_scales, double w_global, int m, int n, int k, double* out,
+                   double* out_abs);
+
 /* ---- comparators ---------------------------------------------------------------- */
 typedef struct {
   double l2_rel;
