@@ -85,6 +85,8 @@ SIGNATURES = {
     "dgpp_minimax_compact_segments": (_I, [_P, _P, _I, _I, _P]),
     "dgpp_launch_moe_accum_ordered": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _I, _P]),
     "dgpp_launch_moe_accum_ordered_f32": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "dgpp_launch_moe_accum_ordered_bf16down": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _P]),
+    "dgpp_launch_moe_accum_ordered_f32_bf16down": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _P]),
     "dgpp_launch_moe_slot_accum": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dgpp_launch_moe_slot_accum_routed_f32": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dgpp_launch_moe_slot_accum_routed_bf16": (_I, [_P, _P, _P, _I, _I, _I, _P]),
@@ -124,6 +126,10 @@ SIGNATURES = {
     "dgpp_launch_swiglu_quantize_rows_nvfp4": (_I, [_P, _P, _Z, _I, _I, _F, _P, _P, _P, _P, _F, _P, _I]),
     "dgpp_launch_moe_grouped_w4a4_bf16": (_I, [_P, _P, _P, _P, _P, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
     "dgpp_launch_moe_grouped_w4a4_f32": (_I, [_P, _P, _P, _P, _P, _I, _I, _P, _I, _P, _Z, _I, _I, _P]),
+    "dgpp_dense_w4a4_supported": (_I, [_I]),
+    "dgpp_launch_dense_w4a4_bf16": (_I, [_P, _P, _Z, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _P]),
+    "dgpp_minimax_quantize_rows_nvfp4": (_I, [_P, _Z, _I, _I, _P, _P, _P, _P]),
+    "dgpp_minimax_swiglu_f32": (_I, [_P, _P, _P, C.c_int64, _F, _F, _P]),
     "dgpp_launch_mxfp8_quantize_rows": (_I, [_P, _Z, _I, _I, _P, _P, _P]),
     "dgpp_launch_minimax_swiglu_mxfp8_rows": (_I, [_P, _P, _Z, _I, _I, _F, _F, _P, _P, _P]),
     "dgpp_launch_mxfp8_gemm_bf16": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _P, _Z, _I]),

@@ -509,15 +509,25 @@ int dgpp_minimax_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* o
   return finish(run_compact_segments(input, output, experts, capacity, as_stream(stream)), "minimax_compact_segments");
 }
 
-static int accum_ordered(void* out, int out_f32, const float* down, size_t down_stride, const int32_t* slot_row,
+static int accum_ordered(void* out, int out_f32, const void* down, size_t down_stride, const int32_t* slot_row,
                          const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens, int top_k,
-                         int hidden, void* stream) {
+                         int hidden, void* stream, int down_bf16 = 0) {
   if (tokens <= 0) return DGPP_OK;
   if (!out || !down || !slot_row || !slot_ids || !slot_w) return fail_arg("moe accum ordered: null pointer");
   if (top_k < 1 || top_k > 16) return fail_arg("moe accum ordered: top_k outside [1, 16]");
-  return finish(run_accum_ordered(out, out_f32, down, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens,
+  return finish(run_accum_ordered(out, out_f32, down, down_bf16, down_stride, slot_row, slot_ids, slot_w, shared_row0, tokens,
                                   top_k, hidden, as_stream(stream)),
                 "moe accum ordered");
+}
+int dgpp_launch_moe_accum_ordered_bf16down(uint16_t* out, const uint16_t* down, size_t down_stride, const int32_t* slot_row,
+                                           const int32_t* slot_ids, const float* slot_w, int tokens, int top_k, int hidden,
+                                           void* stream) {
+  return accum_ordered(out, 0, down, down_stride, slot_row, slot_ids, slot_w, -1, tokens, top_k, hidden, stream, 1);
+}
+int dgpp_launch_moe_accum_ordered_f32_bf16down(float* out, const uint16_t* down, size_t down_stride, const int32_t* slot_row,
+                                               const int32_t* slot_ids, const float* slot_w, int tokens, int top_k, int hidden,
+                                               void* stream) {
+  return accum_ordered(out, 1, down, down_stride, slot_row, slot_ids, slot_w, -1, tokens, top_k, hidden, stream, 1);
 }
 int dgpp_launch_moe_accum_ordered(uint16_t* out, const float* down, size_t down_stride, const int32_t* slot_row,
                                   const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens,

@@ -64,6 +64,11 @@ struct DenseArgs {
   // matrix-core form only: the activation is SwiGLU(act, act_up) with this clamp, computed as the rows are staged
   const uint16_t* act_up = nullptr;
   float limit = 0.f;
+  // matrix-core form, NVFP4 only: `act` holds NVFP4 activation codes (act_stride in BYTES) with these scale rows and
+  // per-row globals (the W4A4 form)
+  const uint8_t* a4_scales = nullptr;
+  size_t a4_scale_stride = 0;
+  const float* a4_gs = nullptr;
 };
 
 template <int FMT, int MAXR, int NB, bool NT>
@@ -697,7 +702,8 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
   const MGeom g = mgeom<FMT>(a.k);
   const unsigned gx = static_cast<unsigned>((a.n + 63) / 64), gy = static_cast<unsigned>((a.m + kTileCols - 1) / kTileCols);
   const size_t need = static_cast<size_t>(g.parts) * a.m * a.n * sizeof(float);
-  const bool split = ws != nullptr && g.parts > 1 && ws_bytes >= need && static_cast<size_t>(gx) * gy < 1024;
+  const bool split = ws != nullptr && g.parts > 1 && ws_bytes >= need && static_cast<size_t>(gx) * gy < 1024 &&
+                     a.a4_scales == nullptr;
   const dim3 grid(gx, gy, split ? g.parts : 1);
   hipError_t err = hipSuccess;
   dispatch_bool(a.once != 0, [&](auto ntc) {
@@ -708,6 +714,9 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
     };
     if constexpr (FMT == kFmtFp8F32) {   // the SwiGLU-staging form exists for the reference's one launcher of it
       if (a.act_up) return go(mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value, true>);
+    }
+    if constexpr (FMT == kFmtNvfp4) {    // the activation-quantized form (never split: its epilogue is its own)
+      if (a.a4_scales) return go(mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value, false, true>);
     }
     go(mfma_dense_kernel<FMT, kMfmaNB, decltype(ntc)::value, false>);
   });

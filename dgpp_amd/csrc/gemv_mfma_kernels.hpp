@@ -159,7 +159,8 @@ __device__ __forceinline__ void store_tile(const f32x4_t& v, float divisor, void
 // `partials` null: all parts in one block, folded and stored. Otherwise blockIdx.z names the ONE part
 // this block computes and its raw sums go to partials[part][row of out][n] (fp32); fold_parts_kernel
 // then adds the parts in the same ascending order — the split form's bits are the unsplit form's.
-template <int FMT, int NB, bool NT, bool SW>
+// A4 (NVFP4 weights, unsplit only): NVFP4 activation rows, the grouped W4A4 kernel's walk and epilogue over rows c0...
+template <int FMT, int NB, bool NT, bool SW, bool A4 = false>
 __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs a, MGeom g, float* partials) {
   extern __shared__ uint4 lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
@@ -168,6 +169,20 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs 
   const int mt = min(kTileCols, a.m - c0);
   const int c = lane & 15;
   f32x4_t sum;
+  if constexpr (A4) {
+    A4Src src;
+    src.scales = a.a4_scales;
+    src.scale_stride = a.a4_scale_stride;
+    src.row_base = c0;
+    block_rows_mfma<FMT, NB, NT, false, true>(a.mat, a.act, a.act_stride, nullptr, mt, a.n, a.k, row0, g, 0, g.parts, lds, sum,
+                                              nullptr, 0.f, src);
+    if (c < mt) {
+      const float mul = a.a4_gs[c0 + c] * (1.0f / load_divisor<FMT>(a.global));
+      const f32x4_t scaled = {sum[0] * mul, sum[1] * mul, sum[2] * mul, sum[3] * mul};
+      store_tile<kFmtMxfp4>(scaled, 1.0f, a.out, a.out_f32, static_cast<size_t>(c0 + c) * a.out_stride, row0, a.n, true);
+    }
+    return;
+  }
   if (partials == nullptr) {
     block_rows_mfma<FMT, NB, NT, SW>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n,
                                  a.k, row0, g, 0, g.parts, lds, sum,

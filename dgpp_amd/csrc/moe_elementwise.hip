@@ -119,6 +119,7 @@ struct ChainArgs {
   const float* weights;      // [tokens, K]
   int shared;                // slot layout: 0 / 1; grouped layout: shared_row0 (< 0: none)
   int K, hidden;
+  int src_bf16 = 0;          // the rows at `src` are BF16 (stride in BF16 elements), widened exactly as they are read
 };
 
 template <int KMAX, bool VEC, bool GROUPED, bool F32>
@@ -154,6 +155,18 @@ __global__ __launch_bounds__(kWaveLanes) void token_chain_kernel(ChainArgs a) {
   const bool live = col < a.hidden;
   float v[KMAX + 1][4];
   auto fetch = [&](int row, float (&dst)[4]) {
+    if (a.src_bf16) {
+      const uint16_t* h = reinterpret_cast<const uint16_t*>(a.src) + static_cast<size_t>(row) * a.src_stride + col;
+      if constexpr (VEC) {
+        const uint2 q = live ? *reinterpret_cast<const uint2*>(h) : make_uint2(0u, 0u);
+        dst[0] = bits_f32(q.x << 16), dst[1] = bits_f32(q.x & 0xFFFF0000u);
+        dst[2] = bits_f32(q.y << 16), dst[3] = bits_f32(q.y & 0xFFFF0000u);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[i] = col + i < a.hidden ? bf16_to_f32(h[i]) : 0.f;
+      }
+      return;
+    }
     const float* p = a.src + static_cast<size_t>(row) * a.src_stride + col;
     if constexpr (VEC) {
       const float4 q = live ? *reinterpret_cast<const float4*>(p) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -202,7 +215,8 @@ __global__ __launch_bounds__(kWaveLanes) void token_chain_kernel(ChainArgs a) {
 template <bool GROUPED>
 hipError_t launch_chain(const ChainArgs& a, int out_f32, int tokens, hipStream_t stream) {
   if (tokens <= 0 || a.hidden <= 0) return hipSuccess;
-  const bool vec = a.hidden % 4 == 0 && a.src_stride % 4 == 0 && (reinterpret_cast<uintptr_t>(a.src) & 15u) == 0 &&
+  const bool vec = a.hidden % 4 == 0 && a.src_stride % 4 == 0 &&
+                   (reinterpret_cast<uintptr_t>(a.src) & (a.src_bf16 ? 7u : 15u)) == 0 &&
                    (reinterpret_cast<uintptr_t>(a.out) & (out_f32 ? 15u : 7u)) == 0;
   const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>((a.hidden + 4 * kWaveLanes - 1) / (4 * kWaveLanes)));
   auto go = [&](auto kmax, auto vc, auto fc) {
@@ -355,12 +369,13 @@ hipError_t run_slot_accum(void* out, int out_f32, int with_shared, const float* 
   return launch_chain<false>(a, out_f32, tokens, stream);
 }
 
-hipError_t run_accum_ordered(void* out, int out_f32, const float* down, size_t down_stride, const int32_t* slot_row,
-                             const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens, int top_k,
-                             int hidden, hipStream_t stream) {
+hipError_t run_accum_ordered(void* out, int out_f32, const void* down, int down_bf16, size_t down_stride,
+                             const int32_t* slot_row, const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens,
+                             int top_k, int hidden, hipStream_t stream) {
   ChainArgs a{};
   a.out = out;
-  a.src = down;
+  a.src = static_cast<const float*>(down);
+  a.src_bf16 = down_bf16;
   a.src_stride = down_stride;
   a.slot_row = slot_row;
   a.slot_ids = slot_ids;

@@ -27,9 +27,10 @@ hipError_t run_accum(float* acc, const float* y, const int32_t* rows, const floa
 hipError_t run_round_bf16(uint16_t* out, const float* acc, int64_t n, hipStream_t stream);
 hipError_t run_slot_accum(void* out, int out_f32, int with_shared, const float* contrib, const float* weights,
                           int tokens, int hidden, int top_k, hipStream_t stream);
-hipError_t run_accum_ordered(void* out, int out_f32, const float* down, size_t down_stride, const int32_t* slot_row,
-                             const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens, int top_k,
-                             int hidden, hipStream_t stream);
+// down_bf16 != 0: the rows at `down` are BF16 (down_stride in BF16 elements).
+hipError_t run_accum_ordered(void* out, int out_f32, const void* down, int down_bf16, size_t down_stride,
+                             const int32_t* slot_row, const int32_t* slot_ids, const float* slot_w, int shared_row0, int tokens,
+                             int top_k, int hidden, hipStream_t stream);
 hipError_t run_segment(const int32_t* ids, int tokens, int top_k, int n_experts, int32_t* rows, int32_t* slot_row,
                        DgppMoeSegment* segs, hipStream_t stream);
 hipError_t run_slot_order(const int32_t* ids, int32_t* order, int32_t* runs, int slots, int top_k, int n_experts,

@@ -56,10 +56,18 @@ struct QuantArgs {
   float static_gs;
   const float* static_gs_dev;
   float limit;
+  int aligned;              // rows may be read as 16-byte vectors
 };
 
 // MODE 0: plain rows; 1: the MoE's SwiGLU of (x, up); 2: the Qwen dense MLP's SwiGLU.
-template <int GPT, int MODE>
+// RECIPE 0: the scale chain of src/kernels/moe_w4a4.cu (above). RECIPE 1: the per-token dynamic producer of
+// src/kernels/minimax_native_moe.cu:36-85 (MODE 0 only), whose chain multiplies by reciprocals:
+//   decode = amax * (1 / 2688);  encode = amax == 0 ? FLT_MAX : 1 / decode;  global = decode
+//   scale  = e4m3_rne_sat(encode * (amax16 * (1 / 6)));  inv = float(scale) == 0 ? 0 : 1 / (float(scale) * (1 / encode))
+//   code   = e2m1_rne_sat(x * inv)      (a zero scale leaves signed zeros: the sign bit of x survives in the code)
+// Every reciprocal here is the correctly rounded one; the reference takes NVIDIA's approximate instruction, whose last
+// bit is its own.
+template <int GPT, int MODE, int RECIPE = 0>
 __global__ __launch_bounds__(kQuantThreads) void nvfp4_quantize_rows_kernel(QuantArgs a) {
   __shared__ float wave_max[kQuantThreads / 64];
   const int row = static_cast<int>(blockIdx.x);
@@ -74,10 +82,16 @@ __global__ __launch_bounds__(kQuantThreads) void nvfp4_quantize_rows_kernel(Quan
     const int g = static_cast<int>(threadIdx.x) + j * kQuantThreads;
     gmax[j] = 0.f;
     if (g < groups) {
-      const uint4* src = reinterpret_cast<const uint4*>(xr + g * 16);
-      const uint4 v0 = src[0], v1 = src[1];
-      w[j][0] = v0.x, w[j][1] = v0.y, w[j][2] = v0.z, w[j][3] = v0.w;
-      w[j][4] = v1.x, w[j][5] = v1.y, w[j][6] = v1.z, w[j][7] = v1.w;
+      if (MODE != 0 || a.aligned) {
+        const uint4* src = reinterpret_cast<const uint4*>(xr + g * 16);
+        const uint4 v0 = src[0], v1 = src[1];
+        w[j][0] = v0.x, w[j][1] = v0.y, w[j][2] = v0.z, w[j][3] = v0.w;
+        w[j][4] = v1.x, w[j][5] = v1.y, w[j][6] = v1.z, w[j][7] = v1.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          w[j][i] = static_cast<uint32_t>(xr[g * 16 + 2 * i]) | (static_cast<uint32_t>(xr[g * 16 + 2 * i + 1]) << 16);
+      }
       if constexpr (MODE != 0) {
         const uint4* us = reinterpret_cast<const uint4*>(ur + g * 16);
         const uint4 u0 = us[0], u1 = us[1];
@@ -109,11 +123,34 @@ __global__ __launch_bounds__(kQuantThreads) void nvfp4_quantize_rows_kernel(Quan
   float row_amax = wave_max[0];
 #pragma unroll
   for (int v = 1; v < kQuantThreads / 64; ++v) row_amax = fmaxf(row_amax, wave_max[v]);
+  uint8_t* scale_row = a.scales + static_cast<size_t>(row) * a.scale_stride;
+  uint8_t* code_row = a.codes + static_cast<size_t>(row) * (a.k / 2);
+  if constexpr (RECIPE == 1) {
+    const float decode = row_amax * (1.f / (6.f * 448.f));
+    const float encode = row_amax == 0.f ? 3.402823466e+38f : 1.f / decode;
+    if (threadIdx.x == 0) a.gs[row] = decode;
+#pragma unroll
+    for (int j = 0; j < GPT; ++j) {
+      const int g = static_cast<int>(threadIdx.x) + j * kQuantThreads;
+      if (g >= groups) continue;
+      const uint8_t sb = f32_to_e4m3(encode * (gmax[j] * (1.f / 6.f)));
+      const float sv = e4m3_to_f32(sb);
+      const float inv = sv == 0.f ? 0.f : 1.f / (sv * (1.f / encode));
+      uint32_t c[2] = {0u, 0u};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t lo = f32_to_e2m1(bits_f32(w[j][i] << 16) * inv);
+        const uint32_t hi = f32_to_e2m1(bits_f32(w[j][i] & 0xFFFF0000u) * inv);
+        c[i >> 2] |= (lo | (hi << 4)) << (8 * (i & 3));
+      }
+      scale_row[g] = sb;
+      *reinterpret_cast<uint2*>(code_row + g * 8) = make_uint2(c[0], c[1]);
+    }
+    return;
+  }
   const float sg = a.static_gs_dev != nullptr ? *a.static_gs_dev : a.static_gs;
   const float global = sg > 0.f ? sg : (row_amax > 0.f ? row_amax / (6.f * 448.f) : 1.f);
   if (threadIdx.x == 0) a.gs[row] = global;
-  uint8_t* scale_row = a.scales + static_cast<size_t>(row) * a.scale_stride;
-  uint8_t* code_row = a.codes + static_cast<size_t>(row) * (a.k / 2);
 #pragma unroll
   for (int j = 0; j < GPT; ++j) {
     const int g = static_cast<int>(threadIdx.x) + j * kQuantThreads;
@@ -139,16 +176,37 @@ __global__ __launch_bounds__(kQuantThreads) void nvfp4_quantize_rows_kernel(Quan
   }
 }
 
-template <int MODE>
+template <int MODE, int RECIPE = 0>
 hipError_t launch_quant(const QuantArgs& a, hipStream_t stream) {
   const int groups = a.k / 16;
   const int gpt = (groups + kQuantThreads - 1) / kQuantThreads;
   const dim3 grid(static_cast<unsigned>(a.rows)), block(kQuantThreads);
-  if (gpt <= 1) hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<1, MODE>), grid, block, 0, stream, a);
-  else if (gpt <= 2) hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<2, MODE>), grid, block, 0, stream, a);
-  else if (gpt <= 4) hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<4, MODE>), grid, block, 0, stream, a);
-  else hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<8, MODE>), grid, block, 0, stream, a);
+  if (gpt <= 1) hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<1, MODE, RECIPE>), grid, block, 0, stream, a);
+  else if (gpt <= 2) hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<2, MODE, RECIPE>), grid, block, 0, stream, a);
+  else if (gpt <= 4) hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<4, MODE, RECIPE>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((nvfp4_quantize_rows_kernel<8, MODE, RECIPE>), grid, block, 0, stream, a);
   return hipGetLastError();
+}
+
+// SwiGLU of the native expert's first GEMM (src/kernels/minimax_native_moe.cu:87-95): FP32 gate / up sums ->
+// bf16((g' / (1 + exp(-alpha g'))) (u' + 1)), g' = min(g, limit), u' = clamp(u, -limit, limit). Four values per lane.
+__global__ __launch_bounds__(256) void swiglu_f32_rows_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                              uint16_t* __restrict__ out, int64_t count, float alpha,
+                                                              float limit, int vec) {
+  const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  if (i0 >= count) return;
+  auto one = [&](float gv, float uv) {
+    const float g = fminf(gv, limit), u = fminf(fmaxf(uv, -limit), limit);
+    return f32_to_bf16((g / (1.f + expf(-alpha * g))) * (u + 1.f));
+  };
+  if (vec && i0 + 4 <= count) {
+    const float4 g = *reinterpret_cast<const float4*>(gate + i0), u = *reinterpret_cast<const float4*>(up + i0);
+    const uint32_t lo = static_cast<uint32_t>(one(g.x, u.x)) | (static_cast<uint32_t>(one(g.y, u.y)) << 16);
+    const uint32_t hi = static_cast<uint32_t>(one(g.z, u.z)) | (static_cast<uint32_t>(one(g.w, u.w)) << 16);
+    *reinterpret_cast<uint2*>(out + i0) = make_uint2(lo, hi);
+    return;
+  }
+  for (int64_t i = i0; i < count && i < i0 + 4; ++i) out[i] = one(gate[i], up[i]);
 }
 
 int quantize(const uint16_t* x, const uint16_t* up, size_t stride, int rows, int k, float limit, uint8_t* codes,
@@ -173,6 +231,7 @@ int quantize(const uint16_t* x, const uint16_t* up, size_t stride, int rows, int
   a.static_gs = static_gs;
   a.static_gs_dev = static_gs_dev;
   a.limit = limit;
+  a.aligned = 1;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const hipError_t err = mode == 0 ? launch_quant<0>(a, st) : (mode == 1 ? launch_quant<1>(a, st) : launch_quant<2>(a, st));
   return report_hip(err, who);
@@ -215,6 +274,41 @@ int grouped_w4a4(const uint8_t* codes, const uint8_t* scales, const float* gs, c
   return report_hip(launch_grouped_mma(kFmtNvfp4, a, n_segs, static_cast<int>(z_ext), static_cast<hipStream_t>(stream)), who);
 }
 
+int dense_w4a4(const uint8_t* a_codes, const uint8_t* a_scales, size_t a_scale_stride, const float* a_gs,
+               const uint8_t* w_codes, const uint8_t* w_scales, const float* w_global, void* out, int out_f32, size_t out_stride,
+               int m, int n, int k, void* stream) {
+  const char* who = "dense w4a4";
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  if (k <= 0 || k % 128 != 0) return report_invalid(std::string(who) + ": k must be a multiple of 128");
+  if (!a_codes || !a_scales || !a_gs || !w_codes || !w_scales || !w_global || !out)
+    return report_invalid(std::string(who) + ": null pointer");
+  if (out_stride < static_cast<size_t>(n)) return report_invalid(std::string(who) + ": out_stride below n");
+  if (a_scale_stride < static_cast<size_t>(k / 16)) return report_invalid(std::string(who) + ": a_scale_stride below k / 16");
+  if (reinterpret_cast<uintptr_t>(a_codes) % 16 != 0 || reinterpret_cast<uintptr_t>(w_codes) % 16 != 0)
+    return report_invalid(std::string(who) + ": code matrices must be 16-byte aligned");
+  if ((m + kTileCols - 1) / kTileCols > 65535) return report_invalid(std::string(who) + ": grid dimension overflow");
+  DenseArgs a;
+  a.act = reinterpret_cast<const uint16_t*>(a_codes);
+  a.act_stride = static_cast<size_t>(k) / 2;   // bytes per code row
+  a.mat.payload = w_codes;
+  a.mat.scales = w_scales;
+  a.mat.divisor = 1.f;
+  a.mat.rs = 0;
+  a.mat.cs = 0;
+  a.global = w_global;
+  a.out = out;
+  a.out_stride = out_stride;
+  a.out_f32 = out_f32;
+  a.m = m;
+  a.n = n;
+  a.k = k;
+  a.once = m <= kTileCols;
+  a.a4_scales = a_scales;
+  a.a4_scale_stride = a_scale_stride;
+  a.a4_gs = a_gs;
+  return report_hip(launch_dense_mma(kFmtNvfp4, a, nullptr, 0, static_cast<hipStream_t>(stream)), who);
+}
+
 }  // namespace
 }  // namespace dgpp_amd
 
@@ -223,6 +317,40 @@ using namespace dgpp_amd;
 extern "C" {
 
 size_t dgpp_nvfp4_act_scale_stride(int k) { return static_cast<size_t>(((k / 16) + 7) / 8 * 8); }
+
+int dgpp_minimax_quantize_rows_nvfp4(const uint16_t* input, size_t stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                     float* globals, void* stream) {
+  const char* who = "minimax_quantize_rows_nvfp4";
+  if (rows <= 0) return DGPP_OK;
+  if (k <= 0 || k > 32768 || k % 128 != 0 || stride < static_cast<size_t>(k))
+    return report_invalid(std::string(who) + ": k must be 128-aligned and <= 32768");
+  if (!input || !codes || !scales || !globals) return report_invalid(std::string(who) + ": null pointer");
+  if (reinterpret_cast<uintptr_t>(codes) % 8 != 0) return report_invalid(std::string(who) + ": codes must be 8-byte aligned");
+  QuantArgs a{};
+  a.x = input;
+  a.stride = stride;
+  a.rows = rows;
+  a.k = k;
+  a.codes = codes;
+  a.scales = scales;
+  a.scale_stride = static_cast<size_t>(k / 16);   // dense: no padding in this producer's layout
+  a.gs = globals;
+  a.aligned = stride % 8 == 0 && reinterpret_cast<uintptr_t>(input) % 16 == 0;
+  return report_hip(launch_quant<0, 1>(a, static_cast<hipStream_t>(stream)), who);
+}
+
+int dgpp_minimax_swiglu_f32(const float* gate, const float* up, uint16_t* output, int64_t count, float alpha, float limit,
+                            void* stream) {
+  const char* who = "minimax_swiglu_f32";
+  if (count <= 0) return DGPP_OK;
+  if (!gate || !up || !output) return report_invalid(std::string(who) + ": null pointer");
+  const int vec = ((reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up)) & 15u) == 0 &&
+                  (reinterpret_cast<uintptr_t>(output) & 7u) == 0;
+  const int64_t lanes = (count + 3) / 4;
+  hipLaunchKernelGGL(swiglu_f32_rows_kernel, dim3(static_cast<unsigned>((lanes + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), gate, up, output, count, alpha, limit, vec);
+  return report_hip(hipGetLastError(), who);
+}
 
 int dgpp_launch_quantize_rows_nvfp4(const uint16_t* x, size_t x_stride, int rows, int k, uint8_t* codes, uint8_t* scales,
                                     float* gs, void* stream, float static_gs, const float* static_gs_dev) {
@@ -246,6 +374,14 @@ int dgpp_launch_moe_grouped_w4a4_f32(const uint8_t* codes, const uint8_t* scales
                                      const DgppMoeSegment* segs, int n_segs, int max_rows, const DgppMoeExpertView* views,
                                      int which, float* out, size_t out_stride, int n, int k, void* stream) {
   return grouped_w4a4(codes, scales, gs, act_rows, segs, n_segs, max_rows, views, which, out, 1, out_stride, n, k, stream);
+}
+
+int dgpp_dense_w4a4_supported(int k) { return k > 0 && k % 128 == 0; }
+
+int dgpp_launch_dense_w4a4_bf16(const uint8_t* a_codes, const uint8_t* a_scales, size_t a_scale_stride, const float* a_gs,
+                                const uint8_t* w_codes, const uint8_t* w_scales, const float* w_global, uint16_t* out,
+                                size_t out_stride, int m, int n, int k, void* stream) {
+  return dense_w4a4(a_codes, a_scales, a_scale_stride, a_gs, w_codes, w_scales, w_global, out, 0, out_stride, m, n, k, stream);
 }
 
 }  // extern "C"

@@ -578,6 +578,34 @@ def launch_moe_grouped_w4a4_bf16(codes, scales, gs, act_rows, segs, n_segs, max_
                                                          _p(views), which, _p(out), out_stride, n, k, _stream(stream)))
 
 
+def dense_w4a4_supported(k: int) -> bool:
+    return bool(_lib.load().dgpp_dense_w4a4_supported(k))
+
+
+def launch_dense_w4a4_bf16(a_codes, a_scales, a_scale_stride, a_gs, w_codes, w_scales, w_global, out, out_stride, m, n, k,
+                           stream=None):
+    _check(_lib.load().dgpp_launch_dense_w4a4_bf16(_p(a_codes), _p(a_scales), a_scale_stride, _p(a_gs), _p(w_codes), _p(w_scales),
+                                                   _p(w_global), _p(out), out_stride, m, n, k, _stream(stream)))
+
+
+def minimax_quantize_rows_nvfp4(x, stride, rows, k, codes, scales, globals_, stream=None):
+    _check(_lib.load().dgpp_minimax_quantize_rows_nvfp4(_p(x), stride, rows, k, _p(codes), _p(scales), _p(globals_), _stream(stream)))
+
+
+def minimax_swiglu_f32(gate, up, out, count, alpha, limit, stream=None):
+    _check(_lib.load().dgpp_minimax_swiglu_f32(_p(gate), _p(up), _p(out), count, alpha, limit, _stream(stream)))
+
+
+def launch_moe_accum_ordered_bf16down(out, down, down_stride, slot_row, slot_ids, slot_w, tokens, top_k, hidden, stream=None):
+    _check(_lib.load().dgpp_launch_moe_accum_ordered_bf16down(_p(out), _p(down), down_stride, _p(slot_row), _p(slot_ids),
+                                                              _p(slot_w), tokens, top_k, hidden, _stream(stream)))
+
+
+def launch_moe_accum_ordered_f32_bf16down(out, down, down_stride, slot_row, slot_ids, slot_w, tokens, top_k, hidden, stream=None):
+    _check(_lib.load().dgpp_launch_moe_accum_ordered_f32_bf16down(_p(out), _p(down), down_stride, _p(slot_row), _p(slot_ids),
+                                                                  _p(slot_w), tokens, top_k, hidden, _stream(stream)))
+
+
 def launch_moe_grouped_w4a4_f32(codes, scales, gs, act_rows, segs, n_segs, max_rows, views, which, out, out_stride, n, k,
                                 stream=None):
     _check(_lib.load().dgpp_launch_moe_grouped_w4a4_f32(_p(codes), _p(scales), _p(gs), _p(act_rows), _p(segs), n_segs, max_rows,

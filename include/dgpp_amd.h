@@ -168,6 +168,14 @@ int dgpp_launch_moe_accum_ordered_f32(float* out, const float* down, size_t down
                                       const int32_t* slot_row, const int32_t* slot_ids,
                                       const float* slot_w, int shared_row0, int tokens, int top_k,
                                       int hidden, void* stream);
+/* src/kernels/glm_moe_launch.hpp:182-191: the same chain over BF16 down rows (the W4A4 grouped chain; no shared row),
+ * rounded to BF16 or left in FP32. down_stride in BF16 elements. */
+int dgpp_launch_moe_accum_ordered_bf16down(uint16_t* out, const uint16_t* down, size_t down_stride, const int32_t* slot_row,
+                                           const int32_t* slot_ids, const float* slot_w, int tokens, int top_k, int hidden,
+                                           void* stream);
+int dgpp_launch_moe_accum_ordered_f32_bf16down(float* out, const uint16_t* down, size_t down_stride, const int32_t* slot_row,
+                                               const int32_t* slot_ids, const float* slot_w, int tokens, int top_k, int hidden,
+                                               void* stream);
 /* src/kernels/glm_moe_launch.hpp:273-283 */
 int dgpp_launch_moe_slot_accum(uint16_t* out, const float* contrib, const float* weights,
                                int tokens, int hidden, int top_k, void* stream);
@@ -516,6 +524,29 @@ int dgpp_launch_moe_grouped_w4a4_bf16(const uint8_t* codes, const uint8_t* scale
 int dgpp_launch_moe_grouped_w4a4_f32(const uint8_t* codes, const uint8_t* scales, const float* gs, const int32_t* act_rows,
                                      const DgppMoeSegment* segs, int n_segs, int max_rows, const DgppMoeExpertView* views,
                                      int which, float* out, size_t out_stride, int n, int k, void* stream);
+
+/* src/kernels/moe_w4a4.hpp:51-71 (dense_w4a4_tma_supported, launch_dense_w4a4_tma_bf16): the dense W4A4 form,
+ * out[m, :n] = act(row) . W^T. The reference stages both code matrices through TMA tensor maps (nvfp4_code_tma_map);
+ * this chip has no such descriptor, so the code matrices arrive as plain pointers ([m, k / 2] and [n, k / 2] bytes,
+ * 16-byte aligned) and the map constructor has no counterpart. a_scales [m, a_scale_stride] and a_gs [m] are the
+ * quantizer's, w_scales [n, k / 16] e4m3, w_global the matrix's device F32 global. k a multiple of 128. Bitwise the
+ * grouped kernel over one segment, as in the reference. */
+int dgpp_dense_w4a4_supported(int k);
+int dgpp_launch_dense_w4a4_bf16(const uint8_t* a_codes, const uint8_t* a_scales, size_t a_scale_stride, const float* a_gs,
+                                const uint8_t* w_codes, const uint8_t* w_scales, const float* w_global, uint16_t* out,
+                                size_t out_stride, int m, int n, int k, void* stream);
+/* src/kernels/minimax_native_moe.hpp:8-13, minimax_native_moe.cu:36-85, :97-107: the per-token dynamic NVFP4 producer of
+ * the native routed experts: BF16 rows [rows, k] (any stride >= k) -> codes [rows, k / 2], e4m3 scales [rows, k / 16]
+ * (dense, no padding), FP32 decode globals [rows] (amax / 2688; 0 for a zero row). Its scale chain multiplies by
+ * reciprocals (see dgpp_amd/csrc/nvfp4_act.hip); they are the correctly rounded ones here, where the reference takes
+ * NVIDIA's approximate reciprocal instruction: a scale byte or a code can differ from the reference's where that
+ * instruction's last bit moves a rounding. k a multiple of 128, <= 32768. */
+int dgpp_minimax_quantize_rows_nvfp4(const uint16_t* input, size_t stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                     float* globals, void* stream);
+/* src/kernels/minimax_native_moe.hpp:15-18, minimax_native_moe.cu:87-95, :109-115: FP32 gate / up sums [count] ->
+ * bf16((g' / (1 + exp(-alpha g'))) (u' + 1)), g' = min(g, limit), u' = clamp(u, -limit, limit). */
+int dgpp_minimax_swiglu_f32(const float* gate, const float* up, uint16_t* output, int64_t count, float alpha, float limit,
+                            void* stream);
 
 /* ---- activation-quantized MXFP8 (W8A8) form ---------------------------------------------------------------------
  * The weights' MXFP8 payload meets activations quantized to MXFP8 on the fly; the products run on the

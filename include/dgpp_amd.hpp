@@ -192,6 +192,18 @@ inline void launch_moe_accum_ordered_f32(float* out, const float* down, size_t d
   detail::check(dgpp_launch_moe_accum_ordered_f32(out, down, down_stride, slot_row, slot_ids, slot_w, shared_row0,
                                                   tokens, top_k, hidden, stream));
 }
+inline void launch_moe_accum_ordered_bf16down(uint16_t* out, const uint16_t* down, size_t down_stride, const int32_t* slot_row,
+                                              const int32_t* slot_ids, const float* slot_w, int tokens, int top_k, int hidden,
+                                              hipStream_t stream) {
+  detail::check(dgpp_launch_moe_accum_ordered_bf16down(out, down, down_stride, slot_row, slot_ids, slot_w, tokens, top_k, hidden,
+                                                       stream));
+}
+inline void launch_moe_accum_ordered_f32_bf16down(float* out, const uint16_t* down, size_t down_stride, const int32_t* slot_row,
+                                                  const int32_t* slot_ids, const float* slot_w, int tokens, int top_k,
+                                                  int hidden, hipStream_t stream) {
+  detail::check(dgpp_launch_moe_accum_ordered_f32_bf16down(out, down, down_stride, slot_row, slot_ids, slot_w, tokens, top_k,
+                                                           hidden, stream));
+}
 inline void launch_moe_slot_accum(uint16_t* out, const float* contrib, const float* weights, int tokens, int hidden,
                                   int top_k, hipStream_t stream) {
   detail::check(dgpp_launch_moe_slot_accum(out, contrib, weights, tokens, hidden, top_k, stream));
@@ -478,6 +490,23 @@ inline void launch_moe_grouped_w4a4_f32(const uint8_t* codes, const uint8_t* sca
                                         int which, float* out, size_t out_stride, int n, int k, hipStream_t stream) {
   detail::check(dgpp_launch_moe_grouped_w4a4_f32(codes, scales, gs, act_rows, segs, n_segs, max_rows, views, which, out,
                                                  out_stride, n, k, stream));
+}
+// The dense form: the reference's TMA tensor maps become the code matrices' plain pointers (src/kernels/moe_w4a4.hpp:51-71).
+inline bool dense_w4a4_supported(int k) { return dgpp_dense_w4a4_supported(k) != 0; }
+inline void launch_dense_w4a4_bf16(const uint8_t* a_codes, const uint8_t* a_scales, size_t a_scale_stride, const float* a_gs,
+                                   const uint8_t* w_codes, const uint8_t* w_scales, const float* w_global, uint16_t* out,
+                                   size_t out_stride, int m, int n, int k, hipStream_t stream) {
+  detail::check(dgpp_launch_dense_w4a4_bf16(a_codes, a_scales, a_scale_stride, a_gs, w_codes, w_scales, w_global, out, out_stride,
+                                            m, n, k, stream));
+}
+// src/kernels/minimax_native_moe.hpp:8-18.
+inline void minimax_quantize_rows_nvfp4(const uint16_t* input, size_t stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                        float* globals, hipStream_t stream) {
+  detail::check(dgpp_minimax_quantize_rows_nvfp4(input, stride, rows, k, codes, scales, globals, stream));
+}
+inline void minimax_swiglu_f32(const float* gate, const float* up, uint16_t* output, int64_t count, float alpha, float limit,
+                               hipStream_t stream) {
+  detail::check(dgpp_minimax_swiglu_f32(gate, up, output, count, alpha, limit, stream));
 }
 
 // src/kernels/mxfp8_gemm.hpp:11-31.

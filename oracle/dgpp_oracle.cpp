@@ -541,6 +541,51 @@ void orc_nvfp4_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k,
   }
 }
 
+// src/kernels/minimax_native_moe.cu:36-85 with every reciprocal correctly rounded (the reference's is NVIDIA's
+// approximate instruction): decode = amax * (1 / 2688), encode = 1 / decode (FLT_MAX for a zero row),
+// scale = e4m3(encode * (amax16 * (1 / 6))), inverse = 1 / (float(scale) * (1 / encode)) (0 for a zero scale).
+void orc_minimax_quantize_rows_nvfp4(const uint16_t* x, int64_t stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                     float* globals) {
+  const int groups = k / 16;
+  for (int r = 0; r < rows; ++r) {
+    const uint16_t* src = x + static_cast<size_t>(r) * stride;
+    float row_max = 0.f;
+    for (int c = 0; c < k; ++c) row_max = std::max(row_max, std::fabs(orc_bf16_to_f32(src[c])));
+    const float decode = row_max * (1.f / (6.f * 448.f));
+    const float encode = row_max == 0.f ? std::numeric_limits<float>::max() : 1.f / decode;
+    globals[r] = decode;
+    for (int g = 0; g < groups; ++g) {
+      float gmax = 0.f;
+      for (int i = 0; i < 16; ++i) gmax = std::max(gmax, std::fabs(orc_bf16_to_f32(src[g * 16 + i])));
+      const float sixth = 1.f / 6.f;
+      const float scaled_max = gmax * sixth;
+      const uint8_t sb = orc_f32_to_e4m3(encode * scaled_max);
+      const float sv = orc_e4m3_to_f32(sb);
+      const float back = 1.f / encode;
+      const float inverse = sv == 0.f ? 0.f : 1.f / (sv * back);
+      scales[static_cast<size_t>(r) * groups + g] = sb;
+      uint8_t* code = codes + static_cast<size_t>(r) * (k / 2) + static_cast<size_t>(g) * 8;
+      for (int i = 0; i < 8; ++i) {
+        const uint8_t lo = orc_f32_to_e2m1(orc_bf16_to_f32(src[g * 16 + 2 * i]) * inverse);
+        const uint8_t hi = orc_f32_to_e2m1(orc_bf16_to_f32(src[g * 16 + 2 * i + 1]) * inverse);
+        code[i] = static_cast<uint8_t>(lo | (hi << 4));
+      }
+    }
+  }
+}
+
+// src/kernels/minimax_native_moe.cu:87-95 in double, rounded once to BF16 (the kernel evaluates it in fp32).
+void orc_minimax_swiglu_f32(const float* gate, const float* up, int64_t count, double alpha, double limit, uint16_t* out,
+                            double* out_exact) {
+  for (int64_t i = 0; i < count; ++i) {
+    const double g = std::min(static_cast<double>(gate[i]), limit);
+    const double u = std::min(std::max(static_cast<double>(up[i]), -limit), limit);
+    const double v = (g / (1.0 + std::exp(-alpha * g))) * (u + 1.0);
+    if (out) out[i] = d2bf16(v);
+    if (out_exact) out_exact[i] = v;
+  }
+}
+
 void orc_w4a4_gemm(const uint8_t* a_codes, const uint8_t* a_scales, int64_t a_scale_stride, const float* a_gs,
                    const uint8_t* w_codes, const uint8_t* w_scales, double w_global, int m, int n, int k, double* out,
                    double* out_abs) {

@@ -176,6 +176,20 @@ void orc_mxfp8_gemm(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w,
  * and an independent numpy float32 evaluation of the same recipe; the conversions are orc_f32_to_e4m3 / orc_f32_to_e2m1. */
 void orc_nvfp4_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, float static_gs, uint8_t* codes,
                              uint8_t* scales, int64_t scale_stride, float* gs);
+/* The per-token dynamic NVFP4 producer of src/kernels/minimax_native_moe.cu:36-85: scales [rows, k / 16] (dense),
+ * globals[rows] = amax * (1 / 2688) (0 for a zero row). The chain of fp32 multiplications by reciprocals is restated
+ * with every reciprocal correctly rounded. PARITY UNPINNED against the reference in that one respect: its reciprocal is
+ * NVIDIA's approximate instruction (rcp.approx.ftz.f32), whose last bit no fixture or closed form available here
+ * fixes (the reference's own test reads fixture folders that are not in its tree). What IS pinned: the restated chain
+ * against an independent numpy float32 evaluation, the decode identity (decoded rows within half a code step), zero
+ * rows, and invariance to how rows are spread over calls (the property the reference's test checks). */
+void orc_minimax_quantize_rows_nvfp4(const uint16_t* x, int64_t stride, int rows, int k, uint8_t* codes, uint8_t* scales,
+                                     float* globals);
+/* src/kernels/minimax_native_moe.cu:87-95 evaluated in double: bf16((g' / (1 + exp(-alpha g'))) (u' + 1)), g' = min(g,
+ * limit), u' = clamp(u, -limit, limit); out (nullable) the BF16 rounding, out_exact (nullable) the unrounded value.
+ * Pinned by closed-form points (g = 0, u = -1, both clamps) and numpy float64. */
+void orc_minimax_swiglu_f32(const float* gate, const float* up, int64_t count, double alpha, double limit, uint16_t* out,
+                            double* out_exact);
 /* out[m, n] = (sum_k e2m1(a) e4m3(sa) * e2m1(w) e4m3(sw)) * gs[m] / w_global in double, and (nullable) the same sum of
  * magnitudes: the fp64 dot of the SAME quantized operands the reference's kernel test compares against
  * (tests/cuda/moe_w4a4_test.cu:193-216, bound |got - dot| < 1e-5 * sum|terms|). Pinned by numpy brute force. */

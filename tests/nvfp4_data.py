@@ -111,3 +111,24 @@ def activation_rows(rows, k, seed, stride=None):
     x = rng.normal(0, 1, (rows, stride)).astype(np.float32)
     x[rng.integers(0, 256, (rows, stride)) == 0] *= 20
     return f32_to_bf16_bits(x)
+
+
+def minimax_quantize_numpy(x_bits, k):
+    """The per-token dynamic producer (src/kernels/minimax_native_moe.cu:36-85) in numpy float32, reciprocals correctly
+    rounded: (codes [rows, k/2], scales [rows, k/16], globals [rows])."""
+    rows = x_bits.shape[0]
+    f = np.float32
+    x = bf16_bits_to_f64(x_bits[:, :k]).astype(np.float32)
+    amax = np.abs(x).max(axis=1)
+    decode = (amax * (f(1.0) / (f(6.0) * f(448.0)))).astype(np.float32)
+    with np.errstate(divide="ignore"):
+        encode = np.where(amax == 0, np.finfo(np.float32).max, f(1.0) / decode).astype(np.float32)
+    xg = x.reshape(rows, k // 16, 16)
+    gmax = np.abs(xg).max(axis=2)
+    sb = e4m3_encode((encode[:, None] * (gmax * (f(1.0) / f(6.0))).astype(np.float32)).astype(np.float32))
+    sv = e4m3_decode(sb).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        inv = np.where(sv == 0, f(0), f(1.0) / (sv * (f(1.0) / encode)[:, None]).astype(np.float32)).astype(np.float32)
+    nib = e2m1_encode((xg * inv[:, :, None]).astype(np.float32)).reshape(rows, k)
+    codes = (nib[:, 0::2] | (nib[:, 1::2] << 4)).astype(np.uint8)
+    return codes, sb.astype(np.uint8), decode

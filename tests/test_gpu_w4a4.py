@@ -174,3 +174,143 @@ def test_w4a4_down_from_the_fused_swiglu_quantizer_and_its_distance_to_w4a16(gpu
     rel = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
     print(f"W4A4 vs W4A16 down rows: relative l2 {rel:.4f}")
     assert 0.0 < rel < 0.25
+
+
+def device_minimax_quantize(x_d, stride, rows, k):
+    codes, scales, glob = dev_empty((rows, k // 2), np.uint8), dev_empty((rows, k // 16), np.uint8), dev_empty(rows, np.float32)
+    L.minimax_quantize_rows_nvfp4(x_d, stride, rows, k, codes, scales, glob)
+    sync()
+    return host(codes), host(scales), host(glob)
+
+
+@pytest.mark.parametrize("k,rows,stride", [(128, 5, 128), (3072, 33, 3072 + 8), (6144, 9, 6144 + 3), (32768, 2, 32768), (1536, 70, 1536)])
+def test_minimax_producer_is_bitwise_the_oracle_and_rows_are_independent(gpu, k, rows, stride):
+    """Bit for bit the oracle's restated chain (reciprocals correctly rounded on both sides), for aligned and unaligned row
+    strides; and the reference test's property (tests/cuda/minimax_native_moe_test.cpp:79-94): the bytes of a row do not
+    depend on how the rows are spread over calls."""
+    from test_oracle_w4a4 import oracle_minimax_quantize
+    x = nd.activation_rows(rows, k, 700 + k, stride=stride)
+    x[rows // 2, :k] = 0
+    x[0, 32:64] = 0
+    x[0, 40] = 0x8000
+    want = oracle_minimax_quantize(x, rows, k)
+    x_d = dev(x)
+    got = device_minimax_quantize(x_d, stride, rows, k)
+    for name, g, w in zip(("codes", "scales", "globals"), got, want):
+        assert np.array_equal(g.view(np.uint8), w.view(np.uint8)), f"{name} k={k} rows={rows} stride={stride}"
+    for chunk in (1, 8, 17):
+        codes, scales, glob = dev_empty((rows, k // 2), np.uint8), dev_empty((rows, k // 16), np.uint8), dev_empty(rows, np.float32)
+        for start in range(0, rows, chunk):
+            n = min(chunk, rows - start)
+            L.minimax_quantize_rows_nvfp4(x_d[start:], stride, n, k, codes[start:], scales[start:], glob[start:])
+        sync()
+        assert np.array_equal(host(codes), got[0]) and np.array_equal(host(scales), got[1]) and np.array_equal(host(glob), got[2])
+
+
+def test_minimax_swiglu_f32_against_the_double_evaluation(gpu):
+    rng = np.random.default_rng(5)
+    n = 70001
+    gate = (rng.normal(0, 3, n)).astype(np.float32)
+    up = (rng.normal(0, 3, n)).astype(np.float32)
+    gate[:4], up[:4] = [0.0, 100.0, -100.0, 3.0], [5.0, 0.5, 0.5, -1.0]
+    want, exact = np.empty(n, np.uint16), np.empty(n)
+    orc.oracle().orc_minimax_swiglu_f32(orc.p(gate), orc.p(up), n, 1.702, 7.0, orc.p(want), orc.p(exact))
+    for off in (0, 1):                                  # the vector path and the unaligned tail path
+        out = dev_empty(n + 1, np.uint16)
+        L.minimax_swiglu_f32(dev(gate)[off:], dev(up)[off:], out[off:], n - off, 1.702, 7.0)
+        sync()
+        got = host(out, np.uint16)[off:n]
+        same = np.mean(got == want[off:])
+        assert same > 0.995, f"{same:.5f} of the values are the correctly rounded ones"
+        ulp = np.abs(hg.bf16_to_f32(got).astype(np.float64) - hg.bf16_to_f32(want[off:]).astype(np.float64))
+        assert np.all(ulp <= np.abs(exact[off:]) * 2.0 ** -7 + 1e-30), "never more than one BF16 step away"
+    assert host(out, np.uint16)[1] == want[1] and want[0] == 0
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 64, 128), (21, 200, 1024), (40, 96, 3072), (16, 130, 6144)])
+def test_dense_w4a4_is_bitwise_the_grouped_kernel_over_one_segment(gpu, m, n, k):
+    """src/kernels/moe_w4a4.hpp:51-58 ("bitwise the grouped kernel over one segment"), and the fp64 bound."""
+    p = moe_data.make_problem(2, k, (n + 15) // 16 * 16, 1, m, "nvfp4", 90 + k, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    mat = p.experts[1][0]                                # gate matrix of expert 1: [>= n, k]; the launches take its first n rows
+    x = nd.activation_rows(m, k, 40 + m)
+    ss = nd.scale_stride(k)
+    codes, scales, gs = dev_empty((m, k // 2), np.uint8), dev_empty((m, ss), np.uint8), dev_empty(m, np.float32)
+    L.launch_quantize_rows_nvfp4(dev(x), k, m, k, codes, scales, gs)
+    seg = dev(np.array([[0, m, 1]], np.int32))
+    want, got = dev_empty((m, n), np.uint16), dev_empty((m, n + 8), np.uint16)
+    L.launch_moe_grouped_w4a4_bf16(codes, scales, gs, None, seg, 1, m, d.views, 0, want, n, n, k)
+    wp, wsc, wg = dev(mat.payload), dev(mat.scales), dev(mat.glob)
+    L.launch_dense_w4a4_bf16(codes, scales, ss, gs, wp, wsc, wg, got, n + 8, m, n, k)
+    sync()
+    g = host(got, np.uint16)[:, :n]
+    assert np.array_equal(g, host(want, np.uint16))
+    ref, mag = np.empty((m, n)), np.empty((m, n))
+    c, s, gg = host(codes), host(scales), host(gs)
+    orc.oracle().orc_w4a4_gemm(orc.p(c), orc.p(s), ss, orc.p(gg), orc.p(mat.payload), orc.p(mat.scales), float(mat.glob[0]), m, n, k,
+                               orc.p(ref), orc.p(mag))
+    err = np.abs(hg.bf16_to_f32(g).astype(np.float64) - ref)
+    assert np.all(err <= 1e-5 * mag + np.abs(ref) * 2.0 ** -8), "the BF16 output: the fp64 bound plus its own rounding"
+
+
+@pytest.mark.parametrize("K,H,T", [(8, 4096, 5), (3, 1000, 9), (16, 512, 2)])
+def test_accum_ordered_over_bf16_down_rows_is_the_f32_chain_over_the_widened_rows(gpu, K, H, T):
+    """src/kernels/glm_moe_launch.hpp:182-191: the ordered chain over BF16 down rows (no shared row)."""
+    rng = np.random.default_rng(K + H)
+    R = T * K
+    stride = H + 4 if H % 4 == 0 else H + 1
+    down = hg.normal_bf16(0x6A0 + H, (R, stride), 1.0)
+    ids = np.stack([rng.permutation(64)[:K] for _ in range(T)]).astype(np.int32)
+    slot_row = rng.permutation(R).astype(np.int32).reshape(T, K)
+    w = rng.uniform(0.05, 1.0, (T, K)).astype(np.float32)
+    d16, d32 = dev(down), dev(hg.bf16_to_f32(down))
+    ids_d, sr_d, w_d = dev(ids), dev(slot_row), dev(w)
+    out_b, out_f, want_b, want_f = dev_empty((T, H), np.uint16), dev_empty((T, H), np.float32), dev_empty((T, H), np.uint16), dev_empty((T, H), np.float32)
+    L.launch_moe_accum_ordered_bf16down(out_b, d16, stride, sr_d, ids_d, w_d, T, K, H)
+    L.launch_moe_accum_ordered_f32_bf16down(out_f, d16, stride, sr_d, ids_d, w_d, T, K, H)
+    L.launch_moe_accum_ordered(want_b, d32, stride, sr_d, ids_d, w_d, -1, T, K, H)
+    L.launch_moe_accum_ordered_f32(want_f, d32, stride, sr_d, ids_d, w_d, -1, T, K, H)
+    sync()
+    assert np.array_equal(host(out_b, np.uint16), host(want_b, np.uint16))
+    assert np.array_equal(host(out_f).view(np.uint32), host(want_f).view(np.uint32))
+    # and the chain itself, on the host: ascending expert id, fma from zero
+    t = T - 1
+    acc = np.zeros(H, np.float32)
+    for j in np.argsort(ids[t], kind="stable"):
+        row = hg.bf16_to_f32(down[slot_row[t, j], :H]).astype(np.float64)
+        acc = (np.float64(w[t, j]) * row + acc.astype(np.float64)).astype(np.float32)      # one rounding: an fma
+    assert np.array_equal(host(out_f)[t].view(np.uint32), acc.view(np.uint32))
+
+
+def test_native_expert_chain_does_not_depend_on_how_rows_are_spread_over_launches(gpu):
+    """tests/cuda/minimax_native_moe_test.cpp:112-165: producer -> grouped W4A4 gate, up (f32) -> SwiGLU (f32 in, BF16 out)
+    -> producer -> grouped W4A4 down (BF16), run over all rows at once and in chunks of 1, 8 and 17 rows: the same bytes."""
+    rows, H, I = 37, 1024, 256
+    p = moe_data.make_problem(1, H, I, 1, rows, "nvfp4", 123, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    x_d = dev(nd.activation_rows(rows, H, 321))
+    codes, scales, glob = dev_empty((rows, H // 2), np.uint8), dev_empty((rows, H // 16), np.uint8), dev_empty(rows, np.float32)
+    gate, up = dev_empty((rows, I), np.float32), dev_empty((rows, I), np.float32)
+    act, out = dev_empty((rows, I), np.uint16), dev_empty((rows, H), np.uint16)
+    ac, asc, ag = dev_empty((rows, I // 2), np.uint8), dev_empty((rows, I // 16), np.uint8), dev_empty(rows, np.float32)
+
+    def run(start, count):
+        seg = dev(np.array([[0, count, 0]], np.int32))
+        L.minimax_quantize_rows_nvfp4(x_d[start:], H, count, H, codes[start:], scales[start:], glob[start:])
+        L.launch_moe_grouped_w4a4_f32(codes[start:], scales[start:], glob[start:], None, seg, 1, count, d.views, 0, gate[start:], I, I, H)
+        L.launch_moe_grouped_w4a4_f32(codes[start:], scales[start:], glob[start:], None, seg, 1, count, d.views, 1, up[start:], I, I, H)
+        L.minimax_swiglu_f32(gate[start:], up[start:], act[start:], count * I, 1.702, 7.0)
+        L.minimax_quantize_rows_nvfp4(act[start:], I, count, I, ac[start:], asc[start:], ag[start:])
+        L.launch_moe_grouped_w4a4_bf16(ac[start:], asc[start:], ag[start:], None, seg, 1, count, d.views, 2, out[start:], H, H, I)
+        sync()
+
+    run(0, rows)
+    first = [host(t).copy() for t in (out, act, gate, up)]
+    assert np.abs(hg.bf16_to_f32(first[0].view(np.uint16))).max() > 0
+    for chunk in (1, 8, 17):
+        for t in (out, act, gate, up):
+            t.zero_()
+        for start in range(0, rows, chunk):
+            run(start, min(chunk, rows - start))
+        for a, t in zip(first, (out, act, gate, up)):
+            assert np.array_equal(a, host(t)), f"chunk {chunk}"

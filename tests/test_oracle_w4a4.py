@@ -95,3 +95,75 @@ def test_launchers_refuse_bad_geometry_without_a_gpu():
     with pytest.raises(L.InvalidArgument):
         L.launch_moe_grouped_w4a4_f32(fake, fake, fake, None, fake, 3, 0, fake, 0, fake, 64, 64, 128)   # max_rows
     L.launch_moe_grouped_w4a4_f32(fake, fake, fake, None, fake, 0, 4, fake, 0, fake, 64, 64, 128)       # no segments
+
+
+def oracle_minimax_quantize(x, rows, k):
+    codes = np.empty((rows, k // 2), np.uint8)
+    scales = np.empty((rows, k // 16), np.uint8)
+    glob = np.empty(rows, np.float32)
+    orc.oracle().orc_minimax_quantize_rows_nvfp4(orc.p(x), x.shape[1], rows, k, orc.p(codes), orc.p(scales), orc.p(glob))
+    return codes, scales, glob
+
+
+@pytest.mark.parametrize("k", [128, 3072, 6144])
+def test_minimax_producer_matches_the_numpy_restatement(k):
+    """What this pins: the restated chain (multiplications by correctly rounded reciprocals). What it cannot: the last
+    bit of the reference's approximate reciprocal instruction (parity unpinned in that respect)."""
+    rows = 7
+    x = nd.activation_rows(rows, k, 300 + k, stride=k + 3)
+    x[2, :k] = 0
+    x[5, 32:64] = 0
+    x[5, 40] = 0x8000                                  # a negative zero in a zero block: its sign survives in the code
+    codes, scales, glob = oracle_minimax_quantize(x, rows, k)
+    want = nd.minimax_quantize_numpy(x, k)
+    assert np.array_equal(glob.view(np.uint32), want[2].view(np.uint32))
+    assert np.array_equal(scales, want[1]) and np.array_equal(codes, want[0])
+    assert glob[2] == 0.0 and not scales[2].any() and not codes[2].any()
+    assert codes[5, 20] == 0x08 and not scales[5, 2:4].any()
+    # the decode identity: rows come back within half a code step (one where the scale byte rounded down)
+    back = nd.dequantize(codes, scales, glob, k)
+    xf = bf16_bits_to_f64(x[:, :k])
+    step = np.repeat(nd.e4m3_decode(scales), 16, axis=1) * glob[:, None].astype(np.float64)
+    assert np.all(np.abs(back - xf) <= step + 1e-30)
+    # the row maximum lands on the top code of the top scale: amax / 2688 * 448 * 6
+    live = [r for r in range(rows) if r != 2]
+    assert np.allclose(np.abs(back[live]).max(axis=1), np.abs(xf[live]).max(axis=1), rtol=2e-6)
+    # rows do not depend on the rows beside them
+    one = oracle_minimax_quantize(np.ascontiguousarray(x[4:5]), 1, k)
+    assert np.array_equal(one[0][0], codes[4]) and np.array_equal(one[1][0], scales[4]) and one[2][0] == glob[4]
+
+
+def test_minimax_swiglu_f32_oracle_closed_form_points():
+    alpha, limit = 1.702, 7.0
+    gate = np.array([0.0, 3.0, 100.0, -100.0, 2.0, 2.0, 1.0], np.float32)
+    up = np.array([5.0, -1.0, 0.5, 0.5, 100.0, -100.0, 0.25], np.float32)
+    out, exact = np.empty(7, np.uint16), np.empty(7)
+    orc.oracle().orc_minimax_swiglu_f32(orc.p(gate), orc.p(up), 7, alpha, limit, orc.p(out), orc.p(exact))
+    sig = lambda v: 1.0 / (1.0 + np.exp(-alpha * v))
+    want = np.array([0.0, 0.0, 7.0 * sig(7.0) * 1.5, -100.0 * sig(-100.0) * 1.5, 2.0 * sig(2.0) * 8.0, 2.0 * sig(2.0) * -6.0,
+                     sig(1.0) * 1.25])
+    assert np.allclose(exact, want, rtol=1e-14, atol=1e-300)
+    assert np.array_equal(out, nd.f32_to_bf16_bits(want.astype(np.float32)))
+
+
+def test_minimax_and_dense_launchers_refuse_bad_geometry_without_a_gpu():
+    from dgpp_amd import launch as L
+    fake = 0x10000
+    for k in (0, 64, 192, 32768 + 128):
+        with pytest.raises(L.InvalidArgument):
+            L.minimax_quantize_rows_nvfp4(fake, 40000, 2, k, fake, fake, fake)
+    with pytest.raises(L.InvalidArgument):
+        L.minimax_quantize_rows_nvfp4(fake, 100, 2, 128, fake, fake, fake)             # stride below k
+    L.minimax_quantize_rows_nvfp4(None, 128, 0, 128, None, None, None)
+    L.minimax_swiglu_f32(None, None, None, 0, 1.702, 7.0)
+    with pytest.raises(L.InvalidArgument):
+        L.minimax_swiglu_f32(fake, None, fake, 5, 1.702, 7.0)
+    assert L.dense_w4a4_supported(128) and L.dense_w4a4_supported(6144) and not L.dense_w4a4_supported(192)
+    with pytest.raises(L.InvalidArgument):
+        L.launch_dense_w4a4_bf16(fake, fake, 8, fake, fake, fake, fake, fake, 64, 4, 64, 192)       # k % 128
+    with pytest.raises(L.InvalidArgument):
+        L.launch_dense_w4a4_bf16(fake, fake, 4, fake, fake, fake, fake, fake, 64, 4, 64, 128)       # scale stride below k / 16
+    with pytest.raises(L.InvalidArgument):
+        L.launch_dense_w4a4_bf16(fake, fake, 8, fake, fake, fake, fake, fake, 32, 4, 64, 128)       # out_stride below n
+    with pytest.raises(L.InvalidArgument):
+        L.launch_moe_accum_ordered_bf16down(fake, fake, 64, fake, fake, fake, 3, 17, 64)            # top_k above 16
