@@ -71,7 +71,7 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5,c5skew,w8a8,qwen_tail,slotbench,readprobe ('' for none; default: c1,c2,c4,c5, none under --tune)")
+                    "separated out of c1,c2,c4,c5,c5skew,w8a8,qwen_tail,slotbench,readprobe,router ('' for none; default: c1,c2,c4,c5, none under --tune)")
     ap.add_argument("--replays", type=int, default=0, help="timed graph replays per measurement (0 = at least 50 and at "
                     "least 1000 steps; a small number keeps a run under a profiler's counters short)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
@@ -711,13 +711,35 @@ def main():
         res["best"] = {k: {"form": v[0], "gbps": v[1], "frac_of_peak": v[1] / HBM_PEAK_GBPS} for k, v in best.items()}
         return res
 
+    def bench_router():
+        """The router's two launches (score rows, selection) at decode batch sizes: the one-row dots kernel against the
+        token-tiled one (from 16 rows on), for the C3 (256 x 4096) and C5 (256 x 6144) router shapes. The gate stays
+        cache-resident here (2-3 MB), as it does between a layer's steps."""
+        res = {}
+        for name, (rE, rH, rK) in (("c3_256x4096", (256, 4096, 8)), ("c5_256x6144", (256, 6144, 8))):
+            rcfg = L.make_config(rH, 64, rE, rK, n_shared_experts=0, routed_scaling_factor=1.0, router_mode=L.ROUTER_SOFTMAX_TOPK)
+            gate = torch.from_numpy(hg.normal_bf16(0xD6990400, (rE, rH), 1.0 / np.sqrt(rH)).view(np.int16)).to(dev)
+            for T in (16, 32, 64, 128):
+                x = torch.from_numpy(hg.normal_bf16(0xD6990401 + T, (T, rH)).view(np.int16)).to(dev)
+                ids, w = torch.empty((T, rK), dtype=torch.int32, device=dev), torch.empty((T, rK), dtype=torch.float32, device=dev)
+                sc, bi = torch.empty((T, rE), dtype=torch.float32, device=dev), torch.empty((T, rE), dtype=torch.float32, device=dev)
+                for tiled, tt in ((False, 0), (True, 2), (True, 4)):
+                    def step(i):
+                        L.launch_moe_router(x, gate, None, ids, w, sc, bi, rcfg, T, stream, None, tiled)
+                    lib.dgpp_tune_set(10, tt)         # tokens per wavefront of the tiled form
+                    sec = time_graph(step, args.steps, args.warmup)
+                    lib.dgpp_tune_set(10, 0)
+                    res[f"{name}_T{T}_{f'tiled{tt}' if tiled else 'one_row'}"] = {"us": sec * 1e6}
+        res["workload"] = "router: score rows + selection, two launches, softmax top-8"
+        return res
+
     other_configs = {}
     configs = args.configs if args.configs is not None else ("" if args.tune else "c1,c2,c4,c5")
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
             other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "c5skew": lambda: bench_c5(True), "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail, "readprobe": bench_readprobe,
-                                   "slotbench": bench_slotbench}[name]()
+                                   "slotbench": bench_slotbench, "router": bench_router}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
 

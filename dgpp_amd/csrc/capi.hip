@@ -378,8 +378,7 @@ int dgpp_moe_config_validate(const DgppMoeConfig* c) {
 int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const float* bias, int32_t* ids,
                            float* weights, float* scores, float* biased, const DgppMoeConfig* cfg, int tokens,
                            void* stream, int* counters, int allow_tiled) {
-  (void)counters;
-  (void)allow_tiled;
+  (void)counters;   // the two-launch form runs either way; the counters stay at rest, as the reference's tiled branch leaves them
   const int rc = dgpp_moe_config_validate(cfg);
   if (rc != DGPP_OK) return rc;
   if (tokens <= 0) return DGPP_OK;
@@ -389,7 +388,7 @@ int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const f
   if (scores == biased) return fail_arg("moe_router: scores and biased must not alias");
   if (cfg->n_experts > 65535 || tokens > 65535) return fail_arg("moe_router: grid dimension overflow");
   int r = finish(run_router_dots(cfg->router_mode, hidden, gate, bias, scores, biased, tokens, cfg->hidden,
-                                 cfg->n_experts, as_stream(stream)),
+                                 cfg->n_experts, as_stream(stream), allow_tiled),
                  "moe_router");
   if (r != DGPP_OK) return r;
   return finish(run_router_select(cfg->router_mode, scores, biased, ids, weights, tokens, cfg->n_experts, cfg->top_k,

@@ -11,7 +11,7 @@
 namespace dgpp_amd {
 
 hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
-                           float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream);
+                           float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream, int allow_tiled = 1);
 hipError_t run_router_select(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
                              int tokens, int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream);
 // tokens <= 16, n_experts <= 512, top_k <= 16; order may be null (selection only).

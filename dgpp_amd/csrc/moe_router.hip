@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include "../../include/dgpp_amd.h"
+#include "gemv_core.hpp"
 #include "moe_misc.hpp"
 #include "moe_rank.hpp"
 #include "numerics.hpp"
@@ -75,6 +76,96 @@ __global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_kernel(
   }
 }
 
+// The same dots for a batch of rows (sixteen and more): a wavefront keeps a TT x EE tile of (token, expert) sums, so a
+// step's TT + EE vector loads feed TT * EE * 8 fmas and a gate row is fetched once per TT tokens instead of once per
+// token. Every (token, expert) sum is still one wavefront's: lane l takes the 16-byte vectors l, l + 64, ... in
+// ascending order, eight fmas each in element order, then the same butterfly - bit for bit the kernel above. Sixteen
+// lanes then finish one score each. Counterpart of the reference's tiled dots (src/kernels/glm_moe.cu:735-835), which
+// stages 16 x 16 tiles in shared memory; here the tile lives in registers and the L2 serves the re-reads.
+constexpr int kTileExperts = 4;
+constexpr int kRouterTiledFromTokens = 32;   // measured: below this the one-row form's many wavefronts win (the reference tiles from 16)
+
+template <int kMode, int TT>
+__global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_tile_kernel(
+    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ gate, const float* __restrict__ bias,
+    float* __restrict__ scores, float* __restrict__ biased, int tokens, int hidden_dim, int n_experts) {
+  constexpr int EE = kTileExperts;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int e0 = (blockIdx.x * kRouterWaves + wave) * EE;
+  const int t0 = blockIdx.y * TT;
+  if (e0 >= n_experts) return;
+  const uint4* x[TT];
+  const uint4* w[EE];
+#pragma unroll
+  for (int i = 0; i < TT; ++i)   // rows past the batch repeat its last row; their sums are never stored
+    x[i] = reinterpret_cast<const uint4*>(hidden + static_cast<size_t>(min(t0 + i, tokens - 1)) * hidden_dim);
+#pragma unroll
+  for (int j = 0; j < EE; ++j)
+    w[j] = reinterpret_cast<const uint4*>(gate + static_cast<size_t>(min(e0 + j, n_experts - 1)) * hidden_dim);
+  float dot[TT][EE];
+#pragma unroll
+  for (int i = 0; i < TT; ++i)
+#pragma unroll
+    for (int j = 0; j < EE; ++j) dot[i][j] = 0.f;
+  const int vecs = hidden_dim / 8;
+  uint4 xn[TT], wn[EE];   // the next step's vectors, in flight while this step's fmas run
+  auto fetch = [&](int v) {
+    const int at = v < vecs ? v : lane;   // past the end: a harmless re-read, never used
+#pragma unroll
+    for (int i = 0; i < TT; ++i) xn[i] = x[i][at];
+#pragma unroll
+    for (int j = 0; j < EE; ++j) wn[j] = w[j][at];
+  };
+  if (lane < vecs) fetch(lane);
+  for (int v = lane; v < vecs; v += kWaveSize) {
+    uint4 xv[TT], wv[EE];
+#pragma unroll
+    for (int i = 0; i < TT; ++i) xv[i] = xn[i];
+#pragma unroll
+    for (int j = 0; j < EE; ++j) wv[j] = wn[j];
+    fetch(v + kWaveSize);
+#pragma unroll
+    for (int i = 0; i < TT; ++i) {
+      const uint32_t xw[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+#pragma unroll
+      for (int j = 0; j < EE; ++j) {
+        const uint32_t ww[4] = {wv[j].x, wv[j].y, wv[j].z, wv[j].w};
+        float d = dot[i][j];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          d = fmaf(bits_f32(xw[q] << 16), bits_f32(ww[q] << 16), d);
+          d = fmaf(bits_f32(xw[q] & 0xFFFF0000u), bits_f32(ww[q] & 0xFFFF0000u), d);
+        }
+        dot[i][j] = d;
+      }
+    }
+  }
+  float mine = 0.f;   // lane i * EE + j finishes the tile's (i, j) score
+#pragma unroll
+  for (int i = 0; i < TT; ++i)
+#pragma unroll
+    for (int j = 0; j < EE; ++j) {
+      const float s = wave_sum(dot[i][j]);
+      if (lane == i * EE + j) mine = s;
+    }
+  const int t = t0 + lane / EE, e = e0 + lane % EE;
+  if (lane >= TT * EE || t >= tokens || e >= n_experts) return;
+  const size_t at = static_cast<size_t>(t) * n_experts + e;
+  if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
+    const float l = bf16_to_f32(f32_to_bf16(mine));
+    scores[at] = l;
+    biased[at] = l;
+  } else {
+    float sc;
+    if (kMode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS)
+      sc = sqrtf(mine > 20.f ? mine : log1pf(expf(mine)));
+    else
+      sc = 1.0f / (1.0f + expf(-mine));
+    scores[at] = sc;
+    biased[at] = sc + bias[e];
+  }
+}
+
 // One wavefront per token, the whole score row in registers (router_select.hpp): 64 * PER_LANE experts.
 template <int kMode, int PER_LANE>
 __global__ __launch_bounds__(kWaveSize) void router_select_reg_kernel(
@@ -131,9 +222,28 @@ __global__ __launch_bounds__(1024) void router_select_order_kernel(
 }  // namespace
 
 hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
-                           float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream) {
+                           float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream, int allow_tiled) {
   const int vec = (hidden_dim % 8 == 0) && ((reinterpret_cast<uintptr_t>(hidden) & 15u) == 0) &&
                   ((reinterpret_cast<uintptr_t>(gate) & 15u) == 0);
+  const int tuned = tune_get(kTuneRouterTile);   // bench / test switch: 2 or 4 forces the tiled form with that tile
+  if (allow_tiled && vec && (tokens >= kRouterTiledFromTokens || tuned > 0)) {
+    // Two tokens per wavefront (more wavefronts in flight) until the batch is large enough that four (fewer gate
+    // re-reads) pays.
+    const int tt = tuned > 0 ? (tuned >= 4 ? 4 : 2) : (tokens >= 128 ? 4 : 2);
+    const dim3 grid((n_experts + kRouterWaves * kTileExperts - 1) / (kRouterWaves * kTileExperts), (tokens + tt - 1) / tt);
+    const dim3 block(kRouterWaves * kWaveSize);
+    auto go = [&](auto kern) {
+      hipLaunchKernelGGL(kern, grid, block, 0, stream, hidden, gate, bias, scores, biased, tokens, hidden_dim, n_experts);
+    };
+    if (mode == DGPP_ROUTER_SOFTMAX_TOPK)
+      tt == 4 ? go(router_dots_tile_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 4>) : go(router_dots_tile_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 2>);
+    else if (mode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS)
+      tt == 4 ? go(router_dots_tile_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS, 4>)
+              : go(router_dots_tile_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS, 2>);
+    else
+      tt == 4 ? go(router_dots_tile_kernel<DGPP_ROUTER_SIGMOID_BIAS, 4>) : go(router_dots_tile_kernel<DGPP_ROUTER_SIGMOID_BIAS, 2>);
+    return hipGetLastError();
+  }
   const dim3 grid((n_experts + kRouterWaves - 1) / kRouterWaves, tokens);
   const dim3 block(kRouterWaves * kWaveSize);
   if (mode == DGPP_ROUTER_SOFTMAX_TOPK)

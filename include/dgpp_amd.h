@@ -102,8 +102,11 @@ typedef struct DgppMoeConfig {
 int dgpp_moe_config_validate(const DgppMoeConfig* cfg);
 
 /* ---- router ------------------------------------------------------------------------------ */
-/* src/kernels/glm_moe_launch.hpp:23 (launch_moe_router). counters (nullable) is accepted for
- * signature parity; the two-kernel form is used either way and the counters stay zero. */
+/* src/kernels/glm_moe_launch.hpp:23 (launch_moe_router). counters (nullable) is accepted for signature parity; the
+ * two-launch form (score rows, then the selection) runs either way and the counters stay zero - hosts that want the
+ * selection off the critical path run it inside a later launch (the extensions below). allow_tiled != 0: from 32 rows
+ * on (the reference: 16) the score rows come from the token-tiled kernel (a gate row fetched once per two or four
+ * tokens), bit for bit the one-row form's values (src/kernels/glm_moe.cu:735-760, :848-866). */
 int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const float* bias,
                            int32_t* ids, float* weights, float* scores, float* biased,
                            const DgppMoeConfig* cfg, int tokens, void* stream, int* counters,

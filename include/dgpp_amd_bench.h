@@ -27,8 +27,9 @@ extern "C" {
  * key 9: 1 keeps the shared expert's passes of the layer driver
  * on the caller's stream, 2 moves them to a second stream beside the routed passes at every batch size (default:
  * from three tokens on); 3 and 4 keep one stream and never / always fold the accumulation into the shared down pass
- * (default: at one token). Outputs do not depend on keys
- * 1 - 4 and 6 - 9; keys 0 and
+ * (default: at one token); key 10: 2 or 4 runs the router's token-tiled score kernel at every batch size with that many tokens per
+ * wavefront (0 = automatic: tiled from 32 rows on, 4 tokens from 128 rows on). Outputs do not depend on keys
+ * 1 - 4 and 6 - 10; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
  * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);

@@ -282,3 +282,33 @@ def test_router_select_order_is_bitwise_select_then_slot_order(gpu, mode, E, K, 
     assert np.array_equal(host(w1), host(w2)) and np.array_equal(host(w1), host(w3))
     assert np.array_equal(host(o1), host(o2))
     assert np.array_equal(np.sort(host(o2)), np.arange(slots))
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("E,H,T", [(96, 512, 16), (258, 1024, 37), (30, 4096, 64), (256, 6144, 19)])
+def test_router_tiled_dots_are_bitwise_the_one_row_form(gpu, mode, E, H, T):
+    """tests/cuda/glm_moe_test.cu moe_router_tiled_dots_are_bitwise_the_warp_form: from sixteen rows on the score rows
+    come from the token-tiled kernel; scores, biased, ids and weights are bit for bit those of the one-row form."""
+    K = 6
+    x = hg.normal_bf16(mode + 11 + E, (T, H))
+    gate = hg.normal_bf16(mode + 19 + H, (E, H), 1.0 / np.sqrt(H))
+    bias = hg.normal_f32(mode + 5, (E,), 0.02)
+    cfg = L.make_config(H, 64, E, K, router_mode=mode, routed_scaling_factor=1.0 if mode == 1 else 2.5)
+    x_d, g_d, b_d = dev(x), dev(gate), (None if mode == 1 else dev(bias))
+    from dgpp_amd import _lib
+    res = []
+    for tiled, tile in ((False, 0), (True, 0), (True, 2), (True, 4)):   # 0: the launcher's own choice for this batch
+        ids_d, w_d = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32)
+        sc_d, bi_d = dev_empty((T, E), np.float32), dev_empty((T, E), np.float32)
+        sc_d.fill_(-7.0), bi_d.fill_(-7.0)
+        _lib.load().dgpp_tune_set(10, tile)
+        try:
+            L.launch_moe_router(x_d, g_d, b_d, ids_d, w_d, sc_d, bi_d, cfg, T, None, None, tiled)
+        finally:
+            _lib.load().dgpp_tune_set(10, 0)
+        sync()
+        res.append([host(t).copy() for t in (sc_d, bi_d, ids_d, w_d)])
+    for other in res[1:]:
+        for a, b, name in zip(res[0], other, ("scores", "biased", "ids", "weights")):
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), name
+        assert not np.any(other[0] == -7.0), "every score of the batch is written"
