@@ -707,6 +707,25 @@ def main():
                         res[key] = {"us": sec * 1e6, "gbps": buf.numel() / sec / 1e9, "us_min": st["us_min"], "us_max": st["us_max"]}
                         if label not in best or res[key]["gbps"] > best[label][1]:
                             best[label] = (key, res[key]["gbps"])
+            if label == "cold_1GiB":
+                # What ONE cold launch of a given size costs (the yardstick for the small-batch GEMV launches, which read
+                # 17 - 60 MB each): successive launches read successive windows of the 1 GiB buffer, so every window has
+                # left the caches by the time it is read again. Time per launch includes the hand-over to the next launch
+                # of the graph, as a layer's dependent launches do.
+                win = {}
+                for w_mib in (16, 32, 48, 64, 128, 256):
+                    nwin = mib // w_mib
+                    wbytes = w_mib << 20
+                    for blocks in (1024, 2048, 4096):
+                        def step(i):
+                            if lib.dgpp_probe_read(buf.data_ptr() + (i % nwin) * wbytes, wbytes, sink.data_ptr(), 0, blocks, 1,
+                                                   stream.cuda_stream) != 0:
+                                raise RuntimeError(lib.dgpp_last_error().decode())
+                        sec = time_graph(step, max(16, nwin), 2)
+                        cur = win.get(w_mib)
+                        if cur is None or sec * 1e6 < cur["us"]:
+                            win[w_mib] = {"us": sec * 1e6, "gbps": wbytes / sec / 1e9, "blocks": blocks}
+                res["cold_window_per_launch"] = {f"{k}MiB": v for k, v in win.items()}
             del buf
         res["best"] = {k: {"form": v[0], "gbps": v[1], "frac_of_peak": v[1] / HBM_PEAK_GBPS} for k, v in best.items()}
         return res
