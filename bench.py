@@ -67,6 +67,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="'layer', 'gate_up' or 'down': run only that timed graph (for profiling)")
     ap.add_argument("--no-others", action="store_true", help="skip the T=1/4/8 side measurements")
+    ap.add_argument("--no-probe", action="store_true",
+                    help="skip the plain-read yardstick (a cold read of the same byte count) beside the two kernel legs")
     ap.add_argument("--eager", action="store_true", help="launch the timed steps eagerly instead of as one HIP graph")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
@@ -185,6 +187,29 @@ def main():
                           "us_max": float(per.max()) * 1e6, "replays": replays, "steps_per_replay": steps})
         return float(np.median(per))
 
+    probe_buf = {}
+
+    def plain_read_us(nbytes):
+        """What ONE cold launch of the library's plain streaming-read probe costs for this many bytes (16-byte loads, a
+        contiguous span per block, nothing computed or stored): successive launches walk successive windows of a 1 GiB
+        buffer, so every window has left the caches when it is read again. The yardstick a weight-streaming launch of
+        the same size is read against; timed like the kernel legs (median of graph replays)."""
+        if "buf" not in probe_buf:
+            probe_buf["buf"] = torch.zeros(1 << 30, dtype=torch.uint8, device=dev)
+            probe_buf["sink"] = torch.zeros(8192, dtype=torch.int32, device=dev)
+        buf, sink = probe_buf["buf"], probe_buf["sink"]
+        nbytes = int(nbytes) // 256 * 256
+        nwin = max(1, buf.numel() // nbytes)
+        best = None
+        for blocks in (1024, 2048, 4096):
+            def step(i):
+                if lib.dgpp_probe_read(buf.data_ptr() + (i % nwin) * nbytes, nbytes, sink.data_ptr(), 0, blocks, 1,
+                                       stream.cuda_stream) != 0:
+                    raise RuntimeError(lib.dgpp_last_error().decode())
+            sec = time_graph(step, max(16, min(nwin, 64)), 2)
+            best = sec if best is None or sec < best else best
+        return best * 1e6
+
     def measure(T, steps, warmup, only=""):
         # a graph holds whole walks of the ring (at least four), so that a replay never meets a layer its predecessor has
         # just left and the few microseconds between two replays stay below one percent of a replay
@@ -239,6 +264,9 @@ def main():
             res["gate_up_us"] = sec_k * 1e6
             res["gate_up_bytes"] = kbytes
             res["gate_up_gbps"] = kbytes / sec_k / 1e9
+            if not args.no_probe:
+                res["gate_up_plain_read_us"] = plain_read_us(kbytes)
+                res["gate_up_frac_of_plain_read"] = res["gate_up_plain_read_us"] / res["gate_up_us"]
         def down(i):   # the layer's second GEMV kernel: token-major down projection + ordered accumulation
             l = i % nL
             L.launch_moe_slot_down_accum_fp4(acts[l], I, layers[l].ids_ptr, layers[l]._views_ptr, H, I, T, K,
@@ -252,6 +280,9 @@ def main():
             res["down_us"] = sec_d * 1e6
             res["down_bytes"] = dbytes
             res["down_gbps"] = dbytes / sec_d / 1e9
+            if not args.no_probe:
+                res["down_plain_read_us"] = plain_read_us(dbytes)
+                res["down_frac_of_plain_read"] = res["down_plain_read_us"] / res["down_us"]
         return res
 
     for lyr in layers:     # device pointer of the layer's expert table, for the single-kernel leg
@@ -923,6 +954,9 @@ def main():
                             "traffic": traffic.get("gate_up") if same_workload else None,
                             "traffic_source": (TRAFFIC_PROFILE + ": " + traffic.get("gate_up_kernel", "")) if same_workload else None,
                             "bytes_per_launch": main_res["gate_up_bytes"], "us_per_launch": main_res["gate_up_us"]}
+        if "gate_up_plain_read_us" in main_res:   # this chip's plain cold read of the same byte count, same timing method
+            line["roofline"]["plain_read_same_bytes_us"] = main_res["gate_up_plain_read_us"]
+            line["roofline"]["frac_of_plain_read"] = main_res["gate_up_frac_of_plain_read"]
         if "down_us" in main_res:
             line["roofline"]["second_kernel"] = {
                 "kernel": "token_down_accum_kernel<MXFP4> (down GEMV + ordered accumulation, bf16 out)",
@@ -930,6 +964,9 @@ def main():
                 "traffic": traffic.get("down") if same_workload else None,
                 "frac": main_res["down_gbps"] / HBM_PEAK_GBPS, "bytes_per_launch": main_res["down_bytes"],
                 "us_per_launch": main_res["down_us"]}
+            if "down_plain_read_us" in main_res:
+                line["roofline"]["second_kernel"]["plain_read_same_bytes_us"] = main_res["down_plain_read_us"]
+                line["roofline"]["second_kernel"]["frac_of_plain_read"] = main_res["down_frac_of_plain_read"]
     print(json.dumps(line))
 
 
