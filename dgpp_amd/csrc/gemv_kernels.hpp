@@ -71,17 +71,21 @@ struct DenseArgs {
   const float* a4_gs = nullptr;
 };
 
-// XV > 0 (one activation row of at most 8 * XV * kBlockThreads aligned elements): the row's loads are issued first, the
-// first row step's weight loads right behind them, and only then is the row committed to LDS - the weight stream
-// starts one memory round trip earlier in every block. Same chain per row as the plain form.
-template <int FMT, int MAXR, int NB, bool NT, int XV = 0>
+template <int FMT, int MAXR, int NB, bool NT>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_kernel(DenseArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  stage_activations<FMT>(a.act, a.act_stride, a.m, a.k, lds);
+  __syncthreads();
+  const float divisor = load_divisor<FMT>(a.global);
   const int rpw = kWave >> g.l2;
   const int wave = threadIdx.x >> 6;
   int row0 = blockIdx.x * block_rows(g, steps) + wave * rpw;
-  auto store = [&](const LaneRow& lr, const float (&acc)[MAXR], float divisor) {
+  for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+    if (row0 >= a.n) break;
+    const auto lr = lane_row<FMT, NT>(a.mat, row0, a.n, a.k, g.l2);
+    float acc[MAXR];
+    row_dots<FMT, MAXR, NB>(lr, g, a.mat.cs, lds, chunks, a.m, acc);
     if (lr.li == 0 && lr.row < a.n) {
 #pragma unroll
       for (int r = 0; r < MAXR; ++r) {
@@ -95,35 +99,6 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_ke
         }
       }
     }
-  };
-  int s = 0;
-  float divisor;
-  if constexpr (XV > 0) {
-    static_assert(MAXR == 1, "the split stage carries one activation row");
-    StageRegs<XV> xr;
-    stage_issue<FMT, XV>(a.act, a.k, threadIdx.x, kBlockThreads, xr);
-    const auto lr = lane_row<FMT, NT>(a.mat, row0, a.n, a.k, g.l2);   // rows past n repeat row n - 1 and are dropped
-    ChunkRegs first[NB];
-    issue_pass<FMT, NB>(lr, 0, g.l2, a.mat.cs, first);
-    divisor = load_divisor<FMT>(a.global);
-    stage_commit<FMT, XV>(xr, a.k, threadIdx.x, kBlockThreads, lds);
-    __syncthreads();
-    float acc[MAXR];
-    row_dots_pre<FMT, MAXR, NB>(lr, g, a.mat.cs, lds, chunks, a.m, first, acc);
-    store(lr, acc, divisor);
-    s = 1;
-    row0 += kWavesPerBlock * rpw;
-  } else {
-    stage_activations<FMT>(a.act, a.act_stride, a.m, a.k, lds);
-    __syncthreads();
-    divisor = load_divisor<FMT>(a.global);
-  }
-  for (; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
-    if (row0 >= a.n) break;
-    const auto lr = lane_row<FMT, NT>(a.mat, row0, a.n, a.k, g.l2);
-    float acc[MAXR];
-    row_dots<FMT, MAXR, NB>(lr, g, a.mat.cs, lds, chunks, a.m, acc);
-    store(lr, acc, divisor);
   }
 }
 
@@ -855,17 +830,7 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
         hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
       });
     };
-    // One aligned row of at most 8192 elements whose weights stream through once: the split-stage form.
-    const bool split = a.m == 1 && a.once != 0 && tune_get(kTuneSplitStage) != 1 && a.k <= 8 * 4 * kBlockThreads &&
-                       (reinterpret_cast<uintptr_t>(a.act) & 15u) == 0 && a.k % 8 == 0;
-    if (split) {
-      auto go_split = [&](auto kern) {
-        err = ensure_lds(kern, lds);
-        if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g, steps);
-      };
-      if (a.k <= 8 * 2 * kBlockThreads) go_split(gemv_dense_kernel<FMT, 1, NB, true, 2>);
-      else go_split(gemv_dense_kernel<FMT, 1, NB, true, 4>);
-    } else if (a.m == 1) go(std::integral_constant<int, 1>{});
+    if (a.m == 1) go(std::integral_constant<int, 1>{});
     else if (a.m == 2) go(std::integral_constant<int, 2>{});
     else if (a.m <= 4) go(std::integral_constant<int, 4>{});
     else go(std::integral_constant<int, 8>{});
