@@ -467,6 +467,31 @@ def main():
         ids5 = torch.empty((cT, cK), dtype=torch.int32, device=dev)
         w5 = torch.empty((cT, cK), dtype=torch.float32, device=dev)
         L.launch_moe_router_select(lg5, lg5, ids5, w5, cfg5, cT, stream)
+
+        # The routed experts in the activation-quantized NVFP4 (W4A4) form, stitched from its launchers: segment, quantize
+        # the token rows, grouped gate and up over the row list, SwiGLU + quantize in one launch, grouped down, ordered
+        # accumulation over the BF16 down rows. Different numerics from the legs beside it (NVFP4 activations).
+        R = cT * cK
+        rows_l, slot_row = torch.empty(R + cT, dtype=torch.int32, device=dev), torch.empty(R, dtype=torch.int32, device=dev)
+        segs4 = torch.empty((cE + 1, 3), dtype=torch.int32, device=dev)
+        ss_h, ss_i = L.nvfp4_act_scale_stride(cH), L.nvfp4_act_scale_stride(cI)
+        xc, xs_, xg = (torch.empty((cT, cH // 2), dtype=torch.uint8, device=dev), torch.empty((cT, ss_h), dtype=torch.uint8, device=dev),
+                       torch.empty(cT, dtype=torch.float32, device=dev))
+        ac4, as4, ag4 = (torch.empty((R, cI // 2), dtype=torch.uint8, device=dev), torch.empty((R, ss_i), dtype=torch.uint8, device=dev),
+                         torch.empty(R, dtype=torch.float32, device=dev))
+        g4, u4 = (torch.empty((R, cI), dtype=torch.int16, device=dev) for _ in range(2))
+        d4 = torch.empty((R, cH), dtype=torch.int16, device=dev)
+
+        def w4a4_chain(ids_t, w_t):
+            def fn(i):
+                L.launch_moe_segment(ids_t, cT, cK, cE, rows_l, slot_row, segs4, stream)
+                L.launch_quantize_rows_nvfp4(x, cH, cT, cH, xc, xs_, xg, stream)
+                L.launch_moe_grouped_w4a4_bf16(xc, xs_, xg, rows_l, segs4, cE, cT, lay.views_ptr, 0, g4, cI, cI, cH, stream)
+                L.launch_moe_grouped_w4a4_bf16(xc, xs_, xg, rows_l, segs4, cE, cT, lay.views_ptr, 1, u4, cI, cI, cH, stream)
+                L.launch_swiglu_quantize_rows_nvfp4(g4, u4, cI, R, cI, float("inf"), ac4, as4, ag4, stream)
+                L.launch_moe_grouped_w4a4_bf16(ac4, as4, ag4, None, segs4, cE, cT, lay.views_ptr, 2, d4, cH, cH, cI, stream)
+                L.launch_moe_accum_ordered_f32_bf16down(routed, d4, cH, slot_row, ids_t, w_t, cT, cK, cH, stream)
+            return fn
         if skew:
             # The same layer under Zipf(1.1) expert popularity: few experts take most tokens, so routed segments reach
             # 16 and more rows - the shape the matrix-core grouped form is for. Routes are given (ids drawn from the
@@ -484,7 +509,8 @@ def main():
                                f"{int(counts.max())} tokens, {int(np.count_nonzero(counts >= 16))} experts with >= 16 tokens",
                    "algorithmic_bytes": nb, "flops": 2.0 * cT * cK * 3 * cI * cH}
             legs = (("decode_slots", lambda i: lay.enqueue_decode_routed(x, cH, ids_z, w_z, None, cT, stream, out_f32=routed)),
-                    ("grouped_matrix_core", lambda i: lay.enqueue_prefill_routed(x, cH, ids_z, w_z, None, cT, stream, out_f32=routed)))
+                    ("grouped_matrix_core", lambda i: lay.enqueue_prefill_routed(x, cH, ids_z, w_z, None, cT, stream, out_f32=routed)),
+                    ("grouped_matrix_core_w4a4", w4a4_chain(ids_z, w_z)))
             for name, fn in legs:
                 sec = time_graph(fn, max(args.steps // 10, 5), 2)
                 res[name] = {"us": sec * 1e6, "gbps": nb / sec / 1e9, "frac_of_peak": nb / sec / 1e9 / HBM_PEAK_GBPS,
@@ -546,6 +572,7 @@ def main():
         for name, fn, nb in (("layer", full, nbytes), ("layer_stitched_from_launchers", stitched, nbytes),
                              ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
                              ("routed_only_matrix_core", routed_mc, uniq * per_expert + cT * cH * 6),
+                             ("routed_only_matrix_core_w4a4", w4a4_chain(ids5, w5), uniq * per_expert + cT * cH * 6),
                              ("shared_only_gemv_launchers", shared_part, shared_bytes + cT * cH * 4),
                              ("shared_only", shared_mc, shared_bytes + cT * cH * 4),
                              ("shared_only_w8a8_scaled_matrix_core", shared_w8a8, shared_bytes + cT * cH * 4),
@@ -738,26 +765,28 @@ def main():
                         res[key] = {"us": sec * 1e6, "gbps": buf.numel() / sec / 1e9, "us_min": st["us_min"], "us_max": st["us_max"]}
                         if label not in best or res[key]["gbps"] > best[label][1]:
                             best[label] = (key, res[key]["gbps"])
-            if label == "cold_1GiB":
-                # What ONE cold launch of a given size costs (the yardstick for the small-batch GEMV launches, which read
-                # 17 - 60 MB each): successive launches read successive windows of the 1 GiB buffer, so every window has
-                # left the caches by the time it is read again. Time per launch includes the hand-over to the next launch
-                # of the graph, as a layer's dependent launches do.
-                win = {}
-                for w_mib in (16, 32, 48, 64, 128, 256):
-                    nwin = mib // w_mib
-                    wbytes = w_mib << 20
-                    for blocks in (1024, 2048, 4096):
-                        def step(i):
-                            if lib.dgpp_probe_read(buf.data_ptr() + (i % nwin) * wbytes, wbytes, sink.data_ptr(), 0, blocks, 1,
-                                                   stream.cuda_stream) != 0:
-                                raise RuntimeError(lib.dgpp_last_error().decode())
-                        sec = time_graph(step, max(16, nwin), 2)
-                        cur = win.get(w_mib)
-                        if cur is None or sec * 1e6 < cur["us"]:
-                            win[w_mib] = {"us": sec * 1e6, "gbps": wbytes / sec / 1e9, "blocks": blocks}
-                res["cold_window_per_launch"] = {f"{k}MiB": v for k, v in win.items()}
             del buf
+        # What ONE cold launch of a given size costs (the yardstick for the small-batch GEMV launches, which read
+        # 17 - 60 MB each): successive launches read successive windows of a 1 GiB buffer, so every window has left the
+        # caches by the time it is read again. Time per launch includes the hand-over to the next launch of the graph, as
+        # a layer's dependent launches do.
+        mib = 1024
+        buf = torch.zeros(mib << 20, dtype=torch.uint8, device=dev)
+        win = {}
+        for w_mib in (16, 32, 48, 64, 128, 256):
+            nwin = mib // w_mib
+            wbytes = w_mib << 20
+            for blocks in (1024, 2048, 4096):
+                def step(i):
+                    if lib.dgpp_probe_read(buf.data_ptr() + (i % nwin) * wbytes, wbytes, sink.data_ptr(), 0, blocks, 1,
+                                           stream.cuda_stream) != 0:
+                        raise RuntimeError(lib.dgpp_last_error().decode())
+                sec = time_graph(step, max(16, nwin), 2)
+                cur = win.get(w_mib)
+                if cur is None or sec * 1e6 < cur["us"]:
+                    win[w_mib] = {"us": sec * 1e6, "gbps": wbytes / sec / 1e9, "blocks": blocks}
+        res["cold_window_per_launch"] = {f"{k}MiB": v for k, v in win.items()}
+        del buf
         res["best"] = {k: {"form": v[0], "gbps": v[1], "frac_of_peak": v[1] / HBM_PEAK_GBPS} for k, v in best.items()}
         return res
 
