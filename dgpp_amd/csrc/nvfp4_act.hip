@@ -347,6 +347,7 @@ int dgpp_minimax_swiglu_f32(const float* gate, const float* up, uint16_t* output
   const int vec = ((reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up)) & 15u) == 0 &&
                   (reinterpret_cast<uintptr_t>(output) & 7u) == 0;
   const int64_t lanes = (count + 3) / 4;
+  if ((lanes + 255) / 256 > 0x7FFFFFFFLL) return report_invalid(std::string(who) + ": grid dimension overflow");
   hipLaunchKernelGGL(swiglu_f32_rows_kernel, dim3(static_cast<unsigned>((lanes + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), gate, up, output, count, alpha, limit, vec);
   return report_hip(hipGetLastError(), who);
