@@ -70,6 +70,11 @@ SIGNATURES = {
     "dgpp_launch_moe_router": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_launch_moe_router_select": (_I, [_P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_router_select_order": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P]),
+    "dgpp_dense_fp4_decode_shape": (_I, [_I, _I, _I, _I]),
+    "dgpp_try_dense_fp4_decode_bf16": (_I, [_P, _Z, _P, _P, _I, _P, _I, _I, _I, _P, _I, _P]),
+    "dgpp_launch_scale_gemm_tile_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
+    "dgpp_launch_scale_gemm_tile_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
+    "dgpp_launch_moe_hash_routes": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P]),
     "dgpp_launch_moe_router_dots": (_I, [_P, _P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu_fp4": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P, _I]),

@@ -396,6 +396,19 @@ int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const f
                 "moe_router");
 }
 
+int dgpp_launch_moe_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float* scores, int32_t* ids,
+                                float* weights, const DgppMoeConfig* cfg, int vocab, int n_tokens, void* stream) {
+  const int rc = dgpp_moe_config_validate(cfg);
+  if (rc != DGPP_OK) return rc;
+  if (n_tokens <= 0) return DGPP_OK;
+  if (!tokens || !tid2eid || !scores || !ids || !weights || vocab <= 0) return fail_arg("moe_hash_routes: null pointer");
+  if (cfg->router_mode == DGPP_ROUTER_SOFTMAX_TOPK)
+    return fail_arg("moe_hash_routes: the softmax router leaves logits, not scores");
+  return finish(run_hash_routes(tokens, tid2eid, scores, ids, weights, n_tokens, vocab, cfg->n_experts, cfg->top_k,
+                                cfg->routed_scaling_factor, cfg->norm_topk_prob ? 1 : 0, as_stream(stream)),
+                "moe_hash_routes");
+}
+
 int dgpp_launch_moe_router_dots(const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
                                 float* biased, const DgppMoeConfig* cfg, int tokens, void* stream) {
   const int rc = dgpp_moe_config_validate(cfg);
@@ -928,6 +941,18 @@ int dgpp_launch_dense_mma_f32(const uint16_t* act, size_t act_stride, const uint
                               float* out, int m, int n, int k, void* stream, size_t out_stride) {
   return dense_mma_fp8(act, act_stride, payload, scales, 0, out, 1, m, n, k, out_stride, 7, 7, nullptr, 0, stream, "dense_mma");
 }
+/* src/kernels/scale_gemm.hpp:173-180: the scale GEMM's tile form (many rows against one pass over the weights): here the
+ * matrix-core dense form with the scale grid's shifts. */
+int dgpp_launch_scale_gemm_tile_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                     const float* w_scales, uint16_t* out, int m, int n, int k, void* stream, int rs, int cs) {
+  return dense_mma_fp8(act, act_row_stride_elems, w_payload, w_scales, 0, out, 0, m, n, k, 0, rs, cs, nullptr, 0, stream,
+                       "scale_gemm_tile");
+}
+int dgpp_launch_scale_gemm_tile_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                    const float* w_scales, float* out, int m, int n, int k, void* stream, int rs, int cs) {
+  return dense_mma_fp8(act, act_row_stride_elems, w_payload, w_scales, 0, out, 1, m, n, k, 0, rs, cs, nullptr, 0, stream,
+                       "scale_gemm_tile");
+}
 int dgpp_launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
                                   uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
                                   void* ws, size_t ws_bytes) {
@@ -1081,6 +1106,21 @@ int dgpp_launch_dense_mma_fp4_prod_bf16(const uint16_t* act, size_t act_stride, 
   if (m <= 0 || n <= 0) return DGPP_OK;
   return grouped_mma_fp4(act, act_stride, seg, 1, m, 0, views, which, out, 0, static_cast<size_t>(n), n, k, stream, nullptr,
                          fp4_group);
+}
+/* src/kernels/dense_fp4_decode.cu:297-308: the small dense NVFP4 shard form. The shape rule is the reference's (one
+ * 16-row tile, n and k up to 17408, k in whole 128-element steps); the launch is the production form's, whose bits the
+ * reference's decode form shares. *launched = 0 and nothing runs when the shape is outside the rule. */
+int dgpp_dense_fp4_decode_shape(int m, int n, int k, int fp4_group) {
+  return fp4_group == 16 && m > 0 && m <= 16 && n > 0 && n <= 17408 && k > 0 && k <= 17408 && k % 128 == 0;
+}
+int dgpp_try_dense_fp4_decode_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
+                                   const DgppMoeExpertView* views, int which, uint16_t* out, int m, int n, int k,
+                                   void* stream, int fp4_group, int* launched) {
+  if (launched) *launched = 0;
+  if (!dgpp_dense_fp4_decode_shape(m, n, k, fp4_group)) return DGPP_OK;
+  const int rc = dgpp_launch_dense_mma_fp4_prod_bf16(act, act_stride, seg, views, which, out, m, n, k, stream, fp4_group);
+  if (rc == DGPP_OK && launched) *launched = 1;
+  return rc;
 }
 /* src/kernels/dense_fp4_decode.cu:310-319: gate and up of one segment; one launch here, the bits of two prod launches. */
 int dgpp_launch_dense_mma_fp4_gate_up_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,

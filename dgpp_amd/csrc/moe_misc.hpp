@@ -10,6 +10,8 @@
 
 namespace dgpp_amd {
 
+hipError_t run_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float* scores, int32_t* ids, float* weights,
+                           int n_tokens, int vocab, int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream);
 hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
                            float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream, int allow_tiled = 1);
 hipError_t run_router_select(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,

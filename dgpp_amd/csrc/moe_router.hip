@@ -219,7 +219,42 @@ __global__ __launch_bounds__(1024) void router_select_order_kernel(
   order[pos] = s;
 }
 
+// Routes taken from a table instead of the scores' top k (src/kernels/glm_moe.cu:917-949): token t's experts are row
+// tokens[t] of tid2eid (ascending ids), its weights the scores at those ids, normalised and scaled as the selection
+// does: the sum runs over the row in order from zero, + 1e-20, one division per weight. One lane per (token, slot);
+// every lane of a token walks the row's sum itself (top_k <= 16 scores out of one or two cache lines), so the routes
+// leave as coalesced stores.
+__global__ __launch_bounds__(256) void hash_routes_kernel(const int64_t* __restrict__ tokens, const int32_t* __restrict__ tid2eid,
+                                                          const float* __restrict__ scores, int32_t* __restrict__ ids,
+                                                          float* __restrict__ weights, int n_tokens, int vocab, int n_experts,
+                                                          int top_k, float scaling, int norm_topk) {
+  const int64_t at = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (at >= static_cast<int64_t>(n_tokens) * top_k) return;
+  const int t = static_cast<int>(at / top_k), i = static_cast<int>(at - static_cast<int64_t>(t) * top_k);
+  int64_t tok = tokens[t];
+  if (tok < 0 || tok >= vocab) tok = 0;   // a padding row: any table row (its output is never read)
+  const int32_t* row = tid2eid + tok * top_k;
+  const float* sc = scores + static_cast<size_t>(t) * n_experts;
+  float denom = 0.f, mine = 0.f;
+  for (int j = 0; j < top_k; ++j) {
+    const float v = sc[row[j]];
+    denom = denom + v;
+    if (j == i) mine = v;
+  }
+  denom = denom + 1e-20f;
+  ids[at] = row[i];
+  weights[at] = norm_topk ? (mine / denom) * scaling : mine * scaling;
+}
+
 }  // namespace
+
+hipError_t run_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float* scores, int32_t* ids, float* weights,
+                           int n_tokens, int vocab, int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream) {
+  const int64_t lanes = static_cast<int64_t>(n_tokens) * top_k;
+  hipLaunchKernelGGL(hash_routes_kernel, dim3(static_cast<unsigned>((lanes + 255) / 256)), dim3(256), 0, stream, tokens, tid2eid,
+                     scores, ids, weights, n_tokens, vocab, n_experts, top_k, scaling, norm_topk);
+  return hipGetLastError();
+}
 
 hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
                            float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream, int allow_tiled) {

@@ -68,6 +68,30 @@ def launch_moe_router(hidden, gate, bias, ids, weights, scores, biased, cfg: Moe
                                               1 if allow_tiled else 0))
 
 
+def dense_fp4_decode_shape(m, n, k, fp4_group=16) -> bool:
+    return bool(_lib.load().dgpp_dense_fp4_decode_shape(m, n, k, fp4_group))
+
+
+def try_dense_fp4_decode_bf16(act, act_stride, seg, views, which, out, m, n, k, stream=None, fp4_group=16) -> bool:
+    launched = C.c_int(0)
+    _check(_lib.load().dgpp_try_dense_fp4_decode_bf16(_p(act), act_stride, _p(seg), _p(views), which, _p(out), m, n, k,
+                                                      _stream(stream), fp4_group, C.addressof(launched)))
+    return bool(launched.value)
+
+
+def launch_scale_gemm_tile_bf16(act, act_stride, w, scales, out, m, n, k, stream=None, rs=7, cs=7):
+    _check(_lib.load().dgpp_launch_scale_gemm_tile_bf16(_p(act), act_stride, _p(w), _p(scales), _p(out), m, n, k, _stream(stream), rs, cs))
+
+
+def launch_scale_gemm_tile_f32(act, act_stride, w, scales, out, m, n, k, stream=None, rs=7, cs=7):
+    _check(_lib.load().dgpp_launch_scale_gemm_tile_f32(_p(act), act_stride, _p(w), _p(scales), _p(out), m, n, k, _stream(stream), rs, cs))
+
+
+def launch_moe_hash_routes(tokens, tid2eid, scores, ids, weights, cfg: MoeConfig, vocab, n_tokens, stream=None):
+    _check(_lib.load().dgpp_launch_moe_hash_routes(_p(tokens), _p(tid2eid), _p(scores), _p(ids), _p(weights), C.addressof(cfg),
+                                                   vocab, n_tokens, _stream(stream)))
+
+
 def launch_moe_router_dots(hidden, gate, bias, scores, biased, cfg: MoeConfig, tokens, stream=None):
     """Extension: the router's score rows without the selection."""
     _check(_lib.load().dgpp_launch_moe_router_dots(_p(hidden), _p(gate), _p(bias), _p(scores), _p(biased), C.addressof(cfg),

@@ -111,6 +111,12 @@ int dgpp_launch_moe_router(const uint16_t* hidden, const uint16_t* gate, const f
                            int32_t* ids, float* weights, float* scores, float* biased,
                            const DgppMoeConfig* cfg, int tokens, void* stream, int* counters,
                            int allow_tiled);
+/* src/kernels/glm_moe_launch.hpp:30-39 (launch_moe_hash_routes): after the router has left every expert's score in
+ * `scores`, the routes are replaced - ids [n_tokens, top_k] = row tokens[t] of tid2eid (int32 [vocab, top_k], rows
+ * ascending), weights the scores at those ids normalised and scaled as the selection does. tokens: device int64
+ * [n_tokens]; a token id outside [0, vocab) reads row 0. Refused in softmax mode (the router leaves logits there). */
+int dgpp_launch_moe_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float* scores, int32_t* ids,
+                                float* weights, const DgppMoeConfig* cfg, int vocab, int n_tokens, void* stream);
 /* Extension (no counterpart in the reference): step 1 of dgpp_launch_moe_router alone - the score rows (`scores`,
  * and `biased` = scores + bias, or the same values in softmax mode) without the selection, for hosts that run the
  * selection inside a later launch (dgpp_launch_moe_router_select_order, dgpp_launch_moe_select_gate_up_swiglu). */
@@ -387,6 +393,14 @@ int dgpp_launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t* up
 int dgpp_launch_dense_mma_fp4_prod_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
                                         const DgppMoeExpertView* views, int which, uint16_t* out, int m, int n, int k,
                                         void* stream, int fp4_group);
+/* src/kernels/glm_moe_launch.hpp:359-365, dense_fp4_decode.cu:297-308: the small dense NVFP4 shard form. The shape
+ * predicate is the reference's (fp4_group 16, 1 <= m <= 16, n and k <= 17408, k % 128 == 0); a shape inside it runs as
+ * dgpp_launch_dense_mma_fp4_prod_bf16 does (the reference's decode form keeps the production kernel's chain) and sets
+ * *launched to 1; outside it nothing runs and *launched is 0, as the reference returns false. */
+int dgpp_dense_fp4_decode_shape(int m, int n, int k, int fp4_group);
+int dgpp_try_dense_fp4_decode_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
+                                   const DgppMoeExpertView* views, int which, uint16_t* out, int m, int n, int k,
+                                   void* stream, int fp4_group, int* launched);
 /* src/kernels/glm_moe_launch.hpp:366-369 (launch_dense_mma_fp4_gate_up_bf16): gate and up of that segment in one
  * launch; the bits of two dgpp_launch_dense_mma_fp4_prod_bf16 calls. */
 int dgpp_launch_dense_mma_fp4_gate_up_bf16(const uint16_t* act, size_t act_stride, const DgppMoeSegment* seg,
@@ -467,6 +481,12 @@ int dgpp_launch_scale_gemm_grid_e8m0_f32(const uint16_t* act, size_t act_row_str
                                          float* out, int m, int n, int k, void* stream,
                                          size_t out_row_stride_elems, int rs, int cs, void* ws,
                                          size_t ws_bytes, int prefill_tile);
+/* src/kernels/scale_gemm.hpp:173-180 (launch_scale_gemm_tile_*): the scale GEMM's tile form for many rows; here the
+ * matrix-core dense form (16 activation rows per pass over the weights). out row stride n. */
+int dgpp_launch_scale_gemm_tile_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                     const float* w_scales, uint16_t* out, int m, int n, int k, void* stream, int rs, int cs);
+int dgpp_launch_scale_gemm_tile_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                    const float* w_scales, float* out, int m, int n, int k, void* stream, int rs, int cs);
 /* src/kernels/scale_gemm.hpp:85-107: up to four [n_i, k] fp8 matrices against the same rows.
  * `problems` is a HOST array. bf16_weight must be null (that form is outside this path). */
 typedef struct DgppFp8GemvProblem {

@@ -112,6 +112,11 @@ inline void launch_moe_router(const uint16_t* hidden, const uint16_t* gate, cons
   detail::check(dgpp_launch_moe_router(hidden, gate, bias, ids, weights, scores, biased, &c, tokens, stream, counters,
                                        allow_tiled ? 1 : 0));
 }
+inline void launch_moe_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float* scores, int32_t* ids,
+                                   float* weights, const GlmMoeConfig& cfg, int vocab, int n_tokens, hipStream_t stream) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_hash_routes(tokens, tid2eid, scores, ids, weights, &c, vocab, n_tokens, stream));
+}
 // The selection half alone (src/kernels/glm_moe.cu:314-329).
 inline void launch_moe_router_select(const float* scores, const float* biased, int32_t* ids, float* weights,
                                      const GlmMoeConfig& cfg, int tokens, hipStream_t stream) {
@@ -533,6 +538,16 @@ inline void launch_dense_mma_fp4_prod_bf16(const uint16_t* act, size_t act_strid
                                            hipStream_t stream, int fp4_group = kFp4Group) {
   detail::check(dgpp_launch_dense_mma_fp4_prod_bf16(act, act_stride, seg, views, which, out, m, n, k, stream, fp4_group));
 }
+inline bool dense_fp4_decode_shape(int m, int n, int k, int fp4_group = kFp4Group) {
+  return dgpp_dense_fp4_decode_shape(m, n, k, fp4_group) != 0;
+}
+inline bool try_dense_fp4_decode_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* seg, const MoeExpertView* views,
+                                      int which, uint16_t* out, int m, int n, int k, hipStream_t stream,
+                                      int fp4_group = kFp4Group) {
+  int launched = 0;
+  detail::check(dgpp_try_dense_fp4_decode_bf16(act, act_stride, seg, views, which, out, m, n, k, stream, fp4_group, &launched));
+  return launched != 0;
+}
 inline void launch_dense_mma_fp4_gate_up_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* seg,
                                               const MoeExpertView* views, uint16_t* gate, uint16_t* up, int m, int n, int k,
                                               hipStream_t stream, int fp4_group = kFp4Group) {
@@ -617,6 +632,16 @@ inline void launch_scale_gemm_grid_e8m0_f32(const uint16_t* act, size_t act_row_
                                                      stream, out_row_stride_elems, rs, cs, ws, ws_bytes, prefill_tile));
 }
 constexpr int kFp8GemvMaxProblems = 4;
+inline void launch_scale_gemm_tile_bf16(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                        const float* w_scales, uint16_t* out, int m, int n, int k, hipStream_t stream,
+                                        int rs = 7, int cs = 7) {
+  detail::check(dgpp_launch_scale_gemm_tile_bf16(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream, rs, cs));
+}
+inline void launch_scale_gemm_tile_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
+                                       const float* w_scales, float* out, int m, int n, int k, hipStream_t stream,
+                                       int rs = 7, int cs = 7) {
+  detail::check(dgpp_launch_scale_gemm_tile_f32(act, act_row_stride_elems, w_payload, w_scales, out, m, n, k, stream, rs, cs));
+}
 inline void launch_scale_gemv_multi_bf16(const Fp8GemvProblem* problems, int n_problems, const uint16_t* act,
                                          size_t act_row_stride_elems, int rows, int k, hipStream_t stream) {
   detail::check(dgpp_launch_scale_gemv_multi_bf16(problems, n_problems, act, act_row_stride_elems, rows, k, stream));

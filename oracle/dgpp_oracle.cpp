@@ -507,6 +507,25 @@ void orc_shared_gate(const uint16_t* x, int64_t x_stride, const uint16_t* g, int
   }
 }
 
+// src/kernels/glm_moe.cu:917-949: routes from a table; the weights' chain in fp32 (fadd from zero in row order, + 1e-20,
+// one division and one multiplication per weight - this file is compiled with -ffp-contract=off).
+void orc_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float* scores, int n_tokens, int vocab,
+                     int n_experts, int top_k, float scaling, int norm_topk, int32_t* ids, float* weights) {
+  for (int t = 0; t < n_tokens; ++t) {
+    int64_t tok = tokens[t];
+    if (tok < 0 || tok >= vocab) tok = 0;
+    const int32_t* row = tid2eid + tok * top_k;
+    float denom = 0.f;
+    for (int i = 0; i < top_k; ++i) denom = denom + scores[static_cast<size_t>(t) * n_experts + row[i]];
+    denom = denom + 1e-20f;
+    for (int i = 0; i < top_k; ++i) {
+      const float v = scores[static_cast<size_t>(t) * n_experts + row[i]];
+      ids[static_cast<size_t>(t) * top_k + i] = row[i];
+      weights[static_cast<size_t>(t) * top_k + i] = norm_topk ? (v / denom) * scaling : v * scaling;
+    }
+  }
+}
+
 // ---- activation-quantized NVFP4 form -----------------------------------------------------------
 // src/kernels/moe_w4a4.cu:139-236: per row a global, per 16 elements an e4m3 scale, e2m1 codes. Plain fp32 operations
 // in the reference's order (this file is compiled with -ffp-contract=off).

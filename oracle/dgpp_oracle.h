@@ -176,6 +176,11 @@ void orc_mxfp8_gemm(const uint8_t* a, const uint8_t* a_scales, const uint8_t* w,
  * and an independent numpy float32 evaluation of the same recipe; the conversions are orc_f32_to_e4m3 / orc_f32_to_e2m1. */
 void orc_nvfp4_quantize_rows(const uint16_t* x, int64_t stride, int rows, int k, float static_gs, uint8_t* codes,
                              uint8_t* scales, int64_t scale_stride, float* gs);
+/* src/kernels/glm_moe.cu:917-949 (hash routing): ids[t] = row tokens[t] of tid2eid (row 0 for a token outside the
+ * vocabulary), weights = scores at those ids, / (their fp32 sum in row order + 1e-20) when norm_topk, * scaling.
+ * Pinned by an independent numpy float32 evaluation (cumulative sums in float32) and closed-form rows. */
+void orc_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float* scores, int n_tokens, int vocab,
+                     int n_experts, int top_k, float scaling, int norm_topk, int32_t* ids, float* weights);
 /* The per-token dynamic NVFP4 producer of src/kernels/minimax_native_moe.cu:36-85: scales [rows, k / 16] (dense),
  * globals[rows] = amax * (1 / 2688) (0 for a zero row). The chain of fp32 multiplications by reciprocals is restated
  * with every reciprocal correctly rounded. PARITY UNPINNED against the reference in that one respect: its reciprocal is

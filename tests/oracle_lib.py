@@ -48,6 +48,7 @@ _SIG = {
     "orc_shared_gate": (None, [_P, _L, _P, _I, _I, _P]),
     "orc_mxfp8_quantize_rows": (None, [_P, _L, _I, _I, _P, _P]),
     "orc_nvfp4_quantize_rows": (None, [_P, _L, _I, _I, C.c_float, _P, _P, _L, _P]),
+    "orc_hash_routes": (None, [_P, _P, _P, _I, _I, _I, _I, _F, _I, _P, _P]),
     "orc_minimax_quantize_rows_nvfp4": (None, [_P, _L, _I, _I, _P, _P, _P]),
     "orc_minimax_swiglu_f32": (None, [_P, _P, C.c_int64, _D, _D, _P, _P]),
     "orc_w4a4_gemm": (None, [_P, _P, _L, _P, _P, _P, C.c_double, _I, _I, _I, _P, _P]),

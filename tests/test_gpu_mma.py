@@ -235,3 +235,46 @@ def test_prefill_path_matches_oracle_and_gemv_launchers_on_the_matrix_core_are_i
         lib.dgpp_tune_set(5, 0)
     assert np.array_equal(out_slots, got), "slot kernels on the matrix core == grouped matrix-core path, bitwise"
     layer.close()
+
+
+@pytest.mark.parametrize("m,n,k,rs,cs", [(33, 96, 1024, 7, 7), (5, 130, 2048, 5, 6), (64, 64, 304, 7, 7)])
+def test_scale_gemm_tile_is_the_matrix_core_dense_form(gpu, m, n, k, rs, cs):
+    """src/kernels/scale_gemm.hpp:173-180: the tile form of the scale GEMM; bitwise launch_mma_gemv_fp8_* (unsplit)."""
+    rng = np.random.default_rng(n + k)
+    w = hg.f32_to_bf16(hg.normal_f32(0x7A0 + n + k, (n, k), 0.02))
+    act = hg.normal_bf16(0x7A1 + n, (m, k))
+    payload, _ = hg.encode_fp8_blocks(w, 128, 128)
+    br, bc = 1 << rs, 1 << cs
+    scales = rng.uniform(0.5, 2.0, ((n + br - 1) // br, (k + bc - 1) // bc)).astype(np.float32) * 1e-3
+    a_d, p_d, s_d = dev(act), dev(payload), dev(scales)
+    tb, tf, want = dev_empty((m, n), np.uint16), dev_empty((m, n), np.float32), dev_empty((m, n), np.uint16)
+    L.launch_scale_gemm_tile_bf16(a_d, k, p_d, s_d, tb, m, n, k, None, rs, cs)
+    L.launch_scale_gemm_tile_f32(a_d, k, p_d, s_d, tf, m, n, k, None, rs, cs)
+    L.launch_mma_gemv_fp8_bf16(a_d, k, p_d, s_d, want, m, n, k, 0, rs, cs, None)
+    sync()
+    got = host(tb, np.uint16)
+    assert np.array_equal(got, host(want, np.uint16))
+    assert np.array_equal(hg.f32_to_bf16(host(tf)), got)
+    check(got, orc.gemv_fp8(act, payload, scales, m, n, k, rs, cs, True), f"scale gemm tile {m}x{n}x{k}")
+
+
+def test_try_dense_fp4_decode_follows_the_shape_rule(gpu):
+    """src/kernels/dense_fp4_decode.cu:297-308: inside the rule the launch is the production form's (same bits), outside
+    it nothing is launched and the call says so."""
+    assert L.dense_fp4_decode_shape(16, 17408, 5120) and L.dense_fp4_decode_shape(1, 64, 128)
+    assert not L.dense_fp4_decode_shape(17, 64, 128) and not L.dense_fp4_decode_shape(4, 64, 192)
+    assert not L.dense_fp4_decode_shape(4, 17409, 128) and not L.dense_fp4_decode_shape(4, 64, 128, 32)
+    E, H, I, m = 2, 1024, 192, 11
+    p = moe_data.make_problem(E, H, I, 1, m, "nvfp4", 19, shared_kind=None, limit=float("inf"), std=0.05)
+    d = DeviceMoe(p)
+    seg = dev(np.array([[0, m, 1]], np.int32))
+    want, got = dev_empty((m, I), np.uint16), dev_empty((m, I), np.uint16)
+    got.fill_(0x1234)
+    L.launch_dense_mma_fp4_prod_bf16(d.x, H, seg, d.views, 1, want, m, I, H, None, 16)
+    assert L.try_dense_fp4_decode_bf16(d.x, H, seg, d.views, 1, got, m, I, H, None, 16) is True
+    sync()
+    assert np.array_equal(host(got, np.uint16), host(want, np.uint16))
+    got.fill_(0x1234)
+    assert L.try_dense_fp4_decode_bf16(d.x, H, seg, d.views, 1, got, m, I, H - 64, None, 16) is False      # k % 128
+    sync()
+    assert np.all(host(got, np.uint16) == 0x1234), "nothing was launched"

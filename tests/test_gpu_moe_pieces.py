@@ -312,3 +312,23 @@ def test_router_tiled_dots_are_bitwise_the_one_row_form(gpu, mode, E, H, T):
         for a, b, name in zip(res[0], other, ("scores", "biased", "ids", "weights")):
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), name
         assert not np.any(other[0] == -7.0), "every score of the batch is written"
+
+
+@pytest.mark.parametrize("norm", [True, False])
+@pytest.mark.parametrize("T,E,K,vocab", [(9, 40, 6, 17), (300, 256, 8, 1000), (1, 384, 16, 3)])
+def test_hash_routes_bit_exact(gpu, norm, T, E, K, vocab):
+    from test_oracle_moe import hash_route_case
+    tokens, table, scores = hash_route_case(T, E, K, vocab, T + E)
+    want_ids, want_w = np.empty((T, K), np.int32), np.empty((T, K), np.float32)
+    orc.oracle().orc_hash_routes(orc.p(tokens), orc.p(table), orc.p(scores), T, vocab, E, K, 2.5, 1 if norm else 0,
+                                 orc.p(want_ids), orc.p(want_w))
+    cfg = L.make_config(64, 64, E, K, router_mode=0, routed_scaling_factor=2.5, norm_topk_prob=norm, n_shared_experts=0)
+    ids_d, w_d = dev_empty((T, K), np.int32), dev_empty((T, K), np.float32)
+    import torch
+    L.launch_moe_hash_routes(torch.from_numpy(tokens).to("cuda:0"), dev(table), dev(scores), ids_d, w_d, cfg, vocab, T)
+    sync()
+    assert np.array_equal(host(ids_d), want_ids)
+    assert np.array_equal(host(w_d).view(np.uint32), want_w.view(np.uint32))
+    soft = L.make_config(64, 64, E, K, router_mode=1, routed_scaling_factor=1.0, n_shared_experts=0)
+    with pytest.raises(L.InvalidArgument):
+        L.launch_moe_hash_routes(torch.from_numpy(tokens).to("cuda:0"), dev(table), dev(scores), ids_d, w_d, soft, vocab, T)

@@ -156,3 +156,36 @@ def test_forward_degenerate_reduces_to_one_expert():
         act = np_ref.f32_to_bf16_f64((silu * ub).astype(np.float32))
         want = np_ref.dequant_fp4(d.payload, d.scales, 32) @ act
         assert np.allclose(raw[t], want, rtol=1e-12, atol=1e-300)
+
+
+def hash_route_case(T, E, K, vocab, seed):
+    rng = np.random.default_rng(seed)
+    table = np.stack([np.sort(rng.permutation(E)[:K]) for _ in range(vocab)]).astype(np.int32)
+    tokens = rng.integers(0, vocab, T).astype(np.int64)
+    tokens[0], tokens[-1] = -5, vocab + 3                      # padding rows read table row 0
+    scores = rng.uniform(0.01, 0.99, (T, E)).astype(np.float32)
+    return tokens, table, scores
+
+
+@pytest.mark.parametrize("norm", [1, 0])
+def test_hash_routes_oracle_against_numpy(norm):
+    """src/kernels/glm_moe.cu:917-949: the routes come from the table, the weights from the scores at those ids."""
+    T, E, K, vocab = 9, 40, 6, 17
+    tokens, table, scores = hash_route_case(T, E, K, vocab, 3)
+    ids, w = np.empty((T, K), np.int32), np.empty((T, K), np.float32)
+    orc.oracle().orc_hash_routes(orc.p(tokens), orc.p(table), orc.p(scores), T, vocab, E, K, 2.5, norm, orc.p(ids), orc.p(w))
+    rows = np.where((tokens < 0) | (tokens >= vocab), 0, tokens)
+    assert np.array_equal(ids, table[rows])
+    sel = np.take_along_axis(scores, table[rows], axis=1)
+    denom = np.zeros(T, np.float32)
+    for j in range(K):                                          # the fp32 chain, one addition at a time
+        denom = (denom + sel[:, j]).astype(np.float32)
+    denom = (denom + np.float32(1e-20)).astype(np.float32)
+    want = ((sel / denom[:, None]).astype(np.float32) * np.float32(2.5)).astype(np.float32) if norm else (sel * np.float32(2.5)).astype(np.float32)
+    assert np.array_equal(w.view(np.uint32), want.view(np.uint32))
+    if norm:
+        assert np.allclose(w.sum(axis=1), 2.5, rtol=1e-6)
+    # all-equal scores: every weight is 1 / K * scaling
+    flat = np.full((T, E), 0.5, np.float32)
+    orc.oracle().orc_hash_routes(orc.p(tokens), orc.p(table), orc.p(flat), T, vocab, E, K, 2.5, 1, orc.p(ids), orc.p(w))
+    assert np.allclose(w, 2.5 / K, rtol=1e-6)
