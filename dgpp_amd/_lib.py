@@ -74,6 +74,8 @@ SIGNATURES = {
     "dgpp_try_dense_fp4_decode_bf16": (_I, [_P, _Z, _P, _P, _I, _P, _I, _I, _I, _P, _I, _P]),
     "dgpp_launch_scale_gemm_tile_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_launch_scale_gemm_tile_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
+    "dgpp_launch_moe_slot_gate_up_swiglu_mixed": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _I, _I,
+                                                        _P, _I, _I]),
     "dgpp_launch_moe_hash_routes": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P]),
     "dgpp_launch_moe_router_dots": (_I, [_P, _P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P]),

@@ -21,6 +21,7 @@ LIB = LIB_DIR / "libdgpp_amd.so"
 HIP_SOURCES = [
     "gemv_mxfp4.hip",
     "gemv_nvfp4.hip",
+    "gemv_mixed.hip",
     "gemv_fp8f32.hip",
     "gemv_fp8e8m0.hip",
     "moe_router.hip",

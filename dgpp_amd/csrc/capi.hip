@@ -792,6 +792,40 @@ int dgpp_launch_moe_slot_gate_up_swiglu_fp4_ex(const uint16_t* x, size_t x_strid
   return finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who);
 }
 
+int dgpp_launch_moe_slot_gate_up_swiglu_mixed(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                                              const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                              int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                              const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                              int act_stride, int slots, int top_k, float limit, int gate_fp4, int fp4_group,
+                                              void* stream, int sh_rs, int sh_cs) {
+  const char* who = "moe_slot_gate_up_mixed";
+  if (slots <= 0) return DGPP_OK;
+  if (fp4_group != 16)
+    return fail_arg(std::string(who) + ": the per-projection form mixes fp8 with NVFP4 (group 16)");
+  int rc = check_fp4_slot(x, ids, views, act, n_routed, k_routed, n_shared, k_shared, -1, fp4_group, who);
+  if (rc != DGPP_OK) return rc;
+  if (k_routed % 16 != 0) return fail_arg(std::string(who) + ": k must be a multiple of 16 (the fp8 core)");
+  if (n_shared > 0 && (!sh_gate_payload || !sh_gate_scales || !sh_up_payload || !sh_up_scales ||
+                       !fp8_shape_ok(sh_gate_payload, k_shared) || !fp8_shape_ok(sh_up_payload, k_shared)))
+    return fail_arg(std::string(who) + ": shared payloads must be 16B-aligned with k % 16 == 0");
+  if (act_stride < n_routed || act_stride < n_shared) return fail_arg(std::string(who) + ": act_stride below n");
+  if (stage_bytes(2, k_routed) + 4096 > kMaxLdsBytes) return fail_arg(std::string(who) + ": k beyond what the two stages hold");
+  SlotArgs a = slot_args(x, x_stride, ids, order, views, act, act_stride, slots, top_k, limit);
+  a.n = n_routed;
+  a.k = k_routed;
+  a.want_shared = 0;
+  a.match = 0;   // one slot per block
+  rc = finish(launch_slot_gate_up_mixed(a, gate_fp4, as_stream(stream)), who);
+  if (rc != DGPP_OK || n_shared == 0) return rc;
+  a = slot_args(x, x_stride, ids, order, views, act, act_stride, slots, top_k, limit);
+  a.n = n_shared;   // the shared slots run the fp8 core on both projections, as the fp4 launcher's do
+  a.k = k_shared;
+  a.want_shared = 1;
+  a.sh[0] = fp8_mat(sh_gate_payload, sh_gate_scales, sh_rs, sh_cs);
+  a.sh[1] = fp8_mat(sh_up_payload, sh_up_scales, sh_rs, sh_cs);
+  return finish(launch_slot_gate_up(kFmtFp8F32, a, as_stream(stream)), who);
+}
+
 int dgpp_launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
                                   const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
                                   int k_shared, const uint8_t* sh_payload, const float* sh_scales, float* out,

@@ -357,6 +357,62 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_
   slot_gate_up_body<FMT, NB, MAXM, SPLIT, NT>(a, g, steps, lds);
 }
 
+// ---- gate / up in different formats (the per-projection form) -------------------------------------------------------
+// One projection of every routed expert is block-FP8 (its table entry's payload / scales / shifts), the other NVFP4
+// (payload / fp4_scales / fp4_global); GATE_FP4 says which (reference: src/kernels/glm_moe.cu:4882-4922). A block takes
+// a tile of rows of ONE slot: the token's row is staged twice, in each core's LDS order; the wavefronts walk the
+// tile's rows of the FP8 matrix with the FP8 core, then of the FP4 matrix with the FP4 core (each with its own row
+// geometry: row_dots, the uniform kernels' chain per row, bit for bit), park the finished dots in LDS, and the SwiGLU
+// runs on the pairs with the uniform kernels' rounding points.
+template <int NB8, int NB4, bool GATE_FP4>
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_mixed_kernel(SlotArgs a, RowGeom g8, RowGeom g4,
+                                                                                            int rows_per_block) {
+  extern __shared__ uint4 lds[];
+  SlotRun<1> run;
+  if (!resolve_run<1>(a, run)) return;
+  const int tile_row0 = static_cast<int>(blockIdx.x) * rows_per_block;
+  if (tile_row0 >= a.n) return;
+  const DgppMoeExpertView& v8 = a.views[run.view_base + (GATE_FP4 ? 1 : 0)];
+  const DgppMoeExpertView& v4 = a.views[run.view_base + (GATE_FP4 ? 0 : 1)];
+  const float *unused = nullptr, *global4 = nullptr;
+  const MatRef m8 = mat_of_view<kFmtFp8F32>(v8, &unused);
+  const MatRef m4 = mat_of_view<kFmtNvfp4>(v4, &global4);
+  const int row_vecs = a.k / 8;
+  uint4* x8 = lds;
+  uint4* x4 = lds + row_vecs;
+  float* d8 = reinterpret_cast<float*>(lds + 2 * row_vecs);   // [rows_per_block] each
+  float* d4 = d8 + rows_per_block;
+  const uint16_t* x = a.x + static_cast<size_t>(run.token[0]) * a.x_stride;
+  stage_activations<kFmtFp8F32>(x, a.x_stride, 1, a.k, x8);
+  stage_activations<kFmtNvfp4>(x, a.x_stride, 1, a.k, x4);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6;
+  const int tile_end = min(a.n, tile_row0 + rows_per_block);
+  {
+    const int rpw = kWave >> g8.l2, chunks = a.k / FmtTraits<kFmtFp8F32>::kElemsPerChunk;
+    for (int row0 = tile_row0 + wave * rpw; row0 < tile_end; row0 += kWavesPerBlock * rpw) {
+      const auto lr = lane_row<kFmtFp8F32, false>(m8, row0, a.n, a.k, g8.l2);
+      float acc[1];
+      row_dots<kFmtFp8F32, 1, NB8>(lr, g8, m8.cs, x8, chunks, 1, acc);
+      if (lr.li == 0 && lr.row < tile_end) d8[lr.row - tile_row0] = finish_dot<kFmtFp8F32>(acc[0], 1.0f);
+    }
+  }
+  {
+    const float divisor = load_divisor<kFmtNvfp4>(global4);
+    const int rpw = kWave >> g4.l2, chunks = a.k / FmtTraits<kFmtNvfp4>::kElemsPerChunk;
+    for (int row0 = tile_row0 + wave * rpw; row0 < tile_end; row0 += kWavesPerBlock * rpw) {
+      const auto lr = lane_row<kFmtNvfp4, false>(m4, row0, a.n, a.k, g4.l2);
+      float acc[1];
+      row_dots<kFmtNvfp4, 1, NB4>(lr, g4, m4.cs, x4, chunks, 1, acc);
+      if (lr.li == 0 && lr.row < tile_end) d4[lr.row - tile_row0] = finish_dot<kFmtNvfp4>(acc[0], divisor);
+    }
+  }
+  __syncthreads();
+  uint16_t* act = static_cast<uint16_t*>(a.out) + static_cast<size_t>(run.slot[0]) * a.out_stride;
+  for (int r = threadIdx.x; tile_row0 + r < tile_end; r += kBlockThreads)
+    act[tile_row0 + r] = GATE_FP4 ? swiglu_bf16(d4[r], d8[r], a.limit) : swiglu_bf16(d8[r], d4[r], a.limit);
+}
+
 // The router's selection and the routed gate/up pass of a ONE-token decode step in one launch: the first
 // wavefront of every block repeats the selection (whole score row in registers: the selection kernel's own
 // code), the ids go to LDS behind the activation stage and the block goes on as slot_gate_up_kernel does.
@@ -651,6 +707,9 @@ hipError_t launch_select_gate_up(int fmt, const SlotArgs& a, const SelectArgs& s
 hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t stream);
 hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
 
+// Routed gate/up + SwiGLU with the two projections in different formats (one block-FP8, one NVFP4).
+hipError_t launch_slot_gate_up_mixed(const SlotArgs& a, int gate_fp4, hipStream_t stream);
+
 // Token-major routed down + accumulation (vector core).
 hipError_t launch_token_down(int fmt, const TokenDownArgs& a, hipStream_t stream);
 template <int FMT> hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipStream_t stream);
@@ -892,6 +951,40 @@ hipError_t launch_slot_gate_up_fmt(const SlotArgs& a, hipStream_t stream) {
   });
   return err != hipSuccess ? err : hipGetLastError();
 }
+
+// The mixed-format gate/up launch (routed slots only; one slot per block - the form is rare enough to go without runs).
+#ifdef DGPP_GEMV_MIXED
+hipError_t launch_slot_gate_up_mixed(const SlotArgs& a, int gate_fp4, hipStream_t stream) {
+  const RowGeom g8 = geom_for<kFmtFp8F32>(a.k), g4 = geom_for<kFmtNvfp4>(a.k);
+  const int step8 = kWavesPerBlock * (kWave >> g8.l2), step4 = kWavesPerBlock * (kWave >> g4.l2);
+  const int unit = step8 > step4 ? step8 : step4;   // both are powers of two: the larger is a multiple of the smaller
+  const long long per_slot = (a.n + unit - 1) / unit;
+  const int steps = pick_steps(per_slot * a.slots);
+  const int rows_per_block = unit * steps;
+  const dim3 grid(static_cast<unsigned>((a.n + rows_per_block - 1) / rows_per_block), static_cast<unsigned>(a.slots));
+  const size_t lds = 2 * stage_bytes(1, a.k) + 2 * static_cast<size_t>(rows_per_block) * sizeof(float);
+  hipError_t err = hipSuccess;
+  // Loads in flight per lane and row: the largest of 4, 2, 1 that divides the lane's chunk count (the chain per row
+  // does not depend on it; the full set of pass widths would square the number of kernels of this rare form).
+  auto pass_width = [](const RowGeom& g) { return g.P % 4 == 0 ? 4 : (g.P % 2 == 0 ? 2 : 1); };
+  dispatch_nb(pass_width(g8), [&](auto n8) {
+    dispatch_nb(pass_width(g4), [&](auto n4) {
+      dispatch_bool(gate_fp4 != 0, [&](auto gf) {
+        constexpr int N8 = decltype(n8)::value, N4 = decltype(n4)::value;
+        if constexpr (N8 > 4 || N8 == 3 || N4 > 4 || N4 == 3) {
+          err = hipErrorInvalidValue;   // never taken: pass_width returns 4, 2 or 1
+          return;
+        } else {
+        auto kern = slot_gate_up_mixed_kernel<N8, N4, decltype(gf)::value>;
+        err = ensure_lds(kern, lds);
+        if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g8, g4, rows_per_block);
+        }
+      });
+    });
+  });
+  return err != hipSuccess ? err : hipGetLastError();
+}
+#endif
 
 // The fused selection + gate/up launch; the caller has checked its limits (capi.hip, select_gate_up_fits).
 template <int FMT>

@@ -238,6 +238,15 @@ def launch_moe_slot_down_fp4(act, act_stride, ids, order, views, n_routed, k_rou
         _p(tile_counter)))
 
 
+def launch_moe_slot_gate_up_swiglu_mixed(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared, sh_gate_payload,
+                                         sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride, slots, top_k, limit,
+                                         gate_fp4, fp4_group=16, stream=None, sh_rs=7, sh_cs=7):
+    _check(_lib.load().dgpp_launch_moe_slot_gate_up_swiglu_mixed(
+        _p(x), x_stride, _p(ids), _p(order), _p(views), n_routed, k_routed, n_shared, k_shared, _p(sh_gate_payload),
+        _p(sh_gate_scales), _p(sh_up_payload), _p(sh_up_scales), _p(act), act_stride, slots, top_k, limit,
+        1 if gate_fp4 else 0, fp4_group, _stream(stream), sh_rs, sh_cs))
+
+
 def launch_moe_slot_gate_up_swiglu_ex(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
                                       sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act, act_stride,
                                       slots, top_k, limit, stream=None, sh_rs=7, sh_cs=7, passes=3):

@@ -281,6 +281,18 @@ int dgpp_launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_stride, 
                                             uint16_t* act, int act_stride, int slots, int top_k,
                                             float limit, void* stream, int shared_view_base,
                                             int fp4_group, int sh_rs, int sh_cs);
+/* src/kernels/glm_moe_launch.hpp:409-425 (launch_moe_slot_gate_up_swiglu_mixed): the per-projection form's gate/up
+ * launch - one projection of every routed expert block-FP8 (its entry's payload / scales / scale shifts), the other
+ * NVFP4 (payload / fp4_scales / fp4_global), gate_fp4 != 0 naming the gate as the NVFP4 one. Each dot is bitwise its
+ * uniform launcher's; the SwiGLU has the same rounding points. fp4_group must be 16; k in the FP4 core's accepted
+ * set and a multiple of 16. The shared slots (n_shared > 0: an FP8 expert on the launch arguments) run as the FP4
+ * launcher's do. */
+int dgpp_launch_moe_slot_gate_up_swiglu_mixed(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                                              const DgppMoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                              int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                              const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                              int act_stride, int slots, int top_k, float limit, int gate_fp4, int fp4_group,
+                                              void* stream, int sh_rs, int sh_cs);
 /* src/kernels/glm_moe_launch.hpp:400-408. tile_counter (two device ints zeroed once by the
  * caller) is accepted for signature parity and left untouched: this build's down kernel uses a
  * static grid. */

@@ -253,6 +253,17 @@ inline void launch_moe_slot_gate_up_swiglu_fp4(const uint16_t* x, size_t x_strid
                                                         sh_up_scales, act, act_stride, slots, top_k, limit, stream,
                                                         shared_view_base, fp4_group, sh_rs, sh_cs));
 }
+inline void launch_moe_slot_gate_up_swiglu_mixed(const uint16_t* x, size_t x_stride, const int32_t* ids, const int32_t* order,
+                                                 const MoeExpertView* views, int n_routed, int k_routed, int n_shared,
+                                                 int k_shared, const uint8_t* sh_gate_payload, const float* sh_gate_scales,
+                                                 const uint8_t* sh_up_payload, const float* sh_up_scales, uint16_t* act,
+                                                 int act_stride, int slots, int top_k, float limit, bool gate_fp4,
+                                                 int fp4_group, hipStream_t stream, int sh_rs = 7, int sh_cs = 7) {
+  detail::check(dgpp_launch_moe_slot_gate_up_swiglu_mixed(x, x_stride, ids, order, views, n_routed, k_routed, n_shared, k_shared,
+                                                          sh_gate_payload, sh_gate_scales, sh_up_payload, sh_up_scales, act,
+                                                          act_stride, slots, top_k, limit, gate_fp4 ? 1 : 0, fp4_group, stream,
+                                                          sh_rs, sh_cs));
+}
 inline void launch_moe_slot_down_fp4(const uint16_t* act, size_t act_stride, const int32_t* ids, const int32_t* order,
                                      const MoeExpertView* views, int n_routed, int k_routed, int n_shared,
                                      int k_shared, const uint8_t* sh_payload, const float* sh_scales, float* out,

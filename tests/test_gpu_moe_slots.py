@@ -383,3 +383,81 @@ def test_fp8_slot_kernels_stage_a_row_wider_than_the_default_lds_ceiling(gpu):
     act, down, out = run_slot_path(p, d, ids, w)
     raw, _ = moe_data.orc_forward(p, ids, w)
     expert_budget(out, raw, "k = 40960 FP8 slots")
+
+
+@pytest.mark.parametrize("gate_fp4", [True, False])
+@pytest.mark.parametrize("H,I,T,K,use_order,shared", [(1024, 160, 3, 2, False, False), (2048, 264, 4, 3, True, True),
+                                                      (512, 96, 1, 4, False, True)])
+def test_mixed_format_gate_up_is_bitwise_the_uniform_cores(gpu, gate_fp4, H, I, T, K, use_order, shared):
+    """src/kernels/glm_moe_launch.hpp:409-425: one projection block-FP8, the other NVFP4; every dot bitwise its uniform
+    launcher's (here: the dense GEMV launchers, the slot kernels' twins), the SwiGLU with the same rounding points; the
+    shared slots run the FP8 core on both projections."""
+    from gpu_util import fp4_matrix, fp4_view, fp8_view, view_table
+    E, limit = 5, 7.0
+    rng = np.random.default_rng(H + I)
+    x = hg.normal_bf16(0xAA0 + H, (T, H))
+    ids = np.stack([np.sort(rng.permutation(E)[:K]) for _ in range(T)]).astype(np.int32)
+    keep, entries, mats = [], [], []
+    for e in range(E):
+        g = moe_data.make_mat("nvfp4" if gate_fp4 else "fp8", I, H, 0xAB0 + 3 * e, 0.05)
+        u = moe_data.make_mat("fp8" if gate_fp4 else "nvfp4", I, H, 0xAB1 + 3 * e, 0.05)
+        mats.append((g, u))
+        for m in (g, u, g):                       # the third entry (down) is not read by this launch
+            pd, sd = dev(m.payload), dev(m.scales)
+            keep += [pd, sd]
+            if m.kind == "fp8":
+                entries.append(fp8_view(pd, sd, m.rs, m.cs))
+            else:
+                gd = dev(m.glob)
+                keep.append(gd)
+                entries.append(fp4_view(pd, sd, gd, 16))
+    views = view_table(entries)
+    SI = 128
+    sh = [moe_data.make_mat("fp8", SI, H, 0xAC0 + j, 0.05) for j in range(2)] if shared else None
+    sh_d = [(dev(m.payload), dev(m.scales)) for m in sh] if shared else [(None, None)] * 2
+    slots = T * (K + 1)
+    x_d, ids_d = dev(x), dev(ids)
+    order = None
+    if use_order:
+        order = dev_empty(slots, np.int32)
+        L.launch_moe_slot_order(ids_d, order, slots, K, E, None, 0)
+    width = max(I, SI)
+    act = dev_empty((slots, width), np.uint16)
+    act.fill_(0x7FC0)
+    L.launch_moe_slot_gate_up_swiglu_mixed(x_d, H, ids_d, order, views, I, H, SI if shared else 0, H if shared else 0,
+                                           sh_d[0][0], sh_d[0][1], sh_d[1][0], sh_d[1][1], act, width, slots, K, limit,
+                                           gate_fp4, 16)
+    sync()
+    got = host(act, np.uint16)
+
+    def dense(m, rows):
+        out = dev_empty((T, rows), np.uint16)
+        if m.kind == "fp8":
+            L.launch_scale_gemm_bf16(x_d, H, dev(m.payload), dev(m.scales), out, T, rows, H, None)
+        else:
+            L.launch_fp4_gemv_bf16(x_d, H, fp4_matrix(dev(m.payload), dev(m.scales), dev(m.glob), rows, H, 16), out, T, rows, H, None)
+        return out
+
+    for e in range(E):
+        gd_, ud_ = dense(mats[e][0], I), dense(mats[e][1], I)
+        want = dev_empty((T, I), np.uint16)
+        L.launch_moe_swiglu_clamp(gd_, ud_, want, T * I, limit, None)
+        sync()
+        w = host(want, np.uint16)
+        for t in range(T):
+            for j in range(K):
+                if ids[t, j] == e:
+                    assert np.array_equal(got[t * (K + 1) + j, :I], w[t]), f"expert {e} token {t}"
+    if shared:
+        gd_, ud_ = dense(sh[0], SI), dense(sh[1], SI)
+        want = dev_empty((T, SI), np.uint16)
+        L.launch_moe_swiglu_clamp(gd_, ud_, want, T * SI, limit, None)
+        sync()
+        w = host(want, np.uint16)
+        for t in range(T):
+            assert np.array_equal(got[t * (K + 1) + K, :SI], w[t]), f"shared slot of token {t}"
+    else:
+        assert np.all(got[K::K + 1] == 0x7FC0), "without a shared expert its slots are left alone"
+    with pytest.raises(L.InvalidArgument):
+        L.launch_moe_slot_gate_up_swiglu_mixed(x_d, H, ids_d, order, views, I, H, 0, 0, None, None, None, None, act, width,
+                                               slots, K, limit, gate_fp4, 32)
