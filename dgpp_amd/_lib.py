@@ -76,6 +76,9 @@ SIGNATURES = {
     "dgpp_launch_scale_gemm_tile_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _I, _I]),
     "dgpp_launch_moe_slot_gate_up_swiglu_mixed": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _F, _I, _I,
                                                         _P, _I, _I]),
+    "dgpp_mma_gemv_shape_ok": (_I, [_P, _P, _Z, _I, _I]),
+    "dgpp_mma_gemv_pair_ok": (_I, [_P, _P, _P, _P, _Z, _I, _I, _I, _I, _P, _Z]),
+    "dgpp_launch_mma_gemv_fp8_bf16_pair": (_I, [_P, _P, _P, _P, _I, _Z, _P, _P, _P, _P, _I, _Z, _Z, _I, _I, _I, _I, _P, _P, _Z]),
     "dgpp_launch_moe_hash_routes": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _P]),
     "dgpp_launch_moe_router_dots": (_I, [_P, _P, _P, _P, _P, _P, _I, _P]),
     "dgpp_launch_moe_select_gate_up_swiglu": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P]),

@@ -956,6 +956,65 @@ static int dense_mma_fp8(const uint16_t* act, size_t act_stride, const uint8_t* 
   return dense_mma(e8m0 ? kFmtFp8E8M0 : kFmtFp8F32, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, out,
                    out_f32, out_stride, m, n, k, ws, ws_bytes, stream, who, act_up, limit);
 }
+/* src/kernels/mma_gemv.cu:895-899: the shape the matrix-core GEMV takes. */
+int dgpp_mma_gemv_shape_ok(const void* w, const void* act, size_t act_stride, int m, int k) {
+  return m >= 1 && k > 0 && (k % 64) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 &&
+         (reinterpret_cast<uintptr_t>(act) & 15u) == 0 && ((act_stride * 2) % 16) == 0;
+}
+/* src/kernels/mma_gemv.cu:921-933: whether two projections may share one launch - a decode batch (at most 32 rows), both
+ * shapes taken, and a workspace that holds both problems' K-part sums (parts(k) * m * (n0 + n1) floats here). */
+int dgpp_mma_gemv_pair_ok(const void* w0, const void* w1, const uint16_t* a0, const uint16_t* a1, size_t act_stride, int m,
+                          int n0, int n1, int k, void* ws, size_t ws_bytes) {
+  if (!ws || m < 1 || m > 32 || n0 <= 0 || n1 <= 0) return 0;
+  if (!dgpp_mma_gemv_shape_ok(w0, a0, act_stride, m, k) || !dgpp_mma_gemv_shape_ok(w1, a1, act_stride, m, k)) return 0;
+  const size_t need = static_cast<size_t>(mgeom<kFmtFp8F32>(k).parts) * m * (static_cast<size_t>(n0) + n1) * sizeof(float);
+  return need <= ws_bytes;
+}
+/* src/kernels/mma_gemv.cu:935-961: two FP8 projections of one k and one batch in ONE launch; every row's chain is its
+ * single launch's (bitwise dgpp_launch_mma_gemv_fp8_bf16 on each). */
+int dgpp_launch_mma_gemv_fp8_bf16_pair(const uint16_t* a0, const uint8_t* w0, const float* s0, uint16_t* o0, int n0,
+                                       size_t stride0, const uint16_t* a1, const uint8_t* w1, const float* s1, uint16_t* o1,
+                                       int n1, size_t stride1, size_t act_stride, int m, int k, int rs, int cs, void* stream,
+                                       void* ws, size_t ws_bytes) {
+  const char* who = "mma_gemv_fp8_pair";
+  if (m <= 0 || (n0 <= 0 && n1 <= 0)) return DGPP_OK;
+  if (n0 <= 0)
+    return dgpp_launch_mma_gemv_fp8_bf16(a1, act_stride, w1, s1, o1, m, n1, k, stride1, rs, cs, stream, ws, ws_bytes);
+  if (n1 <= 0)
+    return dgpp_launch_mma_gemv_fp8_bf16(a0, act_stride, w0, s0, o0, m, n0, k, stride0, rs, cs, stream, ws, ws_bytes);
+  if (!a0 || !a1 || !w0 || !w1 || !s0 || !s1 || !o0 || !o1) return fail_arg(std::string(who) + ": null pointer");
+  const bool row_grid = rs == 0 && cs >= 4;
+  if (!row_grid && (rs < 4 || rs > 7 || cs < 4 || cs > 7))
+    return fail_arg(std::string(who) + ": rs / cs must be 4..7 or a row grid (rs = 0, cs >= 4)");
+  if (k <= 0 || !fp8_shape_ok(w0, k) || !fp8_shape_ok(w1, k))
+    return fail_arg(std::string(who) + ": k must be a positive multiple of 16 with 16-byte aligned payloads");
+  if (stride0 == 0) stride0 = static_cast<size_t>(n0);
+  if (stride1 == 0) stride1 = static_cast<size_t>(n1);
+  if (stride0 < static_cast<size_t>(n0) || stride1 < static_cast<size_t>(n1))
+    return fail_arg(std::string(who) + ": output row stride narrower than n");
+  if ((m + kTileCols - 1) / kTileCols > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
+  DenseArgs p[2];
+  const uint16_t* acts[2] = {a0, a1};
+  const uint8_t* ws_[2] = {w0, w1};
+  const float* ss[2] = {s0, s1};
+  uint16_t* outs[2] = {o0, o1};
+  const int ns[2] = {n0, n1};
+  const size_t strides[2] = {stride0, stride1};
+  for (int i = 0; i < 2; ++i) {
+    p[i].act = acts[i];
+    p[i].act_stride = act_stride;
+    p[i].mat = fp8_mat(ws_[i], ss[i], rs, cs);
+    p[i].global = nullptr;
+    p[i].out = outs[i];
+    p[i].out_stride = strides[i];
+    p[i].out_f32 = 0;
+    p[i].m = m;
+    p[i].n = ns[i];
+    p[i].k = k;
+    p[i].once = m <= kTileCols;
+  }
+  return finish(launch_dense_mma_pair_fp8(p[0], p[1], static_cast<float*>(ws), ws_bytes, as_stream(stream)), who);
+}
 int dgpp_launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t* up, float limit, size_t act_stride,
                                         const uint8_t* w, const float* scales, float* out, int m, int n, int k,
                                         size_t out_stride, int rs, int cs, void* stream) {

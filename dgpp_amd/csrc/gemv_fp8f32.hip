@@ -1,5 +1,6 @@
 // Instantiates the GEMV-core kernels for one weight format (kFmtFp8F32).
 #define DGPP_GEMV_IMPL
+#define DGPP_GEMV_PAIR
 #include "gemv_kernels.hpp"
 
 namespace dgpp_amd {

@@ -716,6 +716,8 @@ template <int FMT> hipError_t launch_token_down_fmt(const TokenDownArgs& a, hipS
 
 // The matrix-core launchers proper (the *_mma_* entry points).
 hipError_t launch_dense_mma(int fmt, const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t stream);
+// Two FP8 (F32 grid) problems of one k and m in one launch; ws as in launch_dense_mma (both problems' partials).
+hipError_t launch_dense_mma_pair_fp8(const DenseArgs& a0, const DenseArgs& a1, float* ws, size_t ws_bytes, hipStream_t stream);
 hipError_t launch_grouped_mma(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
 template <int FMT> hipError_t launch_dense_mma_fmt(const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t stream);
 template <int FMT> hipError_t launch_grouped_mma_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
@@ -787,6 +789,38 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
   }
   return hipGetLastError();
 }
+
+#ifdef DGPP_GEMV_PAIR
+hipError_t launch_dense_mma_pair_fp8(const DenseArgs& a0, const DenseArgs& a1, float* ws, size_t ws_bytes, hipStream_t stream) {
+  constexpr int FMT = kFmtFp8F32;
+  const MGeom g = mgeom<FMT>(a0.k);
+  const unsigned t0 = static_cast<unsigned>((a0.n + 63) / 64), t1 = static_cast<unsigned>((a1.n + 63) / 64);
+  const unsigned gy = static_cast<unsigned>((a0.m + kTileCols - 1) / kTileCols);
+  const size_t need = static_cast<size_t>(g.parts) * a0.m * (static_cast<size_t>(a0.n) + a1.n) * sizeof(float);
+  const bool split = ws != nullptr && g.parts > 1 && ws_bytes >= need && static_cast<size_t>(t0 + t1) * gy < 1024;
+  const dim3 grid(t0 + t1, gy, split ? g.parts : 1);
+  hipError_t err = hipSuccess;
+  dispatch_bool(a0.once != 0, [&](auto ntc) {
+    auto kern = mfma_dense_pair_kernel<FMT, kMfmaNB, decltype(ntc)::value>;
+    constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
+    err = ensure_lds(kern, lds);
+    if (err == hipSuccess)
+      hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a0, a1, static_cast<int>(t0), g, split ? ws : nullptr);
+  });
+  if (err != hipSuccess) return err;
+  if (split) {
+    const DenseArgs* both[2] = {&a0, &a1};
+    float* at = ws;
+    for (const DenseArgs* a : both) {
+      const int64_t total = static_cast<int64_t>(a->m) * a->n;
+      hipLaunchKernelGGL(fold_parts_kernel<FMT>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, stream, at,
+                         g.parts, a->m, a->n, a->global, a->out, a->out_f32, a->out_stride);
+      at += static_cast<size_t>(g.parts) * a->m * a->n;
+    }
+  }
+  return hipGetLastError();
+}
+#endif
 
 template <int FMT>
 hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream) {

@@ -198,6 +198,37 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs 
   store_tile<kFmtMxfp4>(sum, 1.0f, partials, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
 }
 
+// Two dense problems of the same k and m in ONE launch (reference: launch_mma_gemv_fp8_bf16_pair,
+// src/kernels/mma_gemv.cu:935-961 - two dependent-free projections sharing one ramp and drain): the first tiles0 row
+// tiles of the grid belong to problem 0, the rest to problem 1; each block then does what mfma_dense_kernel does for
+// its problem, so every row's chain is its single launch's. Split form: partials of problem 1 follow problem 0's.
+template <int FMT, int NB, bool NT>
+__global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_pair_kernel(DenseArgs a0, DenseArgs a1, int tiles0, MGeom g,
+                                                                           float* partials) {
+  extern __shared__ uint4 lds[];
+  const bool second = static_cast<int>(blockIdx.x) >= tiles0;
+  const DenseArgs& a = second ? a1 : a0;
+  const int bx = static_cast<int>(blockIdx.x) - (second ? tiles0 : 0);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int row0 = (bx * kWavesPerBlock + wave) * kGroupRows;
+  const int c0 = static_cast<int>(blockIdx.y) * kTileCols;
+  const int mt = min(kTileCols, a.m - c0);
+  const int c = lane & 15;
+  f32x4_t sum;
+  if (partials == nullptr) {
+    block_rows_mfma<FMT, NB, NT>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k, row0,
+                                 g, 0, g.parts, lds, sum);
+    store_tile<FMT>(sum, load_divisor<FMT>(a.global), a.out, a.out_f32, static_cast<size_t>(c0 + c) * a.out_stride, row0, a.n,
+                    c < mt);
+    return;
+  }
+  const int part = static_cast<int>(blockIdx.z);
+  block_rows_mfma<FMT, NB, NT>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, nullptr, mt, a.n, a.k, row0, g,
+                               part, part + 1, lds, sum);
+  float* mine = partials + (second ? static_cast<size_t>(g.parts) * a0.m * a0.n : 0);
+  store_tile<kFmtMxfp4>(sum, 1.0f, mine, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
+}
+
 // out[r][j] = finish(((p0 + p1) + p2) + p3) over partials[part][r][j].
 template <int FMT>
 __global__ void fold_parts_kernel(const float* __restrict__ partials, int parts, int m, int n, const float* global,

@@ -469,6 +469,21 @@ def launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per
                                                        _p(act_rows)))
 
 
+def mma_gemv_shape_ok(w, act, act_stride, m, k) -> bool:
+    return bool(_lib.load().dgpp_mma_gemv_shape_ok(_p(w), _p(act), act_stride, m, k))
+
+
+def mma_gemv_pair_ok(w0, w1, a0, a1, act_stride, m, n0, n1, k, ws, ws_bytes) -> bool:
+    return bool(_lib.load().dgpp_mma_gemv_pair_ok(_p(w0), _p(w1), _p(a0), _p(a1), act_stride, m, n0, n1, k, _p(ws), ws_bytes))
+
+
+def launch_mma_gemv_fp8_bf16_pair(a0, w0, s0, o0, n0, stride0, a1, w1, s1, o1, n1, stride1, act_stride, m, k, rs=7, cs=7,
+                                  stream=None, ws=None, ws_bytes=0):
+    _check(_lib.load().dgpp_launch_mma_gemv_fp8_bf16_pair(_p(a0), _p(w0), _p(s0), _p(o0), n0, stride0, _p(a1), _p(w1), _p(s1),
+                                                          _p(o1), n1, stride1, act_stride, m, k, rs, cs, _stream(stream), _p(ws),
+                                                          ws_bytes))
+
+
 def launch_mma_gemv_fp8_swiglu_f32(gate, up, limit, act_stride, w, scales, out, m, n, k, out_stride=0, rs=7, cs=7,
                                    stream=None):
     _check(_lib.load().dgpp_launch_mma_gemv_fp8_swiglu_f32(_p(gate), _p(up), limit, act_stride, _p(w), _p(scales), _p(out),

@@ -394,6 +394,18 @@ int dgpp_launch_moe_grouped_mma_bf16(const uint16_t* act, size_t act_stride, con
 int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, const DgppMoeSegment* segs, int n_segs,
                                     int max_rows, int rows_per_block, const DgppMoeExpertView* views, int which, float* out,
                                     size_t out_stride, int n, int k, void* stream, const int32_t* act_rows);
+/* src/kernels/mma_gemv.hpp:103-104, :119-130 (mma_gemv_shape_ok, mma_gemv_pair_ok, launch_mma_gemv_fp8_bf16_pair): two
+ * FP8 projections of one k against one batch in ONE launch - two dependent-free GEMVs sharing one ramp and drain.
+ * Each row's bits are those of dgpp_launch_mma_gemv_fp8_bf16 on its own problem. act_stride is both activations';
+ * ws (nullable here) holds both problems' K-part sums: parts(k) * m * (n0 + n1) floats. pair_ok mirrors the reference's
+ * conditions that carry over (a workspace, 1 <= m <= 32, both shapes taken, the workspace large enough). */
+int dgpp_mma_gemv_shape_ok(const void* w, const void* act, size_t act_stride, int m, int k);
+int dgpp_mma_gemv_pair_ok(const void* w0, const void* w1, const uint16_t* a0, const uint16_t* a1, size_t act_stride, int m,
+                          int n0, int n1, int k, void* ws, size_t ws_bytes);
+int dgpp_launch_mma_gemv_fp8_bf16_pair(const uint16_t* a0, const uint8_t* w0, const float* s0, uint16_t* o0, int n0,
+                                       size_t stride0, const uint16_t* a1, const uint8_t* w1, const float* s1, uint16_t* o1,
+                                       int n1, size_t stride1, size_t act_stride, int m, int k, int rs, int cs, void* stream,
+                                       void* ws, size_t ws_bytes);
 /* src/kernels/mma_gemv.hpp:86-95 (launch_mma_gemv_fp8_swiglu_f32): out = swiglu(gate, up) x W^T with the activation
  * computed as the rows are staged; bitwise dgpp_launch_moe_swiglu_clamp followed by dgpp_launch_mma_gemv_fp8_f32
  * (unsplit). gate / up: bf16 [m, act_stride], 16-byte aligned rows. */

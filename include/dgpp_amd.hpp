@@ -438,6 +438,20 @@ inline void launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, c
   detail::check(dgpp_launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                                 out_stride, n, k, stream, act_rows));
 }
+inline bool mma_gemv_shape_ok(const void* w, const void* act, size_t act_stride, int m, int k) {
+  return dgpp_mma_gemv_shape_ok(w, act, act_stride, m, k) != 0;
+}
+inline bool mma_gemv_pair_ok(const void* w0, const void* w1, const uint16_t* a0, const uint16_t* a1, size_t act_stride, int m,
+                             int n0, int n1, int k, void* ws, size_t ws_bytes) {
+  return dgpp_mma_gemv_pair_ok(w0, w1, a0, a1, act_stride, m, n0, n1, k, ws, ws_bytes) != 0;
+}
+inline void launch_mma_gemv_fp8_bf16_pair(const uint16_t* a0, const uint8_t* w0, const float* s0, uint16_t* o0, int n0,
+                                          size_t stride0, const uint16_t* a1, const uint8_t* w1, const float* s1, uint16_t* o1,
+                                          int n1, size_t stride1, size_t act_stride, int m, int k, int rs, int cs,
+                                          hipStream_t stream, void* ws, size_t ws_bytes) {
+  detail::check(dgpp_launch_mma_gemv_fp8_bf16_pair(a0, w0, s0, o0, n0, stride0, a1, w1, s1, o1, n1, stride1, act_stride, m, k, rs,
+                                                   cs, stream, ws, ws_bytes));
+}
 inline void launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t* up, float limit, size_t act_stride,
                                            const uint8_t* w, const float* scales, float* out, int m, int n, int k,
                                            size_t out_stride, int rs, int cs, hipStream_t stream) {

@@ -278,3 +278,36 @@ def test_try_dense_fp4_decode_follows_the_shape_rule(gpu):
     assert L.try_dense_fp4_decode_bf16(d.x, H, seg, d.views, 1, got, m, I, H - 64, None, 16) is False      # k % 128
     sync()
     assert np.all(host(got, np.uint16) == 0x1234), "nothing was launched"
+
+
+@pytest.mark.parametrize("m,n0,n1,k,with_ws", [(1, 1536, 576, 7168, True), (8, 200, 130, 2048, False), (20, 96, 300, 1024, True),
+                                                (32, 64, 64, 4096, True)])
+def test_fp8_pair_launch_is_bitwise_the_two_single_launches(gpu, m, n0, n1, k, with_ws):
+    """src/kernels/mma_gemv.hpp:119-130: two projections in one launch, each row's chain its single launch's."""
+    acts = [hg.normal_bf16(0x6B0 + i + n0, (m, k)) for i in range(2)]
+    mats = []
+    for i, n in enumerate((n0, n1)):
+        w = hg.f32_to_bf16(hg.normal_f32(0x6C0 + i + n + k, (n, k), 0.02))
+        mats.append(hg.encode_fp8_blocks(w, 128, 128))
+    a_d = [dev(a) for a in acts]
+    w_d = [(dev(p), dev(s)) for p, s in mats]
+    ws_floats = 4 * m * (n0 + n1)
+    ws = dev_empty(ws_floats, np.float32) if with_ws else None
+    outs = [dev_empty((m, n + 8), np.uint16) for n in (n0, n1)]
+    want = [dev_empty((m, n + 8), np.uint16) for n in (n0, n1)]
+    for t in outs + want:
+        t.zero_()
+    if with_ws:
+        assert L.mma_gemv_pair_ok(w_d[0][0], w_d[1][0], a_d[0], a_d[1], k, m, n0, n1, k, ws, ws_floats * 4)
+    assert not L.mma_gemv_pair_ok(w_d[0][0], w_d[1][0], a_d[0], a_d[1], k, m, n0, n1, k, None, 0)
+    assert not L.mma_gemv_pair_ok(w_d[0][0], w_d[1][0], a_d[0], a_d[1], k, 33, n0, n1, k, ws, ws_floats * 4 if ws is not None else 0)
+    assert L.mma_gemv_shape_ok(w_d[0][0], a_d[0], k, m, k) and not L.mma_gemv_shape_ok(w_d[0][0], a_d[0], k, m, k + 16)
+    L.launch_mma_gemv_fp8_bf16_pair(a_d[0], w_d[0][0], w_d[0][1], outs[0], n0, n0 + 8, a_d[1], w_d[1][0], w_d[1][1], outs[1], n1,
+                                    n1 + 8, k, m, k, 7, 7, None, ws, ws_floats * 4 if with_ws else 0)
+    for i, n in enumerate((n0, n1)):
+        L.launch_mma_gemv_fp8_bf16(a_d[i], k, w_d[i][0], w_d[i][1], want[i], m, n, k, n + 8, 7, 7, None)
+    sync()
+    for i, n in enumerate((n0, n1)):
+        g = host(outs[i], np.uint16)
+        assert np.array_equal(g, host(want[i], np.uint16)), f"problem {i}"
+        check(np.ascontiguousarray(g[:, :n]), orc.gemv_fp8(acts[i], mats[i][0], mats[i][1], m, n, k, 7, 7, True), f"pair problem {i}")
