@@ -438,6 +438,11 @@ inline void launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, c
   detail::check(dgpp_launch_moe_grouped_mma_f32(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                                 out_stride, n, k, stream, act_rows));
 }
+// Timing-sweep knobs of the reference's kernels (src/kernels/glm_moe_launch.hpp:88-90, src/kernels/mma_gemv.hpp:132-135):
+// accepted so that its benchmarks compile; this library's kernels have no counterpart setting and results never depended
+// on them in the reference either.
+inline void moe_set_fp8_ldm(bool) {}
+inline void mma_gemv_set_decode_width(int) {}
 inline bool mma_gemv_shape_ok(const void* w, const void* act, size_t act_stride, int m, int k) {
   return dgpp_mma_gemv_shape_ok(w, act, act_stride, m, k) != 0;
 }
