@@ -73,7 +73,7 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5,c5skew,w8a8,qwen_tail,slotbench,readprobe,router ('' for none; default: c1,c2,c4,c5, none under --tune)")
+                    "separated out of c1,c2,c4,c5,c5skew,w8a8,qwen_tail,slotbench,readprobe,router,pair,dispatch ('' for none; default: c1,c2,c4,c5, none under --tune)")
     ap.add_argument("--replays", type=int, default=0, help="timed graph replays per measurement (0 = at least 50 and at "
                     "least 1000 steps; a small number keeps a run under a profiler's counters short)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
@@ -812,13 +812,93 @@ def main():
         res["workload"] = "router: score rows + selection, two launches, softmax top-8"
         return res
 
+    def bench_pair():
+        """Two FP8 projections of one k in one matrix-core launch against two launches (the reference's decode pair:
+        launch_mma_gemv_fp8_bf16_pair), cold weights, with and without a split-K workspace."""
+        res = {"workload": "two block-FP8 projections (n 1536 and 576, k 7168) of one batch: one launch against two"}
+        k, n0, n1 = 7168, 1536, 576
+        mats = []
+        for i, n in enumerate((n0, n1)):
+            p_, s_ = hg.encode_fp8_blocks(hg.f32_to_bf16(hg.normal_f32(0xD6990500 + i, (n, k), 0.02)), 128, 128)
+            mats.append((torch.from_numpy(p_).to(dev), torch.from_numpy(s_).to(dev)))
+        ring = ring_copies([mats[0][0], mats[0][1], mats[1][0], mats[1][1]], sum(t.numel() for m_ in mats for t in m_[:1]))
+        for m in (1, 8):
+            act = torch.from_numpy(hg.normal_bf16(0xD6990510 + m, (m, k)).view(np.int16)).to(dev)
+            o0 = torch.empty((m, n0), dtype=torch.int16, device=dev)
+            o1 = torch.empty((m, n1), dtype=torch.int16, device=dev)
+            ws = torch.empty(4 * m * (n0 + n1), dtype=torch.float32, device=dev)
+            for use_ws in (False, True):
+                w_, wb = (ws, ws.numel() * 4) if use_ws else (None, 0)
+                def one(i):
+                    r = ring[i % len(ring)]
+                    L.launch_mma_gemv_fp8_bf16_pair(act, r[0], r[1], o0, n0, 0, act, r[2], r[3], o1, n1, 0, k, m, k, 7, 7, stream, w_, wb)
+                def two(i):
+                    r = ring[i % len(ring)]
+                    L.launch_mma_gemv_fp8_bf16(act, k, r[0], r[1], o0, m, n0, k, 0, 7, 7, stream, w_, wb)
+                    L.launch_mma_gemv_fp8_bf16(act, k, r[2], r[3], o1, m, n1, k, 0, 7, 7, stream, w_, wb)
+                tag = f"m{m}_{'split_k' if use_ws else 'unsplit'}"
+                res[tag + "_one_launch"] = {"us": time_graph(one, args.steps, args.warmup) * 1e6}
+                res[tag + "_two_launches"] = {"us": time_graph(two, args.steps, args.warmup) * 1e6}
+        return res
+
+    def bench_dispatch():
+        """What the dense launchers' choice between the two cores rests on: one to eight rows against cold weights of
+        several sizes on the vector core, on the matrix core unsplit, and on the matrix core with a split-K workspace
+        (us per launch; --configs dispatch)."""
+        res = {"workload": "dense GEMV by row count: vector core / matrix core / matrix core with a split-K workspace, cold weights"}
+        cases = [("fp8", 1536, 7168), ("fp8", 4096, 4096), ("fp8", 12288, 6144), ("nvfp4", 2048, 4096), ("nvfp4", 8192, 4096),
+                 ("nvfp4", 17408, 5120), ("mxfp4", 6144, 2048), ("mxfp4", 17408, 5120)]
+        for kind, n, k in cases:
+            w = hg.normal_f32(0xD6990600 + n, (n, k), 0.02)
+            glob = None
+            if kind == "fp8":
+                p_, s_ = hg.encode_fp8_blocks(hg.f32_to_bf16(w), 128, 128)
+            elif kind == "nvfp4":
+                p_, s_, ws2 = hg.encode_nvfp4(w)
+                glob = torch.tensor([1.0 / np.float32(ws2)], dtype=torch.float32, device=dev)
+            else:
+                p_, s_ = hg.encode_mxfp4(w)
+            ring = ring_copies([torch.from_numpy(p_).to(dev), torch.from_numpy(s_).to(dev)], p_.nbytes)
+            mats = None if kind == "fp8" else [L.Fp4Matrix(r[0].data_ptr(), r[1].data_ptr(), glob.data_ptr() if glob is not None else None,
+                                                            n, k, 16 if kind == "nvfp4" else 32, 0, None) for r in ring]
+            for m in (1, 2, 4, 5, 6, 8):
+                act = torch.from_numpy(hg.normal_bf16(0xD6990610 + m, (m, k)).view(np.int16)).to(dev)
+                out = torch.empty((m, n), dtype=torch.int16, device=dev)
+                ws = torch.empty(4 * m * n, dtype=torch.float32, device=dev)
+                row = {}
+                for name, core, w_ in (("vector_core", 1, None), ("matrix_core", 2, None), ("matrix_core_split_k", 2, ws)):
+                    wb = ws.numel() * 4 if w_ is not None else 0
+                    def step(i):
+                        r = i % len(ring)
+                        if kind == "fp8":
+                            L.launch_mma_gemv_fp8_bf16(act, k, ring[r][0], ring[r][1], out, m, n, k, 0, 7, 7, stream, w_, wb)
+                        elif w_ is None:
+                            L.launch_fp4_gemv_bf16(act, k, mats[r], out, m, n, k, stream)
+                        else:
+                            L.launch_mma_gemv_fp4_bf16(act, k, mats[r], out, m, n, k, 0, stream, w_, wb)
+                    lib.dgpp_tune_set(5, core)
+                    row[name] = time_graph(step, 32, 3) * 1e6
+                    lib.dgpp_tune_set(5, 0)
+                lib.dgpp_tune_set(5, 0)
+                def chosen(i):
+                    r = i % len(ring)
+                    if kind == "fp8":
+                        L.launch_mma_gemv_fp8_bf16(act, k, ring[r][0], ring[r][1], out, m, n, k, 0, 7, 7, stream, None, 0)
+                    else:
+                        L.launch_fp4_gemv_bf16(act, k, mats[r], out, m, n, k, stream)
+                row["launcher_without_workspace"] = time_graph(chosen, 32, 3) * 1e6
+                res[f"{kind}_{n}x{k}_m{m}"] = {"us": row["launcher_without_workspace"], **{k_: round(v, 2) for k_, v in row.items()}}
+            del ring, mats
+            torch.cuda.empty_cache()
+        return res
+
     other_configs = {}
     configs = args.configs if args.configs is not None else ("" if args.tune else "c1,c2,c4,c5")
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
             other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "c5skew": lambda: bench_c5(True), "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail, "readprobe": bench_readprobe,
-                                   "slotbench": bench_slotbench, "router": bench_router}[name]()
+                                   "slotbench": bench_slotbench, "router": bench_router, "pair": bench_pair, "dispatch": bench_dispatch}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
 

@@ -84,6 +84,10 @@ hipError_t launch_dense(int fmt, const DenseArgs& a, hipStream_t s) {
     default: return launch_dense_fmt<kFmtMxfp4>(a, s);
   }
 }
+hipError_t launch_dense_multi(int fmt, const DenseArgs* problems, int count, hipStream_t s) {
+  return fmt == kFmtFp8E8M0 ? launch_dense_multi_fmt<kFmtFp8E8M0>(problems, count, s)
+                            : launch_dense_multi_fmt<kFmtFp8F32>(problems, count, s);
+}
 hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t s) {
   switch (fmt) {
     case kFmtFp8F32: return launch_slot_gate_up_fmt<kFmtFp8F32>(a, s);
@@ -138,19 +142,42 @@ hipError_t launch_grouped_mma(int fmt, const GroupedArgs& a, int n_segs, int z_e
 
 namespace {
 
-// Dense projection over m rows. Few rows take the vector-core GEMV in chunks the LDS can stage (each row's chain is
-// the same whatever the chunking); from `mma_from` rows on the call goes to the matrix-core form, which carries 16
-// rows per weight pass (the reference's launchers move to their tensor-core forms as m grows in the same way:
-// src/kernels/scale_gemm.cu:296-339, src/kernels/glm_moe_launch.hpp:363). The two forms differ in fp32 summation
-// order, so a row's bits depend on which side of the boundary the call's m lies - both are held to the same oracle
-// tolerance. `ws` (nullable) is the split-K workspace of the matrix-core form. `out_elem` is 2 (bf16) or 4 (f32).
-constexpr int kFp4MmaFromRows = 5;   // vector core: 8 dot chains per weight beyond 4 rows cost more than the matrix core's decode
-constexpr int kFp8MmaFromRows = 9;   // the vector core's one-pass limit (kMaxActRows)
+// Dense projection over m rows: the vector-core GEMV (up to eight rows per pass over the weights, in chunks the LDS
+// can stage; each row's chain is the same whatever the chunking) or the matrix-core form (16 rows per pass) - the
+// reference's launchers move to their tensor-core forms as m grows in the same way (src/kernels/scale_gemm.cu:296-339,
+// src/kernels/glm_moe_launch.hpp:363). The two forms differ in fp32 summation order, so a row's bits depend on which
+// form its call takes - both are held to the same oracle tolerance. `ws` (nullable) is the split-K workspace of the
+// matrix-core form.
+//
+// Which form, measured on this chip (cold weights; 2048 x 4096 ... 17408 x 5120, one to eight rows):
+// * more rows than one vector pass holds: the matrix core (the vector core would read the weights again per pass);
+// * five to eight rows: the vector core pays a dot chain per row and weight, the matrix core one decode per weight -
+//   but an unsplit matrix-core launch has one block per 64 weight rows, too few to fill the chip unless the matrix is
+//   large: with a split-K workspace the matrix core wins from five rows on (from three for matrices of 48 M weights and
+//   more), without one only for matrices of 64 M weights and more;
+// * up to four rows: the vector core.
+constexpr int kVectorPassRows = kMaxActRows;
+bool dense_takes_matrix_core(int fmt, int m, int n, int k, size_t ws_bytes, bool have_ws, int from_rows) {
+  if (m > kVectorPassRows || m > max_stage_rows(k)) return true;
+  if (from_rows > 0 && m >= from_rows) return true;   // the caller's own boundary (the reference's mma_from_rows)
+  const size_t weights = static_cast<size_t>(n) * static_cast<size_t>(k);
+  int parts = 1;
+  switch (fmt) {
+    case kFmtFp8F32: parts = mgeom<kFmtFp8F32>(k).parts; break;
+    case kFmtFp8E8M0: parts = mgeom<kFmtFp8E8M0>(k).parts; break;
+    case kFmtNvfp4: parts = mgeom<kFmtNvfp4>(k).parts; break;
+    default: parts = mgeom<kFmtMxfp4>(k).parts; break;
+  }
+  const bool split = have_ws && parts > 1 && (n + 63) / 64 < 1024 &&
+                     ws_bytes >= static_cast<size_t>(parts) * m * static_cast<size_t>(n) * sizeof(float);
+  if (split) return m >= 5 || (m >= 3 && weights >= (48u << 20));
+  return m >= 5 && weights >= (64u << 20);
+}
 int dense_rows(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,
-               size_t out_stride, int out_f32, int m, int n, int k, hipStream_t stream, const char* who, int mma_from,
+               size_t out_stride, int out_f32, int m, int n, int k, hipStream_t stream, const char* who, int from_rows,
                void* ws = nullptr, size_t ws_bytes = 0) {
   const int core = tune_get(kTuneCore);   // bench switch: 1 pins the vector core, 2 the matrix core
-  if (core != 1 && (core == 2 || m >= mma_from)) {
+  if (core != 1 && (core == 2 || dense_takes_matrix_core(fmt, m, n, k, ws_bytes, ws != nullptr, from_rows))) {
     if ((m + kTileCols - 1) / kTileCols > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
     DenseArgs a;
     a.act = act;
@@ -208,7 +235,7 @@ int fp4_gemv(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, voi
   mat.rs = 0;
   mat.cs = 0;
   return dense_rows(w->scale_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, mat, w->global_scale, out,
-                    static_cast<size_t>(n), out_f32, m, n, k, as_stream(stream), "fp4_gemv", kFp4MmaFromRows);
+                    static_cast<size_t>(n), out_f32, m, n, k, as_stream(stream), "fp4_gemv", 0);
 }
 
 // src/kernels/scale_gemm.cu:280-365 (launch_scale_gemm) and :406-462 (launch_scale_gemm_grid):
@@ -245,8 +272,7 @@ int scale_gemm(const uint16_t* act, size_t act_stride, const uint8_t* payload, c
   }
   if (!fp8_shape_ok(payload, k))
     return fail_arg(std::string(who) + ": k must be a multiple of 16 with a 16-byte aligned payload");
-  // the caller's own threshold (the reference's mma_from_rows) can only lower the boundary
-  const int mma_from = mma_from_rows > 0 && mma_from_rows < kFp8MmaFromRows ? mma_from_rows : kFp8MmaFromRows;
+  const int mma_from = mma_from_rows > 0 ? mma_from_rows : 0;   // the caller's own boundary can only add matrix-core cases
   return dense_rows(e8m0 ? kFmtFp8E8M0 : kFmtFp8F32, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, o,
                     out_stride, out_f32, m, n, k, as_stream(stream), who, mma_from, ws, ws_bytes);
 }
@@ -956,6 +982,29 @@ static int dense_mma_fp8(const uint16_t* act, size_t act_stride, const uint8_t* 
   return dense_mma(e8m0 ? kFmtFp8E8M0 : kFmtFp8F32, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, out,
                    out_f32, out_stride, m, n, k, ws, ws_bytes, stream, who, act_up, limit);
 }
+// The reference's streaming tensor-core GEMV (launch_mma_gemv_fp8{,e8m0}_*) is its decode form for FP8 weights at every
+// row count. Here a batch that fits one vector-core pass (up to eight rows) runs on the vector core, which is the
+// faster form for it on this chip; from nine rows on the matrix core takes over (ws: its split-K workspace). As with the
+// GEMV-named launchers the two cores differ in summation order and meet the same tolerance.
+static int mma_gemv_fp8(const uint16_t* act, size_t act_stride, const uint8_t* payload, const void* scales, int e8m0, void* out,
+                        int out_f32, int m, int n, int k, size_t out_stride, int rs, int cs, void* ws, size_t ws_bytes,
+                        void* stream, const char* who) {
+  if (m <= 0 || n <= 0) return DGPP_OK;
+  const int fmt = e8m0 ? kFmtFp8E8M0 : kFmtFp8F32;
+  if (tune_get(kTuneCore) == 2 || k <= 0 || (tune_get(kTuneCore) != 1 && dense_takes_matrix_core(fmt, m, n, k, ws_bytes, ws != nullptr, 0)))
+    return dense_mma_fp8(act, act_stride, payload, scales, e8m0, out, out_f32, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream,
+                         who);
+  if (!act || !payload || !scales || !out) return fail_arg(std::string(who) + ": null pointer");
+  const bool row_grid = rs == 0 && cs >= 4;
+  if (!row_grid && (rs < 4 || rs > 7 || cs < 4 || cs > 7))
+    return fail_arg(std::string(who) + ": rs / cs must be 4..7 or a row grid (rs = 0, cs >= 4)");
+  if (k <= 0 || !fp8_shape_ok(payload, k))
+    return fail_arg(std::string(who) + ": k must be a positive multiple of 16 with a 16-byte aligned payload");
+  if (out_stride == 0) out_stride = static_cast<size_t>(n);
+  if (out_stride < static_cast<size_t>(n)) return fail_arg(std::string(who) + ": output row stride narrower than n");
+  return dense_rows(fmt, act, act_stride, fp8_mat(payload, scales, rs, cs), nullptr, out, out_stride, out_f32, m, n, k,
+                    as_stream(stream), who, 0, ws, ws_bytes);
+}
 /* src/kernels/mma_gemv.cu:895-899: the shape the matrix-core GEMV takes. */
 int dgpp_mma_gemv_shape_ok(const void* w, const void* act, size_t act_stride, int m, int k) {
   return m >= 1 && k > 0 && (k % 64) == 0 && (reinterpret_cast<uintptr_t>(w) & 15u) == 0 &&
@@ -993,6 +1042,20 @@ int dgpp_launch_mma_gemv_fp8_bf16_pair(const uint16_t* a0, const uint8_t* w0, co
   if (stride0 < static_cast<size_t>(n0) || stride1 < static_cast<size_t>(n1))
     return fail_arg(std::string(who) + ": output row stride narrower than n");
   if ((m + kTileCols - 1) / kTileCols > 65535) return fail_arg(std::string(who) + ": grid dimension overflow");
+  // Each problem takes the core its single launch would take (so that its bits are that launch's): both on the vector
+  // core -> one vector-core launch over both; both on the matrix core -> one matrix-core launch; one each -> two launches.
+  const int core = tune_get(kTuneCore);
+  auto takes_mma = [&](int n) {
+    if (core == 2) return true;
+    return dense_takes_matrix_core(kFmtFp8F32, m, n, k, ws_bytes, ws != nullptr, 0);
+  };
+  const bool mma0 = takes_mma(n0), mma1 = takes_mma(n1);
+  if (mma0 != mma1 || core == 1) {   // (the bench switch that pins the vector core: the single launchers know how)
+    const int rc = dgpp_launch_mma_gemv_fp8_bf16(a0, act_stride, w0, s0, o0, m, n0, k, stride0, rs, cs, stream, ws, ws_bytes);
+    if (rc != DGPP_OK) return rc;
+    return dgpp_launch_mma_gemv_fp8_bf16(a1, act_stride, w1, s1, o1, m, n1, k, stride1, rs, cs, stream, ws, ws_bytes);
+  }
+  const bool vector_core = !mma0;
   DenseArgs p[2];
   const uint16_t* acts[2] = {a0, a1};
   const uint8_t* ws_[2] = {w0, w1};
@@ -1013,6 +1076,7 @@ int dgpp_launch_mma_gemv_fp8_bf16_pair(const uint16_t* a0, const uint8_t* w0, co
     p[i].k = k;
     p[i].once = m <= kTileCols;
   }
+  if (vector_core) return finish(launch_dense_multi(kFmtFp8F32, p, 2, as_stream(stream)), who);
   return finish(launch_dense_mma_pair_fp8(p[0], p[1], static_cast<float*>(ws), ws_bytes, as_stream(stream)), who);
 }
 int dgpp_launch_mma_gemv_fp8_swiglu_f32(const uint16_t* gate, const uint16_t* up, float limit, size_t act_stride,
@@ -1049,23 +1113,23 @@ int dgpp_launch_scale_gemm_tile_f32(const uint16_t* act, size_t act_row_stride_e
 int dgpp_launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
                                   uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
                                   void* ws, size_t ws_bytes) {
-  return dense_mma_fp8(act, act_stride, w, scales, 0, out, 0, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream, "mma_gemv_fp8");
+  return mma_gemv_fp8(act, act_stride, w, scales, 0, out, 0, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream, "mma_gemv_fp8");
 }
 int dgpp_launch_mma_gemv_fp8_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales, float* out,
                                  int m, int n, int k, size_t out_stride, int rs, int cs, void* stream, void* ws,
                                  size_t ws_bytes) {
-  return dense_mma_fp8(act, act_stride, w, scales, 0, out, 1, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream, "mma_gemv_fp8");
+  return mma_gemv_fp8(act, act_stride, w, scales, 0, out, 1, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream, "mma_gemv_fp8");
 }
 int dgpp_launch_mma_gemv_fp8e8m0_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
                                       uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
                                       void* ws, size_t ws_bytes) {
-  return dense_mma_fp8(act, act_stride, w, scales, 1, out, 0, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream,
+  return mma_gemv_fp8(act, act_stride, w, scales, 1, out, 0, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream,
                        "mma_gemv_fp8e8m0");
 }
 int dgpp_launch_mma_gemv_fp8e8m0_f32(const uint16_t* act, size_t act_stride, const uint8_t* w, const uint8_t* scales,
                                      float* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
                                      void* ws, size_t ws_bytes) {
-  return dense_mma_fp8(act, act_stride, w, scales, 1, out, 1, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream,
+  return mma_gemv_fp8(act, act_stride, w, scales, 1, out, 1, m, n, k, out_stride, rs, cs, ws, ws_bytes, stream,
                        "mma_gemv_fp8e8m0");
 }
 
@@ -1383,6 +1447,27 @@ int dgpp_launch_scale_gemv_multi_bf16(const DgppFp8GemvProblem* problems, int n_
     if (p.bf16_weight) return fail_arg(std::string(who) + ": bf16 problems are outside this library's path");
     if (!p.payload || !p.scales || !p.out || p.n <= 0) return fail_arg(std::string(who) + ": null pointer");
     if (!fp8_shape_ok(p.payload, k)) return fail_arg(std::string(who) + ": k must be a multiple of 16 with aligned payloads");
+  }
+  // One launch over all problems' row tiles where the rows fit one stage (the decode case); otherwise one launch each.
+  if (tune_get(kTuneCore) != 2 && rows <= max_stage_rows(k)) {
+    DenseArgs d[kMaxDenseProblems];
+    for (int i = 0; i < n_problems; ++i) {
+      const DgppFp8GemvProblem& p = problems[i];
+      const size_t out_stride = p.out_stride ? p.out_stride : static_cast<size_t>(p.n);
+      if (out_stride < static_cast<size_t>(p.n)) return fail_arg(std::string(who) + ": output row stride narrower than n");
+      d[i].act = act;
+      d[i].act_stride = act_row_stride_elems;
+      d[i].mat = fp8_mat(p.payload, p.scales, p.rs, p.cs);
+      d[i].global = nullptr;
+      d[i].out = p.out;
+      d[i].out_stride = out_stride;
+      d[i].out_f32 = 0;
+      d[i].m = rows;
+      d[i].n = p.n;
+      d[i].k = k;
+      d[i].once = 1;
+    }
+    return finish(launch_dense_multi(kFmtFp8F32, d, n_problems, as_stream(stream)), who);
   }
   for (int i = 0; i < n_problems; ++i) {
     const DgppFp8GemvProblem& p = problems[i];

@@ -5,5 +5,6 @@
 
 namespace dgpp_amd {
 template hipError_t launch_dense_fmt<kFmtFp8E8M0>(const DenseArgs&, hipStream_t);
+template hipError_t launch_dense_multi_fmt<kFmtFp8E8M0>(const DenseArgs*, int, hipStream_t);
 template hipError_t launch_dense_mma_fmt<kFmtFp8E8M0>(const DenseArgs&, float*, size_t, hipStream_t);
 }  // namespace dgpp_amd

@@ -5,6 +5,7 @@
 
 namespace dgpp_amd {
 template hipError_t launch_dense_fmt<kFmtFp8F32>(const DenseArgs&, hipStream_t);
+template hipError_t launch_dense_multi_fmt<kFmtFp8F32>(const DenseArgs*, int, hipStream_t);
 template hipError_t launch_slot_gate_up_fmt<kFmtFp8F32>(const SlotArgs&, hipStream_t);
 template hipError_t launch_select_gate_up_fmt<kFmtFp8F32>(const SlotArgs&, const SelectArgs&, hipStream_t);
 template hipError_t launch_slot_down_fmt<kFmtFp8F32>(const SlotArgs&, hipStream_t);

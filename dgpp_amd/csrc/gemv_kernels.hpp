@@ -102,6 +102,54 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_ke
   }
 }
 
+// Up to four dense problems of one k and one row count in ONE launch (reference: launch_scale_gemv_multi_bf16,
+// src/kernels/scale_gemm.cu:625-672): the grid is the problems' row tiles laid end to end; a block finds its problem
+// and then does what gemv_dense_kernel does for it, so each output is bitwise its single launch's.
+constexpr int kMaxDenseProblems = 4;
+struct DenseMultiArgs {
+  DenseArgs p[kMaxDenseProblems];
+  int tile_end[kMaxDenseProblems];   // one past the last grid block of each problem
+  int count;
+};
+
+template <int FMT, int MAXR, int NB, bool NT>
+__global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void gemv_dense_multi_kernel(DenseMultiArgs ma, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  int which = 0;
+  const int b = static_cast<int>(blockIdx.x);
+#pragma unroll
+  for (int i = 0; i + 1 < kMaxDenseProblems; ++i)
+    if (i + 1 < ma.count && b >= ma.tile_end[i]) which = i + 1;
+  const DenseArgs& a = ma.p[which];
+  const int bx = b - (which ? ma.tile_end[which - 1] : 0);
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  stage_activations<FMT>(a.act, a.act_stride, a.m, a.k, lds);
+  __syncthreads();
+  const float divisor = load_divisor<FMT>(a.global);
+  const int rpw = kWave >> g.l2;
+  const int wave = threadIdx.x >> 6;
+  int row0 = bx * block_rows(g, steps) + wave * rpw;
+  for (int s = 0; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+    if (row0 >= a.n) break;
+    const auto lr = lane_row<FMT, NT>(a.mat, row0, a.n, a.k, g.l2);
+    float acc[MAXR];
+    row_dots<FMT, MAXR, NB>(lr, g, a.mat.cs, lds, chunks, a.m, acc);
+    if (lr.li == 0 && lr.row < a.n) {
+#pragma unroll
+      for (int r = 0; r < MAXR; ++r) {
+        if (r < a.m) {
+          const float v = finish_dot<FMT>(acc[r], divisor);
+          const size_t at = static_cast<size_t>(r) * a.out_stride + lr.row;
+          if (a.out_f32)
+            static_cast<float*>(a.out)[at] = v;
+          else
+            static_cast<uint16_t*>(a.out)[at] = f32_to_bf16(v);
+        }
+      }
+    }
+  }
+}
+
 // ---- MoE decode slots ----------------------------------------------------------------------------
 // Slot layout (src/kernels/glm_moe_launch.hpp:216-226): slot = t * (top_k + 1) + j, j < top_k the
 // token's j-th routed expert (ascending id), j == top_k the shared expert.
@@ -702,6 +750,9 @@ inline int pick_steps(long long block_steps_total) {
 }
 
 hipError_t launch_dense(int fmt, const DenseArgs& a, hipStream_t stream);
+// `count` problems (<= kMaxDenseProblems) of one k, one row count (<= the rows one stage holds) in one vector-core launch.
+hipError_t launch_dense_multi(int fmt, const DenseArgs* problems, int count, hipStream_t stream);
+template <int FMT> hipError_t launch_dense_multi_fmt(const DenseArgs* problems, int count, hipStream_t stream);
 hipError_t launch_slot_gate_up(int fmt, const SlotArgs& a, hipStream_t stream);
 hipError_t launch_select_gate_up(int fmt, const SlotArgs& a, const SelectArgs& sel, hipStream_t stream);
 hipError_t launch_slot_down(int fmt, const SlotArgs& a, hipStream_t stream);
@@ -926,6 +977,45 @@ hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream) {
     if (a.m == 1) go(std::integral_constant<int, 1>{});
     else if (a.m == 2) go(std::integral_constant<int, 2>{});
     else if (a.m <= 4) go(std::integral_constant<int, 4>{});
+    else go(std::integral_constant<int, 8>{});
+  });
+  return err != hipSuccess ? err : hipGetLastError();
+}
+
+template <int FMT>
+hipError_t launch_dense_multi_fmt(const DenseArgs* problems, int count, hipStream_t stream) {
+  const DenseArgs& first = problems[0];
+  const RowGeom g = geom_for<FMT>(first.k);
+  const int rows_per_step = kWavesPerBlock * (kWave >> g.l2);
+  long long all_steps = 0;
+  for (int i = 0; i < count; ++i) all_steps += (problems[i].n + rows_per_step - 1) / rows_per_step;
+  int steps = pick_steps(all_steps);
+  if (tune_get(kTuneSlotSteps) > 0) steps = tune_get(kTuneSlotSteps);
+  DenseMultiArgs ma{};
+  ma.count = count;
+  long long end = 0;
+  for (int i = 0; i < count; ++i) {
+    ma.p[i] = problems[i];
+    const long long block_steps = (problems[i].n + rows_per_step - 1) / rows_per_step;
+    end += (block_steps + steps - 1) / steps;
+    ma.tile_end[i] = static_cast<int>(end);
+  }
+  if (end > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+  const dim3 grid(static_cast<unsigned>(end));
+  const size_t lds = stage_bytes(first.m, first.k);
+  hipError_t err = hipSuccess;
+  dispatch_nb(g.nb, [&](auto nbc) {
+    constexpr int NB = decltype(nbc)::value;
+    auto go = [&](auto rc) {
+      constexpr int MAXR = decltype(rc)::value;
+      auto kern = gemv_dense_multi_kernel<FMT, MAXR, NB, true>;   // every problem's weights stream through once
+      err = ensure_lds(kern, lds);
+      if (err != hipSuccess) return;
+      hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, ma, g, steps);
+    };
+    if (first.m == 1) go(std::integral_constant<int, 1>{});
+    else if (first.m == 2) go(std::integral_constant<int, 2>{});
+    else if (first.m <= 4) go(std::integral_constant<int, 4>{});
     else go(std::integral_constant<int, 8>{});
   });
   return err != hipSuccess ? err : hipGetLastError();

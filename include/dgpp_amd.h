@@ -375,6 +375,11 @@ int dgpp_launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const D
 #define DGPP_STATIC_SCRATCH_BYTES (8u << 20)
 int dgpp_launch_mma_gemv_fp4_bf16_static(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out,
                                          int m, int n, int k, size_t out_stride, void* stream);
+/* src/kernels/mma_gemv.hpp:70-94 (launch_mma_gemv_fp8{,e8m0}_{bf16,f32}): the reference's streaming tensor-core GEMV for
+ * FP8 weights. The same dispatch as dgpp_launch_scale_gemm_bf16 here: small batches run on the vector core where that
+ * is the faster form on this chip (always up to four rows; five to eight rows without a workspace unless the matrix is
+ * large), the rest on the matrix core with `ws` as its split-K workspace. The two cores differ in fp32 summation order;
+ * both meet the same tolerance against the fp64 oracle. */
 int dgpp_launch_mma_gemv_fp8_bf16(const uint16_t* act, size_t act_stride, const uint8_t* w, const float* scales,
                                   uint16_t* out, int m, int n, int k, size_t out_stride, int rs, int cs, void* stream,
                                   void* ws, size_t ws_bytes);
@@ -396,7 +401,8 @@ int dgpp_launch_moe_grouped_mma_f32(const uint16_t* act, size_t act_stride, cons
                                     size_t out_stride, int n, int k, void* stream, const int32_t* act_rows);
 /* src/kernels/mma_gemv.hpp:103-104, :119-130 (mma_gemv_shape_ok, mma_gemv_pair_ok, launch_mma_gemv_fp8_bf16_pair): two
  * FP8 projections of one k against one batch in ONE launch - two dependent-free GEMVs sharing one ramp and drain.
- * Each row's bits are those of dgpp_launch_mma_gemv_fp8_bf16 on its own problem. act_stride is both activations';
+ * Each row's bits are those of dgpp_launch_mma_gemv_fp8_bf16 on its own problem (up to eight rows: both problems in one
+ * vector-core launch; more: one matrix-core launch). act_stride is both activations';
  * ws (nullable here) holds both problems' K-part sums: parts(k) * m * (n0 + n1) floats. pair_ok mirrors the reference's
  * conditions that carry over (a workspace, 1 <= m <= 32, both shapes taken, the workspace large enough). */
 int dgpp_mma_gemv_shape_ok(const void* w, const void* act, size_t act_stride, int m, int k);
@@ -453,10 +459,14 @@ int dgpp_launch_moe_grouped_mma_fp4_f32(const uint16_t* act, size_t act_stride, 
                                         int fp4_group, int tile_rows);
 
 /* src/kernels/fp4_gemv.hpp:23-32. `w` is a HOST struct holding device pointers.
- * Row-count dispatch: up to 4 rows ride the vector-core GEMV (one weight pass); from 5 rows on the call runs the
- * matrix-core form (16 rows per weight pass), as the reference moves to its tensor-core form as m grows
- * (src/kernels/glm_moe_launch.hpp:363). The two forms sum in different fp32 orders: a row's bits depend on which side
- * of the boundary the call's m lies (never on m otherwise); both are held to the same oracle tolerance. */
+ * Dispatch between the vector-core GEMV (up to eight rows per pass over the weights) or the matrix-core form (16 rows
+ * per pass), chosen by what was measured faster on this chip: more rows than one vector pass holds -> matrix core; five
+ * to eight rows -> matrix core when a split-K workspace is there (then from three rows on for matrices of 48 M weights
+ * and more) or, without one, when the matrix has 64 M weights and more (an unsplit matrix-core launch has one block per
+ * 64 weight rows: too few to fill the chip for smaller matrices); otherwise the vector core.
+ * (This signature carries no workspace.) The reference moves to its tensor-core form as m grows in the same way
+ * (src/kernels/glm_moe_launch.hpp:363). The two forms sum in different fp32 orders: a row's bits depend on which form
+ * its call takes (a function of m, n, k only); both are held to the same oracle tolerance. */
 int dgpp_launch_fp4_gemv_bf16(const uint16_t* act, size_t act_row_stride_elems,
                               const DgppFp4Matrix* w, uint16_t* out, int m, int n, int k,
                               void* stream);
@@ -466,13 +476,17 @@ int dgpp_launch_fp4_gemv_f32(const uint16_t* act, size_t act_row_stride_elems,
 int dgpp_fp4_gemv_accepts(const DgppFp4Matrix* w);
 
 /* ---- dense FP8 block-scaled projection GEMV ------------------------------------------------------------ */
-/* src/kernels/scale_gemm.hpp:57-79. Row-count dispatch (reference: src/kernels/scale_gemm.cu:296-339): up to 8 rows
- * ride the vector-core GEMV in one weight pass; from 9 rows on - or from mma_from_rows on when the caller gives a
- * smaller positive bound - the call runs the matrix-core form (16 rows per weight pass), which uses `ws` / `ws_bytes`
- * (nullable; parts(k) * m * n floats) to split K over blocks when the unsplit grid would leave the chip under-filled.
- * Split and unsplit give the same bits; the two cores sum in different fp32 orders (both held to the same oracle
- * tolerance), so a row's bits depend on which side of the boundary the call's m lies, never on m otherwise.
- * last_row_only / compact_row compute one row and stay on the vector core. */
+/* src/kernels/scale_gemm.hpp:57-79. Dispatch (reference: src/kernels/scale_gemm.cu:296-339) between
+ * the vector-core GEMV (up to eight rows per pass over the weights) or the matrix-core form (16 rows
+ * per pass), chosen by what was measured faster on this chip: more rows than one vector pass holds -> matrix core; five
+ * to eight rows -> matrix core when a split-K workspace is there (then from three rows on for matrices of 48 M weights
+ * and more) or, without one, when the matrix has 64 M weights and more (an unsplit matrix-core launch has one block per
+ * 64 weight rows: too few to fill the chip for smaller matrices); otherwise the vector core.
+ * A positive mma_from_rows adds the calls with m >= mma_from_rows to the matrix-core side. `ws` / `ws_bytes` (nullable;
+ * parts(k) * m * n floats) is the split-K workspace. Split and unsplit give the same bits; the two cores sum in
+ * different fp32 orders (both held to the same oracle tolerance), so a row's bits depend on which form its call takes
+ * (a function of m, n, k and of whether a workspace is given). last_row_only / compact_row compute one row and stay
+ * on the vector core. */
 int dgpp_launch_scale_gemm_bf16(const uint16_t* act, size_t act_row_stride_elems,
                                 const uint8_t* w_payload, const float* w_scales, uint16_t* out,
                                 int m, int n, int k, void* stream, size_t out_row_stride_elems,
@@ -482,8 +496,8 @@ int dgpp_launch_scale_gemm_f32(const uint16_t* act, size_t act_row_stride_elems,
                                int n, int k, void* stream, size_t out_row_stride_elems,
                                int mma_from_rows, int last_row_only, void* ws, size_t ws_bytes,
                                int compact_row);
-/* src/kernels/scale_gemm.hpp:140-149: the same on a stated scale grid; the matrix-core form from 9 rows on (ws as
- * above; decode_mma and prefill_tile are the reference's tuning hints and are accepted unused). */
+/* src/kernels/scale_gemm.hpp:140-149: the same on a stated scale grid, with the same dispatch (ws as above; decode_mma
+ * and prefill_tile are the reference's tuning hints and are accepted unused). */
 int dgpp_launch_scale_gemm_grid_bf16(const uint16_t* act, size_t act_row_stride_elems,
                                      const uint8_t* w_payload, const float* w_scales, uint16_t* out,
                                      int m, int n, int k, void* stream,
@@ -511,7 +525,8 @@ int dgpp_launch_scale_gemm_tile_bf16(const uint16_t* act, size_t act_row_stride_
                                      const float* w_scales, uint16_t* out, int m, int n, int k, void* stream, int rs, int cs);
 int dgpp_launch_scale_gemm_tile_f32(const uint16_t* act, size_t act_row_stride_elems, const uint8_t* w_payload,
                                     const float* w_scales, float* out, int m, int n, int k, void* stream, int rs, int cs);
-/* src/kernels/scale_gemm.hpp:85-107: up to four [n_i, k] fp8 matrices against the same rows.
+/* src/kernels/scale_gemm.hpp:85-107: up to four [n_i, k] fp8 matrices against the same rows, ONE launch (the grid is the
+ * problems' row tiles laid end to end); each output is bitwise the single launcher's.
  * `problems` is a HOST array. bf16_weight must be null (that form is outside this path). */
 typedef struct DgppFp8GemvProblem {
   const uint8_t* payload;

@@ -19,7 +19,7 @@ extern "C" {
  * any weight load is issued (default: activation loads, first weight pass, LDS commit); key 4: 1 keeps
  * the layer driver on the two-launch down + accumulate form; key 5: 2 moves every GEMV launcher to the
  * matrix-core form, 1 keeps the dense launchers on the vector core at every row count (default: the dense launchers
- * move to the matrix core from 5 rows (FP4) / 9 rows (FP8) on); key 6: 1 makes the layer driver compute the slot order for small decode batches too
+ * choose by rows, matrix size and workspace); key 6: 1 makes the layer driver compute the slot order for small decode batches too
  * (default: batches of at most 128 routed slots find the sharers of an expert by ballot, no order);
  * key 7: 1 keeps the selection of a one-token step a launch of its own (default: repeated in the gate/up
  * blocks, dgpp_launch_moe_select_gate_up_swiglu); key 8: row tiles an XCD takes for one token before it turns to the next token in the token-major

@@ -52,7 +52,7 @@ def check(got_bits, raw, label):
 SHAPES = [(1, 520, 4096), (3, 264, 1024), (2, 100, 512), (4, 40, 256), (1, 33, 128), (2, 17, 64), (1, 9, 32),
           (4, 512, 4096), (2, 300, 2048), (1, 390, 5120), (3, 130, 5120), (2, 520, 384), (1, 77, 768), (4, 70, 1536),
           (2, 41, 3072), (1, 20, 12288), (8, 136, 6144), (5, 64, 2560),
-          (16, 200, 2048), (64, 96, 4096), (37, 70, 640)]          # from five rows on: the launcher's matrix-core form
+          (16, 200, 2048), (64, 96, 4096), (37, 70, 640)]          # more rows than one vector pass: the launcher's matrix-core form
 
 
 @pytest.mark.parametrize("m,n,k", SHAPES)
@@ -160,7 +160,7 @@ def make_fp8(m, n, k, seed, br=128, bc=128):
 
 FP8_SHAPES = [(1, 4096, 4096), (1, 520, 4096), (3, 264, 1024), (2, 100, 512), (4, 200, 768), (8, 130, 2048),
               (1, 33, 144), (2, 17, 16), (5, 260, 6144), (1, 70, 7168),
-              (16, 130, 2048), (64, 96, 1024), (9, 40, 304)]           # from nine rows on: the launcher's matrix-core form
+              (16, 130, 2048), (64, 96, 1024), (9, 40, 304)]           # more rows than one vector pass: the launcher's matrix-core form
 
 
 @pytest.mark.parametrize("m,n,k", FP8_SHAPES)

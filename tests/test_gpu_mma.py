@@ -147,7 +147,11 @@ def test_mma_gemv_fp8_swiglu_is_bitwise_swiglu_then_mma_gemv(gpu, m, n, k, limit
     g_d, u_d, p_d, s_d = dev(gate), dev(up), dev(payload), dev(scales)
     act, want, got = dev_empty((m, k), np.uint16), dev_empty((m, n), np.float32), dev_empty((m, n), np.float32)
     L.launch_moe_swiglu_clamp(g_d, u_d, act, m * k, limit, None)
-    L.launch_mma_gemv_fp8_f32(act, k, p_d, s_d, want, m, n, k, 0, 7, 7, None)
+    _lib.load().dgpp_tune_set(5, 2)      # the comparison runs on the matrix core at every row count, as the fused form does
+    try:
+        L.launch_mma_gemv_fp8_f32(act, k, p_d, s_d, want, m, n, k, 0, 7, 7, None)
+    finally:
+        _lib.load().dgpp_tune_set(5, 0)
     L.launch_mma_gemv_fp8_swiglu_f32(g_d, u_d, limit, k, p_d, s_d, got, m, n, k, 0, 7, 7, None)
     sync()
     assert np.array_equal(host(got).view(np.uint32), host(want).view(np.uint32))
@@ -250,7 +254,11 @@ def test_scale_gemm_tile_is_the_matrix_core_dense_form(gpu, m, n, k, rs, cs):
     tb, tf, want = dev_empty((m, n), np.uint16), dev_empty((m, n), np.float32), dev_empty((m, n), np.uint16)
     L.launch_scale_gemm_tile_bf16(a_d, k, p_d, s_d, tb, m, n, k, None, rs, cs)
     L.launch_scale_gemm_tile_f32(a_d, k, p_d, s_d, tf, m, n, k, None, rs, cs)
-    L.launch_mma_gemv_fp8_bf16(a_d, k, p_d, s_d, want, m, n, k, 0, rs, cs, None)
+    _lib.load().dgpp_tune_set(5, 2)      # the matrix-core form at every row count
+    try:
+        L.launch_mma_gemv_fp8_bf16(a_d, k, p_d, s_d, want, m, n, k, 0, rs, cs, None)
+    finally:
+        _lib.load().dgpp_tune_set(5, 0)
     sync()
     got = host(tb, np.uint16)
     assert np.array_equal(got, host(want, np.uint16))
