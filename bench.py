@@ -544,6 +544,17 @@ def main():
             L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
             L.launch_moe_round_bf16(out, routed, cT * cH, stream)
 
+        sws = torch.empty(4 * cT * max(cSI, cH), dtype=torch.float32, device=dev)   # split-K workspace: parts(k) * m * n floats
+
+        def shared_part_ws(i):   # the same launchers given a split-K workspace
+            nb_ = sws.numel() * 4
+            L.launch_scale_gemm_grid_e8m0_bf16(x, cH, sh[0][0], sh[0][1], g_d, cT, cSI, cH, stream, 0, 0, 5, sws, nb_)
+            L.launch_scale_gemm_grid_e8m0_bf16(x, cH, sh[1][0], sh[1][1], u_d, cT, cSI, cH, stream, 0, 0, 5, sws, nb_)
+            L.launch_moe_swiglu_clamp(g_d, u_d, a_d, cT * cSI, float("inf"), stream)
+            L.launch_scale_gemm_grid_e8m0_f32(a_d, cSI, sh[2][0], sh[2][1], shared_down, cT, cH, cSI, stream, 0, 0, 5, sws, nb_)
+            L.launch_moe_accum(routed, shared_down, rows_id, ones, cT, cH, stream)
+            L.launch_moe_round_bf16(out, routed, cT * cH, stream)
+
         def stitched(i):        # the shared expert through the GEMV-named launchers (they take the matrix core at 64 rows)
             routed_part(i)
             shared_part(i)
@@ -574,6 +585,7 @@ def main():
                              ("routed_only_matrix_core", routed_mc, uniq * per_expert + cT * cH * 6),
                              ("routed_only_matrix_core_w4a4", w4a4_chain(ids5, w5), uniq * per_expert + cT * cH * 6),
                              ("shared_only_gemv_launchers", shared_part, shared_bytes + cT * cH * 4),
+                             ("shared_only_gemv_launchers_split_k_workspace", shared_part_ws, shared_bytes + cT * cH * 4),
                              ("shared_only", shared_mc, shared_bytes + cT * cH * 4),
                              ("shared_only_w8a8_scaled_matrix_core", shared_w8a8, shared_bytes + cT * cH * 4),
                              ("layer_with_w8a8_shared", full_w8a8, nbytes)):
