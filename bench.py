@@ -468,30 +468,11 @@ def main():
         w5 = torch.empty((cT, cK), dtype=torch.float32, device=dev)
         L.launch_moe_router_select(lg5, lg5, ids5, w5, cfg5, cT, stream)
 
-        # The routed experts in the activation-quantized NVFP4 (W4A4) form, stitched from its launchers: segment, quantize
+        # The routed experts in the activation-quantized NVFP4 (W4A4) form, the layer driver's leg of it: segment, quantize
         # the token rows, grouped gate and up over the row list, SwiGLU + quantize in one launch, grouped down, ordered
         # accumulation over the BF16 down rows. Different numerics from the legs beside it (NVFP4 activations).
-        R = cT * cK
-        rows_l, slot_row = torch.empty(R + cT, dtype=torch.int32, device=dev), torch.empty(R, dtype=torch.int32, device=dev)
-        segs4 = torch.empty((cE + 1, 3), dtype=torch.int32, device=dev)
-        ss_h, ss_i = L.nvfp4_act_scale_stride(cH), L.nvfp4_act_scale_stride(cI)
-        xc, xs_, xg = (torch.empty((cT, cH // 2), dtype=torch.uint8, device=dev), torch.empty((cT, ss_h), dtype=torch.uint8, device=dev),
-                       torch.empty(cT, dtype=torch.float32, device=dev))
-        ac4, as4, ag4 = (torch.empty((R, cI // 2), dtype=torch.uint8, device=dev), torch.empty((R, ss_i), dtype=torch.uint8, device=dev),
-                         torch.empty(R, dtype=torch.float32, device=dev))
-        g4, u4 = (torch.empty((R, cI), dtype=torch.int16, device=dev) for _ in range(2))
-        d4 = torch.empty((R, cH), dtype=torch.int16, device=dev)
-
         def w4a4_chain(ids_t, w_t):
-            def fn(i):
-                L.launch_moe_segment(ids_t, cT, cK, cE, rows_l, slot_row, segs4, stream)
-                L.launch_quantize_rows_nvfp4(x, cH, cT, cH, xc, xs_, xg, stream)
-                L.launch_moe_grouped_w4a4_bf16(xc, xs_, xg, rows_l, segs4, cE, cT, lay.views_ptr, 0, g4, cI, cI, cH, stream)
-                L.launch_moe_grouped_w4a4_bf16(xc, xs_, xg, rows_l, segs4, cE, cT, lay.views_ptr, 1, u4, cI, cI, cH, stream)
-                L.launch_swiglu_quantize_rows_nvfp4(g4, u4, cI, R, cI, float("inf"), ac4, as4, ag4, stream)
-                L.launch_moe_grouped_w4a4_bf16(ac4, as4, ag4, None, segs4, cE, cT, lay.views_ptr, 2, d4, cH, cH, cI, stream)
-                L.launch_moe_accum_ordered_f32_bf16down(routed, d4, cH, slot_row, ids_t, w_t, cT, cK, cH, stream)
-            return fn
+            return lambda i: lay.enqueue_prefill_routed_w4a4(x, cH, ids_t, w_t, None, cT, stream, out_f32=routed)
         if skew:
             # The same layer under Zipf(1.1) expert popularity: few experts take most tokens, so routed segments reach
             # 16 and more rows - the shape the matrix-core grouped form is for. Routes are given (ids drawn from the

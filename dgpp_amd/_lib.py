@@ -208,6 +208,7 @@ LAYER_SIGNATURES = {
     "dgpp_moe_layer_enqueue_decode_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_grouped_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
+    "dgpp_moe_layer_enqueue_prefill_routed_w4a4": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_moe_layer_views": (_P, [_P]),
     "dgpp_moe_layer_ids": (_P, [_P]),
     "dgpp_moe_layer_weights": (_P, [_P]),

@@ -20,7 +20,7 @@ size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 // Buffer sizes in bytes, in the order they are carved (each rounded to 256).
 struct Layout {
   size_t views, ids, weights, scores, biased, order, slot_act, slot_down, acc, counter, rows, slot_row, segs, gather,
-      gate, up, sh_gate, sh_up, sh_act, sh_down, sh_ws, rows_id, ones, total;
+      gate, up, sh_gate, sh_up, sh_act, sh_down, sh_ws, rows_id, ones, q_codes, q_scales, q_gs, total;
 };
 Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t n_views, bool dense_shared) {
   const size_t M = static_cast<size_t>(std::max(max_tokens, 0)), H = c.hidden, K = c.top_k, E = c.n_experts;
@@ -51,9 +51,14 @@ Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t
     l.rows_id = align_up(M * 4);
     l.ones = align_up(M * 4);
   }
+  // The activation-quantized (W4A4) leg's operand rows: the token rows at K = hidden, then the slot rows at K = inter.
+  const size_t qk = std::max(H, static_cast<size_t>(std::max(c.inter, 0)));
+  l.q_codes = align_up(slots * (qk / 2));
+  l.q_scales = align_up(slots * nvfp4_act_scale_stride(static_cast<int>(qk)));
+  l.q_gs = align_up(slots * 4);
   l.total = l.views + l.ids + l.weights + l.scores + l.biased + l.order + l.slot_act + l.slot_down + l.acc + l.counter +
             l.rows + l.slot_row + l.segs + l.gather + l.gate + l.up + l.sh_gate + l.sh_up + l.sh_act + l.sh_down + l.sh_ws +
-            l.rows_id + l.ones;
+            l.rows_id + l.ones + l.q_codes + l.q_scales + l.q_gs;
   return l;
 }
 
@@ -174,6 +179,9 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
     hip_ok(hipMemcpy(d_rows_id_, idv.data(), idv.size() * 4, hipMemcpyHostToDevice), "GlmMoeLayer: row list upload");
     hip_ok(hipMemcpy(d_ones_, onev.data(), onev.size() * 4, hipMemcpyHostToDevice), "GlmMoeLayer: unit weights upload");
   }
+  d_q_codes_ = carve(l.q_codes);
+  d_q_scales_ = carve(l.q_scales);
+  d_q_gs_ = reinterpret_cast<float*>(carve(l.q_gs));
   // The device expert table is uploaded once (the reference's capture form prepares a per-binding
   // device table once too, src/models/glm/moe_layer.cpp:364-396); the counter pair is zero at rest.
   hip_ok(hipMemcpy(d_views_, w.views.data(), w.views.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
@@ -459,6 +467,48 @@ void GlmMoeLayer::enqueue_prefill_routed(const uint16_t* x, size_t x_stride, con
     launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
 }
 
+// The reference's W4A4 prefill chain (src/models/glm/moe_layer.cpp:1122-1135 the token rows' quantizer, :1217-1219
+// gate / up over the routed row list, :1306-1316 SwiGLU inside the second quantizer when no shared segment rides
+// along, :1268-1272 the down projection in bf16 or f32, :690 the accumulation from bf16 down rows).
+void GlmMoeLayer::enqueue_prefill_routed_w4a4(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                                              uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
+                                              const float* act_scales_dev, bool f32_down) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  if (w_.format != GlmExpertFormat::Nvfp4)
+    throw std::invalid_argument("GlmMoeLayer: the activation-quantized path takes NVFP4 experts");
+  if (has_shared())
+    throw std::invalid_argument("GlmMoeLayer: the grouped path here covers the routed experts (no shared segment)");
+  const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter, E = cfg_.n_experts;
+  if (H % 64 != 0 || I % 64 != 0)
+    throw std::invalid_argument("GlmMoeLayer: the activation-quantized path needs hidden and inter in multiples of 64");
+  const int tk = tokens * K;
+  launch_moe_segment(ids, tokens, K, E, d_rows_, d_slot_row_, d_segs_, stream);
+  launch_quantize_rows_nvfp4(x, x_stride, tokens, H, d_q_codes_, d_q_scales_, d_q_gs_, stream, 0.f, act_scales_dev);
+  launch_moe_grouped_w4a4_bf16(d_q_codes_, d_q_scales_, d_q_gs_, d_rows_, d_segs_, E, tokens, d_views_, 0, d_gate_, I, I, H,
+                               stream);
+  launch_moe_grouped_w4a4_bf16(d_q_codes_, d_q_scales_, d_q_gs_, d_rows_, d_segs_, E, tokens, d_views_, 1, d_up_, I, I, H,
+                               stream);
+  launch_swiglu_quantize_rows_nvfp4(d_gate_, d_up_, I, tk, I, cfg_.swiglu_limit, d_q_codes_, d_q_scales_, d_q_gs_, stream, 0.f,
+                                    act_scales_dev ? act_scales_dev + 1 : nullptr);
+  if (f32_down) {
+    launch_moe_grouped_w4a4_f32(d_q_codes_, d_q_scales_, d_q_gs_, nullptr, d_segs_, E, tokens, d_views_, 2, d_slot_down_, H, H,
+                                I, stream);
+    if (out_f32)
+      launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+    else
+      launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+  } else {
+    uint16_t* down = reinterpret_cast<uint16_t*>(d_slot_down_);
+    launch_moe_grouped_w4a4_bf16(d_q_codes_, d_q_scales_, d_q_gs_, nullptr, d_segs_, E, tokens, d_views_, 2, down, H, H, I,
+                                 stream);
+    if (out_f32)
+      launch_moe_accum_ordered_f32_bf16down(out_f32, down, H, d_slot_row_, ids, weights, tokens, K, H, stream);
+    else
+      launch_moe_accum_ordered_bf16down(out_bf16, down, H, d_slot_row_, ids, weights, tokens, K, H, stream);
+  }
+}
+
 }  // namespace dgpp
 
 // ---- C wrappers -------------------------------------------------------------------------------------------
@@ -563,6 +613,14 @@ int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* l, const uint16_t* x, si
                                           void* stream) {
   return guarded([&] {
     l->impl.enqueue_prefill_routed(x, x_stride, ids, weights, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
+  });
+}
+int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                               const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
+                                               void* stream, const float* act_scales_dev, int f32_down) {
+  return guarded([&] {
+    l->impl.enqueue_prefill_routed_w4a4(x, x_stride, ids, weights, out_bf16, out_f32, tokens,
+                                        static_cast<hipStream_t>(stream), act_scales_dev, f32_down != 0);
   });
 }
 const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* l) { return l->impl.views(); }

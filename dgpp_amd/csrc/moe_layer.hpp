@@ -54,6 +54,13 @@ class GlmMoeLayer {
   void enqueue_prefill_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                               uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
 
+  // The activation-quantized (W4A4) form of the same chain for NVFP4 experts: token rows and SwiGLU rows go through the
+  // NVFP4 row quantizer. act_scales_dev: null (a global per row from the row's own maximum) or a DEVICE pair
+  // {token rows' global, SwiGLU rows' global}. The down rows are bf16 unless f32_down.
+  void enqueue_prefill_routed_w4a4(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                                   uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
+                                   const float* act_scales_dev = nullptr, bool f32_down = false);
+
   const MoeExpertView* views() const { return d_views_; }
   const int32_t* ids() const { return d_ids_; }
   const float* weights() const { return d_weights_; }
@@ -98,6 +105,9 @@ class GlmMoeLayer {
   uint16_t* d_gather_ = nullptr;     // [rows_total, hidden]
   uint16_t* d_gate_ = nullptr;       // [rows_total, max_inter]
   uint16_t* d_up_ = nullptr;
+  uint8_t* d_q_codes_ = nullptr;     // W4A4 operand rows: codes [slots, max(hidden, inter) / 2], scale bytes, globals
+  uint8_t* d_q_scales_ = nullptr;
+  float* d_q_gs_ = nullptr;
   // dense shared expert: gate / up / SwiGLU rows [tokens, shared_inter], unrounded down rows [tokens, hidden], the
   // split-K workspace of its projections, and the identity row list / unit weights of the last chain step
   uint16_t* d_sh_gate_ = nullptr;

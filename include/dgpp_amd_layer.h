@@ -77,6 +77,15 @@ int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* layer, const uint16_t* x
 int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, const int32_t* ids,
                                           const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
                                           void* stream);
+/* The activation-quantized (W4A4) form of that chain for NVFP4 experts (src/models/glm/moe_layer.cpp:1122-1135,
+ * 1217-1219, 1268-1272, 1306-1316): token rows -> NVFP4 row quantizer -> grouped W4A4 gate, up over the routed row list
+ * -> SwiGLU inside the second quantizer -> grouped W4A4 down (bf16 rows, or f32 when f32_down is non-zero, the
+ * reference's DGPP_MOE_W4A4_F32_DOWN) -> ordered accumulation. act_scales_dev: null for a global per row, or a
+ * DEVICE pair {token rows' global, SwiGLU rows' global} (the reference's act_scales_dev). hidden and inter must
+ * be multiples of 64. Bitwise the same launchers called one by one. */
+int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, const int32_t* ids,
+                                               const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
+                                               void* stream, const float* act_scales_dev, int f32_down);
 /* Device pointers of the last routes the layer computed: ids int32 [tokens, top_k], weights f32. */
 const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* layer); /* the device expert table */
 const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* layer);

@@ -314,3 +314,74 @@ def test_native_expert_chain_does_not_depend_on_how_rows_are_spread_over_launche
             run(start, min(chunk, rows - start))
         for a, t in zip(first, (out, act, gate, up)):
             assert np.array_equal(a, host(t)), f"chunk {chunk}"
+
+
+@pytest.mark.parametrize("static_gs,f32_down,out_kind", [(False, False, "bf16"), (True, False, "f32"), (False, True, "f32"),
+                                                          (True, True, "bf16")])
+def test_layer_w4a4_leg_is_bitwise_the_launchers_called_one_by_one(gpu, static_gs, f32_down, out_kind):
+    """The layer driver's activation-quantized chain (the reference's W4A4 prefill form,
+    src/models/glm/moe_layer.cpp:1122-1135, 1217-1219, 1268-1272, 1306-1316) gives the bits of the same launchers stitched
+    by hand over buffers of the caller's own, stays within a few per cent of the BF16-activation chain, and refuses
+    a layer whose experts are not NVFP4."""
+    from test_gpu_moe_layer import make_layer
+    E, H, I, K, T = 9, 1024, 192, 3, 27
+    p = moe_data.make_problem(E, H, I, K, T, "nvfp4", 311, shared_kind=None, limit=7.0, std=0.05)
+    d = DeviceMoe(p)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    ids_d, w_d = dev(ids), dev(w)
+    layer = make_layer(p, d, 1, 1.0, T)
+    pair = dev(np.array([2e-3, 1e-2], dtype=np.float32)) if static_gs else None
+    R = T * K
+    out_dtype = np.uint16 if out_kind == "bf16" else np.float32
+    got_d = dev_empty((T, H), out_dtype)
+    kw = {"out_f32": got_d} if out_kind == "f32" else {}
+    layer.enqueue_prefill_routed_w4a4(d.x, H, ids_d, w_d, None if out_kind == "f32" else got_d, T, None,
+                                      act_scales_dev=pair, f32_down=f32_down, **kw)
+    sync()
+    got = host(got_d, out_dtype)
+    # the same chain by hand
+    rows_d, sr_d, segs_d = dev_empty(R + T, np.int32), dev_empty(R, np.int32), dev_empty((E + 1, 3), np.int32)
+    L.launch_moe_segment(ids_d, T, K, E, rows_d, sr_d, segs_d, None)
+    tc, ts, tg = dev_empty((T, H // 2), np.uint8), dev_empty((T, nd.scale_stride(H)), np.uint8), dev_empty(T, np.float32)
+    L.launch_quantize_rows_nvfp4(d.x, H, T, H, tc, ts, tg, None, static_gs_dev=pair)
+    gate, up = dev_empty((R, I), np.uint16), dev_empty((R, I), np.uint16)
+    L.launch_moe_grouped_w4a4_bf16(tc, ts, tg, rows_d, segs_d, E, T, d.views, 0, gate, I, I, H)
+    L.launch_moe_grouped_w4a4_bf16(tc, ts, tg, rows_d, segs_d, E, T, d.views, 1, up, I, I, H)
+    ac, as_, ag = dev_empty((R, I // 2), np.uint8), dev_empty((R, nd.scale_stride(I)), np.uint8), dev_empty(R, np.float32)
+    second = pair[1:] if static_gs else None
+    L.launch_swiglu_quantize_rows_nvfp4(gate, up, I, R, I, 7.0, ac, as_, ag, None, static_gs_dev=second)
+    want_d = dev_empty((T, H), out_dtype)
+    if f32_down:
+        down = dev_empty((R, H), np.float32)
+        L.launch_moe_grouped_w4a4_f32(ac, as_, ag, None, segs_d, E, T, d.views, 2, down, H, H, I)
+        if out_kind == "f32":
+            L.launch_moe_accum_ordered_f32(want_d, down, H, sr_d, ids_d, w_d, -1, T, K, H, None)
+        else:
+            L.launch_moe_accum_ordered(want_d, down, H, sr_d, ids_d, w_d, -1, T, K, H, None)
+    else:
+        down = dev_empty((R, H), np.uint16)
+        L.launch_moe_grouped_w4a4_bf16(ac, as_, ag, None, segs_d, E, T, d.views, 2, down, H, H, I)
+        if out_kind == "f32":
+            L.launch_moe_accum_ordered_f32_bf16down(want_d, down, H, sr_d, ids_d, w_d, T, K, H, None)
+        else:
+            L.launch_moe_accum_ordered_bf16down(want_d, down, H, sr_d, ids_d, w_d, T, K, H, None)
+    sync()
+    assert np.array_equal(got, host(want_d, out_dtype))
+    # distance to the BF16-activation chain over the same routes
+    ref_d = dev_empty((T, H), np.float32)
+    layer.enqueue_prefill_routed(d.x, H, ids_d, w_d, None, T, None, out_f32=ref_d)
+    sync()
+    ref = host(ref_d).astype(np.float64)
+    val = hg.bf16_to_f32(got).astype(np.float64) if out_kind == "bf16" else got.astype(np.float64)
+    rel = float(np.linalg.norm(val - ref) / np.linalg.norm(ref))
+    assert np.isfinite(rel) and rel > 0.0
+    if not static_gs:
+        assert rel < 0.25, rel
+    layer.close()
+    p8 = moe_data.make_problem(4, 512, 128, 2, 8, "fp8", 5, shared_kind=None, limit=7.0, std=0.05)
+    d8 = DeviceMoe(p8)
+    i8, w8, _, _ = moe_data.orc_router(p8, 1, 1.0, True)
+    layer8 = make_layer(p8, d8, 1, 1.0, 8)
+    with pytest.raises(L.InvalidArgument):
+        layer8.enqueue_prefill_routed_w4a4(d8.x, 512, dev(i8), dev(w8), dev_empty((8, 512), np.uint16), 8)
+    layer8.close()
