@@ -196,6 +196,14 @@ class MoeLayerDesc(C.Structure):
     ]
 
 
+class MoeResidentDesc(C.Structure):
+    """include/dgpp_amd_layer.h: DgppMoeResidentDesc."""
+    _fields_ = [
+        ("cfg", MoeConfig), ("max_tokens", C.c_int32), ("rank", C.c_int32), ("world", C.c_int32), ("routed", C.c_void_p),
+        ("shared", C.c_void_p), ("shared_inter", C.c_int64), ("router_weight", C.c_void_p), ("router_bias", C.c_void_p),
+    ]
+
+
 # include/dgpp_amd_layer.h
 LAYER_SIGNATURES = {
     "dgpp_moe_layer_last_error": (C.c_char_p, []),
@@ -209,6 +217,12 @@ LAYER_SIGNATURES = {
     "dgpp_moe_layer_enqueue_grouped_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill_routed_w4a4": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P, _P, _I]),
+    "dgpp_moe_resident_last_error": (C.c_char_p, []),
+    "dgpp_moe_resident_load": (_I, [_P, _P]),
+    "dgpp_moe_resident_destroy": (None, [_P]),
+    "dgpp_moe_resident_layer": (_P, [_P]),
+    "dgpp_moe_resident_weight_bytes": (C.c_size_t, [_P]),
+    "dgpp_moe_resident_inter": (_I, [_P]),
     "dgpp_moe_layer_views": (_P, [_P]),
     "dgpp_moe_layer_ids": (_P, [_P]),
     "dgpp_moe_layer_weights": (_P, [_P]),

@@ -34,7 +34,7 @@ HIP_SOURCES = [
 ]
 HOST_SOURCES = ["host_codec.cpp", "loader.cpp"]
 # Host C++ that needs the HIP runtime headers (compiled by hipcc as plain host code).
-HIP_HOST_SOURCES = ["moe_layer.cpp"]
+HIP_HOST_SOURCES = ["moe_layer.cpp", "moe_resident.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # Packed-FP32 instruction selection is switched off for all device code.

@@ -6,7 +6,7 @@ from __future__ import annotations
 import ctypes as C
 
 from . import _lib
-from ._lib import MoeConfig, MoeExpertView, MoeLayerDesc
+from ._lib import MoeConfig, MoeExpertView, MoeLayerDesc, MoeResidentDesc
 from .launch import InvalidArgument, _p, _stream
 
 EXPERTS_FP8, EXPERTS_NVFP4, EXPERTS_MXFP4 = 0, 1, 2
@@ -101,3 +101,43 @@ class MoeLayer:
     @property
     def weights_ptr(self) -> int:
         return self._lib.dgpp_moe_layer_weights(self._h)
+
+
+class ResidentMoeLayer(MoeLayer):
+    """A layer made resident from what a loader.*_moe_bind_layer call found: this rank's slices of the expert matrices
+    (gate / up rows [rank * inter / world, ...), the matching columns of down) are uploaded into one device allocation
+    that the object owns together with the layer driver over it. The shards must be open during construction only."""
+
+    def __init__(self, cfg: MoeConfig, max_tokens: int, routed, *, shared=None, shared_inter: int = 0, router_weight=None,
+                 router_bias=None, rank: int = 0, world: int = 1):
+        from .loader import MoeMatrixTensors
+        self._lib = _lib.load()
+        flat = [m for expert in routed for m in expert]
+        r_arr = (MoeMatrixTensors * len(flat))(*flat)
+        s_arr = (MoeMatrixTensors * 3)(*shared) if shared else None
+        d = MoeResidentDesc()
+        d.cfg = cfg
+        d.max_tokens, d.rank, d.world = max_tokens, rank, world
+        d.routed = C.addressof(r_arr)
+        d.shared = C.addressof(s_arr) if s_arr is not None else None
+        d.shared_inter = shared_inter if shared else 0
+        d.router_weight = C.addressof(router_weight) if router_weight is not None else None
+        d.router_bias = C.addressof(router_bias) if router_bias is not None else None
+        handle = C.c_void_p()
+        rc = self._lib.dgpp_moe_resident_load(C.addressof(d), C.addressof(handle))
+        if rc != 0:
+            msg = self._lib.dgpp_moe_resident_last_error().decode()
+            raise InvalidArgument(msg) if rc == 1 else RuntimeError(msg)
+        self._resident = handle
+        self._h = C.c_void_p(self._lib.dgpp_moe_resident_layer(handle))
+        self.cfg = cfg
+        self.weight_bytes = self._lib.dgpp_moe_resident_weight_bytes(handle)
+        self.inter = self._lib.dgpp_moe_resident_inter(handle)
+
+    def close(self):
+        if getattr(self, "_resident", None):
+            self._lib.dgpp_moe_resident_destroy(self._resident)   # the layer goes with it
+            self._resident = None
+            self._h = None
+
+    __del__ = close

@@ -10,6 +10,7 @@
 #define DGPP_AMD_LAYER_H
 
 #include "dgpp_amd.h"
+#include "dgpp_amd_loader.h"
 
 #ifdef __cplusplus
 extern "C" {
@@ -90,6 +91,33 @@ int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* layer, const uint16
 const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* layer); /* the device expert table */
 const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* layer);
 const float* dgpp_moe_layer_weights(const DgppMoeLayer* layer);
+
+/* ---- a bound layer made resident in one call -----------------------------------------------------------------
+ * Reference: the resident build of a MoE layer, src/models/glm/loader.cpp:418-471 (router, shared expert, every
+ * routed expert cut to the rank's slice of the intermediate dimension, NVFP4 globals gathered into one array), with
+ * the slicing rules of src/models/quant_matrix.hpp:67-96 (block-FP8 grids re-blocked at gcd(128, start, count)) and
+ * :140-164 (FP4 column slices on scale-group boundaries). Takes what a dgpp_*_moe_bind_layer call found (host
+ * addresses inside the mapped shards, which must stay open during the call), uploads this rank's slices into ONE
+ * device allocation and creates the layer driver over them. Not a launcher: it allocates, copies and synchronizes. */
+typedef struct DgppMoeResident DgppMoeResident;
+typedef struct DgppMoeResidentDesc {
+  DgppMoeConfig cfg;                    /* the checkpoint's (unsliced) geometry */
+  int32_t max_tokens;
+  int32_t rank, world;                  /* gate / up rows [rank * inter / world, ...), the matching columns of down */
+  const DgppMoeMatrixTensors* routed;   /* [n_experts * 3] gate, up, down: block FP8 (F32 or BF16 grid), NVFP4 in its three
+                                           spellings, or MXFP4 */
+  const DgppMoeMatrixTensors* shared;   /* [3] or null: block FP8 (slot top_k of every token), the routed experts' FP4
+                                           format and width (a table entry), or MXFP8 (dense projections of its own width) */
+  int64_t shared_inter;                 /* the shared expert's unsliced width (0: none) */
+  const DgppTensorInfo* router_weight;  /* BF16 [n_experts, hidden], or null */
+  const DgppTensorInfo* router_bias;    /* F32 or BF16 [n_experts], or null */
+} DgppMoeResidentDesc;
+const char* dgpp_moe_resident_last_error(void);
+int dgpp_moe_resident_load(const DgppMoeResidentDesc* desc, DgppMoeResident** out);
+void dgpp_moe_resident_destroy(DgppMoeResident* resident);   /* the layer and the weights */
+DgppMoeLayer* dgpp_moe_resident_layer(DgppMoeResident* resident);           /* owned by the resident */
+size_t dgpp_moe_resident_weight_bytes(const DgppMoeResident* resident);     /* device bytes of the weights' allocation */
+int dgpp_moe_resident_inter(const DgppMoeResident* resident);               /* the rank's expert width, inter / world */
 
 #ifdef __cplusplus
 }

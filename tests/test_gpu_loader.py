@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import moe_data
-from dgpp_amd import _lib, launch as L, loader as LD, moe_layer as ML
+from dgpp_amd import _lib, hostgen as hg, launch as L, loader as LD, moe_layer as ML
 from gpu_util import DeviceMoe, dev, dev_empty, host, sync, view_table
 from test_gpu_moe_layer import make_layer
 
@@ -23,7 +23,7 @@ def write_checkpoint(path, tensors, dtypes=None):
     """A safetensors file from numpy arrays (header JSON + payload, 8-byte padded header)."""
     header, payload, at = {}, [], 0
     for name, a in tensors.items():
-        a = np.ascontiguousarray(a)
+        a = np.asarray(a, order="C")   # keeps a scalar tensor's empty shape
         dt = (dtypes or {}).get(name, _DT[a.dtype])
         header[name] = {"dtype": dt, "shape": list(a.shape), "data_offsets": [at, at + a.nbytes]}
         payload.append(a.tobytes())
@@ -236,3 +236,161 @@ def test_layer_bound_by_the_glm_tensor_names_is_bitwise_the_layer_from_the_array
     assert host(want, np.uint16).any()
     ref_layer.close()
     got_layer.close()
+
+
+def _checkpoint_tensors(p, family):
+    """The problem's tensors under a model family's names: 'glm' (block FP8 or NVFP4 in the engine's own spelling, the
+    shared expert block FP8), 'mimo' (MXFP4), 'minimax' (compressed-tensors NVFP4, MXFP8 shared expert)."""
+    tensors, dtypes = {}, {}
+    if family == "glm":
+        pre = "model.layers.3."
+        tensors[pre + "mlp.gate.weight"], dtypes[pre + "mlp.gate.weight"] = p.router_gate, "BF16"
+        tensors[pre + "mlp.gate.e_score_correction_bias"] = p.router_bias
+
+        def put(base, m):
+            if m.kind == "fp8":
+                tensors[base], dtypes[base] = m.payload, "F8_E4M3"
+                tensors[base + "_scale_inv"] = m.scales
+            else:
+                tensors[base + "_packed"] = m.payload
+                tensors[base + "_scale"], dtypes[base + "_scale"] = m.scales, "F8_E4M3"
+                tensors[base + "_global_scale"] = m.glob
+        for e, mats in enumerate(p.experts):
+            for m, proj in zip(mats, PROJ):
+                put(f"{pre}mlp.experts.{e}.{proj}.weight", m)
+        if p.shared:
+            for m, proj in zip(p.shared, PROJ):
+                put(f"{pre}mlp.shared_experts.{proj}.weight", m)
+        return pre, tensors, dtypes
+    if family == "mimo":
+        pre = "model.layers.2.mlp."
+        tensors[pre + "gate.weight"], dtypes[pre + "gate.weight"] = p.router_gate, "BF16"
+        tensors[pre + "gate.e_score_correction_bias"] = p.router_bias
+        for e, mats in enumerate(p.experts):
+            for m, proj in zip(mats, PROJ):
+                tensors[f"{pre}experts.{e}.{proj}.weight"] = m.payload
+                tensors[f"{pre}experts.{e}.{proj}.weight_scale"] = m.scales
+        return pre, tensors, dtypes
+    pre = "language_model.model.layers.4.block_sparse_moe."
+    tensors[pre + "gate.weight"] = hg.bf16_to_f32(p.router_gate)
+    tensors[pre + "e_score_correction_bias"] = p.router_bias
+    for e, mats in enumerate(p.experts):
+        for m, w in zip(mats, ("w1", "w3", "w2")):
+            tensors[f"{pre}experts.{e}.{w}.weight_packed"] = m.payload
+            tensors[f"{pre}experts.{e}.{w}.weight_scale"], dtypes[f"{pre}experts.{e}.{w}.weight_scale"] = m.scales, "F8_E4M3"
+            tensors[f"{pre}experts.{e}.{w}.weight_global_scale"] = np.float32(m.glob[0])
+    if p.shared:
+        for m, proj in zip(p.shared, PROJ):
+            base = f"{pre}shared_experts.{proj}.weight"
+            tensors[base], dtypes[base] = m.payload, "F8_E4M3"
+            tensors[base + "_scale_inv"] = m.scales
+    return pre, tensors, dtypes
+
+
+RESIDENT_CASES = [
+    # family, kind, shared kind, E, H, I, shared I, K, T, world
+    ("glm", "fp8", "fp8", 8, 512, 128, 256, 2, 3, 1),
+    ("glm", "fp8", "fp8", 6, 512, 256, 256, 2, 4, 2),       # slices of 128: views of the grid as it is
+    ("glm", "fp8", None, 8, 512, 384, 0, 2, 3, 2),          # slices of 192: rank 1's grids re-blocked at 64
+    ("glm", "nvfp4", None, 8, 512, 256, 0, 4, 5, 2),
+    ("mimo", "mxfp4", None, 12, 1024, 512, 0, 8, 6, 4),
+    ("minimax", "nvfp4", "mxfp8", 6, 512, 128, 192, 2, 5, 1),
+    ("minimax", "nvfp4", "mxfp8", 6, 512, 128, 192, 2, 5, 2),
+]
+
+
+@pytest.mark.parametrize("family,kind,shared,E,H,I,sI,K,T,world", RESIDENT_CASES)
+def test_resident_layer_from_a_bound_checkpoint_is_bitwise_the_hand_sliced_layer(gpu, tmp_path, family, kind, shared, E, H, I, sI,
+                                                                                 K, T, world):
+    """One call from a family's binding to a layer on the device (the reference's resident build of a MoE layer,
+    src/models/glm/loader.cpp:418-471): every rank's layer gives the bits of the layer built by hand from the same
+    slices (rows of gate / up, columns of down, cut with the loader's slice functions and uploaded one by one)."""
+    from test_gpu_moe_tp_slices import cols_slice, rows_slice
+    p = moe_data.make_problem(E, H, I, K, T, kind, 7100 + E + world, shared_kind=shared, shared_I=sI or None, limit=7.0, std=0.05)
+    pre, tensors, dtypes = _checkpoint_tensors(p, family)
+    names = sorted(tensors)
+    paths = []
+    for i in range(2):
+        paths.append(str(tmp_path / f"model-0000{i + 1}-of-00002.safetensors"))
+        write_checkpoint(paths[-1], {n: np.asarray(tensors[n]) for n in names[i::2]}, dtypes)
+    mode = 0
+    cfg = L.make_config(H, I, E, K, n_shared_experts=1 if shared else 0, routed_scaling_factor=2.5, swiglu_limit=p.limit, router_mode=mode)
+    files = [LD.SafetensorsFile(x) for x in paths]
+    layers = []
+    try:
+        if family == "glm":
+            rw, rb, sh, routed = LD.glm_moe_bind_layer(files, pre, E, H, I, LD.BIND_FP8 if kind == "fp8" else LD.BIND_NVFP4, sI)
+        elif family == "mimo":
+            (rw, rb, routed), sh = LD.mimo_moe_bind_layer(files, pre, E, H, I), None
+        else:
+            rw, rb, sh, routed = LD.minimax_moe_bind_layer(files, pre, E, H, I, sI)
+            rw = None   # this family's router weight is F32: the scores come from the caller
+        for r in range(world):
+            layers.append(ML.ResidentMoeLayer(cfg, T, routed, shared=sh, shared_inter=sI, router_weight=rw, router_bias=rb,
+                                              rank=r, world=world))
+        with pytest.raises(L.InvalidArgument):
+            ML.ResidentMoeLayer(cfg, T, routed, shared=sh, shared_inter=sI, router_weight=rw, router_bias=rb, rank=world, world=world)
+        with pytest.raises(L.InvalidArgument):
+            ML.ResidentMoeLayer(cfg, T, routed, shared=sh, shared_inter=sI, rank=0, world=7)
+    finally:
+        for f in files:
+            f.close()   # the resident layers own device copies: the shards may go
+    ids, w, _, _ = moe_data.orc_router(p, mode, 2.5, True)
+    ids_d, w_d, x_d = dev(ids), dev(w), dev(p.x)
+    M, SM = I // world, (sI // world if shared else 0)
+    for r, layer in enumerate(layers):
+        assert layer.inter == M and layer.weight_bytes > 0
+        q = moe_data.MoeProblem(E, H, M, K, T, kind, shared, SM, limit=p.limit)
+        q.x, q.router_gate, q.router_bias = p.x, p.router_gate, p.router_bias
+
+        def rows(m, width):
+            if world == 1:
+                return m
+            if m.kind == "fp8" and (r * width) % 128 != 0:
+                whole = LD.QuantMatrix(m.payload.ctypes.data, m.scales.ctypes.data, None, m.rows, m.cols, 128, 128)
+                payload, scales, v = LD.quant_slice(whole, 0, r * width, width)
+                ok, rs, cs = LD.quant_scale_shifts(v)
+                assert ok
+                return moe_data.Mat("fp8", width, m.cols, payload, scales, rs=rs, cs=cs)
+            if m.kind == "mxfp8":
+                return moe_data.Mat("mxfp8", width, m.cols, np.ascontiguousarray(m.payload[r * width:(r + 1) * width]),
+                                    np.ascontiguousarray(m.scales[r * width:(r + 1) * width]), rs=0, cs=5)
+            return rows_slice(m, r * width, width)
+
+        def cols(m, width):
+            if world == 1:
+                return m
+            if m.kind == "mxfp8":
+                c0 = r * width
+                return moe_data.Mat("mxfp8", m.rows, width, np.ascontiguousarray(m.payload[:, c0:c0 + width]),
+                                    np.ascontiguousarray(m.scales[:, c0 // 32:(c0 + width) // 32]), rs=0, cs=5)
+            return cols_slice(m, r * width, width)
+        for g, u, dn in p.experts:
+            q.experts.append([rows(g, M), rows(u, M), cols(dn, M)])
+        out_r, out_h = dev_empty((T, H), np.uint16), dev_empty((T, H), np.uint16)
+        if shared == "mxfp8":
+            q.shared = [rows(p.shared[0], SM), rows(p.shared[1], SM), cols(p.shared[2], SM)]
+            d = DeviceMoe(moe_data.MoeProblem(E, H, M, K, T, kind, None, M, experts=q.experts, x=p.x, limit=p.limit))
+            views = list((L.MoeExpertView * (d.views.numel() // 96)).from_buffer_copy(bytes(host(d.views))))
+            shd = [(dev(m.payload), dev(m.scales)) for m in q.shared]
+            cfg_r = L.make_config(H, M, E, K, n_shared_experts=1, routed_scaling_factor=2.5, swiglu_limit=p.limit, router_mode=mode)
+            hand = ML.MoeLayer(cfg_r, ML.EXPERTS_NVFP4, views, T, shared_inter=SM, sh_payload=[t[0] for t in shd],
+                               sh_scales_e8m0=[t[1] for t in shd])
+        else:
+            if shared:
+                q.shared = [rows(p.shared[0], SM), rows(p.shared[1], SM), cols(p.shared[2], SM)]
+            d = DeviceMoe(q)
+            hand = make_layer(q, d, mode, 2.5, T)
+        hand.enqueue_decode_routed(x_d, H, ids_d, w_d, out_h, T)
+        layer.enqueue_decode_routed(x_d, H, ids_d, w_d, out_r, T)
+        sync()
+        assert np.array_equal(host(out_r, np.uint16), host(out_h, np.uint16)), f"rank {r}"
+        assert host(out_h, np.uint16).any()
+        if family != "minimax":   # the router came along: the whole step from the hidden rows
+            out_r.zero_()
+            hand.enqueue_decode(x_d, H, out_h, T)
+            layer.enqueue_decode(x_d, H, out_r, T)
+            sync()
+            assert np.array_equal(host(out_r, np.uint16), host(out_h, np.uint16)), f"rank {r}: with the router"
+        hand.close()
+        layer.close()

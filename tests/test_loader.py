@@ -365,6 +365,15 @@ def test_glm_moe_layer_binding_finds_every_tensor_across_shards(tmp_path, fmt):
         # no shared expert, no bias: nothing of them is looked up
         rw2, rb2, sh2, routed2 = LD.glm_moe_bind_layer(files, prefix, E, H, I, fmt, 0, with_bias=False)
         assert rb2 is None and sh2 is None and len(routed2) == E
+        # the resident build refuses what it cannot slice before it touches a device
+        from dgpp_amd import launch as L, moe_layer as ML
+        cfg = L.make_config(H, I, E, 2, n_shared_experts=1)
+        for kw, text in ((dict(rank=2, world=2), "rank must lie"), (dict(rank=0, world=3), "must divide by world"),
+                         (dict(rank=0, world=32), "re-block" if fmt == LD.BIND_FP8 else "whole scale groups")):
+            with pytest.raises(L.InvalidArgument, match=text):
+                ML.ResidentMoeLayer(cfg, 4, routed, shared=shared, shared_inter=S, router_weight=rw, router_bias=rb, **kw)
+        with pytest.raises(L.InvalidArgument, match="does not have the layer's geometry"):
+            ML.ResidentMoeLayer(L.make_config(H, I * 2, E, 2), 4, routed)
     finally:
         for f in files:
             f.close()
