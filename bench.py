@@ -550,6 +550,9 @@ def main():
         def full(i):
             lay1.enqueue_decode_scores(x, cH, lg5, lg5, out, cT, stream)
 
+        def full_mc(i):   # the same layer through the driver's matrix-core grouped path (routes given)
+            lay1.enqueue_prefill_routed(x, cH, ids5, w5, out, cT, stream)
+
         def full_w8a8(i):
             routed_part(i)
             shared_w8a8(i)
@@ -561,7 +564,8 @@ def main():
         res = {"workload": f"C5 NVFP4 routed MoE (256 experts, hidden 6144, inter 2048, top-8, {uniq} distinct; decode slots) "
                            f"+ MXFP8 shared expert (inter 4096, dense projections: launch_scale_gemm_grid_e8m0_*, the matrix-core form at 64 rows) as ONE layer-driver call, T=64; routed expert weights = device copies of {G} generated experts",
                "algorithmic_bytes": nbytes}
-        for name, fn, nb in (("layer", full, nbytes), ("layer_stitched_from_launchers", stitched, nbytes),
+        for name, fn, nb in (("layer", full, nbytes), ("layer_matrix_core", full_mc, nbytes),
+                             ("layer_stitched_from_launchers", stitched, nbytes),
                              ("routed_only", routed_part, uniq * per_expert + cT * cH * 6),
                              ("routed_only_matrix_core", routed_mc, uniq * per_expert + cT * cH * 6),
                              ("routed_only_matrix_core_w4a4", w4a4_chain(ids5, w5), uniq * per_expert + cT * cH * 6),

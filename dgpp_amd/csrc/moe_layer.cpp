@@ -20,7 +20,7 @@ size_t align_up(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
 // Buffer sizes in bytes, in the order they are carved (each rounded to 256).
 struct Layout {
   size_t views, ids, weights, scores, biased, order, slot_act, slot_down, acc, counter, rows, slot_row, segs, gather,
-      gate, up, sh_gate, sh_up, sh_act, sh_down, sh_ws, rows_id, ones, q_codes, q_scales, q_gs, total;
+      gate, up, sh_gate, sh_up, sh_act, sh_down, sh_ws, rows_id, ones, q_codes, q_scales, q_gs, sh_views, total;
 };
 Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t n_views, bool dense_shared) {
   const size_t M = static_cast<size_t>(std::max(max_tokens, 0)), H = c.hidden, K = c.top_k, E = c.n_experts;
@@ -56,9 +56,12 @@ Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t
   l.q_codes = align_up(slots * (qk / 2));
   l.q_scales = align_up(slots * nvfp4_act_scale_stride(static_cast<int>(qk)));
   l.q_gs = align_up(slots * 4);
+  // A block-FP8 shared expert handed over by pointers, as the table entries the grouped launchers read (its segment
+  // names expert n_experts).
+  l.sh_views = align_up((E + 1) * 3 * sizeof(MoeExpertView));
   l.total = l.views + l.ids + l.weights + l.scores + l.biased + l.order + l.slot_act + l.slot_down + l.acc + l.counter +
             l.rows + l.slot_row + l.segs + l.gather + l.gate + l.up + l.sh_gate + l.sh_up + l.sh_act + l.sh_down + l.sh_ws +
-            l.rows_id + l.ones + l.q_codes + l.q_scales + l.q_gs;
+            l.rows_id + l.ones + l.q_codes + l.q_scales + l.q_gs + l.sh_views;
   return l;
 }
 
@@ -182,6 +185,20 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   d_q_codes_ = carve(l.q_codes);
   d_q_scales_ = carve(l.q_scales);
   d_q_gs_ = reinterpret_cast<float*>(carve(l.q_gs));
+  d_sh_views_ = reinterpret_cast<MoeExpertView*>(carve(l.sh_views));
+  if (w.shared_inter > 0 && !w.shared_in_table && !e8m0_shared) {
+    std::vector<MoeExpertView> table((E + 1) * 3);
+    for (int i = 0; i < 3; ++i) {
+      MoeExpertView& v = table[E * 3 + static_cast<size_t>(i)];
+      v.payload = w.sh_payload[i];
+      v.scales = w.sh_scales[i];
+      v.scale_shift_rows = w.sh_rs;
+      v.scale_shift_cols = w.sh_cs;
+      v.fp4_group = kFp4Group;
+    }
+    hip_ok(hipMemcpy(d_sh_views_, table.data(), table.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
+           "GlmMoeLayer: shared table upload");
+  }
   // The device expert table is uploaded once (the reference's capture form prepares a per-binding
   // device table once too, src/models/glm/moe_layer.cpp:364-396); the counter pair is zero at rest.
   hip_ok(hipMemcpy(d_views_, w.views.data(), w.views.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
@@ -443,28 +460,60 @@ void GlmMoeLayer::enqueue_prefill_routed(const uint16_t* x, size_t x_stride, con
                                          uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream) {
   if (tokens <= 0) return;
   check_tokens(tokens);
-  if (has_shared())
-    throw std::invalid_argument("GlmMoeLayer: the grouped path here covers the routed experts (no shared segment)");
+  if (out_bf16 == nullptr && out_f32 == nullptr) throw std::invalid_argument("GlmMoeLayer: no output buffer");
+  if (dense_shared()) {
+    const int H = cfg_.hidden;
+    // As in the decode chain: the routed rows unrounded, the shared expert's dense projections beside them on the
+    // side stream, then a = fma(1, shared, a) and the one rounding.
+    float* acc = out_f32 ? out_f32 : d_acc_;
+    StreamFork fork{stream, side_, fork_, join_};
+    fork.begin();
+    dense_shared_chain(x, x_stride, tokens, side_);
+    prefill_chain(x, x_stride, ids, weights, nullptr, acc, tokens, stream, /*with_shared=*/false);
+    fork.end();
+    launch_moe_accum(acc, d_sh_down_, d_rows_id_, d_ones_, tokens, H, stream);
+    if (!out_f32) launch_moe_round_bf16(out_bf16, acc, static_cast<int64_t>(tokens) * H, stream);
+    return;
+  }
+  prefill_chain(x, x_stride, ids, weights, out_bf16, out_f32, tokens, stream, has_shared());
+}
+
+// Segments -> gate + up + SwiGLU -> down -> ordered accumulation on the matrix core. with_shared: the shared expert
+// is segment n_experts (every token, in token order, rows [tokens * top_k, ...) of the slot buffers; the reference's
+// shared_seg, src/models/glm/moe_layer.cpp:1293-1296, 1335-1336) and ends every token's chain with weight 1.
+void GlmMoeLayer::prefill_chain(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
+                                uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream, bool with_shared) {
   const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter, E = cfg_.n_experts;
   const int tk = tokens * K;
+  const bool fp8 = w_.format == GlmExpertFormat::Fp8;
+  const bool in_table = with_shared && w_.shared_in_table;   // the routed experts' format and width: one more segment
+  const size_t stride = with_shared ? static_cast<size_t>(max_inter_) : static_cast<size_t>(I);
+  const int n_segs = in_table ? E + 1 : E;
   launch_moe_segment(ids, tokens, K, E, d_rows_, d_slot_row_, d_segs_, stream);
   const int max_rows = tokens;
   // gate + up + SwiGLU in one launch (the bits of the two grouped launches and the elementwise kernel)
-  if (w_.format == GlmExpertFormat::Fp8)
-    launch_moe_grouped_mma_gate_up_swiglu(x, x_stride, d_segs_, E, max_rows, 0, d_views_, d_slot_act_, I, I, H,
+  if (fp8)
+    launch_moe_grouped_mma_gate_up_swiglu(x, x_stride, d_segs_, n_segs, max_rows, 0, d_views_, d_slot_act_, stride, I, H,
                                           cfg_.swiglu_limit, stream, d_rows_);
   else
-    launch_moe_grouped_mma_gate_up_swiglu_fp4(x, x_stride, d_segs_, E, max_rows, 0, d_views_, d_slot_act_, I, I, H,
+    launch_moe_grouped_mma_gate_up_swiglu_fp4(x, x_stride, d_segs_, n_segs, max_rows, 0, d_views_, d_slot_act_, stride, I, H,
                                               cfg_.swiglu_limit, stream, d_rows_, fp4_group_);
-  if (w_.format == GlmExpertFormat::Fp8)
-    launch_moe_grouped_mma_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream);
+  if (with_shared && !in_table)   // a block-FP8 shared expert of its own width
+    launch_moe_grouped_mma_gate_up_swiglu(x, x_stride, d_segs_ + E, 1, max_rows, 0, d_sh_views_, d_slot_act_, stride,
+                                          w_.shared_inter, H, cfg_.swiglu_limit, stream, d_rows_);
+  if (fp8)
+    launch_moe_grouped_mma_f32(d_slot_act_, stride, d_segs_, n_segs, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream);
   else
-    launch_moe_grouped_mma_fp4_f32(d_slot_act_, I, d_segs_, E, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream,
+    launch_moe_grouped_mma_fp4_f32(d_slot_act_, stride, d_segs_, n_segs, max_rows, 0, d_views_, 2, d_slot_down_, H, H, I, stream,
                                    nullptr, fp4_group_);
+  if (with_shared && !in_table)
+    launch_moe_grouped_mma_f32(d_slot_act_, stride, d_segs_ + E, 1, max_rows, 0, d_sh_views_, 2, d_slot_down_, H, H,
+                               w_.shared_inter, stream);
+  const int shared_row0 = with_shared ? tk : -1;
   if (out_f32)
-    launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+    launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, shared_row0, tokens, K, H, stream);
   else
-    launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+    launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, shared_row0, tokens, K, H, stream);
 }
 
 // The reference's W4A4 prefill chain (src/models/glm/moe_layer.cpp:1122-1135 the token rows' quantizer, :1217-1219

@@ -50,7 +50,8 @@ class GlmMoeLayer {
                              uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
   void enqueue_grouped_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                               uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
-  // The same through the matrix-core grouped launchers (gather folded in, 16 token rows per weight pass).
+  // The same through the matrix-core grouped launchers (gather folded in, 16 token rows per weight pass); a layer's
+  // shared expert rides along as the segment of every token (or as dense projections beside, the MXFP8 form).
   void enqueue_prefill_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                               uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
 
@@ -73,6 +74,8 @@ class GlmMoeLayer {
   void check_tokens(int tokens) const;
   bool needs_order(int tokens) const;
   void dense_shared_chain(const uint16_t* x, size_t x_stride, int tokens, hipStream_t stream);
+  void prefill_chain(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights, uint16_t* out_bf16,
+                     float* out_f32, int tokens, hipStream_t stream, bool with_shared);
   void expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                           uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
                           bool order_ready = false, const float* sel_scores = nullptr, const float* sel_biased = nullptr,
@@ -108,6 +111,7 @@ class GlmMoeLayer {
   uint8_t* d_q_codes_ = nullptr;     // W4A4 operand rows: codes [slots, max(hidden, inter) / 2], scale bytes, globals
   uint8_t* d_q_scales_ = nullptr;
   float* d_q_gs_ = nullptr;
+  MoeExpertView* d_sh_views_ = nullptr;   // [(n_experts + 1) * 3]: a block-FP8 shared expert as segment n_experts' entries
   // dense shared expert: gate / up / SwiGLU rows [tokens, shared_inter], unrounded down rows [tokens, hidden], the
   // split-K workspace of its projections, and the identity row list / unit weights of the last chain step
   uint16_t* d_sh_gate_ = nullptr;

@@ -74,7 +74,10 @@ int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* layer, const uint16_t* x
                                           const int32_t* ids, const float* weights, uint16_t* out_bf16,
                                           float* out_f32, int tokens, void* stream);
 /* The grouped path through the matrix-core launchers (the reference's prefill form,
- * src/models/glm/moe_layer.cpp:775-817): gather folded into the gate / up launches. */
+ * src/models/glm/moe_layer.cpp:775-817): gather folded into the gate / up launches. A layer's shared expert rides
+ * along as the segment of every token behind the routed rows (:1293-1296, 1335-1336; a table entry joins the routed
+ * launches, a block-FP8 one of its own width takes a launch of its own per projection) and ends every token's chain
+ * with weight 1; the dense MXFP8 form runs beside the routed chain as in the decode path. */
 int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, const int32_t* ids,
                                           const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
                                           void* stream);

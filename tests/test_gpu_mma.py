@@ -319,3 +319,45 @@ def test_fp8_pair_launch_is_bitwise_the_two_single_launches(gpu, m, n0, n1, k, w
         g = host(outs[i], np.uint16)
         assert np.array_equal(g, host(want[i], np.uint16)), f"problem {i}"
         check(np.ascontiguousarray(g[:, :n]), orc.gemv_fp8(acts[i], mats[i][0], mats[i][1], m, n, k, 7, 7, True), f"pair problem {i}")
+
+
+@pytest.mark.parametrize("kind,shared,sI", [("fp8", "fp8", 384), ("nvfp4", "fp8", 128), ("nvfp4", "nvfp4", 256),
+                                            ("mxfp4", "mxfp4", 256), ("nvfp4", "mxfp8", 192)])
+def test_prefill_path_with_a_shared_expert(gpu, kind, shared, sI):
+    """The layer's matrix-core grouped path with the shared expert riding along (the reference's shared_seg,
+    src/models/glm/moe_layer.cpp:1293-1296, 1335-1336): a table entry joins the routed launches as segment n_experts, a
+    block-FP8 expert of its own width takes its own launches, the MXFP8 form runs as dense projections beside. Held to
+    the oracle's layer budget, and bitwise the decode-slot chain of the same layer with its kernels on the matrix core."""
+    from dgpp_amd import moe_layer as ML
+    from test_gpu_moe_layer import make_layer
+    from test_gpu_moe_slots import expert_budget
+    E, H, I, K, T = 10, 1024, 256, 4, 19
+    p = moe_data.make_problem(E, H, I, K, T, kind, 91, shared_kind=shared, shared_I=sI, limit=7.0, std=0.05)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    if shared == "mxfp8":
+        routed_only = moe_data.MoeProblem(E, H, I, K, T, kind, None, I, experts=p.experts, x=p.x, limit=p.limit)
+        d = DeviceMoe(routed_only)
+        views = list((L.MoeExpertView * (d.views.numel() // 96)).from_buffer_copy(bytes(host(d.views))))
+        shd = [(dev(m.payload), dev(m.scales)) for m in p.shared]
+        cfg = L.make_config(H, I, E, K, n_shared_experts=1, routed_scaling_factor=1.0, swiglu_limit=p.limit, router_mode=1)
+        layer = ML.MoeLayer(cfg, ML.EXPERTS_NVFP4, views, T, shared_inter=sI, sh_payload=[t[0] for t in shd],
+                            sh_scales_e8m0=[t[1] for t in shd])
+    else:
+        d = DeviceMoe(p)
+        layer = make_layer(p, d, 1, 1.0, T)
+    ids_d, w_d = dev(ids), dev(w)
+    out, out2 = dev_empty((T, H), np.uint16), dev_empty((T, H), np.uint16)
+    layer.enqueue_prefill_routed(d.x, H, ids_d, w_d, out, T)
+    sync()
+    got = host(out, np.uint16)
+    raw, _ = moe_data.orc_forward(p, ids, w)
+    expert_budget(got, raw, f"prefill {kind} + shared {shared}")
+    lib = _lib.load()
+    lib.dgpp_tune_set(5, 2)
+    try:
+        layer.enqueue_decode_routed(d.x, H, ids_d, w_d, out2, T)
+        sync()
+    finally:
+        lib.dgpp_tune_set(5, 0)
+    assert np.array_equal(host(out2, np.uint16), got), "decode-slot chain on the matrix core == grouped matrix-core path, bitwise"
+    layer.close()
