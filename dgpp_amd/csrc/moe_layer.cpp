@@ -524,14 +524,22 @@ void GlmMoeLayer::enqueue_prefill_routed_w4a4(const uint16_t* x, size_t x_stride
                                               const float* act_scales_dev, bool f32_down) {
   if (tokens <= 0) return;
   check_tokens(tokens);
+  if (out_bf16 == nullptr && out_f32 == nullptr) throw std::invalid_argument("GlmMoeLayer: no output buffer");
   if (w_.format != GlmExpertFormat::Nvfp4)
     throw std::invalid_argument("GlmMoeLayer: the activation-quantized path takes NVFP4 experts");
-  if (has_shared())
-    throw std::invalid_argument("GlmMoeLayer: the grouped path here covers the routed experts (no shared segment)");
   const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter, E = cfg_.n_experts;
   if (H % 64 != 0 || I % 64 != 0)
     throw std::invalid_argument("GlmMoeLayer: the activation-quantized path needs hidden and inter in multiples of 64");
   const int tk = tokens * K;
+  const bool dense = dense_shared();
+  const bool seg_shared = has_shared() && !dense;   // the shared expert's rows keep BF16 activations behind the routed rows
+  float* acc = dense ? (out_f32 ? out_f32 : d_acc_) : out_f32;
+  uint16_t* rounded = dense ? nullptr : out_bf16;
+  StreamFork fork{stream, side_, fork_, join_};
+  if (dense) {
+    fork.begin();
+    dense_shared_chain(x, x_stride, tokens, side_);
+  }
   launch_moe_segment(ids, tokens, K, E, d_rows_, d_slot_row_, d_segs_, stream);
   launch_quantize_rows_nvfp4(x, x_stride, tokens, H, d_q_codes_, d_q_scales_, d_q_gs_, stream, 0.f, act_scales_dev);
   launch_moe_grouped_w4a4_bf16(d_q_codes_, d_q_scales_, d_q_gs_, d_rows_, d_segs_, E, tokens, d_views_, 0, d_gate_, I, I, H,
@@ -540,21 +548,43 @@ void GlmMoeLayer::enqueue_prefill_routed_w4a4(const uint16_t* x, size_t x_stride
                                stream);
   launch_swiglu_quantize_rows_nvfp4(d_gate_, d_up_, I, tk, I, cfg_.swiglu_limit, d_q_codes_, d_q_scales_, d_q_gs_, stream, 0.f,
                                     act_scales_dev ? act_scales_dev + 1 : nullptr);
-  if (f32_down) {
+  if (seg_shared) {
+    const MoeExpertView* table = w_.shared_in_table ? d_views_ : d_sh_views_;
+    const int SI = w_.shared_inter;
+    const size_t stride = static_cast<size_t>(max_inter_);
+    if (w_.shared_in_table)
+      launch_moe_grouped_mma_gate_up_swiglu_fp4(x, x_stride, d_segs_ + E, 1, tokens, 0, table, d_slot_act_, stride, SI, H,
+                                                cfg_.swiglu_limit, stream, d_rows_, fp4_group_);
+    else
+      launch_moe_grouped_mma_gate_up_swiglu(x, x_stride, d_segs_ + E, 1, tokens, 0, table, d_slot_act_, stride, SI, H,
+                                            cfg_.swiglu_limit, stream, d_rows_);
+    if (w_.shared_in_table)
+      launch_moe_grouped_mma_fp4_f32(d_slot_act_, stride, d_segs_ + E, 1, tokens, 0, table, 2, d_slot_down_, H, H, SI, stream,
+                                     nullptr, fp4_group_);
+    else
+      launch_moe_grouped_mma_f32(d_slot_act_, stride, d_segs_ + E, 1, tokens, 0, table, 2, d_slot_down_, H, H, SI, stream);
+  }
+  if (f32_down || seg_shared) {   // the shared rows are fp32: so are the routed ones (src/models/glm/moe_layer.cpp:1121)
     launch_moe_grouped_w4a4_f32(d_q_codes_, d_q_scales_, d_q_gs_, nullptr, d_segs_, E, tokens, d_views_, 2, d_slot_down_, H, H,
                                 I, stream);
-    if (out_f32)
-      launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+    const int shared_row0 = seg_shared ? tk : -1;
+    if (acc)
+      launch_moe_accum_ordered_f32(acc, d_slot_down_, H, d_slot_row_, ids, weights, shared_row0, tokens, K, H, stream);
     else
-      launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, -1, tokens, K, H, stream);
+      launch_moe_accum_ordered(rounded, d_slot_down_, H, d_slot_row_, ids, weights, shared_row0, tokens, K, H, stream);
   } else {
     uint16_t* down = reinterpret_cast<uint16_t*>(d_slot_down_);
     launch_moe_grouped_w4a4_bf16(d_q_codes_, d_q_scales_, d_q_gs_, nullptr, d_segs_, E, tokens, d_views_, 2, down, H, H, I,
                                  stream);
-    if (out_f32)
-      launch_moe_accum_ordered_f32_bf16down(out_f32, down, H, d_slot_row_, ids, weights, tokens, K, H, stream);
+    if (acc)
+      launch_moe_accum_ordered_f32_bf16down(acc, down, H, d_slot_row_, ids, weights, tokens, K, H, stream);
     else
-      launch_moe_accum_ordered_bf16down(out_bf16, down, H, d_slot_row_, ids, weights, tokens, K, H, stream);
+      launch_moe_accum_ordered_bf16down(rounded, down, H, d_slot_row_, ids, weights, tokens, K, H, stream);
+  }
+  if (dense) {
+    fork.end();
+    launch_moe_accum(acc, d_sh_down_, d_rows_id_, d_ones_, tokens, H, stream);
+    if (!out_f32) launch_moe_round_bf16(out_bf16, acc, static_cast<int64_t>(tokens) * H, stream);
   }
 }
 

@@ -57,7 +57,8 @@ class GlmMoeLayer {
 
   // The activation-quantized (W4A4) form of the same chain for NVFP4 experts: token rows and SwiGLU rows go through the
   // NVFP4 row quantizer. act_scales_dev: null (a global per row from the row's own maximum) or a DEVICE pair
-  // {token rows' global, SwiGLU rows' global}. The down rows are bf16 unless f32_down.
+  // {token rows' global, SwiGLU rows' global}. The down rows are bf16 unless f32_down or a shared expert's fp32 rows
+  // sit behind them; the shared expert keeps BF16 activations (its segment, or dense projections beside).
   void enqueue_prefill_routed_w4a4(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                                    uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
                                    const float* act_scales_dev = nullptr, bool f32_down = false);

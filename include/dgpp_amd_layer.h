@@ -86,7 +86,8 @@ int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* layer, const uint16_t* x
  * -> SwiGLU inside the second quantizer -> grouped W4A4 down (bf16 rows, or f32 when f32_down is non-zero, the
  * reference's DGPP_MOE_W4A4_F32_DOWN) -> ordered accumulation. act_scales_dev: null for a global per row, or a
  * DEVICE pair {token rows' global, SwiGLU rows' global} (the reference's act_scales_dev). hidden and inter must
- * be multiples of 64. Bitwise the same launchers called one by one. */
+ * be multiples of 64. Bitwise the same launchers called one by one. A shared expert keeps BF16 activations: its
+ * segment's rows sit behind the routed rows (then every down row is f32, :1121), the MXFP8 form runs beside. */
 int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, const int32_t* ids,
                                                const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
                                                void* stream, const float* act_scales_dev, int f32_down);

@@ -385,3 +385,47 @@ def test_layer_w4a4_leg_is_bitwise_the_launchers_called_one_by_one(gpu, static_g
     with pytest.raises(L.InvalidArgument):
         layer8.enqueue_prefill_routed_w4a4(d8.x, 512, dev(i8), dev(w8), dev_empty((8, 512), np.uint16), 8)
     layer8.close()
+
+
+@pytest.mark.parametrize("shared,sI", [("nvfp4", 192), ("fp8", 128), ("mxfp8", 256)])
+def test_layer_w4a4_leg_with_a_shared_expert(gpu, shared, sI):
+    """With a shared expert the activation-quantized chain keeps that expert on BF16 activations (the reference's
+    shared_seg beside W4A4 routed rows, src/models/glm/moe_layer.cpp:1121, 1293-1296, 1317-1336): the token's chain is
+    the routed W4A4 chain over fp32 down rows with the shared row added last, weight 1, one rounding. The shared row is
+    taken from the BF16-activation path with all routing weights zero; the sum must match bit for bit."""
+    from dgpp_amd import moe_layer as ML
+    from test_gpu_moe_layer import make_layer
+    E, H, I, K, T = 7, 1024, 192, 3, 21
+    p = moe_data.make_problem(E, H, I, K, T, "nvfp4", 419, shared_kind=shared, shared_I=sI, limit=7.0, std=0.05)
+    ids, w, _, _ = moe_data.orc_router(p, 1, 1.0, True)
+    ids_d, w_d, zero_d = dev(ids), dev(w), dev(np.zeros_like(w))
+    routed_only = moe_data.MoeProblem(E, H, I, K, T, "nvfp4", None, I, experts=p.experts, x=p.x, router_gate=p.router_gate,
+                                      router_bias=p.router_bias, limit=p.limit)
+    d_ro = DeviceMoe(routed_only)
+    layer_ro = make_layer(routed_only, d_ro, 1, 1.0, T)
+    if shared == "mxfp8":
+        views = list((L.MoeExpertView * (d_ro.views.numel() // 96)).from_buffer_copy(bytes(host(d_ro.views))))
+        shd = [(dev(m.payload), dev(m.scales)) for m in p.shared]
+        cfg = L.make_config(H, I, E, K, n_shared_experts=1, routed_scaling_factor=1.0, swiglu_limit=p.limit, router_mode=1)
+        layer = ML.MoeLayer(cfg, ML.EXPERTS_NVFP4, views, T, shared_inter=sI, sh_payload=[t[0] for t in shd],
+                            sh_scales_e8m0=[t[1] for t in shd])
+        x_d = d_ro.x
+    else:
+        d = DeviceMoe(p)
+        layer = make_layer(p, d, 1, 1.0, T)
+        x_d = d.x
+    a_d, s_d, got_d = (dev_empty((T, H), np.float32) for _ in range(3))
+    got_b = dev_empty((T, H), np.uint16)
+    # a shared segment's fp32 rows make the routed down rows fp32 too; beside dense projections they stay BF16
+    layer_ro.enqueue_prefill_routed_w4a4(x_d, H, ids_d, w_d, None, T, None, out_f32=a_d, f32_down=shared != "mxfp8")
+    layer.enqueue_prefill_routed(x_d, H, ids_d, zero_d, None, T, None, out_f32=s_d)
+    layer.enqueue_prefill_routed_w4a4(x_d, H, ids_d, w_d, None, T, None, out_f32=got_d)
+    layer.enqueue_prefill_routed_w4a4(x_d, H, ids_d, w_d, got_b, T, None)
+    sync()
+    a, s = host(a_d), host(s_d)
+    assert np.any(s != 0) and np.any(a != 0)
+    want = (a + s).astype(np.float32)
+    assert np.array_equal(host(got_d).view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(host(got_b, np.uint16), hg.f32_to_bf16(want))
+    layer.close()
+    layer_ro.close()
