@@ -114,6 +114,43 @@ __device__ __forceinline__ void decode_frags(const ChunkRegs& ch, Frag (&f)[MTra
   }
 }
 
+// The FP16 operands of an NVFP4 lane load, for kernels whose activations are FP16 as well (the W4A4 form: both
+// operands are e2m1 x e4m3 products, six significant bits in [2^-10, 2688], exact in FP16). The scaled conversion
+// applies the scale's exponent; its mantissa, 1 + m / 8, is one packed FP16 multiply per pair: 1.25 instructions
+// per element against the 2 of the BF16 route (convert to f32, multiply, pack).
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+union FragH {
+  f16x8_t v;
+  f16x2_t p[4];
+};
+// (2^e, 1 + m / 8 in both halves) of an e4m3 scale given as f32: the conversion's scale operand and the multiplier.
+__device__ __forceinline__ void split_scale_f16(float s, float& pow2, f16x2_t& mant) {
+  const uint32_t bits = f32_bits(s);
+  pow2 = bits_f32(bits & 0x7F800000u);
+  const uint32_t h = ((bits >> 13) & 0x0380u) | 0x3C00u;
+  mant = __builtin_bit_cast(f16x2_t, h | (h << 16));
+}
+__device__ __forceinline__ void decode_frags_nvfp4_f16(const ChunkRegs& ch, FragH (&f)[4]) {
+  const uint32_t w[4] = {ch.w.x, ch.w.y, ch.w.z, ch.w.w};
+  float e0, e1;
+  f16x2_t m0, m1;
+  split_scale_f16(__builtin_amdgcn_cvt_f32_fp8(ch.s, 0), e0, m0);
+  split_scale_f16(__builtin_amdgcn_cvt_f32_fp8(ch.s, 1), e1, m1);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float e = q < 2 ? e0 : e1;
+    const f16x2_t m = q < 2 ? m0 : m1;
+    f[q].p[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[q], e, 0) * m;
+    f[q].p[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[q], e, 1) * m;
+    f[q].p[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[q], e, 2) * m;
+    f[q].p[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w[q], e, 3) * m;
+  }
+}
+__device__ __forceinline__ f32x4_t mfma_f16(const FragH& a, const uint4& b, f32x4_t acc) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.v, __builtin_bit_cast(f16x8_t, b), acc, 0, 0, 0);
+}
+
 __device__ __forceinline__ f32x4_t mfma_bf16(const Frag& a, const uint4& b, f32x4_t acc) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
 }
@@ -274,20 +311,29 @@ __device__ __forceinline__ uint32_t load_scale(const ScaleLane& sl, int step, in
 }
 
 // acc += the chunk whose tile sits in `region` (operand reads) with block scales sc[0 .. 3]; `valid` steps.
-template <int FMT>
+// H16: the stage holds FP16 activations and the weights decode to FP16 (NVFP4 only).
+template <int FMT, bool H16 = false>
 __device__ __forceinline__ void mfma_tile(const uint4* __restrict__ region, const uint32_t (&sc)[4],
                                           const uint4* __restrict__ lane_stage, int m, int valid, f32x4_t& acc) {
   constexpr int kSub = MTraits<FMT>::kSub;
+  static_assert(!H16 || FMT == kFmtNvfp4, "the FP16 route decodes NVFP4");
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     if (i < valid) {
       ChunkRegs ch;
       ch.w = tile_operand(region, i);
       ch.s = sc[i];
-      Frag f[kSub];
-      decode_frags<FMT>(ch, f);
+      if constexpr (H16) {
+        FragH f[4];
+        decode_frags_nvfp4_f16(ch, f);
 #pragma unroll
-      for (int j = 0; j < kSub; ++j) acc = mfma_bf16(f[j], lane_stage[(i * 4 * kSub + j) * m], acc);
+        for (int j = 0; j < kSub; ++j) acc = mfma_f16(f[j], lane_stage[(i * 4 * kSub + j) * m], acc);
+      } else {
+        Frag f[kSub];
+        decode_frags<FMT>(ch, f);
+#pragma unroll
+        for (int j = 0; j < kSub; ++j) acc = mfma_bf16(f[j], lane_stage[(i * 4 * kSub + j) * m], acc);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   }

@@ -22,8 +22,9 @@ constexpr int kMfmaNB = 4;          // lane loads in flight per row group and pa
 // block must call.
 // Activation rows that arrive already quantized to NVFP4 (the W4A4 form): e2m1 codes [rows, k / 2], one e4m3 scale per
 // 16 elements [rows, scale_stride]; the row's fp32 global is applied by the caller's epilogue. A row's eight-element
-// block decodes to eight BF16 values exactly (e2m1 x e4m3 needs six significant bits), so the matrix core multiplies
-// the same numbers a block-scaled FP4 x FP4 instruction would.
+// block decodes to eight FP16 values exactly (e2m1 x e4m3 needs six significant bits and stays inside [2^-10, 2688]),
+// and so do the weights in this form: the matrix core multiplies the same numbers a block-scaled FP4 x FP4
+// instruction would, with FP16 operands.
 struct A4Src {
   const uint8_t* scales = nullptr;
   size_t scale_stride = 0;
@@ -33,18 +34,15 @@ __device__ __forceinline__ uint4 load_act_block_nvfp4(const uint8_t* __restrict_
                                                       int k0, int k) {
   if (k0 >= k) return make_uint4(0u, 0u, 0u, 0u);
   const uint32_t codes = *reinterpret_cast<const uint32_t*>(codes_row + (k0 >> 1));
-  const float s = __builtin_amdgcn_cvt_f32_fp8(static_cast<uint32_t>(scale_row[k0 >> 4]), 0);
-  uint32_t o[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    f32x2_t v;
-    if (q == 0) v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 0);
-    else if (q == 1) v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 1);
-    else if (q == 2) v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 2);
-    else v = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(codes, 1.0f, 3);
-    o[q] = __builtin_bit_cast(uint32_t, pack_bf16(v.x * s, v.y * s));
-  }
-  return make_uint4(o[0], o[1], o[2], o[3]);
+  float e;
+  f16x2_t m;
+  split_scale_f16(__builtin_amdgcn_cvt_f32_fp8(static_cast<uint32_t>(scale_row[k0 >> 4]), 0), e, m);
+  const f16x2_t v0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, e, 0) * m;
+  const f16x2_t v1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, e, 1) * m;
+  const f16x2_t v2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, e, 2) * m;
+  const f16x2_t v3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(codes, e, 3) * m;
+  return make_uint4(__builtin_bit_cast(uint32_t, v0), __builtin_bit_cast(uint32_t, v1), __builtin_bit_cast(uint32_t, v2),
+                    __builtin_bit_cast(uint32_t, v3));
 }
 
 constexpr int kTileBatch = 2;   // 8 KB in flight per wavefront; more tiles cost registers, and blocks per CU count for more
@@ -126,7 +124,7 @@ __device__ __forceinline__ void block_rows_mfma(const MatRef& mat, const uint16_
     for (int d = 0; d < kTileBatch; ++d) {
       if (d < tiles) {
         commit_tile(region, tile[d]);   // the region's earlier reads were issued before: LDS keeps a wavefront's order
-        mfma_tile<FMT>(region, sc[d], lds + (d * NB * kStepBlocks + (lane >> 4) * kSub) * mt + cc, mt, valid[d], acc);
+        mfma_tile<FMT, A4>(region, sc[d], lds + (d * NB * kStepBlocks + (lane >> 4) * kSub) * mt + cc, mt, valid[d], acc);
         if ((t0 + d + 1) % cpp == 0) {   // a part ends: it joins the running sum, ((p0 + p1) + p2) + p3
           sum = (t0 + d + 1 == (p_lo + 1) * cpp) ? acc : sum + acc;
           acc = f32x4_t{0.f, 0.f, 0.f, 0.f};

@@ -558,7 +558,7 @@ int dgpp_launch_fp8_dequant_blocks_e8m0(const uint8_t* payload, const uint8_t* s
  * scale, e2m1 codes: x ~= e2m1 * scale * gs). Its numerics are those of src/kernels/moe_w4a4.cu, not of the
  * BF16-activation launchers above: the activations carry NVFP4 rounding. The quantizers reproduce the reference's
  * recipe bit for bit (a chain of single IEEE fp32 operations). The GEMM multiplies the exactly decoded operands on the
- * BF16 matrix core with FP32 accumulation (this chip's block-scaled FP4 instruction takes one power-of-two scale per 32
+ * FP16 matrix core with FP32 accumulation (this chip's block-scaled FP4 instruction takes one power-of-two scale per 32
  * elements; NVFP4 carries an e4m3 per 16) and is held, like the reference's kernel, to the fp64 dot of the same
  * quantized operands: |got - dot| < 1e-5 * sum |terms| (tests/cuda/moe_w4a4_test.cu:193-216). */
 /* src/kernels/moe_w4a4.hpp:15, moe_w4a4.cu:596: the activation scale buffer's row stride in bytes: k / 16 rounded up to 8. */
