@@ -840,7 +840,8 @@ def main():
 
     def bench_dispatch():
         """What the dense launchers' choice between the two cores rests on: one to eight rows against cold weights of
-        several sizes on the vector core, on the matrix core unsplit, and on the matrix core with a split-K workspace
+        several sizes on the vector core, on the matrix core unsplit (row tiles only, or the K parts side by side inside
+        sixteen-wavefront blocks), and on the matrix core with a split-K workspace
         (us per launch; --configs dispatch)."""
         res = {"workload": "dense GEMV by row count: vector core / matrix core / matrix core with a split-K workspace, cold weights"}
         cases = [("fp8", 1536, 7168), ("fp8", 4096, 4096), ("fp8", 12288, 6144), ("nvfp4", 2048, 4096), ("nvfp4", 8192, 4096),
@@ -863,7 +864,8 @@ def main():
                 out = torch.empty((m, n), dtype=torch.int16, device=dev)
                 ws = torch.empty(4 * m * n, dtype=torch.float32, device=dev)
                 row = {}
-                for name, core, w_ in (("vector_core", 1, None), ("matrix_core", 2, None), ("matrix_core_split_k", 2, ws)):
+                for name, core, w_, teams in (("vector_core", 1, None, 0), ("matrix_core", 2, None, 1),
+                                              ("matrix_core_parts_side_by_side", 2, None, 2), ("matrix_core_split_k", 2, ws, 0)):
                     wb = ws.numel() * 4 if w_ is not None else 0
                     def step(i):
                         r = i % len(ring)
@@ -874,8 +876,10 @@ def main():
                         else:
                             L.launch_mma_gemv_fp4_bf16(act, k, mats[r], out, m, n, k, 0, stream, w_, wb)
                     lib.dgpp_tune_set(5, core)
+                    lib.dgpp_tune_set(11, teams)   # K parts side by side in sixteen-wavefront blocks: 1 never, 2 always
                     row[name] = time_graph(step, 32, 3) * 1e6
                     lib.dgpp_tune_set(5, 0)
+                    lib.dgpp_tune_set(11, 0)
                 lib.dgpp_tune_set(5, 0)
                 def chosen(i):
                     r = i % len(ring)

@@ -154,8 +154,12 @@ namespace {
 // * five to eight rows: the vector core pays a dot chain per row and weight, the matrix core one decode per weight -
 //   but an unsplit matrix-core launch has one block per 64 weight rows, too few to fill the chip unless the matrix is
 //   large: with a split-K workspace the matrix core wins from five rows on (from three for matrices of 48 M weights and
-//   more), without one only for matrices of 64 M weights and more;
-// * up to four rows: the vector core.
+//   more). Without one, rows of 4096 elements and more run the four parts of K side by side inside a block while the
+//   row tiles fit one round of the chip (dense_mfma_team_row_groups): then six rows and more take the matrix core for
+//   matrices of 8 M weights (block FP8: the vector core needs two passes there) or 32 M weights (FP4) and more, and
+//   matrices of 64 M weights from four (FP8) or five (FP4) rows on; otherwise only matrices of 64 M weights and
+//   more, from five rows on;
+// * up to four rows (three of a large matrix): the vector core.
 constexpr int kVectorPassRows = kMaxActRows;
 bool dense_takes_matrix_core(int fmt, int m, int n, int k, size_t ws_bytes, bool have_ws, int from_rows) {
   if (m > kVectorPassRows || m > max_stage_rows(k)) return true;
@@ -171,6 +175,13 @@ bool dense_takes_matrix_core(int fmt, int m, int n, int k, size_t ws_bytes, bool
   const bool split = have_ws && parts > 1 && (n + 63) / 64 < 1024 &&
                      ws_bytes >= static_cast<size_t>(parts) * m * static_cast<size_t>(n) * sizeof(float);
   if (split) return m >= 5 || (m >= 3 && weights >= (48u << 20));
+  if (dense_mfma_team_row_groups(parts, m, n, true) != 0) {
+    // the parts of K side by side inside a block: block FP8 from six rows on (the vector core takes two passes there),
+    // FP4 from six rows on for matrices of 32 M weights and more; large matrices from four rows on
+    const bool fp8 = fmt == kFmtFp8F32 || fmt == kFmtFp8E8M0;
+    if (m >= 6 && weights >= ((fp8 ? 8u : 32u) << 20)) return true;
+    return m >= (fp8 ? 4 : 5) && weights >= (64u << 20);
+  }
   return m >= 5 && weights >= (64u << 20);
 }
 int dense_rows(int fmt, const uint16_t* act, size_t act_stride, const MatRef& mat, const float* global, void* out,

@@ -795,6 +795,21 @@ inline int max_stage_rows(int k) {
   return static_cast<int>(fit < 1 ? 1 : (fit > kMaxActRows ? kMaxActRows : fit));
 }
 
+// Row groups per block of the dense matrix-core launch that runs the four parts of K side by side inside a block
+// (0: the row-tile form). Four up to one round of the chip's 256 CUs - one such block fills a CU, and 272 tiles, two
+// rounds with the second nearly empty, measured slower than the row-tile form; two (blocks half the size, two to a CU)
+// for up to eight activation rows when the row tiles just exceed a round. Bench switch 11: 1 never, 2 four, 3 two.
+constexpr size_t kTeamsMaxTiles = 256;
+constexpr size_t kTeamsMaxTilesHalf = 320;
+inline int dense_mfma_team_row_groups(int parts, int m, int n, bool plain) {
+  const int knob = tune_get(kTuneTeams);
+  if (!plain || parts != 4 || knob == 1) return 0;
+  const size_t tiles = static_cast<size_t>((n + 63) / 64) * static_cast<size_t>((m + 15) / 16);
+  if (knob == 2 || tiles <= kTeamsMaxTiles) return 4;
+  if ((knob == 3 || tiles <= kTeamsMaxTilesHalf) && m <= 8) return 2;
+  return 0;
+}
+
 // The bodies, included by the per-format translation units.
 #ifdef DGPP_GEMV_IMPL
 template <class F>
@@ -809,6 +824,7 @@ inline bool use_mfma_core() { return tune_get(kTuneCore) == 2; }
 
 // `ws` (nullable) holds parts * m * n floats: the K parts then run in separate blocks and a second
 // launch folds them (same bits); worth it only when the unsplit grid leaves the chip under-filled.
+
 template <int FMT>
 hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, size_t ws_bytes) {
   const MGeom g = mgeom<FMT>(a.k);
@@ -818,6 +834,24 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
                      a.a4_scales == nullptr;
   const dim3 grid(gx, gy, split ? g.parts : 1);
   hipError_t err = hipSuccess;
+  // Without a workspace the four parts of K run side by side inside a block while the row tiles alone would leave
+  // most SIMDs one wavefront.
+  const int rg = dense_mfma_team_row_groups(g.parts, a.m, a.n, !split && a.act_up == nullptr && a.a4_scales == nullptr);
+  if (rg != 0) {
+    dispatch_bool(a.once != 0, [&](auto ntc) {
+      auto launch = [&](auto rgc) {
+        constexpr int RG = decltype(rgc)::value;
+        auto kern = mfma_dense_teams_kernel<FMT, kMfmaNB, decltype(ntc)::value, RG>;
+        constexpr size_t lds = TeamShape<RG>::kLdsUnits * sizeof(uint4);
+        err = ensure_lds(kern, lds);
+        const unsigned bx = static_cast<unsigned>((a.n + RG * kGroupRows - 1) / (RG * kGroupRows));
+        if (err == hipSuccess) hipLaunchKernelGGL(kern, dim3(bx, gy), dim3(TeamShape<RG>::kThreads), lds, stream, a, g);
+      };
+      if (rg == 4) launch(std::integral_constant<int, 4>{});
+      else launch(std::integral_constant<int, 2>{});
+    });
+    return err != hipSuccess ? err : hipGetLastError();
+  }
   dispatch_bool(a.once != 0, [&](auto ntc) {
     auto go = [&](auto kern) {
       constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);

@@ -196,6 +196,117 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_dense_kernel(DenseArgs 
   store_tile<kFmtMxfp4>(sum, 1.0f, partials, 1, (static_cast<size_t>(part) * a.m + c0 + c) * a.n, row0, a.n, c < mt);
 }
 
+// ---- K parts side by side inside one block ---------------------------------------------------------------------
+// A dense launch whose row tiles barely fill the chip leaves one wavefront per SIMD walking all of K on its own.
+// Here a block is sixteen wavefronts: TEAM t (four of them, one per row group) walks part t of K, so the four parts
+// of a row group run side by side and the block folds them in LDS in the unsplit form's order, ((p0 + p1) + p2) + p3:
+// the same bits, no workspace, no second launch. A team shares its own activation stage; the barriers are
+// block-wide, which is sound because every part is walked as the same number of tiles (a trailing part's missing
+// steps are zero loads).
+// RG row groups per block (four, or two with half the stage for up to eight activation rows: two such blocks share
+// a CU, which evens out a grid that just exceeds one round of the larger blocks).
+template <int RG>
+struct TeamShape {
+  static constexpr int kTeamThreads = RG * kWave;                     // the wavefronts that share one part of K
+  static constexpr int kThreads = kMaxParts * kTeamThreads;
+  static constexpr int kStage = kStageUnits * RG / kWavesPerBlock;    // 16-byte units of one team's activation stage
+  static constexpr int kLdsUnits = kMaxParts * kStage + (kThreads / kWave) * kTileUnits;
+};
+
+template <int FMT, int NB, bool NT, int RG>
+__device__ __forceinline__ void team_rows_mfma(const MatRef& mat, const uint16_t* __restrict__ act, size_t act_stride, int mt,
+                                               int n, int k, int row0, const MGeom& g, int team, uint4* __restrict__ lds,
+                                               f32x4_t& sum) {
+  static_assert(NB == 4, "a tile is four steps");
+  using S = TeamShape<RG>;
+  constexpr int kSub = MTraits<FMT>::kSub;
+  constexpr int kStepBlocks = MTraits<FMT>::kStepBlocks;
+  constexpr int kStepElems = MTraits<FMT>::kStepElems;
+  constexpr int kStageRegs = S::kStage / S::kTeamThreads;
+  const int chunks = k / MTraits<FMT>::kLoadElems;
+  const int lane = threadIdx.x & (kWave - 1), tid = threadIdx.x % S::kTeamThreads;
+  const WideLane wl = wide_lane<FMT>(mat, row0, n, k);
+  const ScaleLane sl = scale_lane<FMT>(mat, row0, n, k);
+  uint4* stage = lds + team * S::kStage;
+  uint4* region = lds + kMaxParts * S::kStage + (threadIdx.x >> 6) * kTileUnits;
+  const int cc = min(lane & 15, mt - 1);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(act) & 15u) == 0) && ((act_stride & 7u) == 0);
+  const int cpp = g.part_steps / NB;
+  const int batch = max(1, min(kTileBatch, S::kStage / (mt * kStepBlocks * NB)));
+  const int t_lo = team * cpp, t_hi = t_lo + cpp;
+  int unit_kb[kStageRegs];
+  size_t unit_row[kStageRegs];
+#pragma unroll
+  for (int i = 0; i < kStageRegs; ++i) {
+    const int idx = tid + i * S::kTeamThreads;
+    const int kb = idx / mt, c = idx - kb * mt;
+    unit_kb[i] = kb;
+    unit_row[i] = static_cast<size_t>(c) * act_stride;
+  }
+  f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+  for (int t0 = t_lo; t0 < t_hi; t0 += batch) {
+    const int tiles = min(batch, t_hi - t0);
+    uint4 tile[kTileBatch][4];
+    uint32_t sc[kTileBatch][4];
+    int valid[kTileBatch];
+#pragma unroll
+    for (int d = 0; d < kTileBatch; ++d) {
+      const int step0 = (t0 + d) * NB;
+      valid[d] = d < tiles ? max(0, min(NB, g.steps - step0)) : 0;
+      issue_tile<NT>(wl, valid[d] > 0 ? step0 : g.steps, tile[d]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sc[d][i] = load_scale<FMT>(sl, i < valid[d] ? step0 + i : g.steps, chunks, mat.cs);
+    }
+    const int units = tiles * NB * kStepBlocks * mt;
+    const int k_base = t0 * NB * kStepElems;
+    uint4 pre[kStageRegs];
+#pragma unroll
+    for (int i = 0; i < kStageRegs; ++i) {
+      pre[i] = make_uint4(0u, 0u, 0u, 0u);
+      if (tid + i * S::kTeamThreads < units) pre[i] = load_act_block(act + unit_row[i], k_base + unit_kb[i] * 8, k, aligned);
+    }
+    __syncthreads();   // every team's readers of the batch before are through
+#pragma unroll
+    for (int i = 0; i < kStageRegs; ++i)
+      if (tid + i * S::kTeamThreads < units) stage[tid + i * S::kTeamThreads] = pre[i];
+    __syncthreads();
+#pragma unroll
+    for (int d = 0; d < kTileBatch; ++d) {
+      if (d < tiles) {
+        commit_tile(region, tile[d]);
+        mfma_tile<FMT>(region, sc[d], stage + (d * NB * kStepBlocks + (lane >> 4) * kSub) * mt + cc, mt, valid[d], acc);
+      }
+    }
+  }
+  sum = acc;
+}
+
+template <int FMT, int NB, bool NT, int RG>
+__global__ __launch_bounds__(TeamShape<RG>::kThreads) void mfma_dense_teams_kernel(DenseArgs a, MGeom g) {
+  extern __shared__ uint4 lds[];
+  using S = TeamShape<RG>;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  const int team = wave / RG, rg = wave % RG;
+  const int row0 = (static_cast<int>(blockIdx.x) * RG + rg) * kGroupRows;
+  const int c0 = static_cast<int>(blockIdx.y) * kTileCols;
+  const int mt = min(kTileCols, a.m - c0);
+  f32x4_t sum;
+  team_rows_mfma<FMT, NB, NT, RG>(a.mat, a.act + static_cast<size_t>(c0) * a.act_stride, a.act_stride, mt, a.n, a.k, row0, g, team,
+                                  lds, sum);
+  // every wavefront parks its part's sums in its own tile region (its last operand reads were issued before: LDS
+  // keeps a wavefront's order); team 0 folds the four parts of its row groups in ascending order and stores
+  uint4* regions = lds + kMaxParts * S::kStage;
+  regions[wave * kTileUnits + lane] = __builtin_bit_cast(uint4, sum);
+  __syncthreads();
+  if (team != 0) return;
+  f32x4_t s = sum;
+  s = s + __builtin_bit_cast(f32x4_t, regions[(RG + rg) * kTileUnits + lane]);
+  s = (s + __builtin_bit_cast(f32x4_t, regions[(2 * RG + rg) * kTileUnits + lane])) +
+      __builtin_bit_cast(f32x4_t, regions[(3 * RG + rg) * kTileUnits + lane]);
+  const int c = lane & 15;
+  store_tile<FMT>(s, load_divisor<FMT>(a.global), a.out, a.out_f32, static_cast<size_t>(c0 + c) * a.out_stride, row0, a.n, c < mt);
+}
+
 // Two dense problems of the same k and m in ONE launch (reference: launch_mma_gemv_fp8_bf16_pair,
 // src/kernels/mma_gemv.cu:935-961 - two dependent-free projections sharing one ramp and drain): the first tiles0 row
 // tiles of the grid belong to problem 0, the rest to problem 1; each block then does what mfma_dense_kernel does for

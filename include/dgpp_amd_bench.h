@@ -28,8 +28,11 @@ extern "C" {
  * on the caller's stream, 2 moves them to a second stream beside the routed passes at every batch size (default:
  * from three tokens on); 3 and 4 keep one stream and never / always fold the accumulation into the shared down pass
  * (default: at one token); key 10: 2 or 4 runs the router's token-tiled score kernel at every batch size with that many tokens per
- * wavefront (0 = automatic: tiled from 32 rows on, 4 tokens from 128 rows on). Outputs do not depend on keys
- * 1 - 4 and 6 - 10; keys 0 and
+ * wavefront (0 = automatic: tiled from 32 rows on, 4 tokens from 128 rows on); key 11: the dense matrix-core launch
+ * without a workspace that runs the four parts of K side by side inside a block: 1 never, 2 always with four row groups
+ * per block, 3 with two for up to eight rows (0 = automatic: four while the row tiles fit one round of the chip, two for up
+ * to a round and a quarter). Outputs do not depend on keys
+ * 1 - 4 and 6 - 11; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
  * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);

@@ -361,3 +361,50 @@ def test_prefill_path_with_a_shared_expert(gpu, kind, shared, sI):
         lib.dgpp_tune_set(5, 0)
     assert np.array_equal(host(out2, np.uint16), got), "decode-slot chain on the matrix core == grouped matrix-core path, bitwise"
     layer.close()
+
+
+@pytest.mark.parametrize("kind,m,n,k", [("fp8", 9, 200, 4096), ("e8m0", 64, 130, 6144), ("nvfp4", 8, 530, 5120), ("mxfp4", 16, 64, 4096),
+                                        ("nvfp4", 3, 48, 8192)])
+def test_parts_of_k_side_by_side_in_a_block_give_the_row_tile_forms_bits(gpu, kind, m, n, k):
+    """The dense matrix-core launch without a workspace that gives each of the four parts of K to its own wavefronts
+    of a block and folds them in LDS (four row groups per block, or two for up to eight rows): the bits of the form
+    that walks the parts one after the other, whatever the bench switch picks."""
+    lib = _lib.load()
+    w = hg.normal_f32(0x7EA0 + n + k, (n, k), 0.02)
+    act = hg.normal_bf16(0x7EA1 + n, (m, k))
+    a_d = dev(act)
+    if kind in ("fp8", "e8m0"):
+        payload, scales = hg.encode_mxfp8(w) if kind == "e8m0" else hg.encode_fp8_blocks(hg.f32_to_bf16(w), 128, 128)
+        p_d, s_d = dev(payload), dev(scales)
+        fn = L.launch_mma_gemv_fp8e8m0_f32 if kind == "e8m0" else L.launch_mma_gemv_fp8_f32
+        rs, cs = (0, 5) if kind == "e8m0" else (7, 7)
+
+        def run(out):
+            fn(a_d, k, p_d, s_d, out, m, n, k, 0, rs, cs, None)
+    else:
+        if kind == "nvfp4":
+            payload, scales, ws2 = hg.encode_nvfp4(w)
+            g_d = dev(np.array([1.0 / np.float32(ws2)], np.float32))
+        else:
+            (payload, scales), g_d = hg.encode_mxfp4(w), None
+        p_d, s_d = dev(payload), dev(scales)
+        wm = fp4_matrix(p_d, s_d, g_d, n, k, 16 if kind == "nvfp4" else 32)
+
+        def run(out):
+            L.launch_mma_gemv_fp4_f32(a_d, k, wm, out, m, n, k, 0, None)
+    outs = {}
+    lib.dgpp_tune_set(5, 2)
+    try:
+        for knob in (1, 2, 3) if m <= 8 else (1, 2):
+            lib.dgpp_tune_set(11, knob)
+            outs[knob] = dev_empty((m, n), np.float32)
+            outs[knob].fill_(-7.0)
+            run(outs[knob])
+        sync()
+    finally:
+        lib.dgpp_tune_set(11, 0)
+        lib.dgpp_tune_set(5, 0)
+    want = host(outs[1])
+    assert np.all(want != -7.0)
+    for knob, o in outs.items():
+        assert np.array_equal(host(o).view(np.uint32), want.view(np.uint32)), f"switch {knob}"
