@@ -216,6 +216,7 @@ LAYER_SIGNATURES = {
     "dgpp_moe_layer_enqueue_decode_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_grouped_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
+    "dgpp_moe_layer_enqueue_prefill": (_I, [_P, _P, _Z, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill_routed_w4a4": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_moe_resident_last_error": (C.c_char_p, []),
     "dgpp_moe_resident_load": (_I, [_P, _P]),

@@ -478,6 +478,19 @@ void GlmMoeLayer::enqueue_prefill_routed(const uint16_t* x, size_t x_stride, con
   prefill_chain(x, x_stride, ids, weights, out_bf16, out_f32, tokens, stream, has_shared());
 }
 
+// The whole prefill step from the hidden rows (reference: GlmMoeLayer::enqueue_prefill, src/models/glm/moe_layer.cpp:775-812
+// - route on the device, then the grouped chain, nothing waits on the host): score rows, selection, enqueue_prefill_routed
+// over the layer's own ids and weights.
+void GlmMoeLayer::enqueue_prefill(const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32, int tokens,
+                                  hipStream_t stream) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  if (!w_.router_gate) throw std::invalid_argument("GlmMoeLayer: the router gate is not bound");
+  launch_moe_router_dots(x, w_.router_gate, w_.router_bias, d_scores_, d_biased_, cfg_, tokens, stream);
+  launch_moe_router_select(d_scores_, d_biased_, d_ids_, d_weights_, cfg_, tokens, stream);
+  enqueue_prefill_routed(x, x_stride, d_ids_, d_weights_, out_bf16, out_f32, tokens, stream);
+}
+
 // Segments -> gate + up + SwiGLU -> down -> ordered accumulation on the matrix core. with_shared: the shared expert
 // is segment n_experts (every token, in token order, rows [tokens * top_k, ...) of the slot buffers; the reference's
 // shared_seg, src/models/glm/moe_layer.cpp:1293-1296, 1335-1336) and ends every token's chain with weight 1.
@@ -693,6 +706,10 @@ int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* l, const uint16_t* x, si
   return guarded([&] {
     l->impl.enqueue_prefill_routed(x, x_stride, ids, weights, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream));
   });
+}
+int dgpp_moe_layer_enqueue_prefill(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32,
+                                   int tokens, void* stream) {
+  return guarded([&] { l->impl.enqueue_prefill(x, x_stride, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream)); });
 }
 int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, const int32_t* ids,
                                                const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,

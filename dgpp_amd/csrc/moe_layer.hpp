@@ -55,6 +55,8 @@ class GlmMoeLayer {
   void enqueue_prefill_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                               uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
 
+  // The same from the hidden rows: score rows, selection, then the chain above over the layer's own routes.
+  void enqueue_prefill(const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
   // The activation-quantized (W4A4) form of the same chain for NVFP4 experts: token rows and SwiGLU rows go through the
   // NVFP4 row quantizer. act_scales_dev: null (a global per row from the row's own maximum) or a DEVICE pair
   // {token rows' global, SwiGLU rows' global}. The down rows are bf16 unless f32_down or a shared expert's fp32 rows

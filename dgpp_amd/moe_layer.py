@@ -83,6 +83,10 @@ class MoeLayer:
         _check(self._lib.dgpp_moe_layer_enqueue_prefill_routed(self._h, _p(x), x_stride, _p(ids), _p(weights),
                                                                _p(out_bf16), _p(out_f32), tokens, _stream(stream)))
 
+    def enqueue_prefill(self, x, x_stride, out_bf16, tokens, stream=None, out_f32=None):
+        _check(self._lib.dgpp_moe_layer_enqueue_prefill(self._h, _p(x), x_stride, _p(out_bf16), _p(out_f32), tokens,
+                                                        _stream(stream)))
+
     def enqueue_prefill_routed_w4a4(self, x, x_stride, ids, weights, out_bf16, tokens, stream=None, out_f32=None,
                                     act_scales_dev=None, f32_down=False):
         _check(self._lib.dgpp_moe_layer_enqueue_prefill_routed_w4a4(self._h, _p(x), x_stride, _p(ids), _p(weights),

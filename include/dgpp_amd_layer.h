@@ -81,6 +81,10 @@ int dgpp_moe_layer_enqueue_grouped_routed(DgppMoeLayer* layer, const uint16_t* x
 int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, const int32_t* ids,
                                           const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
                                           void* stream);
+/* The same from the hidden rows (GlmMoeLayer::enqueue_prefill, src/models/glm/moe_layer.cpp:775-812: routing stays on the
+ * device, nothing waits on the host): score rows, selection, then the chain above over the layer's own ids and weights. */
+int dgpp_moe_layer_enqueue_prefill(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32,
+                                   int tokens, void* stream);
 /* The activation-quantized (W4A4) form of that chain for NVFP4 experts (src/models/glm/moe_layer.cpp:1122-1135,
  * 1217-1219, 1268-1272, 1306-1316): token rows -> NVFP4 row quantizer -> grouped W4A4 gate, up over the routed row list
  * -> SwiGLU inside the second quantizer -> grouped W4A4 down (bf16 rows, or f32 when f32_down is non-zero, the

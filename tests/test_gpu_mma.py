@@ -360,6 +360,14 @@ def test_prefill_path_with_a_shared_expert(gpu, kind, shared, sI):
     finally:
         lib.dgpp_tune_set(5, 0)
     assert np.array_equal(host(out2, np.uint16), got), "decode-slot chain on the matrix core == grouped matrix-core path, bitwise"
+    # the whole step from the hidden rows: the layer routes on the device, then runs the same chain over its own routes
+    out3, out4 = dev_empty((T, H), np.uint16), dev_empty((T, H), np.uint16)
+    if shared != "mxfp8":   # (that layer was built without a router gate)
+        layer.enqueue_prefill(d.x, H, out3, T)
+        layer.enqueue_prefill_routed(d.x, H, layer.ids_ptr, layer.weights_ptr, out4, T)
+        sync()
+        assert np.array_equal(host(out3, np.uint16), host(out4, np.uint16)) and host(out3, np.uint16).any()
+        expert_budget(host(out3, np.uint16), raw, f"prefill from the hidden rows {kind} + shared {shared}")
     layer.close()
 
 
