@@ -217,6 +217,9 @@ LAYER_SIGNATURES = {
     "dgpp_moe_layer_enqueue_grouped_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill_routed": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill": (_I, [_P, _P, _Z, _P, _P, _I, _P]),
+    "dgpp_moe_layer_route_prefill_rows": (_I, [_P, _P, _Z, _I, _I, _P]),
+    "dgpp_moe_layer_enqueue_prefill_phased": (_I, [_P, _P, _Z, _I, _P]),
+    "dgpp_moe_layer_accumulate_prefill_rows": (_I, [_P, _P, _P, _I, _I, _I, _P]),
     "dgpp_moe_layer_enqueue_prefill_routed_w4a4": (_I, [_P, _P, _Z, _P, _P, _P, _P, _I, _P, _P, _I]),
     "dgpp_moe_resident_last_error": (C.c_char_p, []),
     "dgpp_moe_resident_load": (_I, [_P, _P]),

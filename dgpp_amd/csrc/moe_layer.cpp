@@ -495,7 +495,8 @@ void GlmMoeLayer::enqueue_prefill(const uint16_t* x, size_t x_stride, uint16_t* 
 // is segment n_experts (every token, in token order, rows [tokens * top_k, ...) of the slot buffers; the reference's
 // shared_seg, src/models/glm/moe_layer.cpp:1293-1296, 1335-1336) and ends every token's chain with weight 1.
 void GlmMoeLayer::prefill_chain(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
-                                uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream, bool with_shared) {
+                                uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream, bool with_shared,
+                                bool accumulate) {
   const int K = cfg_.top_k, H = cfg_.hidden, I = cfg_.inter, E = cfg_.n_experts;
   const int tk = tokens * K;
   const bool fp8 = w_.format == GlmExpertFormat::Fp8;
@@ -522,11 +523,48 @@ void GlmMoeLayer::prefill_chain(const uint16_t* x, size_t x_stride, const int32_
   if (with_shared && !in_table)
     launch_moe_grouped_mma_f32(d_slot_act_, stride, d_segs_ + E, 1, max_rows, 0, d_sh_views_, 2, d_slot_down_, H, H,
                                w_.shared_inter, stream);
+  if (!accumulate) return;
   const int shared_row0 = with_shared ? tk : -1;
   if (out_f32)
     launch_moe_accum_ordered_f32(out_f32, d_slot_down_, H, d_slot_row_, ids, weights, shared_row0, tokens, K, H, stream);
   else
     launch_moe_accum_ordered(out_bf16, d_slot_down_, H, d_slot_row_, ids, weights, shared_row0, tokens, K, H, stream);
+}
+
+// The prefill in phases (reference: route_prefill_rows / enqueue_prefill_phased / accumulate_prefill_rows,
+// src/models/glm/moe_layer.cpp:843-904, for a caller that overlaps other work with the per-row ends of the layer): the
+// router over a block of rows ahead of the chain, the chain over all rows without its accumulation, the accumulation
+// per block of rows. The same kernels per row as enqueue_prefill: bitwise its output.
+void GlmMoeLayer::route_prefill_rows(const uint16_t* x, size_t x_stride, int r0, int rows, hipStream_t stream) {
+  if (rows <= 0) return;
+  if (r0 < 0 || r0 > max_tokens_ - rows) throw std::invalid_argument("GlmMoeLayer: the row block exceeds the layer's max_tokens");
+  if (!w_.router_gate) throw std::invalid_argument("GlmMoeLayer: the router gate is not bound");
+  const size_t E = static_cast<size_t>(cfg_.n_experts), K = static_cast<size_t>(cfg_.top_k), at = static_cast<size_t>(r0);
+  launch_moe_router_dots(x + at * x_stride, w_.router_gate, w_.router_bias, d_scores_ + at * E, d_biased_ + at * E, cfg_, rows,
+                         stream);
+  launch_moe_router_select(d_scores_ + at * E, d_biased_ + at * E, d_ids_ + at * K, d_weights_ + at * K, cfg_, rows, stream);
+}
+void GlmMoeLayer::enqueue_prefill_phased(const uint16_t* x, size_t x_stride, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return;
+  check_tokens(tokens);
+  if (dense_shared()) throw std::invalid_argument("GlmMoeLayer: the phased prefill takes the shared expert as a segment");
+  prefill_chain(x, x_stride, d_ids_, d_weights_, nullptr, nullptr, tokens, stream, has_shared(), /*accumulate=*/false);
+}
+void GlmMoeLayer::accumulate_prefill_rows(uint16_t* out_bf16, float* out_f32, int tokens, int r0, int rows, hipStream_t stream) {
+  if (rows <= 0) return;
+  check_tokens(tokens);
+  if (out_bf16 == nullptr && out_f32 == nullptr) throw std::invalid_argument("GlmMoeLayer: no output buffer");
+  if (r0 < 0 || r0 > tokens - rows) throw std::invalid_argument("GlmMoeLayer: the row block lies outside the batch");
+  if (dense_shared()) throw std::invalid_argument("GlmMoeLayer: the phased prefill takes the shared expert as a segment");
+  const int K = cfg_.top_k, H = cfg_.hidden;
+  const size_t at = static_cast<size_t>(r0);
+  const int shared_row0 = has_shared() ? tokens * K + r0 : -1;
+  if (out_f32)
+    launch_moe_accum_ordered_f32(out_f32 + at * H, d_slot_down_, H, d_slot_row_ + at * K, d_ids_ + at * K, d_weights_ + at * K,
+                                 shared_row0, rows, K, H, stream);
+  else
+    launch_moe_accum_ordered(out_bf16 + at * H, d_slot_down_, H, d_slot_row_ + at * K, d_ids_ + at * K, d_weights_ + at * K,
+                             shared_row0, rows, K, H, stream);
 }
 
 // The reference's W4A4 prefill chain (src/models/glm/moe_layer.cpp:1122-1135 the token rows' quantizer, :1217-1219
@@ -710,6 +748,16 @@ int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* l, const uint16_t* x, si
 int dgpp_moe_layer_enqueue_prefill(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32,
                                    int tokens, void* stream) {
   return guarded([&] { l->impl.enqueue_prefill(x, x_stride, out_bf16, out_f32, tokens, static_cast<hipStream_t>(stream)); });
+}
+int dgpp_moe_layer_route_prefill_rows(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, int r0, int rows, void* stream) {
+  return guarded([&] { l->impl.route_prefill_rows(x, x_stride, r0, rows, static_cast<hipStream_t>(stream)); });
+}
+int dgpp_moe_layer_enqueue_prefill_phased(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, int tokens, void* stream) {
+  return guarded([&] { l->impl.enqueue_prefill_phased(x, x_stride, tokens, static_cast<hipStream_t>(stream)); });
+}
+int dgpp_moe_layer_accumulate_prefill_rows(DgppMoeLayer* l, uint16_t* out_bf16, float* out_f32, int tokens, int r0, int rows,
+                                           void* stream) {
+  return guarded([&] { l->impl.accumulate_prefill_rows(out_bf16, out_f32, tokens, r0, rows, static_cast<hipStream_t>(stream)); });
 }
 int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* l, const uint16_t* x, size_t x_stride, const int32_t* ids,
                                                const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,

@@ -57,6 +57,11 @@ class GlmMoeLayer {
 
   // The same from the hidden rows: score rows, selection, then the chain above over the layer's own routes.
   void enqueue_prefill(const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
+  // The prefill in phases over the layer's own routes: the router over rows [r0, r0 + rows), the chain over all rows
+  // without its accumulation, the accumulation of rows [r0, r0 + rows) into out[r0 ...]. Bitwise enqueue_prefill.
+  void route_prefill_rows(const uint16_t* x, size_t x_stride, int r0, int rows, hipStream_t stream);
+  void enqueue_prefill_phased(const uint16_t* x, size_t x_stride, int tokens, hipStream_t stream);
+  void accumulate_prefill_rows(uint16_t* out_bf16, float* out_f32, int tokens, int r0, int rows, hipStream_t stream);
   // The activation-quantized (W4A4) form of the same chain for NVFP4 experts: token rows and SwiGLU rows go through the
   // NVFP4 row quantizer. act_scales_dev: null (a global per row from the row's own maximum) or a DEVICE pair
   // {token rows' global, SwiGLU rows' global}. The down rows are bf16 unless f32_down or a shared expert's fp32 rows
@@ -78,7 +83,7 @@ class GlmMoeLayer {
   bool needs_order(int tokens) const;
   void dense_shared_chain(const uint16_t* x, size_t x_stride, int tokens, hipStream_t stream);
   void prefill_chain(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights, uint16_t* out_bf16,
-                     float* out_f32, int tokens, hipStream_t stream, bool with_shared);
+                     float* out_f32, int tokens, hipStream_t stream, bool with_shared, bool accumulate = true);
   void expert_chain_slots(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
                           uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream,
                           bool order_ready = false, const float* sel_scores = nullptr, const float* sel_biased = nullptr,

@@ -87,6 +87,16 @@ class MoeLayer:
         _check(self._lib.dgpp_moe_layer_enqueue_prefill(self._h, _p(x), x_stride, _p(out_bf16), _p(out_f32), tokens,
                                                         _stream(stream)))
 
+    def route_prefill_rows(self, x, x_stride, r0, rows, stream=None):
+        _check(self._lib.dgpp_moe_layer_route_prefill_rows(self._h, _p(x), x_stride, r0, rows, _stream(stream)))
+
+    def enqueue_prefill_phased(self, x, x_stride, tokens, stream=None):
+        _check(self._lib.dgpp_moe_layer_enqueue_prefill_phased(self._h, _p(x), x_stride, tokens, _stream(stream)))
+
+    def accumulate_prefill_rows(self, out_bf16, tokens, r0, rows, stream=None, out_f32=None):
+        _check(self._lib.dgpp_moe_layer_accumulate_prefill_rows(self._h, _p(out_bf16), _p(out_f32), tokens, r0, rows,
+                                                                _stream(stream)))
+
     def enqueue_prefill_routed_w4a4(self, x, x_stride, ids, weights, out_bf16, tokens, stream=None, out_f32=None,
                                     act_scales_dev=None, f32_down=False):
         _check(self._lib.dgpp_moe_layer_enqueue_prefill_routed_w4a4(self._h, _p(x), x_stride, _p(ids), _p(weights),

@@ -85,6 +85,15 @@ int dgpp_moe_layer_enqueue_prefill_routed(DgppMoeLayer* layer, const uint16_t* x
  * device, nothing waits on the host): score rows, selection, then the chain above over the layer's own ids and weights. */
 int dgpp_moe_layer_enqueue_prefill(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32,
                                    int tokens, void* stream);
+/* The prefill in phases (route_prefill_rows / enqueue_prefill_phased / accumulate_prefill_rows,
+ * src/models/glm/moe_layer.cpp:843-904), for a caller that overlaps other work with the per-row ends of the layer: the router
+ * over rows [r0, r0 + rows) of x (x points at row 0), then the chain over all `tokens` rows without its accumulation, then
+ * the accumulation of rows [r0, r0 + rows) into out[r0 ...] (out points at row 0). The same kernels per row as
+ * dgpp_moe_layer_enqueue_prefill: bitwise its output. The shared expert rides as a segment (not the dense MXFP8 form). */
+int dgpp_moe_layer_route_prefill_rows(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, int r0, int rows, void* stream);
+int dgpp_moe_layer_enqueue_prefill_phased(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, int tokens, void* stream);
+int dgpp_moe_layer_accumulate_prefill_rows(DgppMoeLayer* layer, uint16_t* out_bf16, float* out_f32, int tokens, int r0, int rows,
+                                           void* stream);
 /* The activation-quantized (W4A4) form of that chain for NVFP4 experts (src/models/glm/moe_layer.cpp:1122-1135,
  * 1217-1219, 1268-1272, 1306-1316): token rows -> NVFP4 row quantizer -> grouped W4A4 gate, up over the routed row list
  * -> SwiGLU inside the second quantizer -> grouped W4A4 down (bf16 rows, or f32 when f32_down is non-zero, the

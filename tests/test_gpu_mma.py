@@ -368,6 +368,22 @@ def test_prefill_path_with_a_shared_expert(gpu, kind, shared, sI):
         sync()
         assert np.array_equal(host(out3, np.uint16), host(out4, np.uint16)) and host(out3, np.uint16).any()
         expert_budget(host(out3, np.uint16), raw, f"prefill from the hidden rows {kind} + shared {shared}")
+        # the same in phases: the router over two row blocks, the chain, the accumulation per block
+        out5 = dev_empty((T, H), np.uint16)
+        out5.fill_(0x7F7F)
+        cut = 7
+        layer.route_prefill_rows(d.x, H, cut, T - cut)
+        layer.route_prefill_rows(d.x, H, 0, cut)
+        layer.enqueue_prefill_phased(d.x, H, T)
+        layer.accumulate_prefill_rows(out5, T, cut, T - cut)
+        layer.accumulate_prefill_rows(out5, T, 0, cut)
+        sync()
+        assert np.array_equal(host(out5, np.uint16), host(out3, np.uint16)), "phased == whole"
+        with pytest.raises(L.InvalidArgument):
+            layer.accumulate_prefill_rows(out5, T, T - 2, 5)
+    else:
+        with pytest.raises(L.InvalidArgument):
+            layer.enqueue_prefill_phased(d.x, H, T)
     layer.close()
 
 
