@@ -388,11 +388,11 @@ def test_prefill_path_with_a_shared_expert(gpu, kind, shared, sI):
 
 
 @pytest.mark.parametrize("kind,m,n,k", [("fp8", 9, 200, 4096), ("e8m0", 64, 130, 6144), ("nvfp4", 8, 530, 5120), ("mxfp4", 16, 64, 4096),
-                                        ("nvfp4", 3, 48, 8192)])
+                                        ("nvfp4", 3, 48, 8192), ("mxfp4", 8, 16500, 4096), ("fp8", 16, 20470, 4096)])
 def test_parts_of_k_side_by_side_in_a_block_give_the_row_tile_forms_bits(gpu, kind, m, n, k):
     """The dense matrix-core launch without a workspace that gives each of the four parts of K to its own wavefronts
     of a block and folds them in LDS (four row groups per block, or two for up to eight rows): the bits of the form
-    that walks the parts one after the other, whatever the bench switch picks."""
+    that walks the parts one after the other, whatever the bench switch or the automatic rule picks."""
     lib = _lib.load()
     w = hg.normal_f32(0x7EA0 + n + k, (n, k), 0.02)
     act = hg.normal_bf16(0x7EA1 + n, (m, k))
@@ -419,7 +419,7 @@ def test_parts_of_k_side_by_side_in_a_block_give_the_row_tile_forms_bits(gpu, ki
     outs = {}
     lib.dgpp_tune_set(5, 2)
     try:
-        for knob in (1, 2, 3) if m <= 8 else (1, 2):
+        for knob in (1, 0, 2, 3) if m <= 8 else (1, 0, 2):   # 0: the automatic rule
             lib.dgpp_tune_set(11, knob)
             outs[knob] = dev_empty((m, n), np.float32)
             outs[knob].fill_(-7.0)
