@@ -110,6 +110,14 @@ SIGNATURES = {
     "dgpp_launch_moe_slot_down_fp4_ex": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _P, _I, _P, _P]),
     "dgpp_launch_moe_slot_down_accum": (_I, [_P, _Z, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P]),
     "dgpp_launch_moe_slot_down_accum_fp4": (_I, [_P, _Z, _P, _P, _I, _I, _I, _I, _P, _P, _P, _P, _I]),
+    "dgpp_moe_slot_chain_ready_bytes": (C.c_size_t, [_I, _I]),
+    "dgpp_launch_moe_slot_chain": (_I, [_P, _Z, _P, _P, _I, _I, _P, _I, _I, _I, _F, _P, _P, _P, _P, _P, C.c_uint, _P]),
+    "dgpp_launch_moe_select_slot_chain": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P, _P, _P, _P, C.c_uint,
+                                               _P]),
+    "dgpp_launch_moe_select_slot_chain_fp4": (_I, [_P, _P, _P, _P, _P, _I, _P, _Z, _P, _I, _I, _P, _I, _F, _P, _P, _P, _P,
+                                                   C.c_uint, _P, _I]),
+    "dgpp_launch_moe_slot_chain_fp4": (_I, [_P, _Z, _P, _P, _I, _I, _P, _I, _I, _I, _F, _P, _P, _P, _P, _P, C.c_uint, _P,
+                                            _I]),
     "dgpp_launch_dense_mma_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _Z]),
     "dgpp_launch_dense_mma_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _P, _Z]),
     "dgpp_launch_dense_mma_fp4_bf16": (_I, [_P, _Z, _P, _P, _I, _I, _I, _P]),
@@ -228,6 +236,7 @@ LAYER_SIGNATURES = {
     "dgpp_moe_resident_weight_bytes": (C.c_size_t, [_P]),
     "dgpp_moe_resident_inter": (_I, [_P]),
     "dgpp_moe_layer_views": (_P, [_P]),
+    "dgpp_moe_layer_check": (_I, [_P, _P]),
     "dgpp_moe_layer_ids": (_P, [_P]),
     "dgpp_moe_layer_weights": (_P, [_P]),
 }

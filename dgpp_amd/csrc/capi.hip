@@ -116,6 +116,13 @@ hipError_t launch_grouped(int fmt, const GroupedArgs& a, int n_segs, int z_ext, 
     default: return launch_grouped_fmt<kFmtMxfp4>(a, n_segs, z_ext, s);
   }
 }
+hipError_t launch_slot_chain(int fmt, const ChainArgs& c, const SelectArgs* sel, hipStream_t s) {
+  switch (fmt) {
+    case kFmtFp8F32: return launch_slot_chain_fmt<kFmtFp8F32>(c, sel, s);
+    case kFmtNvfp4: return launch_slot_chain_fmt<kFmtNvfp4>(c, sel, s);
+    default: return launch_slot_chain_fmt<kFmtMxfp4>(c, sel, s);
+  }
+}
 hipError_t launch_token_down(int fmt, const TokenDownArgs& a, hipStream_t s) {
   switch (fmt) {
     case kFmtFp8F32: return launch_token_down_fmt<kFmtFp8F32>(a, s);
@@ -953,6 +960,136 @@ int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, 
     return fail_arg(std::string(who) + ": k must be a multiple of 32 in the fp4 core's compiled set");
   return slot_down_accum(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, act, act_stride, ids, views, n, k, tokens, top_k, weights,
                          out_bf16, out_f32, stream, who);
+}
+
+// The routed chain of a small decode batch in one launch (no counterpart in the reference, which runs
+// launch_moe_slot_gate_up_swiglu*, launch_moe_slot_down* and launch_moe_slot_accum_routed_* back to back). Problems
+// outside the one-launch form run as the two launches it stands for; the bits are the same either way.
+static int slot_chain(int fmt, const uint16_t* x, size_t x_stride, const int32_t* ids, const DgppMoeExpertView* views,
+                      int inter, int hidden, uint16_t* act, int act_stride, int tokens, int top_k, float limit,
+                      const float* weights, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status, unsigned spins,
+                      void* stream, int fp4_group, const char* who, const SelectArgs* sel = nullptr,
+                      const DgppMoeConfig* cfg = nullptr) {
+  if (tokens <= 0) return DGPP_OK;
+  if (!x || !ids || !views || !act || !weights || (!out_bf16 && !out_f32)) return fail_arg(std::string(who) + ": null pointer");
+  if (inter <= 0 || hidden <= 0 || top_k <= 0 || top_k > 16) return fail_arg(std::string(who) + ": degenerate dims (top_k 1..16)");
+  if (act_stride < inter) return fail_arg(std::string(who) + ": act_stride below the expert width");
+  ChainArgs c{};
+  const int slots = tokens * (top_k + 1);
+  c.gu = slot_args(x, x_stride, ids, nullptr, views, act, act_stride, slots, top_k, limit);
+  c.gu.n = inter;
+  c.gu.k = hidden;
+  c.dn.act = act;
+  c.dn.act_stride = static_cast<size_t>(act_stride);
+  c.dn.ids = ids;
+  c.dn.views = views;
+  c.dn.weights = weights;
+  c.dn.out = out_f32 ? static_cast<void*>(out_f32) : static_cast<void*>(out_bf16);
+  c.dn.out_f32 = out_f32 != nullptr;
+  c.dn.n = hidden;
+  c.dn.k = inter;
+  c.dn.tokens = tokens;
+  c.dn.top_k = top_k;
+  c.ready = ready;
+  c.status = status;
+  c.spins = spins;
+  bool one = ready != nullptr && status != nullptr && tune_get(kTuneChain) != 1 && slot_chain_fits(c);
+  if (one && sel != nullptr)   // the selection inside the launch: one token whose score row fits a wavefront's registers
+    one = tokens == 1 && top_k <= kWave && sel->n_experts <= 8 * kWave && tune_get(kTuneSelectAlone) != 1;
+  if (one) {
+    if (fmt == kFmtFp8F32) {
+      one = hidden % 16 == 0 && inter % 16 == 0 && slot_chain_widths_ok<kFmtFp8F32>(hidden, inter);
+    } else {
+      one = fp4_k_supported(hidden) && fp4_k_compiled(hidden, fp4_group) && fp4_k_supported(inter) &&
+            fp4_k_compiled(inter, fp4_group) &&
+            (fmt == kFmtNvfp4 ? slot_chain_widths_ok<kFmtNvfp4>(hidden, inter) : slot_chain_widths_ok<kFmtMxfp4>(hidden, inter));
+    }
+  }
+  if (!one) {
+    int rc;
+    if (sel != nullptr) {   // selection (+ gate/up where that form fits), then the token-major down launch
+      if (fmt == kFmtFp8F32)
+        rc = dgpp_launch_moe_select_gate_up_swiglu(sel->scores, sel->biased, sel->ids, sel->weights, cfg, tokens, x, x_stride, views,
+                                                   inter, hidden, act, act_stride, limit, stream);
+      else
+        rc = dgpp_launch_moe_select_gate_up_swiglu_fp4(sel->scores, sel->biased, sel->ids, sel->weights, cfg, tokens, x, x_stride,
+                                                       views, inter, hidden, act, act_stride, limit, stream, fp4_group);
+    } else if (fmt == kFmtFp8F32) {
+      rc = dgpp_launch_moe_slot_gate_up_swiglu(x, x_stride, ids, nullptr, views, inter, hidden, 0, 0, nullptr, nullptr, nullptr,
+                                               nullptr, act, act_stride, slots, top_k, limit, stream, 7, 7);
+    } else {
+      rc = dgpp_launch_moe_slot_gate_up_swiglu_fp4(x, x_stride, ids, nullptr, views, inter, hidden, 0, 0, nullptr, nullptr, nullptr,
+                                                   nullptr, act, act_stride, slots, top_k, limit, stream, -1, fp4_group, 7, 7);
+    }
+    if (rc != DGPP_OK) return rc;
+    if (fmt == kFmtFp8F32)
+      return dgpp_launch_moe_slot_down_accum(act, static_cast<size_t>(act_stride), ids, views, hidden, inter, tokens, top_k,
+                                             weights, out_bf16, out_f32, stream);
+    return dgpp_launch_moe_slot_down_accum_fp4(act, static_cast<size_t>(act_stride), ids, views, hidden, inter, tokens, top_k,
+                                               weights, out_bf16, out_f32, stream, fp4_group);
+  }
+  return finish(launch_slot_chain(fmt, c, sel, as_stream(stream)), who);
+}
+// The same with the router's selection inside the launch (one token; more tokens select first and go on as above).
+static int select_slot_chain(int fmt, const float* scores, const float* biased, int32_t* ids, float* weights,
+                             const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                             const DgppMoeExpertView* views, int inter, int hidden, uint16_t* act, int act_stride, float limit,
+                             uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status, unsigned spins, void* stream,
+                             int fp4_group, const char* who) {
+  const int rc = dgpp_moe_config_validate(cfg);
+  if (rc != DGPP_OK) return rc;
+  if (tokens <= 0) return DGPP_OK;
+  if (!scores || !biased || !ids || !weights) return fail_arg(std::string(who) + ": null pointer");
+  SelectArgs sel;
+  sel.scores = scores;
+  sel.biased = biased;
+  sel.ids = ids;
+  sel.weights = weights;
+  sel.mode = cfg->router_mode;
+  sel.n_experts = cfg->n_experts;
+  sel.scaling = cfg->routed_scaling_factor;
+  sel.norm_topk = cfg->norm_topk_prob ? 1 : 0;
+  return slot_chain(fmt, x, x_stride, ids, views, inter, hidden, act, act_stride, tokens, cfg->top_k, limit, weights, out_bf16,
+                    out_f32, ready, status, spins, stream, fp4_group, who, &sel, cfg);
+}
+size_t dgpp_moe_slot_chain_ready_bytes(int tokens, int top_k) {
+  if (tokens <= 0 || top_k <= 0) return 0;
+  return static_cast<size_t>(tokens) * static_cast<size_t>(top_k) * kReadyStride * sizeof(uint32_t);
+}
+int dgpp_launch_moe_slot_chain(const uint16_t* x, size_t x_stride, const int32_t* ids, const DgppMoeExpertView* views,
+                               int inter, int hidden, uint16_t* act, int act_stride, int tokens, int top_k, float limit,
+                               const float* weights, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                               unsigned spins, void* stream) {
+  return slot_chain(kFmtFp8F32, x, x_stride, ids, views, inter, hidden, act, act_stride, tokens, top_k, limit, weights, out_bf16,
+                    out_f32, ready, status, spins, stream, 0, "moe_slot_chain");
+}
+int dgpp_launch_moe_slot_chain_fp4(const uint16_t* x, size_t x_stride, const int32_t* ids, const DgppMoeExpertView* views,
+                                   int inter, int hidden, uint16_t* act, int act_stride, int tokens, int top_k, float limit,
+                                   const float* weights, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                   unsigned spins, void* stream, int fp4_group) {
+  const char* who = "moe_slot_chain_fp4";
+  if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
+  return slot_chain(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, x, x_stride, ids, views, inter, hidden, act, act_stride, tokens,
+                    top_k, limit, weights, out_bf16, out_f32, ready, status, spins, stream, fp4_group, who);
+}
+
+int dgpp_launch_moe_select_slot_chain(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                      const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                      const DgppMoeExpertView* views, int inter, int hidden, uint16_t* act, int act_stride,
+                                      float limit, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                      unsigned spins, void* stream) {
+  return select_slot_chain(kFmtFp8F32, scores, biased, ids, weights, cfg, tokens, x, x_stride, views, inter, hidden, act, act_stride,
+                           limit, out_bf16, out_f32, ready, status, spins, stream, 0, "moe_select_slot_chain");
+}
+int dgpp_launch_moe_select_slot_chain_fp4(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                          const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                          const DgppMoeExpertView* views, int inter, int hidden, uint16_t* act, int act_stride,
+                                          float limit, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                          unsigned spins, void* stream, int fp4_group) {
+  const char* who = "moe_select_slot_chain_fp4";
+  if (fp4_group != 16 && fp4_group != 32) return fail_arg(std::string(who) + ": the fp4 scale group must be 16 or 32");
+  return select_slot_chain(fp4_group == 16 ? kFmtNvfp4 : kFmtMxfp4, scores, biased, ids, weights, cfg, tokens, x, x_stride, views,
+                           inter, hidden, act, act_stride, limit, out_bf16, out_f32, ready, status, spins, stream, fp4_group, who);
 }
 
 // ---- matrix-core launchers (src/kernels/glm_moe_launch.hpp:103-125, :311-345; src/kernels/mma_gemv.hpp:65-85) -----

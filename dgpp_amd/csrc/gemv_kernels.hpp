@@ -230,8 +230,7 @@ __device__ __forceinline__ int slot_key(const SlotArgs& a, int slot, int& token)
 }
 
 template <int MAXM>
-__device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& run) {
-  const int p = static_cast<int>(blockIdx.y);
+__device__ __forceinline__ bool resolve_run_at(const SlotArgs& a, SlotRun<MAXM>& run, int p) {
   if (p >= a.slots) return false;
   const int slot0 = a.order ? a.order[p] : p;
   int token0;
@@ -324,13 +323,31 @@ __device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& ru
   }
   return true;
 }
+template <int MAXM>
+__device__ __forceinline__ bool resolve_run(const SlotArgs& a, SlotRun<MAXM>& run) {
+  return resolve_run_at<MAXM>(a, run, static_cast<int>(blockIdx.y));
+}
 
-template <int FMT, int NB, int MAXM, bool SPLIT, bool NT>
-__device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGeom& g, int steps, uint4* __restrict__ lds) {
+// What a gate/up block of the one-launch chain (gemv_chain.hpp) does beyond storing its act values: the values go
+// out as agent-scope stores (written through to where every XCD reads them) and, once every wavefront's stores
+// have been acknowledged, one thread counts the block in on the readiness word of each slot it served.
+struct SlotPublish {
+  unsigned* ready;   // one word per routed slot (index token * top_k + j), `stride` words apart
+  int stride;
+  unsigned wrap;     // the word goes back to zero after wrap + 1 increments
+};
+
+// `p` names the block's position (its slot, or its place in `order`), `tile` its row tile. WAVES wavefronts per
+// block; PUBLISH: the chain form above.
+template <int FMT, int NB, int MAXM, bool SPLIT, bool NT, int WAVES = kWavesPerBlock, bool PUBLISH = false>
+__device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGeom& g, int steps, uint4* __restrict__ lds,
+                                                  int p, int tile, const SlotPublish* pub = nullptr) {
+  constexpr int kThreads = WAVES * kWave;
   SlotRun<MAXM> run;
-  if (!resolve_run<MAXM>(a, run)) return;
-  const int rows_per_block = block_rows(g, steps);
-  if (static_cast<int>(blockIdx.x) * rows_per_block >= a.n) return;
+  if (!resolve_run_at<MAXM>(a, run, p)) return;
+  const int rpw = kWave >> g.l2;
+  const int rows_per_block = WAVES * rpw * steps;
+  if (tile * rows_per_block >= a.n) return;
   MatRef mg, mu;
   const float *gg = nullptr, *gu = nullptr;
   if (run.view_base >= 0) {
@@ -342,13 +359,12 @@ __device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGe
   }
   const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
   const int row_vecs = FmtTraits<FMT>::kPieces * chunks;
-  const int rpw = kWave >> g.l2;
   const int wave = threadIdx.x >> 6;
-  int row0 = blockIdx.x * rows_per_block + wave * rpw;
+  int row0 = tile * rows_per_block + wave * rpw;
   uint16_t* act = static_cast<uint16_t*>(a.out);
   // Fast set-up (rows of at most 4096 aligned elements): activation loads, then the first step's weight
   // loads, then the LDS commit and the barrier — the weights travel while the block sets up.
-  constexpr int XV = kSplitStageVecs;
+  constexpr int XV = (kSplitStageVecs * kBlockThreads + kThreads - 1) / kThreads;
   const auto lg = lane_row<FMT, NT>(mg, row0, a.n, a.k, g.l2);
   const auto lu = lane_row<FMT, NT>(mu, row0, a.n, a.k, g.l2);
   ChunkRegs fg[NB], fu[NB];
@@ -356,12 +372,12 @@ __device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGe
     StageRegs<XV> xr[MAXM];
 #pragma unroll
     for (int r = 0; r < MAXM; ++r)   // every register set is loaded (unused run entries repeat row 0): no partial state
-      stage_issue<FMT, XV>(a.x + static_cast<size_t>(run.token[r]) * a.x_stride, a.k, threadIdx.x, kBlockThreads, xr[r]);
+      stage_issue<FMT, XV>(a.x + static_cast<size_t>(run.token[r]) * a.x_stride, a.k, threadIdx.x, kThreads, xr[r]);
     issue_pass<FMT, NB>(lg, 0, g.l2, mg.cs, fg);
     issue_pass<FMT, NB>(lu, 0, g.l2, mu.cs, fu);
 #pragma unroll
     for (int r = 0; r < MAXM; ++r)
-      if (r < run.m) stage_commit<FMT, XV>(xr[r], a.k, threadIdx.x, kBlockThreads, lds + r * row_vecs);
+      if (r < run.m) stage_commit<FMT, XV>(xr[r], a.k, threadIdx.x, kThreads, lds + r * row_vecs);
   } else {
 #pragma unroll
     for (int r = 0; r < MAXM; ++r)
@@ -374,9 +390,12 @@ __device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGe
     if (l.li == 0 && l.row < a.n) {
 #pragma unroll
       for (int r = 0; r < MAXM; ++r)
-        if (r < run.m)
-          act[static_cast<size_t>(run.slot[r]) * a.out_stride + l.row] =
-              swiglu_bf16(finish_dot<FMT>(ag[r], dg), finish_dot<FMT>(au[r], du), a.limit);
+        if (r < run.m) {
+          const uint16_t v = swiglu_bf16(finish_dot<FMT>(ag[r], dg), finish_dot<FMT>(au[r], du), a.limit);
+          uint16_t* at = act + static_cast<size_t>(run.slot[r]) * a.out_stride + l.row;
+          if constexpr (PUBLISH) __hip_atomic_store(at, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else *at = v;
+        }
     }
   };
   int s = 0;
@@ -387,9 +406,9 @@ __device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGe
       finish(lg, ag, au);
     }
     s = 1;
-    row0 += kWavesPerBlock * rpw;
+    row0 += WAVES * rpw;
   }
-  for (; s < steps; ++s, row0 += kWavesPerBlock * rpw) {
+  for (; s < steps; ++s, row0 += WAVES * rpw) {
     if (row0 >= a.n) break;
     const auto l2g = lane_row<FMT, NT>(mg, row0, a.n, a.k, g.l2);
     const auto l2u = lane_row<FMT, NT>(mu, row0, a.n, a.k, g.l2);
@@ -397,12 +416,22 @@ __device__ __forceinline__ void slot_gate_up_body(const SlotArgs& a, const RowGe
     row_dots_pair<FMT, NB, MAXM>(l2g, l2u, g, mg.cs, mu.cs, lds, chunks, run.m, ag, au);
     finish(l2g, ag, au);
   }
+  if constexpr (PUBLISH) {
+    // vmcnt(0): every act store of this wavefront has been acknowledged by the memory side (a block barrier alone
+    // does not wait for outstanding stores); then the block is counted in, once per slot of its run.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < MAXM; ++r)
+      if (r < run.m && static_cast<int>(threadIdx.x) == r)
+        atomicInc(pub->ready + static_cast<size_t>(run.slot[r] - run.token[r]) * pub->stride, pub->wrap);
+  }
 }
 
 template <int FMT, int NB, int MAXM, bool SPLIT, bool NT>
 __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void slot_gate_up_kernel(SlotArgs a, RowGeom g, int steps) {
   extern __shared__ uint4 lds[];
-  slot_gate_up_body<FMT, NB, MAXM, SPLIT, NT>(a, g, steps, lds);
+  slot_gate_up_body<FMT, NB, MAXM, SPLIT, NT>(a, g, steps, lds, static_cast<int>(blockIdx.y), static_cast<int>(blockIdx.x));
 }
 
 // ---- gate / up in different formats (the per-projection form) -------------------------------------------------------
@@ -499,7 +528,7 @@ __global__ __launch_bounds__(kBlockThreads, kMinWavesPerSimd) void select_gate_u
   __syncthreads();
   SlotArgs b = a;
   b.ids = ids;
-  slot_gate_up_body<FMT, NB, 1, true, true>(b, g, steps, lds);
+  slot_gate_up_body<FMT, NB, 1, true, true>(b, g, steps, lds, static_cast<int>(blockIdx.y), static_cast<int>(blockIdx.x));
 }
 
 // Down rows of a run of slots, unrounded f32.
@@ -576,9 +605,50 @@ struct TokenDownArgs {
   int xcd_group;            // row tiles an XCD takes for one token before it turns to the next token (see the kernel)
 };
 
-template <int FMT, int NB, bool SPLIT>
-__global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a, RowGeom g, int steps) {
-  extern __shared__ uint4 lds[];
+// What a down block of the one-launch chain (gemv_chain.hpp) waits for: its slot's readiness word reaching `need`
+// (the gate/up blocks that serve a slot). The wait is bounded: after `spins` polls the wavefront reports through
+// `status` and goes on with whatever the row holds, so every wavefront of the grid exits.
+struct SlotAwait {
+  unsigned* ready;
+  int stride;
+  unsigned need;
+  unsigned wrap;
+  unsigned spins;
+  int* status;
+};
+// A word above `wrap` was never zeroed by its owner: not ready, and the wait will run out.
+__device__ __forceinline__ bool slot_ready_now(const unsigned* word, unsigned need, unsigned wrap) {
+  const unsigned v = static_cast<unsigned>(
+      __builtin_amdgcn_readfirstlane(static_cast<int>(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))));
+  return v >= need && v <= wrap;
+}
+__device__ __forceinline__ bool slot_wait(const unsigned* word, unsigned need, unsigned wrap, unsigned spins) {
+  for (unsigned i = 0; i < spins; ++i) {
+    if (slot_ready_now(word, need, wrap)) return true;
+    __builtin_amdgcn_s_sleep(16);
+  }
+  return false;
+}
+// stage_issue over a row other XCDs have just written: agent-scope loads (they pass this XCD's L2), 8 bytes each.
+template <int FMT, int XV>
+__device__ __forceinline__ void stage_issue_agent(const uint16_t* __restrict__ x, int k, int tid, int threads, StageRegs<XV>& r) {
+  const int vecs = k / 8;
+#pragma unroll
+  for (int i = 0; i < XV; ++i) {
+    const int v = tid + i * threads;
+    const unsigned long long* src = reinterpret_cast<const unsigned long long*>(x + static_cast<size_t>(v < vecs ? v : 0) * 8);
+    const unsigned long long lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    r.v[i] = make_uint4(static_cast<unsigned>(lo), static_cast<unsigned>(lo >> 32), static_cast<unsigned>(hi),
+                        static_cast<unsigned>(hi >> 32));
+  }
+}
+
+// The body of token_down_accum_kernel for block `b` of its grid. CHAIN: the act rows come from gate/up blocks of the
+// same launch (`aw`); wavefronts beyond top_k (a block sized for the gate/up part) only join the barrier.
+template <int FMT, int NB, bool SPLIT, bool CHAIN>
+__device__ __forceinline__ void token_down_body(const TokenDownArgs& a, const RowGeom& g, int steps, uint4* __restrict__ lds,
+                                                int b, const SlotAwait* aw = nullptr) {
   constexpr int kPieces = FmtTraits<FMT>::kPieces;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
   // Block -> (row tile, token). Consecutive blocks go to the chip's eight XCDs in turn (block b runs on XCD b % 8 as
@@ -589,7 +659,6 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
   // better order while few tokens share experts.
   int t, tile;
   {
-    const int b = static_cast<int>(blockIdx.x);
     const int G = a.xcd_group;
     if (G > 0) {     // tiles is a multiple of 8 * G
       const int seq = b >> 3;
@@ -606,47 +675,70 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
   const int rpw = kWave >> g.l2;
   const int rows_per_block = rpw * steps;
   const int tile_row0 = tile * rows_per_block;
-  uint4* my_x = lds + wave * row_vecs;
   float* part = reinterpret_cast<float*>(lds + a.top_k * row_vecs);   // [top_k][rows_per_block]
-  const float* gd = nullptr;
-  const MatRef md = mat_of_view<FMT>(a.views[a.ids[static_cast<size_t>(t) * a.top_k + wave] * 3 + 2], &gd);
-  // This wavefront's activation row, in the core's [piece][chunk] order. Fast set-up (a row of at most 1024
-  // aligned elements): activation loads, then the first step's weight loads, then the LDS commit.
-  const uint16_t* x = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + wave) * a.act_stride;
-  const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
-  constexpr int XV = kSplitStageVecs;
-  const auto lr = lane_row<FMT, true>(md, tile_row0, a.n, a.k, g.l2);
-  ChunkRegs first[NB];
-  if constexpr (SPLIT) {
-    StageRegs<XV> xr;
-    stage_issue<FMT, XV>(x, a.k, lane, kWave, xr);
-    issue_pass<FMT, NB>(lr, 0, g.l2, md.cs, first);
-    stage_commit<FMT, XV>(xr, a.k, lane, kWave, my_x);
-  } else {
-    for (int v = lane; v < row_vecs; v += kWave) {
-      const int c = v / kPieces, q = v - c * kPieces;
-      my_x[q * chunks + c] = load_vec8(x, v, aligned);
+  if (!CHAIN || wave < a.top_k) {
+    uint4* my_x = lds + wave * row_vecs;
+    const float* gd = nullptr;
+    const MatRef md = mat_of_view<FMT>(a.views[a.ids[static_cast<size_t>(t) * a.top_k + wave] * 3 + 2], &gd);
+    // This wavefront's activation row, in the core's [piece][chunk] order. Fast set-up (a row of at most 1024
+    // aligned elements): activation loads, then the first step's weight loads, then the LDS commit.
+    const uint16_t* x = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + wave) * a.act_stride;
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+    constexpr int XV = kSplitStageVecs;
+    const auto lr = lane_row<FMT, true>(md, tile_row0, a.n, a.k, g.l2);
+    ChunkRegs first[NB];
+    if constexpr (CHAIN) {
+      // The slot's row is complete once every gate/up block that serves it has counted itself in. Ready at the first
+      // look (the common case: gate/up blocks precede the down blocks in the grid): row first, then weights, as
+      // below. Otherwise the first weight loads go out before the wait.
+      static_assert(SPLIT, "the chain form stages a wavefront's row from registers");
+      unsigned* word = aw->ready + (static_cast<size_t>(t) * a.top_k + wave) * aw->stride;
+      StageRegs<XV> xr;
+      bool ok = slot_ready_now(word, aw->need, aw->wrap);
+      if (ok) {
+        stage_issue_agent<FMT, XV>(x, a.k, lane, kWave, xr);
+        issue_pass<FMT, NB>(lr, 0, g.l2, md.cs, first);
+      } else {
+        issue_pass<FMT, NB>(lr, 0, g.l2, md.cs, first);
+        ok = slot_wait(word, aw->need, aw->wrap, aw->spins);
+        stage_issue_agent<FMT, XV>(x, a.k, lane, kWave, xr);
+      }
+      if (lane == 0) {
+        atomicInc(word, aw->wrap);                 // this reader is through: the last one returns the word to zero
+        if (!ok) *aw->status = 1;
+      }
+      stage_commit<FMT, XV>(xr, a.k, lane, kWave, my_x);
+    } else if constexpr (SPLIT) {
+      StageRegs<XV> xr;
+      stage_issue<FMT, XV>(x, a.k, lane, kWave, xr);
+      issue_pass<FMT, NB>(lr, 0, g.l2, md.cs, first);
+      stage_commit<FMT, XV>(xr, a.k, lane, kWave, my_x);
+    } else {
+      for (int v = lane; v < row_vecs; v += kWave) {
+        const int c = v / kPieces, q = v - c * kPieces;
+        my_x[q * chunks + c] = load_vec8(x, v, aligned);
+      }
     }
-  }
-  // The staged row is this wavefront's own: LDS keeps a wavefront's writes and reads in order, no block barrier.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  const float dd = load_divisor<FMT>(gd);
-  int s = 0;
-  if constexpr (SPLIT) {
-    float acc[1];
-    row_dots_pre<FMT, 1, NB>(lr, g, md.cs, my_x, chunks, 1, first, acc);   // tile_row0 < n: the grid covers n
-    if (lr.li == 0) part[wave * rows_per_block + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
-    s = 1;
-  }
-  for (; s < steps; ++s) {
-    const int row0 = tile_row0 + s * rpw;
-    if (row0 >= a.n) break;
-    const auto l2 = lane_row<FMT, true>(md, row0, a.n, a.k, g.l2);
-    float acc[1];
-    row_dots<FMT, 1, NB>(l2, g, md.cs, my_x, chunks, 1, acc);
-    if (l2.li == 0) part[wave * rows_per_block + s * rpw + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
+    // The staged row is this wavefront's own: LDS keeps a wavefront's writes and reads in order, no block barrier.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float dd = load_divisor<FMT>(gd);
+    int s = 0;
+    if constexpr (SPLIT) {
+      float acc[1];
+      row_dots_pre<FMT, 1, NB>(lr, g, md.cs, my_x, chunks, 1, first, acc);   // tile_row0 < n: the grid covers n
+      if (lr.li == 0) part[wave * rows_per_block + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
+      s = 1;
+    }
+    for (; s < steps; ++s) {
+      const int row0 = tile_row0 + s * rpw;
+      if (row0 >= a.n) break;
+      const auto l2 = lane_row<FMT, true>(md, row0, a.n, a.k, g.l2);
+      float acc[1];
+      row_dots<FMT, 1, NB>(l2, g, md.cs, my_x, chunks, 1, acc);
+      if (l2.li == 0) part[wave * rows_per_block + s * rpw + (lane >> g.l2)] = finish_dot<FMT>(acc[0], dd);
+    }
   }
   __syncthreads();
   for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
@@ -661,6 +753,140 @@ __global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a,
     else
       static_cast<uint16_t*>(a.out)[at] = f32_to_bf16(v);
   }
+}
+
+// The token-major down + accumulation block with FOUR wavefronts, each carrying two routed slots of the token (j and
+// j + 4): the form a launch takes whose blocks must match the gate/up blocks' size and register budget (the one-launch
+// chain). A wavefront keeps two row passes in flight - its two slots' - where the eight-wavefront block relies on
+// twice the wavefronts per SIMD. Per (row, slot) the chain is row_dots', the fold the same: the same bits.
+// top_k <= 8, rows of at most 1024 aligned elements. CHAIN as in token_down_body.
+template <int FMT, int NB, bool CHAIN>
+__device__ __forceinline__ void token_down_pair_body(const TokenDownArgs& a, const RowGeom& g, int steps, uint4* __restrict__ lds,
+                                                     int b, const SlotAwait* aw = nullptr) {
+  constexpr int kPieces = FmtTraits<FMT>::kPieces;
+  constexpr int XV = kSplitStageVecs;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+  int t, tile;
+  {
+    const int G = a.xcd_group;
+    if (G > 0) {     // tiles is a multiple of 8 * G (see token_down_body)
+      const int seq = b >> 3;
+      const int gi = seq % G, rest = seq / G;
+      t = rest % a.tokens;
+      tile = ((rest / a.tokens) * G + gi) * 8 + (b & 7);
+    } else {
+      t = b / a.tiles;
+      tile = b - t * a.tiles;
+    }
+  }
+  const int chunks = a.k / FmtTraits<FMT>::kElemsPerChunk;
+  const int row_vecs = kPieces * chunks;
+  const int rpw = kWave >> g.l2;
+  const int rows_per_block = rpw * steps;
+  const int tile_row0 = tile * rows_per_block;
+  float* part = reinterpret_cast<float*>(lds + a.top_k * row_vecs);   // [top_k][rows_per_block]
+  const int j0 = wave, j1 = wave + kWavesPerBlock;
+  if (j0 < a.top_k) {
+    const bool two = j1 < a.top_k;
+    const int jb = two ? j1 : j0;
+    const size_t r0 = static_cast<size_t>(t) * a.top_k + j0, r1 = static_cast<size_t>(t) * a.top_k + jb;
+    // wave-uniform by construction: saying so keeps the table entries in scalar registers
+    const int e0 = __builtin_amdgcn_readfirstlane(a.ids[r0]), e1 = __builtin_amdgcn_readfirstlane(a.ids[r1]);
+    unsigned v0 = 0, v1 = 0;
+    unsigned *w0 = nullptr, *w1 = nullptr;
+    if constexpr (CHAIN) {
+      // The readiness words are asked for before the table entries: their trip to the memory side runs beside the
+      // ids -> entry -> address chain.
+      w0 = aw->ready + r0 * aw->stride;
+      w1 = aw->ready + r1 * aw->stride;
+      v0 = __hip_atomic_load(w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v1 = __hip_atomic_load(w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const float *gd0 = nullptr, *gd1 = nullptr;
+    const MatRef m0 = mat_of_view<FMT>(a.views[e0 * 3 + 2], &gd0);
+    const MatRef m1 = mat_of_view<FMT>(a.views[e1 * 3 + 2], &gd1);
+    const uint16_t* x0 = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + j0) * a.act_stride;
+    const uint16_t* x1 = a.act + (static_cast<size_t>(t) * (a.top_k + 1) + jb) * a.act_stride;
+    uint4* my0 = lds + j0 * row_vecs;
+    uint4* my1 = lds + jb * row_vecs;
+    auto lr0 = lane_row<FMT, true>(m0, tile_row0, a.n, a.k, g.l2);
+    auto lr1 = lane_row<FMT, true>(m1, tile_row0, a.n, a.k, g.l2);
+    ChunkRegs f0[NB], f1[NB];
+    StageRegs<XV> xa, xb;
+    if constexpr (CHAIN) {
+      auto ready = [&](unsigned v) {
+        const unsigned u = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(v)));
+        return u >= aw->need && u <= aw->wrap;
+      };
+      // The first weight passes go out before the rows are looked for: they travel while the wavefront waits.
+      issue_pass<FMT, NB>(lr0, 0, g.l2, m0.cs, f0);
+      if (two) issue_pass<FMT, NB>(lr1, 0, g.l2, m1.cs, f1);
+      bool ok = ready(v0) && (!two || ready(v1));
+      if (!ok) {
+        ok = slot_wait(w0, aw->need, aw->wrap, aw->spins);
+        if (two) ok = slot_wait(w1, aw->need, aw->wrap, aw->spins) && ok;
+      }
+      stage_issue_agent<FMT, XV>(x0, a.k, lane, kWave, xa);
+      if (two) stage_issue_agent<FMT, XV>(x1, a.k, lane, kWave, xb);
+      if (lane == 0) {
+        atomicInc(w0, aw->wrap);                   // this reader is through: the last one returns the word to zero
+        if (two) atomicInc(w1, aw->wrap);
+        if (!ok) *aw->status = 1;
+      }
+    } else {
+      stage_issue<FMT, XV>(x0, a.k, lane, kWave, xa);
+      if (two) stage_issue<FMT, XV>(x1, a.k, lane, kWave, xb);
+      issue_pass<FMT, NB>(lr0, 0, g.l2, m0.cs, f0);
+      if (two) issue_pass<FMT, NB>(lr1, 0, g.l2, m1.cs, f1);
+    }
+    stage_commit<FMT, XV>(xa, a.k, lane, kWave, my0);
+    if (two) stage_commit<FMT, XV>(xb, a.k, lane, kWave, my1);
+    // The staged rows are this wavefront's own: LDS keeps a wavefront's writes and reads in order, no block barrier.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float dd0 = load_divisor<FMT>(gd0), dd1 = load_divisor<FMT>(gd1);
+    for (int s = 0; s < steps; ++s) {
+      const int row0 = tile_row0 + s * rpw;
+      if (row0 >= a.n) break;
+      const bool more = s + 1 < steps && row0 + rpw < a.n;
+      const int at = s * rpw + (lane >> g.l2);
+      float acc[1];
+      row_dots_pre<FMT, 1, NB>(lr0, g, m0.cs, my0, chunks, 1, f0, acc);
+      if (lr0.li == 0) part[j0 * rows_per_block + at] = finish_dot<FMT>(acc[0], dd0);
+      if (more) {   // this slot's next row group goes out while the other slot's current one is consumed
+        lr0 = lane_row<FMT, true>(m0, row0 + rpw, a.n, a.k, g.l2);
+        issue_pass<FMT, NB>(lr0, 0, g.l2, m0.cs, f0);
+      }
+      if (two) {
+        row_dots_pre<FMT, 1, NB>(lr1, g, m1.cs, my1, chunks, 1, f1, acc);
+        if (lr1.li == 0) part[j1 * rows_per_block + at] = finish_dot<FMT>(acc[0], dd1);
+        if (more) {
+          lr1 = lane_row<FMT, true>(m1, row0 + rpw, a.n, a.k, g.l2);
+          issue_pass<FMT, NB>(lr1, 0, g.l2, m1.cs, f1);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int r = threadIdx.x; r < rows_per_block; r += blockDim.x) {
+    const int row = tile_row0 + r;
+    if (row >= a.n) break;
+    float v = 0.f;
+    for (int j = 0; j < a.top_k; ++j)
+      v = fmaf(a.weights[static_cast<size_t>(t) * a.top_k + j], part[j * rows_per_block + r], v);
+    const size_t at = static_cast<size_t>(t) * a.n + row;
+    if (a.out_f32)
+      static_cast<float*>(a.out)[at] = v;
+    else
+      static_cast<uint16_t*>(a.out)[at] = f32_to_bf16(v);
+  }
+}
+
+template <int FMT, int NB, bool SPLIT>
+__global__ __launch_bounds__(1024) void token_down_accum_kernel(TokenDownArgs a, RowGeom g, int steps) {
+  extern __shared__ uint4 lds[];
+  token_down_body<FMT, NB, SPLIT, false>(a, g, steps, lds, static_cast<int>(blockIdx.x));
 }
 
 // ---- grouped (segment-major) twin ------------------------------------------------------------------
@@ -772,6 +998,45 @@ hipError_t launch_dense_mma_pair_fp8(const DenseArgs& a0, const DenseArgs& a1, f
 hipError_t launch_grouped_mma(int fmt, const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
 template <int FMT> hipError_t launch_dense_mma_fmt(const DenseArgs& a, float* ws, size_t ws_bytes, hipStream_t stream);
 template <int FMT> hipError_t launch_grouped_mma_fmt(const GroupedArgs& a, int n_segs, int z_ext, hipStream_t stream);
+
+// ---- the routed chain in one launch (gemv_chain.hpp) -------------------------------------------------------
+constexpr int kReadyStride = 32;            // words between two slots' readiness words: a 128-byte line each
+constexpr unsigned kChainDefaultSpins = 1u << 18;
+
+struct ChainArgs {
+  SlotArgs gu;        // x rows, ids, views, out = act [slots, out_stride], n = inter, k = hidden
+  TokenDownArgs dn;   // act rows, ids, views, weights, out, n = hidden, k = inter
+  unsigned* ready;    // [tokens * top_k * kReadyStride], zero at rest
+  int* status;        // one word, raised when a wait gave up
+  int gu_tiles;       // gate/up row tiles per slot
+  int gu_blocks;      // gu_tiles * tokens * top_k
+  unsigned spins;
+};
+
+// Whether the one-launch form takes this problem (otherwise the caller runs the two launches).
+inline bool slot_chain_fits(const ChainArgs& c) {
+  const SlotArgs& u = c.gu;
+  const TokenDownArgs& d = c.dn;
+  const int K = u.top_k;
+  if (K < 1 || K > 8 || d.tokens < 1 || d.tokens * K > 128) return false;
+  if (tune_get(kTuneCore) == 2 || tune_get(kTuneSplitStage) == 1) return false;
+  // the fast set-ups of both parts: whole rows held in registers between their loads and the LDS commit
+  if (u.k > 8 * kSplitStageVecs * kBlockThreads || (u.x_stride & 7u) != 0 || (reinterpret_cast<uintptr_t>(u.x) & 15u) != 0) return false;
+  if (d.k > 8 * kSplitStageVecs * kWave || (d.act_stride & 7u) != 0 || (reinterpret_cast<uintptr_t>(d.act) & 15u) != 0) return false;
+  return true;
+}
+
+// The pass widths the chain kernel is compiled for (a lane's loads in flight per row and pass: 1, 2 or 4).
+template <int FMT>
+inline bool slot_chain_widths_ok(int k_gate_up, int k_down) {
+  const int a = geom_for<FMT>(k_gate_up).nb, b = geom_for<FMT>(k_down).nb;
+  auto ok = [](int nb) { return nb == 1 || nb == 2 || nb == 4; };
+  return ok(a) && ok(b);
+}
+
+// `sel` non-null: one token, the selection repeated by every block (select_chain_kernel).
+hipError_t launch_slot_chain(int fmt, const ChainArgs& c, const SelectArgs* sel, hipStream_t stream);
+template <int FMT> hipError_t launch_slot_chain_fmt(const ChainArgs& c, const SelectArgs* sel, hipStream_t stream);
 
 // Per-format implementations.
 template <int FMT> hipError_t launch_dense_fmt(const DenseArgs& a, hipStream_t stream);

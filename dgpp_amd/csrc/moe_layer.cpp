@@ -36,7 +36,8 @@ Layout layout_of(const GlmMoeConfig& c, int max_tokens, int shared_inter, size_t
   l.slot_act = align_up(slots * I * 2);
   l.slot_down = align_up(slots * H * 4);
   l.acc = align_up(M * H * 4);
-  l.counter = align_up(2 * sizeof(int));
+  // the stealing pair, the one-launch chain's status word (at +64 bytes) and its readiness words (from +256 bytes)
+  l.counter = align_up(256 + M * K * 128);
   l.rows = align_up(slots * 4);
   l.slot_row = align_up(M * K * 4);
   l.segs = align_up((E + 1) * sizeof(MoeSegment));
@@ -161,6 +162,9 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   d_slot_down_ = reinterpret_cast<float*>(carve(l.slot_down));
   d_acc_ = reinterpret_cast<float*>(carve(l.acc));
   d_tile_counter_ = reinterpret_cast<int*>(carve(l.counter));
+  d_chain_status_ = d_tile_counter_ + 16;
+  d_chain_ready_ = reinterpret_cast<uint32_t*>(d_tile_counter_ + 64);
+  counter_bytes_ = l.counter;
   d_rows_ = reinterpret_cast<int32_t*>(carve(l.rows));
   d_slot_row_ = reinterpret_cast<int32_t*>(carve(l.slot_row));
   d_segs_ = reinterpret_cast<MoeSegment*>(carve(l.segs));
@@ -203,7 +207,7 @@ GlmMoeLayer::GlmMoeLayer(const GlmMoeConfig& cfg, const GlmMoeLayerWeights& w, i
   // device table once too, src/models/glm/moe_layer.cpp:364-396); the counter pair is zero at rest.
   hip_ok(hipMemcpy(d_views_, w.views.data(), w.views.size() * sizeof(MoeExpertView), hipMemcpyHostToDevice),
          "GlmMoeLayer: table upload");
-  hip_ok(hipMemset(d_tile_counter_, 0, 2 * sizeof(int)), "GlmMoeLayer: counter");
+  hip_ok(hipMemset(d_tile_counter_, 0, counter_bytes_), "GlmMoeLayer: counters");
   if (has_shared()) {
     hip_ok(hipStreamCreateWithFlags(&side_, hipStreamNonBlocking), "GlmMoeLayer: side stream");
     hip_ok(hipEventCreateWithFlags(&fork_, hipEventDisableTiming), "GlmMoeLayer: event");
@@ -234,6 +238,18 @@ bool GlmMoeLayer::needs_order(int tokens) const {
   if (tokens <= 1 || tokens * (cfg_.top_k + 1) > 1024) return false;
   if (dgpp_tune_get(6) == 1) return true;
   return tokens * cfg_.top_k > 128;   // up to 128 routed slots the gate/up kernel finds the sharers of an expert by ballot
+}
+
+// Waits for `stream` and reads the one-launch chain's status word: a launch whose bounded wait ran out has
+// produced nothing valid. The counters are put back to rest before the error is raised.
+void GlmMoeLayer::check(hipStream_t stream) {
+  hip_ok(hipStreamSynchronize(stream), "GlmMoeLayer: check");
+  int status = 0;
+  hip_ok(hipMemcpy(&status, d_chain_status_, sizeof(int), hipMemcpyDeviceToHost), "GlmMoeLayer: check");
+  if (status == 0) return;
+  hip_ok(hipMemset(d_tile_counter_, 0, counter_bytes_), "GlmMoeLayer: counters");
+  throw std::runtime_error("GlmMoeLayer: a one-launch expert chain gave up waiting for its gate/up rows; the output of "
+                           "that call is invalid");
 }
 
 void GlmMoeLayer::check_tokens(int tokens) const {
@@ -352,7 +368,24 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
   };
   const float* fold_w = fold_accum ? weights : nullptr;
   uint16_t* fold_o = fold_accum ? out_bf16 : nullptr;
+  // Routed only, a small batch: gate/up, down and the accumulation in ONE launch (dgpp_launch_moe_slot_chain*), with
+  // the selection of a one-token step inside it. Measured slower than the launches it stands for on this chip at
+  // every batch size (one register budget for both parts, and the readers' polls of the readiness words), so the
+  // driver takes it only under bench switch 12 = 2.
+  const bool one_launch = token_major && !fused && dgpp_tune_get(12) == 2;
+  const bool one_launch_sel = token_major && fused && dgpp_tune_get(12) == 2;
   if (w_.format == GlmExpertFormat::Fp8) {
+    if (one_launch_sel) {
+      launch_moe_select_slot_chain(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
+                                   d_slot_act_, max_inter_, cfg_.swiglu_limit, out_bf16, out_f32, d_chain_ready_,
+                                   d_chain_status_, stream);
+      return;
+    }
+    if (one_launch) {
+      launch_moe_slot_chain(x, x_stride, ids, d_views_, I, H, d_slot_act_, max_inter_, tokens, K, cfg_.swiglu_limit, weights,
+                            out_bf16, out_f32, d_chain_ready_, d_chain_status_, stream);
+      return;
+    }
     if (fused) {
       launch_moe_select_gate_up_swiglu(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
                                        d_slot_act_, max_inter_, cfg_.swiglu_limit, stream);
@@ -378,6 +411,17 @@ void GlmMoeLayer::expert_chain_slots(const uint16_t* x, size_t x_stride, const i
     });
   } else {
     const int base = w_.shared_in_table ? cfg_.n_experts * 3 : -1;
+    if (one_launch_sel) {
+      launch_moe_select_slot_chain_fp4(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I, H,
+                                       d_slot_act_, max_inter_, cfg_.swiglu_limit, out_bf16, out_f32, d_chain_ready_,
+                                       d_chain_status_, stream, fp4_group_);
+      return;
+    }
+    if (one_launch) {
+      launch_moe_slot_chain_fp4(x, x_stride, ids, d_views_, I, H, d_slot_act_, max_inter_, tokens, K, cfg_.swiglu_limit,
+                                weights, out_bf16, out_f32, d_chain_ready_, d_chain_status_, stream, fp4_group_);
+      return;
+    }
     if (fused) {
       launch_moe_select_gate_up_swiglu_fp4(sel_scores, sel_biased, d_ids_, d_weights_, cfg_, tokens, x, x_stride, d_views_, I,
                                            H, d_slot_act_, max_inter_, cfg_.swiglu_limit, stream, fp4_group_);
@@ -766,6 +810,9 @@ int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* l, const uint16_t* 
     l->impl.enqueue_prefill_routed_w4a4(x, x_stride, ids, weights, out_bf16, out_f32, tokens,
                                         static_cast<hipStream_t>(stream), act_scales_dev, f32_down != 0);
   });
+}
+int dgpp_moe_layer_check(DgppMoeLayer* l, void* stream) {
+  return guarded([&] { l->impl.check(static_cast<hipStream_t>(stream)); });
 }
 const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* l) { return l->impl.views(); }
 const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* l) { return l->impl.ids(); }

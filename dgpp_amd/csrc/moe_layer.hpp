@@ -44,6 +44,9 @@ class GlmMoeLayer {
   // out_f32 non-null: the unrounded chain goes there and out_bf16 is not written.
   void enqueue_decode(const uint16_t* x, size_t x_stride, uint16_t* out_bf16, float* out_f32, int tokens,
                       hipStream_t stream);
+  // Synchronizes `stream` and throws std::runtime_error when a one-launch expert chain enqueued on it gave up its
+  // bounded wait (its output is then invalid); the counters are back at rest afterwards.
+  void check(hipStream_t stream);
   void enqueue_decode_scores(const uint16_t* x, size_t x_stride, const float* scores, const float* biased,
                              uint16_t* out_bf16, float* out_f32, int tokens, hipStream_t stream);
   void enqueue_decode_routed(const uint16_t* x, size_t x_stride, const int32_t* ids, const float* weights,
@@ -106,6 +109,9 @@ class GlmMoeLayer {
   float* d_slot_down_ = nullptr;     // [slots, hidden]
   float* d_acc_ = nullptr;           // [tokens, hidden]
   int* d_tile_counter_ = nullptr;    // [2]
+  int* d_chain_status_ = nullptr;    // raised by a one-launch chain whose bounded wait ran out
+  uint32_t* d_chain_ready_ = nullptr;   // the one-launch chain's readiness words, zero at rest
+  size_t counter_bytes_ = 0;
   // The shared expert's passes run beside the routed ones: a second stream of the default priority, forked from
   // and joined to the caller's stream with two events (created only for a layer with a shared expert).
   hipStream_t side_ = nullptr;

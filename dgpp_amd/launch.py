@@ -300,6 +300,45 @@ def launch_moe_slot_down_accum_fp4(act, act_stride, ids, views, n, k, tokens, to
                                                            fp4_group))
 
 
+def moe_slot_chain_ready_bytes(tokens, top_k):
+    return int(_lib.load().dgpp_moe_slot_chain_ready_bytes(tokens, top_k))
+
+
+def launch_moe_slot_chain(x, x_stride, ids, views, inter, hidden, act, act_stride, tokens, top_k, limit, weights, out_bf16,
+                          out_f32, ready, status, spins=0, stream=None):
+    """Extension: the routed chain (gate/up + SwiGLU, down, accumulation) of a small decode batch in one launch (FP8)."""
+    _check(_lib.load().dgpp_launch_moe_slot_chain(_p(x), x_stride, _p(ids), _p(views), inter, hidden, _p(act), act_stride,
+                                                  tokens, top_k, limit, _p(weights), _p(out_bf16), _p(out_f32), _p(ready),
+                                                  _p(status), spins, _stream(stream)))
+
+
+def launch_moe_slot_chain_fp4(x, x_stride, ids, views, inter, hidden, act, act_stride, tokens, top_k, limit, weights,
+                              out_bf16, out_f32, ready, status, spins=0, stream=None, fp4_group=16):
+    """Extension: the routed chain of a small decode batch in one launch (NVFP4 / MXFP4 experts)."""
+    _check(_lib.load().dgpp_launch_moe_slot_chain_fp4(_p(x), x_stride, _p(ids), _p(views), inter, hidden, _p(act), act_stride,
+                                                      tokens, top_k, limit, _p(weights), _p(out_bf16), _p(out_f32),
+                                                      _p(ready), _p(status), spins, _stream(stream), fp4_group))
+
+
+def launch_moe_select_slot_chain(scores, biased, ids, weights, cfg: MoeConfig, tokens, x, x_stride, views, inter, hidden, act,
+                                 act_stride, limit, out_bf16, out_f32, ready, status, spins=0, stream=None):
+    """Extension: selection + the routed chain in one launch for a one-token step (FP8; ids and weights are outputs)."""
+    _check(_lib.load().dgpp_launch_moe_select_slot_chain(_p(scores), _p(biased), _p(ids), _p(weights), C.addressof(cfg), tokens,
+                                                         _p(x), x_stride, _p(views), inter, hidden, _p(act), act_stride, limit,
+                                                         _p(out_bf16), _p(out_f32), _p(ready), _p(status), spins,
+                                                         _stream(stream)))
+
+
+def launch_moe_select_slot_chain_fp4(scores, biased, ids, weights, cfg: MoeConfig, tokens, x, x_stride, views, inter, hidden,
+                                     act, act_stride, limit, out_bf16, out_f32, ready, status, spins=0, stream=None,
+                                     fp4_group=16):
+    """Extension: selection + the routed chain in one launch for a one-token step (NVFP4 / MXFP4)."""
+    _check(_lib.load().dgpp_launch_moe_select_slot_chain_fp4(_p(scores), _p(biased), _p(ids), _p(weights), C.addressof(cfg),
+                                                             tokens, _p(x), x_stride, _p(views), inter, hidden, _p(act),
+                                                             act_stride, limit, _p(out_bf16), _p(out_f32), _p(ready),
+                                                             _p(status), spins, _stream(stream), fp4_group))
+
+
 # ---- grouped twins ---------------------------------------------------------------------------------------
 def launch_moe_grouped_gemv_bf16(act, act_stride, segs, n_segs, max_rows, rows_per_block, views, which, out,
                                  out_stride, n, k, stream=None):

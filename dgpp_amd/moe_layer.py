@@ -75,6 +75,10 @@ class MoeLayer:
         _check(self._lib.dgpp_moe_layer_enqueue_decode_routed(self._h, _p(x), x_stride, _p(ids), _p(weights),
                                                               _p(out_bf16), _p(out_f32), tokens, _stream(stream)))
 
+    def check(self, stream=None):
+        """Synchronizes the stream; raises when a one-launch expert chain on it gave up its bounded wait."""
+        _check(self._lib.dgpp_moe_layer_check(self._h, _stream(stream)))
+
     def enqueue_grouped_routed(self, x, x_stride, ids, weights, out_bf16, tokens, stream=None, out_f32=None):
         _check(self._lib.dgpp_moe_layer_enqueue_grouped_routed(self._h, _p(x), x_stride, _p(ids), _p(weights),
                                                                _p(out_bf16), _p(out_f32), tokens, _stream(stream)))

@@ -319,6 +319,47 @@ int dgpp_launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_stride, 
                                         const float* weights, uint16_t* out_bf16, float* out_f32, void* stream,
                                         int fp4_group);
 
+/* Extension (no counterpart in the reference, whose decode walk runs launch_moe_slot_gate_up_swiglu*,
+ * launch_moe_slot_down* and launch_moe_slot_accum_routed_* back to back, src/models/glm/moe_layer.cpp:1641-1677):
+ * the routed experts' whole chain of a small decode batch in ONE launch. The gate/up + SwiGLU blocks lead the
+ * grid, the token-major down + accumulation blocks follow it and read a slot's act row once the slot's
+ * readiness word says that every gate/up block that serves it has stored its values. Bit-identical to the
+ * launches it stands for. x: token rows [tokens, x_stride]; act: scratch [tokens * (top_k + 1), act_stride]
+ * (slot = t * (top_k + 1) + j, as the slot launchers lay it out); weights: [tokens, top_k]; out_f32 (when given)
+ * or out_bf16: [tokens, hidden]. `ready`: dgpp_moe_slot_chain_ready_bytes(tokens, top_k) bytes of device memory the
+ * caller zeroes ONCE; every launch leaves them zero (as the reference's counters are left,
+ * src/kernels/glm_moe.cu:2092-2099), so a captured launch replays without a memset. `status`: one device int the
+ * caller zeroes once; a wavefront whose bounded wait (`spins` polls, 0 = the default) ran out raises it and
+ * finishes with whatever the row held — a non-zero status after a synchronisation means the launch's output
+ * is invalid (and `ready` must be zeroed again). Launches that share `ready` must not overlap. Problems outside
+ * the one-launch form (more than 128 routed slots, top_k above 8, rows that do not fit the register stages,
+ * ready or status null) run as the launches above, same bits. Routed slots only. */
+size_t dgpp_moe_slot_chain_ready_bytes(int tokens, int top_k);
+int dgpp_launch_moe_slot_chain(const uint16_t* x, size_t x_stride, const int32_t* ids, const DgppMoeExpertView* views,
+                               int inter, int hidden, uint16_t* act, int act_stride, int tokens, int top_k, float limit,
+                               const float* weights, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                               unsigned spins, void* stream);
+int dgpp_launch_moe_slot_chain_fp4(const uint16_t* x, size_t x_stride, const int32_t* ids, const DgppMoeExpertView* views,
+                                   int inter, int hidden, uint16_t* act, int act_stride, int tokens, int top_k, float limit,
+                                   const float* weights, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                   unsigned spins, void* stream, int fp4_group);
+
+/* The same with the router's selection inside the launch (the reference's fused form selects inside its router
+ * launch, src/kernels/glm_moe.cu:840-890; here a one-token step is ONE launch from score rows to the output row):
+ * every block's first wavefront repeats the selection, block 0 stores ids / weights [tokens, top_k] for the caller.
+ * One token and at most 512 experts take that form; anything else runs dgpp_launch_moe_select_gate_up_swiglu* (or the
+ * selection alone) and goes on as dgpp_launch_moe_slot_chain* would. Same bits. */
+int dgpp_launch_moe_select_slot_chain(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                      const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                      const DgppMoeExpertView* views, int inter, int hidden, uint16_t* act, int act_stride,
+                                      float limit, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                      unsigned spins, void* stream);
+int dgpp_launch_moe_select_slot_chain_fp4(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                          const DgppMoeConfig* cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                          const DgppMoeExpertView* views, int inter, int hidden, uint16_t* act, int act_stride,
+                                          float limit, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                          unsigned spins, void* stream, int fp4_group);
+
 /* src/kernels/glm_moe_launch.hpp:77-87 */
 int dgpp_launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride,
                                       const DgppMoeSegment* segs, int n_segs, int max_rows,

@@ -332,6 +332,40 @@ inline void launch_moe_slot_down_accum_fp4(const uint16_t* act, size_t act_strid
   detail::check(dgpp_launch_moe_slot_down_accum_fp4(act, act_stride, ids, views, n, k, tokens, top_k, weights, out_bf16,
                                                     out_f32, stream, fp4_group));
 }
+inline size_t moe_slot_chain_ready_bytes(int tokens, int top_k) { return dgpp_moe_slot_chain_ready_bytes(tokens, top_k); }
+inline void launch_moe_slot_chain(const uint16_t* x, size_t x_stride, const int32_t* ids, const MoeExpertView* views, int inter,
+                                  int hidden, uint16_t* act, int act_stride, int tokens, int top_k, float limit,
+                                  const float* weights, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                  hipStream_t stream, unsigned spins = 0) {
+  detail::check(dgpp_launch_moe_slot_chain(x, x_stride, ids, views, inter, hidden, act, act_stride, tokens, top_k, limit,
+                                           weights, out_bf16, out_f32, ready, status, spins, stream));
+}
+inline void launch_moe_slot_chain_fp4(const uint16_t* x, size_t x_stride, const int32_t* ids, const MoeExpertView* views,
+                                      int inter, int hidden, uint16_t* act, int act_stride, int tokens, int top_k, float limit,
+                                      const float* weights, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                      hipStream_t stream, int fp4_group = kFp4Group, unsigned spins = 0) {
+  detail::check(dgpp_launch_moe_slot_chain_fp4(x, x_stride, ids, views, inter, hidden, act, act_stride, tokens, top_k, limit,
+                                               weights, out_bf16, out_f32, ready, status, spins, stream, fp4_group));
+}
+inline void launch_moe_select_slot_chain(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                         const GlmMoeConfig& cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                         const MoeExpertView* views, int inter, int hidden, uint16_t* act, int act_stride,
+                                         float limit, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                         hipStream_t stream, unsigned spins = 0) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_select_slot_chain(scores, biased, ids, weights, &c, tokens, x, x_stride, views, inter, hidden, act,
+                                                  act_stride, limit, out_bf16, out_f32, ready, status, spins, stream));
+}
+inline void launch_moe_select_slot_chain_fp4(const float* scores, const float* biased, int32_t* ids, float* weights,
+                                             const GlmMoeConfig& cfg, int tokens, const uint16_t* x, size_t x_stride,
+                                             const MoeExpertView* views, int inter, int hidden, uint16_t* act, int act_stride,
+                                             float limit, uint16_t* out_bf16, float* out_f32, uint32_t* ready, int* status,
+                                             hipStream_t stream, int fp4_group = kFp4Group, unsigned spins = 0) {
+  const DgppMoeConfig c = cfg.c_config();
+  detail::check(dgpp_launch_moe_select_slot_chain_fp4(scores, biased, ids, weights, &c, tokens, x, x_stride, views, inter, hidden,
+                                                      act, act_stride, limit, out_bf16, out_f32, ready, status, spins, stream,
+                                                      fp4_group));
+}
 inline void launch_moe_grouped_gemv_bf16(const uint16_t* act, size_t act_stride, const MoeSegment* segs, int n_segs,
                                          int max_rows, int rows_per_block, const MoeExpertView* views, int which,
                                          uint16_t* out, size_t out_stride, int n, int k, hipStream_t stream) {

@@ -31,8 +31,10 @@ extern "C" {
  * wavefront (0 = automatic: tiled from 32 rows on, 4 tokens from 128 rows on); key 11: the dense matrix-core launch
  * without a workspace that runs the four parts of K side by side inside a block: 1 never, 2 always with four row groups
  * per block, 3 with two for up to eight rows (0 = automatic: four while the row tiles fit one round of the chip, two for up
- * to a round and a quarter). Outputs do not depend on keys
- * 1 - 4 and 6 - 11; keys 0 and
+ * to a round and a quarter); key 12: 1 makes dgpp_launch_moe_slot_chain* run the launches the one-launch chain stands for, 2 makes
+ * the layer driver take the one-launch chain for small routed-only decode batches (default: the driver runs the
+ * launches; the chain measured slower); key 13: row steps per wavefront of the chain's down part (0 = automatic). Outputs do not depend on keys
+ * 1 - 4 and 6 - 13; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
  * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);

@@ -104,6 +104,12 @@ int dgpp_moe_layer_accumulate_prefill_rows(DgppMoeLayer* layer, uint16_t* out_bf
 int dgpp_moe_layer_enqueue_prefill_routed_w4a4(DgppMoeLayer* layer, const uint16_t* x, size_t x_stride, const int32_t* ids,
                                                const float* weights, uint16_t* out_bf16, float* out_f32, int tokens,
                                                void* stream, const float* act_scales_dev, int f32_down);
+/* Waits for `stream` and reports whether a decode call enqueued on it ended with its one-launch expert chain
+ * (dgpp_launch_moe_slot_chain*) giving up the bounded wait for its gate/up rows: DGPP_RUNTIME_ERROR then (that
+ * call's output is invalid; the layer's counters are back at rest), DGPP_OK otherwise. Synchronizes: not for
+ * use under stream capture. No counterpart in the reference, whose launches wait for each other at launch
+ * boundaries only. */
+int dgpp_moe_layer_check(DgppMoeLayer* layer, void* stream);
 /* Device pointers of the last routes the layer computed: ids int32 [tokens, top_k], weights f32. */
 const DgppMoeExpertView* dgpp_moe_layer_views(const DgppMoeLayer* layer); /* the device expert table */
 const int32_t* dgpp_moe_layer_ids(const DgppMoeLayer* layer);
