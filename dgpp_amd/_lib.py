@@ -93,6 +93,7 @@ SIGNATURES = {
     "dgpp_moe_run_groups_max": (_I, [_I]),
     "dgpp_launch_moe_slot_order": (_I, [_P, _P, _I, _I, _I, _P, _I, _P]),
     "dgpp_minimax_compact_segments": (_I, [_P, _P, _I, _I, _P]),
+    "dgpp_minimax_router": (_I, [_P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P]),
     "dgpp_launch_moe_accum_ordered": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _I, _P]),
     "dgpp_launch_moe_accum_ordered_f32": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _I, _P]),
     "dgpp_launch_moe_accum_ordered_bf16down": (_I, [_P, _P, _Z, _P, _P, _P, _I, _I, _I, _P]),

@@ -17,6 +17,10 @@ CSRC = PKG / "csrc"
 BUILD = PKG / "_build"
 LIB_DIR = PKG / "lib"
 LIB = LIB_DIR / "libdgpp_amd.so"
+# A C++ host program over include/dgpp_amd.hpp (reference-style host code calling the dgpp::launch_* names), run by
+# the GPU tests as a subprocess.
+HOST_PROGRAM_SRC = PKG.parent / "tests" / "cpp" / "host_program.cpp"
+HOST_PROGRAM = LIB_DIR / "dgpp_host_program"
 
 HIP_SOURCES = [
     "gemv_mxfp4.hip",
@@ -88,6 +92,11 @@ def build(force: bool = True, jobs: int = 6) -> Path:
     with cf.ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(_run, tasks))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB), *map(str, objs)])
+    if HOST_PROGRAM_SRC.exists() and (force or not HOST_PROGRAM.exists() or
+                                      HOST_PROGRAM.stat().st_mtime < max(HOST_PROGRAM_SRC.stat().st_mtime, LIB.stat().st_mtime)):
+        # host code only (no kernels of its own): it finds the library next to itself
+        _run([HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++17", str(HOST_PROGRAM_SRC), "-o", str(HOST_PROGRAM),
+              f"-L{LIB_DIR}", "-ldgpp_amd", "-Wl,-rpath,$ORIGIN"])
     return LIB
 
 

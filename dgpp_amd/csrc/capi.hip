@@ -558,6 +558,16 @@ int dgpp_launch_moe_slot_order(const int32_t* ids, int32_t* order, int slots, in
                 "moe_slot_order");
 }
 
+int dgpp_minimax_router(const uint16_t* x, const float* gate, const float* bias, int rows, int hidden, int experts, int topk,
+                        float factor, float* scores, int32_t* ids, float* weights, void* stream) {
+  const char* who = "minimax_router";
+  if (rows <= 0) return DGPP_OK;
+  if (experts <= 0 || topk <= 0 || topk > 16 || topk > experts) return fail_arg(std::string(who) + ": MiniMax router shape");
+  if (experts > 4096) return fail_arg(std::string(who) + ": at most 4096 experts (the score row lives in a wavefront's registers)");
+  if (hidden <= 0 || rows > 65535) return fail_arg(std::string(who) + ": degenerate dims");
+  if (!x || !gate || !bias || !scores || !ids || !weights) return fail_arg(std::string(who) + ": null pointer");
+  return finish(run_minimax_router(x, gate, bias, rows, hidden, experts, topk, factor, scores, ids, weights, as_stream(stream)), who);
+}
 int dgpp_minimax_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* output, int experts, int capacity,
                                   void* stream) {
   if (!input || !output || input == output || experts < 1 || experts > 1024 || capacity < 1 || capacity > experts)

@@ -1,9 +1,10 @@
 // Token -> expert grouping of the MoE path: segments (a stable counting sort), the decode slots' expert order,
 // the tile list and the compaction of non-empty segments. Every output is an integer, bit-exact contract.
 //
-// Reference counterparts: src/models/glm/moe_layer.cpp:634-659 (the host grouping that is the specification),
-// src/kernels/glm_moe.cu:465-517 (slot order), :1382-1439 (segmentation), :1553-1569 (tile list);
-// src/kernels/minimax.cu:33-50 (segment compaction).
+// What each output must hold is fixed by the reference: src/models/glm/moe_layer.cpp:634-659 (the host grouping that is
+// the specification), src/kernels/glm_moe.cu:465-517 (slot order, runs, group list), :1382-1439 (segmentation),
+// :1553-1569 (tile list); src/kernels/minimax.cu:33-50 (segment compaction). How it is computed is this chip's:
+// wavefront ballots with mbcnt prefix counts, DPP prefix sums, scalar-side running totals.
 #include <hip/hip_runtime.h>
 #include <limits.h>
 #include <stdint.h>
@@ -17,67 +18,87 @@ namespace {
 
 constexpr int kWaveSize = 64;
 
+// ---- wavefront primitives ------------------------------------------------------------------------
+// How many lanes below this one have their bit set in a ballot.
+__device__ __forceinline__ int lanes_below(unsigned long long mask) {
+  return static_cast<int>(__builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(mask >> 32),
+                                                    __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u)));
+}
+template <int kCtrl, int kRowMask>
+__device__ __forceinline__ int dpp_take(int v) {   // lanes the move does not reach read 0
+  return __builtin_amdgcn_update_dpp(0, v, kCtrl, kRowMask, 0xF, false);
+}
+// Inclusive prefix sum over the wavefront: four shifts inside each row of sixteen lanes, then the two row
+// broadcasts that carry a row's total into the rows after it.
+__device__ __forceinline__ int wave_prefix_incl(int v) {
+  v += dpp_take<0x111, 0xF>(v);   // row_shr:1
+  v += dpp_take<0x112, 0xF>(v);   // row_shr:2
+  v += dpp_take<0x114, 0xF>(v);   // row_shr:4
+  v += dpp_take<0x118, 0xF>(v);   // row_shr:8
+  v += dpp_take<0x142, 0xA>(v);   // row_bcast:15 into rows 1 and 3
+  v += dpp_take<0x143, 0xC>(v);   // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // ---- grouping ------------------------------------------------------------------------------------
-// One block per expert plus one for the shared segment, ONE launch: a block derives its own
-// segment start as the number of ids below its expert (no cross-block dependency), then places
-// its (token, slot) pairs in (token, slot) order with a block scan over match flags — the host
-// path's stable counting sort, src/models/glm/moe_layer.cpp:634-659.
-constexpr int kSegThreads = 256;
-__global__ __launch_bounds__(kSegThreads) void segment_kernel(const int32_t* __restrict__ ids, int tokens, int K,
-                                                              int E, int32_t* __restrict__ rows,
-                                                              int32_t* __restrict__ slot_row,
-                                                              DgppMoeSegment* __restrict__ segs) {
-  __shared__ int s_wave[16];
-  __shared__ int s_less, s_equal;
-  const int e = blockIdx.x;
+// The host path's stable counting sort (src/models/glm/moe_layer.cpp:634-659) with ONE WAVEFRONT per expert
+// and no LDS, barrier or atomic: the wavefront reads the routed ids sixty-four at a time; two ballots per read
+// count, on the scalar side, the ids that sort before its expert (its segment's first row) and its own (the
+// segment's length). A second walk places the matches in (token, slot) order: a match's row is the segment's
+// rows placed so far plus the matching lanes below it (mbcnt of the ballot). One launch; the wavefront after the
+// last expert writes the shared segment.
+constexpr int kSegWaves = 4;
+__global__ __launch_bounds__(kSegWaves * kWaveSize) void segment_kernel(const int32_t* __restrict__ ids, int tokens, int K,
+                                                                         int E, int32_t* __restrict__ rows,
+                                                                         int32_t* __restrict__ slot_row,
+                                                                         DgppMoeSegment* __restrict__ segs) {
+  const int lane = threadIdx.x & (kWaveSize - 1);
+  const int e = blockIdx.x * kSegWaves + (threadIdx.x >> 6);
+  if (e > E) return;
   const int tk = tokens * K;
   if (e == E) {  // the shared expert: every token once more, after the routed rows
-    for (int t = threadIdx.x; t < tokens; t += kSegThreads) rows[tk + t] = t;
-    if (threadIdx.x == 0) segs[E] = DgppMoeSegment{tk, tokens, E};
+    for (int t = lane; t < tokens; t += kWaveSize) rows[tk + t] = t;
+    if (lane == 0) segs[E] = DgppMoeSegment{tk, tokens, E};
     return;
   }
-  if (threadIdx.x == 0) {
-    s_less = 0;
-    s_equal = 0;
+  int before = 0, own = 0;
+  for (int first = 0; first < tk; first += kWaveSize) {
+    const int i = first + lane;
+    const int id = i < tk ? ids[i] : INT_MAX;
+    before += __builtin_popcountll(__builtin_amdgcn_ballot_w64(id < e));
+    own += __builtin_popcountll(__builtin_amdgcn_ballot_w64(id == e));
   }
-  __syncthreads();
-  int less = 0, equal = 0;
-  for (int i = threadIdx.x; i < tk; i += kSegThreads) {
-    const int id = ids[i];
-    less += id < e;
-    equal += id == e;
-  }
-  // Integer sums: the order of the atomic adds does not change the result.
-  if (less) atomicAdd(&s_less, less);
-  if (equal) atomicAdd(&s_equal, equal);
-  __syncthreads();
-  const int row0 = s_less, count = s_equal;
-  if (threadIdx.x == 0) segs[e] = DgppMoeSegment{row0, count, e};
-  if (count == 0) return;
-  int running = row0;
-  for (int base = 0; base < tk; base += kSegThreads) {
-    const int i = base + threadIdx.x;
-    const int flag = (i < tk && ids[i] == e) ? 1 : 0;
-    int total = 0;
-    const int excl = block_exclusive_scan(flag, s_wave, &total);
-    if (flag) {
-      const int pos = running + excl;
-      rows[pos] = i / K;
-      slot_row[i] = pos;
+  if (lane == 0) segs[e] = DgppMoeSegment{before, own, e};
+  if (own == 0) return;
+  int placed = before;
+  for (int first = 0; first < tk && placed < before + own; first += kWaveSize) {
+    const int i = first + lane;
+    const bool hit = i < tk && ids[i] == e;
+    const unsigned long long hits = __builtin_amdgcn_ballot_w64(hit);
+    if (hit) {
+      const int at = placed + lanes_below(hits);
+      rows[at] = i / K;
+      slot_row[i] = at;
     }
-    running += total;
+    placed += __builtin_popcountll(hits);
   }
 }
 
-// One block, one thread per slot: rank by (key, slot), key = expert id or E for the shared slot.
+// One block, one thread per slot: rank by (key, slot), key = expert id or E for the shared slot. With `runs`: the
+// length of every run of equal experts at its first position (0 elsewhere) and, behind it, the list of 64-row
+// groups of the runs longer than a 16-row tile (src/kernels/glm_moe.cu:465-517 defines both). Run starts are found
+// by ballot; a run's length is the distance to the next start, read off the ballots (this wavefront's mask above
+// the lane, else the first set bit of a later wavefront's); a run's first list entry is an exclusive prefix sum of
+// the group counts (wavefront scan, wavefront totals through LDS).
 __global__ void slot_order_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ order,
                                   int32_t* __restrict__ runs, int slots, int top_k, int n_experts,
                                   int shared_early) {
-  extern __shared__ __align__(16) int32_t so_lds[];  // keys [slots padded to 4]; with runs: sorted [slots], groups [slots]
+  extern __shared__ __align__(16) int32_t so_lds[];  // keys [slots padded to 4]; with runs: sorted [slots]
+  __shared__ unsigned long long s_starts[16];
+  __shared__ int s_groups[16];
   const int padded = (slots + 3) & ~3;
   int32_t* keys = so_lds;
   int32_t* sorted = keys + padded;
-  int32_t* groups = sorted + slots;
   const int s = threadIdx.x;
   if (s < slots) {
     const int t = s / (top_k + 1), j = s - t * (top_k + 1);
@@ -99,27 +120,45 @@ __global__ void slot_order_kernel(const int32_t* __restrict__ ids, int32_t* __re
   if (!runs) return;
   __syncthreads();
   constexpr int kTileRows = 16, kGroupRows = 64;
-  int len = 0;
-  if (s < slots) {
-    if (s == 0 || sorted[s - 1] != sorted[s]) {
-      len = 1;
-      while (s + len < slots && sorted[s + len] == sorted[s]) ++len;
-    }
-    runs[s] = len;
-    groups[s] = len > kTileRows ? (len + kGroupRows - 1) / kGroupRows : 0;
-  }
+  const int lane = s & (kWaveSize - 1), wave = s >> 6, n_waves = static_cast<int>(blockDim.x) >> 6;
+  const bool starts_run = s < slots && (s == 0 || sorted[s - 1] != sorted[s]);
+  const unsigned long long mask = __builtin_amdgcn_ballot_w64(starts_run);
+  if (lane == 0) s_starts[wave] = mask;
   __syncthreads();
-  if (s < slots) {
-    int base = 0;
-    for (int o = 0; o < s; ++o) base += groups[o];
-    int32_t* list = runs + slots;
-    for (int g = 0; g < groups[s]; ++g) {
-      const int r0 = g * kGroupRows;
-      list[base + g] = (s + r0) | (min(kGroupRows, len - r0) << 16);
+  int next = slots;   // the position of the next run's start
+  {
+    const unsigned long long above = lane < kWaveSize - 1 ? mask >> (lane + 1) : 0ull;
+    if (above != 0ull) {
+      next = s + 1 + __builtin_ctzll(above);
+    } else {
+      for (int w = wave + 1; w < n_waves; ++w) {
+        const unsigned long long m = s_starts[w];
+        if (m != 0ull) {
+          next = w * kWaveSize + __builtin_ctzll(m);
+          break;
+        }
+      }
     }
-    if (s == slots - 1)
-      for (int i = base + groups[s]; i < slots / (kTileRows + 1) + 1; ++i) list[i] = -1;
   }
+  const int len = starts_run ? next - s : 0;
+  const int n_groups = len > kTileRows ? (len + kGroupRows - 1) / kGroupRows : 0;
+  if (s < slots) runs[s] = len;
+  const int upto = wave_prefix_incl(n_groups);
+  if (lane == kWaveSize - 1) s_groups[wave] = upto;
+  __syncthreads();
+  int first_entry = upto - n_groups, listed = 0;
+  for (int w = 0; w < n_waves; ++w) {
+    const int c = s_groups[w];
+    if (w < wave) first_entry += c;
+    listed += c;
+  }
+  int32_t* list = runs + slots;
+  for (int g = 0; g < n_groups; ++g) {
+    const int r0 = g * kGroupRows;
+    list[first_entry + g] = (s + r0) | (min(kGroupRows, len - r0) << 16);
+  }
+  const int capacity = slots / (kTileRows + 1) + 1;   // the list's entries beyond the groups read -1
+  for (int i = listed + s; i < capacity; i += static_cast<int>(blockDim.x)) list[i] = -1;
 }
 
 // The same order from several blocks (no run list): every block builds all sort keys in its LDS and ranks its own
@@ -168,31 +207,42 @@ __global__ __launch_bounds__(kOrderThreads) void slot_order_wide_kernel(const in
   order[pos] = s;
 }
 
-constexpr int kTileThreads = 256;
-__global__ __launch_bounds__(kTileThreads) void tile_list_kernel(const DgppMoeSegment* __restrict__ segs, int n_segs,
-                                                                 int tile_rows, DgppMoeTile* __restrict__ tiles,
-                                                                 int32_t* __restrict__ count) {
-  __shared__ int s_wave[16];
-  int running = 0;
-  for (int base = 0; base < n_segs; base += kTileThreads) {
-    const int e = base + threadIdx.x;
-    const int rows = e < n_segs ? segs[e].rows : 0;
-    const int mine = (rows + tile_rows - 1) / tile_rows;
-    int total = 0;
-    const int excl = block_exclusive_scan(mine, s_wave, &total);
-    for (int j = 0; j < mine; ++j) tiles[running + excl + j] = DgppMoeTile{e, j * tile_rows};
-    running += total;
+// The (segment, first row) tiles of every segment, in segment order, and their count: ONE wavefront walks the
+// segments sixty-four at a time; a segment's first tile is the tiles emitted so far plus the wavefront prefix sum of
+// the tile counts below its lane (no LDS, no barrier), and each lane writes its own segment's tiles.
+__global__ __launch_bounds__(kWaveSize) void tile_list_kernel(const DgppMoeSegment* __restrict__ segs, int n_segs,
+                                                               int tile_rows, DgppMoeTile* __restrict__ tiles,
+                                                               int32_t* __restrict__ count) {
+  const int lane = threadIdx.x;
+  int emitted = 0;
+  for (int first = 0; first < n_segs; first += kWaveSize) {
+    const int seg = first + lane;
+    const int n_tiles = seg < n_segs ? (segs[seg].rows + tile_rows - 1) / tile_rows : 0;
+    const int upto = wave_prefix_incl(n_tiles);
+    DgppMoeTile* out = tiles + emitted + upto - n_tiles;
+    for (int j = 0; j < n_tiles; ++j) out[j] = DgppMoeTile{seg, j * tile_rows};
+    emitted += __builtin_amdgcn_readlane(upto, kWaveSize - 1);
   }
-  if (threadIdx.x == 0) *count = running;
+  if (lane == 0) *count = emitted;
 }
 
+// Stable compaction of the non-empty segments (src/kernels/minimax.cu:33-50): a live segment's place is the live
+// lanes below it in its wavefront's ballot plus the live counts of the wavefronts before; entries past the live
+// ones read zero.
 __global__ void compact_segments_kernel(const DgppMoeSegment* __restrict__ input, DgppMoeSegment* __restrict__ output,
                                         int experts, int capacity) {
-  __shared__ int s_wave[16];
-  const int e = threadIdx.x;
-  const int live = (e < experts && input[e].rows > 0) ? 1 : 0;
-  int total = 0;
-  const int at = block_exclusive_scan(live, s_wave, &total);
+  __shared__ int s_live[16];
+  const int e = threadIdx.x, lane = e & (kWaveSize - 1), wave = e >> 6, n_waves = static_cast<int>(blockDim.x) >> 6;
+  const bool live = e < experts && input[e].rows > 0;
+  const unsigned long long mask = __builtin_amdgcn_ballot_w64(live);
+  if (lane == 0) s_live[wave] = __builtin_popcountll(mask);
+  __syncthreads();
+  int at = lanes_below(mask), total = 0;
+  for (int w = 0; w < n_waves; ++w) {
+    const int c = s_live[w];
+    if (w < wave) at += c;
+    total += c;
+  }
   if (live && at < capacity) output[at] = input[e];
   if (e >= total && e < capacity) output[e] = DgppMoeSegment{0, 0, 0};
 }
@@ -201,8 +251,8 @@ __global__ void compact_segments_kernel(const DgppMoeSegment* __restrict__ input
 
 hipError_t run_segment(const int32_t* ids, int tokens, int top_k, int n_experts, int32_t* rows, int32_t* slot_row,
                        DgppMoeSegment* segs, hipStream_t stream) {
-  hipLaunchKernelGGL(segment_kernel, dim3(n_experts + 1), dim3(kSegThreads), 0, stream, ids, tokens, top_k, n_experts,
-                     rows, slot_row, segs);
+  hipLaunchKernelGGL(segment_kernel, dim3((n_experts + 1 + kSegWaves - 1) / kSegWaves), dim3(kSegWaves * kWaveSize), 0, stream,
+                     ids, tokens, top_k, n_experts, rows, slot_row, segs);
   return hipGetLastError();
 }
 
@@ -215,7 +265,7 @@ hipError_t run_slot_order(const int32_t* ids, int32_t* order, int32_t* runs, int
     return hipGetLastError();
   }
   const int threads = (slots + kWaveSize - 1) / kWaveSize * kWaveSize;
-  const size_t lds = (static_cast<size_t>((slots + 3) & ~3) + (runs ? 2 * static_cast<size_t>(slots) : 0)) * sizeof(int32_t);
+  const size_t lds = (static_cast<size_t>((slots + 3) & ~3) + (runs ? static_cast<size_t>(slots) : 0)) * sizeof(int32_t);
   hipLaunchKernelGGL(slot_order_kernel, dim3(1), dim3(threads), lds, stream, ids, order, runs, slots, top_k, n_experts,
                      shared_early);
   return hipGetLastError();
@@ -223,7 +273,7 @@ hipError_t run_slot_order(const int32_t* ids, int32_t* order, int32_t* runs, int
 
 hipError_t run_tile_list(const DgppMoeSegment* segs, int n_segs, int tile_rows, DgppMoeTile* tiles, int32_t* count,
                          hipStream_t stream) {
-  hipLaunchKernelGGL(tile_list_kernel, dim3(1), dim3(kTileThreads), 0, stream, segs, n_segs, tile_rows, tiles, count);
+  hipLaunchKernelGGL(tile_list_kernel, dim3(1), dim3(kWaveSize), 0, stream, segs, n_segs, tile_rows, tiles, count);
   return hipGetLastError();
 }
 

@@ -16,6 +16,8 @@ hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gat
                            float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream, int allow_tiled = 1);
 hipError_t run_router_select(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
                              int tokens, int n_experts, int top_k, float scaling, int norm_topk, hipStream_t stream);
+hipError_t run_minimax_router(const uint16_t* x, const float* gate, const float* bias, int rows, int hidden, int experts,
+                              int top_k, float factor, float* scores, int32_t* ids, float* weights, hipStream_t stream);
 // tokens <= 16, n_experts <= 512, top_k <= 16; order may be null (selection only).
 hipError_t run_router_select_order(int mode, const float* scores, const float* biased, int32_t* ids, float* weights,
                                    int32_t* order, int tokens, int n_experts, int top_k, float scaling, int norm_topk,

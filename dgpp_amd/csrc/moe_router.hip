@@ -27,42 +27,13 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 // ---- router ---------------------------------------------------------------------------------
-// One wavefront per (expert, token): lanes stride the hidden vector in 16-byte vectors, each
-// lane an fp32 fma chain in k order, then the butterfly.
-constexpr int kRouterWaves = 4;
-
+// A finished dot becomes the token's score for the expert, and the score the selection ranks by
+// (src/kernels/glm_moe.cu:86-196 defines the three modes).
 template <int kMode>
-__global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_kernel(
-    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ gate, const float* __restrict__ bias,
-    float* __restrict__ scores, float* __restrict__ biased, int tokens, int hidden_dim, int n_experts,
-    int vector_loads) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int e = blockIdx.x * kRouterWaves + wave;
-  const int t = blockIdx.y;
-  if (e >= n_experts || t >= tokens) return;
-  const uint16_t* x = hidden + static_cast<size_t>(t) * hidden_dim;
-  const uint16_t* w = gate + static_cast<size_t>(e) * hidden_dim;
-  float dot = 0.f;
-  if (vector_loads) {
-    const int vecs = hidden_dim / 8;
-    for (int v = lane; v < vecs; v += kWaveSize) {
-      const uint4 xv = reinterpret_cast<const uint4*>(x)[v];
-      const uint4 wv = reinterpret_cast<const uint4*>(w)[v];
-      const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w}, ww[4] = {wv.x, wv.y, wv.z, wv.w};
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        dot = fmaf(bits_f32(xw[q] << 16), bits_f32(ww[q] << 16), dot);
-        dot = fmaf(bits_f32(xw[q] & 0xFFFF0000u), bits_f32(ww[q] & 0xFFFF0000u), dot);
-      }
-    }
-  } else {
-    for (int k = lane; k < hidden_dim; k += kWaveSize) dot = fmaf(bf16_to_f32(x[k]), bf16_to_f32(w[k]), dot);
-  }
-  dot = wave_sum(dot);
-  if (lane != 0) return;
-  const size_t at = static_cast<size_t>(t) * n_experts + e;
+__device__ __forceinline__ void store_score(float dot, const float* __restrict__ bias, int e, size_t at,
+                                            float* __restrict__ scores, float* __restrict__ biased) {
   if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
-    const float l = bf16_to_f32(f32_to_bf16(dot));
+    const float l = bf16_to_f32(f32_to_bf16(dot));   // the logit row is bf16-rounded
     scores[at] = l;
     biased[at] = l;
   } else {
@@ -76,20 +47,21 @@ __global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_kernel(
   }
 }
 
-// The same dots for a batch of rows (sixteen and more): a wavefront keeps a TT x EE tile of (token, expert) sums, so a
-// step's TT + EE vector loads feed TT * EE * 8 fmas and a gate row is fetched once per TT tokens instead of once per
-// token. Every (token, expert) sum is still one wavefront's: lane l takes the 16-byte vectors l, l + 64, ... in
-// ascending order, eight fmas each in element order, then the same butterfly - bit for bit the kernel above. Sixteen
-// lanes then finish one score each. Counterpart of the reference's tiled dots (src/kernels/glm_moe.cu:735-835), which
-// stages 16 x 16 tiles in shared memory; here the tile lives in registers and the L2 serves the re-reads.
+// The score rows of a batch. A wavefront keeps a TT x EE tile of (token, expert) sums in registers: a step's TT + EE
+// 16-byte vector loads feed TT * EE * 8 fmas, the next step's vectors are in flight while this step's fmas run, and a
+// gate row is fetched once per TT tokens. Every (token, expert) sum is one wavefront's: lane l takes the vectors l,
+// l + 64, ... in ascending order, eight fmas each in element order, then the butterfly - so the bits do not depend on
+// the tile. TT = EE = 1 is the decode form (one wavefront per (token, expert): the most wavefronts in flight), larger
+// tiles serve batches. The tile lives in registers and the L2 serves the re-reads, where the reference stages 16 x 16
+// tiles in shared memory (src/kernels/glm_moe.cu:735-835).
+constexpr int kRouterWaves = 4;
 constexpr int kTileExperts = 4;
 constexpr int kRouterTiledFromTokens = 32;   // measured: below this the one-row form's many wavefronts win (the reference tiles from 16)
 
-template <int kMode, int TT>
+template <int kMode, int TT, int EE>
 __global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_tile_kernel(
     const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ gate, const float* __restrict__ bias,
     float* __restrict__ scores, float* __restrict__ biased, int tokens, int hidden_dim, int n_experts) {
-  constexpr int EE = kTileExperts;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int e0 = (blockIdx.x * kRouterWaves + wave) * EE;
   const int t0 = blockIdx.y * TT;
@@ -150,19 +122,73 @@ __global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_tile_ker
     }
   const int t = t0 + lane / EE, e = e0 + lane % EE;
   if (lane >= TT * EE || t >= tokens || e >= n_experts) return;
-  const size_t at = static_cast<size_t>(t) * n_experts + e;
-  if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
-    const float l = bf16_to_f32(f32_to_bf16(mine));
-    scores[at] = l;
-    biased[at] = l;
+  store_score<kMode>(mine, bias, e, static_cast<size_t>(t) * n_experts + e, scores, biased);
+}
+
+// Rows that cannot be read as aligned 16-byte vectors (hidden not a multiple of eight, unaligned pointers): a
+// wavefront per (token, expert), lanes a stride of 64 elements apart.
+template <int kMode>
+__global__ __launch_bounds__(kRouterWaves * kWaveSize) void router_dots_unaligned_kernel(
+    const uint16_t* __restrict__ hidden, const uint16_t* __restrict__ gate, const float* __restrict__ bias,
+    float* __restrict__ scores, float* __restrict__ biased, int tokens, int hidden_dim, int n_experts) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * kRouterWaves + (threadIdx.x >> 6), t = blockIdx.y;
+  if (e >= n_experts || t >= tokens) return;
+  const uint16_t* x = hidden + static_cast<size_t>(t) * hidden_dim;
+  const uint16_t* w = gate + static_cast<size_t>(e) * hidden_dim;
+  float dot = 0.f;
+  for (int k = lane; k < hidden_dim; k += kWaveSize) dot = fmaf(bf16_to_f32(x[k]), bf16_to_f32(w[k]), dot);
+  dot = wave_sum(dot);
+  if (lane == 0) store_score<kMode>(dot, bias, e, static_cast<size_t>(t) * n_experts + e, scores, biased);
+}
+
+// ---- the MiniMax router (src/kernels/minimax.hpp:56-60, src/kernels/minimax.cu:397-440) ---------------------------
+// FP32 gate rows against BF16 token rows; the score is the sigmoid of the FP32 dot and is what the weights are made
+// of, the bias enters the ranking only. One wavefront per (row, expert): lane l takes the eight-element groups l,
+// l + 64, ... in ascending order (one 16-byte load of the token row, two of the gate row), eight fmas each in element
+// order, then the butterfly; rows that are not 32-byte aligned groups go element by element.
+__global__ __launch_bounds__(kRouterWaves * kWaveSize) void minimax_router_dots_kernel(
+    const uint16_t* __restrict__ x, const float* __restrict__ gate, float* __restrict__ scores, int rows, int hidden,
+    int experts, int vectors) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * kRouterWaves + (threadIdx.x >> 6), r = blockIdx.y;
+  if (e >= experts || r >= rows) return;
+  const uint16_t* xr = x + static_cast<size_t>(r) * hidden;
+  const float* w = gate + static_cast<size_t>(e) * hidden;
+  float dot = 0.f;
+  if (vectors) {
+    for (int v = lane; v < hidden / 8; v += kWaveSize) {
+      const uint4 xv = reinterpret_cast<const uint4*>(xr)[v];
+      const float4 w0 = reinterpret_cast<const float4*>(w)[2 * v], w1 = reinterpret_cast<const float4*>(w)[2 * v + 1];
+      dot = fmaf(bits_f32(xv.x << 16), w0.x, dot);
+      dot = fmaf(bits_f32(xv.x & 0xFFFF0000u), w0.y, dot);
+      dot = fmaf(bits_f32(xv.y << 16), w0.z, dot);
+      dot = fmaf(bits_f32(xv.y & 0xFFFF0000u), w0.w, dot);
+      dot = fmaf(bits_f32(xv.z << 16), w1.x, dot);
+      dot = fmaf(bits_f32(xv.z & 0xFFFF0000u), w1.y, dot);
+      dot = fmaf(bits_f32(xv.w << 16), w1.z, dot);
+      dot = fmaf(bits_f32(xv.w & 0xFFFF0000u), w1.w, dot);
+    }
   } else {
-    float sc;
-    if (kMode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS)
-      sc = sqrtf(mine > 20.f ? mine : log1pf(expf(mine)));
-    else
-      sc = 1.0f / (1.0f + expf(-mine));
-    scores[at] = sc;
-    biased[at] = sc + bias[e];
+    for (int k = lane; k < hidden; k += kWaveSize) dot = fmaf(bf16_to_f32(xr[k]), w[k], dot);
+  }
+  dot = wave_sum(dot);
+  if (lane == 0) scores[static_cast<size_t>(r) * experts + e] = 1.0f / (1.0f + expf(-dot));
+}
+template <int PER_LANE>
+__global__ __launch_bounds__(kWaveSize) void minimax_router_select_kernel(const float* __restrict__ scores,
+                                                                          const float* __restrict__ bias,
+                                                                          int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                                          int rows, int experts, int top_k, float factor) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  if (r >= rows) return;
+  int id;
+  float w;
+  select_token<DGPP_ROUTER_SIGMOID_BIAS, PER_LANE, true>(scores + static_cast<size_t>(r) * experts, bias, experts, top_k, factor, 1,
+                                                         lane, id, w);
+  if (lane < top_k) {
+    ids[static_cast<size_t>(r) * top_k + lane] = id;
+    weights[static_cast<size_t>(r) * top_k + lane] = w;
   }
 }
 
@@ -256,40 +282,44 @@ hipError_t run_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const 
   return hipGetLastError();
 }
 
+template <int TT, int EE>
+static void launch_dots_tile(int mode, dim3 grid, hipStream_t stream, const uint16_t* hidden, const uint16_t* gate,
+                             const float* bias, float* scores, float* biased, int tokens, int hidden_dim, int n_experts) {
+  const dim3 block(kRouterWaves * kWaveSize);
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, grid, block, 0, stream, hidden, gate, bias, scores, biased, tokens, hidden_dim, n_experts);
+  };
+  if (mode == DGPP_ROUTER_SOFTMAX_TOPK) go(router_dots_tile_kernel<DGPP_ROUTER_SOFTMAX_TOPK, TT, EE>);
+  else if (mode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS) go(router_dots_tile_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS, TT, EE>);
+  else go(router_dots_tile_kernel<DGPP_ROUTER_SIGMOID_BIAS, TT, EE>);
+}
+
 hipError_t run_router_dots(int mode, const uint16_t* hidden, const uint16_t* gate, const float* bias, float* scores,
                            float* biased, int tokens, int hidden_dim, int n_experts, hipStream_t stream, int allow_tiled) {
-  const int vec = (hidden_dim % 8 == 0) && ((reinterpret_cast<uintptr_t>(hidden) & 15u) == 0) &&
-                  ((reinterpret_cast<uintptr_t>(gate) & 15u) == 0);
+  const bool vec = (hidden_dim % 8 == 0) && ((reinterpret_cast<uintptr_t>(hidden) & 15u) == 0) &&
+                   ((reinterpret_cast<uintptr_t>(gate) & 15u) == 0);
+  if (!vec) {
+    const dim3 grid((n_experts + kRouterWaves - 1) / kRouterWaves, tokens), block(kRouterWaves * kWaveSize);
+    auto go = [&](auto kern) {
+      hipLaunchKernelGGL(kern, grid, block, 0, stream, hidden, gate, bias, scores, biased, tokens, hidden_dim, n_experts);
+    };
+    if (mode == DGPP_ROUTER_SOFTMAX_TOPK) go(router_dots_unaligned_kernel<DGPP_ROUTER_SOFTMAX_TOPK>);
+    else if (mode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS) go(router_dots_unaligned_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS>);
+    else go(router_dots_unaligned_kernel<DGPP_ROUTER_SIGMOID_BIAS>);
+    return hipGetLastError();
+  }
   const int tuned = tune_get(kTuneRouterTile);   // bench / test switch: 2 or 4 forces the tiled form with that tile
-  if (allow_tiled && vec && (tokens >= kRouterTiledFromTokens || tuned > 0)) {
+  if (allow_tiled && (tokens >= kRouterTiledFromTokens || tuned > 0)) {
     // Two tokens per wavefront (more wavefronts in flight) until the batch is large enough that four (fewer gate
     // re-reads) pays.
     const int tt = tuned > 0 ? (tuned >= 4 ? 4 : 2) : (tokens >= 128 ? 4 : 2);
     const dim3 grid((n_experts + kRouterWaves * kTileExperts - 1) / (kRouterWaves * kTileExperts), (tokens + tt - 1) / tt);
-    const dim3 block(kRouterWaves * kWaveSize);
-    auto go = [&](auto kern) {
-      hipLaunchKernelGGL(kern, grid, block, 0, stream, hidden, gate, bias, scores, biased, tokens, hidden_dim, n_experts);
-    };
-    if (mode == DGPP_ROUTER_SOFTMAX_TOPK)
-      tt == 4 ? go(router_dots_tile_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 4>) : go(router_dots_tile_kernel<DGPP_ROUTER_SOFTMAX_TOPK, 2>);
-    else if (mode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS)
-      tt == 4 ? go(router_dots_tile_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS, 4>)
-              : go(router_dots_tile_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS, 2>);
-    else
-      tt == 4 ? go(router_dots_tile_kernel<DGPP_ROUTER_SIGMOID_BIAS, 4>) : go(router_dots_tile_kernel<DGPP_ROUTER_SIGMOID_BIAS, 2>);
+    if (tt == 4) launch_dots_tile<4, kTileExperts>(mode, grid, stream, hidden, gate, bias, scores, biased, tokens, hidden_dim, n_experts);
+    else launch_dots_tile<2, kTileExperts>(mode, grid, stream, hidden, gate, bias, scores, biased, tokens, hidden_dim, n_experts);
     return hipGetLastError();
   }
   const dim3 grid((n_experts + kRouterWaves - 1) / kRouterWaves, tokens);
-  const dim3 block(kRouterWaves * kWaveSize);
-  if (mode == DGPP_ROUTER_SOFTMAX_TOPK)
-    hipLaunchKernelGGL(router_dots_kernel<DGPP_ROUTER_SOFTMAX_TOPK>, grid, block, 0, stream, hidden, gate, bias, scores,
-                       biased, tokens, hidden_dim, n_experts, vec);
-  else if (mode == DGPP_ROUTER_SQRT_SOFTPLUS_BIAS)
-    hipLaunchKernelGGL(router_dots_kernel<DGPP_ROUTER_SQRT_SOFTPLUS_BIAS>, grid, block, 0, stream, hidden, gate, bias,
-                       scores, biased, tokens, hidden_dim, n_experts, vec);
-  else
-    hipLaunchKernelGGL(router_dots_kernel<DGPP_ROUTER_SIGMOID_BIAS>, grid, block, 0, stream, hidden, gate, bias, scores,
-                       biased, tokens, hidden_dim, n_experts, vec);
+  launch_dots_tile<1, 1>(mode, grid, stream, hidden, gate, bias, scores, biased, tokens, hidden_dim, n_experts);
   return hipGetLastError();
 }
 
@@ -318,6 +348,24 @@ hipError_t run_router_select(int mode, const float* scores, const float* biased,
     launch_select_mode<DGPP_ROUTER_SOFTMAX_TOPK>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
   else
     launch_select_mode<DGPP_ROUTER_SIGMOID_BIAS>(scores, biased, ids, weights, tokens, n_experts, top_k, scaling, norm_topk, stream);
+  return hipGetLastError();
+}
+
+hipError_t run_minimax_router(const uint16_t* x, const float* gate, const float* bias, int rows, int hidden, int experts,
+                              int top_k, float factor, float* scores, int32_t* ids, float* weights, hipStream_t stream) {
+  if (experts > 64 * kWaveSize) return hipErrorInvalidValue;
+  const int vectors = hidden % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(gate) & 15u) == 0;
+  hipLaunchKernelGGL(minimax_router_dots_kernel, dim3((experts + kRouterWaves - 1) / kRouterWaves, rows),
+                     dim3(kRouterWaves * kWaveSize), 0, stream, x, gate, scores, rows, hidden, experts, vectors);
+  const int per_lane = (experts + kWaveSize - 1) / kWaveSize;
+  auto go = [&](auto kern) {
+    hipLaunchKernelGGL(kern, dim3(rows), dim3(kWaveSize), 0, stream, scores, bias, ids, weights, rows, experts, top_k, factor);
+  };
+  if (per_lane <= 4) go(minimax_router_select_kernel<4>);
+  else if (per_lane <= 8) go(minimax_router_select_kernel<8>);
+  else if (per_lane <= 16) go(minimax_router_select_kernel<16>);
+  else if (per_lane <= 32) go(minimax_router_select_kernel<32>);
+  else go(minimax_router_select_kernel<64>);
   return hipGetLastError();
 }
 

@@ -74,7 +74,9 @@ __device__ __forceinline__ uint32_t order_key(float v) {
 
 // One wavefront selects for one token. On return lane p < top_k holds the token's p-th expert in
 // ascending id order and its final weight; no private arrays, no LDS.
-template <int kMode, int PER_LANE>
+// kAddBias: `biased` holds the per-expert bias and the ranking value is scores[e] + bias[e], formed here; the weights
+// are then score / max(sum, 1e-20) * scaling, never narrowed (the MiniMax router, src/kernels/minimax.cu:409-440).
+template <int kMode, int PER_LANE, bool kAddBias = false>
 __device__ __forceinline__ void select_token(const float* __restrict__ scores, const float* __restrict__ biased,
                                              int n_experts, int top_k, float scaling, int norm_topk, int lane,
                                              int& out_id, float& out_w) {
@@ -93,7 +95,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ scores, c
     for (int j = 0; j < PER_LANE; ++j) {
       const bool live = lane + j * kWaveSize < n_experts;
       sc[j] = live ? raw_s[j] : -INFINITY;
-      key[j] = live ? order_key(raw_b[j]) : 0u;
+      key[j] = live ? order_key(kAddBias ? raw_s[j] + raw_b[j] : raw_b[j]) : 0u;
     }
   }
   if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) {
@@ -151,7 +153,8 @@ __device__ __forceinline__ void select_token(const float* __restrict__ scores, c
   const float sw = __shfl(my_w, src);
   float denom = 0.f;
   for (int i = 0; i < top_k; ++i) denom += row_lane(sw, i);   // fp32 adds in id order
-  denom += 1e-20f;
+  if (kAddBias) denom = fmaxf(denom, 1e-20f);
+  else denom += 1e-20f;
   float w = norm_topk ? (sw / denom) * scaling : sw * scaling;
   if (kMode == DGPP_ROUTER_SOFTMAX_TOPK) w = bf16_to_f32(f32_to_bf16(w));
   out_id = sid;

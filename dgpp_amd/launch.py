@@ -168,6 +168,12 @@ def launch_moe_slot_order(ids, order, slots, top_k, n_experts, stream=None, shar
                                                   1 if shared_early else 0, _p(runs)))
 
 
+def minimax_router(x, gate, bias, rows, hidden, experts, topk, factor, scores, ids, weights, stream=None):
+    """src/kernels/minimax.hpp:56-60: FP32 gate, sigmoid scores, bias for the ranking only, FP32 weights."""
+    _check(_lib.load().dgpp_minimax_router(_p(x), _p(gate), _p(bias), rows, hidden, experts, topk, factor, _p(scores), _p(ids),
+                                           _p(weights), _stream(stream)))
+
+
 def minimax_compact_segments(input, output, experts, capacity, stream=None):
     _check(_lib.load().dgpp_minimax_compact_segments(_p(input), _p(output), experts, capacity, _stream(stream)))
 

@@ -163,6 +163,14 @@ int dgpp_launch_moe_tile_list(const DgppMoeSegment* segs, int n_segs, int tile_r
 int dgpp_moe_run_groups_max(int slots);
 int dgpp_launch_moe_slot_order(const int32_t* ids, int32_t* order, int slots, int top_k,
                                int n_experts, void* stream, int shared_early, int32_t* runs);
+/* src/kernels/minimax.hpp:56-60 (minimax_router; kernels src/kernels/minimax.cu:397-440): the MiniMax router. x: BF16
+ * token rows [rows, hidden]; gate: FP32 [experts, hidden]; scores (out) [rows, experts] = sigmoid of the FP32 dot. The
+ * top-k is taken by scores + bias (strict '>' : the lower id wins a tie), ids come back ascending, and
+ * weights = score / max(sum of the picked scores in id order, 1e-20) * factor, FP32, never narrowed. rows <= 0 returns
+ * at once; experts <= 0, topk outside 1..16 or above experts is an invalid argument. At most 4096 experts. */
+int dgpp_minimax_router(const uint16_t* x, const float* gate, const float* bias, int rows, int hidden, int experts, int topk,
+                        float factor, float* scores, int32_t* ids, float* weights, void* stream);
+
 /* src/kernels/minimax.hpp:11 */
 int dgpp_minimax_compact_segments(const DgppMoeSegment* input, DgppMoeSegment* output,
                                   int experts, int capacity, void* stream);

@@ -394,6 +394,10 @@ inline void launch_moe_grouped_gemv_fp4_f32(const uint16_t* act, size_t act_stri
 }
 
 // ---- src/kernels/minimax.hpp:11 -----------------------------------------------------------------------
+inline void minimax_router(const uint16_t* x, const float* gate, const float* bias, int rows, int hidden, int experts, int topk,
+                           float factor, float* scores, int32_t* ids, float* weights, hipStream_t stream) {
+  detail::check(dgpp_minimax_router(x, gate, bias, rows, hidden, experts, topk, factor, scores, ids, weights, stream));
+}
 inline void minimax_compact_segments(const MoeSegment* input, MoeSegment* output, int experts, int capacity,
                                      hipStream_t stream) {
   detail::check(dgpp_minimax_compact_segments(input, output, experts, capacity, stream));

@@ -605,6 +605,43 @@ void orc_minimax_swiglu_f32(const float* gate, const float* up, int64_t count, d
   }
 }
 
+// The MiniMax router as its CPU statement does it (src/models/minimax/reference.cpp:96-113) and its kernels
+// (src/kernels/minimax.cu:409-440), in FP32 throughout: ranking by score + bias (ties to the lower id), ids
+// ascending, weights = score / max(sum in id order, 1e-20) * factor. `scores` are the sigmoid scores themselves
+// (the device's, when a device selection is checked against this).
+void orc_minimax_route_scores(const float* scores, const float* bias, int rows, int experts, int topk, float factor,
+                              int32_t* ids, float* weights) {
+  std::vector<int> order(static_cast<size_t>(experts));
+  for (int r = 0; r < rows; ++r) {
+    const float* row = scores + static_cast<size_t>(r) * experts;
+    for (int e = 0; e < experts; ++e) order[static_cast<size_t>(e)] = e;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+      const float sa = row[a] + bias[a], sb = row[b] + bias[b];
+      return sa == sb ? a < b : sa > sb;
+    });
+    std::vector<int> picked(order.begin(), order.begin() + topk);
+    std::sort(picked.begin(), picked.end());
+    float sum = 0.f;
+    for (int e : picked) sum += row[e];
+    for (int j = 0; j < topk; ++j) {
+      ids[static_cast<size_t>(r) * topk + j] = picked[static_cast<size_t>(j)];
+      weights[static_cast<size_t>(r) * topk + j] = row[picked[static_cast<size_t>(j)]] / std::max(sum, 1e-20f) * factor;
+    }
+  }
+}
+// scores[r, e] = sigmoid(dot(x[r], gate[e])) with the dot in double (x BF16 bits, gate FP32): what the device's FP32
+// chain is held against. src/kernels/minimax.cu:397-408
+void orc_minimax_router_scores(const uint16_t* x, const float* gate, int rows, int hidden, int experts, double* scores) {
+  for (int r = 0; r < rows; ++r)
+    for (int e = 0; e < experts; ++e) {
+      double dot = 0.0;
+      for (int k = 0; k < hidden; ++k)
+        dot += bf16d(x[static_cast<size_t>(r) * hidden + k]) *
+               static_cast<double>(gate[static_cast<size_t>(e) * hidden + k]);
+      scores[static_cast<size_t>(r) * experts + e] = 1.0 / (1.0 + std::exp(-dot));
+    }
+}
+
 void orc_w4a4_gemm(const uint8_t* a_codes, const uint8_t* a_scales, int64_t a_scale_stride, const float* a_gs,
                    const uint8_t* w_codes, const uint8_t* w_scales, double w_global, int m, int n, int k, double* out,
                    double* out_abs) {

@@ -190,6 +190,13 @@ void orc_hash_routes(const int64_t* tokens, const int32_t* tid2eid, const float*
  * rows, and invariance to how rows are spread over calls (the property the reference's test checks). */
 void orc_minimax_quantize_rows_nvfp4(const uint16_t* x, int64_t stride, int rows, int k, uint8_t* codes, uint8_t* scales,
                                      float* globals);
+/* The MiniMax router: selection and weights from sigmoid scores, FP32 throughout (ranking by score + bias, ties to
+ * the lower id, ids ascending, weights = score / max(sum in id order, 1e-20) * factor).
+ * src/models/minimax/reference.cpp:96-113; src/kernels/minimax.cu:409-440 */
+void orc_minimax_route_scores(const float* scores, const float* bias, int rows, int experts, int topk, float factor,
+                              int32_t* ids, float* weights);
+/* scores[r, e] = sigmoid(dot(x[r], gate[e])), dot in double; x BF16 bits, gate FP32. src/kernels/minimax.cu:397-408 */
+void orc_minimax_router_scores(const uint16_t* x, const float* gate, int rows, int hidden, int experts, double* scores);
 /* src/kernels/minimax_native_moe.cu:87-95 evaluated in double: bf16((g' / (1 + exp(-alpha g'))) (u' + 1)), g' = min(g,
  * limit), u' = clamp(u, -limit, limit); out (nullable) the BF16 rounding, out_exact (nullable) the unrounded value.
  * Pinned by closed-form points (g = 0, u = -1, both clamps) and numpy float64. */

@@ -14,6 +14,7 @@
 #include "loaders/fp8_quant.hpp"
 #include "loaders/nvfp4_quant.hpp"
 #include "models/glm/moe_reference.hpp"
+#include "models/minimax/reference.hpp"
 
 using namespace dgpp;
 
@@ -51,6 +52,23 @@ void ref_nvfp4_encode_row(const float* row, int64_t cols, float ws2, uint8_t* pa
 }
 void ref_fp8_encode_block128(const uint16_t* src, int64_t rows, int64_t cols, uint8_t* payload, float* scales) {
   fp8_quant::encode_block128(src, static_cast<size_t>(cols), rows, cols, payload, scales, 1);
+}
+
+// The reference's MiniMax routing statement (src/models/minimax/reference.cpp:96-113) for one row of logits.
+int ref_minimax_route(const float* logits, const float* bias, int experts, int topk, float factor, int32_t* ids,
+                      float* weights) {
+  try {
+    std::vector<int> i;
+    std::vector<float> w;
+    dgpp::minimax_ref::route(logits, bias, experts, topk, factor, i, w);
+    for (int j = 0; j < topk; ++j) {
+      ids[j] = i[static_cast<size_t>(j)];
+      weights[j] = w[static_cast<size_t>(j)];
+    }
+    return 0;
+  } catch (const std::exception&) {
+    return 1;
+  }
 }
 
 // Router oracle: returns 0, or 1 when the reference threw.

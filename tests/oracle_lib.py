@@ -51,6 +51,8 @@ _SIG = {
     "orc_hash_routes": (None, [_P, _P, _P, _I, _I, _I, _I, _F, _I, _P, _P]),
     "orc_minimax_quantize_rows_nvfp4": (None, [_P, _L, _I, _I, _P, _P, _P]),
     "orc_minimax_swiglu_f32": (None, [_P, _P, C.c_int64, _D, _D, _P, _P]),
+    "orc_minimax_route_scores": (None, [_P, _P, _I, _I, _I, _F, _P, _P]),
+    "orc_minimax_router_scores": (None, [_P, _P, _I, _I, _I, _P]),
     "orc_w4a4_gemm": (None, [_P, _P, _L, _P, _P, _P, C.c_double, _I, _I, _I, _P, _P]),
     "orc_swiglu_oai": (None, [_P, _P, _L, _I, _I, _F, _F, _P, _P]),
     "orc_mxfp8_gemm": (None, [_P, _P, _P, _P, _I, _I, _I, _P, _P]),
@@ -66,6 +68,7 @@ _REF_SIG = {
     "ref_nvfp4_tensor_scale": (_F, [_F]),
     "ref_nvfp4_encode_row": (None, [_P, _L, _F, _P, _P]),
     "ref_fp8_encode_block128": (None, [_P, _L, _L, _P, _P]),
+    "ref_minimax_route": (_I, [_P, _P, _I, _I, _F, _P, _P]),
     "ref_router": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P]),
     "ref_moe_forward": (_I, [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _P, _P, _P, _L, _P, _L, _I, _I, _I, _P, _L, _P,
                              _L, _P, _L, _P]),
