@@ -38,8 +38,22 @@ GATE_UP_BYTES = 2 * (I * H // 2 + I * H // 32)
 TRAFFIC_PROFILE = "profiles/moe_gemv_kernels_mxfp4_c3_t8_hbm_counters.txt"
 
 
+# The sources that define the two profiled kernels: the counter summary names the digest of the build it was taken
+# from, and its figures are used only while the tree's digest is the same (a kernel body can change without its name).
+KERNEL_SOURCES = ("gemv_core.hpp", "gemv_kernels.hpp", "swiglu.hpp", "numerics.hpp", "router_select.hpp")
+
+
+def kernel_source_digest():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        h.update((ROOT / "dgpp_amd" / "csrc" / name).read_bytes())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic():
-    """{"gate_up": bytes, "down": bytes, "gate_up_kernel": name, "down_kernel": name} from the counter summary, or {}."""
+    """{"gate_up": bytes, "down": bytes, "gate_up_kernel": name, "down_kernel": name, "digest": ...} from the counter
+    summary, or {}; {"stale": digest} when the summary was taken from other kernel sources than the tree holds."""
     out = {}
     try:
         text = (ROOT / TRAFFIC_PROFILE).read_text()
@@ -50,6 +64,14 @@ def measured_traffic():
         if len(part) >= 4 and part[0] == "traffic_bytes_per_launch":
             out[part[1]] = float(part[2])
             out[part[1] + "_kernel"] = " ".join(part[3:])
+        if len(part) >= 2 and part[0] == "kernel_source_digest":
+            out["digest"] = part[1]
+    try:
+        now = kernel_source_digest()
+    except OSError:
+        return {}
+    if out.get("digest") != now:
+        return {"stale": out.get("digest"), "tree": now}
     return out
 
 
@@ -1012,7 +1034,9 @@ def main():
                 cpu = {"value": bytes_ref / t_ref / 1e9, "unit": "GB/s", "cores": 1, "kind": "reference",
                        "sample": f"{n_ref} T=1 passes of the reference's own glm_moe_ref_forward (compiled from its sources: router "
                                  f"GEMV + 8 routed MXFP4 experts + the shared expert it always runs = {bytes_ref / 1e6:.1f} MB per "
-                                 "pass), one thread as the reference runs it",
+                                 "pass), one thread as the reference runs it. NOT the GPU's workload one to one: a GPU T=1 "
+                                 f"pass is 8 routed experts and no router GEMV ({(K * EXPERT_BYTES) / 1e6:.1f} MB); compare the GB/s, "
+                                 "not us_per_layer. `port` times exactly the GPU's T=1 workload (8 experts, given logits)",
                        "us_per_layer": t_ref * 1e6,
                        "port_equals_reference_bits": bool(np.array_equal(port_bits, ref_out)),
                        "gpu_vs_cpu_max_rel": port.pop("gpu_vs_cpu_max_rel"),
@@ -1062,7 +1086,11 @@ def main():
                             "achieved": main_res["gate_up_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                             "frac": main_res["gate_up_gbps"] / HBM_PEAK_GBPS,
                             "traffic": traffic.get("gate_up") if same_workload else None,
-                            "traffic_source": (TRAFFIC_PROFILE + ": " + traffic.get("gate_up_kernel", "")) if same_workload else None,
+                            "traffic_source": ((TRAFFIC_PROFILE + ": " + traffic.get("gate_up_kernel", "") + ", kernel sources " +
+                                                traffic["digest"]) if "digest" in traffic else
+                                               (TRAFFIC_PROFILE + " was taken from kernel sources " + str(traffic.get("stale")) +
+                                                ", the tree holds " + str(traffic.get("tree")) + ": not used")
+                                               if "stale" in traffic else None) if same_workload else None,
                             "bytes_per_launch": main_res["gate_up_bytes"], "us_per_launch": main_res["gate_up_us"]}
         if "gate_up_plain_read_us" in main_res:   # this chip's plain cold read of the same byte count, same timing method
             line["roofline"]["plain_read_same_bytes_us"] = main_res["gate_up_plain_read_us"]

@@ -126,6 +126,7 @@ SIGNATURES = {
     "dgpp_launch_mma_gemv_fp4_bf16": (_I, [_P, _Z, _P, _P, _I, _I, _I, _Z, _P, _P, _Z]),
     "dgpp_launch_mma_gemv_fp4_f32": (_I, [_P, _Z, _P, _P, _I, _I, _I, _Z, _P, _P, _Z]),
     "dgpp_launch_mma_gemv_fp4_bf16_static": (_I, [_P, _Z, _P, _P, _I, _I, _I, _Z, _P]),
+    "dgpp_static_scratch_release": (_I, []),
     "dgpp_launch_mma_gemv_fp8_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
     "dgpp_launch_mma_gemv_fp8_f32": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),
     "dgpp_launch_mma_gemv_fp8e8m0_bf16": (_I, [_P, _Z, _P, _P, _P, _I, _I, _I, _Z, _I, _I, _P, _P, _Z]),

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <limits.h>
+#include <atomic>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -62,8 +63,14 @@ MatRef fp8_mat(const uint8_t* payload, const void* scales, int rs, int cs) {
 }  // namespace
 
 namespace dgpp_amd {
-static int g_tune[kTuneCount] = {0};
-int tune_get(int key) { return key >= 0 && key < kTuneCount ? g_tune[key] : 0; }
+// The measurement switches: relaxed atomics (a harness may set one while another thread launches; every launch reads a
+// switch once). A build with -DDGPP_NO_TUNE compiles them out: every switch reads 0 and dgpp_tune_set does nothing.
+#ifdef DGPP_NO_TUNE
+int tune_get(int) { return 0; }
+#else
+static std::atomic<int> g_tune[kTuneCount];
+int tune_get(int key) { return key >= 0 && key < kTuneCount ? g_tune[key].load(std::memory_order_relaxed) : 0; }
+#endif
 
 hipError_t ensure_lds_impl(const void* kernel, size_t bytes) {
   static std::mutex mu;
@@ -401,7 +408,12 @@ int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, 
   return finish(run_probe_read(src, bytes, sink, nontemporal, blocks, span, as_stream(stream)), who);
 }
 void dgpp_tune_set(int key, int value) {
-  if (key >= 0 && key < kTuneCount) g_tune[key] = value;
+#ifndef DGPP_NO_TUNE
+  if (key >= 0 && key < kTuneCount) g_tune[key].store(value, std::memory_order_relaxed);
+#else
+  (void)key;
+  (void)value;
+#endif
 }
 int dgpp_tune_get(int key) { return tune_get(key); }
 
@@ -1334,8 +1346,14 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 namespace {
 std::mutex g_scratch_mu;
 void* g_scratch_ptr[kMaxDevices] = {nullptr};
-// The device address of `scratch` on the current device (looked up on the first call there).
-int static_scratch(void** ptr, const char* who) {
+// The stream a device's array is bound to: launches on ONE stream follow each other, launches on two could overlap and
+// race on the array, so a second stream is refused until the caller releases the binding (dgpp_static_scratch_release,
+// after it has made sure the bound stream's work is done).
+void* g_scratch_stream[kMaxDevices] = {nullptr};
+bool g_scratch_bound[kMaxDevices] = {false};
+inline bool dense_mma_would_split(int parts, int m, int n) { return dense_mfma_would_split(parts, m, n); }
+// The device address of `scratch` on the current device (looked up on the first call there), bound to `stream`.
+int static_scratch(void** ptr, void* stream, const char* who) {
   int device = -1;
   hipError_t err = hipGetDevice(&device);
   if (err != hipSuccess) return finish(err, who);
@@ -1348,6 +1366,11 @@ int static_scratch(void** ptr, const char* who) {
     if (p == nullptr) return fail_arg(std::string(who) + ": the scratch array has no address on this device");
     g_scratch_ptr[device] = p;
   }
+  if (g_scratch_bound[device] && g_scratch_stream[device] != stream)
+    return fail_arg(std::string(who) + ": the static workspace of this device is in use by another stream (calls that "
+                    "overlap would race on it); finish that stream's work and call dgpp_static_scratch_release first");
+  g_scratch_bound[device] = true;
+  g_scratch_stream[device] = stream;
   *ptr = g_scratch_ptr[device];
   return DGPP_OK;
 }
@@ -1358,16 +1381,28 @@ int dgpp_launch_mma_gemv_fp4_bf16_static(const uint16_t* act, size_t act_stride,
   const char* who = "mma_gemv_fp4_static";
   if (m <= 0 || n <= 0) return DGPP_OK;
   if (k <= 0 || k % 32 != 0) return fail_arg(std::string(who) + ": k must be a positive multiple of 32");
-  const size_t parts = static_cast<size_t>(w && w->scale_group == 32 ? mgeom<kFmtMxfp4>(k).parts : mgeom<kFmtNvfp4>(k).parts);
-  const size_t need = parts * static_cast<size_t>(m) * static_cast<size_t>(n) * sizeof(float);
+  const int parts = w && w->scale_group == 32 ? mgeom<kFmtMxfp4>(k).parts : mgeom<kFmtNvfp4>(k).parts;
+  // Only the split form uses the workspace: a launch that would run unsplit anyway (one part, or row tiles that fill
+  // the chip by themselves) needs none and is never refused for its size.
+  if (!dense_mma_would_split(parts, m, n)) return dense_mma_fp4(act, act_stride, w, out, 0, m, n, k, stream, out_stride, nullptr, 0);
+  const size_t need = static_cast<size_t>(parts) * static_cast<size_t>(m) * static_cast<size_t>(n) * sizeof(float);
   if (need > kStaticScratchBytes)
     return fail_arg(std::string(who) + ": parts(k) * m * n floats (" + std::to_string(need) + " bytes) exceed the " +
                     std::to_string(kStaticScratchBytes) + "-byte static workspace; pass a workspace of your own to "
                     "dgpp_launch_mma_gemv_fp4_bf16");
   void* ws = nullptr;
-  const int rc = static_scratch(&ws, who);
+  const int rc = static_scratch(&ws, stream, who);
   if (rc != DGPP_OK) return rc;
   return dense_mma_fp4(act, act_stride, w, out, 0, m, n, k, stream, out_stride, ws, kStaticScratchBytes);
+}
+int dgpp_static_scratch_release(void) {
+  int device = -1;
+  const hipError_t err = hipGetDevice(&device);
+  if (err != hipSuccess) return finish(err, "static_scratch_release");
+  if (device < 0 || device >= kMaxDevices) return fail_arg("static_scratch_release: device ordinal beyond the per-device table");
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  g_scratch_bound[device] = false;
+  return DGPP_OK;
 }
 int dgpp_launch_dense_mma_fp4_bf16(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out, int m,
                                    int n, int k, void* stream) {

@@ -1060,6 +1060,12 @@ inline int max_stage_rows(int k) {
   return static_cast<int>(fit < 1 ? 1 : (fit > kMaxActRows ? kMaxActRows : fit));
 }
 
+// Whether the dense matrix-core launch runs its K parts in separate blocks through a workspace when it is given one
+// that is large enough (launch_dense_mfma's rule): more than one part, and row tiles that leave the chip under-filled.
+inline bool dense_mfma_would_split(int parts, int m, int n) {
+  return parts > 1 && static_cast<size_t>((n + 63) / 64) * static_cast<size_t>((m + 15) / 16) < 1024;
+}
+
 // Row groups per block of the dense matrix-core launch that runs the four parts of K side by side inside a block
 // (0: the row-tile form). Four up to one round of the chip's 256 CUs - one such block fills a CU, and 272 tiles, two
 // rounds with the second nearly empty, measured slower than the row-tile form; two (blocks half the size, two to a CU)
@@ -1095,8 +1101,7 @@ hipError_t launch_dense_mfma(const DenseArgs& a, hipStream_t stream, float* ws, 
   const MGeom g = mgeom<FMT>(a.k);
   const unsigned gx = static_cast<unsigned>((a.n + 63) / 64), gy = static_cast<unsigned>((a.m + kTileCols - 1) / kTileCols);
   const size_t need = static_cast<size_t>(g.parts) * a.m * a.n * sizeof(float);
-  const bool split = ws != nullptr && g.parts > 1 && ws_bytes >= need && static_cast<size_t>(gx) * gy < 1024 &&
-                     a.a4_scales == nullptr;
+  const bool split = ws != nullptr && ws_bytes >= need && dense_mfma_would_split(g.parts, a.m, a.n) && a.a4_scales == nullptr;
   const dim3 grid(gx, gy, split ? g.parts : 1);
   hipError_t err = hipSuccess;
   // Without a workspace the four parts of K run side by side inside a block while the row tiles alone would leave

@@ -145,6 +145,23 @@ DeviceMatrix place(const DgppMoeMatrixTensors& t, const Cut& c, Bump& bump, bool
   }
   if (dry) return d;
   if (!t.payload.data || !t.scales.data) refuse("a bound tensor has no data");
+  {
+    // The copies below read whole rows of the UNSLICED tensors at sizes derived from the payload's shape: a
+    // description whose byte counts do not cover them (hand-filled, or inconsistent) is refused before any read.
+    const Kind whole_kind = kind_of(t.format);
+    uint64_t need_payload, need_scales;
+    if (whole_kind == Kind::Fp8) {
+      need_payload = static_cast<uint64_t>(rows) * static_cast<uint64_t>(cols);
+      need_scales = static_cast<uint64_t>((rows + 127) / 128) * static_cast<uint64_t>((cols + 127) / 128) *
+                    (t.format == DGPP_BIND_FP8_BF16_SCALES ? 2u : 4u);
+    } else {
+      const int64_t group = whole_kind == Kind::Fp4 ? fp4_group_of(t.format) : 32;
+      need_payload = static_cast<uint64_t>(rows) * static_cast<uint64_t>(whole_kind == Kind::Fp4 ? cols / 2 : cols);
+      need_scales = static_cast<uint64_t>(rows) * static_cast<uint64_t>(cols / group);
+    }
+    if (rows <= 0 || cols <= 0 || t.payload.nbytes < need_payload || t.scales.nbytes < need_scales)
+      refuse("a bound tensor's byte count does not cover the matrix its shape describes");
+  }
   const uint8_t* payload = static_cast<const uint8_t*>(t.payload.data);
   const uint8_t* scales = static_cast<const uint8_t*>(t.scales.data);
   if (kind == Kind::Fp8) {

@@ -643,6 +643,11 @@ def launch_mma_gemv_fp4_bf16_static(act, act_stride, w: Fp4Matrix, out, m, n, k,
                                                             out_stride, _stream(stream)))
 
 
+def static_scratch_release():
+    """Frees the static workspace's binding to a stream (call once that stream's work is done)."""
+    _check(_lib.load().dgpp_static_scratch_release())
+
+
 def launch_mma_gemv_fp4_f32(act, act_stride, w: Fp4Matrix, out, m, n, k, out_stride=0, stream=None, ws=None, ws_bytes=0):
     _check(_lib.load().dgpp_launch_mma_gemv_fp4_f32(_p(act), act_stride, C.addressof(w), _p(out), m, n, k, out_stride,
                                                     _stream(stream), _p(ws), ws_bytes))

@@ -418,12 +418,18 @@ int dgpp_launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const D
  * under HIP graph capture, tight serving loops, harnesses that forbid allocation): the split-K partial sums go to a
  * workspace of DGPP_STATIC_SCRATCH_BYTES that the library holds in a file-scope device array (each GPU the library runs
  * on keeps its own copy until the process ends). The call allocates nothing and gives dgpp_launch_mma_gemv_fp4_bf16's
- * bits. parts(k) * m * n floats (parts = 4 from k = 4096, 2 from k = 2048, else 1) beyond the static workspace are
- * refused with DGPP_INVALID_ARGUMENT. Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two
- * streams, two threads) race; calls on one stream do not. The first call on a device looks the array's address up. */
+ * bits. Only launches that would run split use the workspace (more than one K part: parts = 4 from k = 4096, 2 from
+ * k = 2048; and fewer than 1024 tiles of 64 weight rows x 16 activation rows); of those, parts(k) * m * n floats
+ * beyond the static workspace are refused with DGPP_INVALID_ARGUMENT. Every other launch runs unsplit, uses no
+ * workspace and is never refused for its size. Every split call on a GPU shares that GPU's array, so the array is
+ * BOUND to the stream of the first split call: a split call on another stream of that GPU is refused with
+ * DGPP_INVALID_ARGUMENT (calls on two streams could overlap and race on the array; calls on one stream follow each
+ * other) until dgpp_static_scratch_release() - to be called once the bound stream's work is done - frees the
+ * binding. The first split call on a device looks the array's address up. */
 #define DGPP_STATIC_SCRATCH_BYTES (8u << 20)
 int dgpp_launch_mma_gemv_fp4_bf16_static(const uint16_t* act, size_t act_stride, const DgppFp4Matrix* w, uint16_t* out,
                                          int m, int n, int k, size_t out_stride, void* stream);
+int dgpp_static_scratch_release(void);
 /* src/kernels/mma_gemv.hpp:70-94 (launch_mma_gemv_fp8{,e8m0}_{bf16,f32}): the reference's streaming tensor-core GEMV for
  * FP8 weights. The same dispatch as dgpp_launch_scale_gemm_bf16 here: small batches run on the vector core where that
  * is the faster form on this chip (always up to four rows; five to eight rows without a workspace unless the matrix is

@@ -436,6 +436,12 @@ inline void launch_mma_gemv_fp4_bf16(const uint16_t* act, size_t act_stride, con
                                      size_t ws_bytes = 0) {
   detail::check(dgpp_launch_mma_gemv_fp4_bf16(act, act_stride, &w, out, m, n, k, out_stride, stream, ws, ws_bytes));
 }
+// The same on the library's own static workspace: allocates nothing (for callers that cannot allocate one).
+inline void launch_mma_gemv_fp4_bf16_static(const uint16_t* act, size_t act_stride, const GlmFp4Matrix& w, uint16_t* out, int m,
+                                            int n, int k, size_t out_stride, hipStream_t stream) {
+  detail::check(dgpp_launch_mma_gemv_fp4_bf16_static(act, act_stride, &w, out, m, n, k, out_stride, stream));
+}
+inline void static_scratch_release() { detail::check(dgpp_static_scratch_release()); }
 inline void launch_mma_gemv_fp4_f32(const uint16_t* act, size_t act_stride, const GlmFp4Matrix& w, float* out, int m, int n,
                                     int k, size_t out_stride, hipStream_t stream, void* ws = nullptr, size_t ws_bytes = 0) {
   detail::check(dgpp_launch_mma_gemv_fp4_f32(act, act_stride, &w, out, m, n, k, out_stride, stream, ws, ws_bytes));

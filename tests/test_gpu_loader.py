@@ -332,6 +332,16 @@ def test_resident_layer_from_a_bound_checkpoint_is_bitwise_the_hand_sliced_layer
             ML.ResidentMoeLayer(cfg, T, routed, shared=sh, shared_inter=sI, router_weight=rw, router_bias=rb, rank=world, world=world)
         with pytest.raises(L.InvalidArgument):
             ML.ResidentMoeLayer(cfg, T, routed, shared=sh, shared_inter=sI, rank=0, world=7)
+        # a description whose byte counts do not cover the matrix its shape describes is refused before any copy
+        for field in ("scales", "payload"):
+            info = getattr(routed[1][0], field)
+            kept = info.nbytes
+            info.nbytes = kept - 1
+            try:
+                with pytest.raises(L.InvalidArgument, match="byte count"):
+                    ML.ResidentMoeLayer(cfg, T, routed, shared=sh, shared_inter=sI, router_weight=rw, router_bias=rb, rank=0, world=world)
+            finally:
+                info.nbytes = kept
     finally:
         for f in files:
             f.close()   # the resident layers own device copies: the shards may go
