@@ -170,7 +170,8 @@ def test_c5_nvfp4_routed_plus_mxfp8_shared(gpu):
     """C5 at full size. The whole layer is ONE call of the layer driver (NVFP4 routed experts in decode slots, the MXFP8
     shared expert of its own width as dense projections beside them, combined last with weight 1): bitwise the chain
     stitched from the loose launchers, and held to the oracle on twelve tokens spread over the batch whose routes reach
-    at least 32 distinct generated experts."""
+    at least 32 distinct generated experts. The same layer is then routed by the MiniMax router from an FP32 gate
+    (routes and FP32 weights equal the oracle's bit for bit) and six of its tokens are held to the oracle."""
     E, H, I, K, T, SI = 256, 6144, 2048, 8, 64, 4096
     BASE, G = 10, 40                         # BASE generated experts; expert e uses variant e % G of them (variant g is
                                              # base expert g % BASE with its rows rotated by 64 * (g // BASE): other weights)
@@ -236,7 +237,28 @@ def test_c5_nvfp4_routed_plus_mxfp8_shared(gpu):
     layer1.enqueue_decode_routed(x_d, H, dev(ids[:13]), dev(w[:13]), out1b, 13)
     sync()
     assert np.array_equal(host(out1b, np.uint16), got[:13]), "rows do not depend on the batch they ride in"
+    # the same layer routed by its donor family's router (src/kernels/minimax.hpp:56-60: FP32 gate, sigmoid scores, the
+    # bias in the ranking only, FP32 weights never narrowed): routes equal the oracle's, six tokens against the oracle
+    rng = np.random.default_rng(0xC5)
+    gate = (rng.normal(0, 1.0, (E, H)) / np.sqrt(H)).astype(np.float32)
+    bias = rng.normal(0, 0.1, E).astype(np.float32)
+    sc_d, ids_d, w_d = dev_empty((T, E), np.float32), dev_empty((T, K), np.int32), dev_empty((T, K), np.float32)
+    L.minimax_router(x_d, dev(gate), dev(bias), T, H, E, K, 2.5, sc_d, ids_d, w_d)
+    out_mm = dev_empty((T, H), np.uint16)
+    layer1.enqueue_decode_routed(x_d, H, ids_d, w_d, out_mm, T)
+    sync()
+    scores_mm = np.ascontiguousarray(host(sc_d, np.float32))
+    ids_mm, w_mm = np.empty((T, K), np.int32), np.empty((T, K), np.float32)
+    orc.oracle().orc_minimax_route_scores(orc.p(scores_mm), orc.p(bias), T, E, K, 2.5, orc.p(ids_mm), orc.p(w_mm))
+    assert np.array_equal(host(ids_d, np.int32), ids_mm), "MiniMax routes"
+    assert np.array_equal(host(w_d, np.float32).view(np.uint32), w_mm.view(np.uint32)), "MiniMax weights, FP32 bit for bit"
     layer1.close()
+    sample_mm = [1, 14, 27, 39, 50, 62]
+    orc_experts_mm = [m.orc() for e in range(E) for m in gen[e % G][1]]
+    raw_mm, _ = orc.moe_forward(np.ascontiguousarray(x[sample_mm]), np.ascontiguousarray(ids_mm[sample_mm]),
+                                np.ascontiguousarray(w_mm[sample_mm]), H, I, SI, orc_experts_mm, [m.orc() for m in sh],
+                                float("inf"), threads=8)
+    expert_budget(np.ascontiguousarray(host(out_mm, np.uint16)[sample_mm]), raw_mm, "C5 routed by the MiniMax router")
     # twelve tokens against the oracle (routed NVFP4 chain + MXFP8 shared expert)
     sample = [0, 5, 11, 17, 23, 29, 34, 40, 46, 52, 58, 63]
     assert len({int(e) % G for e in ids[sample].ravel()}) >= 32, "the sampled tokens must reach >= 32 distinct generated experts"
