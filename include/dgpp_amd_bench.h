@@ -11,8 +11,10 @@
 extern "C" {
 #endif
 
-/* Bench A/B switches, process-wide, not thread-safe against concurrent launches (the reference
- * keeps such a switch in its launcher header too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90).
+/* Bench A/B switches, process-wide relaxed atomics (a set that races a launch is defined: the launch takes the old or
+ * the new value), 0 everywhere = the product behaviour; a library built with -DDGPP_NO_TUNE leaves them out
+ * (dgpp_tune_set stores nothing, dgpp_tune_get returns 0). The reference keeps such a switch in its launcher header
+ * too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90.
  * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: slots of one expert a
  * decode-slot block serves together (0 = default: 2 gate/up, 4 down; 1 = one slot per block);
  * key 2: row steps per block of the slot launches (0 = automatic); key 3: 1 stages activations before
