@@ -109,6 +109,7 @@ def main():
               "dimension with a single all-reduce after the layer; no multi-GPU figure is produced). "
               "Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+    os.environ.setdefault("DGPP_AMD_BENCH", "1")   # the A/B legs steer the library's measurement switches: opt in
     import torch
     from dgpp_amd import _lib, hostgen as hg, launch as L, moe_layer as ML
 
@@ -116,6 +117,10 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     lib = _lib.load()   # fails loudly when the HIP library has not been built
+    if not lib.dgpp_tune_enabled():
+        print("bench.py: the library's measurement switches are off (DGPP_AMD_BENCH is set to something other than 1, "
+              "or the library was built with -DDGPP_NO_TUNE): the A/B legs would all time the default form", file=sys.stderr)
+        sys.exit(1)
     for kv in filter(None, args.tune.split(",")):
         k, v = kv.split("=")
         lib.dgpp_tune_set(int(k), int(v))

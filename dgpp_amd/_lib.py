@@ -247,6 +247,7 @@ LAYER_SIGNATURES = {
 BENCH_SIGNATURES = {
     "dgpp_tune_set": (None, [_I, _I]),
     "dgpp_tune_get": (_I, [_I]),
+    "dgpp_tune_enabled": (_I, []),
     "dgpp_probe_copy": (_I, [_P, _P, C.c_size_t, _P]),
     "dgpp_probe_read": (_I, [_P, C.c_size_t, _P, _I, _I, _I, _P]),
 }

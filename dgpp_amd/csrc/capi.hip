@@ -4,6 +4,7 @@
 
 #include <limits.h>
 #include <atomic>
+#include <cstdlib>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -407,9 +408,23 @@ int dgpp_probe_read(const void* src, size_t bytes, void* sink, int nontemporal, 
     return fail_arg(std::string(who) + ": bytes and the pointer must be multiples of 16");
   return finish(run_probe_read(src, bytes, sink, nontemporal, blocks, span, as_stream(stream)), who);
 }
+// The switches take values only in a process that asked for them before its first call here (environment
+// DGPP_AMD_BENCH=1, read once): a host that merely links the library cannot have its launches steered by another
+// component's call.
+int dgpp_tune_enabled(void) {
+#ifndef DGPP_NO_TUNE
+  static const bool on = [] {
+    const char* e = std::getenv("DGPP_AMD_BENCH");
+    return e != nullptr && e[0] == '1' && e[1] == '\0';
+  }();
+  return on ? 1 : 0;
+#else
+  return 0;
+#endif
+}
 void dgpp_tune_set(int key, int value) {
 #ifndef DGPP_NO_TUNE
-  if (key >= 0 && key < kTuneCount) g_tune[key].store(value, std::memory_order_relaxed);
+  if (dgpp_tune_enabled() && key >= 0 && key < kTuneCount) g_tune[key].store(value, std::memory_order_relaxed);
 #else
   (void)key;
   (void)value;

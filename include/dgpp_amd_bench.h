@@ -12,7 +12,8 @@ extern "C" {
 #endif
 
 /* Bench A/B switches, process-wide relaxed atomics (a set that races a launch is defined: the launch takes the old or
- * the new value), 0 everywhere = the product behaviour; a library built with -DDGPP_NO_TUNE leaves them out
+ * the new value), 0 everywhere = the product behaviour. They are inert unless the process opted in through the
+ * environment (DGPP_AMD_BENCH=1, see dgpp_tune_enabled); a library built with -DDGPP_NO_TUNE leaves them out
  * (dgpp_tune_set stores nothing, dgpp_tune_get returns 0). The reference keeps such a switch in its launcher header
  * too: moe_set_fp8_ldm, src/kernels/glm_moe_launch.hpp:90.
  * key 0: preferred chunks per lane of the row geometry (0 = default 4); key 1: slots of one expert a
@@ -41,6 +42,10 @@ extern "C" {
  * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);
 int dgpp_tune_get(int key);
+/* 1 when the process opted in: the switches take values only if the environment held DGPP_AMD_BENCH=1 at the first
+ * call of dgpp_tune_set / dgpp_tune_enabled (read once). Without it dgpp_tune_set stores nothing and every launcher
+ * runs its measured default, whatever any component of the process calls. */
+int dgpp_tune_enabled(void);
 
 /* Measurement aid with no counterpart in the reference: a plain streaming copy of `bytes`
  * (a multiple of 16; both pointers 16-byte aligned) on `stream`. A profiler's HBM byte counters

@@ -1,3 +1,4 @@
+import os
 import sys
 from pathlib import Path
 
@@ -7,6 +8,10 @@ ROOT = Path(__file__).resolve().parent.parent
 for q in (str(ROOT), str(ROOT / "tests")):
     if q not in sys.path:
         sys.path.insert(0, q)
+
+
+# The tests that compare kernel forms steer the library's measurement switches: opt in before the library loads.
+os.environ.setdefault("DGPP_AMD_BENCH", "1")
 
 
 def pytest_configure(config):

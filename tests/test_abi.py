@@ -150,3 +150,21 @@ def test_slot_ex_launchers_refuse_what_they_cannot_honour():
             down(256, 1, fake, fake, fp4)            # the accumulation rides the shared pass, which is not run
         with pytest.raises(L.InvalidArgument):
             down(0, 3, fake, fake, fp4)              # ... or does not exist
+
+
+def test_measurement_switches_are_inert_unless_the_process_opted_in():
+    """dgpp_tune_set steers launcher choices for the benchmark and the form-comparison tests. A process that did not
+    ask for that (no DGPP_AMD_BENCH=1 in its environment when the library is first asked) keeps every switch at 0
+    whatever is called; one that did gets what it sets."""
+    import os
+    import subprocess
+    import sys
+    code = ("import ctypes, sys; lib = ctypes.CDLL(sys.argv[1]); lib.dgpp_tune_set(12, 2); lib.dgpp_tune_set(5, 1); "
+            "print(lib.dgpp_tune_enabled(), lib.dgpp_tune_get(12), lib.dgpp_tune_get(5))")
+    path = str(_lib.LIB_PATH)
+    env = {k: v for k, v in os.environ.items() if k != "DGPP_AMD_BENCH"}
+    off = subprocess.run([sys.executable, "-c", code, path], env=env, capture_output=True, text=True, check=True)
+    assert off.stdout.split() == ["0", "0", "0"]
+    env["DGPP_AMD_BENCH"] = "1"
+    on = subprocess.run([sys.executable, "-c", code, path], env=env, capture_output=True, text=True, check=True)
+    assert on.stdout.split() == ["1", "2", "1"]
