@@ -95,7 +95,7 @@ def parse():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MiB",
                     help="also run the library's plain copy kernel over this many MiB three times (counter calibration)")
     ap.add_argument("--configs", default=None, help="other benchmark configurations to time beside the headline, comma "
-                    "separated out of c1,c2,c4,c5,c5skew,w8a8,qwen_tail,slotbench,readprobe,router,pair,dispatch ('' for none; default: c1,c2,c4,c5, none under --tune)")
+                    "separated out of c1,c2,c2round,c4,c5,c5skew,w8a8,qwen_tail,slotbench,readprobe,router,pair,dispatch ('' for none; default: c1,c2,c4,c5, none under --tune)")
     ap.add_argument("--replays", type=int, default=0, help="timed graph replays per measurement (0 = at least 50 and at "
                     "least 1000 steps; a small number keeps a run under a profiler's counters short)")
     ap.add_argument("--tune", default="", help="bench A/B switches as key=value,... (dgpp_tune_set)")
@@ -392,6 +392,37 @@ def main():
             res[f"batch{m}_matrix_core_split_k"] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9,
                                                     "frac_of_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
         res["workload"] = "C2 dense NVFP4 GEMV 17408x5120 (gate_up shape), batch 1 and 8 (one weight pass)"
+        return res
+
+    def bench_c2round():
+        """C2's matrix at eight rows with the row count varied around what one resident round of the chip holds (1024 row
+        groups of 16 rows x four K parts = 4096 wavefront slots): 16384 rows fill one round exactly, 17408 (C2) and 20480
+        need a second."""
+        k, m = 5120, 8
+        res = {"workload": "dense NVFP4 GEMV [n x 5120], batch 8, n = 16384 / 17408 / 20480: the matrix-core forms around one "
+                           "resident round (4096 wavefront tasks)"}
+        act = torch.from_numpy(hg.normal_bf16(0xD6990021, (m, k)).view(np.int16)).to(dev)
+        for n in (16384, 17408, 20480):
+            payload, scales, ws2 = hg.encode_nvfp4(hg.normal_f32(0xD6990020, (n, k), 0.02))
+            glob = torch.tensor([1.0 / np.float32(ws2)], dtype=torch.float32, device=dev)
+            ring = ring_copies([torch.from_numpy(payload).to(dev), torch.from_numpy(scales).to(dev)],
+                               payload.nbytes + scales.nbytes)
+            mats = [L.Fp4Matrix(r[0].data_ptr(), r[1].data_ptr(), glob.data_ptr(), n, k, 16, 0, None) for r in ring]
+            out = torch.empty((len(ring), m, n), dtype=torch.int16, device=dev)
+            ws = torch.empty(4 * m * n, dtype=torch.float32, device=dev)
+            nbytes = n * k // 2 + n * k // 16 + 4 + m * (k * 2 + n * 2)
+            legs = {
+                "launcher": lambda i: L.launch_fp4_gemv_bf16(act, k, mats[i % len(ring)], out[i % len(ring)], m, n, k, stream),
+                "matrix_core_no_workspace": lambda i: L.launch_dense_mma_fp4_bf16(act, k, mats[i % len(ring)], out[i % len(ring)], m, n, k, stream),
+                "matrix_core_split_k": lambda i: L.launch_mma_gemv_fp4_bf16(act, k, mats[i % len(ring)], out[i % len(ring)], m, n, k, 0, stream,
+                                                                            ws, ws.numel() * 4),
+            }
+            row = {"row_groups_x_parts": (n // 16) * 4}
+            for name, fn in legs.items():
+                sec = time_graph(fn, args.steps, args.warmup)
+                row[name] = {"us": sec * 1e6, "gbps": nbytes / sec / 1e9}
+            res[f"n{n}"] = row
+            del ring, mats, out, ws
         return res
 
     def expert_table(per_expert_views, n_exp):
@@ -925,7 +956,7 @@ def main():
     if not args.only:
         for name in filter(None, configs.split(",")):
             t0 = time.time()
-            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c4": bench_c4, "c5": bench_c5, "c5skew": lambda: bench_c5(True), "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail, "readprobe": bench_readprobe,
+            other_configs[name] = {"c1": bench_c1, "c2": bench_c2, "c2round": bench_c2round, "c4": bench_c4, "c5": bench_c5, "c5skew": lambda: bench_c5(True), "w8a8": bench_w8a8, "qwen_tail": bench_qwen_tail, "readprobe": bench_readprobe,
                                    "slotbench": bench_slotbench, "router": bench_router, "pair": bench_pair, "dispatch": bench_dispatch}[name]()
             other_configs[name]["setup_and_run_seconds"] = time.time() - t0
             torch.cuda.empty_cache()
