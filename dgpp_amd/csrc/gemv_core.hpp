@@ -67,7 +67,7 @@ struct RowGeom {
 };
 // Bench A/B switches (host side, process-wide; 0 = the default behaviour). Set through
 // dgpp_tune_set; launchers read them when they pick a geometry or a kernel form.
-enum : int { kTunePreferP = 0, kTuneSlotRun = 1, kTuneSlotSteps = 2, kTuneSplitStage = 3, kTuneCore = 5, kTuneSelectAlone = 7, kTuneXcdGroup = 8, kTuneRouterTile = 10, kTuneTeams = 11, kTuneChain = 12, kTuneChainDownSteps = 13, kTuneCount = 14 };
+enum : int { kTunePreferP = 0, kTuneSlotRun = 1, kTuneSlotSteps = 2, kTuneSplitStage = 3, kTuneCore = 5, kTuneSelectAlone = 7, kTuneXcdGroup = 8, kTuneRouterTile = 10, kTuneTeams = 11, kTuneChain = 12, kTuneChainDownSteps = 13, kTuneGateUpWalks = 14, kTuneCount = 15 };
 int tune_get(int key);
 
 __host__ __device__ inline RowGeom row_geom(int chunks, int prefer_p = 4) {

@@ -1193,12 +1193,26 @@ hipError_t launch_grouped_mfma(const GroupedArgs& a, int n_segs, int z_ext, hipS
       return err != hipSuccess ? err : hipGetLastError();
     }
   }
+  // gate + up in one launch: while the grid is small (a few rounds of the chip) a block's wavefronts split into gate
+  // walkers and up walkers - twice the blocks, half the walk each (C4 100 -> 90 us); a large grid keeps every wavefront
+  // on both walks (C5: 1100 us against 1140 us split).
+  // (bench / test switch 14: 1 never splits, 2 always)
+  const int walks = tune_get(kTuneGateUpWalks);
+  const bool split_walks = a.gate_up != 0 && walks != 1 && (walks == 2 || static_cast<size_t>(grid.x) * grid.y * grid.z <= 2048);
   dispatch_bool(a.once != 0, [&](auto ntc) {
     dispatch_bool(a.gate_up != 0, [&](auto guc) {
-      auto kern = mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value, decltype(guc)::value>;
-      constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
-      err = ensure_lds(kern, lds);
-      if (err == hipSuccess) hipLaunchKernelGGL(kern, grid, dim3(kBlockThreads), lds, stream, a, g);
+      dispatch_bool(split_walks, [&](auto swc) {
+        constexpr bool GU = decltype(guc)::value, GUW = decltype(swc)::value;
+        if constexpr (GUW && !GU) {
+          err = hipErrorInvalidValue;   // not reached: split_walks implies gate_up
+        } else {
+          auto kern = mfma_grouped_kernel<FMT, kMfmaNB, decltype(ntc)::value, GU, false, GUW>;
+          constexpr size_t lds = kBlockMfmaLdsUnits * sizeof(uint4);
+          const dim3 gu_grid(static_cast<unsigned>((a.n + 31) / 32), grid.y, grid.z);
+          err = ensure_lds(kern, lds);
+          if (err == hipSuccess) hipLaunchKernelGGL(kern, GUW ? gu_grid : grid, dim3(kBlockThreads), lds, stream, a, g);
+        }
+      });
     });
   });
   return err != hipSuccess ? err : hipGetLastError();

@@ -366,9 +366,11 @@ __global__ void fold_parts_kernel(const float* __restrict__ partials, int parts,
 
 // GU: the block computes its rows of the segment's gate AND up matrices (two walks over K, the same
 // activations) and stores SwiGLU(bf16(gate), bf16(up)) — the bits of two launches and the elementwise kernel.
+// GUW (with GU): the block's wavefronts split into gate walkers and up walkers (32 rows of each per block, grid.x twice
+// as long) instead of every wavefront walking both matrices in turn: the same bits, taken for small grids.
 // A4 (NVFP4 experts only, GU false): the activations are NVFP4 rows (a.act the codes, a.act_stride bytes per row,
 // a.a4_scales / a.a4_gs); out = acc * (gs[row] * (1 / global)), the reference's epilogue (src/kernels/moe_w4a4.cu:424).
-template <int FMT, int NB, bool NT, bool GU, bool A4 = false>
+template <int FMT, int NB, bool NT, bool GU, bool A4 = false, bool GUW = false>
 __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedArgs a, MGeom g) {
   extern __shared__ uint4 lds[];
   const DgppMoeSegment seg = a.segs[blockIdx.y];
@@ -387,7 +389,39 @@ __global__ __launch_bounds__(kBlockThreads, 2) void mfma_grouped_kernel(GroupedA
     const size_t first = static_cast<size_t>(seg.row0 + c0);
     const uint16_t* act = a.act_rows ? a.act : a.act + first * a.act_stride;
     const int32_t* rows = a.act_rows ? a.act_rows + first : nullptr;
-    if constexpr (GU) {
+    if constexpr (GU && GUW) {
+      // Two wavefronts walk gate rows, the other two the SAME rows of up (a block covers 32 rows of each): every
+      // wavefront makes one walk - the one-matrix kernel's register budget, a wavefront more per SIMD than two walks
+      // in turn cost - and the block's one activation stage serves both matrices. The up sums meet the gate sums in LDS.
+      const int which = wave >> 1;
+      const int row0g = (static_cast<int>(blockIdx.x) * 2 + (wave & 1)) * kGroupRows;
+      const MatRef mw = mat_of_view<FMT>(a.views[seg.expert * 3 + which], &gp2);
+      f32x4_t t;
+      block_rows_mfma<FMT, NB, NT>(mw, act, a.act_stride, rows, mt, a.n, a.k, row0g, g, 0, g.parts, lds, t);
+      // an up wavefront parks its sums in its own tile region (its last operand reads were issued before: LDS keeps a
+      // wavefront's order); the gate wavefront of the same rows takes them after the barrier
+      uint4* regions = lds + kStageUnits;
+      if (which == 1) regions[wave * kTileUnits + lane] = __builtin_bit_cast(uint4, t);
+      __syncthreads();
+      if (which == 0) {
+        const f32x4_t sum_up = __builtin_bit_cast(f32x4_t, regions[(wave + 2) * kTileUnits + lane]);
+        const float *gp_up = nullptr;
+        (void)mat_of_view<FMT>(a.views[seg.expert * 3 + 1], &gp_up);
+        const float divisor_up = load_divisor<FMT>(gp_up);
+        sum = t;
+        if (a.gate_up == 2) {
+          store_tile<FMT>(sum, divisor, a.out, 0, (first + c) * a.out_stride, row0g, a.n, c < mt);
+          store_tile<FMT>(sum_up, divisor_up, a.out_up, 0, (first + c) * a.out_stride, row0g, a.n, c < mt);
+        } else if (c < mt) {
+          uint16_t* out = static_cast<uint16_t*>(a.out) + (first + c) * a.out_stride;
+          const int r = row0g + (lane >> 4) * 4;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (r + i < a.n)
+              out[r + i] = swiglu_bf16(finish_dot<FMT>(sum[i], divisor), finish_dot<FMT>(sum_up[i], divisor_up), a.limit);
+        }
+      }
+    } else if constexpr (GU) {
       // one compiled walk, run for the gate matrix and again for the up matrix (kept a loop: register budget)
       f32x4_t sum_up = {0.f, 0.f, 0.f, 0.f};
       float divisor_up = 1.f;

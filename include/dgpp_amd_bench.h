@@ -36,8 +36,10 @@ extern "C" {
  * per block, 3 with two for up to eight rows (0 = automatic: four while the row tiles fit one round of the chip, two for up
  * to a round and a quarter); key 12: 1 makes dgpp_launch_moe_slot_chain* run the launches the one-launch chain stands for, 2 makes
  * the layer driver take the one-launch chain for small routed-only decode batches (default: the driver runs the
- * launches; the chain measured slower); key 13: row steps per wavefront of the chain's down part (0 = automatic). Outputs do not depend on keys
- * 1 - 4 and 6 - 13; keys 0 and
+ * launches; the chain measured slower); key 13: row steps per wavefront of the chain's down part (0 = automatic);
+ * key 14: the fused gate + up matrix-core grouped launch: 1 = every wavefront walks both matrices in turn, 2 = the block's
+ * wavefronts split into gate walkers and up walkers (0 = automatic: split while the grid is at most 2048 blocks). Outputs do not
+ * depend on keys 1 - 4 and 6 - 14; keys 0 and
  * 5 change the fp32 summation order (every GEMV launcher follows them alike, so the launchers stay
  * bitwise twins of each other). */
 void dgpp_tune_set(int key, int value);

@@ -173,6 +173,16 @@ def test_dense_mma_fp4_prod_and_gate_up_are_the_grouped_kernel_on_one_segment(gp
     L.launch_dense_mma_fp4_prod_bf16(d.x, H, seg, d.views, 1, u1, m, I, H, None, d.fp4_group)
     L.launch_dense_mma_fp4_gate_up_bf16(d.x, H, seg, d.views, g2, u2, m, I, H, None, d.fp4_group)
     L.launch_moe_grouped_mma_fp4_bf16(d.x, H, seg, 1, m, 0, d.views, 0, gg, I, I, H, None, None, d.fp4_group)
+    from dgpp_amd import _lib
+    for form in (1, 2):   # both forms of the paired kernel (wavefronts walking both matrices / split into gate and up walkers)
+        g3, u3 = dev_empty((m, I), np.uint16), dev_empty((m, I), np.uint16)
+        _lib.load().dgpp_tune_set(14, form)
+        try:
+            L.launch_dense_mma_fp4_gate_up_bf16(d.x, H, seg, d.views, g3, u3, m, I, H, None, d.fp4_group)
+        finally:
+            _lib.load().dgpp_tune_set(14, 0)
+        sync()
+        assert np.array_equal(host(g3, np.uint16), host(g2, np.uint16)) and np.array_equal(host(u3, np.uint16), host(u2, np.uint16))
     sync()
     assert np.array_equal(host(g1, np.uint16), host(gg, np.uint16))
     assert np.array_equal(host(g1, np.uint16), host(g2, np.uint16)) and np.array_equal(host(u1, np.uint16), host(u2, np.uint16))
@@ -209,6 +219,22 @@ def test_grouped_mma_gate_up_swiglu_is_bitwise_the_three_launches(gpu, kind, lim
     sync()
     assert np.array_equal(host(got, np.uint16), host(want, np.uint16))
     assert np.array_equal(host(got_z, np.uint16), host(want, np.uint16)), "the z split does not change a row"
+    # both forms of the fused kernel: every wavefront walking gate and up in turn (1), and the block's wavefronts split
+    # into gate walkers and up walkers (2; what a small grid takes by itself)
+    from dgpp_amd import _lib
+    for form in (1, 2):
+        again = dev_empty((T * K, I), np.uint16)
+        _lib.load().dgpp_tune_set(14, form)
+        try:
+            if kind == "fp8":
+                L.launch_moe_grouped_mma_gate_up_swiglu(d.x, H, segs_d, E, T, 0, d.views, again, I, I, H, limit, None, rows_d)
+            else:
+                L.launch_moe_grouped_mma_gate_up_swiglu_fp4(d.x, H, segs_d, E, T, 0, d.views, again, I, I, H, limit, None, rows_d,
+                                                            d.fp4_group)
+        finally:
+            _lib.load().dgpp_tune_set(14, 0)
+        sync()
+        assert np.array_equal(host(again, np.uint16), host(want, np.uint16)), f"fused gate + up form {form}"
     with pytest.raises(L.InvalidArgument):
         L.launch_moe_grouped_mma_gate_up_swiglu(d.x, H, segs_d, E, 0, 0, d.views, got, I, I, H, limit, None, rows_d)
 
